@@ -1,0 +1,310 @@
+/* ------------------------------------------------------------------------ */
+/* ocean_hip.h -- C ABI of the MI355X (gfx950) device library for Ocean's   */
+/* core module.                                                             */
+/*                                                                          */
+/* Every entry point is plain C: pointers, sizes, byte strides and an       */
+/* opaque stream handle (a hipStream_t). The library replaces the Solid GPU */
+/* foundation (solid_gpu_<op>_<type> / solid_gpu_<op>[dtype] tables,        */
+/* solid/src/core/gpu/solid_core_gpu.src:42-439) and the CUDA runtime and   */
+/* cuBLAS calls made by Ocean's GPU device module (files in src/core/gpu). The */
+/* reference exports one symbol per (operation, type); this library takes   */
+/* the operation and the element type as leading integer arguments, so that */
+/* a lookup `solid_gpu_add[dtype](...)` becomes `och_binary(OCH_ADD, dtype, */
+/* ...)` with the remaining arguments unchanged.                            */
+/*                                                                          */
+/* Conventions (same as Solid, solid_core_gpu.src:20-28):                   */
+/*   - sizes are element counts, strides are in BYTES and may be zero       */
+/*     (broadcast) or, for source operands, negative;                       */
+/*   - at most OCH_MAX_DIMS dimensions;                                     */
+/*   - all device pointers belong to the current HIP device;                */
+/*   - functions return 0 on success and -1 on error; och_last_error()      */
+/*     returns the message (cf. solid_errmsg, solid error.h:24-35).         */
+/* All launches are asynchronous on the given stream unless stated.         */
+/* ------------------------------------------------------------------------ */
+#ifndef OCEAN_HIP_H
+#define OCEAN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OCH_MAX_DIMS 8
+
+/* Element types; numbering identical to OcDType (include/ocean/base/dtype.h:29-36)
+   and to Solid's type index (solid/include/solid/base/generic/dtype_macros.h:133-147). */
+typedef enum {
+   OCH_BOOL = 0, OCH_UINT8, OCH_UINT16, OCH_UINT32, OCH_UINT64,
+   OCH_INT8, OCH_INT16, OCH_INT32, OCH_INT64,
+   OCH_HALF, OCH_FLOAT, OCH_DOUBLE,
+   OCH_CHALF, OCH_CFLOAT, OCH_CDOUBLE,
+   OCH_DTYPE_COUNT
+} och_dtype;
+
+/* Scalar passed by value; mirrors solid_scalar (solid/include/solid/base/generic/scalar.h:30-50). */
+typedef struct { uint16_t real, imag; } och_chalf;
+typedef struct { float    real, imag; } och_cfloat;
+typedef struct { double   real, imag; } och_cdouble;
+typedef union {
+   uint8_t  _bool;  uint8_t  _uint8; uint16_t _uint16; uint32_t _uint32; uint64_t _uint64;
+   int8_t   _int8;  int16_t  _int16; int32_t  _int32;  int64_t  _int64;
+   uint16_t _half;  float    _float; double   _double;
+   och_chalf _chalf; och_cfloat _cfloat; och_cdouble _cdouble;
+} och_scalar;
+
+typedef void *och_stream;   /* hipStream_t */
+typedef void *och_event;    /* hipEvent_t  */
+
+/* Element size in bytes per dtype (solid_gpu_type_size[], solid_core_gpu.src:34). */
+extern const int och_type_size[OCH_DTYPE_COUNT];
+
+/* Message of the most recent failure in the calling thread. */
+const char *och_last_error(void);
+
+/* ======================================================================== */
+/* Device, stream, event and memory glue                                    */
+/* Replaces: src/core/gpu/device_gpu.c:155-420 (warm-up, streams, events),  */
+/*           src/core/gpu/storage_gpu.c:61-302 (alloc/free/copy/zero),      */
+/*           src/core/gpu/cuda.c:67-120 (set device, sticky status),        */
+/*           solid/src/base/gpu/solid_gpu.c:28-236 (property cache).        */
+/* ======================================================================== */
+typedef struct {
+   char     name[256];
+   char     arch[64];                 /* e.g. "gfx950:sramecc+:xnack-" */
+   size_t   total_global_mem;
+   size_t   shared_mem_per_block;     /* LDS bytes per workgroup */
+   int      multiprocessor_count;     /* compute units */
+   int      wavefront_size;
+   int      max_threads_per_block;
+   int      max_threads_per_multiprocessor;
+   int      clock_rate_khz;
+   int      memory_clock_rate_khz;
+   int      memory_bus_width;
+   int      l2_cache_size;
+   int      pci_bus_id, pci_device_id, pci_domain_id;
+   int      concurrent_kernels;
+   int      ecc_enabled;
+} och_device_prop;
+
+int och_device_count(int *count);                          /* device_gpu.c:184 cudaGetDeviceCount */
+int och_device_set(int device);                            /* cuda.c:67 OcCuda_setDevice */
+int och_device_get(int *device);
+int och_device_properties(int device, och_device_prop *p); /* device_gpu.c:471-637 */
+int och_device_can_access_peer(int device, int peer, int *result); /* device_gpu.c:447-454 */
+int och_device_warmup(int device);                         /* device_gpu.c:155-172 + template_dummy.cu:21-37 */
+int och_device_synchronize(void);
+
+int och_stream_create(och_stream *stream);                 /* device_gpu.c:251-288 */
+int och_stream_destroy(och_stream stream);                 /* device_gpu.c:324-346 */
+int och_stream_synchronize(och_stream stream);             /* device_gpu.c:374-382 */
+int och_stream_wait_event(och_stream stream, och_event event); /* device_gpu.c:411-420 */
+int och_event_create(och_event *event, int timing);        /* device_gpu.c:292-320; timing=0: disable timing */
+int och_event_destroy(och_event event);                    /* device_gpu.c:350-370 */
+int och_event_record(och_event event, och_stream stream);  /* device_gpu.c:398-407 */
+int och_event_synchronize(och_event event);                /* device_gpu.c:386-394 */
+int och_event_elapsed_ms(och_event start, och_event stop, float *ms);
+
+/* Stream-ordered allocation: the block is usable by work enqueued on `stream`
+   after the call and is returned to the device pool in stream order.
+   Replaces cudaMalloc/cudaFree of storage_gpu.c:83-95,107-116. */
+int och_malloc_async(void **ptr, size_t nbytes, och_stream stream);
+int och_free_async(void *ptr, och_stream stream);
+int och_malloc_host(void **ptr, size_t nbytes);            /* pinned host memory */
+int och_free_host(void *ptr);
+int och_memcpy_dtod_async(void *dst, const void *src, size_t nbytes, och_stream stream); /* storage_gpu.c:120-161 */
+int och_memcpy_peer_async(void *dst, int dst_device, const void *src, int src_device, size_t nbytes, och_stream stream);
+int och_memcpy_htod(void *dst, const void *src, size_t nbytes, och_stream stream);  /* storage_gpu.c:165-189; returns after completion */
+int och_memcpy_dtoh(void *dst, const void *src, size_t nbytes, och_stream stream);  /* storage_gpu.c:194-221; returns after completion */
+int och_memcpy_htod_async(void *dst, const void *src, size_t nbytes, och_stream stream);
+int och_memcpy_dtoh_async(void *dst, const void *src, size_t nbytes, och_stream stream);
+int och_memset_async(void *dst, int value, size_t nbytes, och_stream stream);       /* storage_gpu.c:283-302 */
+
+/* ======================================================================== */
+/* Fill, steps (elemwise1)                                                  */
+/* Replaces solid_gpu_fill / fill_nan / masked_fill (template_fill.cu:35-82)*/
+/* and steps_int64/double/cdouble (template_steps.cu:31-57).                */
+/* fill_nan follows the CPU semantics (only NaN entries are replaced,       */
+/* unary_ops.h:332-334,669-672); the reference GPU kernel overwrote all.    */
+/* ======================================================================== */
+int och_fill(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+             void *ptr, och_scalar value, och_stream stream);
+int och_fill_nan(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+                 void *ptr, och_scalar value, och_stream stream);
+/* ptr1: data (dtype), ptr2: mask (bool) */
+int och_masked_fill(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides1,
+                    void *ptr1, const ptrdiff_t *strides2, void *ptr2,
+                    och_scalar value, och_stream stream);
+int och_steps_int64(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+                    void *ptr, int64_t offset, int64_t step, och_stream stream);
+int och_steps_double(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+                     void *ptr, double offset, double step, och_stream stream);
+int och_steps_cdouble(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+                      void *ptr, och_cdouble offset, och_cdouble step, och_stream stream);
+
+/* ======================================================================== */
+/* Copy with type conversion, byteswap                                      */
+/* och_copy replaces solid_gpu_copy[src][dst] (template_copy.cu:55-86):     */
+/*   operand 1 is the source, operand 2 the destination; the shapes may     */
+/*   differ as long as the element counts match (reshape copy).             */
+/* och_byteswap / och_byteswap_copy have no GPU counterpart in the          */
+/*   reference; they replace solid_cpu_byteswap (template_byteswap.c:27-34) */
+/*   and solid_cpu_byteswap_copy (template_copy.c:79-89): each real part is */
+/*   byte-reversed; byteswap_copy reverses the SOURCE element first and     */
+/*   then converts (dtype_assign.h:297-371).                                */
+/* ======================================================================== */
+int och_copy(int dtype_src, int dtype_dst,
+             int ndims1, const size_t *size1, const ptrdiff_t *strides1, void *ptr1,
+             int ndims2, const size_t *size2, const ptrdiff_t *strides2, void *ptr2,
+             och_stream stream);
+int och_byteswap_copy(int dtype_src, int dtype_dst,
+             int ndims1, const size_t *size1, const ptrdiff_t *strides1, void *ptr1,
+             int ndims2, const size_t *size2, const ptrdiff_t *strides2, void *ptr2,
+             och_stream stream);
+int och_byteswap(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+                 void *ptr, och_stream stream);
+
+/* ======================================================================== */
+/* Unary elementwise: y = f(x)  (template_unary.cu:52-244)                  */
+/* Order follows include/ocean/core/generic/generate_tensor_unary.h:19-62.  */
+/* ptr2/strides2 NULL selects the in-place form. Output type: same as the   */
+/* input except OCH_ABSOLUTE on complex (real part type) and OCH_IS* (bool).*/
+/* ======================================================================== */
+typedef enum {
+   OCH_NEGATIVE = 0, OCH_BITWISE_NOT, OCH_LOGICAL_NOT, OCH_CONJ, OCH_RECIPROCAL,
+   OCH_SIN, OCH_COS, OCH_TAN, OCH_SINH, OCH_COSH, OCH_TANH,
+   OCH_ARCSIN, OCH_ARCCOS, OCH_ARCTAN, OCH_ARCSINH, OCH_ARCCOSH, OCH_ARCTANH,
+   OCH_SQRT, OCH_CBRT, OCH_SQUARE, OCH_EXP, OCH_EXP2, OCH_EXP10, OCH_EXPM1,
+   OCH_LOG, OCH_LOG2, OCH_LOG10, OCH_LOG1P,
+   OCH_ABSOLUTE, OCH_FABS, OCH_SIGN, OCH_CEIL, OCH_FLOOR, OCH_TRUNC, OCH_ROUND,
+   OCH_ISINF, OCH_ISNAN, OCH_ISFINITE, OCH_ISPOSINF, OCH_ISNEGINF,
+   OCH_UNARY_COUNT
+} och_unary_op;
+
+int och_unary(int op, int dtype, int ndims, const size_t *size,
+              const ptrdiff_t *strides1, void *ptr1,
+              const ptrdiff_t *strides2, void *ptr2, och_stream stream);
+int och_unary_supported(int op, int dtype);   /* LUT entry != 0, ocean_solid.h:131-140 */
+int och_unary_result_dtype(int op, int dtype);
+
+/* ======================================================================== */
+/* Binary elementwise: z = f(x, y)  (template_binary.cu:35-264)             */
+/* Order follows include/ocean/core/generic/generate_tensor_binary.h:19-47. */
+/* Operand 2 has type int8 for the bit shifts and int16 for integer/bool    */
+/* power (template_binary.cu:201,261); comparisons write bool.              */
+/* ptr3/strides3 NULL selects the in-place form z = x.                      */
+/* ======================================================================== */
+typedef enum {
+   OCH_ADD = 0, OCH_SUBTRACT, OCH_MULTIPLY, OCH_DIVIDE, OCH_TRUE_DIVIDE, OCH_FLOOR_DIVIDE,
+   OCH_POWER, OCH_MOD, OCH_FMOD,
+   OCH_MIN, OCH_MAX, OCH_FMIN, OCH_FMAX,
+   OCH_LT, OCH_LE, OCH_EQ, OCH_NE, OCH_GE, OCH_GT,
+   OCH_BITWISE_AND, OCH_BITWISE_OR, OCH_BITWISE_XOR,
+   OCH_LOGICAL_AND, OCH_LOGICAL_OR, OCH_LOGICAL_XOR,
+   OCH_BITSHIFT_LEFT, OCH_BITSHIFT_RIGHT,
+   OCH_BINARY_COUNT
+} och_binary_op;
+
+int och_binary(int op, int dtype, int ndims, const size_t *size,
+               const ptrdiff_t *strides1, void *ptr1,
+               const ptrdiff_t *strides2, void *ptr2,
+               const ptrdiff_t *strides3, void *ptr3, och_stream stream);
+int och_binary_supported(int op, int dtype);
+int och_binary_operand2_dtype(int op, int dtype);
+int och_binary_result_dtype(int op, int dtype);
+
+/* ======================================================================== */
+/* Full reductions (template_reduce_all.cu:54-88; reduce_all.h:365-414)     */
+/* One launch; the scalar result is written to host memory at `result` in   */
+/* the op's result type and the call returns after the stream has finished  */
+/* the reduction (the reference synchronises too, reduce_all.h:404-410).    */
+/* Result types (reduce_ops.h): any/all/all_*: bool (uint8); nnz: uint64;   */
+/* sum/prod: uint64 | int64 | same float; sum_abs/maximum_abs/minimum_abs/  */
+/* norm*: magnitude type (ints: uint64 for sum_abs, unsigned twin for       */
+/* max/min abs, double for norms); maximum/minimum: same as input.          */
+/* `buffer` may be NULL (the library then uses a per-device scratch block); */
+/* otherwise it must hold och_reduce_all_buffer_size() bytes.               */
+/* bound/lower/upper are given in the tensor's own dtype.                   */
+/* ======================================================================== */
+typedef enum {
+   OCH_R_ANY = 0, OCH_R_ALL, OCH_R_ALL_FINITE, OCH_R_ANY_INF, OCH_R_ANY_NAN,
+   OCH_R_NNZ, OCH_R_NNZ_NAN,
+   OCH_R_ALL_LT, OCH_R_ALL_LE, OCH_R_ALL_GT, OCH_R_ALL_GE,
+   OCH_R_ALL_GTLT, OCH_R_ALL_GTLE, OCH_R_ALL_GELT, OCH_R_ALL_GELE,
+   OCH_R_SUM, OCH_R_SUM_NAN, OCH_R_PROD, OCH_R_PROD_NAN,
+   OCH_R_SUM_ABS, OCH_R_SUM_ABS_NAN,
+   OCH_R_MAXIMUM, OCH_R_MINIMUM, OCH_R_MAXIMUM_ABS, OCH_R_MINIMUM_ABS,
+   OCH_R_NORM, OCH_R_NORM_NAN, OCH_R_NORM2, OCH_R_NORM2_NAN,
+   OCH_REDUCE_COUNT
+} och_reduce_op;
+
+size_t och_reduce_all_buffer_size(void);     /* solid_gpu_reduce_get_buffer_size, op/reduce_all.c:111-123 */
+int och_reduce_supported(int op, int dtype);
+int och_reduce_result_dtype(int op, int dtype);
+int och_reduce_all(int op, int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+                   void *ptr, const och_scalar *param1, const och_scalar *param2, double p,
+                   void *result, void *buffer, och_stream stream);
+/* Same reduction, result left in device memory at `dresult`; no host synchronisation. */
+int och_reduce_all_device(int op, int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+                   void *ptr, const och_scalar *param1, const och_scalar *param2, double p,
+                   void *dresult, void *buffer, och_stream stream);
+
+/* ======================================================================== */
+/* Axis reductions (template_reduce_axis.cu:54-80; reduce_axis.h:563-597)   */
+/* The configuration mirrors solid_gpu_reduce_axis_config: outer dimensions */
+/* (size/strides1 for the source, strides2 for the destination) and the     */
+/* reduced dimensions (rsize/rstrides into the source), as produced by      */
+/* OcSolid_analyzeReduceAxis (ocean_solid.c:382-462).                       */
+/* ======================================================================== */
+typedef struct {
+   int        ndims;                      /* outer (kept) dimensions */
+   size_t     size[OCH_MAX_DIMS];
+   ptrdiff_t  strides1[OCH_MAX_DIMS];     /* source strides of kept dims */
+   ptrdiff_t  strides2[OCH_MAX_DIMS];     /* destination strides */
+   int        rdims;                      /* reduced dimensions */
+   size_t     rsize[OCH_MAX_DIMS];
+   ptrdiff_t  rstrides[OCH_MAX_DIMS];
+   void      *ptr1;                       /* source */
+   void      *ptr2;                       /* destination, element type = reduce result dtype */
+   och_stream stream;
+} och_reduce_axis_config;
+
+int och_reduce_axis(int op, int dtype, const och_reduce_axis_config *config, double p);
+
+/* ======================================================================== */
+/* GEMM: C <- alpha * op(A) * op(B) + beta * C, column-major, ld in elements*/
+/* Replaces cublas{S,D,C,Z}gemm dispatch (src/core/gpu/op/tensor_blas_gpu.c */
+/* :132-231) and solid_gpu_gemm for bool/integers (template_blas.cu:99-237).*/
+/* trans in {'N','T','C'}. alpha/beta point to one element of `dtype` in    */
+/* host memory (scalar_mode_host != 0) or device memory.                    */
+/* bool uses OR/AND arithmetic (template_blas.cu).                          */
+/* ======================================================================== */
+int och_gemm(int dtype, char transA, char transB, size_t M, size_t N, size_t K,
+             const void *alpha, const void *A, ptrdiff_t ldA,
+             const void *B, ptrdiff_t ldB,
+             const void *beta, void *C, ptrdiff_t ldC,
+             int scalar_mode_host, och_stream stream);
+int och_gemm_supported(int dtype);
+
+/* ======================================================================== */
+/* Index operations (template_index.cu:37-57, index1.h:182, index2.h:188)   */
+/* ======================================================================== */
+int och_add_if_negative(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+                        void *ptr, och_scalar value, och_stream stream);
+int och_index_to_offset(int dtype, int nstrides, const int64_t *strides, ptrdiff_t stride_reduce,
+                        size_t nelem, ptrdiff_t stride1, void *ptr1,
+                        ptrdiff_t stride2, void *ptr2, och_stream stream);
+int och_get_index(int dtype, int ndims, const size_t *size, int64_t **offsets,
+                  const ptrdiff_t *strides1, void *ptr1,
+                  const ptrdiff_t *strides2, void *ptr2, och_stream stream);
+int och_set_index(int dtype, int ndims, const size_t *size, int64_t **offsets,
+                  const ptrdiff_t *strides1, void *ptr1,
+                  const ptrdiff_t *strides2, void *ptr2, och_stream stream);
+int och_fill_index(int dtype, int ndims, const size_t *size, int64_t **offsets,
+                   const ptrdiff_t *strides, void *ptr, och_scalar value, och_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,422 @@
+/* Strided / broadcast elementwise engine for gfx950.
+ *
+ * Replaces the reference's elemwise1/2/3 kernel families and their host-side
+ * analysers (solid/include/solid/core/gpu/apply_elemwise{1,2,3}.h,
+ * solid/src/core/gpu/op/apply_elemwise{,1,2,3}.c). Design:
+ *   - operands are normalised on the host: unit dimensions dropped, the
+ *     destination's strides made positive and sorted ascending, mergeable
+ *     dimensions merged, so that a contiguous tensor is one dimension;
+ *   - one thread handles groups of VEC consecutive elements of dimension 0;
+ *     operands whose dimension-0 stride equals their element size and whose
+ *     addresses are 16-byte aligned use one <=128-bit access per group, other
+ *     operands (strided, broadcast) use VEC element accesses;
+ *   - the index of a group is decomposed with multiply-high division by
+ *     invariant integers; one-dimensional problems need no division;
+ *   - 32-bit group indices; larger tensors are cut on the host.
+ */
+#pragma once
+#include "och_common.h"
+#include "och_dtypes.h"
+
+namespace och {
+
+/* ---- division by an invariant 32-bit integer d >= 2 ---------------------- */
+struct FastDiv { uint32_t d, m, s; };
+
+static inline FastDiv make_fastdiv(uint32_t d)
+{  /* q = (t + ((n - t) >> 1)) >> s with t = mulhi(m, n); exact for all 32-bit n */
+   FastDiv f; f.d = d; f.m = 0; f.s = 0;
+   if (d < 2) return f;
+   uint32_t L = 0; while ((1ull << L) < d) L++;
+   f.m = (uint32_t)((((1ull << L) - d) << 32) / d + 1);
+   f.s = L - 1;
+   return f;
+}
+OCH_HD uint32_t fastdiv(uint32_t n, const FastDiv &f)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+   uint32_t t = __umulhi(f.m, n);
+#else
+   uint32_t t = (uint32_t)(((uint64_t)f.m * n) >> 32);
+#endif
+   return (t + ((n - t) >> 1)) >> f.s;
+}
+
+/* ---- kernel parameters ---------------------------------------------------- */
+template <int NOPS> struct EwParams
+{
+   char    *ptr[NOPS];
+   int64_t  gstride[NOPS];                 /* byte step of one group (VEC elements) along dim 0 */
+   int64_t  estride[NOPS];                 /* byte step of one element along dim 0 */
+   int64_t  stride[NOPS][OCH_MAX_DIMS];    /* byte strides of dims 1.. (index 0 unused) */
+   FastDiv  div[OCH_MAX_DIMS];             /* div[0]: groups along dim 0, div[d]: size of dim d */
+   uint32_t ngroups;                       /* total number of groups */
+   uint64_t group0;                        /* first flat element index (for index-dependent ops) */
+   int      ndims;
+   int      vecmode[NOPS];                 /* 1: aligned unit stride, one wide access per group */
+};
+
+template <class T, int VEC> struct alignas((sizeof(T) * VEC) > 16 ? 16 : (sizeof(T) * VEC)) Pack { T v[VEC]; };
+
+template <class T, int VEC>
+OCH_D void load_pack(Pack<T, VEC> &p, const char *addr, int64_t estride, int vec)
+{
+   if (vec) p = *reinterpret_cast<const Pack<T, VEC> *>(addr);
+   else
+   {
+#pragma unroll
+      for (int k = 0; k < VEC; k++) p.v[k] = *reinterpret_cast<const T *>(addr + k * estride);
+   }
+}
+template <class T, int VEC>
+OCH_D void store_pack(const Pack<T, VEC> &p, char *addr, int64_t estride, int vec)
+{
+   if (vec) *reinterpret_cast<Pack<T, VEC> *>(addr) = p;
+   else
+   {
+#pragma unroll
+      for (int k = 0; k < VEC; k++) *reinterpret_cast<T *>(addr + k * estride) = p.v[k];
+   }
+}
+
+template <int NOPS>
+OCH_D void group_offsets(const EwParams<NOPS> &p, uint32_t g, int64_t (&off)[NOPS])
+{
+   if (p.ndims == 1)
+   {
+#pragma unroll
+      for (int k = 0; k < NOPS; k++) off[k] = (int64_t)g * p.gstride[k];
+   }
+   else
+   {  uint32_t q = fastdiv(g, p.div[0]);
+      uint32_t i = g - q * p.div[0].d;
+#pragma unroll
+      for (int k = 0; k < NOPS; k++) off[k] = (int64_t)i * p.gstride[k];
+      for (int d = 1; d < p.ndims - 1; d++)
+      {  uint32_t q2 = fastdiv(q, p.div[d]);
+         i = q - q2 * p.div[d].d; q = q2;
+#pragma unroll
+         for (int k = 0; k < NOPS; k++) off[k] += (int64_t)i * p.stride[k][d];
+      }
+#pragma unroll
+      for (int k = 0; k < NOPS; k++) off[k] += (int64_t)q * p.stride[k][p.ndims - 1];
+   }
+}
+
+#define OCH_EW_BLOCK 256
+
+/* z = f(x, y) */
+template <class F, int VEC, int UNR, bool FAST>
+__global__ __launch_bounds__(OCH_EW_BLOCK) void ew3_kernel(const EwParams<3> p)
+{
+   typedef typename F::A A; typedef typename F::B B; typedef typename F::R R;
+   const uint32_t base = blockIdx.x * (OCH_EW_BLOCK * UNR) + threadIdx.x;
+   Pack<A, VEC> a[UNR]; Pack<B, VEC> b[UNR]; int64_t off[UNR][3];
+#pragma unroll
+   for (int u = 0; u < UNR; u++)
+   {  uint32_t g = base + u * OCH_EW_BLOCK;
+      if (g < p.ngroups)
+      {  group_offsets<3>(p, g, off[u]);
+         load_pack<A, VEC>(a[u], p.ptr[0] + off[u][0], p.estride[0], FAST || p.vecmode[0]);
+         load_pack<B, VEC>(b[u], p.ptr[1] + off[u][1], p.estride[1], FAST || p.vecmode[1]);
+      }
+   }
+#pragma unroll
+   for (int u = 0; u < UNR; u++)
+   {  uint32_t g = base + u * OCH_EW_BLOCK;
+      if (g < p.ngroups)
+      {  Pack<R, VEC> r;
+#pragma unroll
+         for (int k = 0; k < VEC; k++) r.v[k] = F::f(a[u].v[k], b[u].v[k]);
+         store_pack<R, VEC>(r, p.ptr[2] + off[u][2], p.estride[2], FAST || p.vecmode[2]);
+      }
+   }
+}
+
+/* y = f(x) */
+template <class F, int VEC, int UNR, bool FAST>
+__global__ __launch_bounds__(OCH_EW_BLOCK) void ew2_kernel(const EwParams<2> p)
+{
+   typedef typename F::A A; typedef typename F::R R;
+   const uint32_t base = blockIdx.x * (OCH_EW_BLOCK * UNR) + threadIdx.x;
+   Pack<A, VEC> a[UNR]; int64_t off[UNR][2];
+#pragma unroll
+   for (int u = 0; u < UNR; u++)
+   {  uint32_t g = base + u * OCH_EW_BLOCK;
+      if (g < p.ngroups)
+      {  group_offsets<2>(p, g, off[u]);
+         load_pack<A, VEC>(a[u], p.ptr[0] + off[u][0], p.estride[0], FAST || p.vecmode[0]);
+      }
+   }
+#pragma unroll
+   for (int u = 0; u < UNR; u++)
+   {  uint32_t g = base + u * OCH_EW_BLOCK;
+      if (g < p.ngroups)
+      {  Pack<R, VEC> r;
+#pragma unroll
+         for (int k = 0; k < VEC; k++) r.v[k] = F::f(a[u].v[k]);
+         store_pack<R, VEC>(r, p.ptr[1] + off[u][1], p.estride[1], FAST || p.vecmode[1]);
+      }
+   }
+}
+
+/* x = f(x, flat index, param): fill, conditional fill, steps. F::RMW tells whether the
+   old value is read. The flat index counts elements in the order of the NORMALISED
+   dimensions, so index-dependent functors are launched without reordering. */
+template <class F, int VEC, int UNR, bool FAST>
+__global__ __launch_bounds__(OCH_EW_BLOCK) void ew1_kernel(const EwParams<1> p, const typename F::Param prm)
+{
+   typedef typename F::R R;
+   const uint32_t base = blockIdx.x * (OCH_EW_BLOCK * UNR) + threadIdx.x;
+#pragma unroll
+   for (int u = 0; u < UNR; u++)
+   {  uint32_t g = base + u * OCH_EW_BLOCK;
+      if (g < p.ngroups)
+      {  int64_t off[1];
+         group_offsets<1>(p, g, off);
+         Pack<R, VEC> r;
+         if constexpr (F::RMW) load_pack<R, VEC>(r, p.ptr[0] + off[0], p.estride[0], FAST || p.vecmode[0]);
+#pragma unroll
+         for (int k = 0; k < VEC; k++) r.v[k] = F::f(r.v[k], p.group0 + (uint64_t)g * VEC + k, prm);
+         store_pack<R, VEC>(r, p.ptr[0] + off[0], p.estride[0], FAST || p.vecmode[0]);
+      }
+   }
+}
+
+/* ---- host side: normalisation --------------------------------------------- */
+template <int NOPS> struct EwShape
+{
+   int      ndims;
+   uint64_t size[OCH_MAX_DIMS];
+   int64_t  stride[NOPS][OCH_MAX_DIMS];
+   char    *ptr[NOPS];
+   uint64_t nelem;
+};
+
+/* key: operand whose strides drive sorting (the destination). reorder=false keeps the
+   caller's dimension order and stride signs (needed when the flat index matters).
+   Returns -1 on bad input. */
+template <int NOPS>
+static int ew_normalize(EwShape<NOPS> &s, int ndims, const size_t *size,
+                        const ptrdiff_t *const strides[NOPS], void *const ptr[NOPS],
+                        int key, bool reorder)
+{
+   if (ndims < 0 || ndims > OCH_MAX_DIMS) return set_error("invalid number of dimensions (%d)", ndims);
+   s.nelem = 1; s.ndims = 0;
+   for (int k = 0; k < NOPS; k++) s.ptr[k] = (char *)ptr[k];
+   for (int d = 0; d < ndims; d++) s.nelem *= size[d];
+   if (s.nelem == 0) return 0;
+   for (int d = 0; d < ndims; d++)
+   {  if (size[d] == 1) continue;
+      int j = s.ndims++;
+      s.size[j] = size[d];
+      for (int k = 0; k < NOPS; k++) s.stride[k][j] = strides[k][d];
+      if (reorder && s.stride[key][j] < 0)
+      {  for (int k = 0; k < NOPS; k++)
+         {  s.ptr[k] += s.stride[k][j] * (int64_t)(size[d] - 1);
+            s.stride[k][j] = -s.stride[k][j];
+         }
+      }
+   }
+   if (reorder)
+   {  for (int i = 1; i < s.ndims; i++)          /* insertion sort, ascending key strides */
+      {  for (int j = i; j > 0; j--)
+         {  bool swap = false;
+            if (s.stride[key][j - 1] > s.stride[key][j]) swap = true;
+            else if (s.stride[key][j - 1] == s.stride[key][j])
+            {  for (int k = 0; k < NOPS; k++)
+               {  if (s.stride[k][j - 1] == s.stride[k][j]) continue;
+                  swap = s.stride[k][j - 1] > s.stride[k][j]; break;
+               }
+            }
+            if (!swap) break;
+            uint64_t t = s.size[j]; s.size[j] = s.size[j - 1]; s.size[j - 1] = t;
+            for (int k = 0; k < NOPS; k++)
+            {  int64_t r = s.stride[k][j]; s.stride[k][j] = s.stride[k][j - 1]; s.stride[k][j - 1] = r; }
+         }
+      }
+   }
+   if (s.ndims > 1)
+   {  int j = 0;
+      for (int i = 1; i < s.ndims; i++)
+      {  bool merge = true;
+         for (int k = 0; k < NOPS; k++)
+            if (s.stride[k][i] != s.stride[k][j] * (int64_t)s.size[j]) { merge = false; break; }
+         if (merge) s.size[j] *= s.size[i];
+         else
+         {  j++; s.size[j] = s.size[i];
+            for (int k = 0; k < NOPS; k++) s.stride[k][j] = s.stride[k][i];
+         }
+      }
+      s.ndims = j + 1;
+   }
+   if (s.ndims == 0)
+   {  s.ndims = 1; s.size[0] = 1;
+      for (int k = 0; k < NOPS; k++) s.stride[k][0] = 0;
+   }
+   return 0;
+}
+
+/* Launcher signature: (shape with every size < 2^32 and nelem < 2^32, vec flag, first flat index) */
+template <int NOPS, class L>
+static int ew_launch_chunked(EwShape<NOPS> s, uint64_t flat0, L &&launch)
+{
+   const uint64_t LIMIT = 0xFFFF0000ull;          /* keeps block base + thread offset from wrapping */
+   if (s.nelem == 0) return 0;
+   if (s.nelem <= LIMIT) return launch(s, flat0);
+   int last = s.ndims - 1;
+   uint64_t inner = s.nelem / s.size[last];
+   uint64_t chunk = (s.ndims == 1) ? (1ull << 30) : (inner <= LIMIT ? LIMIT / inner : 0);
+   if (chunk >= 1)
+   {  for (uint64_t start = 0; start < s.size[last]; start += chunk)
+      {  EwShape<NOPS> c = s;
+         c.size[last] = (s.size[last] - start < chunk) ? (s.size[last] - start) : chunk;
+         c.nelem = inner * c.size[last];
+         for (int k = 0; k < NOPS; k++) c.ptr[k] = s.ptr[k] + (int64_t)start * s.stride[k][last];
+         if (launch(c, flat0 + start * inner) != 0) return -1;
+      }
+      return 0;
+   }
+   for (uint64_t i = 0; i < s.size[last]; i++)
+   {  EwShape<NOPS> c = s;
+      c.ndims = last; c.nelem = inner;
+      for (int k = 0; k < NOPS; k++) c.ptr[k] = s.ptr[k] + (int64_t)i * s.stride[k][last];
+      if (ew_launch_chunked<NOPS>(c, flat0 + i * inner, launch) != 0) return -1;
+   }
+   return 0;
+}
+
+/* Fill kernel parameters for a VEC-wide launch; returns false when VEC does not fit */
+template <int NOPS>
+static bool ew_params(EwParams<NOPS> &p, const EwShape<NOPS> &s, int vec, const int elemsize[NOPS], uint64_t flat0)
+{
+   if (s.size[0] % vec != 0) return false;
+   p.ndims = s.ndims;
+   p.ngroups = (uint32_t)(s.nelem / vec);
+   p.group0 = flat0;
+   p.div[0] = make_fastdiv((uint32_t)(s.size[0] / vec));
+   for (int d = 1; d < s.ndims; d++) p.div[d] = make_fastdiv((uint32_t)s.size[d]);
+   for (int k = 0; k < NOPS; k++)
+   {  p.ptr[k] = s.ptr[k];
+      p.estride[k] = s.stride[k][0];
+      p.gstride[k] = s.stride[k][0] * vec;
+      for (int d = 0; d < OCH_MAX_DIMS; d++) p.stride[k][d] = (d < s.ndims) ? s.stride[k][d] : 0;
+      int width = elemsize[k] * vec; if (width > 16) width = 16;
+      bool v = (s.stride[k][0] == elemsize[k]) && (((uintptr_t)s.ptr[k]) % width == 0);
+      for (int d = 1; d < s.ndims && v; d++) if (s.stride[k][d] % width != 0) v = false;
+      p.vecmode[k] = v ? 1 : 0;
+   }
+   return true;
+}
+
+template <class T> constexpr int vec_for() { return (16 / (int)sizeof(T)) > 0 ? (16 / (int)sizeof(T)) : 1; }
+template <class A, class B, class C> constexpr int vec_for3()
+{  constexpr int m = sizeof(A) > sizeof(B) ? (sizeof(A) > sizeof(C) ? sizeof(A) : sizeof(C)) : (sizeof(B) > sizeof(C) ? sizeof(B) : sizeof(C));
+   return (16 / m) > 0 ? (16 / m) : 1;
+}
+
+#define OCH_EW_UNR 4
+
+/* ---- generic launchers ------------------------------------------------------ */
+/* Picks the kernel variant for one (chunk of a) normalised shape:
+     wide  : every operand has aligned unit stride along dim 0 -> VEC-wide accesses only
+     mixed : dim 0 divisible by VEC, some operands strided or broadcast
+     single: one element per thread (odd sizes); for 1-D shapes only the tail uses it   */
+template <int NOPS, class LW, class LM, class LS>
+static int ew_dispatch(const EwShape<NOPS> &s, uint64_t flat0, int vec, const int (&es)[NOPS],
+                       LW &&wide, LM &&mixed, LS &&single)
+{
+   EwParams<NOPS> p;
+   auto run = [&](const EwShape<NOPS> &sh, uint64_t f0) -> bool
+   {  if (vec <= 1 || !ew_params<NOPS>(p, sh, vec, es, f0)) return false;
+      bool all = true;
+      for (int k = 0; k < NOPS; k++) all = all && p.vecmode[k];
+      if (all) wide(p, (p.ngroups + OCH_EW_BLOCK * OCH_EW_UNR - 1) / (OCH_EW_BLOCK * OCH_EW_UNR));
+      else     mixed(p, (p.ngroups + OCH_EW_BLOCK * 2 - 1) / (OCH_EW_BLOCK * 2));
+      return true;
+   };
+   if (!run(s, flat0))
+   {  if (vec > 1 && s.ndims == 1 && s.size[0] > (uint64_t)vec)
+      {  EwShape<NOPS> body = s, tail = s;
+         body.size[0] = s.size[0] - s.size[0] % vec; body.nelem = body.size[0];
+         tail.size[0] = s.size[0] % vec; tail.nelem = tail.size[0];
+         for (int k = 0; k < NOPS; k++) tail.ptr[k] = s.ptr[k] + (int64_t)body.size[0] * s.stride[k][0];
+         run(body, flat0);
+         ew_params<NOPS>(p, tail, 1, es, flat0 + body.nelem);
+         single(p, 1u);
+      }
+      else
+      {  ew_params<NOPS>(p, s, 1, es, flat0);
+         single(p, (p.ngroups + OCH_EW_BLOCK - 1) / OCH_EW_BLOCK);
+      }
+   }
+   OCH_CHECK_LAUNCH();
+   return 0;
+}
+
+template <class F>
+static int launch_ew3(int ndims, const size_t *size,
+                      const ptrdiff_t *st1, void *p1, const ptrdiff_t *st2, void *p2,
+                      const ptrdiff_t *st3, void *p3, hipStream_t stream)
+{
+   typedef typename F::A A; typedef typename F::B B; typedef typename F::R R;
+   constexpr int VEC = vec_for3<A, B, R>();
+   const ptrdiff_t *strides[3] = { st1, st2, st3 }; void *ptrs[3] = { p1, p2, p3 };
+   EwShape<3> shape;
+   if (ew_normalize<3>(shape, ndims, size, strides, ptrs, 2, true) != 0) return -1;
+   const int es[3] = { (int)sizeof(A), (int)sizeof(B), (int)sizeof(R) };
+   return ew_launch_chunked<3>(shape, 0, [&](const EwShape<3> &s, uint64_t flat0) -> int
+   {  return ew_dispatch<3>(s, flat0, VEC, es,
+         [&](const EwParams<3> &p, uint32_t blocks)
+         {  hipLaunchKernelGGL((ew3_kernel<F, VEC, OCH_EW_UNR, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
+         [&](const EwParams<3> &p, uint32_t blocks)
+         {  hipLaunchKernelGGL((ew3_kernel<F, VEC, 2, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
+         [&](const EwParams<3> &p, uint32_t blocks)
+         {  hipLaunchKernelGGL((ew3_kernel<F, 1, 1, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); });
+   });
+}
+
+template <class F>
+static int launch_ew2(int ndims, const size_t *size,
+                      const ptrdiff_t *st1, void *p1, const ptrdiff_t *st2, void *p2, hipStream_t stream)
+{
+   typedef typename F::A A; typedef typename F::R R;
+   constexpr int VEC = vec_for3<A, A, R>();
+   const ptrdiff_t *strides[2] = { st1, st2 }; void *ptrs[2] = { p1, p2 };
+   EwShape<2> shape;
+   if (ew_normalize<2>(shape, ndims, size, strides, ptrs, 1, true) != 0) return -1;
+   const int es[2] = { (int)sizeof(A), (int)sizeof(R) };
+   return ew_launch_chunked<2>(shape, 0, [&](const EwShape<2> &s, uint64_t flat0) -> int
+   {  return ew_dispatch<2>(s, flat0, VEC, es,
+         [&](const EwParams<2> &p, uint32_t blocks)
+         {  hipLaunchKernelGGL((ew2_kernel<F, VEC, OCH_EW_UNR, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
+         [&](const EwParams<2> &p, uint32_t blocks)
+         {  hipLaunchKernelGGL((ew2_kernel<F, VEC, 2, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
+         [&](const EwParams<2> &p, uint32_t blocks)
+         {  hipLaunchKernelGGL((ew2_kernel<F, 1, 1, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); });
+   });
+}
+
+/* reorder=false for functors that use the flat index */
+template <class F>
+static int launch_ew1(int ndims, const size_t *size, const ptrdiff_t *st, void *ptr,
+                      const typename F::Param &prm, bool reorder, hipStream_t stream)
+{
+   typedef typename F::R R;
+   constexpr int VEC = vec_for<R>();
+   const ptrdiff_t *strides[1] = { st }; void *ptrs[1] = { ptr };
+   EwShape<1> shape;
+   if (ew_normalize<1>(shape, ndims, size, strides, ptrs, 0, reorder) != 0) return -1;
+   const int es[1] = { (int)sizeof(R) };
+   return ew_launch_chunked<1>(shape, 0, [&](const EwShape<1> &s, uint64_t flat0) -> int
+   {  return ew_dispatch<1>(s, flat0, VEC, es,
+         [&](const EwParams<1> &p, uint32_t blocks)
+         {  hipLaunchKernelGGL((ew1_kernel<F, VEC, OCH_EW_UNR, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p, prm); },
+         [&](const EwParams<1> &p, uint32_t blocks)
+         {  hipLaunchKernelGGL((ew1_kernel<F, VEC, 2, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p, prm); },
+         [&](const EwParams<1> &p, uint32_t blocks)
+         {  hipLaunchKernelGGL((ew1_kernel<F, 1, 1, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p, prm); });
+   });
+}
+
+} /* namespace och */

@@ -1,0 +1,143 @@
+/* Device, stream, event and memory glue plus error reporting.
+ * Counterpart of src/core/gpu/device_gpu.c:155-420, storage_gpu.c:61-302,
+ * cuda.c:67-120 and solid/src/base/gpu/solid_gpu.c:28-236 in the reference,
+ * written against the HIP runtime: one hipStream_t per stream handle,
+ * stream-ordered allocation from the device's default memory pool. */
+#include "och_common.h"
+#include <string.h>
+
+namespace och {
+static thread_local char g_errmsg[512] = "";
+int set_error(const char *fmt, ...)
+{
+   va_list ap; va_start(ap, fmt); vsnprintf(g_errmsg, sizeof(g_errmsg), fmt, ap); va_end(ap);
+   return -1;
+}
+void clear_error() { g_errmsg[0] = 0; }
+__global__ void warmup_kernel(int *p) { if (p) *p = 1; }
+}
+
+extern "C" {
+
+const int och_type_size[OCH_DTYPE_COUNT] = { 1, 1, 2, 4, 8, 1, 2, 4, 8, 2, 4, 8, 4, 8, 16 };
+
+const char *och_last_error(void) { return och::g_errmsg; }
+
+int och_device_count(int *count)
+{
+   hipError_t e = hipGetDeviceCount(count);
+   if (e == hipErrorNoDevice) { *count = 0; (void)hipGetLastError(); return 0; }
+   OCH_CHECK_HIP(e);
+   return 0;
+}
+int och_device_set(int device) { OCH_CHECK_HIP(hipSetDevice(device)); return 0; }
+int och_device_get(int *device) { OCH_CHECK_HIP(hipGetDevice(device)); return 0; }
+
+int och_device_properties(int device, och_device_prop *p)
+{
+   hipDeviceProp_t d;
+   OCH_CHECK_HIP(hipGetDeviceProperties(&d, device));
+   memset(p, 0, sizeof(*p));
+   strncpy(p->name, d.name, sizeof(p->name) - 1);
+   strncpy(p->arch, d.gcnArchName, sizeof(p->arch) - 1);
+   p->total_global_mem = d.totalGlobalMem;
+   p->shared_mem_per_block = d.sharedMemPerBlock;
+   p->multiprocessor_count = d.multiProcessorCount;
+   p->wavefront_size = d.warpSize;
+   p->max_threads_per_block = d.maxThreadsPerBlock;
+   p->max_threads_per_multiprocessor = d.maxThreadsPerMultiProcessor;
+   p->clock_rate_khz = d.clockRate;
+   p->memory_clock_rate_khz = d.memoryClockRate;
+   p->memory_bus_width = d.memoryBusWidth;
+   p->l2_cache_size = d.l2CacheSize;
+   p->pci_bus_id = d.pciBusID; p->pci_device_id = d.pciDeviceID; p->pci_domain_id = d.pciDomainID;
+   p->concurrent_kernels = d.concurrentKernels;
+   p->ecc_enabled = d.ECCEnabled;
+   return 0;
+}
+
+int och_device_can_access_peer(int device, int peer, int *result)
+{
+   OCH_CHECK_HIP(hipDeviceCanAccessPeer(result, device, peer));
+   return 0;
+}
+
+int och_device_warmup(int device)
+{  /* pay the runtime's first-use cost (context, code object load) up front */
+   int prev;
+   OCH_CHECK_HIP(hipGetDevice(&prev));
+   OCH_CHECK_HIP(hipSetDevice(device));
+   hipLaunchKernelGGL(och::warmup_kernel, dim3(1), dim3(1), 0, 0, (int *)nullptr);
+   OCH_CHECK_LAUNCH();
+   OCH_CHECK_HIP(hipDeviceSynchronize());
+   OCH_CHECK_HIP(hipSetDevice(prev));
+   return 0;
+}
+int och_device_synchronize(void) { OCH_CHECK_HIP(hipDeviceSynchronize()); return 0; }
+
+int och_stream_create(och_stream *stream)
+{
+   hipStream_t s;
+   OCH_CHECK_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+   *stream = (och_stream)s; return 0;
+}
+int och_stream_destroy(och_stream stream) { OCH_CHECK_HIP(hipStreamDestroy((hipStream_t)stream)); return 0; }
+int och_stream_synchronize(och_stream stream) { OCH_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream)); return 0; }
+int och_stream_wait_event(och_stream stream, och_event event)
+{  OCH_CHECK_HIP(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0)); return 0; }
+
+int och_event_create(och_event *event, int timing)
+{
+   hipEvent_t e;
+   OCH_CHECK_HIP(hipEventCreateWithFlags(&e, timing ? hipEventDefault : hipEventDisableTiming));
+   *event = (och_event)e; return 0;
+}
+int och_event_destroy(och_event event) { OCH_CHECK_HIP(hipEventDestroy((hipEvent_t)event)); return 0; }
+int och_event_record(och_event event, och_stream stream)
+{  OCH_CHECK_HIP(hipEventRecord((hipEvent_t)event, (hipStream_t)stream)); return 0; }
+int och_event_synchronize(och_event event) { OCH_CHECK_HIP(hipEventSynchronize((hipEvent_t)event)); return 0; }
+int och_event_elapsed_ms(och_event start, och_event stop, float *ms)
+{  OCH_CHECK_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop)); return 0; }
+
+int och_malloc_async(void **ptr, size_t nbytes, och_stream stream)
+{
+   *ptr = nullptr;
+   if (nbytes == 0) return 0;
+   OCH_CHECK_HIP(hipMallocAsync(ptr, nbytes, (hipStream_t)stream));
+   return 0;
+}
+int och_free_async(void *ptr, och_stream stream)
+{
+   if (ptr == nullptr) return 0;
+   OCH_CHECK_HIP(hipFreeAsync(ptr, (hipStream_t)stream));
+   return 0;
+}
+int och_malloc_host(void **ptr, size_t nbytes) { OCH_CHECK_HIP(hipHostMalloc(ptr, nbytes ? nbytes : 1, hipHostMallocDefault)); return 0; }
+int och_free_host(void *ptr) { if (ptr) OCH_CHECK_HIP(hipHostFree(ptr)); return 0; }
+
+int och_memcpy_dtod_async(void *dst, const void *src, size_t nbytes, och_stream stream)
+{  if (nbytes) OCH_CHECK_HIP(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToDevice, (hipStream_t)stream)); return 0; }
+int och_memcpy_peer_async(void *dst, int dst_device, const void *src, int src_device, size_t nbytes, och_stream stream)
+{  if (nbytes) OCH_CHECK_HIP(hipMemcpyPeerAsync(dst, dst_device, src, src_device, nbytes, (hipStream_t)stream)); return 0; }
+int och_memcpy_htod_async(void *dst, const void *src, size_t nbytes, och_stream stream)
+{  if (nbytes) OCH_CHECK_HIP(hipMemcpyAsync(dst, src, nbytes, hipMemcpyHostToDevice, (hipStream_t)stream)); return 0; }
+int och_memcpy_dtoh_async(void *dst, const void *src, size_t nbytes, och_stream stream)
+{  if (nbytes) OCH_CHECK_HIP(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, (hipStream_t)stream)); return 0; }
+int och_memcpy_htod(void *dst, const void *src, size_t nbytes, och_stream stream)
+{
+   if (nbytes == 0) return 0;
+   OCH_CHECK_HIP(hipMemcpyAsync(dst, src, nbytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+   OCH_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));
+   return 0;
+}
+int och_memcpy_dtoh(void *dst, const void *src, size_t nbytes, och_stream stream)
+{
+   if (nbytes == 0) return 0;
+   OCH_CHECK_HIP(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, (hipStream_t)stream));
+   OCH_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));
+   return 0;
+}
+int och_memset_async(void *dst, int value, size_t nbytes, och_stream stream)
+{  if (nbytes) OCH_CHECK_HIP(hipMemsetAsync(dst, value, nbytes, (hipStream_t)stream)); return 0; }
+
+} /* extern "C" */

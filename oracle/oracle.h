@@ -1,0 +1,76 @@
+/* TEST INFRASTRUCTURE -- CPU oracle for the MI355X device library.
+ *
+ * A restatement in plain C (+OpenMP) of the arithmetic and of the threading
+ * policy of Ocean's CPU path (Solid CPU kernels, solid/src/core/cpu/ and
+ * solid/include/solid/core/{cpu,generic}/). It exists to check the HIP
+ * kernels and to time a CPU baseline. Nothing in the product links, loads or
+ * calls it; only tests/, the smoke check and the benchmark's cpu_baseline leg
+ * may. Operation and type numbering are those of include/ocean_hip.h.
+ * All pointers are host pointers; strides are in bytes.
+ */
+#ifndef ORACLE_H
+#define ORACLE_H
+#include <stddef.h>
+#include <stdint.h>
+#include "../include/ocean_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* nthreads: number of OpenMP threads the CPU module would use for one- and
+   two-operand loops (<= 1: serial). Three-operand (binary) loops are always serial. */
+int oracle_max_threads(void);
+
+int oracle_binary(int op, int dtype, int ndims, const size_t *size,
+                  const ptrdiff_t *strides1, void *ptr1, const ptrdiff_t *strides2, void *ptr2,
+                  const ptrdiff_t *strides3, void *ptr3);
+int oracle_binary_supported(int op, int dtype);
+int oracle_unary(int op, int dtype, int ndims, const size_t *size,
+                 const ptrdiff_t *strides1, void *ptr1, const ptrdiff_t *strides2, void *ptr2, int nthreads);
+int oracle_unary_supported(int op, int dtype);
+
+int oracle_copy(int dtype_src, int dtype_dst,
+                int ndims1, const size_t *size1, const ptrdiff_t *strides1, void *ptr1,
+                int ndims2, const size_t *size2, const ptrdiff_t *strides2, void *ptr2, int nthreads);
+int oracle_byteswap_copy(int dtype_src, int dtype_dst,
+                int ndims1, const size_t *size1, const ptrdiff_t *strides1, void *ptr1,
+                int ndims2, const size_t *size2, const ptrdiff_t *strides2, void *ptr2, int nthreads);
+int oracle_byteswap(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr, int nthreads);
+
+int oracle_fill(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr,
+                och_scalar value, int nthreads);
+int oracle_fill_nan(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr,
+                och_scalar value, int nthreads);
+int oracle_masked_fill(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides1, void *ptr1,
+                const ptrdiff_t *strides2, void *ptr2, och_scalar value, int nthreads);
+int oracle_steps_int64(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr,
+                int64_t offset, int64_t step, int nthreads);
+int oracle_steps_double(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr,
+                double offset, double step, int nthreads);
+int oracle_steps_cdouble(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr,
+                och_cdouble offset, och_cdouble step, int nthreads);
+
+/* Full reductions with the CPU module's threading: per-thread partials over contiguous
+   index ranges (threads capped so each gets >= 512 elements), folded in thread order. */
+int oracle_reduce_all(int op, int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+                void *ptr, const och_scalar *param1, const och_scalar *param2, double p,
+                void *result, int nthreads);
+int oracle_reduce_supported(int op, int dtype);
+int oracle_reduce_result_dtype(int op, int dtype);
+/* Axis reduction; configuration as och_reduce_axis_config (stream ignored). Serial. */
+int oracle_reduce_axis(int op, int dtype, const och_reduce_axis_config *config, double p);
+
+/* Column-major GEMM, textbook triple loop; accumulation in the element type. */
+int oracle_gemm(int dtype, char transA, char transB, size_t M, size_t N, size_t K,
+                const void *alpha, const void *A, ptrdiff_t ldA, const void *B, ptrdiff_t ldB,
+                const void *beta, void *C, ptrdiff_t ldC, int nthreads);
+
+/* Software half precision (half.c) exposed for exhaustive tests */
+float    oracle_half_to_float(uint16_t h);
+uint16_t oracle_float_to_half(float f);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
