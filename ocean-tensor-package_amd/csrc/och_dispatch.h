@@ -33,6 +33,9 @@ template <template <class> class OP, int TS> struct Row3 { static const ew3_fn f
 template <template <class> class OP, int TS> const ew3_fn Row3<OP, TS>::fn[DT_COUNT] = { OCH_FOR_ALL_TYPES(OCH_X) };
 #undef OCH_X
 
+template <class F, bool OK> struct Pick2 { static constexpr ew2_fn fn = nullptr; };
+template <class F> struct Pick2<F, true> { static constexpr ew2_fn fn = &launch_ew2<F>; };
+
 static inline int dtype_ok(int dtype) { return dtype >= 0 && dtype < DT_COUNT; }
 
 } /* namespace och */
