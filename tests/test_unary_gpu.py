@@ -21,9 +21,9 @@ import ocean_hip as oh
 pytestmark = pytest.mark.gpu
 N = 2051
 
-EXACT = {"negative", "bitwise_not", "logical_not", "conj", "reciprocal", "square", "fabs", "sign", "ceil", "floor",
+EXACT = {"negative", "bitwise_not", "logical_not", "conj", "reciprocal", "square", "sign", "ceil", "floor",
          "trunc", "round", "isinf", "isnan", "isfinite", "isposinf", "isneginf"}
-EXACT_REAL_ONLY = {"sqrt", "absolute"}       # complex versions use hypot
+EXACT_REAL_ONLY = {"sqrt", "absolute", "fabs"}       # complex versions use hypot
 
 
 def input_data(name, dtype, rng):
@@ -37,7 +37,7 @@ def input_data(name, dtype, rng):
         return d
     if dtype == H.BOOL:
         return H.random_data(dtype, N, rng)
-    if name in EXACT or name in ("sqrt", "absolute"):
+    if name in EXACT or name in EXACT_REAL_ONLY:
         d = H.random_data(dtype, N, rng, "special")
         if name == "sqrt" and dtype in H.COMPLEX_TYPES:
             d = H.random_data(dtype, N, rng, "general")
@@ -94,6 +94,8 @@ def compare(name, dtype, rdtype, got, want):
         assert np.all(np.abs(g - w) <= 4e-3 * np.maximum(np.abs(w), 1e-2))
     else:
         tol = 2e-5 if rdtype == H.CFLOAT else 1e-12
+        if name == "cbrt":
+            tol = 2e-5          # the CPU table evaluates pow in single precision for every type
         assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-3)), "%s %s" % (name, H.NAMES[dtype])
 
 
