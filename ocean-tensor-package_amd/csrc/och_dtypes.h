@@ -103,7 +103,7 @@ OCH_HD half_t float_to_half(float f)
    half_t r;
    if (ex < 112u) { r.v = 0; return r; }
    if (ex > 143u)
-   {  if (ex == 255u && d != 0) r.v = 0x7E00;    /* quiet NaN, sign dropped */
+   {  if (ex == 255u && d != 0) r.v = 0x7F00;    /* quiet NaN pattern 0x7F00, sign dropped */
       else r.v = (uint16_t)(s | 0x7C00u);
       return r;
    }

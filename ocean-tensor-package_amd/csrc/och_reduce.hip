@@ -1,0 +1,95 @@
+/* C ABI of the full reductions (och_reduce_all and its queries) and the per-device
+ * scratch they use when the caller supplies none. */
+#include "och_reduce_all.h"
+#include <mutex>
+#include <string.h>
+
+namespace och {
+red_fn reduce_lookup_a(int op, int dtype);
+red_fn reduce_lookup_b(int op, int dtype);
+red_fn reduce_lookup_c(int op, int dtype);
+red_fn reduce_lookup_d(int op, int dtype);
+static_assert((int)R_COUNT == (int)OCH_REDUCE_COUNT && (int)R_NORM2_NAN == (int)OCH_R_NORM2_NAN && (int)R_SUM == (int)OCH_R_SUM,
+              "operation lists out of step");
+
+static red_fn reduce_lookup(int op, int dtype)
+{
+   if (dtype < 0 || dtype >= DT_COUNT || op < 0 || op >= OCH_REDUCE_COUNT) return nullptr;
+   if (op <= 7) return reduce_lookup_a(op, dtype);
+   if (op <= 14) return reduce_lookup_b(op, dtype);
+   if (op <= 20) return reduce_lookup_c(op, dtype);
+   return reduce_lookup_d(op, dtype);
+}
+
+#define OCH_MAX_DEVICES 64
+static RedContext g_ctx[OCH_MAX_DEVICES];
+static bool g_ctx_ready[OCH_MAX_DEVICES];
+static std::mutex g_ctx_mutex;
+
+int red_context(RedContext **out)
+{
+   int dev;
+   OCH_CHECK_HIP(hipGetDevice(&dev));
+   if (dev < 0 || dev >= OCH_MAX_DEVICES) return set_error("device index %d out of range", dev);
+   std::lock_guard<std::mutex> lock(g_ctx_mutex);
+   if (!g_ctx_ready[dev])
+   {  void *scratch = nullptr, *host = nullptr;
+      OCH_CHECK_HIP(hipMalloc(&scratch, OCH_RED_SCRATCH));
+      OCH_CHECK_HIP(hipMemset(scratch, 0, OCH_RED_SCRATCH));
+      OCH_CHECK_HIP(hipHostMalloc(&host, 64, hipHostMallocDefault));
+      g_ctx[dev].scratch = (char *)scratch; g_ctx[dev].host_result = host;
+      g_ctx_ready[dev] = true;
+   }
+   *out = &g_ctx[dev];
+   return 0;
+}
+}  /* namespace och */
+
+using namespace och;
+
+extern "C" size_t och_reduce_all_buffer_size(void) { return OCH_RED_SCRATCH; }
+extern "C" int och_reduce_supported(int op, int dtype) { return reduce_lookup(op, dtype) != nullptr; }
+
+extern "C" int och_reduce_result_dtype(int op, int dtype)
+{
+   if (!och_reduce_supported(op, dtype)) return -1;
+   const bool isbool = dtype == OCH_BOOL, isuint = dtype >= OCH_UINT8 && dtype <= OCH_UINT64;
+   const bool issint = dtype >= OCH_INT8 && dtype <= OCH_INT64, iscomplex = dtype >= OCH_CHALF;
+   const int abstype = iscomplex ? dtype - 3 : (issint ? dtype - 4 : dtype);
+   if (op <= OCH_R_ANY_NAN || (op >= OCH_R_ALL_LT && op <= OCH_R_ALL_GELE)) return OCH_BOOL;
+   if (op == OCH_R_NNZ || op == OCH_R_NNZ_NAN) return OCH_UINT64;
+   if (op >= OCH_R_SUM && op <= OCH_R_PROD_NAN) return (isbool || isuint) ? OCH_UINT64 : (issint ? OCH_INT64 : dtype);
+   if (op == OCH_R_SUM_ABS || op == OCH_R_SUM_ABS_NAN) return (isbool || isuint || issint) ? OCH_UINT64 : abstype;
+   if (op == OCH_R_MAXIMUM || op == OCH_R_MINIMUM) return dtype;
+   if (op == OCH_R_MAXIMUM_ABS || op == OCH_R_MINIMUM_ABS) return abstype;
+   return (isbool || isuint || issint) ? OCH_DOUBLE : abstype;      /* norms */
+}
+
+extern "C" int och_reduce_all_device(int op, int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+                   void *ptr, const och_scalar *param1, const och_scalar *param2, double p,
+                   void *dresult, void *buffer, och_stream stream)
+{
+   red_fn fn = reduce_lookup(op, dtype);
+   if (fn == nullptr) return set_error("reduction %d is not available for data type %d", op, dtype);
+   char *scratch = (char *)buffer;
+   if (scratch == nullptr)
+   {  RedContext *ctx;
+      if (red_context(&ctx) != 0) return -1;
+      scratch = ctx->scratch;
+   }
+   return fn(ndims, size, strides, ptr, param1, param2, p, dresult, scratch, buffer != nullptr, as_stream(stream));
+}
+
+extern "C" int och_reduce_all(int op, int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+                   void *ptr, const och_scalar *param1, const och_scalar *param2, double p,
+                   void *result, void *buffer, och_stream stream)
+{
+   RedContext *ctx;
+   if (red_context(&ctx) != 0) return -1;
+   /* the kernel writes the scalar straight into pinned host memory; one synchronisation */
+   if (och_reduce_all_device(op, dtype, ndims, size, strides, ptr, param1, param2, p, ctx->host_result, buffer, stream) != 0) return -1;
+   OCH_CHECK_HIP(hipStreamSynchronize(as_stream(stream)));
+   int rd = och_reduce_result_dtype(op, dtype);
+   memcpy(result, ctx->host_result, och_type_size[rd]);
+   return 0;
+}

@@ -1,0 +1,201 @@
+/* Single-launch full reduction for gfx950.
+ *
+ * Replaces the reference's accumulate + finalize kernel pair followed by a blocking copy
+ * (solid/include/solid/core/gpu/reduce_all.h:136-274,365-414). One kernel:
+ *   grid-stride loop with <=128-bit loads, four independent loads in flight per thread
+ *   -> 64-lane butterfly (shuffle) inside each wave -> LDS combine of the block's waves
+ *   -> one partial per block in a scratch buffer -> the block that takes the last ticket
+ *   (atomic counter) folds all partials in index order and writes the result.
+ * The fold order depends only on the launch geometry, so results are reproducible run to run.
+ * The result pointer may be device memory or device-visible pinned host memory.
+ */
+#pragma once
+#include "och_elemwise.h"
+#include "och_reduce_ops.h"
+#include <string.h>
+
+namespace och {
+
+#define OCH_RED_BLOCK 256
+#define OCH_RED_UNR 4
+#define OCH_RED_MAX_BLOCKS 2048
+#define OCH_RED_SLOT 16                               /* bytes per partial */
+#define OCH_RED_SCRATCH (OCH_RED_MAX_BLOCKS * OCH_RED_SLOT + 256)
+
+template <class A> OCH_D A shfl_xor_any(A v, int mask)
+{
+   constexpr int NW = (sizeof(A) + 3) / 4;
+   union { A a; int w[NW]; } u;
+   for (int i = 0; i < NW; i++) u.w[i] = 0;
+   u.a = v;
+#pragma unroll
+   for (int i = 0; i < NW; i++) u.w[i] = __shfl_xor(u.w[i], mask, 64);
+   return u.a;
+}
+
+/* read an accumulator that another workgroup wrote: word-wise volatile loads */
+template <class A> OCH_D A load_shared_global(const char *addr)
+{
+   constexpr int NW = (sizeof(A) + 3) / 4;
+   union { A a; unsigned int w[NW]; } u;
+#pragma unroll
+   for (int i = 0; i < NW; i++) u.w[i] = reinterpret_cast<const volatile unsigned int *>(addr)[i];
+   return u.a;
+}
+
+/* reduce across the 256 threads of a block; the result is valid in thread 0 */
+template <class RD> OCH_D typename RD::Acc block_reduce(typename RD::Acc a, typename RD::Acc *lds)
+{
+   typedef typename RD::Acc Acc;
+#pragma unroll
+   for (int m = 32; m >= 1; m >>= 1) a = RD::combine(a, shfl_xor_any<Acc>(a, m));
+   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+   if (lane == 0) lds[wave] = a;
+   __syncthreads();
+   if (threadIdx.x == 0)
+   {
+#pragma unroll
+      for (int w = 1; w < OCH_RED_BLOCK / 64; w++) a = RD::combine(a, lds[w]);
+   }
+   return a;
+}
+
+struct RedParams
+{
+   EwParams<1> ew;             /* source layout; ew.ngroups unused when flat */
+   uint64_t ngroups;           /* total groups (VEC elements each) */
+   char *partials;             /* OCH_RED_MAX_BLOCKS slots */
+   unsigned int *counter;      /* ticket counter, zero on entry, zero again on exit */
+   void *result;
+   char *tail;                 /* flat layout only: elements left over after the last full group */
+   int   ntail;
+};
+
+template <class RD, class T, int VEC>
+__global__ __launch_bounds__(OCH_RED_BLOCK) void reduce_all_kernel(const RedParams p, const typename RD::Param prm)
+{
+   typedef typename RD::Acc Acc;
+   __shared__ Acc lds[OCH_RED_BLOCK / 64];
+   __shared__ unsigned int ticket;
+   Acc acc = RD::identity();
+   const uint64_t stride = (uint64_t)gridDim.x * OCH_RED_BLOCK;
+   uint64_t g = (uint64_t)blockIdx.x * OCH_RED_BLOCK + threadIdx.x;
+   const bool flat = (p.ew.ndims == 1);
+   /* main loop: OCH_RED_UNR groups per trip, loads first */
+   for (; g + (OCH_RED_UNR - 1) * stride < p.ngroups; g += OCH_RED_UNR * stride)
+   {  Pack<T, VEC> v[OCH_RED_UNR];
+#pragma unroll
+      for (int u = 0; u < OCH_RED_UNR; u++)
+      {  int64_t off[1];
+         if (flat) off[0] = (int64_t)(g + u * stride) * p.ew.gstride[0];
+         else group_offsets<1>(p.ew, (uint32_t)(g + u * stride), off);
+         load_pack<T, VEC>(v[u], p.ew.ptr[0] + off[0], p.ew.estride[0], p.ew.vecmode[0]);
+      }
+#pragma unroll
+      for (int u = 0; u < OCH_RED_UNR; u++)
+#pragma unroll
+         for (int k = 0; k < VEC; k++) acc = RD::combine(acc, RD::load(v[u].v[k], prm));
+   }
+   for (; g < p.ngroups; g += stride)
+   {  Pack<T, VEC> v; int64_t off[1];
+      if (flat) off[0] = (int64_t)g * p.ew.gstride[0];
+      else group_offsets<1>(p.ew, (uint32_t)g, off);
+      load_pack<T, VEC>(v, p.ew.ptr[0] + off[0], p.ew.estride[0], p.ew.vecmode[0]);
+#pragma unroll
+      for (int k = 0; k < VEC; k++) acc = RD::combine(acc, RD::load(v.v[k], prm));
+   }
+   if (blockIdx.x == 0 && (int)threadIdx.x < p.ntail)
+      acc = RD::combine(acc, RD::load(*reinterpret_cast<const T *>(p.tail + (int64_t)threadIdx.x * p.ew.estride[0]), prm));
+   acc = block_reduce<RD>(acc, lds);
+   if (threadIdx.x == 0)
+   {  *reinterpret_cast<Acc *>(p.partials + (size_t)blockIdx.x * OCH_RED_SLOT) = acc;
+      __threadfence();
+      ticket = atomicAdd(p.counter, 1u);
+   }
+   __syncthreads();
+   if (ticket != gridDim.x - 1) return;
+   /* last block: fold the partials in index order */
+   __threadfence();
+   acc = RD::identity();
+   for (unsigned int b = threadIdx.x; b < gridDim.x; b += OCH_RED_BLOCK)
+      acc = RD::combine(acc, load_shared_global<Acc>(p.partials + (size_t)b * OCH_RED_SLOT));
+   __syncthreads();
+   acc = block_reduce<RD>(acc, lds);
+   if (threadIdx.x == 0)
+   {  *reinterpret_cast<typename RD::Res *>(p.result) = RD::finalize(acc, prm);
+      *p.counter = 0;
+   }
+}
+
+/* per-device scratch and pinned result slot used when the caller passes no buffer */
+struct RedContext { char *scratch; void *host_result; };
+int red_context(RedContext **ctx);
+
+typedef int (*red_fn)(int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr,
+                      const och_scalar *b1, const och_scalar *b2, double pnorm,
+                      void *dresult, char *scratch, bool zero_counter, hipStream_t stream);
+
+template <class T, int OP>
+static int launch_reduce_all(int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr,
+                             const och_scalar *b1, const och_scalar *b2, double pnorm,
+                             void *dresult, char *scratch, bool zero_counter, hipStream_t stream)
+{
+   typedef Reduce<T, OP> RD;
+   static_assert(sizeof(typename RD::Acc) <= OCH_RED_SLOT, "accumulator does not fit a partial slot");
+   typename RD::Param prm;
+   memset(&prm, 0, sizeof(prm));
+   if (b1) memcpy(&prm.bound1, b1, sizeof(T));
+   if (b2) memcpy(&prm.bound2, b2, sizeof(T));
+   prm.phalf = pnorm / 2; prm.pinv = (pnorm != 0) ? 1.0 / pnorm : 0.0;
+
+   const ptrdiff_t *st[1] = { strides }; void *pp[1] = { ptr };
+   EwShape<1> shape;
+   if (ew_normalize<1>(shape, ndims, size, st, pp, 0, true) != 0) return -1;
+   if (shape.nelem == 0 && RD::NEEDS_DATA) return set_error("reduction of an empty tensor is undefined for this operation");
+   if (shape.ndims > 1 && shape.nelem > 0xFFFF0000ull) return set_error("strided reduction of more than 2^32 elements is not supported");
+
+   RedParams p;
+   memset(&p, 0, sizeof(p));
+   constexpr int VEC = vec_for<T>();
+   const int es[1] = { (int)sizeof(T) };
+   int vec = 1;
+   if (shape.nelem > 0)
+   {  EwShape<1> s32 = shape;                     /* ew_params works on 32-bit group counts: fill by hand when flat */
+      if (shape.ndims == 1)
+      {  uint64_t n = shape.size[0];
+         bool wide = (VEC > 1) && (n >= (uint64_t)VEC) && (shape.stride[0][0] == (int64_t)sizeof(T)) &&
+                     (((uintptr_t)shape.ptr[0]) % (sizeof(T) * VEC > 16 ? 16 : sizeof(T) * VEC) == 0);
+         vec = wide ? VEC : 1;
+         p.ntail = (int)(n % vec);
+         p.tail = shape.ptr[0] + (int64_t)(n - n % vec) * shape.stride[0][0];
+         p.ew.ndims = 1; p.ew.ptr[0] = shape.ptr[0];
+         p.ew.estride[0] = shape.stride[0][0]; p.ew.gstride[0] = shape.stride[0][0] * vec;
+         p.ew.vecmode[0] = wide ? 1 : ((shape.stride[0][0] == (int64_t)sizeof(T)) && (((uintptr_t)shape.ptr[0]) % alignof(Pack<T, 1>) == 0));
+         p.ngroups = n / vec;
+      }
+      else
+      {  vec = (VEC > 1 && ew_params<1>(p.ew, s32, VEC, es, 0)) ? VEC : 1;
+         if (vec == 1) ew_params<1>(p.ew, s32, 1, es, 0);
+         p.ngroups = p.ew.ngroups;
+      }
+   }
+   p.partials = scratch;
+   p.counter = reinterpret_cast<unsigned int *>(scratch + OCH_RED_MAX_BLOCKS * OCH_RED_SLOT);
+   p.result = dresult;
+   if (zero_counter) OCH_CHECK_HIP(hipMemsetAsync(p.counter, 0, sizeof(unsigned int), stream));
+   uint64_t want = (p.ngroups + (uint64_t)OCH_RED_BLOCK * OCH_RED_UNR - 1) / ((uint64_t)OCH_RED_BLOCK * OCH_RED_UNR);
+   unsigned int blocks = (unsigned int)(want < 1 ? 1 : (want > OCH_RED_MAX_BLOCKS ? OCH_RED_MAX_BLOCKS : want));
+   if (vec > 1) hipLaunchKernelGGL((reduce_all_kernel<RD, T, VEC>), dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
+   else         hipLaunchKernelGGL((reduce_all_kernel<RD, T, 1>),   dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
+   OCH_CHECK_LAUNCH();
+   return 0;
+}
+
+template <class T, int OP, bool OK> struct PickR { static constexpr red_fn fn = nullptr; };
+template <class T, int OP> struct PickR<T, OP, true> { static constexpr red_fn fn = &launch_reduce_all<T, OP>; };
+template <int OP> struct RowR { static const red_fn fn[DT_COUNT]; };
+#define OCH_X(T) PickR<T, OP, reduce_defined<T, OP>()>::fn,
+template <int OP> const red_fn RowR<OP>::fn[DT_COUNT] = { OCH_FOR_ALL_TYPES(OCH_X) };
+#undef OCH_X
+
+} /* namespace och */

@@ -54,24 +54,33 @@ class CDouble(C.Structure):
     _fields_ = [("real", C.c_double), ("imag", C.c_double)]
 
 
-class Scalar(C.Union):
+class ScalarUnion(C.Union):
     _fields_ = [("_bool", C.c_uint8), ("_uint8", C.c_uint8), ("_uint16", C.c_uint16), ("_uint32", C.c_uint32),
                 ("_uint64", C.c_uint64), ("_int8", C.c_int8), ("_int16", C.c_int16), ("_int32", C.c_int32),
                 ("_int64", C.c_int64), ("_half", C.c_uint16), ("_float", C.c_float), ("_double", C.c_double),
                 ("_chalf", CHalf), ("_cfloat", CFloat), ("_cdouble", CDouble)]
 
 
+class Scalar(C.Structure):
+    """och_scalar as ctypes can pass it BY VALUE. libffi lays a ctypes Union out like a struct of all
+    members, which breaks the x86-64 calling convention; the C union's two eightbytes classify as
+    INTEGER and SSE, exactly like this two-field structure of the same 16 bytes."""
+    _fields_ = [("lo", C.c_uint64), ("hi", C.c_double)]
+
+
 def make_scalar(dtype, value):
-    """Scalar union holding `value` as element type `dtype` (half types take bit patterns)."""
-    s = Scalar()
-    C.memset(C.byref(s), 0, C.sizeof(s))
+    """Scalar holding `value` as element type `dtype` (half types take bit patterns)."""
+    u = ScalarUnion()
+    C.memset(C.byref(u), 0, C.sizeof(u))
     name = "_" + DTYPE_NAMES[dtype]
     if dtype in (CHALF, CFLOAT, CDOUBLE):
         re, im = (value if isinstance(value, tuple) else (value.real, value.imag))
-        f = getattr(s, name)
+        f = getattr(u, name)
         f.real, f.imag = re, im
     else:
-        setattr(s, name, value)
+        setattr(u, name, value)
+    s = Scalar()
+    C.memmove(C.byref(s), C.byref(u), C.sizeof(s))
     return s
 
 

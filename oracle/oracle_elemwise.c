@@ -23,202 +23,9 @@ float    oracle_half_to_float(uint16_t h) { return o_half_to_float(h); }
 uint16_t oracle_float_to_half(float f)    { return o_float_to_half(f); }
 
 /* ---- instantiate the per-type operation loops ----------------------------- */
-
-#define K_BOOL 1
-#define K_UINT 0
-#define K_SINT 0
-#define K_FLOAT 0
-#define K_COMPLEX 0
-#define TN bool
-#define T o_bool
-#define PN bool
-#define WN bool
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef PN
-#undef WN
-#undef K_BOOL
-#define K_BOOL 0
-
-#undef K_UINT
-#define K_UINT 1
-#define TN uint8
-#define T uint8_t
-#define UT uint8_t
-#define PN uint8
-#define WN uint8
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef UT
-#undef PN
-#undef WN
-#define TN uint16
-#define T uint16_t
-#define UT uint16_t
-#define PN uint16
-#define WN uint16
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef UT
-#undef PN
-#undef WN
-#define TN uint32
-#define T uint32_t
-#define UT uint32_t
-#define PN uint32
-#define WN uint32
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef UT
-#undef PN
-#undef WN
-#define TN uint64
-#define T uint64_t
-#define UT uint64_t
-#define PN uint64
-#define WN uint64
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef UT
-#undef PN
-#undef WN
-#undef K_UINT
-#define K_UINT 0
-
-#undef K_SINT
-#define K_SINT 1
-#define TN int8
-#define T int8_t
-#define UT uint8_t
-#define PN int8
-#define WN int8
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef UT
-#undef PN
-#undef WN
-#define TN int16
-#define T int16_t
-#define UT uint16_t
-#define PN int16
-#define WN int16
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef UT
-#undef PN
-#undef WN
-#define TN int32
-#define T int32_t
-#define UT uint32_t
-#define PN int32
-#define WN int32
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef UT
-#undef PN
-#undef WN
-#define TN int64
-#define T int64_t
-#define UT uint64_t
-#define PN int64
-#define WN int64
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef UT
-#undef PN
-#undef WN
-#undef K_SINT
-#define K_SINT 0
-
-#undef K_FLOAT
-#define K_FLOAT 1
-#define TN half
-#define T o_half
-#define PN half
-#define WN float
-#define W float
-#define MF(fn) fn##f
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef PN
-#define TN float
-#define T float
-#define PN float
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef PN
-#undef WN
-#undef W
-#undef MF
-#define TN double
-#define T double
-#define PN double
-#define WN double
-#define W double
-#define MF(fn) fn
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef PN
-#undef WN
-#undef W
-#undef MF
-#undef K_FLOAT
-#define K_FLOAT 0
-
-#undef K_COMPLEX
-#define K_COMPLEX 1
-#define TN chalf
-#define T o_chalf
-#define PN half
-#define WN float
-#define W float
-#define MF(fn) fn##f
-#define HALF_OR_INF ((o_half)0xFC00)     /* the CPU table's half-precision infinity constant */
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef PN
-#undef HALF_OR_INF
-#define TN cfloat
-#define T o_cfloat
-#define PN float
-#define HALF_OR_INF ((float)(1. / 0.))
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef PN
-#undef WN
-#undef W
-#undef MF
-#undef HALF_OR_INF
-#define TN cdouble
-#define T o_cdouble
-#define PN double
-#define WN double
-#define W double
-#define MF(fn) fn
-#define HALF_OR_INF ((double)(1. / 0.))
-#include "oracle_ops_tmpl.h"
-#undef TN
-#undef T
-#undef PN
-#undef WN
-#undef W
-#undef MF
-#undef HALF_OR_INF
-#undef K_COMPLEX
+#define O_TMPL_FILE "oracle_ops_tmpl.h"
+#include "oracle_foreach_type.h"
+#undef O_TMPL_FILE
 
 /* ---- tables ------------------------------------------------------------------ */
 typedef int (*o_bin_fn)(int, const size_t *, const ptrdiff_t *, void *, const ptrdiff_t *, void *, const ptrdiff_t *, void *);

@@ -64,7 +64,7 @@ static inline o_half o_float_to_half(float f)
    e = (uint16_t)((e & 0x7FFF) >> 7);
    if (e < 127 - 15) return 0;                       /* zero and underflow */
    if (e > 127 + 16)
-   {  if (e == 255 && mant != 0) return 0x7E00;      /* NaN */
+   {  if (e == 255 && mant != 0) return 0x7F00;      /* NaN (the quiet-NaN pattern of half.h:26) */
       return (o_half)(sign | 0x7C00);                /* infinity and overflow */
    }
    e = (uint16_t)(e - (127 - 15));

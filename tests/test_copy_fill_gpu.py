@@ -1,0 +1,199 @@
+"""Parity of copy / cast / byteswap / fill / steps kernels with the CPU oracle (bit-exact).
+
+Reference tests of the same kind: examples/python/gpu/tensors/tensor_copy_01..09.py (zero
+stride broadcast copies, byteswapped sources, cross-dtype), tensor_dtype_cast_01.py,
+ocean_cast_01.py, tensor_fill_01.py, tensor_fillnan_01.py, ocean_linspace_03.py.
+Float -> integer conversions use in-range values only (out-of-range is undefined in the
+reference, dtype_assign.h:109).
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import helpers as H
+import ocean_hip as oh
+
+pytestmark = pytest.mark.gpu
+orc = H.orc
+
+
+def source_values(ts, td, n, rng):
+    x = H.random_data(ts, n, rng, "full" if ts in H.INT_TYPES and oh.TYPE_SIZE[ts] <= 2 else "general")
+    if ts in H.FLOAT_TYPES + H.COMPLEX_TYPES and td in H.INT_TYPES:
+        hi = min(120, int(np.iinfo(H.storage(td)).max))
+        lo = -hi if np.iinfo(H.storage(td)).min < 0 else 0
+        v = rng.uniform(lo, hi, n)
+        if ts == H.HALF:
+            x = H.f32_to_half_bits(v.astype(np.float32))
+        elif ts == H.CHALF:
+            x["real"] = H.f32_to_half_bits(v.astype(np.float32))
+        elif ts in H.COMPLEX_TYPES:
+            x = np.empty(n, H.storage(ts)); x.real, x.imag = v, rng.uniform(-5, 5, n)
+        else:
+            x = v.astype(H.storage(ts))
+    elif ts in H.FLOAT_TYPES + H.COMPLEX_TYPES:
+        x = H.random_data(ts, n, rng, "special")
+    return x
+
+
+PAIRS = [(s, d) for s in H.ALL_TYPES for d in H.ALL_TYPES]
+
+
+@pytest.mark.parametrize("ts,td", PAIRS, ids=["%s-%s" % (H.NAMES[s], H.NAMES[d]) for s, d in PAIRS])
+def test_cast_copy_all_pairs(hip, stream, ts, td):
+    """och_copy and och_byteswap_copy for all 15 x 15 type pairs, contiguous and step-2 source."""
+    rng = np.random.default_rng(300 + ts * 15 + td)
+    n = 1030
+    for swap in (0, 1):
+        for step in (1, 2):
+            xd = source_values(ts, td, n * step, rng)
+            if swap:
+                assert orc.lib.oracle_byteswap(ts, 1, oh.sizes([n * step]), oh.strides([oh.TYPE_SIZE[ts]]), orc.ptr(xd), 1) == 0
+            x = H.Operand(xd, xd[::step], ts).upload(stream)
+            y = H.Operand.contiguous(np.zeros(n, H.storage(td)), td).upload(stream)
+            gfn = oh.lib.och_byteswap_copy if swap else oh.lib.och_copy
+            cfn = orc.lib.oracle_byteswap_copy if swap else orc.lib.oracle_copy
+            oh.check(gfn(ts, td, 1, oh.sizes([n]), oh.strides(x.strides), x.dptr(), 1, oh.sizes([n]), oh.strides(y.strides), y.dptr(), stream.handle))
+            want = y.parent.copy()
+            assert cfn(ts, td, 1, oh.sizes([n]), oh.strides(x.strides), x.hptr(), 1, oh.sizes([n]), oh.strides(y.strides), y.hptr(want), 2) == 0
+            got = y.download()
+            x.free(); y.free()
+            H.assert_same_bytes(got, want, "%s -> %s swap=%d step=%d" % (H.NAMES[ts], H.NAMES[td], swap, step))
+
+
+@pytest.mark.parametrize("ts,td", [(H.FLOAT, H.FLOAT), (H.INT16, H.FLOAT), (H.CFLOAT, H.CDOUBLE), (H.DOUBLE, H.INT32), (H.UINT8, H.BOOL)],
+                         ids=lambda v: H.NAMES[v] if isinstance(v, int) else None)
+def test_reshape_and_strided_copy(hip, stream, ts, td):
+    """Different shapes with equal element count (reshape copy), transposed and broadcast sources."""
+    rng = np.random.default_rng(17 + ts)
+    # reshape: source 12 x 10 view (step 2 rows) -> destination 8 x 15, both column-major walks
+    src_parent = source_values(ts, td, 24 * 10, rng).reshape(10, 24)       # numpy (10,24): fastest index last
+    sv = src_parent.T[::2, :]                                              # shape (12,10), strides (2*es, 24*es)
+    dst_parent = np.zeros((15, 8), H.storage(td))
+    dv = dst_parent.T                                                      # shape (8,15) column-major
+    x = H.Operand(src_parent, sv, ts).upload(stream)
+    y = H.Operand(dst_parent, dv, td).upload(stream)
+    oh.check(oh.lib.och_copy(ts, td, 2, oh.sizes(x.shape), oh.strides(x.strides), x.dptr(), 2, oh.sizes(y.shape), oh.strides(y.strides), y.dptr(), stream.handle))
+    want = dst_parent.copy()
+    assert orc.lib.oracle_copy(ts, td, 2, oh.sizes(x.shape), oh.strides(x.strides), x.hptr(), 2, oh.sizes(y.shape), oh.strides(y.strides), y.hptr(want), 1) == 0
+    H.assert_same_bytes(y.download(), want, "reshape copy")
+    x.free(); y.free()
+    # broadcast source (zero stride) into a transposed destination
+    row = source_values(ts, td, 33, rng).reshape(1, 33)
+    bv = np.broadcast_to(row, (21, 33))
+    dst_parent = np.zeros((33, 21), H.storage(td))
+    x = H.Operand(row, bv, ts).upload(stream)
+    y = H.Operand(dst_parent, dst_parent.T, td).upload(stream)
+    oh.check(oh.lib.och_copy(ts, td, 2, oh.sizes(x.shape), oh.strides(x.strides), x.dptr(), 2, oh.sizes(y.shape), oh.strides(y.strides), y.dptr(), stream.handle))
+    want = dst_parent.copy()
+    assert orc.lib.oracle_copy(ts, td, 2, oh.sizes(x.shape), oh.strides(x.strides), x.hptr(), 2, oh.sizes(y.shape), oh.strides(y.strides), y.hptr(want), 1) == 0
+    H.assert_same_bytes(y.download(), want, "broadcast copy")
+    x.free(); y.free()
+
+
+@pytest.mark.parametrize("dtype", H.ALL_TYPES, ids=[H.NAMES[d] for d in H.ALL_TYPES])
+def test_byteswap_in_place(hip, stream, dtype):
+    rng = np.random.default_rng(5 + dtype)
+    parent = H.random_data(dtype, 40 * 23, rng).reshape(23, 40)
+    x = H.Operand(parent, parent[::2, 1::3], dtype).upload(stream)
+    oh.check(oh.lib.och_byteswap(dtype, 2, oh.sizes(x.shape), oh.strides(x.strides), x.dptr(), stream.handle))
+    want = parent.copy()
+    assert orc.lib.oracle_byteswap(dtype, 2, oh.sizes(x.shape), oh.strides(x.strides), x.hptr(want), 1) == 0
+    got = x.download()
+    H.assert_same_bytes(got.view(np.uint8), want.view(np.uint8), "byteswap %s" % H.NAMES[dtype])
+    # swapping twice restores the original bytes
+    oh.check(oh.lib.och_byteswap(dtype, 2, oh.sizes(x.shape), oh.strides(x.strides), x.dptr(), stream.handle))
+    H.assert_same_bytes(x.download().view(np.uint8), parent.view(np.uint8), "double byteswap")
+    x.free()
+
+
+def scalar_for(dtype, rng):
+    v = H.random_data(dtype, 1, rng, "general")
+    s = oh.Scalar()
+    C.memset(C.byref(s), 0, C.sizeof(s))
+    C.memmove(C.byref(s), v.ctypes.data, v.dtype.itemsize)
+    return s
+
+
+@pytest.mark.parametrize("dtype", H.ALL_TYPES, ids=[H.NAMES[d] for d in H.ALL_TYPES])
+def test_fill_family(hip, stream, dtype):
+    rng = np.random.default_rng(60 + dtype)
+    value = scalar_for(dtype, rng)
+    parent = H.random_data(dtype, 50 * 31, rng, "special" if dtype >= H.HALF else "general").reshape(31, 50)
+    view = parent[1::2, ::3]
+    mask_parent = rng.integers(0, 2, size=(50, 31)).astype(np.uint8)
+    mview = mask_parent.T[1::2, ::3]
+    for what in ("fill", "fill_nan", "masked_fill"):
+        if what == "fill_nan" and dtype < H.HALF:
+            assert oh.lib.och_fill_nan(dtype, 1, oh.sizes([1]), oh.strides([1]), None, value, stream.handle) == -1
+            continue
+        x = H.Operand(parent, view, dtype).upload(stream)
+        want = parent.copy()
+        if what == "masked_fill":
+            m = H.Operand(mask_parent, mview, H.BOOL).upload(stream)
+            oh.check(oh.lib.och_masked_fill(dtype, 2, oh.sizes(x.shape), oh.strides(x.strides), x.dptr(), oh.strides(m.strides), m.dptr(), value, stream.handle))
+            assert orc.lib.oracle_masked_fill(dtype, 2, oh.sizes(x.shape), oh.strides(x.strides), x.hptr(want), oh.strides(m.strides), m.hptr(), value, 2) == 0
+            m.free()
+        else:
+            gfn = getattr(oh.lib, "och_" + what); cfn = getattr(orc.lib, "oracle_" + what)
+            oh.check(gfn(dtype, 2, oh.sizes(x.shape), oh.strides(x.strides), x.dptr(), value, stream.handle))
+            assert cfn(dtype, 2, oh.sizes(x.shape), oh.strides(x.strides), x.hptr(want), value, 2) == 0
+        got = x.download()
+        x.free()
+        H.assert_same_bytes(got.view(np.uint8), want.view(np.uint8), "%s %s" % (what, H.NAMES[dtype]))
+
+
+@pytest.mark.parametrize("dtype", H.ALL_TYPES, ids=[H.NAMES[d] for d in H.ALL_TYPES])
+def test_steps(hip, stream, dtype):
+    """arange / linspace building blocks: value = offset + index * step with the flat index taken in
+    the caller's dimension order."""
+    n0, n1 = 37, 9
+    parent = np.zeros((n1, 2 * n0), H.storage(dtype))
+    view = parent[:, ::2].T                                               # shape (n0, n1), dim 0 strided
+    cases = [("int64", (3, 2)), ("double", (0.25, 0.5)), ("cdouble", (oh.CDouble(1.0, -2.0), oh.CDouble(0.5, 0.25)))]
+    if dtype in (H.BOOL, H.UINT8, H.INT8):
+        cases[0] = ("int64", (0, 1) if dtype != H.BOOL else (0, 0))
+        cases[1] = ("double", (0.0, 0.25))
+        cases[2] = ("cdouble", (oh.CDouble(0.0, 0.0), oh.CDouble(0.25, 0.125)))
+    for kind, (a, b) in cases:
+        x = H.Operand(parent, view, dtype).upload(stream)
+        want = parent.copy()
+        gfn = getattr(oh.lib, "och_steps_" + kind); cfn = getattr(orc.lib, "oracle_steps_" + kind)
+        oh.check(gfn(dtype, 2, oh.sizes(x.shape), oh.strides(x.strides), x.dptr(), a, b, stream.handle))
+        assert cfn(dtype, 2, oh.sizes(x.shape), oh.strides(x.strides), x.hptr(want), a, b, 2) == 0
+        got = x.download()
+        x.free()
+        H.assert_same_bytes(got.view(np.uint8), want.view(np.uint8), "steps_%s %s" % (kind, H.NAMES[dtype]))
+
+
+def test_config4_cast_byteswap(hip, stream):
+    """BASELINE config 4 at reduced size plus the full-size round-trip property:
+    int16 3-D tensor (full int16 range, stored byteswapped, step-2 slice) -> contiguous float32, and
+    complex64 -> complex128."""
+    rng = np.random.default_rng(4)
+    d0, d1, d2 = 256, 64, 16
+    parent = rng.integers(-32768, 32767, size=(d2, d1, 2 * d0), dtype=np.int16, endpoint=True)
+    swapped = parent.byteswap()                       # bytes as a big-endian producer would have written them
+    view = swapped.transpose(2, 1, 0)[::2]            # Ocean order: dim 0 fastest, step 2 along it
+    assert view.shape == (d0, d1, d2)
+    x = H.Operand(swapped, view, H.INT16).upload(stream)
+    out = np.zeros((d2, d1, d0), np.float32)
+    y = H.Operand(out, out.transpose(2, 1, 0), H.FLOAT).upload(stream)
+    oh.check(oh.lib.och_byteswap_copy(H.INT16, H.FLOAT, 3, oh.sizes(x.shape), oh.strides(x.strides), x.dptr(),
+                                      3, oh.sizes(y.shape), oh.strides(y.strides), y.dptr(), stream.handle))
+    want = out.copy()
+    assert orc.lib.oracle_byteswap_copy(H.INT16, H.FLOAT, 3, oh.sizes(x.shape), oh.strides(x.strides), x.hptr(),
+                                        3, oh.sizes(y.shape), oh.strides(y.strides), y.hptr(want), 4) == 0
+    got = y.download()
+    x.free(); y.free()
+    H.assert_same_bytes(got, want, "config 4a")
+    H.assert_same_bytes(got, parent[:, :, ::2].astype(np.float32), "config 4a vs numpy")     # closed form: exact conversion
+    n = 1 << 20
+    z = (rng.uniform(-1, 1, n) + 1j * rng.uniform(-1, 1, n)).astype(np.complex64)
+    x = H.Operand.contiguous(z, H.CFLOAT).upload(stream)
+    y = H.Operand.contiguous(np.zeros(n, np.complex128), H.CDOUBLE).upload(stream)
+    oh.check(oh.lib.och_copy(H.CFLOAT, H.CDOUBLE, 1, oh.sizes([n]), oh.strides([8]), x.dptr(), 1, oh.sizes([n]), oh.strides([16]), y.dptr(), stream.handle))
+    got = y.download()
+    x.free(); y.free()
+    H.assert_same_bytes(got, z.astype(np.complex128), "config 4b")

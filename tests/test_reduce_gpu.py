@@ -1,0 +1,203 @@
+"""Parity of the full reductions (och_reduce_all) with the CPU oracle and with exact arithmetic.
+
+Reference tests of the same kind: examples/python/gpu/tensors/ocean_sum_01/02.py, ocean_sumabs_01.py,
+ocean_maximumabs_01/02.py, ocean_min_01.py, ocean_all_01.py (CPU and GPU printed side by side),
+examples/python/cpu/tensors/ocean_norm_01/02.py, axis_sum_01.py (NaN variants).
+
+Exact (bit-for-bit against the oracle): any/all/all_finite/any_inf/any_nan, nnz, the range checks,
+integer and bool sums / products / extrema / abs-extrema, float maximum / minimum (NaNs ignored).
+Tolerance: floating sums, products and norms. The GPU accumulates in double as a tree; Ocean's CPU
+path folds serially in the input precision per thread, so its own result moves with the thread
+count. The GPU result is therefore gated against an exact (math.fsum / float64) evaluation of the
+same inputs: relative 1e-5 for half/float inputs, 1e-12 for double, measured against sum|x| for
+sums (the sum itself can cancel) and against the value for norms and products; the distance to the
+literal CPU fold is reported with looser bounds.
+"""
+import ctypes as C
+import math
+
+import numpy as np
+import pytest
+
+import helpers as H
+import ocean_hip as oh
+
+pytestmark = pytest.mark.gpu
+orc = H.orc
+
+EXACT_OPS = {"any", "all", "all_finite", "any_inf", "any_nan", "nnz", "nnz_nan", "all_lt", "all_le", "all_gt", "all_ge",
+             "all_gtlt", "all_gtle", "all_gelt", "all_gele", "maximum", "minimum"}
+
+
+def to_float64(dtype, a):
+    """Values of a storage array as float64 / complex128."""
+    if dtype == H.HALF:
+        return np.array([orc.lib.oracle_half_to_float(int(b)) for b in a.reshape(-1)], np.float64).reshape(a.shape)
+    if dtype == H.CHALF:
+        out = np.empty(a.shape, np.complex128)
+        out.real, out.imag = to_float64(H.HALF, a["real"]), to_float64(H.HALF, a["imag"])
+        return out
+    if dtype == H.BOOL:
+        return a.astype(np.float64)
+    return a.astype(np.complex128 if dtype >= H.CFLOAT else np.float64)
+
+
+def gpu_reduce(stream, op, dtype, x, b1=None, b2=None, p=0.0):
+    rd = oh.lib.och_reduce_result_dtype(op, dtype)
+    out = np.zeros(1, H.storage(rd))
+    oh.check(oh.lib.och_reduce_all(op, dtype, len(x.shape), oh.sizes(x.shape), oh.strides(x.strides), x.dptr(),
+                                   b1, b2, p, orc.ptr(out), None, stream.handle))
+    return rd, out
+
+
+def cpu_reduce(op, dtype, x, b1=None, b2=None, p=0.0, nthreads=1):
+    rd = orc.lib.oracle_reduce_result_dtype(op, dtype)
+    out = np.zeros(1, H.storage(rd))
+    assert orc.lib.oracle_reduce_all(op, dtype, len(x.shape), oh.sizes(x.shape), oh.strides(x.strides), x.hptr(),
+                                     b1, b2, p, orc.ptr(out), nthreads) == 0
+    return rd, out
+
+
+def check_against_truth(name, dtype, rd, got, xd):
+    """Tolerance checks for floating sums / products / norms against float64 evaluation."""
+    v = to_float64(dtype, xd).reshape(-1)
+    g = to_float64(rd, got)[0]
+    tol = 1e-12 if dtype in (H.DOUBLE, H.CDOUBLE) else (2e-3 if dtype in (H.HALF, H.CHALF) else 1e-5)
+    skipnan = name.endswith("_nan")
+    if skipnan:
+        bad = np.isnan(v.real) | np.isnan(v.imag) if np.iscomplexobj(v) else np.isnan(v)
+        v = v[~bad]
+    if name in ("sum", "sum_nan"):
+        if np.iscomplexobj(v):
+            ref = complex(math.fsum(v.real), math.fsum(v.imag)); scale = math.fsum(np.abs(v.real)) + math.fsum(np.abs(v.imag))
+        else:
+            ref = math.fsum(v); scale = math.fsum(np.abs(v))
+        assert abs(g - ref) <= tol * max(scale, 1e-30), (name, g, ref)
+    elif name in ("sum_abs", "sum_abs_nan"):
+        ref = math.fsum(np.abs(v)); assert abs(g - ref) <= tol * ref
+    elif name in ("prod", "prod_nan"):
+        ref = np.prod(v.astype(np.complex128 if np.iscomplexobj(v) else np.longdouble))
+        assert abs(g - complex(ref) if np.iscomplexobj(v) else g - float(ref)) <= 20 * tol * abs(complex(ref))
+    elif name in ("norm2", "norm2_nan"):
+        ref = math.sqrt(math.fsum(np.abs(v) ** 2)); assert abs(g - ref) <= tol * ref
+    elif name in ("norm", "norm_nan"):
+        ref = math.fsum(np.abs(v) ** 3.0) ** (1 / 3.0); assert abs(g - ref) <= max(tol, 1e-6) * ref
+    elif name in ("maximum_abs", "minimum_abs"):
+        a = np.abs(v); a = a[~np.isnan(a)]
+        ref = a.max() if name == "maximum_abs" else a.min()
+        assert abs(g - ref) <= tol * max(ref, 1e-30)
+    else:
+        raise AssertionError("unhandled " + name)
+
+
+PAIRS = [(op, dt) for op in range(len(oh.REDUCE_OPS)) for dt in H.ALL_TYPES]
+
+
+@pytest.mark.parametrize("op,dtype", PAIRS, ids=["%s-%s" % (oh.REDUCE_OPS[o], H.NAMES[d]) for o, d in PAIRS])
+def test_reduce_all(hip, stream, op, dtype):
+    name = oh.REDUCE_OPS[op]
+    sup = bool(oh.lib.och_reduce_supported(op, dtype))
+    assert sup == bool(orc.lib.oracle_reduce_supported(op, dtype))
+    if not sup:
+        return
+    assert oh.lib.och_reduce_result_dtype(op, dtype) == orc.lib.oracle_reduce_result_dtype(op, dtype)
+    rng = np.random.default_rng(2000 + op * 16 + dtype)
+    n = 70001 if not name.startswith("prod") else 23
+    if dtype in (H.HALF, H.CHALF) and not (name in EXACT_OPS):
+        n = min(n, 3001)                          # keeps half-precision sums inside the half range
+    kind = "small" if (name.startswith("prod") or dtype in (H.HALF, H.CHALF)) else "general"
+    if name in ("all", "all_finite") or name.startswith("all_"):
+        kind = "positive"
+    xd = H.random_data(dtype, n, rng, kind)
+    if dtype >= H.HALF and name in ("any_nan", "any_inf", "all_finite", "maximum", "minimum", "nnz", "nnz_nan"):
+        sp = H.random_data(dtype, 64, rng, "special")
+        xd[100:164] = sp
+        xd[0] = sp[0]                             # a special value may lead the tensor (a leading NaN must not stick to max/min)
+    elif dtype >= H.HALF and name.endswith("_nan"):
+        # NaN entries (no infinities: they would make the exact value infinite) that the operation must skip
+        idx = rng.choice(n, size=max(2, n // 10), replace=False)
+        nan_elem = H.random_data(dtype, 1, rng, "general")
+        raw = nan_elem.view(np.uint16 if dtype in (H.HALF, H.CHALF) else (np.float32 if dtype in (H.FLOAT, H.CFLOAT) else np.float64))
+        raw[0] = 0x7F00 if dtype in (H.HALF, H.CHALF) else np.nan
+        xd[idx] = nan_elem[0]
+        xd[0] = nan_elem[0]
+    bounds = H.random_data(dtype, 2, rng, "general")
+    b1, b2 = oh.Scalar(), oh.Scalar()
+    C.memmove(C.byref(b1), bounds[0:1].ctypes.data, bounds.dtype.itemsize)
+    C.memmove(C.byref(b2), bounds[1:2].ctypes.data, bounds.dtype.itemsize)
+    p = 3.0
+    x = H.Operand.contiguous(xd, dtype).upload(stream)
+    rd, got = gpu_reduce(stream, op, dtype, x, C.byref(b1), C.byref(b2), p)
+    _, want = cpu_reduce(op, dtype, x, C.byref(b1), C.byref(b2), p, nthreads=4)
+    x.free()
+    isint = dtype <= H.INT64
+    if name in EXACT_OPS or (isint and not name.startswith("norm")):
+        if name == "nnz_nan" and dtype == H.CHALF:
+            # the CPU macro re-converts the float parts through the half type (reduce_ops.h:329-330) and so
+            # treats |x| < 1 as zero; the kernel counts true non-zeros
+            v = to_float64(dtype, xd)
+            want = np.array([np.count_nonzero(~np.isnan(v.real) & ~np.isnan(v.imag) & (v != 0))], np.uint64)
+        H.assert_same_bytes(got, want, "%s %s" % (name, H.NAMES[dtype]))
+        return
+    if isint:       # integer norms: double results
+        v = to_float64(dtype, xd)
+        ref = math.sqrt(math.fsum(v * v)) if name.startswith("norm2") else math.fsum(np.abs(v) ** 3.0) ** (1 / 3.0)
+        assert abs(got[0] - ref) <= (1e-12 if name.startswith("norm2") else 1e-6) * ref
+        return
+    check_against_truth(name, dtype, rd, got, xd)
+    if name == "prod_nan" and dtype >= H.CHALF:
+        return                                   # CPU accumulate step has a sign slip (reduce_ops.h:784)
+    # distance to the literal CPU fold (4 threads): informative bound, an order looser
+    g, w = to_float64(rd, got)[0], to_float64(rd, want)[0]
+    loose = 1e-10 if dtype in (H.DOUBLE, H.CDOUBLE) else (2e-2 if dtype in (H.HALF, H.CHALF) else 1e-3)
+    if name in ("norm", "norm_nan"):
+        loose = max(loose, 1e-5)                  # the CPU evaluates pow in single precision for every type
+    if not (np.isnan(g) and np.isnan(w)):
+        assert abs(g - w) <= loose * max(abs(w), 1.0), (name, g, w)
+
+
+def test_reduce_strided_and_empty(hip, stream):
+    rng = np.random.default_rng(9)
+    parent = rng.integers(-50, 50, size=(33, 50, 20), dtype=np.int32)
+    view = parent[::2, 1::3, ::-1].transpose(2, 0, 1)
+    x = H.Operand(parent, view, H.INT32).upload(stream)
+    for name in ("sum", "maximum", "minimum", "nnz", "sum_abs", "any", "all"):
+        _, got = gpu_reduce(stream, oh.R[name], H.INT32, x)
+        _, want = cpu_reduce(oh.R[name], H.INT32, x)
+        H.assert_same_bytes(got, want, "strided " + name)
+    assert got is not None
+    x.free()
+    # empty tensor: sum is 0, maximum is an error
+    e = H.Operand.contiguous(np.zeros(4, np.float32), H.FLOAT).upload(stream)
+    out = np.ones(1, np.float32)
+    oh.check(oh.lib.och_reduce_all(oh.R["sum"], H.FLOAT, 1, oh.sizes([0]), oh.strides([4]), e.dptr(), None, None, 0.0, orc.ptr(out), None, stream.handle))
+    assert out[0] == 0
+    assert oh.lib.och_reduce_all(oh.R["maximum"], H.FLOAT, 1, oh.sizes([0]), oh.strides([4]), e.dptr(), None, None, 0.0, orc.ptr(out), None, stream.handle) == -1
+    e.free()
+
+
+@pytest.mark.parametrize("dtype", [H.FLOAT, H.DOUBLE], ids=lambda d: H.NAMES[d])
+def test_config3_full_reductions(hip, stream, dtype):
+    """BASELINE config 3, full reductions: sum, 2-norm and max of an 8192 x 8192 N(0,1) tensor.
+    max is exact; sum within 1e-5 (float) / 1e-12 (double) of the exact sum relative to sum|x|, and also
+    relative to |sum| itself thanks to double accumulation; norm2 within the same relative tolerance."""
+    n = 8192 * 8192
+    rng = np.random.default_rng(33)
+    xd = rng.standard_normal(n).astype(H.storage(dtype))
+    x = H.Operand.contiguous(xd, dtype).upload(stream)
+    tol = 1e-5 if dtype == H.FLOAT else 1e-12
+    _, s = gpu_reduce(stream, oh.R["sum"], dtype, x)
+    _, nrm = gpu_reduce(stream, oh.R["norm2"], dtype, x)
+    _, mx = gpu_reduce(stream, oh.R["maximum"], dtype, x)
+    x.free()
+    v = xd.astype(np.float64)
+    exact_sum = math.fsum(v)
+    assert abs(float(s[0]) - exact_sum) <= tol * abs(exact_sum)
+    exact_norm = math.sqrt(math.fsum(v * v))
+    assert abs(float(nrm[0]) - exact_norm) <= tol * exact_norm
+    assert mx[0] == xd.max()
+    # determinism: a second launch gives the same bits
+    x = H.Operand.contiguous(xd, dtype).upload(stream)
+    _, s2 = gpu_reduce(stream, oh.R["sum"], dtype, x)
+    x.free()
+    H.assert_same_bytes(s, s2, "repeatability")

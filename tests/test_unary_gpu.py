@@ -39,7 +39,7 @@ def input_data(name, dtype, rng):
         return H.random_data(dtype, N, rng)
     if name in EXACT or name in EXACT_REAL_ONLY:
         d = H.random_data(dtype, N, rng, "special")
-        if name == "sqrt" and dtype in H.COMPLEX_TYPES:
+        if name in EXACT_REAL_ONLY and dtype in H.COMPLEX_TYPES:
             d = H.random_data(dtype, N, rng, "general")
         return d
     small = {"arcsin", "arccos", "arctanh"}
