@@ -1,0 +1,179 @@
+/* Axis reductions for gfx950: dst[outer] = reduce over the reduced dimensions of src.
+ *
+ * Replaces the three kernel modes of solid/include/solid/core/gpu/reduce_axis.h:142-597 and
+ * their host-side planner (solid/src/core/gpu/op/reduce_axis.c:22-315). Two kernel shapes:
+ *   thread-per-output  : neighbouring threads own neighbouring outputs; used when the outer
+ *                        dimension is the fast one in memory, so every load instruction of a
+ *                        wave is contiguous; four loads in flight per thread
+ *   group-per-output   : a wave (64) or a block (256) strides over the reduced range of one
+ *                        output and combines with a shuffle butterfly (+ LDS for blocks); used
+ *                        when the reduced dimension is the fast one in memory
+ * Accumulator types, NaN rules and result types are those of the full reductions.
+ */
+#pragma once
+#include "och_reduce_all.h"
+
+namespace och {
+
+struct AxisParams
+{
+   char    *src, *dst;
+   int      nd, rd;
+   FastDiv  div[OCH_MAX_DIMS], rdiv[OCH_MAX_DIMS];
+   int64_t  st1[OCH_MAX_DIMS], st2[OCH_MAX_DIMS], rst[OCH_MAX_DIMS];
+   uint32_t nout, relem, rsize0, rrows;          /* relem = rsize0 * rrows */
+};
+
+OCH_D void axis_outer_offsets(const AxisParams &p, uint32_t o, int64_t &o1, int64_t &o2)
+{
+   o1 = 0; o2 = 0;
+   uint32_t q = o;
+   for (int d = 0; d < p.nd - 1; d++)
+   {  uint32_t q2 = fastdiv(q, p.div[d]); uint32_t i = q - q2 * p.div[d].d; q = q2;
+      o1 += (int64_t)i * p.st1[d]; o2 += (int64_t)i * p.st2[d];
+   }
+   if (p.nd > 0) { o1 += (int64_t)q * p.st1[p.nd - 1]; o2 += (int64_t)q * p.st2[p.nd - 1]; }
+}
+
+/* offset of row r of the reduced range (all reduced dimensions but the first) */
+OCH_D int64_t axis_row_offset(const AxisParams &p, uint32_t r)
+{
+   int64_t off = 0; uint32_t q = r;
+   for (int d = 1; d < p.rd - 1; d++)
+   {  uint32_t q2 = fastdiv(q, p.rdiv[d]); off += (int64_t)(q - q2 * p.rdiv[d].d) * p.rst[d]; q = q2; }
+   if (p.rd > 1) off += (int64_t)q * p.rst[p.rd - 1];
+   return off;
+}
+
+template <class RD, class T>
+__global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, const typename RD::Param prm)
+{
+   typedef typename RD::Acc Acc;
+   uint32_t o = blockIdx.x * 256 + threadIdx.x;
+   if (o >= p.nout) return;
+   int64_t o1, o2;
+   axis_outer_offsets(p, o, o1, o2);
+   const char *base = p.src + o1;
+   Acc acc = RD::identity();
+   const int64_t s0 = p.rst[0];
+   for (uint32_t r = 0; r < p.rrows; r++)
+   {  const char *row = base + axis_row_offset(p, r);
+      uint32_t i = 0;
+      for (; i + 4 <= p.rsize0; i += 4)
+      {  T v0 = *reinterpret_cast<const T *>(row + (int64_t)(i + 0) * s0);
+         T v1 = *reinterpret_cast<const T *>(row + (int64_t)(i + 1) * s0);
+         T v2 = *reinterpret_cast<const T *>(row + (int64_t)(i + 2) * s0);
+         T v3 = *reinterpret_cast<const T *>(row + (int64_t)(i + 3) * s0);
+         acc = RD::combine(acc, RD::load(v0, prm)); acc = RD::combine(acc, RD::load(v1, prm));
+         acc = RD::combine(acc, RD::load(v2, prm)); acc = RD::combine(acc, RD::load(v3, prm));
+      }
+      for (; i < p.rsize0; i++) acc = RD::combine(acc, RD::load(*reinterpret_cast<const T *>(row + (int64_t)i * s0), prm));
+   }
+   *reinterpret_cast<typename RD::Res *>(p.dst + o2) = RD::finalize(acc, prm);
+}
+
+/* GROUP threads cooperate on one output; GROUP is 64 (one wave) or 256 (the whole block) */
+template <class RD, class T, int GROUP>
+__global__ __launch_bounds__(256) void axis_group_kernel(const AxisParams p, const typename RD::Param prm)
+{
+   typedef typename RD::Acc Acc;
+   __shared__ Acc lds[4];
+   constexpr int PER_BLOCK = 256 / GROUP;
+   const uint32_t lane = threadIdx.x % GROUP;
+   const uint32_t o = blockIdx.x * PER_BLOCK + threadIdx.x / GROUP;
+   const bool active = o < p.nout;
+   Acc acc = RD::identity();
+   int64_t o1 = 0, o2 = 0;
+   if (active)
+   {  axis_outer_offsets(p, o, o1, o2);
+      const char *base = p.src + o1;
+      const int64_t s0 = p.rst[0];
+      if (p.rd <= 1)
+      {  uint32_t i = lane;
+         for (; i + 3 * GROUP < p.rsize0; i += 4 * GROUP)
+         {  T v0 = *reinterpret_cast<const T *>(base + (int64_t)i * s0);
+            T v1 = *reinterpret_cast<const T *>(base + (int64_t)(i + GROUP) * s0);
+            T v2 = *reinterpret_cast<const T *>(base + (int64_t)(i + 2 * GROUP) * s0);
+            T v3 = *reinterpret_cast<const T *>(base + (int64_t)(i + 3 * GROUP) * s0);
+            acc = RD::combine(acc, RD::load(v0, prm)); acc = RD::combine(acc, RD::load(v1, prm));
+            acc = RD::combine(acc, RD::load(v2, prm)); acc = RD::combine(acc, RD::load(v3, prm));
+         }
+         for (; i < p.rsize0; i += GROUP) acc = RD::combine(acc, RD::load(*reinterpret_cast<const T *>(base + (int64_t)i * s0), prm));
+      }
+      else
+      {  for (uint32_t j = lane; j < p.relem; j += GROUP)
+         {  uint32_t r = fastdiv(j, p.rdiv[0]); uint32_t i = j - r * p.rdiv[0].d;
+            acc = RD::combine(acc, RD::load(*reinterpret_cast<const T *>(base + axis_row_offset(p, r) + (int64_t)i * s0), prm));
+         }
+      }
+   }
+#pragma unroll
+   for (int m = 32; m >= 1; m >>= 1) acc = RD::combine(acc, shfl_xor_any<Acc>(acc, m));
+   if constexpr (GROUP == 256)
+   {  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = acc;
+      __syncthreads();
+      if (threadIdx.x == 0) { acc = RD::combine(RD::combine(lds[0], lds[1]), RD::combine(lds[2], lds[3])); }
+   }
+   if (active && lane == 0) *reinterpret_cast<typename RD::Res *>(p.dst + o2) = RD::finalize(acc, prm);
+}
+
+typedef int (*axis_fn)(const och_reduce_axis_config *c, double pnorm);
+
+template <class T, int OP>
+static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
+{
+   typedef Reduce<T, OP> RD;
+   if (c->ndims < 0 || c->ndims > OCH_MAX_DIMS || c->rdims < 0 || c->rdims > OCH_MAX_DIMS)
+      return set_error("invalid number of dimensions (%d, %d)", c->ndims, c->rdims);
+   typename RD::Param prm;
+   memset(&prm, 0, sizeof(prm));
+   prm.phalf = pnorm / 2; prm.pinv = (pnorm != 0) ? 1.0 / pnorm : 0.0;
+   uint64_t nout = 1, relem = 1;
+   for (int d = 0; d < c->ndims; d++) nout *= c->size[d];
+   for (int d = 0; d < c->rdims; d++) relem *= c->rsize[d];
+   if (nout == 0) return 0;
+   if (relem == 0 && RD::NEEDS_DATA) return set_error("reduction over an empty range is undefined for this operation");
+   if (nout > 0xFFFFFF00ull || relem > 0xFFFFFF00ull) return set_error("axis reduction with more than 2^32 outputs or reduced elements is not supported");
+
+   AxisParams p;
+   memset(&p, 0, sizeof(p));
+   p.src = (char *)c->ptr1; p.dst = (char *)c->ptr2;
+   /* drop unit dimensions */
+   for (int d = 0; d < c->ndims; d++)
+   {  if (c->size[d] == 1) continue;
+      p.div[p.nd] = make_fastdiv((uint32_t)c->size[d]); p.st1[p.nd] = c->strides1[d]; p.st2[p.nd] = c->strides2[d]; p.nd++;
+   }
+   uint64_t rs0 = 1;
+   for (int d = 0; d < c->rdims; d++)
+   {  if (c->rsize[d] == 1) continue;
+      if (p.rd == 0) rs0 = c->rsize[d];
+      p.rdiv[p.rd] = make_fastdiv((uint32_t)c->rsize[d]); p.rst[p.rd] = c->rstrides[d]; p.rd++;
+   }
+   p.nout = (uint32_t)nout; p.relem = (uint32_t)relem;
+   p.rsize0 = (relem == 0) ? 0 : (uint32_t)rs0;
+   p.rrows = (relem == 0) ? 0 : (uint32_t)(relem / rs0);
+   hipStream_t stream = as_stream(c->stream);
+
+   /* which side is the fast one in memory? */
+   int64_t outer_fast = (p.nd > 0) ? (p.st1[0] < 0 ? -p.st1[0] : p.st1[0]) : INT64_MAX;
+   for (int d = 1; d < p.nd; d++) { int64_t a = p.st1[d] < 0 ? -p.st1[d] : p.st1[d]; if (a < outer_fast) outer_fast = a; }
+   int64_t red_fast = (p.rd > 0) ? (p.rst[0] < 0 ? -p.rst[0] : p.rst[0]) : INT64_MAX;
+   bool cooperative = (p.rd > 0) && ((red_fast < outer_fast) || (nout < 16384 && relem >= 256));
+   if (!cooperative)
+      hipLaunchKernelGGL((axis_thread_kernel<RD, T>), dim3((p.nout + 255) / 256), dim3(256), 0, stream, p, prm);
+   else if (relem <= 2048 && nout >= 1024)
+      hipLaunchKernelGGL((axis_group_kernel<RD, T, 64>), dim3((p.nout + 3) / 4), dim3(256), 0, stream, p, prm);
+   else
+      hipLaunchKernelGGL((axis_group_kernel<RD, T, 256>), dim3(p.nout), dim3(256), 0, stream, p, prm);
+   OCH_CHECK_LAUNCH();
+   return 0;
+}
+
+template <class T, int OP, bool OK> struct PickA { static constexpr axis_fn fn = nullptr; };
+template <class T, int OP> struct PickA<T, OP, true> { static constexpr axis_fn fn = &launch_reduce_axis<T, OP>; };
+template <int OP> struct RowA { static const axis_fn fn[DT_COUNT]; };
+#define OCH_X(T) PickA<T, OP, reduce_defined<T, OP>()>::fn,
+template <int OP> const axis_fn RowA<OP>::fn[DT_COUNT] = { OCH_FOR_ALL_TYPES(OCH_X) };
+#undef OCH_X
+
+} /* namespace och */

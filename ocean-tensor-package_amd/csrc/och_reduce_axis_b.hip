@@ -1,0 +1,15 @@
+/* Axis-reduction kernels, operations: 15 16 17 18 */
+#include "och_reduce_axis.h"
+namespace och {
+axis_fn axis_lookup_b(int op, int dtype)
+{
+   switch (op)
+   {
+      case 15: return RowA<15>::fn[dtype];
+      case 16: return RowA<16>::fn[dtype];
+      case 17: return RowA<17>::fn[dtype];
+      case 18: return RowA<18>::fn[dtype];
+   }
+   return nullptr;
+}
+}

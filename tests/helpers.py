@@ -198,3 +198,26 @@ def cpu_unary(op, dtype, a, z, zparent, nthreads=1):
     st = orc.lib.oracle_unary(op, dtype, len(z.shape), oh.sizes(z.shape), oh.strides(a.strides), a.hptr(),
                               oh.strides(z.strides), z.hptr(zparent), nthreads)
     assert st == 0
+
+
+def axis_config(src, dst, axes, stream=None, device=True):
+    """och_reduce_axis_config for reducing `axes` of Operand src into Operand dst (dst has the kept
+    dimensions only), prepared the way OcSolid_analyzeReduceAxis does: kept dimensions sorted by
+    destination stride, reduced dimensions by source stride, unit dimensions dropped."""
+    cfg = oh.ReduceAxisConfig()
+    kept = [d for d in range(len(src.shape)) if d not in axes]
+    outer = [(src.shape[d], src.strides[d], dst.strides[i]) for i, d in enumerate(kept) if src.shape[d] != 1]
+    outer.sort(key=lambda t: abs(t[2]))
+    inner = sorted([(src.shape[d], src.strides[d]) for d in axes if src.shape[d] != 1], key=lambda t: abs(t[1]))
+    cfg.ndims = len(outer)
+    for i, (n, s1, s2) in enumerate(outer):
+        cfg.size[i], cfg.strides1[i], cfg.strides2[i] = n, s1, s2
+    cfg.rdims = len(inner)
+    for i, (n, s) in enumerate(inner):
+        cfg.rsize[i], cfg.rstrides[i] = n, s
+    if device:
+        cfg.ptr1, cfg.ptr2 = src.dptr().value, dst.dptr().value
+        cfg.stream = stream.handle if stream is not None else None
+    else:
+        cfg.ptr1, cfg.ptr2 = src.hptr().value, dst.hptr().value
+    return cfg

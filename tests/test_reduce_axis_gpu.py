@@ -1,0 +1,133 @@
+"""Parity of the axis reductions (och_reduce_axis) with the CPU oracle.
+
+Reference tests of the same kind: examples/python/gpu/tensors/ocean_axis_reduce_04.py,
+tensor_axis_norm2_01.py (against numpy.linalg.norm), examples/python/cpu/tensors/
+axis_reduce_01..04.py (int8 -> int64 sums, several axes), axis_sum_01.py (NaN variants).
+Exact for logical / counting / integer / extrema operations; floating sums and norms within
+1e-5 (half 2e-3, double 1e-12) of a float64 evaluation, relative to the sum of magnitudes.
+"""
+import numpy as np
+import pytest
+
+import helpers as H
+import ocean_hip as oh
+
+pytestmark = pytest.mark.gpu
+orc = H.orc
+
+AXIS_OPS = ["any", "all", "all_finite", "any_inf", "any_nan", "nnz", "nnz_nan", "sum", "sum_nan", "prod", "prod_nan",
+            "sum_abs", "sum_abs_nan", "maximum", "minimum", "maximum_abs", "minimum_abs", "norm", "norm_nan", "norm2", "norm2_nan"]
+EXACT = {"any", "all", "all_finite", "any_inf", "any_nan", "nnz", "nnz_nan", "maximum", "minimum"}
+
+
+def to_f64(dtype, a):
+    if dtype == H.HALF:
+        return np.array([orc.lib.oracle_half_to_float(int(b)) for b in a.reshape(-1)], np.float64).reshape(a.shape)
+    if dtype == H.CHALF:
+        out = np.empty(a.shape, np.complex128)
+        out.real, out.imag = to_f64(H.HALF, a["real"]), to_f64(H.HALF, a["imag"])
+        return out
+    return a.astype(np.complex128 if dtype >= H.CFLOAT else np.float64)
+
+
+def run_case(stream, name, dtype, parent, view, axes, p=3.0):
+    op = oh.R[name]
+    rd = oh.lib.och_reduce_result_dtype(op, dtype)
+    kept_shape = [n for d, n in enumerate(view.shape) if d not in axes]
+    out_parent = np.zeros(kept_shape[::-1] if kept_shape else (1,), H.storage(rd))     # column-major destination
+    out_view = out_parent.T if kept_shape else out_parent.reshape(())
+    src = H.Operand(parent, view, dtype).upload(stream)
+    dst = H.Operand(out_parent, out_view, rd).upload(stream)
+    cfg = H.axis_config(src, dst, axes, stream)
+    oh.check(oh.lib.och_reduce_axis(op, dtype, cfg, p))
+    got = dst.download()
+    want = out_parent.copy()
+    dsth = H.Operand(want, want.T if kept_shape else want.reshape(()), rd)
+    cfgh = H.axis_config(src, dsth, axes, device=False)
+    assert orc.lib.oracle_reduce_axis(op, dtype, cfgh, p) == 0
+    src.free(); dst.free()
+    return rd, got, want
+
+
+CASES = [(n, d) for n in AXIS_OPS for d in H.ALL_TYPES]
+
+
+@pytest.mark.parametrize("name,dtype", CASES, ids=["%s-%s" % (n, H.NAMES[d]) for n, d in CASES])
+def test_axis_all_ops(hip, stream, name, dtype):
+    op = oh.R[name]
+    if not oh.lib.och_reduce_supported(op, dtype):
+        cfg = oh.ReduceAxisConfig()
+        assert oh.lib.och_reduce_axis(op, dtype, cfg, 0.0) == -1
+        return
+    rng = np.random.default_rng(500 + op * 16 + dtype)
+    small = name.startswith("prod") or dtype in (H.HALF, H.CHALF)
+    shape = (6, 5, 7) if name.startswith("prod") else (37, 20, 11)
+    parent = H.random_data(dtype, int(np.prod(shape)), rng, "small" if small else "general").reshape(shape[::-1])
+    view = parent.T                                  # Ocean order: dimension 0 fastest
+    if dtype >= H.HALF and name in ("any_nan", "any_inf", "all_finite", "maximum", "minimum", "nnz", "nnz_nan"):
+        flat = parent.reshape(-1)
+        flat[3:19] = H.random_data(dtype, 16, rng, "special")
+    for axes in ([0], [1], [2], [0, 2], [0, 1, 2]):
+        rd, got, want = run_case(stream, name, dtype, parent, view, axes)
+        what = "%s %s axes=%s" % (name, H.NAMES[dtype], axes)
+        isint = dtype <= H.INT64
+        if name in EXACT or (isint and not name.startswith("norm")):
+            if name == "nnz_nan" and dtype == H.CHALF:
+                continue                              # CPU macro quirk, see test_reduce_gpu.py
+            H.assert_same_bytes(got, want, what)
+            continue
+        if name == "prod_nan" and dtype >= H.CHALF:
+            continue                                  # CPU accumulate step has a sign slip (reduce_ops.h:784)
+        g, w = to_f64(rd, got), to_f64(rd, want)
+        tol = 1e-12 if dtype in (H.DOUBLE, H.CDOUBLE) else (4e-3 if dtype in (H.HALF, H.CHALF) else 1e-5)
+        if name in ("norm", "norm_nan"):
+            tol = max(tol, 1e-5)                      # CPU pow is single precision
+        v = to_f64(dtype, view)
+        scale = np.abs(v).sum(axis=tuple(axes)).T if name.startswith("sum") else np.abs(w)
+        if name.startswith("prod"):
+            tol *= 50
+        with np.errstate(invalid="ignore"):
+            ok = (g == w) | (np.abs(g - w) <= tol * np.maximum(np.abs(np.asarray(scale)), 1e-6))
+        assert np.all(ok), what
+
+
+def test_axis_layouts(hip, stream):
+    """Non-contiguous sources: sliced / transposed views, reduction along the fast and the slow axis,
+    single-output and no-reduction corner cases."""
+    rng = np.random.default_rng(2)
+    parent = rng.integers(-99, 99, size=(24, 40, 64), dtype=np.int32)
+    view = parent[::2, 1::3, ::-2].transpose(2, 0, 1)          # shape (32, 12, 13), mixed strides
+    for axes in ([0], [1], [2], [1, 2], [0, 1], [0, 1, 2], []):
+        for name in ("sum", "maximum", "nnz"):
+            rd, got, want = run_case(stream, name, H.INT32, parent, view, axes)
+            H.assert_same_bytes(got, want, "%s axes=%s" % (name, axes))
+    # long reduction, few outputs (block-per-output path) and many outputs, short reduction
+    big = rng.integers(-9, 9, size=(3, 50000), dtype=np.int16)
+    rd, got, want = run_case(stream, "sum", H.INT16, big, big.T, [0])
+    H.assert_same_bytes(got, want, "long reduction")
+    wide = rng.integers(-9, 9, size=(5, 70000), dtype=np.int8)
+    rd, got, want = run_case(stream, "sum", H.INT8, wide, wide.T, [1])
+    H.assert_same_bytes(got, want, "many outputs")
+    assert rd == H.INT64
+
+
+@pytest.mark.parametrize("dtype", [H.FLOAT, H.DOUBLE], ids=lambda d: H.NAMES[d])
+def test_config3_axis_reductions(hip, stream, dtype):
+    """BASELINE config 3, axis part: sum and min along axis 0 and axis 1 of a 3-D 512 x 512 x 256
+    non-contiguous view (cut from a larger parent so that no two dimensions merge), N(0,1) data.
+    min is exact; sum within 1e-5 / 1e-12 of the float64 result relative to the sum of magnitudes."""
+    rng = np.random.default_rng(303)
+    st = H.storage(dtype)
+    parent = rng.standard_normal((258, 514, 516)).astype(st)
+    view = parent[1:257, 1:513, 2:514].transpose(2, 1, 0)       # (512, 512, 256): dim 0 unit stride, padded pitches
+    assert view.shape == (512, 512, 256)
+    v64 = view.astype(np.float64)
+    tol = 1e-5 if dtype == H.FLOAT else 1e-12
+    for axis in (0, 1):
+        rd, got, want = run_case(stream, "sum", dtype, parent, view, [axis])
+        ref = v64.sum(axis=axis).T
+        scale = np.abs(v64).sum(axis=axis).T
+        assert np.all(np.abs(got.astype(np.float64) - ref) <= tol * scale), "axis %d sum" % axis
+        rd, got, want = run_case(stream, "minimum", dtype, parent, view, [axis])
+        H.assert_same_bytes(got, want, "axis %d min" % axis)
+        H.assert_same_bytes(got, view.min(axis=axis).T.copy(), "axis %d min vs numpy" % axis)
