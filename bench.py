@@ -1,0 +1,304 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X device module on BASELINE.json's configurations (one GPU).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only-step]
+
+One "step" is one pass of configuration 2 through the device library, as Ocean's interface
+layer would issue it for   Z = (A.T + r + I) * F   with
+    A  float64 4096 x 4096, used through its transposed view (non-unit strides)
+    r  float64 1 x 4096 row, broadcast along dimension 0 (zero stride)
+    I  int32 4096 x 4096, auto-cast to float64 by a converting copy
+    F  float32 4096 x 4096 stored byte-swapped, brought to native float64 by a swapping copy
+i.e. five launches: add(A.T, r) -> Z ; copy(I) -> TI ; add(Z, TI) -> Z ; byteswap_copy(F) -> TF ;
+multiply(Z, TF) -> Z.  Values are U(-10, 10) from a fixed seed; inputs are resident in HBM before
+the timed region.  value = algorithmic bytes of the step / time (GB/s): every logical input element
+read once, every output element written once, the broadcast row counted once.
+
+Printed: ONE JSON line with the driver's fields plus
+    roofline      dominant kernel of the step: algorithmic bytes per launch / mean launch time
+                  (HIP events on the launch stream) against the 8 TB/s HBM peak
+    kernels       the same figure for every kernel of the step
+    configs       short measurements of configurations 1, 3, 4 and 5 (GB/s or TFLOP/s)
+    cpu_baseline  the CPU oracle (a port of Ocean's CPU path with its threading policy:
+                  binary operations serial, copies over all cores) timed on this host on the
+                  same full-size step
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "ocean-tensor-package_amd"))
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK = {"float": 157.3, "double": 78.6, "cfloat": 157.3, "cdouble": 78.6}
+
+N2 = 4096
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only-step", action="store_true", help="time the configuration-2 step only (for profiling)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (every figure here is a one-GPU figure)" % args.gpus)
+
+    import numpy as np
+    import ocean_hip as oh
+
+    oh.check(oh.lib.och_device_set(0))
+    oh.check(oh.lib.och_device_warmup(0))
+    prop = oh.device_properties(0)
+    stream = oh.Stream()
+    lib = oh.lib
+    B, R = oh.B, oh.R
+    F32, F64, I32, I16, CF, CD = oh.FLOAT, oh.DOUBLE, oh.INT32, oh.INT16, oh.CFLOAT, oh.CDOUBLE
+
+    def time_launches(fn, reps=20, warm=3):
+        """mean duration in ms of one call of fn(), measured with events on the launch stream"""
+        for _ in range(warm):
+            fn()
+        e0, e1 = oh.Event(), oh.Event()
+        e0.record(stream)
+        for _ in range(reps):
+            fn()
+        e1.record(stream)
+        e1.synchronize()
+        ms = e0.elapsed_ms(e1) / reps
+        e0.destroy(); e1.destroy()
+        return ms
+
+    # ------------------------------------------------------------------ configuration 2
+    n = N2
+    rng = np.random.default_rng(20240)
+    hostA = rng.uniform(-10, 10, (n, n))
+    hostR = rng.uniform(-10, 10, n)
+    hostI = rng.integers(-10, 10, (n, n), endpoint=True).astype(np.int32)
+    hostF = rng.uniform(-10, 10, (n, n)).astype(np.float32)
+    hostFs = hostF.byteswap()
+    NSETS = 2
+    sets = []
+    for _ in range(NSETS):
+        s = {"A": oh.to_device(hostA, stream), "r": oh.to_device(hostR, stream), "I": oh.to_device(hostI, stream),
+             "F": oh.to_device(hostFs, stream), "Z": oh.DeviceBuffer(8 * n * n, stream),
+             "TI": oh.DeviceBuffer(8 * n * n, stream), "TF": oh.DeviceBuffer(8 * n * n, stream)}
+        sets.append(s)
+    shape = oh.sizes([n, n])
+    st_f64, st_f64_T, st_row = oh.strides([8, 8 * n]), oh.strides([8 * n, 8]), oh.strides([0, 8])
+    st_i32, st_f32 = oh.strides([4, 4 * n]), oh.strides([4, 4 * n])
+    h = stream.handle
+
+    def k_add_transposed(s):
+        oh.check(lib.och_binary(B["add"], F64, 2, shape, st_f64_T, s["A"].ptr, st_row, s["r"].ptr, st_f64, s["Z"].ptr, h))
+
+    def k_cast_i32(s):
+        oh.check(lib.och_copy(I32, F64, 2, shape, st_i32, s["I"].ptr, 2, shape, st_f64, s["TI"].ptr, h))
+
+    def k_add(s):
+        oh.check(lib.och_binary(B["add"], F64, 2, shape, st_f64, s["Z"].ptr, st_f64, s["TI"].ptr, st_f64, s["Z"].ptr, h))
+
+    def k_cast_swapped(s):
+        oh.check(lib.och_byteswap_copy(F32, F64, 2, shape, st_f32, s["F"].ptr, 2, shape, st_f64, s["TF"].ptr, h))
+
+    def k_multiply(s):
+        oh.check(lib.och_binary(B["multiply"], F64, 2, shape, st_f64, s["Z"].ptr, st_f64, s["TF"].ptr, st_f64, s["Z"].ptr, h))
+
+    nn = n * n
+    step_kernels = [
+        ("add f64: transposed view + row broadcast", k_add_transposed, 8 * nn * 2 + 8 * n),
+        ("copy int32 -> f64", k_cast_i32, 12 * nn),
+        ("add f64 contiguous", k_add, 24 * nn),
+        ("byteswap_copy f32 (swapped) -> f64", k_cast_swapped, 12 * nn),
+        ("multiply f64 contiguous", k_multiply, 24 * nn),
+    ]
+    step_bytes = sum(b for _, _, b in step_kernels)
+
+    def step(i):
+        s = sets[i % NSETS]
+        for _, fn, _ in step_kernels:
+            fn(s)
+
+    for i in range(args.warmup):
+        step(i)
+    stream.synchronize()
+    oh.check(lib.och_device_synchronize())
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    stream.synchronize()
+    oh.check(lib.och_device_synchronize())
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / max(args.steps, 1)
+    value = step_bytes / ms_per_step / 1e6
+
+    result = {
+        "metric": "elementwise/reduction HBM GB/s (% of peak); fp32/fp64 GEMM TFLOP/s",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f64", "data": "synthetic",
+        "config": {"workload": "config 2: Z = (A.T + r + I) * F, float64 4096x4096 transposed view + 1x4096 row broadcast, "
+                               "int32 operand cast to float64, byteswapped float32 operand; 5 launches, %.1f MB algorithmic" % (step_bytes / 1e6),
+                   "device": prop.arch.decode(), "compute_units": prop.multiprocessor_count,
+                   "percent_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1)},
+    }
+    if args.only_step:
+        print(json.dumps(result))
+        return
+
+    # per-kernel roofline of the step
+    kernels = []
+    for name, fn, nbytes in step_kernels:
+        ms = time_launches(lambda fn=fn: fn(sets[0]))
+        kernels.append({"kernel": name, "ms": round(ms, 4), "algorithmic_MB": round(nbytes / 1e6, 1),
+                        "GBps": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 3)})
+    dom = max(kernels, key=lambda k: k["ms"])
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get(dom["kernel"])
+    result["roofline"] = {"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(dom["GBps"] / HBM_PEAK_GBS, 3), "traffic": traffic}
+    result["kernels"] = kernels
+    for s in sets:
+        for b in s.values():
+            b.free()
+    stream.synchronize()
+
+    configs = {}
+
+    def gbps(nbytes, ms):
+        return {"ms": round(ms, 4), "GBps": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 3)}
+
+    # ------------------------------------------------------------------ configuration 1
+    n1 = 1 << 24
+    x, y, t, z = [oh.DeviceBuffer(4 * n1, stream) for _ in range(4)]
+    x.upload(rng.uniform(-1, 1, n1).astype(np.float32)); y.upload(rng.uniform(-1, 1, n1).astype(np.float32))
+    s1, st1 = oh.sizes([n1]), oh.strides([4])
+    ms_mul = time_launches(lambda: oh.check(lib.och_binary(B["multiply"], F32, 1, s1, st1, x.ptr, st1, y.ptr, st1, t.ptr, h)))
+    ms_add = time_launches(lambda: oh.check(lib.och_binary(B["add"], F32, 1, s1, st1, t.ptr, st1, x.ptr, st1, z.ptr, h)))
+    configs["c1_scale_f32_2^24"] = gbps(12 * n1, ms_mul)
+    configs["c1_add_f32_2^24"] = gbps(12 * n1, ms_add)
+    for b in (x, y, t, z):
+        b.free()
+
+    # ------------------------------------------------------------------ configuration 3
+    n3 = 8192 * 8192
+    for dt, es, nm in ((F32, 4, "f32"), (F64, 8, "f64")):
+        buf = oh.DeviceBuffer(es * n3, stream)
+        chunk = rng.standard_normal(1 << 22).astype(np.float32 if es == 4 else np.float64)
+        for off in range(0, n3, 1 << 22):
+            buf.upload(chunk, offset=off * es)
+        dres = oh.DeviceBuffer(64, stream)
+        s3, st3 = oh.sizes([n3]), oh.strides([es])
+        for opn in ("sum", "norm2", "maximum"):
+            ms = time_launches(lambda: oh.check(lib.och_reduce_all_device(R[opn], dt, 1, s3, st3, buf.ptr, None, None, 0.0, dres.ptr, None, h)), reps=10)
+            configs["c3_%s_%s_8192^2" % (opn, nm)] = gbps(es * n3, ms)
+        # axis reductions on a 512 x 512 x 256 view with padded pitches (no two dimensions merge);
+        # the view lives in a parent of (512+4) x (512+2) x 256 elements
+        d0, d1, d2 = 512, 512, 256
+        p0, p1 = (d0 + 4) * es, (d0 + 4) * (d1 + 2) * es
+        parent_bytes = p1 * d2
+        extent = (d0 - 1) * es + (d1 - 1) * p0 + (d2 - 1) * p1 + es
+        assert extent <= parent_bytes, "axis view exceeds its parent buffer"
+        abuf = oh.DeviceBuffer(parent_bytes, stream)
+        for off in range(0, parent_bytes, chunk.nbytes):
+            m = min(chunk.nbytes, parent_bytes - off) // chunk.itemsize
+            abuf.upload(chunk[:m], offset=off)
+        out = oh.DeviceBuffer(es * d0 * d1, stream)
+        for axis, keep in ((0, (d1, d2)), (1, (d0, d2))):
+            cfg = oh.ReduceAxisConfig()
+            cfg.ndims = 2
+            if axis == 0:
+                cfg.size[0], cfg.size[1] = d1, d2; cfg.strides1[0], cfg.strides1[1] = p0, p1
+                cfg.rsize[0], cfg.rstrides[0] = d0, es
+            else:
+                cfg.size[0], cfg.size[1] = d0, d2; cfg.strides1[0], cfg.strides1[1] = es, p1
+                cfg.rsize[0], cfg.rstrides[0] = d1, p0
+            cfg.strides2[0], cfg.strides2[1] = es, es * keep[0]
+            assert es * keep[0] * keep[1] <= es * d0 * d1
+            cfg.rdims = 1; cfg.ptr1, cfg.ptr2, cfg.stream = abuf.ptr.value, out.ptr.value, h
+            for opn in ("sum", "minimum"):
+                ms = time_launches(lambda: oh.check(lib.och_reduce_axis(R[opn], dt, C.byref(cfg), 0.0)), reps=10)
+                configs["c3_axis%d_%s_%s_512x512x256" % (axis, opn, nm)] = gbps(es * (d0 * d1 * d2 + keep[0] * keep[1]), ms)
+        abuf.free()
+        for b in (buf, dres, out):
+            b.free()
+
+    # ------------------------------------------------------------------ configuration 4
+    d0, d1, d2 = 1024, 1024, 64
+    n4 = d0 * d1 * d2
+    src = oh.DeviceBuffer(2 * 2 * n4, stream); dst = oh.DeviceBuffer(4 * n4, stream)
+    chunk = rng.integers(-32768, 32767, 1 << 22, dtype=np.int16, endpoint=True)
+    for off in range(0, 2 * n4, 1 << 22):
+        src.upload(chunk, offset=off * 2)
+    sz4 = oh.sizes([d0, d1, d2])
+    st_src, st_dst = oh.strides([4, 4 * d0, 4 * d0 * d1]), oh.strides([4, 4 * d0, 4 * d0 * d1])
+    ms = time_launches(lambda: oh.check(lib.och_byteswap_copy(I16, F32, 3, sz4, st_src, src.ptr, 3, sz4, st_dst, dst.ptr, h)), reps=10)
+    configs["c4_int16_swapped_step2_to_f32_1024x1024x64"] = gbps(6 * n4, ms)
+    src.free(); dst.free()
+    n4b = 1 << 26
+    src = oh.DeviceBuffer(8 * n4b, stream); dst = oh.DeviceBuffer(16 * n4b, stream)
+    oh.check(lib.och_memset_async(src.ptr, 0, 8 * n4b, h))
+    s4, sa, sb = oh.sizes([n4b]), oh.strides([8]), oh.strides([16])
+    ms = time_launches(lambda: oh.check(lib.och_copy(CF, CD, 1, s4, sa, src.ptr, 1, s4, sb, dst.ptr, h)), reps=10)
+    configs["c4_cfloat_to_cdouble_2^26"] = gbps(24 * n4b, ms)
+    src.free(); dst.free()
+
+    # ------------------------------------------------------------------ configuration 5 (GEMM)
+    if "och_gemm" not in oh.MISSING:
+        for dt, es, nm, dim, flop_per_mac in ((F64, 8, "double", 8192, 2), (F32, 4, "float", 8192, 2), (CF, 8, "cfloat", 4096, 8)):
+            if not lib.och_gemm_supported(dt):
+                continue
+            a, b, c = [oh.DeviceBuffer(es * dim * dim, stream) for _ in range(3)]
+            block = rng.uniform(-1, 1, 1 << 22).astype(np.float32 if nm != "double" else np.float64)
+            for buf in (a, b):
+                for off in range(0, es * dim * dim, block.nbytes):
+                    buf.upload(block[: (min(block.nbytes, es * dim * dim - off)) // block.itemsize], offset=off)
+            one = np.array([1, 0], dtype=block.dtype); zero = np.zeros(2, dtype=block.dtype)
+            for ta, tb in ((b"N", b"N"), (b"T", b"N"), (b"N", b"T")):
+                fn = lambda: oh.check(lib.och_gemm(dt, ta, tb, dim, dim, dim, one.ctypes.data, a.ptr, dim, b.ptr, dim,
+                                                   zero.ctypes.data, c.ptr, dim, 1, h))
+                ms = time_launches(fn, reps=3, warm=1)
+                tf = flop_per_mac * dim ** 3 / ms / 1e9
+                configs["c5_gemm_%s_%d_%s%s" % (nm, dim, ta.decode(), tb.decode())] = {
+                    "ms": round(ms, 3), "TFLOPs": round(tf, 2), "frac": round(tf / MFMA_PEAK[nm], 3)}
+            for buf in (a, b, c):
+                buf.free()
+    result["configs"] = configs
+
+    # ------------------------------------------------------------------ CPU baseline (oracle, Ocean's threading policy)
+    if not args.no_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        import oracle_lib as orc
+        orc.setup(oh)
+        threads = orc.lib.oracle_max_threads()
+        Z = np.empty((n, n)); TI = np.empty((n, n)); TF = np.empty((n, n))
+        p = orc.ptr
+
+        def cpu_step():
+            assert orc.lib.oracle_binary(B["add"], F64, 2, shape, st_f64_T, p(hostA), st_row, p(hostR), st_f64, p(Z)) == 0
+            assert orc.lib.oracle_copy(I32, F64, 2, shape, st_i32, p(hostI), 2, shape, st_f64, p(TI), threads) == 0
+            assert orc.lib.oracle_binary(B["add"], F64, 2, shape, st_f64, p(Z), st_f64, p(TI), st_f64, p(Z)) == 0
+            assert orc.lib.oracle_byteswap_copy(F32, F64, 2, shape, st_f32, p(hostFs), 2, shape, st_f64, p(TF), threads) == 0
+            assert orc.lib.oracle_binary(B["multiply"], F64, 2, shape, st_f64, p(Z), st_f64, p(TF), st_f64, p(Z)) == 0
+
+        cpu_step()
+        reps, t0 = 0, time.perf_counter()
+        while reps < 5 and (time.perf_counter() - t0) < 20:
+            cpu_step(); reps += 1
+        cpu_ms = (time.perf_counter() - t0) * 1e3 / reps
+        result["cpu_baseline"] = {"value": round(step_bytes / cpu_ms / 1e6, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+                                  "sample": "%d full-size configuration-2 steps (binary operations serial, copies on %d threads, as in Ocean's CPU module)" % (reps, threads),
+                                  "ms_per_step": round(cpu_ms, 1)}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -15,6 +15,7 @@
  *   - 32-bit group indices; larger tensors are cut on the host.
  */
 #pragma once
+#include <string.h>
 #include "och_common.h"
 #include "och_dtypes.h"
 
@@ -58,10 +59,41 @@ template <int NOPS> struct EwParams
 
 template <class T, int VEC> struct alignas((sizeof(T) * VEC) > 16 ? 16 : (sizeof(T) * VEC)) Pack { T v[VEC]; };
 
+template <class T> constexpr int vec_for_c() { return (16 / (int)sizeof(T)) > 0 ? (16 / (int)sizeof(T)) : 1; }
+
+/* Wide accesses go through a native vector type of the pack's byte width, so that the compiler
+   keeps them as ONE load/store instruction (an aggregate copy is split into element accesses
+   and may then be merged with the strided path into element-wise loads). */
+typedef unsigned int och_u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int och_u32x4 __attribute__((ext_vector_type(4)));
+template <int BYTES> struct RawVec;
+template <> struct RawVec<1>  { typedef uint8_t  type; };
+template <> struct RawVec<2>  { typedef uint16_t type; };
+template <> struct RawVec<4>  { typedef uint32_t type; };
+template <> struct RawVec<8>  { typedef och_u32x2 type; };
+template <> struct RawVec<16> { typedef och_u32x4 type; };
+
+template <class T, int VEC>
+OCH_D void load_wide(Pack<T, VEC> &p, const char *addr)
+{
+   static_assert(sizeof(Pack<T, VEC>) <= 16, "pack wider than 128 bits");
+   typedef typename RawVec<sizeof(Pack<T, VEC>)>::type V;
+   V raw = *reinterpret_cast<const V *>(addr);
+   __builtin_memcpy(&p, &raw, sizeof(V));
+}
+template <class T, int VEC>
+OCH_D void store_wide(const Pack<T, VEC> &p, char *addr)
+{
+   typedef typename RawVec<sizeof(Pack<T, VEC>)>::type V;
+   V raw;
+   __builtin_memcpy(&raw, &p, sizeof(V));
+   *reinterpret_cast<V *>(addr) = raw;
+}
+
 template <class T, int VEC>
 OCH_D void load_pack(Pack<T, VEC> &p, const char *addr, int64_t estride, int vec)
 {
-   if (vec) p = *reinterpret_cast<const Pack<T, VEC> *>(addr);
+   if (vec) load_wide<T, VEC>(p, addr);
    else
    {
 #pragma unroll
@@ -71,7 +103,7 @@ OCH_D void load_pack(Pack<T, VEC> &p, const char *addr, int64_t estride, int vec
 template <class T, int VEC>
 OCH_D void store_pack(const Pack<T, VEC> &p, char *addr, int64_t estride, int vec)
 {
-   if (vec) *reinterpret_cast<Pack<T, VEC> *>(addr) = p;
+   if (vec) store_wide<T, VEC>(p, addr);
    else
    {
 #pragma unroll
@@ -179,6 +211,142 @@ __global__ __launch_bounds__(OCH_EW_BLOCK) void ew1_kernel(const EwParams<1> p, 
 #pragma unroll
          for (int k = 0; k < VEC; k++) r.v[k] = F::f(r.v[k], p.group0 + (uint64_t)g * VEC + k, prm);
          store_pack<R, VEC>(r, p.ptr[0] + off[0], p.estride[0], FAST || p.vecmode[0]);
+      }
+   }
+}
+
+
+/* ---- tiled kernels for transposed operands ----------------------------------
+   When an input is contiguous along a dimension other than the output's fastest one (a
+   transposed view), reading it in output order touches one element per cache line. These
+   kernels work on TILE x TILE blocks of (dimension 0, dimension d1): such an input is read
+   with 128-bit loads along d1, parked transposed in LDS, and then consumed in output order;
+   the other operands are accessed directly along dimension 0. */
+#define OCH_TILE_THREADS 256
+template <int NOPS> struct TileParams
+{
+   char    *ptr[NOPS];
+   int64_t  s0[NOPS], s1[NOPS];             /* byte strides along dimension 0 and along d1 */
+   int64_t  so[NOPS][OCH_MAX_DIMS];         /* byte strides of the remaining (outer) dimensions */
+   FastDiv  odiv[OCH_MAX_DIMS];
+   uint32_t n0, n1;                         /* extents of dimension 0 and d1 */
+   int      nouter;
+   int      trans[NOPS];                    /* read through LDS */
+   int      vecmode[NOPS];                  /* direct access may use VEC-wide loads/stores */
+   int      lds_off[NOPS];                  /* byte offset of the operand's LDS tile */
+};
+
+constexpr int tile_dim(size_t maxsize) { return maxsize >= 16 ? 32 : 64; }
+template <class T> constexpr int tile_pitch(int tile) { return tile + (sizeof(T) >= 4 ? 1 : 4 / (int)sizeof(T)); }
+template <class T> constexpr int tile_bytes(int tile) { return ((tile * tile_pitch<T>(tile) * (int)sizeof(T)) + 15) / 16 * 16; }
+
+template <class T, int TILE>
+OCH_D void tile_stage(T *lds, const char *base, int64_t s0, uint32_t n0, uint32_t n1)
+{
+   constexpr int VK = vec_for_c<T>();
+   constexpr int LPR = TILE / VK;                        /* lanes per row (fixed index along dimension 0) */
+   constexpr int RPP = OCH_TILE_THREADS / LPR;           /* rows per pass */
+   constexpr int PASSES = (TILE + RPP - 1) / RPP;
+   constexpr int PITCH = tile_pitch<T>(TILE);
+   const uint32_t i1 = (threadIdx.x % LPR) * VK, row = threadIdx.x / LPR;
+   Pack<T, VK> v[PASSES];
+#pragma unroll
+   for (int u = 0; u < PASSES; u++)
+   {  uint32_t i0 = row + u * RPP;
+      if (i0 < n0 && i1 < n1) load_wide<T, VK>(v[u], base + (int64_t)i0 * s0 + (int64_t)i1 * (int64_t)sizeof(T));
+   }
+#pragma unroll
+   for (int u = 0; u < PASSES; u++)
+   {  uint32_t i0 = row + u * RPP;
+      if (i0 < n0 && i1 < n1)
+      {
+#pragma unroll
+         for (int j = 0; j < VK; j++) lds[(i1 + j) * PITCH + i0] = v[u].v[j];
+      }
+   }
+}
+
+template <int NOPS>
+OCH_D void tile_origin(const TileParams<NOPS> &p, int tile, int64_t (&off)[NOPS])
+{
+   uint32_t q = blockIdx.z;
+#pragma unroll
+   for (int k = 0; k < NOPS; k++)
+      off[k] = (int64_t)blockIdx.x * tile * p.s0[k] + (int64_t)blockIdx.y * tile * p.s1[k];
+   for (int d = 0; d < p.nouter; d++)
+   {  uint32_t q2 = fastdiv(q, p.odiv[d]);
+      uint32_t i = q - q2 * p.odiv[d].d; q = q2;
+#pragma unroll
+      for (int k = 0; k < NOPS; k++) off[k] += (int64_t)i * p.so[k][d];
+   }
+}
+
+template <class F, int VEC>
+__global__ __launch_bounds__(OCH_TILE_THREADS) void ew3_tile_kernel(const TileParams<3> p)
+{
+   typedef typename F::A A; typedef typename F::B B; typedef typename F::R R;
+   constexpr size_t MAXS = sizeof(A) > sizeof(B) ? (sizeof(A) > sizeof(R) ? sizeof(A) : sizeof(R)) : (sizeof(B) > sizeof(R) ? sizeof(B) : sizeof(R));
+   constexpr int TILE = tile_dim(MAXS);
+   extern __shared__ __align__(16) char och_tile_lds[];
+   A *la = reinterpret_cast<A *>(och_tile_lds + p.lds_off[0]);
+   B *lb = reinterpret_cast<B *>(och_tile_lds + p.lds_off[1]);
+   int64_t off[3];
+   tile_origin<3>(p, TILE, off);
+   const uint32_t r0 = p.n0 - blockIdx.x * TILE, r1 = p.n1 - blockIdx.y * TILE;
+   const uint32_t n0 = r0 < (uint32_t)TILE ? r0 : TILE, n1 = r1 < (uint32_t)TILE ? r1 : TILE;
+   if (p.trans[0]) tile_stage<A, TILE>(la, p.ptr[0] + off[0], p.s0[0], n0, n1);
+   if (p.trans[1]) tile_stage<B, TILE>(lb, p.ptr[1] + off[1], p.s0[1], n0, n1);
+   __syncthreads();
+   constexpr int LPC = TILE / VEC, CPP = OCH_TILE_THREADS / LPC, PASSES = (TILE + CPP - 1) / CPP;
+   const uint32_t i0 = (threadIdx.x % LPC) * VEC, col = threadIdx.x / LPC;
+#pragma unroll
+   for (int u = 0; u < PASSES; u++)
+   {  uint32_t i1 = col + u * CPP;
+      if (i0 < n0 && i1 < n1)
+      {  Pack<A, VEC> a; Pack<B, VEC> b; Pack<R, VEC> r;
+         if (p.trans[0])
+         {
+#pragma unroll
+            for (int k = 0; k < VEC; k++) a.v[k] = la[i1 * tile_pitch<A>(TILE) + i0 + k];
+         }
+         else load_pack<A, VEC>(a, p.ptr[0] + off[0] + (int64_t)i0 * p.s0[0] + (int64_t)i1 * p.s1[0], p.s0[0], p.vecmode[0]);
+         if (p.trans[1])
+         {
+#pragma unroll
+            for (int k = 0; k < VEC; k++) b.v[k] = lb[i1 * tile_pitch<B>(TILE) + i0 + k];
+         }
+         else load_pack<B, VEC>(b, p.ptr[1] + off[1] + (int64_t)i0 * p.s0[1] + (int64_t)i1 * p.s1[1], p.s0[1], p.vecmode[1]);
+#pragma unroll
+         for (int k = 0; k < VEC; k++) r.v[k] = F::f(a.v[k], b.v[k]);
+         store_pack<R, VEC>(r, p.ptr[2] + off[2] + (int64_t)i0 * p.s0[2] + (int64_t)i1 * p.s1[2], p.s0[2], p.vecmode[2]);
+      }
+   }
+}
+
+template <class F, int VEC>
+__global__ __launch_bounds__(OCH_TILE_THREADS) void ew2_tile_kernel(const TileParams<2> p)
+{
+   typedef typename F::A A; typedef typename F::R R;
+   constexpr size_t MAXS = sizeof(A) > sizeof(R) ? sizeof(A) : sizeof(R);
+   constexpr int TILE = tile_dim(MAXS);
+   extern __shared__ __align__(16) char och_tile_lds[];
+   A *la = reinterpret_cast<A *>(och_tile_lds);
+   int64_t off[2];
+   tile_origin<2>(p, TILE, off);
+   const uint32_t r0 = p.n0 - blockIdx.x * TILE, r1 = p.n1 - blockIdx.y * TILE;
+   const uint32_t n0 = r0 < (uint32_t)TILE ? r0 : TILE, n1 = r1 < (uint32_t)TILE ? r1 : TILE;
+   tile_stage<A, TILE>(la, p.ptr[0] + off[0], p.s0[0], n0, n1);
+   __syncthreads();
+   constexpr int LPC = TILE / VEC, CPP = OCH_TILE_THREADS / LPC, PASSES = (TILE + CPP - 1) / CPP;
+   const uint32_t i0 = (threadIdx.x % LPC) * VEC, col = threadIdx.x / LPC;
+#pragma unroll
+   for (int u = 0; u < PASSES; u++)
+   {  uint32_t i1 = col + u * CPP;
+      if (i0 < n0 && i1 < n1)
+      {  Pack<R, VEC> r;
+#pragma unroll
+         for (int k = 0; k < VEC; k++) r.v[k] = F::f(la[i1 * tile_pitch<A>(TILE) + i0 + k]);
+         store_pack<R, VEC>(r, p.ptr[1] + off[1] + (int64_t)i0 * p.s0[1] + (int64_t)i1 * p.s1[1], p.s0[1], p.vecmode[1]);
       }
    }
 }
@@ -354,6 +522,56 @@ static int ew_dispatch(const EwShape<NOPS> &s, uint64_t flat0, int vec, const in
    return 0;
 }
 
+
+/* Decide whether a normalised shape should run on the tiled kernels and fill their parameters.
+   The output (last operand) must have unit stride along dimension 0; the inputs that are
+   contiguous along one other dimension d1 (and strided along dimension 0) go through LDS. */
+template <int NOPS>
+static bool ew_tile_params(TileParams<NOPS> &t, const EwShape<NOPS> &s, const int (&es)[NOPS], int tile, int vec,
+                           dim3 &grid, size_t &lds_bytes, const int (&tilebytes)[NOPS])
+{
+   const int out = NOPS - 1;
+   if (s.ndims < 2 || s.stride[out][0] != es[out]) return false;
+   if (s.size[0] % vec != 0 || s.size[0] < 16) return false;
+   auto is_trans = [&](int k, int d)
+   {  return s.stride[k][d] == es[k] && s.stride[k][0] != es[k] && s.stride[k][0] != 0; };
+   int d1 = -1;
+   for (int d = 1; d < s.ndims && d1 < 0; d++)
+      for (int k = 0; k < out; k++) if (is_trans(k, d)) { d1 = d; break; }
+   if (d1 < 0 || s.size[d1] < 16) return false;
+   memset(&t, 0, sizeof(t));
+   bool any = false; size_t lds = 0;
+   for (int k = 0; k < NOPS; k++)
+   {  t.ptr[k] = s.ptr[k]; t.s0[k] = s.stride[k][0]; t.s1[k] = s.stride[k][d1];
+      bool tr = (k != out) && is_trans(k, d1);
+      if (tr)
+      {  int vk = 16 / es[k]; if (vk < 1) vk = 1;
+         if (s.size[d1] % vk != 0 || ((uintptr_t)s.ptr[k]) % 16 != 0) tr = false;
+         for (int d = 0; d < s.ndims && tr; d++) if (d != d1 && s.stride[k][d] % 16 != 0) tr = false;
+      }
+      t.trans[k] = tr ? 1 : 0;
+      if (tr) { any = true; t.lds_off[k] = (int)lds; lds += tilebytes[k]; }
+      int width = es[k] * vec; if (width > 16) width = 16;
+      bool v = (s.stride[k][0] == es[k]) && (((uintptr_t)s.ptr[k]) % width == 0);
+      for (int d = 1; d < s.ndims && v; d++) if (s.stride[k][d] % width != 0) v = false;
+      t.vecmode[k] = v ? 1 : 0;
+   }
+   if (!any || lds > 64 * 1024) return false;
+   uint64_t outer = 1; t.nouter = 0;
+   for (int d = 1; d < s.ndims; d++)
+   {  if (d == d1) continue;
+      t.odiv[t.nouter] = make_fastdiv((uint32_t)s.size[d]);
+      for (int k = 0; k < NOPS; k++) t.so[k][t.nouter] = s.stride[k][d];
+      t.nouter++; outer *= s.size[d];
+   }
+   uint64_t tiles0 = (s.size[0] + tile - 1) / tile, tiles1 = (s.size[d1] + tile - 1) / tile;
+   if (outer > 65535 || tiles1 > 65535 || tiles0 > 0x7FFFFFFFull) return false;
+   t.n0 = (uint32_t)s.size[0]; t.n1 = (uint32_t)s.size[d1];
+   grid = dim3((unsigned)tiles0, (unsigned)tiles1, (unsigned)outer);
+   lds_bytes = lds;
+   return true;
+}
+
 template <class F>
 static int launch_ew3(int ndims, const size_t *size,
                       const ptrdiff_t *st1, void *p1, const ptrdiff_t *st2, void *p2,
@@ -366,7 +584,16 @@ static int launch_ew3(int ndims, const size_t *size,
    if (ew_normalize<3>(shape, ndims, size, strides, ptrs, 2, true) != 0) return -1;
    const int es[3] = { (int)sizeof(A), (int)sizeof(B), (int)sizeof(R) };
    return ew_launch_chunked<3>(shape, 0, [&](const EwShape<3> &s, uint64_t flat0) -> int
-   {  return ew_dispatch<3>(s, flat0, VEC, es,
+   {  constexpr size_t MAXS = sizeof(A) > sizeof(B) ? (sizeof(A) > sizeof(R) ? sizeof(A) : sizeof(R)) : (sizeof(B) > sizeof(R) ? sizeof(B) : sizeof(R));
+      constexpr int TILE = tile_dim(MAXS);
+      const int tb[3] = { tile_bytes<A>(TILE), tile_bytes<B>(TILE), 0 };
+      TileParams<3> tp; dim3 grid; size_t lds;
+      if (ew_tile_params<3>(tp, s, es, TILE, VEC, grid, lds, tb))
+      {  hipLaunchKernelGGL((ew3_tile_kernel<F, VEC>), grid, dim3(OCH_TILE_THREADS), lds, stream, tp);
+         OCH_CHECK_LAUNCH();
+         return 0;
+      }
+      return ew_dispatch<3>(s, flat0, VEC, es,
          [&](const EwParams<3> &p, uint32_t blocks)
          {  hipLaunchKernelGGL((ew3_kernel<F, VEC, OCH_EW_UNR, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
          [&](const EwParams<3> &p, uint32_t blocks)
@@ -387,7 +614,16 @@ static int launch_ew2(int ndims, const size_t *size,
    if (ew_normalize<2>(shape, ndims, size, strides, ptrs, 1, true) != 0) return -1;
    const int es[2] = { (int)sizeof(A), (int)sizeof(R) };
    return ew_launch_chunked<2>(shape, 0, [&](const EwShape<2> &s, uint64_t flat0) -> int
-   {  return ew_dispatch<2>(s, flat0, VEC, es,
+   {  constexpr size_t MAXS = sizeof(A) > sizeof(R) ? sizeof(A) : sizeof(R);
+      constexpr int TILE = tile_dim(MAXS);
+      const int tb[2] = { tile_bytes<A>(TILE), 0 };
+      TileParams<2> tp; dim3 grid; size_t lds;
+      if (ew_tile_params<2>(tp, s, es, TILE, VEC, grid, lds, tb))
+      {  hipLaunchKernelGGL((ew2_tile_kernel<F, VEC>), grid, dim3(OCH_TILE_THREADS), lds, stream, tp);
+         OCH_CHECK_LAUNCH();
+         return 0;
+      }
+      return ew_dispatch<2>(s, flat0, VEC, es,
          [&](const EwParams<2> &p, uint32_t blocks)
          {  hipLaunchKernelGGL((ew2_kernel<F, VEC, OCH_EW_UNR, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
          [&](const EwParams<2> &p, uint32_t blocks)

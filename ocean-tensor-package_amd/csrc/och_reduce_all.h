@@ -64,6 +64,7 @@ struct RedParams
 {
    EwParams<1> ew;             /* source layout; ew.ngroups unused when flat */
    uint64_t ngroups;           /* total groups (VEC elements each) */
+   uint64_t per_block;         /* groups per block: block b reduces the contiguous range starting at b * per_block */
    char *partials;             /* OCH_RED_MAX_BLOCKS slots */
    unsigned int *counter;      /* ticket counter, zero on entry, zero again on exit */
    void *result;
@@ -71,39 +72,51 @@ struct RedParams
    int   ntail;
 };
 
-template <class RD, class T, int VEC>
+/* WIDE: flat, unit-stride, aligned source read with VEC-wide loads (compile-time, so that the
+   loads stay single 128-bit instructions); otherwise VEC is 1 and any layout is accepted. */
+template <class RD, class T, int VEC, bool WIDE>
 __global__ __launch_bounds__(OCH_RED_BLOCK) void reduce_all_kernel(const RedParams p, const typename RD::Param prm)
 {
    typedef typename RD::Acc Acc;
    __shared__ Acc lds[OCH_RED_BLOCK / 64];
    __shared__ unsigned int ticket;
-   Acc acc = RD::identity();
-   const uint64_t stride = (uint64_t)gridDim.x * OCH_RED_BLOCK;
-   uint64_t g = (uint64_t)blockIdx.x * OCH_RED_BLOCK + threadIdx.x;
-   const bool flat = (p.ew.ndims == 1);
-   /* main loop: OCH_RED_UNR groups per trip, loads first */
-   for (; g + (OCH_RED_UNR - 1) * stride < p.ngroups; g += OCH_RED_UNR * stride)
+   Acc part[OCH_RED_UNR];
+#pragma unroll
+   for (int u = 0; u < OCH_RED_UNR; u++) part[u] = RD::identity();
+   /* every block walks one contiguous range of groups, OCH_RED_BLOCK groups per step, so that
+      the loads in flight stay close together in memory (a grid-wide stride is a large power of
+      two and lands the concurrent loads on the same memory channels) */
+   const uint64_t stride = OCH_RED_BLOCK;
+   uint64_t g = (uint64_t)blockIdx.x * p.per_block + threadIdx.x;
+   uint64_t end = (uint64_t)blockIdx.x * p.per_block + p.per_block;
+   if (end > p.ngroups) end = p.ngroups;
+   const bool flat = WIDE || (p.ew.ndims == 1);
+   /* main loop: OCH_RED_UNR independent groups per trip, loads first, one accumulator per group */
+   for (; g + (OCH_RED_UNR - 1) * stride < end; g += OCH_RED_UNR * stride)
    {  Pack<T, VEC> v[OCH_RED_UNR];
 #pragma unroll
       for (int u = 0; u < OCH_RED_UNR; u++)
       {  int64_t off[1];
          if (flat) off[0] = (int64_t)(g + u * stride) * p.ew.gstride[0];
          else group_offsets<1>(p.ew, (uint32_t)(g + u * stride), off);
-         load_pack<T, VEC>(v[u], p.ew.ptr[0] + off[0], p.ew.estride[0], p.ew.vecmode[0]);
+         load_pack<T, VEC>(v[u], p.ew.ptr[0] + off[0], p.ew.estride[0], WIDE);
       }
 #pragma unroll
-      for (int u = 0; u < OCH_RED_UNR; u++)
+      for (int k = 0; k < VEC; k++)
 #pragma unroll
-         for (int k = 0; k < VEC; k++) acc = RD::combine(acc, RD::load(v[u].v[k], prm));
+         for (int u = 0; u < OCH_RED_UNR; u++) part[u] = RD::combine(part[u], RD::load(v[u].v[k], prm));
    }
-   for (; g < p.ngroups; g += stride)
+   for (; g < end; g += stride)
    {  Pack<T, VEC> v; int64_t off[1];
       if (flat) off[0] = (int64_t)g * p.ew.gstride[0];
       else group_offsets<1>(p.ew, (uint32_t)g, off);
-      load_pack<T, VEC>(v, p.ew.ptr[0] + off[0], p.ew.estride[0], p.ew.vecmode[0]);
+      load_pack<T, VEC>(v, p.ew.ptr[0] + off[0], p.ew.estride[0], WIDE);
 #pragma unroll
-      for (int k = 0; k < VEC; k++) acc = RD::combine(acc, RD::load(v.v[k], prm));
+      for (int k = 0; k < VEC; k++) part[0] = RD::combine(part[0], RD::load(v.v[k], prm));
    }
+   Acc acc = part[0];
+#pragma unroll
+   for (int u = 1; u < OCH_RED_UNR; u++) acc = RD::combine(acc, part[u]);
    if (blockIdx.x == 0 && (int)threadIdx.x < p.ntail)
       acc = RD::combine(acc, RD::load(*reinterpret_cast<const T *>(p.tail + (int64_t)threadIdx.x * p.ew.estride[0]), prm));
    acc = block_reduce<RD>(acc, lds);
@@ -158,24 +171,21 @@ static int launch_reduce_all(int ndims, const size_t *size, const ptrdiff_t *str
    memset(&p, 0, sizeof(p));
    constexpr int VEC = vec_for<T>();
    const int es[1] = { (int)sizeof(T) };
-   int vec = 1;
+   bool wide_launch = false;
    if (shape.nelem > 0)
-   {  EwShape<1> s32 = shape;                     /* ew_params works on 32-bit group counts: fill by hand when flat */
-      if (shape.ndims == 1)
+   {  if (shape.ndims == 1)
       {  uint64_t n = shape.size[0];
-         bool wide = (VEC > 1) && (n >= (uint64_t)VEC) && (shape.stride[0][0] == (int64_t)sizeof(T)) &&
-                     (((uintptr_t)shape.ptr[0]) % (sizeof(T) * VEC > 16 ? 16 : sizeof(T) * VEC) == 0);
-         vec = wide ? VEC : 1;
-         p.ntail = (int)(n % vec);
-         p.tail = shape.ptr[0] + (int64_t)(n - n % vec) * shape.stride[0][0];
+         constexpr size_t width = (sizeof(T) * VEC > 16) ? 16 : sizeof(T) * VEC;
+         wide_launch = (n >= (uint64_t)VEC) && (shape.stride[0][0] == (int64_t)sizeof(T)) && (((uintptr_t)shape.ptr[0]) % width == 0);
+         int vec = wide_launch ? VEC : 1;
          p.ew.ndims = 1; p.ew.ptr[0] = shape.ptr[0];
          p.ew.estride[0] = shape.stride[0][0]; p.ew.gstride[0] = shape.stride[0][0] * vec;
-         p.ew.vecmode[0] = wide ? 1 : ((shape.stride[0][0] == (int64_t)sizeof(T)) && (((uintptr_t)shape.ptr[0]) % alignof(Pack<T, 1>) == 0));
          p.ngroups = n / vec;
+         p.ntail = (int)(n % vec);
+         p.tail = shape.ptr[0] + (int64_t)(n - n % vec) * shape.stride[0][0];
       }
       else
-      {  vec = (VEC > 1 && ew_params<1>(p.ew, s32, VEC, es, 0)) ? VEC : 1;
-         if (vec == 1) ew_params<1>(p.ew, s32, 1, es, 0);
+      {  ew_params<1>(p.ew, shape, 1, es, 0);
          p.ngroups = p.ew.ngroups;
       }
    }
@@ -185,8 +195,12 @@ static int launch_reduce_all(int ndims, const size_t *size, const ptrdiff_t *str
    if (zero_counter) OCH_CHECK_HIP(hipMemsetAsync(p.counter, 0, sizeof(unsigned int), stream));
    uint64_t want = (p.ngroups + (uint64_t)OCH_RED_BLOCK * OCH_RED_UNR - 1) / ((uint64_t)OCH_RED_BLOCK * OCH_RED_UNR);
    unsigned int blocks = (unsigned int)(want < 1 ? 1 : (want > OCH_RED_MAX_BLOCKS ? OCH_RED_MAX_BLOCKS : want));
-   if (vec > 1) hipLaunchKernelGGL((reduce_all_kernel<RD, T, VEC>), dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
-   else         hipLaunchKernelGGL((reduce_all_kernel<RD, T, 1>),   dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
+   {  const uint64_t step = (uint64_t)OCH_RED_BLOCK * OCH_RED_UNR;
+      uint64_t per = (p.ngroups + blocks - 1) / blocks;
+      p.per_block = (per + step - 1) / step * step;
+   }
+   if (wide_launch) hipLaunchKernelGGL((reduce_all_kernel<RD, T, VEC, true>), dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
+   else             hipLaunchKernelGGL((reduce_all_kernel<RD, T, 1, false>),  dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
    OCH_CHECK_LAUNCH();
    return 0;
 }
