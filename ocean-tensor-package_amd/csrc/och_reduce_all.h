@@ -2,12 +2,19 @@
  *
  * Replaces the reference's accumulate + finalize kernel pair followed by a blocking copy
  * (solid/include/solid/core/gpu/reduce_all.h:136-274,365-414). One kernel:
- *   grid-stride loop with <=128-bit loads, four independent loads in flight per thread
- *   -> 64-lane butterfly (shuffle) inside each wave -> LDS combine of the block's waves
- *   -> one partial per block in a scratch buffer -> the block that takes the last ticket
- *   (atomic counter) folds all partials in index order and writes the result.
+ *   every block streams one contiguous range with <=128-bit loads, four independent loads in
+ *   flight per thread -> 64-lane butterfly (shuffle) inside each wave -> LDS combine of the
+ *   block's waves -> one partial per block in a scratch buffer -> the block that takes the last
+ *   ticket (atomic counter) folds all partials in index order and writes the result.
  * The fold order depends only on the launch geometry, so results are reproducible run to run.
  * The result pointer may be device memory or device-visible pinned host memory.
+ *
+ * Cross-block hand-over: partials are written and read with relaxed agent-scope atomics (they
+ * bypass the per-XCD L2, which is not coherent between XCDs), the writer waits for its stores
+ * to complete and then takes its ticket with a relaxed agent-scope atomic add. A full
+ * agent-scope fence per block (L2 write-back + invalidate) serialises at ~30 ns per block and
+ * was measured to halve the streaming rate; the ticket itself costs ~5 ns per block, which is
+ * why the grid is capped at two blocks per compute unit.
  */
 #pragma once
 #include "och_elemwise.h"
@@ -18,7 +25,7 @@ namespace och {
 
 #define OCH_RED_BLOCK 256
 #define OCH_RED_UNR 4
-#define OCH_RED_MAX_BLOCKS 2048
+#define OCH_RED_MAX_BLOCKS 512
 #define OCH_RED_SLOT 16                               /* bytes per partial */
 #define OCH_RED_SCRATCH (OCH_RED_MAX_BLOCKS * OCH_RED_SLOT + 256)
 
@@ -33,14 +40,26 @@ template <class A> OCH_D A shfl_xor_any(A v, int mask)
    return u.a;
 }
 
-/* read an accumulator that another workgroup wrote: word-wise volatile loads */
+/* read / write an accumulator shared between workgroups: word-wise relaxed agent-scope atomics */
 template <class A> OCH_D A load_shared_global(const char *addr)
 {
    constexpr int NW = (sizeof(A) + 3) / 4;
    union { A a; unsigned int w[NW]; } u;
 #pragma unroll
-   for (int i = 0; i < NW; i++) u.w[i] = reinterpret_cast<const volatile unsigned int *>(addr)[i];
+   for (int i = 0; i < NW; i++)
+      u.w[i] = __hip_atomic_load(reinterpret_cast<const unsigned int *>(addr) + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
    return u.a;
+}
+template <class A> OCH_D void store_shared_global(char *addr, const A &a)
+{
+   constexpr int NW = (sizeof(A) + 3) / 4;
+   union { A a; unsigned int w[NW]; } u;
+#pragma unroll
+   for (int i = 0; i < NW; i++) u.w[i] = 0;
+   u.a = a;
+#pragma unroll
+   for (int i = 0; i < NW; i++)
+      __hip_atomic_store(reinterpret_cast<unsigned int *>(addr) + i, u.w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 /* reduce across the 256 threads of a block; the result is valid in thread 0 */
@@ -121,14 +140,13 @@ __global__ __launch_bounds__(OCH_RED_BLOCK) void reduce_all_kernel(const RedPara
       acc = RD::combine(acc, RD::load(*reinterpret_cast<const T *>(p.tail + (int64_t)threadIdx.x * p.ew.estride[0]), prm));
    acc = block_reduce<RD>(acc, lds);
    if (threadIdx.x == 0)
-   {  *reinterpret_cast<Acc *>(p.partials + (size_t)blockIdx.x * OCH_RED_SLOT) = acc;
-      __threadfence();
-      ticket = atomicAdd(p.counter, 1u);
+   {  store_shared_global<Acc>(p.partials + (size_t)blockIdx.x * OCH_RED_SLOT, acc);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");            /* the write-through stores above have completed */
+      ticket = __hip_atomic_fetch_add(p.counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
    }
    __syncthreads();
    if (ticket != gridDim.x - 1) return;
-   /* last block: fold the partials in index order */
-   __threadfence();
+   /* last block: every partial is in memory; fold them in index order */
    acc = RD::identity();
    for (unsigned int b = threadIdx.x; b < gridDim.x; b += OCH_RED_BLOCK)
       acc = RD::combine(acc, load_shared_global<Acc>(p.partials + (size_t)b * OCH_RED_SLOT));

@@ -4,7 +4,8 @@
  * their host-side planner (solid/src/core/gpu/op/reduce_axis.c:22-315). Two kernel shapes:
  *   thread-per-output  : neighbouring threads own neighbouring outputs; used when the outer
  *                        dimension is the fast one in memory, so every load instruction of a
- *                        wave is contiguous; four loads in flight per thread
+ *                        wave is contiguous; eight loads in flight per thread, and four waves
+ *                        share each group of 64 outputs when there are few outputs
  *   group-per-output   : a wave (64) or a block (256) strides over the reduced range of one
  *                        output and combines with a shuffle butterfly (+ LDS for blocks); used
  *                        when the reduced dimension is the fast one in memory
@@ -45,31 +46,67 @@ OCH_D int64_t axis_row_offset(const AxisParams &p, uint32_t r)
    return off;
 }
 
-template <class RD, class T>
+/* Neighbouring threads own neighbouring outputs: VEC consecutive outputs each (one 128-bit load
+   covers them; needs unit source stride along the first outer dimension). SPLIT slices (waves
+   when SPLIT is 4) share each output: slice s takes elements s, s + SPLIT, ... of every row of
+   the reduced range and the slices are folded through LDS in slice order. */
+template <class RD, class T, int SPLIT, int VEC>
 __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, const typename RD::Param prm)
 {
    typedef typename RD::Acc Acc;
-   uint32_t o = blockIdx.x * 256 + threadIdx.x;
-   if (o >= p.nout) return;
-   int64_t o1, o2;
-   axis_outer_offsets(p, o, o1, o2);
-   const char *base = p.src + o1;
-   Acc acc = RD::identity();
-   const int64_t s0 = p.rst[0];
-   for (uint32_t r = 0; r < p.rrows; r++)
-   {  const char *row = base + axis_row_offset(p, r);
-      uint32_t i = 0;
-      for (; i + 4 <= p.rsize0; i += 4)
-      {  T v0 = *reinterpret_cast<const T *>(row + (int64_t)(i + 0) * s0);
-         T v1 = *reinterpret_cast<const T *>(row + (int64_t)(i + 1) * s0);
-         T v2 = *reinterpret_cast<const T *>(row + (int64_t)(i + 2) * s0);
-         T v3 = *reinterpret_cast<const T *>(row + (int64_t)(i + 3) * s0);
-         acc = RD::combine(acc, RD::load(v0, prm)); acc = RD::combine(acc, RD::load(v1, prm));
-         acc = RD::combine(acc, RD::load(v2, prm)); acc = RD::combine(acc, RD::load(v3, prm));
+   constexpr int OPB = 256 / SPLIT;                 /* output groups per block */
+   constexpr int UNR = (VEC > 1) ? 4 : 8;
+   __shared__ Acc lds[SPLIT > 1 ? 256 * VEC : 1];
+   const uint32_t slice = threadIdx.x / OPB, ol = threadIdx.x % OPB;
+   const uint32_t o = (blockIdx.x * OPB + ol) * VEC;
+   const bool active = o < p.nout;
+   Acc acc[VEC];
+#pragma unroll
+   for (int k = 0; k < VEC; k++) acc[k] = RD::identity();
+   int64_t o1 = 0, o2 = 0;
+   if (active)
+   {  axis_outer_offsets(p, o, o1, o2);
+      const char *base = p.src + o1;
+      const int64_t s0 = p.rst[0];
+      for (uint32_t r = 0; r < p.rrows; r++)
+      {  const char *row = base + ((p.rd > 1) ? axis_row_offset(p, r) : 0);
+         uint32_t i = slice;
+         for (; i + (UNR - 1) * SPLIT < p.rsize0; i += UNR * SPLIT)
+         {  Pack<T, VEC> v[UNR];
+#pragma unroll
+            for (int u = 0; u < UNR; u++) load_wide<T, VEC>(v[u], row + (int64_t)(i + u * SPLIT) * s0);
+#pragma unroll
+            for (int u = 0; u < UNR; u++)
+#pragma unroll
+               for (int k = 0; k < VEC; k++) acc[k] = RD::combine(acc[k], RD::load(v[u].v[k], prm));
+         }
+         for (; i < p.rsize0; i += SPLIT)
+         {  Pack<T, VEC> v;
+            load_wide<T, VEC>(v, row + (int64_t)i * s0);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) acc[k] = RD::combine(acc[k], RD::load(v.v[k], prm));
+         }
       }
-      for (; i < p.rsize0; i++) acc = RD::combine(acc, RD::load(*reinterpret_cast<const T *>(row + (int64_t)i * s0), prm));
    }
-   *reinterpret_cast<typename RD::Res *>(p.dst + o2) = RD::finalize(acc, prm);
+   if constexpr (SPLIT > 1)
+   {
+#pragma unroll
+      for (int k = 0; k < VEC; k++) lds[k * 256 + threadIdx.x] = acc[k];
+      __syncthreads();
+      if (slice == 0)
+      {
+#pragma unroll
+         for (int s2 = 1; s2 < SPLIT; s2++)
+#pragma unroll
+            for (int k = 0; k < VEC; k++) acc[k] = RD::combine(acc[k], lds[k * 256 + s2 * OPB + ol]);
+      }
+   }
+   if (active && slice == 0)
+   {
+#pragma unroll
+      for (int k = 0; k < VEC; k++)
+         *reinterpret_cast<typename RD::Res *>(p.dst + o2 + (int64_t)k * p.st2[0]) = RD::finalize(acc[k], prm);
+   }
 }
 
 /* GROUP threads cooperate on one output; GROUP is 64 (one wave) or 256 (the whole block) */
@@ -160,7 +197,23 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
    int64_t red_fast = (p.rd > 0) ? (p.rst[0] < 0 ? -p.rst[0] : p.rst[0]) : INT64_MAX;
    bool cooperative = (p.rd > 0) && ((red_fast < outer_fast) || (nout < 16384 && relem >= 256));
    if (!cooperative)
-      hipLaunchKernelGGL((axis_thread_kernel<RD, T>), dim3((p.nout + 255) / 256), dim3(256), 0, stream, p, prm);
+   {  /* VEC outputs per thread when the first outer dimension has unit source stride and
+         everything is 16-byte aligned; four waves per output group while there are few groups */
+      constexpr int VEC = vec_for<T>();
+      bool wide = (VEC > 1) && p.nd > 0 && p.st1[0] == (int64_t)sizeof(T) && (p.div[0].d % VEC == 0) && (((uintptr_t)p.src) % 16 == 0);
+      for (int d = 1; d < p.nd && wide; d++) if (p.st1[d] % 16 != 0) wide = false;
+      for (int d = 0; d < p.rd && wide; d++) if (p.rst[d] % 16 != 0) wide = false;
+      const uint64_t groups = wide ? nout / VEC : nout;
+      const bool split = groups < (1u << 20) && p.rsize0 >= 16;
+      if (wide && split)
+         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 4, VEC>), dim3((unsigned)((groups + 63) / 64)), dim3(256), 0, stream, p, prm);
+      else if (wide)
+         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, VEC>), dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, stream, p, prm);
+      else if (split)
+         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 4, 1>), dim3((p.nout + 63) / 64), dim3(256), 0, stream, p, prm);
+      else
+         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, 1>), dim3((p.nout + 255) / 256), dim3(256), 0, stream, p, prm);
+   }
    else if (relem <= 2048 && nout >= 1024)
       hipLaunchKernelGGL((axis_group_kernel<RD, T, 64>), dim3((p.nout + 3) / 4), dim3(256), 0, stream, p, prm);
    else
