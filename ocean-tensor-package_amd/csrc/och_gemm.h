@@ -1,0 +1,331 @@
+/* GEMM kernels for gfx950: C <- alpha * op(A) * op(B) + beta * C, column-major.
+ *
+ * Replaces the cuBLAS dispatch of src/core/gpu/op/tensor_blas_gpu.c:132-231 (float, double,
+ * cfloat, cdouble: MFMA kernels below) and the tiled integer kernels of
+ * solid/src/core/gpu/template_blas.cu:99-160 (bool, integers, half: the generic kernel).
+ *
+ * MFMA kernel: a block of four waves owns a (2*WM) x (2*WN) tile of C; each wave a WM x WN
+ * sub-tile made of v_mfma_f64_16x16x4_f64 / v_mfma_f32_32x32x2_f32 tiles held in registers.
+ * Per K step the block stages a (2*WM) x KT slab of op(A) and a KT x (2*WN) slab of op(B)
+ * through LDS in k-major order (As[k][m], Bs[k][n]); so both the "m/n-contiguous" and the
+ * "k-contiguous" (transposed) memory layouts end up in the same LDS layout and the inner loop
+ * does not depend on the transposition flags. Global loads of slab s+1 are issued before the
+ * MFMAs of slab s and written to the other LDS buffer afterwards (one barrier per slab).
+ * Complex types keep real and imaginary planes apart in LDS and use four real MFMAs per tile
+ * (the sign of imag(A) is flipped in a register for the real part; conjugation flips the
+ * sign when the plane is written).
+ */
+#pragma once
+#include "och_common.h"
+#include "och_dtypes.h"
+#include <string.h>
+
+namespace och {
+
+typedef double och_f64x4  __attribute__((ext_vector_type(4)));
+typedef float  och_f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int och_gu32x4 __attribute__((ext_vector_type(4)));
+
+/* One MFMA tile. Operands: lane l supplies A(row l % T, k = l / T) and B(k = l / T, col l % T);
+   accumulator register r of lane l is C(acc_row(l, r), l % T). */
+template <class R> struct Mfma;
+template <> struct Mfma<double>
+{  static constexpr int T = 16, TK = 4, NACC = 4;
+   typedef och_f64x4 Acc;
+   static __device__ __forceinline__ Acc mma(double a, double b, Acc c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+   static __device__ __forceinline__ int acc_row(int lane, int r) { return 4 * r + (lane >> 4); }
+};
+template <> struct Mfma<float>
+{  static constexpr int T = 32, TK = 2, NACC = 16;
+   typedef och_f32x16 Acc;
+   static __device__ __forceinline__ Acc mma(float a, float b, Acc c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
+   static __device__ __forceinline__ int acc_row(int lane, int r) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+};
+
+template <class R> struct GemmParams
+{
+   const char *A, *B; char *C;
+   int64_t  ldA, ldB, ldC;              /* in elements */
+   uint32_t M, N, K;
+   R        alpha[2], beta[2];          /* (re, im) when the scalars live in host memory */
+   const R *alpha_dev, *beta_dev;       /* non-null: read the scalar from device memory */
+   int      conjA, conjB;
+   uint32_t tiles_m, tiles_n;
+};
+
+#define OCH_GEMM_THREADS 256
+
+/* Moves a BMN x KT slab of an operand from global memory to registers (fetch) and from there
+   to its k-major LDS planes (stash). KC: the operand is contiguous along k in memory. */
+template <class R, bool CPLX, bool KC, bool EDGE, int BMN, int KT>
+struct SlabLoader
+{
+   static constexpr int NPL = CPLX ? 2 : 1;
+   static constexpr int ES = (int)sizeof(R) * NPL;
+   static constexpr int VE = 16 / ES;                              /* elements per 128-bit load */
+   static constexpr int NV = BMN * KT / VE / OCH_GEMM_THREADS;     /* loads per thread */
+   static_assert(NV >= 1 && (BMN * KT) % (VE * OCH_GEMM_THREADS) == 0, "slab does not divide among the threads");
+   R reg[NV][VE * NPL];
+
+   static __device__ __forceinline__ void where(int v, uint32_t &mn, uint32_t &k)
+   {  const uint32_t q = threadIdx.x + OCH_GEMM_THREADS * v;
+      if (!KC) { mn = (q % (BMN / VE)) * VE; k = q / (BMN / VE); }
+      else     { k = (q % (KT / VE)) * VE;   mn = q / (KT / VE); }
+   }
+   /* mat: operand origin; element (mn, k) of op(.) lives at mn + k * ld (!KC) or k + mn * ld (KC) */
+   __device__ __forceinline__ void fetch(const char *mat, int64_t ld, uint32_t mn0, uint32_t k0, uint32_t MN, uint32_t K)
+   {
+#pragma unroll
+      for (int v = 0; v < NV; v++)
+      {  uint32_t mn, k; where(v, mn, k);
+         const int64_t gm = (int64_t)mn0 + mn, gk = (int64_t)k0 + k;
+         if (!EDGE)
+         {  const char *addr = mat + (KC ? (gk + gm * ld) : (gm + gk * ld)) * ES;
+            och_gu32x4 raw = *reinterpret_cast<const och_gu32x4 *>(addr);
+            __builtin_memcpy(&reg[v][0], &raw, 16);
+         }
+         else
+         {
+#pragma unroll
+            for (int e = 0; e < VE; e++)
+            {  const int64_t em = gm + (KC ? 0 : e), ek = gk + (KC ? e : 0);
+               const bool ok = (em < (int64_t)MN) && (ek < (int64_t)K);
+               const R *src = reinterpret_cast<const R *>(mat + (KC ? (ek + em * ld) : (em + ek * ld)) * ES);
+#pragma unroll
+               for (int c = 0; c < NPL; c++) reg[v][e * NPL + c] = ok ? src[c] : (R)0;
+            }
+         }
+      }
+   }
+   /* planes: plane 0 of this operand in the current LDS buffer; row pitch in reals */
+   __device__ __forceinline__ void stash(R *planes, int pitch, bool conj) const
+   {
+#pragma unroll
+      for (int v = 0; v < NV; v++)
+      {  uint32_t mn, k; where(v, mn, k);
+#pragma unroll
+         for (int e = 0; e < VE; e++)
+         {  const uint32_t em = mn + (KC ? 0 : e), ek = k + (KC ? e : 0);
+            planes[ek * pitch + em] = reg[v][e * NPL];
+            if (CPLX) planes[(KT + ek) * pitch + em] = conj ? -reg[v][e * NPL + 1] : reg[v][e * NPL + 1];
+         }
+      }
+   }
+};
+
+template <class R, bool CPLX, bool AKC, bool BKC, bool EDGE, int WM, int WN, int KT>
+__global__ __launch_bounds__(OCH_GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmParams<R> p)
+{
+   typedef Mfma<R> MM;
+   typedef typename MM::Acc Acc;
+   constexpr int T = MM::T, TK = MM::TK;
+   constexpr int BM = 2 * WM, BN = 2 * WN, NPL = CPLX ? 2 : 1;
+   constexpr int TMS = WM / T, TNS = WN / T;
+   constexpr int PAD = 32 / (int)sizeof(R);
+   constexpr int PA = BM + PAD, PB = BN + PAD;
+   constexpr int BUF = NPL * KT * (PA + PB);
+   __shared__ __align__(16) R lds[2 * BUF];
+
+   const uint32_t tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
+   const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+   const int wm = (wave & 1) * WM, wn = (wave >> 1) * WN;
+
+   Acc acc[TMS][TNS], acci[CPLX ? TMS : 1][CPLX ? TNS : 1];
+#pragma unroll
+   for (int i = 0; i < TMS; i++)
+#pragma unroll
+      for (int j = 0; j < TNS; j++)
+      {
+#pragma unroll
+         for (int r = 0; r < MM::NACC; r++) { acc[i][j][r] = 0; if (CPLX) acci[i][j][r] = 0; }
+      }
+
+   SlabLoader<R, CPLX, AKC, EDGE, BM, KT> la;
+   SlabLoader<R, CPLX, BKC, EDGE, BN, KT> lb;
+   const uint32_t nslabs = (p.K + KT - 1) / KT;
+   if (nslabs > 0)
+   {  la.fetch(p.A, p.ldA, m0, 0, p.M, p.K);
+      lb.fetch(p.B, p.ldB, n0, 0, p.N, p.K);
+      la.stash(lds, PA, p.conjA);
+      lb.stash(lds + NPL * KT * PA, PB, p.conjB);
+   }
+   __syncthreads();
+   for (uint32_t s = 0; s < nslabs; s++)
+   {  const R *As = lds + (s & 1) * BUF, *Bs = As + NPL * KT * PA;
+      const bool more = s + 1 < nslabs;
+      if (more)
+      {  la.fetch(p.A, p.ldA, m0, (s + 1) * KT, p.M, p.K);
+         lb.fetch(p.B, p.ldB, n0, (s + 1) * KT, p.N, p.K);
+      }
+#pragma unroll
+      for (int ks = 0; ks < KT / TK; ks++)
+      {  const int k = ks * TK + lane / T;
+         R a[TMS], b[TNS], ai[CPLX ? TMS : 1], bi[CPLX ? TNS : 1];
+#pragma unroll
+         for (int i = 0; i < TMS; i++)
+         {  a[i] = As[k * PA + wm + i * T + lane % T];
+            if (CPLX) ai[i] = As[(KT + k) * PA + wm + i * T + lane % T];
+         }
+#pragma unroll
+         for (int j = 0; j < TNS; j++)
+         {  b[j] = Bs[k * PB + wn + j * T + lane % T];
+            if (CPLX) bi[j] = Bs[(KT + k) * PB + wn + j * T + lane % T];
+         }
+#pragma unroll
+         for (int i = 0; i < TMS; i++)
+#pragma unroll
+            for (int j = 0; j < TNS; j++)
+            {  acc[i][j] = MM::mma(a[i], b[j], acc[i][j]);
+               if (CPLX)
+               {  acc[i][j]  = MM::mma(-ai[i], bi[j], acc[i][j]);
+                  acci[i][j] = MM::mma(a[i], bi[j], acci[i][j]);
+                  acci[i][j] = MM::mma(ai[i], b[j], acci[i][j]);
+               }
+            }
+      }
+      if (more)
+      {  R *An = lds + ((s + 1) & 1) * BUF;
+         la.stash(An, PA, p.conjA);
+         lb.stash(An + NPL * KT * PA, PB, p.conjB);
+      }
+      __syncthreads();
+   }
+
+   /* epilogue */
+   R alr = p.alpha[0], ali = p.alpha[1], ber = p.beta[0], bei = p.beta[1];
+   if (p.alpha_dev) { alr = p.alpha_dev[0]; if (CPLX) ali = p.alpha_dev[1]; }
+   if (p.beta_dev)  { ber = p.beta_dev[0];  if (CPLX) bei = p.beta_dev[1]; }
+   const bool use_c = CPLX ? (ber != 0 || bei != 0) : (ber != 0);
+#pragma unroll
+   for (int i = 0; i < TMS; i++)
+#pragma unroll
+      for (int j = 0; j < TNS; j++)
+      {  const uint32_t col = n0 + wn + j * T + lane % T;
+#pragma unroll
+         for (int r = 0; r < MM::NACC; r++)
+         {  const uint32_t row = m0 + wm + i * T + MM::acc_row(lane, r);
+            if (EDGE && (row >= p.M || col >= p.N)) continue;
+            R *c = reinterpret_cast<R *>(p.C + ((int64_t)row + (int64_t)col * p.ldC) * (int64_t)(sizeof(R) * NPL));
+            if (!CPLX)
+            {  R v = alr * acc[i][j][r];
+               if (use_c) v += ber * c[0];
+               c[0] = v;
+            }
+            else
+            {  const R sr = acc[i][j][r], si = acci[i][j][r];
+               R vr = alr * sr - ali * si, vi = alr * si + ali * sr;
+               if (use_c) { const R cr = c[0], ci = c[1]; vr += ber * cr - bei * ci; vi += ber * ci + bei * cr; }
+               c[0] = vr; c[1] = vi;
+            }
+         }
+      }
+}
+
+/* Few outputs (dot products, tiny C): one block per element of C strides over K. Accumulates
+   in double; the four partial sums of the waves are folded in wave order. */
+template <class R, bool CPLX>
+__global__ __launch_bounds__(256) void gemm_dot_kernel(const GemmParams<R> p, int64_t sAm, int64_t sAk, int64_t sBk, int64_t sBn)
+{
+   constexpr int NPL = CPLX ? 2 : 1;
+   __shared__ double lds[8];
+   const uint32_t row = blockIdx.x % p.M, col = blockIdx.x / p.M;
+   const R *a = reinterpret_cast<const R *>(p.A) + (int64_t)row * sAm * NPL;
+   const R *b = reinterpret_cast<const R *>(p.B) + (int64_t)col * sBn * NPL;
+   double sr = 0, si = 0;
+   for (uint32_t k = threadIdx.x; k < p.K; k += 256)
+   {  const R *x = a + (int64_t)k * sAk * NPL, *y = b + (int64_t)k * sBk * NPL;
+      if (!CPLX) sr += (double)x[0] * (double)y[0];
+      else
+      {  const double xr = x[0], xi = p.conjA ? -(double)x[1] : (double)x[1];
+         const double yr = y[0], yi = p.conjB ? -(double)y[1] : (double)y[1];
+         sr += xr * yr - xi * yi; si += xr * yi + xi * yr;
+      }
+   }
+#pragma unroll
+   for (int m = 32; m >= 1; m >>= 1) { sr += __shfl_xor(sr, m, 64); if (CPLX) si += __shfl_xor(si, m, 64); }
+   if ((threadIdx.x & 63) == 0) { lds[(threadIdx.x >> 6) * 2] = sr; lds[(threadIdx.x >> 6) * 2 + 1] = si; }
+   __syncthreads();
+   if (threadIdx.x != 0) return;
+   sr = ((lds[0] + lds[2]) + lds[4]) + lds[6];
+   si = ((lds[1] + lds[3]) + lds[5]) + lds[7];
+   R alr = p.alpha[0], ali = p.alpha[1], ber = p.beta[0], bei = p.beta[1];
+   if (p.alpha_dev) { alr = p.alpha_dev[0]; if (CPLX) ali = p.alpha_dev[1]; }
+   if (p.beta_dev)  { ber = p.beta_dev[0];  if (CPLX) bei = p.beta_dev[1]; }
+   R *c = reinterpret_cast<R *>(p.C) + ((int64_t)row + (int64_t)col * p.ldC) * NPL;
+   if (!CPLX)
+   {  double v = (double)alr * sr;
+      if (ber != 0) v += (double)ber * (double)c[0];
+      c[0] = (R)v;
+   }
+   else
+   {  double vr = (double)alr * sr - (double)ali * si, vi = (double)alr * si + (double)ali * sr;
+      if (ber != 0 || bei != 0)
+      {  const double cr = c[0], ci = c[1];
+         vr += (double)ber * cr - (double)bei * ci; vi += (double)ber * ci + (double)bei * cr;
+      }
+      c[0] = (R)vr; c[1] = (R)vi;
+   }
+}
+
+/* host side ------------------------------------------------------------------ */
+struct GemmArgs
+{
+   char transA, transB;
+   size_t M, N, K;
+   const void *alpha, *beta;
+   const void *A, *B; void *C;
+   ptrdiff_t ldA, ldB, ldC;
+   int scalar_mode_host;
+   hipStream_t stream;
+};
+
+template <class R, bool CPLX, int WM, int WN, int KT>
+static int launch_gemm_mfma(const GemmArgs &g)
+{
+   constexpr int NPL = CPLX ? 2 : 1;
+   constexpr int ES = (int)sizeof(R) * NPL;
+   constexpr int BM = 2 * WM, BN = 2 * WN;
+   GemmParams<R> p;
+   memset(&p, 0, sizeof(p));
+   p.A = (const char *)g.A; p.B = (const char *)g.B; p.C = (char *)g.C;
+   p.ldA = g.ldA; p.ldB = g.ldB; p.ldC = g.ldC;
+   p.M = (uint32_t)g.M; p.N = (uint32_t)g.N; p.K = (uint32_t)g.K;
+   if (g.scalar_mode_host)
+   {  memcpy(p.alpha, g.alpha, ES); memcpy(p.beta, g.beta, ES); }
+   else
+   {  p.alpha_dev = (const R *)g.alpha; p.beta_dev = (const R *)g.beta; }
+   const bool akc = (g.transA != 'N'), bkc = (g.transB == 'N');
+   p.conjA = CPLX && (g.transA == 'C'); p.conjB = CPLX && (g.transB == 'C');
+
+   if (g.M * g.N <= 256 && g.K >= 64)
+   {  /* op(A)(m,k) = A[m*sAm + k*sAk], op(B)(k,n) = B[k*sBk + n*sBn] */
+      const int64_t sAm = akc ? g.ldA : 1, sAk = akc ? 1 : g.ldA, sBk = bkc ? 1 : g.ldB, sBn = bkc ? g.ldB : 1;
+      hipLaunchKernelGGL((gemm_dot_kernel<R, CPLX>), dim3((unsigned)(g.M * g.N)), dim3(256), 0, g.stream, p, sAm, sAk, sBk, sBn);
+      OCH_CHECK_LAUNCH();
+      return 0;
+   }
+   p.tiles_m = (uint32_t)((g.M + BM - 1) / BM); p.tiles_n = (uint32_t)((g.N + BN - 1) / BN);
+   const uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
+   if (blocks > 0x7FFFFFFFull) return set_error("gemm: too many tiles");
+   auto aligned = [&](const void *ptr, ptrdiff_t ld) { return ((uintptr_t)ptr % 16 == 0) && (((int64_t)ld * ES) % 16 == 0); };
+   const bool edge = !(g.M % BM == 0 && g.N % BN == 0 && g.K % KT == 0 && aligned(g.A, g.ldA) && aligned(g.B, g.ldB));
+   const dim3 grid((unsigned)blocks), block(OCH_GEMM_THREADS);
+#define OCH_GEMM_LAUNCH(AK, BK)                                                                             \
+   do { if (edge) hipLaunchKernelGGL((gemm_mfma_kernel<R, CPLX, AK, BK, true, WM, WN, KT>), grid, block, 0, g.stream, p);  \
+        else      hipLaunchKernelGGL((gemm_mfma_kernel<R, CPLX, AK, BK, false, WM, WN, KT>), grid, block, 0, g.stream, p); } while (0)
+   if (!akc && !bkc) OCH_GEMM_LAUNCH(false, false);
+   else if (!akc)    OCH_GEMM_LAUNCH(false, true);
+   else if (!bkc)    OCH_GEMM_LAUNCH(true, false);
+   else              OCH_GEMM_LAUNCH(true, true);
+#undef OCH_GEMM_LAUNCH
+   OCH_CHECK_LAUNCH();
+   return 0;
+}
+
+int gemm_float(const GemmArgs &g);
+int gemm_double(const GemmArgs &g);
+int gemm_cfloat(const GemmArgs &g);
+int gemm_cdouble(const GemmArgs &g);
+
+} /* namespace och */

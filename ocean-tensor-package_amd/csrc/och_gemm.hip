@@ -1,0 +1,161 @@
+/* och_gemm entry point, argument checks, and the generic tiled kernel for bool, integers and
+ * half (solid/src/core/gpu/template_blas.cu:99-160 uses one thread per element of C and a
+ * square LDS tile; here each thread owns a 4 x 4 patch of a 64 x 64 tile).
+ * bool: + is OR, * is AND. Integers wrap. half multiplies and accumulates in float. */
+#include "och_gemm.h"
+#include "../../include/ocean_hip.h"
+
+namespace och {
+
+template <class T> struct GemmElem;     /* W: LDS / accumulator type */
+template <class T, class WT> struct GemmInt
+{  typedef WT W;
+   static __device__ W load(T x) { return (W)x; }
+   static __device__ W fma(W s, W a, W b) { return (W)(s + a * b); }
+   static __device__ T finish(W s, W alpha, W beta, T c) { return (T)(W)(alpha * s + beta * (W)c); }
+};
+template <> struct GemmElem<uint8_t>  : GemmInt<uint8_t, uint32_t> {};
+template <> struct GemmElem<uint16_t> : GemmInt<uint16_t, uint32_t> {};
+template <> struct GemmElem<uint32_t> : GemmInt<uint32_t, uint32_t> {};
+template <> struct GemmElem<uint64_t> : GemmInt<uint64_t, uint64_t> {};
+template <> struct GemmElem<int8_t>   : GemmInt<int8_t, uint32_t> {};
+template <> struct GemmElem<int16_t>  : GemmInt<int16_t, uint32_t> {};
+template <> struct GemmElem<int32_t>  : GemmInt<int32_t, uint32_t> {};
+template <> struct GemmElem<int64_t>  : GemmInt<int64_t, uint64_t> {};
+template <> struct GemmElem<obool>
+{  typedef uint32_t W;
+   static __device__ W load(obool x) { return x.v ? 1u : 0u; }
+   static __device__ W fma(W s, W a, W b) { return s | (a & b); }
+   static __device__ obool finish(W s, W alpha, W beta, obool c) { obool r; r.v = ((s & alpha) | (beta & (c.v ? 1u : 0u))) ? 1 : 0; return r; }
+};
+template <> struct GemmElem<half_t>
+{  typedef float W;
+   static __device__ W load(half_t x) { return half_to_float(x); }
+   static __device__ W fma(W s, W a, W b) { return s + a * b; }
+   static __device__ half_t finish(W s, W alpha, W beta, half_t c)
+   {  float v = alpha * s;
+      if (beta != 0) v += beta * half_to_float(c);
+      return float_to_half(v);
+   }
+};
+
+#define GT 64      /* tile edge */
+#define GK 16      /* K slab */
+template <class T>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(uint32_t M, uint32_t N, uint32_t K,
+      T alpha_host, T beta_host, const T *alpha_dev, const T *beta_dev,
+      const T *A, int64_t sAm, int64_t sAk, const T *B, int64_t sBk, int64_t sBn, T *C, int64_t ldC)
+{
+   typedef GemmElem<T> E; typedef typename E::W W;
+   __shared__ W As[GK][GT + 1], Bs[GK][GT + 1];
+   const uint32_t tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+   const uint32_t m0 = blockIdx.x * GT, n0 = blockIdx.y * GT;
+   W acc[4][4];
+#pragma unroll
+   for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) acc[i][j] = 0;
+   for (uint32_t k0 = 0; k0 < K; k0 += GK)
+   {
+#pragma unroll
+      for (int v = 0; v < 4; v++)
+      {  const uint32_t q = threadIdx.x + 256 * v;
+         const uint32_t mm = q % GT, kk = q / GT;
+         const uint32_t gm = m0 + mm, gn = n0 + mm, gk = k0 + kk;
+         As[kk][mm] = (gm < M && gk < K) ? E::load(A[(int64_t)gm * sAm + (int64_t)gk * sAk]) : (W)0;
+         Bs[kk][mm] = (gn < N && gk < K) ? E::load(B[(int64_t)gk * sBk + (int64_t)gn * sBn]) : (W)0;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int kk = 0; kk < GK; kk++)
+      {  W a[4], b[4];
+#pragma unroll
+         for (int i = 0; i < 4; i++) { a[i] = As[kk][tx + 16 * i]; b[i] = Bs[kk][ty + 16 * i]; }
+#pragma unroll
+         for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[i][j] = E::fma(acc[i][j], a[i], b[j]);
+      }
+      __syncthreads();
+   }
+   const W alpha = E::load(alpha_dev ? *alpha_dev : alpha_host), beta = E::load(beta_dev ? *beta_dev : beta_host);
+#pragma unroll
+   for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+      {  const uint32_t row = m0 + tx + 16 * i, col = n0 + ty + 16 * j;
+         if (row < M && col < N)
+         {  T *c = C + (int64_t)row + (int64_t)col * ldC;
+            *c = E::finish(acc[i][j], alpha, beta, *c);
+         }
+      }
+}
+
+template <class T> static int gemm_generic(const GemmArgs &g)
+{
+   T alpha, beta; memset(&alpha, 0, sizeof(T)); memset(&beta, 0, sizeof(T));
+   const T *adev = nullptr, *bdev = nullptr;
+   if (g.scalar_mode_host) { memcpy(&alpha, g.alpha, sizeof(T)); memcpy(&beta, g.beta, sizeof(T)); }
+   else { adev = (const T *)g.alpha; bdev = (const T *)g.beta; }
+   const bool ta = (g.transA != 'N'), tb = (g.transB != 'N');
+   const int64_t sAm = ta ? g.ldA : 1, sAk = ta ? 1 : g.ldA, sBk = tb ? g.ldB : 1, sBn = tb ? 1 : g.ldB;
+   const uint64_t gx = (g.M + GT - 1) / GT, gy = (g.N + GT - 1) / GT;
+   if (gy > 65535) return set_error("gemm: N = %zu is too large for this data type", g.N);
+   hipLaunchKernelGGL((gemm_generic_kernel<T>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, g.stream,
+                      (uint32_t)g.M, (uint32_t)g.N, (uint32_t)g.K, alpha, beta, adev, bdev,
+                      (const T *)g.A, sAm, sAk, (const T *)g.B, sBk, sBn, (T *)g.C, (int64_t)g.ldC);
+   OCH_CHECK_LAUNCH();
+   return 0;
+}
+
+static char norm_trans(char t)
+{  if (t == 'N' || t == 'n') return 'N';
+   if (t == 'T' || t == 't') return 'T';
+   if (t == 'C' || t == 'c') return 'C';
+   return 0;
+}
+
+} /* namespace och */
+
+using namespace och;
+
+extern "C" int och_gemm_supported(int dtype)
+{  return (dtype >= 0 && dtype < DT_COUNT && dtype != OCH_CHALF) ? 1 : 0; }
+
+extern "C" int och_gemm(int dtype, char transA, char transB, size_t M, size_t N, size_t K,
+                        const void *alpha, const void *A, ptrdiff_t ldA, const void *B, ptrdiff_t ldB,
+                        const void *beta, void *C, ptrdiff_t ldC, int scalar_mode_host, och_stream stream)
+{
+   if (!och_gemm_supported(dtype)) return set_error("gemm is not available for data type %d", dtype);
+   GemmArgs g;
+   g.transA = norm_trans(transA); g.transB = norm_trans(transB);
+   if (!g.transA || !g.transB) return set_error("gemm: invalid transposition mode ('%c', '%c')", transA, transB);
+   if (M == 0 || N == 0) return 0;                       /* empty result: tensor_blas_gpu.c:96 */
+   if (M > 0xFFFFFF00ull || N > 0xFFFFFF00ull || K > 0xFFFFFF00ull) return set_error("gemm: dimensions beyond 2^32 are not supported");
+   const size_t rowsA = (g.transA == 'N') ? M : K, rowsB = (g.transB == 'N') ? K : N;
+   if (K > 0 && (ldA < (ptrdiff_t)(rowsA ? rowsA : 1) || ldB < (ptrdiff_t)(rowsB ? rowsB : 1)))
+      return set_error("gemm: leading dimension smaller than the number of rows (ldA = %td, ldB = %td)", ldA, ldB);
+   if (ldC < (ptrdiff_t)M) return set_error("gemm: ldC = %td is smaller than M = %zu", ldC, M);
+   if (!alpha || !beta || !C || (K > 0 && (!A || !B))) return set_error("gemm: null pointer argument");
+   g.M = M; g.N = N; g.K = K; g.alpha = alpha; g.beta = beta; g.A = A; g.B = B; g.C = C;
+   g.ldA = ldA; g.ldB = ldB; g.ldC = ldC; g.scalar_mode_host = scalar_mode_host; g.stream = as_stream(stream);
+   if (dtype < OCH_CHALF && g.transA == 'C') g.transA = 'T';   /* conjugating a real matrix is the identity */
+   if (dtype < OCH_CHALF && g.transB == 'C') g.transB = 'T';
+   switch (dtype)
+   {  case OCH_BOOL:    return gemm_generic<obool>(g);
+      case OCH_UINT8:   return gemm_generic<uint8_t>(g);
+      case OCH_UINT16:  return gemm_generic<uint16_t>(g);
+      case OCH_UINT32:  return gemm_generic<uint32_t>(g);
+      case OCH_UINT64:  return gemm_generic<uint64_t>(g);
+      case OCH_INT8:    return gemm_generic<int8_t>(g);
+      case OCH_INT16:   return gemm_generic<int16_t>(g);
+      case OCH_INT32:   return gemm_generic<int32_t>(g);
+      case OCH_INT64:   return gemm_generic<int64_t>(g);
+      case OCH_HALF:    return gemm_generic<half_t>(g);
+      case OCH_FLOAT:   return gemm_float(g);
+      case OCH_DOUBLE:  return gemm_double(g);
+      case OCH_CFLOAT:  return gemm_cfloat(g);
+      case OCH_CDOUBLE: return gemm_cdouble(g);
+   }
+   return set_error("gemm is not available for data type %d", dtype);
+}

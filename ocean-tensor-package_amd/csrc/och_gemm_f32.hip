@@ -1,0 +1,3 @@
+/* float GEMM: 128 x 128 block tile, 64 x 64 per wave (2 x 2 tiles of 32x32x2), K slab 16 */
+#include "och_gemm.h"
+namespace och { int gemm_float(const GemmArgs &g) { return launch_gemm_mfma<float, false, 64, 64, 16>(g); } }

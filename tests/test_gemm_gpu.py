@@ -1,0 +1,225 @@
+"""Parity of och_gemm with the CPU oracle (textbook triple loop, long-double accumulation).
+
+Mirrors examples/python/cpu/tensors/ocean_gemm_01..11.py and examples/python/gpu/tensors/
+ocean_gemm_01/10/11.py (modes N/T/C, vector shapes, empty operands, alpha/beta variants) and
+ocean_multiply_02.py (bool GEMM = OR/AND), extended to every supported type.
+
+Bars: bool and integers bit-exact (wrap-around arithmetic). Floating point: normwise
+    ||C_gpu - C_oracle||_F <= tol * (|alpha| * || |A| |B| ||_F + |beta| * ||C_0||_F)
+with tol = 1e-5 (float, cfloat), 1e-13 (double, cdouble) and 2e-3 (half: products and sums
+are accumulated in float and rounded to half once).
+The full-size products (8192^3 double/float, 4096^3 cfloat) are checked with random probe
+vectors: C x must equal alpha * A (B x) + beta * C_0 x (Freivalds), to the same bars.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import helpers as H
+import ocean_hip as oh
+
+orc = H.orc
+pytestmark = pytest.mark.gpu
+
+GEMM_TYPES = [d for d in H.ALL_TYPES if d != H.CHALF]
+TOL = {H.HALF: 2e-3, H.FLOAT: 1e-5, H.CFLOAT: 1e-5, H.DOUBLE: 1e-13, H.CDOUBLE: 1e-13}
+
+
+def as_float(dtype, a):
+    """numpy float/complex view of stored data (half bits -> float32)."""
+    if dtype == H.HALF:
+        return a.view(np.float16).astype(np.float64)
+    return a
+
+
+def matrix(dtype, rows, cols, ld, rng):
+    """Column-major rows x cols matrix inside an ld x cols parent; the padding rows hold junk
+    that must never be read into the result."""
+    flat = H.random_data(dtype, ld * max(cols, 1), rng, "small")
+    return flat
+
+
+def scalar_of(dtype, value):
+    st = H.storage(dtype)
+    if dtype == H.HALF:
+        return H.f32_to_half_bits(np.array([value], np.float32))
+    if dtype == H.BOOL:
+        return np.array([1 if value else 0], np.uint8)
+    return np.array([value]).astype(st)
+
+
+def run_case(stream, dtype, ta, tb, M, N, K, alpha, beta, rng, device_scalars=False, pad=3):
+    rowsA, colsA = (M, K) if ta == "N" else (K, M)
+    rowsB, colsB = (K, N) if tb == "N" else (N, K)
+    ldA, ldB, ldC = max(rowsA, 1) + pad, max(rowsB, 1) + pad, max(M, 1) + pad
+    A = matrix(dtype, rowsA, colsA, ldA, rng)
+    B = matrix(dtype, rowsB, colsB, ldB, rng)
+    C0 = matrix(dtype, M, N, ldC, rng)
+    al, be = scalar_of(dtype, alpha), scalar_of(dtype, beta)
+    dA, dB, dC = oh.to_device(A, stream), oh.to_device(B, stream), oh.to_device(C0, stream)
+    if device_scalars:
+        dal, dbe = oh.to_device(al, stream), oh.to_device(be, stream)
+        pal, pbe, mode = dal.ptr, dbe.ptr, 0
+    else:
+        pal, pbe, mode = orc.ptr(al), orc.ptr(be), 1
+    oh.check(oh.lib.och_gemm(dtype, ta.encode(), tb.encode(), M, N, K, pal, dA.ptr, ldA, dB.ptr, ldB, pbe, dC.ptr, ldC, mode, stream.handle))
+    got = dC.download(C0.dtype, C0.size)
+    want = C0.copy()
+    assert orc.lib.oracle_gemm(dtype, ta.encode(), tb.encode(), M, N, K, orc.ptr(al), orc.ptr(A), ldA, orc.ptr(B), ldB,
+                               orc.ptr(be), orc.ptr(want), ldC, 4) == 0
+    for b in (dA, dB, dC):
+        b.free()
+    what = "%s %s%s %dx%dx%d alpha=%r beta=%r" % (H.NAMES[dtype], ta, tb, M, N, K, alpha, beta)
+    if dtype not in TOL:
+        H.assert_same_bytes(got, want, what)
+        return
+    g, w = as_float(dtype, got).reshape(-1, ldC), as_float(dtype, want).reshape(-1, ldC)      # (cols, ld)
+    # padding rows untouched
+    H.assert_same_bytes(got.reshape(-1, ldC)[:, M:], C0.reshape(-1, ldC)[:, M:], what + " (padding)")
+    a = np.abs(as_float(dtype, A).reshape(-1, ldA)[:colsA, :rowsA])
+    b = np.abs(as_float(dtype, B).reshape(-1, ldB)[:colsB, :rowsB])
+    opa = a.T if ta == "N" else a                 # (M, K) in row-major numpy terms
+    opb = b.T if tb == "N" else b
+    scale = abs(alpha) * np.linalg.norm(opa @ opb) + abs(beta) * np.linalg.norm(as_float(dtype, C0).reshape(-1, ldC)[:N, :M])
+    err = np.linalg.norm((g - w)[:N, :M])
+    assert np.isfinite(err) and err <= TOL[dtype] * max(scale, 1e-30), "%s: error %.3e, bound %.3e" % (what, err, TOL[dtype] * scale)
+
+
+SHAPES = [(70, 50, 90), (128, 128, 64), (256, 128, 16), (130, 257, 33), (1, 1, 300), (1, 1, 4096), (3, 2, 1000),
+          (200, 1, 64), (1, 200, 77), (64, 64, 1), (5, 3, 0), (17, 1, 1)]
+
+
+@pytest.mark.parametrize("dtype", GEMM_TYPES, ids=[H.NAMES[d] for d in GEMM_TYPES])
+def test_gemm_all_types(hip, stream, dtype):
+    assert oh.lib.och_gemm_supported(dtype) == 1
+    rng = np.random.default_rng(500 + dtype)
+    modes = ["N", "T"] + (["C"] if dtype in H.COMPLEX_TYPES else [])
+    cplx = dtype in H.COMPLEX_TYPES
+    for (M, N, K) in SHAPES:
+        for ta in modes:
+            for tb in modes:
+                alpha, beta = (1, 0)
+                if (M + N + K + len(ta + tb)) % 2 == 0:
+                    alpha, beta = ((2 - 1j, -1 + 0.5j) if cplx else (2, -1)) if dtype != H.BOOL else (1, 1)
+                if dtype in (H.UINT8, H.UINT16, H.UINT32, H.UINT64) and beta == -1:
+                    beta = 3
+                run_case(stream, dtype, ta, tb, M, N, K, alpha, beta, rng)
+
+
+@pytest.mark.parametrize("dtype", [H.INT32, H.HALF, H.FLOAT, H.DOUBLE, H.CFLOAT, H.CDOUBLE, H.BOOL], ids=lambda d: H.NAMES[d])
+def test_gemm_scalars(hip, stream, dtype):
+    """alpha / beta in device memory, zero alpha, beta = 0 with NaN in C (C must not be read)."""
+    rng = np.random.default_rng(600 + dtype)
+    run_case(stream, dtype, "N", "T", 96, 80, 40, 1, 1, rng, device_scalars=True)
+    run_case(stream, dtype, "T", "N", 128, 128, 128, 1, 0, rng, device_scalars=True, pad=0)
+    run_case(stream, dtype, "N", "N", 33, 65, 20, 0, 1, rng)
+    run_case(stream, dtype, "N", "N", 1, 1, 512, 1, 1, rng, device_scalars=True)
+    if dtype in (H.FLOAT, H.DOUBLE, H.CFLOAT, H.CDOUBLE):
+        st = H.storage(dtype)
+        M, N, K = 128, 128, 32
+        A = H.random_data(dtype, M * K, rng, "small"); B = H.random_data(dtype, K * N, rng, "small")
+        C0 = np.full(M * N, np.nan, st)
+        dA, dB, dC = oh.to_device(A, stream), oh.to_device(B, stream), oh.to_device(C0, stream)
+        one, zero = scalar_of(dtype, 1), scalar_of(dtype, 0)
+        oh.check(oh.lib.och_gemm(dtype, b"N", b"N", M, N, K, orc.ptr(one), dA.ptr, M, dB.ptr, K, orc.ptr(zero), dC.ptr, M, 1, stream.handle))
+        got = dC.download(st, M * N)
+        assert np.isfinite(got.view(np.float32 if st in (np.float32, np.complex64) else np.float64)).all(), "beta = 0 must ignore C"
+        for b in (dA, dB, dC):
+            b.free()
+
+
+def test_gemm_errors_and_empty(hip, stream):
+    rng = np.random.default_rng(7)
+    one = np.ones(1)
+    buf = oh.to_device(rng.uniform(-1, 1, 64), stream)
+    # empty result: no-op, returns success
+    assert oh.lib.och_gemm(H.DOUBLE, b"N", b"N", 0, 5, 3, orc.ptr(one), buf.ptr, 1, buf.ptr, 3, orc.ptr(one), buf.ptr, 1, 1, stream.handle) == 0
+    assert oh.lib.och_gemm(H.DOUBLE, b"N", b"N", 5, 0, 3, orc.ptr(one), buf.ptr, 5, buf.ptr, 3, orc.ptr(one), buf.ptr, 5, 1, stream.handle) == 0
+    # chalf is not supported, as in the reference
+    assert oh.lib.och_gemm_supported(H.CHALF) == 0
+    assert oh.lib.och_gemm(H.CHALF, b"N", b"N", 2, 2, 2, orc.ptr(one), buf.ptr, 2, buf.ptr, 2, orc.ptr(one), buf.ptr, 2, 1, stream.handle) != 0
+    assert b"not available" in oh.lib.och_last_error()
+    assert oh.lib.och_gemm(H.DOUBLE, b"X", b"N", 2, 2, 2, orc.ptr(one), buf.ptr, 2, buf.ptr, 2, orc.ptr(one), buf.ptr, 2, 1, stream.handle) != 0
+    assert oh.lib.och_gemm(H.DOUBLE, b"N", b"N", 4, 2, 2, orc.ptr(one), buf.ptr, 2, buf.ptr, 2, orc.ptr(one), buf.ptr, 4, 1, stream.handle) != 0
+    assert b"leading dimension" in oh.lib.och_last_error()
+    buf.free()
+
+
+FULL = [(H.DOUBLE, 8192, "N", "N"), (H.DOUBLE, 8192, "T", "N"), (H.FLOAT, 8192, "N", "T"), (H.FLOAT, 8192, "N", "N"),
+        (H.CFLOAT, 4096, "C", "N"), (H.CFLOAT, 4096, "N", "N"), (H.CDOUBLE, 2048, "N", "C")]
+
+
+@pytest.mark.parametrize("dtype,n,ta,tb", FULL, ids=["%s-%d-%s%s" % (H.NAMES[d], n, a, b) for d, n, a, b in FULL])
+def test_gemm_full_size_probe(hip, stream, dtype, n, ta, tb):
+    """Benchmark-size products checked with probe vectors (no O(n^3) work on the host)."""
+    rng = np.random.default_rng(800 + dtype + n)
+    st = H.storage(dtype)
+    cplx = dtype in H.COMPLEX_TYPES
+
+    def rand():
+        a = rng.uniform(-1, 1, n * n).astype(st if not cplx else (np.float32 if dtype == H.CFLOAT else np.float64))
+        if cplx:
+            a = (a + 1j * rng.uniform(-1, 1, n * n)).astype(st)
+        return a.reshape(n, n)                           # numpy (col, row): column-major matrix
+    A, B, C0 = rand(), rand(), rand()
+    alpha, beta = ((0.5 - 0.25j, -1.5 + 1j) if cplx else (0.5, -1.5))
+    al, be = scalar_of(dtype, alpha), scalar_of(dtype, beta)
+    dA, dB, dC = oh.to_device(A, stream), oh.to_device(B, stream), oh.to_device(C0, stream)
+    oh.check(oh.lib.och_gemm(dtype, ta.encode(), tb.encode(), n, n, n, orc.ptr(al), dA.ptr, n, dB.ptr, n, orc.ptr(be), dC.ptr, n, 1, stream.handle))
+    got = dC.download(st, n * n).reshape(n, n)
+    for b in (dA, dB, dC):
+        b.free()
+    wide = np.complex128 if cplx else np.float64
+
+    def op(Mx, t):          # the mathematical matrix op(M) as a numpy array indexed [row, col]
+        m = Mx.T            # column-major storage -> [row, col]
+        return m if t == "N" else (m.T if t == "T" else m.conj().T)
+    X = rng.uniform(-1, 1, (n, 4)).astype(wide)
+    opA, opB = op(A, ta), op(B, tb)
+    want = alpha * (opA.astype(wide) @ (opB.astype(wide) @ X)) + beta * (C0.T.astype(wide) @ X)
+    have = got.T.astype(wide) @ X
+    scale = abs(alpha) * np.linalg.norm(np.abs(opA).astype(np.float64) @ (np.abs(opB).astype(np.float64) @ np.abs(X))) \
+        + abs(beta) * np.linalg.norm(np.abs(C0.T).astype(np.float64) @ np.abs(X))
+    err = np.linalg.norm(have - want)
+    assert err <= TOL[dtype] * scale, "probe error %.3e, bound %.3e" % (err, TOL[dtype] * scale)
+    # and one directly computed row and column
+    i = int(rng.integers(0, n))
+    row = alpha * (opA[i, :].astype(wide) @ opB.astype(wide)) + beta * C0.T[i, :].astype(wide)
+    assert np.linalg.norm(got.T[i, :] - row) <= TOL[dtype] * (np.linalg.norm(np.abs(opA[i, :]).astype(np.float64) @ np.abs(opB).astype(np.float64)) * abs(alpha)
+                                                              + abs(beta) * np.linalg.norm(C0.T[i, :]))
+
+
+def test_mgs_qr_pattern(hip, stream):
+    """Modified Gram-Schmidt on a 512 x 48 double matrix driven the way the reference example does
+    it: per pair one dot product (gemm with M = N = 1, result kept on the device), one rank-1 update
+    (gemm with K = 1 reading that device scalar) and per column a norm and a scale."""
+    rng = np.random.default_rng(11)
+    m, n = 512, 48
+    A = rng.uniform(-1, 1, (n, m))                       # column j = A[j, :]
+    Q = oh.to_device(A, stream)
+    R = oh.to_device(np.zeros((n, n)), stream)           # R[j, i] = r_ij (column-major n x n)
+    one, zero, minus = np.ones(1), np.zeros(1), -np.ones(1)
+    done, dzero, dminus = oh.to_device(one, stream), oh.to_device(zero, stream), oh.to_device(minus, stream)
+    inv = oh.DeviceBuffer(8, stream)
+    col = lambda j: C.c_void_p(Q.address + 8 * m * j)
+    rij = lambda i, j: C.c_void_p(R.address + 8 * (i + n * j))
+    nrm = np.zeros(1)
+    ref = A.copy(); Rref = np.zeros((n, n))
+    for j in range(n):
+        for i in range(j):
+            # r_ij = q_i' a_j  (device scalar), a_j -= q_i r_ij
+            oh.check(oh.lib.och_gemm(H.DOUBLE, b"T", b"N", 1, 1, m, dminus.ptr, col(i), m, col(j), m, dzero.ptr, rij(i, j), 1, 0, stream.handle))
+            oh.check(oh.lib.och_gemm(H.DOUBLE, b"N", b"N", m, 1, 1, done.ptr, col(i), m, rij(i, j), 1, done.ptr, col(j), m, 0, stream.handle))
+            r = ref[i] @ ref[j]; Rref[j, i] = r; ref[j] -= r * ref[i]
+        oh.check(oh.lib.och_reduce_all(oh.R["norm2"], H.DOUBLE, 1, oh.sizes([m]), oh.strides([8]), col(j), None, None, 0.0, orc.ptr(nrm), None, stream.handle))
+        inv.upload(np.array([1.0 / nrm[0]]))
+        oh.check(oh.lib.och_binary(oh.B["multiply"], H.DOUBLE, 1, oh.sizes([m]), oh.strides([8]), col(j), oh.strides([0]), inv.ptr,
+                                   oh.strides([8]), col(j), stream.handle))
+        nr = np.linalg.norm(ref[j]); Rref[j, j] = nr; ref[j] /= nr
+    Qg = Q.download(np.float64, n * m).reshape(n, m)
+    Rg = -R.download(np.float64, n * n).reshape(n, n)     # the dot products were stored negated (alpha = -1)
+    assert np.abs(Qg @ Qg.T - np.eye(n)).max() < 1e-12
+    assert np.abs(Qg - ref).max() < 1e-11
+    off = ~np.eye(n, dtype=bool)
+    assert np.abs(Rg[off] - Rref[off]).max() < 1e-11
