@@ -1,0 +1,152 @@
+/* Index operations: add-if-negative, index-to-offset, gather / scatter / fill through per-dimension
+ * offset tables. Replaces solid/src/core/gpu/template_index.cu:37-200 and the kernels of
+ * solid/include/solid/core/gpu/index1.h:182-215, index2.h:188-230.
+ *
+ * Offset tables: for dimension d, offsets[d] is either NULL (the element offset advances by
+ * index * strides[d]) or a device array of size[d] byte offsets. Gather, scatter and fill move
+ * raw elements, so one kernel per element size serves every data type.
+ */
+#include "och_elemwise.h"
+#include "och_dispatch.h"
+
+namespace och {
+
+template <class T> struct AddIfNegOp
+{  typedef T R; struct Param { T value; }; static constexpr bool RMW = true;
+   static OCH_D R f(R x, uint64_t, const Param &p) { return (x < 0) ? (R)(x + p.value) : x; }
+};
+template <class T> static T idx_scalar_as(const och_scalar &s) { T v; memcpy(&v, &s, sizeof(T)); return v; }
+
+struct IndexParams
+{
+   uint64_t       size[OCH_MAX_DIMS];
+   const int64_t *offsets[OCH_MAX_DIMS];
+   int64_t        strides1[OCH_MAX_DIMS], strides2[OCH_MAX_DIMS];
+   char          *ptr1, *ptr2;
+   uint64_t       nelem;
+   int            ndims;
+};
+struct ToOffsetStrides { int64_t s[OCH_MAX_DIMS]; };
+
+template <class T>
+__global__ __launch_bounds__(256) void index_to_offset_kernel(uint64_t nelem, int nstrides, const ToOffsetStrides st,
+      int64_t stride_reduce, const char *src, int64_t stride1, char *dst, int64_t stride2)
+{
+   uint64_t j = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+   if (j >= nelem) return;
+   int64_t s = 0;
+   for (int i = 0; i < nstrides; i++)
+      s += st.s[i] * (int64_t)*reinterpret_cast<const T *>(src + (int64_t)j * stride1 + (int64_t)i * stride_reduce);
+   *reinterpret_cast<int64_t *>(dst + (int64_t)j * stride2) = s;
+}
+
+/* MODE 0: gather  *ptr2 = *ptr1(indexed);  1: scatter  *ptr1(indexed) = *ptr2;  2: fill  *ptr1(indexed) = value */
+template <class E, int MODE>
+__global__ __launch_bounds__(256) void index_kernel(const IndexParams p, const E value)
+{
+   for (uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x; idx < p.nelem; idx += (uint64_t)gridDim.x * 256)
+   {  uint64_t q = idx; int64_t o1 = 0, o2 = 0;
+      for (int d = 0; d < p.ndims; d++)
+      {  uint64_t s = q % p.size[d]; q /= p.size[d];
+         o1 += p.offsets[d] ? p.offsets[d][s] : (int64_t)s * p.strides1[d];
+         if (MODE != 2) o2 += (int64_t)s * p.strides2[d];
+      }
+      E *a = reinterpret_cast<E *>(p.ptr1 + o1);
+      if (MODE == 0) *reinterpret_cast<E *>(p.ptr2 + o2) = *a;
+      else if (MODE == 1) *a = *reinterpret_cast<const E *>(p.ptr2 + o2);
+      else *a = value;
+   }
+}
+
+struct alignas(4) E4 { unsigned char b[4]; };
+struct alignas(8) E8 { unsigned char b[8]; };
+struct alignas(8) E16 { unsigned char b[16]; };      /* cdouble is 8-byte aligned */
+struct alignas(2) E2 { unsigned char b[2]; };
+struct E1 { unsigned char b[1]; };
+
+template <class E, int MODE>
+static int launch_index(const IndexParams &p, const och_scalar &value, hipStream_t stream)
+{  E v; memcpy(&v, &value, sizeof(E));
+   uint64_t blocks = (p.nelem + 255) / 256; if (blocks > 65536) blocks = 65536;
+   hipLaunchKernelGGL((index_kernel<E, MODE>), dim3((unsigned)blocks), dim3(256), 0, stream, p, v);
+   OCH_CHECK_LAUNCH();
+   return 0;
+}
+
+template <int MODE>
+static int index_op(int dtype, int ndims, const size_t *size, int64_t **offsets, const ptrdiff_t *strides1, void *ptr1,
+                    const ptrdiff_t *strides2, void *ptr2, const och_scalar &value, hipStream_t stream)
+{
+   if (!dtype_ok(dtype)) return set_error("invalid data type (%d)", dtype);
+   if (ndims < 0 || ndims > OCH_MAX_DIMS) return set_error("invalid number of dimensions (%d)", ndims);
+   IndexParams p; memset(&p, 0, sizeof(p));
+   p.ndims = ndims; p.nelem = 1; p.ptr1 = (char *)ptr1; p.ptr2 = (char *)ptr2;
+   for (int d = 0; d < ndims; d++)
+   {  p.size[d] = size[d]; p.nelem *= size[d];
+      p.offsets[d] = offsets ? offsets[d] : nullptr;
+      p.strides1[d] = strides1 ? strides1[d] : 0;
+      p.strides2[d] = (MODE != 2 && strides2) ? strides2[d] : 0;
+   }
+   if (p.nelem == 0) return 0;
+   switch (och_type_size[dtype])
+   {  case 1:  return launch_index<E1, MODE>(p, value, stream);
+      case 2:  return launch_index<E2, MODE>(p, value, stream);
+      case 4:  return launch_index<E4, MODE>(p, value, stream);
+      case 8:  return launch_index<E8, MODE>(p, value, stream);
+      case 16: return launch_index<E16, MODE>(p, value, stream);
+   }
+   return set_error("unsupported element size");
+}
+
+} /* namespace och */
+
+using namespace och;
+
+extern "C" int och_add_if_negative(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr,
+                                   och_scalar value, och_stream stream)
+{
+   switch (dtype)
+   {
+#define OCH_CASE(T, ID) case ID: { AddIfNegOp<T>::Param prm; prm.value = idx_scalar_as<T>(value); \
+                        return launch_ew1<AddIfNegOp<T>>(ndims, size, strides, ptr, prm, true, as_stream(stream)); }
+      OCH_CASE(int8_t, OCH_INT8) OCH_CASE(int16_t, OCH_INT16) OCH_CASE(int32_t, OCH_INT32) OCH_CASE(int64_t, OCH_INT64)
+#undef OCH_CASE
+   }
+   return set_error("add_if_negative is available for signed integer types only (got %d)", dtype);
+}
+
+extern "C" int och_index_to_offset(int dtype, int nstrides, const int64_t *strides, ptrdiff_t stride_reduce, size_t nelem,
+                                   ptrdiff_t stride1, void *ptr1, ptrdiff_t stride2, void *ptr2, och_stream stream)
+{
+   if (nstrides < 0 || nstrides > OCH_MAX_DIMS) return set_error("invalid number of strides (%d)", nstrides);
+   if (nelem == 0) return 0;
+   ToOffsetStrides st; memset(&st, 0, sizeof(st));
+   for (int i = 0; i < nstrides; i++) st.s[i] = strides[i];
+   const dim3 grid((unsigned)((nelem + 255) / 256)), block(256);
+   if (nelem > 0xFFFFFF00ull * 256ull) return set_error("index_to_offset: too many elements");
+   switch (dtype)
+   {
+#define OCH_CASE(T, ID) case ID: hipLaunchKernelGGL((index_to_offset_kernel<T>), grid, block, 0, as_stream(stream), (uint64_t)nelem, nstrides, st, \
+                           (int64_t)stride_reduce, (const char *)ptr1, (int64_t)stride1, (char *)ptr2, (int64_t)stride2); break;
+      OCH_CASE(uint8_t, OCH_UINT8) OCH_CASE(uint16_t, OCH_UINT16) OCH_CASE(uint32_t, OCH_UINT32) OCH_CASE(uint64_t, OCH_UINT64)
+      OCH_CASE(int8_t, OCH_INT8) OCH_CASE(int16_t, OCH_INT16) OCH_CASE(int32_t, OCH_INT32) OCH_CASE(int64_t, OCH_INT64)
+#undef OCH_CASE
+      default: return set_error("index_to_offset is available for integer types only (got %d)", dtype);
+   }
+   OCH_CHECK_LAUNCH();
+   return 0;
+}
+
+extern "C" int och_get_index(int dtype, int ndims, const size_t *size, int64_t **offsets, const ptrdiff_t *strides1, void *ptr1,
+                             const ptrdiff_t *strides2, void *ptr2, och_stream stream)
+{  och_scalar zero; memset(&zero, 0, sizeof(zero));
+   return index_op<0>(dtype, ndims, size, offsets, strides1, ptr1, strides2, ptr2, zero, as_stream(stream));
+}
+extern "C" int och_set_index(int dtype, int ndims, const size_t *size, int64_t **offsets, const ptrdiff_t *strides1, void *ptr1,
+                             const ptrdiff_t *strides2, void *ptr2, och_stream stream)
+{  och_scalar zero; memset(&zero, 0, sizeof(zero));
+   return index_op<1>(dtype, ndims, size, offsets, strides1, ptr1, strides2, ptr2, zero, as_stream(stream));
+}
+extern "C" int och_fill_index(int dtype, int ndims, const size_t *size, int64_t **offsets, const ptrdiff_t *strides, void *ptr,
+                              och_scalar value, och_stream stream)
+{  return index_op<2>(dtype, ndims, size, offsets, strides, ptr, nullptr, nullptr, value, as_stream(stream)); }

@@ -66,6 +66,16 @@ int oracle_gemm(int dtype, char transA, char transB, size_t M, size_t N, size_t 
                 const void *alpha, const void *A, ptrdiff_t ldA, const void *B, ptrdiff_t ldB,
                 const void *beta, void *C, ptrdiff_t ldC, int nthreads);
 
+/* Index operations (template_index.c): per-dimension offset tables or strides. */
+int oracle_add_if_negative(int dtype, int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr, och_scalar value);
+int oracle_index_to_offset(int dtype, int nstrides, const int64_t *strides, ptrdiff_t stride_reduce, size_t nelem,
+                ptrdiff_t stride1, const void *ptr1, ptrdiff_t stride2, void *ptr2);
+int oracle_get_index(int dtype, int ndims, const size_t *size, int64_t **offsets, const ptrdiff_t *strides1, void *ptr1,
+                const ptrdiff_t *strides2, void *ptr2);
+int oracle_set_index(int dtype, int ndims, const size_t *size, int64_t **offsets, const ptrdiff_t *strides1, void *ptr1,
+                const ptrdiff_t *strides2, void *ptr2);
+int oracle_fill_index(int dtype, int ndims, const size_t *size, int64_t **offsets, const ptrdiff_t *strides, void *ptr, och_scalar value);
+
 /* Software half precision (half.c) exposed for exhaustive tests */
 float    oracle_half_to_float(uint16_t h);
 uint16_t oracle_float_to_half(float f);

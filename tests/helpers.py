@@ -221,3 +221,12 @@ def axis_config(src, dst, axes, stream=None, device=True):
     else:
         cfg.ptr1, cfg.ptr2 = src.hptr().value, dst.hptr().value
     return cfg
+
+
+def raw_scalar(element):
+    """och_scalar holding the bytes of one stored element (numpy array of size 1, any storage type)."""
+    a = np.ascontiguousarray(element).reshape(-1)[:1]
+    s = oh.Scalar()
+    C.memset(C.byref(s), 0, C.sizeof(s))
+    C.memmove(C.byref(s), a.ctypes.data, a.itemsize)
+    return s

@@ -50,6 +50,11 @@ def setup(oh):
         ("oracle_reduce_axis", _i, [_i, _i, C.POINTER(oh.ReduceAxisConfig), C.c_double]),
         ("oracle_gemm", _i, [_i, C.c_char, C.c_char, C.c_size_t, C.c_size_t, C.c_size_t, _vp, _vp, C.c_ssize_t, _vp,
                             C.c_ssize_t, _vp, _vp, C.c_ssize_t, _i]),
+        ("oracle_add_if_negative", _i, [_i, _i, _sz, _st, _vp, S]),
+        ("oracle_index_to_offset", _i, [_i, _i, C.POINTER(C.c_int64), C.c_ssize_t, C.c_size_t, C.c_ssize_t, _vp, C.c_ssize_t, _vp]),
+        ("oracle_get_index", _i, [_i, _i, _sz, C.POINTER(C.POINTER(C.c_int64)), _st, _vp, _st, _vp]),
+        ("oracle_set_index", _i, [_i, _i, _sz, C.POINTER(C.POINTER(C.c_int64)), _st, _vp, _st, _vp]),
+        ("oracle_fill_index", _i, [_i, _i, _sz, C.POINTER(C.POINTER(C.c_int64)), _st, _vp, S]),
     ]:
         if hasattr(lib, name):
             _proto(getattr(lib, name), res, args)
