@@ -148,23 +148,39 @@ def main():
                    "percent_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 1)},
     }
     if args.only_step:
+        # one plain float64 -> float64 copy of known size (134.2 MB read, 134.2 MB written): the
+        # yardstick that scales the FETCH_SIZE / WRITE_SIZE counters of a profiling run
+        oh.check(lib.och_copy(F64, F64, 2, shape, st_f64, sets[0]["TI"].ptr, 2, shape, st_f64, sets[0]["TF"].ptr, h))
+        stream.synchronize()
         print(json.dumps(result))
         return
 
     # per-kernel roofline of the step
     kernels = []
     for name, fn, nbytes in step_kernels:
-        ms = time_launches(lambda fn=fn: fn(sets[0]))
+        turn = [0]
+
+        def rotating(fn=fn, turn=turn):          # alternate the buffer sets, as the step loop does
+            turn[0] += 1
+            fn(sets[turn[0] % NSETS])
+        ms = time_launches(rotating)
         kernels.append({"kernel": name, "ms": round(ms, 4), "algorithmic_MB": round(nbytes / 1e6, 1),
                         "GBps": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 3)})
     dom = max(kernels, key=lambda k: k["ms"])
-    traffic = None
+    # HBM bytes per launch of that kernel as counted by rocprofv3 (FETCH_SIZE + WRITE_SIZE, scaled by a
+    # copy kernel of known size; profiles/elementwise_config2_hbm_traffic.txt), over the same duration
+    traffic, traffic_bytes = None, None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get(dom["kernel"])
+            t = json.load(f).get(dom["kernel"])
+        if t:
+            traffic_bytes = t["fetch_bytes"] + t["write_bytes"]
+            traffic = round(traffic_bytes / dom["ms"] / 1e6, 1)
     result["roofline"] = {"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": round(dom["GBps"] / HBM_PEAK_GBS, 3), "traffic": traffic}
+                          "frac": round(dom["GBps"] / HBM_PEAK_GBS, 3), "traffic": traffic,
+                          "algorithmic_bytes_per_launch": next(b for nm, _, b in step_kernels if nm == dom["kernel"]),
+                          "traffic_bytes_per_launch": traffic_bytes, "launch_ms": dom["ms"]}
     result["kernels"] = kernels
     for s in sets:
         for b in s.values():
