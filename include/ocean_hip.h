@@ -304,6 +304,33 @@ int och_set_index(int dtype, int ndims, const size_t *size, int64_t **offsets,
 int och_fill_index(int dtype, int ndims, const size_t *size, int64_t **offsets,
                    const ptrdiff_t *strides, void *ptr, och_scalar value, och_stream stream);
 
+/* ======================================================================== */
+/* Launch analysis of an elementwise call, without launching anything.      */
+/* Reports what the library derives from the operands before a launch, the  */
+/* counterpart of solid_gpu_elemwise{1,2,3}_analyze (src/core/gpu/op/       */
+/* apply_elemwise3.c:43-156: drop unit dimensions, sort, merge, pick a      */
+/* kernel): the normalised shape (dimensions sorted by the strides of the   */
+/* last operand, negative strides of that operand flipped, mergeable        */
+/* dimensions merged), the byte offset this adds to each pointer, the       */
+/* kernel family, the elements per thread-level access, the number of       */
+/* launches, and the multiply-shift constants that replace the division by  */
+/* each dimension in the kernels. The last operand is the destination.      */
+/* Needs no GPU.                                                            */
+/* ======================================================================== */
+enum { OCH_KERNEL_WIDE = 0, OCH_KERNEL_MIXED = 1, OCH_KERNEL_SINGLE = 2, OCH_KERNEL_TILED = 3 };
+typedef struct {
+   int        ndims;
+   size_t     size[OCH_MAX_DIMS];
+   ptrdiff_t  strides[3][OCH_MAX_DIMS];
+   ptrdiff_t  offset[3];
+   int        kernel;                     /* OCH_KERNEL_* of the first launch */
+   int        vec;                        /* elements per access in that launch */
+   int        launches;                   /* kernel launches for the whole call */
+   unsigned   div_d[OCH_MAX_DIMS], div_m[OCH_MAX_DIMS], div_s1[OCH_MAX_DIMS], div_s2[OCH_MAX_DIMS];
+} och_elemwise_plan;
+int och_elemwise_analyze(int noperands, const int *elemsize, int ndims, const size_t *size,
+                         const ptrdiff_t *const *strides, void *const *ptrs, och_elemwise_plan *plan);
+
 #ifdef __cplusplus
 }
 #endif

@@ -22,15 +22,16 @@
 namespace och {
 
 /* ---- division by an invariant 32-bit integer d >= 2 ---------------------- */
-struct FastDiv { uint32_t d, m, s; };
+struct FastDiv { uint32_t d, m; uint16_t s1, s2; };
 
 static inline FastDiv make_fastdiv(uint32_t d)
-{  /* q = (t + ((n - t) >> 1)) >> s with t = mulhi(m, n); exact for all 32-bit n */
-   FastDiv f; f.d = d; f.m = 0; f.s = 0;
+{  /* q = (t + ((n - t) >> s1)) >> s2 with t = mulhi(m, n), L = ceil(log2 d), m = floor(2^32 (2^L - d) / d) + 1,
+      s1 = min(L, 1), s2 = max(L - 1, 0); exact for all 32-bit n and every d >= 1 (d = 1 gives m = 1, s1 = s2 = 0) */
+   FastDiv f; f.d = d; f.m = 1; f.s1 = 0; f.s2 = 0;
    if (d < 2) return f;
    uint32_t L = 0; while ((1ull << L) < d) L++;
    f.m = (uint32_t)((((1ull << L) - d) << 32) / d + 1);
-   f.s = L - 1;
+   f.s1 = 1; f.s2 = (uint16_t)(L - 1);
    return f;
 }
 OCH_HD uint32_t fastdiv(uint32_t n, const FastDiv &f)
@@ -40,7 +41,7 @@ OCH_HD uint32_t fastdiv(uint32_t n, const FastDiv &f)
 #else
    uint32_t t = (uint32_t)(((uint64_t)f.m * n) >> 32);
 #endif
-   return (t + ((n - t) >> 1)) >> f.s;
+   return (t + ((n - t) >> f.s1)) >> f.s2;
 }
 
 /* ---- kernel parameters ---------------------------------------------------- */

@@ -84,6 +84,26 @@ def make_scalar(dtype, value):
     return s
 
 
+class ElemwisePlan(C.Structure):
+    _fields_ = [("ndims", C.c_int), ("size", C.c_size_t * 8), ("strides", (C.c_ssize_t * 8) * 3), ("offset", C.c_ssize_t * 3),
+                ("kernel", C.c_int), ("vec", C.c_int), ("launches", C.c_int),
+                ("div_d", C.c_uint * 8), ("div_m", C.c_uint * 8), ("div_s1", C.c_uint * 8), ("div_s2", C.c_uint * 8)]
+
+
+KERNEL_WIDE, KERNEL_MIXED, KERNEL_SINGLE, KERNEL_TILED = 0, 1, 2, 3
+
+
+def elemwise_analyze(elemsizes, size, strides_per_operand, addresses):
+    """och_elemwise_analyze for operands given by element size, byte strides and base address."""
+    n = len(elemsizes)
+    es = (C.c_int * n)(*elemsizes)
+    st = (_st * n)(*[strides(s) for s in strides_per_operand])
+    pp = (_vp * n)(*addresses)
+    plan = ElemwisePlan()
+    check(lib.och_elemwise_analyze(n, es, len(size), sizes(size), st, pp, C.byref(plan)))
+    return plan
+
+
 class DeviceProp(C.Structure):
     _fields_ = [("name", C.c_char * 256), ("arch", C.c_char * 64), ("total_global_mem", C.c_size_t),
                 ("shared_mem_per_block", C.c_size_t), ("multiprocessor_count", C.c_int), ("wavefront_size", C.c_int),
@@ -165,6 +185,7 @@ PROTOTYPES = {
     "och_get_index": (_i, [_i, _i, _sz, C.POINTER(C.POINTER(C.c_int64)), _st, _vp, _st, _vp, _vp]),
     "och_set_index": (_i, [_i, _i, _sz, C.POINTER(C.POINTER(C.c_int64)), _st, _vp, _st, _vp, _vp]),
     "och_fill_index": (_i, [_i, _i, _sz, C.POINTER(C.POINTER(C.c_int64)), _st, _vp, Scalar, _vp]),
+    "och_elemwise_analyze": (_i, [_i, C.POINTER(_i), _i, _sz, C.POINTER(_st), C.POINTER(_vp), C.c_void_p]),
 }
 
 

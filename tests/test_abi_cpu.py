@@ -1,0 +1,194 @@
+"""CPU-side checks of the C-ABI library and its host logic (no GPU needed):
+  * the shared library loads and exports every function that include/ocean_hip.h declares,
+    and the Python binding declares a prototype for each of them;
+  * the support / result-type tables agree with the oracle's, which follow the reference's
+    function tables (solid_core_gpu.src:42-439 lists the same (operation, type) pairs as the CPU);
+  * the launch analysis (normalisation: drop, flip, sort, merge; kernel choice; chunking) keeps
+    the set of element offsets of every operand, checked by brute-force enumeration, and its
+    multiply-shift division constants divide exactly.
+"""
+import ctypes as C
+import itertools
+import os
+import re
+
+import numpy as np
+import pytest
+
+import helpers as H
+import ocean_hip as oh
+
+orc = H.orc
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "ocean_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(och_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_function():
+    names = declared_functions()
+    assert len(names) >= 58
+    raw = C.CDLL(oh.LIB_PATH)
+    missing = [n for n in names if not hasattr(raw, n)]
+    assert not missing, "not exported: %s" % missing
+    assert oh.MISSING == []
+    unbound = [n for n in names if n not in oh.PROTOTYPES]
+    assert not unbound, "no prototype in the binding: %s" % unbound
+    stale = [n for n in oh.PROTOTYPES if n not in names]
+    assert not stale, "binding declares functions the header does not: %s" % stale
+
+
+def test_type_sizes_and_error_message():
+    sizes = (C.c_int * 15).in_dll(oh.lib, "och_type_size")
+    assert list(sizes) == [1, 1, 2, 4, 8, 1, 2, 4, 8, 2, 4, 8, 4, 8, 16]
+    assert oh.lib.och_binary_supported(999, 0) == 0
+    assert oh.lib.och_gemm_supported(H.CHALF) == 0
+    plan = oh.ElemwisePlan()
+    assert oh.lib.och_elemwise_analyze(4, None, 0, None, None, None, C.byref(plan)) != 0
+    assert len(oh.lib.och_last_error()) > 0
+
+
+def test_support_tables_match_oracle():
+    for op in range(len(oh.BINARY_OPS)):
+        for dt in H.ALL_TYPES:
+            assert bool(oh.lib.och_binary_supported(op, dt)) == bool(orc.lib.oracle_binary_supported(op, dt)), (oh.BINARY_OPS[op], dt)
+    for op in range(len(oh.UNARY_OPS)):
+        for dt in H.ALL_TYPES:
+            assert bool(oh.lib.och_unary_supported(op, dt)) == bool(orc.lib.oracle_unary_supported(op, dt)), (oh.UNARY_OPS[op], dt)
+    for op in range(len(oh.REDUCE_OPS)):
+        for dt in H.ALL_TYPES:
+            sup = bool(oh.lib.och_reduce_supported(op, dt))
+            assert sup == bool(orc.lib.oracle_reduce_supported(op, dt)), (oh.REDUCE_OPS[op], dt)
+            if sup:
+                assert oh.lib.och_reduce_result_dtype(op, dt) == orc.lib.oracle_reduce_result_dtype(op, dt)
+
+
+def fastdiv(n, d, m, s1, s2):
+    t = (m * n) >> 32
+    return (t + ((n - t) >> s1)) >> s2
+
+
+def test_division_constants_exact():
+    """The kernels divide by dimension sizes with q = (t + ((n - t) >> s1)) >> s2, t = mulhi(m, n)."""
+    rng = np.random.default_rng(1)
+    divisors = [1, 2, 3, 4, 5, 7, 255, 256, 257, 641, 65535, 65536, 65537, (1 << 31) - 1, 1 << 31, (1 << 31) + 1, (1 << 32) - 1]
+    divisors += [int(x) for x in rng.integers(1, 1 << 32, 40)]
+    for d in divisors:
+        # a 2-D shape whose first dimension cannot merge with the second: dim 0 keeps size d
+        if d > 0x7FFF0000 or d < 2:             # (the whole shape must stay below 2^32 elements for one launch)
+            continue
+        plan = oh.elemwise_analyze([1], [d, 2], [[1, 2 * d + 3]], [0x10000])
+        assert plan.ndims == 2 and plan.launches == 1
+        for i in range(plan.ndims):
+            dd, m, s1, s2 = plan.div_d[i], plan.div_m[i], plan.div_s1[i], plan.div_s2[i]
+            assert dd >= 1
+            probes = [0, 1, dd - 1, dd, dd + 1, 2 * dd - 1, 2 * dd, (1 << 32) - 1, (1 << 32) - dd, (1 << 31)] + [int(x) for x in rng.integers(0, 1 << 32, 200)]
+            for n in probes:
+                if 0 <= n < (1 << 32):
+                    assert fastdiv(n, dd, m, s1, s2) == n // dd, (n, dd)
+    # exhaustive for small divisors over a 16-bit range plus the top of the 32-bit range
+    for d in range(1, 70):
+        plan = oh.elemwise_analyze([1], [d * 16, 2], [[1, 16 * d + 16]], [0x10000])
+        dd, m, s1, s2 = plan.div_d[0], plan.div_m[0], plan.div_s1[0], plan.div_s2[0]
+        n = np.concatenate([np.arange(0, 1 << 16, dtype=np.uint64), np.arange((1 << 32) - (1 << 12), 1 << 32, dtype=np.uint64)])
+        t = (np.uint64(m) * n) >> np.uint64(32)
+        q = (t + ((n - t) >> np.uint64(s1))) >> np.uint64(s2)
+        assert np.array_equal(q, n // np.uint64(dd)), dd
+
+
+def offsets_of(size, strides, base=0):
+    """Multiset of byte offsets visited by a strided operand."""
+    off = np.zeros([1] * 0, dtype=np.int64) + base
+    grids = np.meshgrid(*[np.arange(n, dtype=np.int64) for n in size], indexing="ij") if size else []
+    total = np.zeros(tuple(size), dtype=np.int64) + base
+    for g, s in zip(grids, strides):
+        total = total + g * s
+    return total
+
+
+def joint_offsets(size, strides_list, bases):
+    """Set of offset tuples (one entry per operand) visited together."""
+    cols = [offsets_of(size, st, b).reshape(-1) for st, b in zip(strides_list, bases)]
+    rows = np.stack(cols, axis=1)
+    return rows[np.lexsort(rows.T[::-1])]
+
+
+CASES = []
+_rng = np.random.default_rng(99)
+for _ in range(300):
+    nd = int(_rng.integers(0, 6))
+    size = [int(x) for x in _rng.choice([1, 1, 2, 3, 4, 5, 8, 16], size=nd)]
+    nops = int(_rng.integers(1, 4))
+    es = [int(x) for x in _rng.choice([1, 2, 4, 8, 16], size=nops)]
+    strides_list = []
+    for k in range(nops):
+        # a permuted, possibly padded, possibly reversed or broadcast layout
+        perm = _rng.permutation(nd)
+        st = [0] * nd
+        acc = es[k]
+        for d in perm:
+            mode = _rng.integers(0, 8)
+            if mode == 0 and k < nops - 1:
+                st[d] = 0                      # broadcast (inputs only)
+            else:
+                st[d] = acc * (-1 if mode == 1 else 1)
+                acc *= size[d] * (2 if mode == 2 else 1)
+        strides_list.append(st)
+    CASES.append((size, es, strides_list))
+
+
+@pytest.mark.parametrize("case", range(len(CASES)))
+def test_normalisation_preserves_offsets(case):
+    size, es, strides_list = CASES[case]
+    bases = [1 << 20] * len(es)
+    plan = oh.elemwise_analyze(es, size, strides_list, bases)
+    nelem = int(np.prod(size)) if size else 1
+    if nelem == 0:
+        assert plan.ndims == 0
+        return
+    nsize = [plan.size[d] for d in range(plan.ndims)]
+    assert int(np.prod(nsize)) == nelem
+    nstr = [[plan.strides[k][d] for d in range(plan.ndims)] for k in range(len(es))]
+    nbase = [bases[k] + plan.offset[k] for k in range(len(es))]
+    assert np.array_equal(joint_offsets(size, strides_list, bases), joint_offsets(nsize, nstr, nbase))
+    # canonical form: no unit dimensions (unless scalar), destination strides ascending and non-negative
+    key = nstr[-1]
+    if plan.ndims > 1:
+        assert all(n > 1 for n in nsize)
+    assert all(s >= 0 for s in key) or plan.ndims == 1
+    assert key == sorted(key)
+    # no two neighbouring dimensions are still mergeable
+    for d in range(plan.ndims - 1):
+        assert not all(nstr[k][d + 1] == nstr[k][d] * nsize[d] for k in range(len(es)))
+    assert plan.kernel in (oh.KERNEL_WIDE, oh.KERNEL_MIXED, oh.KERNEL_SINGLE, oh.KERNEL_TILED)
+    if plan.kernel != oh.KERNEL_SINGLE:
+        assert nsize[0] % plan.vec == 0 or plan.ndims == 1
+
+
+def test_kernel_choice():
+    a = 1 << 20
+    n = 4096
+    # contiguous float64 add: wide, 2 elements per access
+    p = oh.elemwise_analyze([8, 8, 8], [n, n], [[8, 8 * n]] * 3, [a, a, a])
+    assert (p.ndims, p.kernel, p.vec, p.launches) == (1, oh.KERNEL_WIDE, 2, 1)
+    # transposed input + row broadcast: tiled
+    p = oh.elemwise_analyze([8, 8, 8], [n, n], [[8 * n, 8], [0, 8], [8, 8 * n]], [a, a, a])
+    assert (p.ndims, p.kernel) == (2, oh.KERNEL_TILED)
+    # step-2 source: mixed
+    p = oh.elemwise_analyze([2, 4], [1024, 64], [[4, 4096], [4, 4096]], [a, a])
+    assert p.kernel == oh.KERNEL_MIXED and p.vec == 4
+    # odd length: vector body + scalar tail
+    p = oh.elemwise_analyze([4, 4, 4], [4099], [[4]] * 3, [a, a, a])
+    assert (p.kernel, p.launches) == (oh.KERNEL_WIDE, 2)
+    # misaligned pointer: cannot use wide accesses
+    p = oh.elemwise_analyze([4, 4, 4], [4096], [[4]] * 3, [a + 4, a, a])
+    assert p.kernel == oh.KERNEL_MIXED
+    # more than 2^32 elements: several launches
+    p = oh.elemwise_analyze([1], [1 << 33], [[1]], [a])
+    assert p.launches == 8 and p.kernel == oh.KERNEL_WIDE
+    # first dimension equal to the vector width (one group per row: divisor 1)
+    p = oh.elemwise_analyze([4, 4], [4, 5], [[4, 32], [4, 16]], [a, a])
+    assert p.div_d[0] == 1 and fastdiv(12345, 1, p.div_m[0], p.div_s1[0], p.div_s2[0]) == 12345

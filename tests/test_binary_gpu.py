@@ -190,3 +190,26 @@ def test_config1_scale_add_fp32(hip, stream):
     H.assert_same_bytes(got, zw, "config 1")
     # closed form: two separately rounded IEEE operations
     H.assert_same_bytes(got, (xd * yd) + xd, "config 1 vs numpy")
+
+
+@pytest.mark.parametrize("dtype", [H.INT8, H.INT16, H.FLOAT, H.DOUBLE, H.CFLOAT], ids=lambda d: H.NAMES[d])
+def test_binary_first_dimension_equals_access_width(hip, stream, dtype):
+    """Rows of exactly one 128-bit access (16 int8, 8 int16, 4 float, 2 double, 2 cfloat elements) with a
+    padded pitch: one group per row, so the group index is divided by one."""
+    op = oh.B["add"]
+    rng = np.random.default_rng(4242 + dtype)
+    w = 16 // oh.TYPE_SIZE[dtype]
+    for rows in (5, 64, 1000):
+        A = H.random_data(dtype, rows * 2 * w, rng).reshape(rows, 2 * w)
+        Bm = H.random_data(dtype, rows * 3 * w, rng).reshape(rows, 3 * w)
+        Z = np.zeros((rows, 2 * w), dtype=H.storage(dtype))
+        x = H.Operand(A, A[:, :w], dtype).upload(stream)
+        y = H.Operand(Bm, Bm[:, w:2 * w], dtype).upload(stream)
+        z = H.Operand(Z, Z[:, :w], dtype).upload(stream)
+        H.gpu_binary(stream, op, dtype, x, y, z)
+        want = Z.copy()
+        H.cpu_binary(op, dtype, x, y, z, want)
+        got = z.download()
+        for t in (x, y, z):
+            t.free()
+        H.assert_same_bytes(got, want, "rows of one access, %d rows" % rows)
