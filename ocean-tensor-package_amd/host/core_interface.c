@@ -1,0 +1,317 @@
+/* A small device-independent front end over the module table: what Ocean's interface layer does
+ * before it reaches a device function, restricted to the cases the benchmark configurations and
+ * the tests exercise. Follows src/core/interface/tensor_itf.c (copy :777-1041, ensure :1226-1304,
+ * binary :3983-4133, reductions :5299-5514, axis reductions :5522-5766, gemm :5951-6778) and
+ * src/core/generic/tensor_op.c:141-423 (common type, automatic casts, broadcasting, allocation).
+ */
+#include "ocean_host.h"
+#include <stdlib.h>
+#include <string.h>
+
+#define MODULE_OR_FAIL(m, device) OcModuleCore *m = OcModuleCore_forDevice(device); \
+   if (m == NULL) return OcErrorMessage("No core module is registered for device %s", (device) ? (device)->name : "(null)")
+
+/* ---- copy between any two tensors ------------------------------------------------------- */
+static int host_copy_same_type(OcTensor *src, OcTensor *dst)
+{  OcSize idx[OC_TENSOR_MAX_DIMS] = { 0 }, jdx[OC_TENSOR_MAX_DIMS] = { 0 }, i; int d, es = src->elemsize;
+   for (i = 0; i < src->nelem; i++)
+   {  OcIndex so = 0, dof = 0;
+      for (d = 0; d < src->ndims; d++) so += idx[d] * src->strides[d];
+      for (d = 0; d < dst->ndims; d++) dof += jdx[d] * dst->strides[d];
+      memcpy(OcTensor_data(dst) + dof, OcTensor_data(src) + so, (size_t)es);
+      for (d = 0; d < src->ndims; d++) { if (++idx[d] < src->size[d]) break; idx[d] = 0; }
+      for (d = 0; d < dst->ndims; d++) { if (++jdx[d] < dst->size[d]) break; jdx[d] = 0; }
+   }
+   return 0;
+}
+int OcTensor_copy(OcTensor *src, OcTensor *dst)
+{  if (src->nelem != dst->nelem) return OcErrorMessage("Mismatch in the number of elements in tensor copy");
+   if (src->device == OcCPU && dst->device == OcCPU)
+   {  if (src->dtype != dst->dtype || OcTensor_isByteswapped(src) != OcTensor_isByteswapped(dst))
+         return OcErrorMessage("Converting copies between host tensors need the CPU device module, which is not part of this build");
+      return host_copy_same_type(src, dst);
+   }
+   if (src->device == OcCPU) { MODULE_OR_FAIL(m, dst->device); return m->Tensor_copyFromCPU(src, dst); }
+   if (dst->device == OcCPU) { MODULE_OR_FAIL(m, src->device); return m->Tensor_copyToCPU(src, dst); }
+   {  MODULE_OR_FAIL(m, dst->device); return m->Tensor_copy(src, dst); }
+}
+
+/* Replace *tensor by a native-order tensor of the requested type on the requested device when it is not one
+   already (tensor_itf.c:1226-1304). The replacement is a new column-major tensor; the old reference is released. */
+int OcTensor_ensure(OcTensor **tensor, OcDType dtype, OcDevice *device)
+{  OcTensor *t = *tensor, *r;
+   if (dtype == OcDTypeNone) dtype = t->dtype;
+   if (device == NULL) device = t->device;
+   if (t->dtype == dtype && t->device == device && !OcTensor_isByteswapped(t)) return 0;
+   if ((r = OcTensor_create(t->ndims, t->size, NULL, dtype, device)) == NULL) return -1;
+   if (OcTensor_copy(t, r) != 0) { OcDecrefTensor(r); return -1; }
+   OcDecrefTensor(t);
+   *tensor = r;
+   return 0;
+}
+int OcTensor_fill(OcTensor *tensor, OcScalar *value)
+{  MODULE_OR_FAIL(m, tensor->device);
+   return m->Tensor_fill(tensor, value);
+}
+
+/* ---- elementwise -------------------------------------------------------------------------- */
+typedef int (*oc_binary_fn)(OcTensor *, OcTensor *, OcTensor *);
+typedef int (*oc_unary_fn)(OcTensor *, OcTensor *);
+#define OC_NBINARY 27
+#define OC_NUNARY 40
+
+/* broadcast shape of two tensors: dimensions align from the first; missing trailing dimensions count as 1 */
+static int broadcast_shape(OcTensor *a, OcTensor *b, int *ndims, OcSize *size)
+{  int i, n = a->ndims > b->ndims ? a->ndims : b->ndims;
+   for (i = 0; i < n; i++)
+   {  OcSize sa = i < a->ndims ? a->size[i] : 1, sb = i < b->ndims ? b->size[i] : 1;
+      if (sa != sb && sa != 1 && sb != 1) return OcErrorMessage("Tensor dimensions are not compatible (dimension %d: %td and %td)", i, sa, sb);
+      size[i] = (sa == 1) ? sb : sa;
+   }
+   *ndims = n;
+   return 0;
+}
+int OcTensor_binary(int op, OcTensor *src1, OcTensor *src2, OcTensor **dst)
+{  OcTensor *a = NULL, *b = NULL, *va = NULL, *vb = NULL, *out = NULL; OcSize size[OC_TENSOR_MAX_DIMS]; int ndims = 0, result = -1;
+   OcDevice *device = src1->device != OcCPU ? src1->device : (src2->device != OcCPU ? src2->device : ((*dst) ? (*dst)->device : OcCPU));
+   OcDType dtype, dtype2, rtype; oc_binary_fn fn; int is_compare = (op >= 13 && op <= 18), is_shift = (op >= 25), is_logical = (op >= 22 && op <= 24);
+   if (op < 0 || op >= OC_NBINARY) return OcErrorMessage("Invalid binary operation index (%d)", op);
+   {  MODULE_OR_FAIL(m, device);
+      fn = ((oc_binary_fn *)&m->Tensor_add)[op];
+      if (fn == NULL) return OcErrorMessage("Tensor operation is not supported on device %s", device->name);
+   }
+   /* common type of the operands; shifts keep the type of the first operand and take int8 counts,
+      integer powers take int16 exponents, logical operations work on bool */
+   dtype = is_shift ? src1->dtype : OcDType_getCommonType(src1->dtype, src2->dtype);
+   if (is_logical) dtype = OcDTypeBool;
+   dtype2 = dtype;
+   if (is_shift) dtype2 = OcDTypeInt8;
+   if (op == 6 && !OcDType_isFloat(dtype)) dtype2 = OcDTypeInt16;
+   rtype = is_compare ? OcDTypeBool : dtype;
+   a = OcIncrefTensor(src1); b = OcIncrefTensor(src2);
+   if (OcTensor_ensure(&a, dtype, device) != 0 || OcTensor_ensure(&b, dtype2, device) != 0) goto final;
+   if (broadcast_shape(a, b, &ndims, size) != 0) goto final;
+   if ((va = OcTensor_broadcastTo(a, ndims, size)) == NULL || (vb = OcTensor_broadcastTo(b, ndims, size)) == NULL) goto final;
+   if (*dst == NULL)
+   {  if ((out = OcTensor_create(ndims, size, NULL, rtype, device)) == NULL) goto final;
+      result = fn(va, vb, out);
+      if (result == 0) { *dst = out; out = NULL; }
+   }
+   else if ((*dst)->dtype == rtype && (*dst)->device == device && !OcTensor_isByteswapped(*dst))
+   {  OcTensor *vd = OcTensor_broadcastTo(*dst, ndims, size);          /* shape check: must not actually broadcast */
+      int i, ok = (vd != NULL);
+      for (i = 0; ok && i < ndims; i++) if ((i < (*dst)->ndims ? (*dst)->size[i] : 1) != size[i]) ok = 0;
+      if (!ok) { if (vd) OcDecrefTensor(vd); if (vd) OcErrorMessage("Destination size does not match the operands"); goto final; }
+      result = fn(va, vb, vd);
+      OcDecrefTensor(vd);
+   }
+   else
+   {  /* compute in the working type, then convert into the caller's destination */
+      if ((out = OcTensor_create(ndims, size, NULL, rtype, device)) == NULL) goto final;
+      if (fn(va, vb, out) != 0) goto final;
+      result = OcTensor_copy(out, *dst);
+   }
+final:
+   if (out) OcDecrefTensor(out);
+   if (va) OcDecrefTensor(va);
+   if (vb) OcDecrefTensor(vb);
+   if (a) OcDecrefTensor(a);
+   if (b) OcDecrefTensor(b);
+   return result;
+}
+int OcTensor_unary(int op, OcTensor *src, OcTensor **dst)
+{  OcTensor *a = NULL, *out = NULL; oc_unary_fn fn; int result = -1; OcDType rtype;
+   if (op < 0 || op >= OC_NUNARY) return OcErrorMessage("Invalid unary operation index (%d)", op);
+   {  MODULE_OR_FAIL(m, src->device);
+      fn = ((oc_unary_fn *)&m->Tensor_negative)[op];
+      if (fn == NULL) return OcErrorMessage("Tensor operation is not supported on device %s", src->device->name);
+   }
+   a = OcIncrefTensor(src);
+   if (OcTensor_ensure(&a, a->dtype, a->device) != 0) goto final;
+   rtype = a->dtype;
+   if (op >= 35) rtype = OcDTypeBool;                                       /* isinf ... isneginf */
+   if (op == 28 && OcDType_isComplex(a->dtype)) rtype = OcDType_getBaseType(a->dtype);   /* absolute of complex is real */
+   if (*dst && (*dst)->dtype == rtype && (*dst)->device == a->device && !OcTensor_isByteswapped(*dst)) result = fn(a, *dst);
+   else
+   {  if ((out = OcTensor_create(a->ndims, a->size, NULL, rtype, a->device)) == NULL) goto final;
+      if ((result = fn(a, out)) != 0) goto final;
+      if (*dst) result = OcTensor_copy(out, *dst); else { *dst = out; out = NULL; }
+   }
+final:
+   if (out) OcDecrefTensor(out);
+   if (a) OcDecrefTensor(a);
+   return result;
+}
+
+/* ---- reductions ------------------------------------------------------------------------------ */
+int OcTensor_reduceAll(int which, OcTensor *tensor, double p, OcScalar *result)
+{  OcTensor *a = OcIncrefTensor(tensor); int r = -1;
+   if (OcTensor_ensure(&a, a->dtype, a->device) == 0)          /* native byte order (tensor_itf.c:5308) */
+   {  OcModuleCore *m = OcModuleCore_forDevice(a->device);
+      if (m == NULL) OcErrorMessage("No core module is registered for device %s", a->device->name);
+      else switch (which)
+      {  case 15: r = m->Tensor_sum(a, result); break;        case 16: r = m->Tensor_sumNaN(a, result); break;
+         case 17: r = m->Tensor_prod(a, result); break;       case 18: r = m->Tensor_prodNaN(a, result); break;
+         case 19: r = m->Tensor_sumAbs(a, result); break;     case 20: r = m->Tensor_sumAbsNaN(a, result); break;
+         case 21: r = m->Tensor_maximum(a, result); break;    case 22: r = m->Tensor_minimum(a, result); break;
+         case 23: r = m->Tensor_maximumAbs(a, result); break; case 24: r = m->Tensor_minimumAbs(a, result); break;
+         case 25: r = m->Tensor_norm(a, p, result); break;    case 26: r = m->Tensor_normNaN(a, p, result); break;
+         case 27: r = m->Tensor_norm2(a, result); break;      case 28: r = m->Tensor_norm2NaN(a, result); break;
+         default: OcErrorMessage("Reduction %d does not return a scalar", which);
+      }
+   }
+   OcDecrefTensor(a);
+   return r;
+}
+int OcTensor_sum(OcTensor *t, OcScalar *r)     { return OcTensor_reduceAll(15, t, 0.0, r); }
+int OcTensor_maximum(OcTensor *t, OcScalar *r) { return OcTensor_reduceAll(21, t, 0.0, r); }
+int OcTensor_norm2(OcTensor *t, OcScalar *r)   { return OcTensor_reduceAll(27, t, 0.0, r); }
+
+typedef int (*oc_axis_fn)(OcTensor *, int, int *, OcTensor *);
+static OcDType reduce_result_type(int which, OcDType d)
+{  int isbool = (d == OcDTypeBool), isuint = (d >= OcDTypeUInt8 && d <= OcDTypeUInt64), issint = (d >= OcDTypeInt8 && d <= OcDTypeInt64);
+   OcDType mag = OcDType_isComplex(d) ? OcDType_getBaseType(d) : (issint ? (OcDType)(d - 4) : d);
+   if (which <= 4) return OcDTypeBool;
+   if (which <= 6) return OcDTypeUInt64;
+   if (which >= 15 && which <= 18) return (isbool || isuint) ? OcDTypeUInt64 : (issint ? OcDTypeInt64 : d);
+   if (which == 19 || which == 20) return (isbool || isuint || issint) ? OcDTypeUInt64 : mag;
+   if (which == 21 || which == 22) return d;
+   if (which == 23 || which == 24) return mag;
+   return (isbool || isuint || issint) ? OcDTypeDouble : mag;
+}
+/* axes validated, made unique and non-negative (tensor_itf.c:5537-5554); dst created when *dst is NULL */
+int OcTensor_axisReduce(int which, OcTensor *src, int n, int *axes, int keepdims, double p, OcTensor **dst)
+{  int flag[OC_TENSOR_MAX_DIMS] = { 0 }, ax[OC_TENSOR_MAX_DIMS], i, j, nd = 0, r = -1; OcSize size[OC_TENSOR_MAX_DIMS];
+   OcTensor *a, *out = NULL; OcModuleCore *m; OcDType rtype;
+   static const int order[] = { 0, 1, 2, 3, 4, 5, 6, 15, 17, 16, 18, 19, 20, 22, 21, 24, 23, 27, 28 };   /* table order of the axis block */
+   for (i = 0, j = 0; i < n; i++)
+   {  int k = axes[i] < 0 ? axes[i] + src->ndims : axes[i];
+      if (k < 0 || k >= src->ndims) return OcErrorMessage("Axis index %d out of range", axes[i]);
+      if (flag[k]) return OcErrorMessage("Repeated axis index %d", axes[i]);
+      flag[k] = 1; ax[j++] = k;
+   }
+   for (i = 0; i < src->ndims; i++) { if (!flag[i]) size[nd++] = src->size[i]; else if (keepdims) size[nd++] = 1; }
+   a = OcIncrefTensor(src);
+   if (OcTensor_ensure(&a, a->dtype, a->device) != 0) goto final;
+   if ((m = OcModuleCore_forDevice(a->device)) == NULL) { OcErrorMessage("No core module is registered for device %s", a->device->name); goto final; }
+   rtype = reduce_result_type(which, a->dtype);
+   if (*dst && (*dst)->dtype == rtype && (*dst)->device == a->device && !OcTensor_isByteswapped(*dst)) out = OcIncrefTensor(*dst);
+   else if ((out = OcTensor_create(nd, size, NULL, rtype, a->device)) == NULL) goto final;
+   if (out->ndims != nd) { OcErrorMessage("Destination has %d dimensions, expected %d", out->ndims, nd); goto final; }
+   for (i = 0; i < nd; i++) if (out->size[i] != size[i]) { OcErrorMessage("Destination size mismatch in dimension %d", i); goto final; }
+   if (which == 25) r = m->Tensor_axisNorm(a, p, j, ax, out);
+   else if (which == 26) r = m->Tensor_axisNormNaN(a, p, j, ax, out);
+   else
+   {  oc_axis_fn fn = NULL;
+      for (i = 0; i < (int)(sizeof(order) / sizeof(order[0])); i++) if (order[i] == which) fn = ((oc_axis_fn *)&m->Tensor_axisAny)[i];
+      if (fn == NULL) { OcErrorMessage("Axis reduction %d is not available", which); goto final; }
+      r = fn(a, j, ax, out);
+   }
+   if (r == 0 && *dst == NULL) { *dst = out; out = NULL; }
+   else if (r == 0 && *dst != out) r = OcTensor_copy(out, *dst);
+final:
+   if (out) OcDecrefTensor(out);
+   OcDecrefTensor(a);
+   return r;
+}
+
+/* ---- GEMM ---------------------------------------------------------------------------------------- */
+/* C <- alpha op(A) op(B) + beta C. Operands are brought to one type; an operand whose columns are not
+   contiguous is either used through the opposite transposition (when its rows are contiguous) or copied
+   (tensor_itf.c:6137-6778); alpha and beta become one-element host tensors of that type (:5951-5992). */
+static OcTensor *scalar_tensor(OcScalar *s, OcDType dtype, double fallback)
+{  OcSize one = 1; OcTensor *t = OcTensor_create(0, &one, NULL, dtype, OcCPU); char *p;
+   double re = fallback, im = 0;
+   if (t == NULL) return NULL;
+   if (s)
+      switch (s->dtype)
+      {  case OcDTypeBool: re = s->value.sBool; break;      case OcDTypeUInt8: re = s->value.sUInt8; break;
+         case OcDTypeUInt16: re = s->value.sUInt16; break;  case OcDTypeUInt32: re = s->value.sUInt32; break;
+         case OcDTypeUInt64: re = (double)s->value.sUInt64; break; case OcDTypeInt8: re = s->value.sInt8; break;
+         case OcDTypeInt16: re = s->value.sInt16; break;    case OcDTypeInt32: re = s->value.sInt32; break;
+         case OcDTypeInt64: re = (double)s->value.sInt64; break;   case OcDTypeFloat: re = s->value.sFloat; break;
+         case OcDTypeDouble: re = s->value.sDouble; break;
+         case OcDTypeCFloat: re = s->value.sCFloat.real; im = s->value.sCFloat.imag; break;
+         case OcDTypeCDouble: re = s->value.sCDouble.real; im = s->value.sCDouble.imag; break;
+         default: OcErrorMessage("Half-precision scalars are not supported by this front end"); OcDecrefTensor(t); return NULL;
+      }
+   p = OcTensor_data(t);
+   switch (dtype)
+   {  case OcDTypeBool: *(OcBool *)p = (re != 0); break;       case OcDTypeUInt8: *(OcUInt8 *)p = (OcUInt8)re; break;
+      case OcDTypeUInt16: *(OcUInt16 *)p = (OcUInt16)re; break; case OcDTypeUInt32: *(OcUInt32 *)p = (OcUInt32)re; break;
+      case OcDTypeUInt64: *(OcUInt64 *)p = (OcUInt64)re; break; case OcDTypeInt8: *(OcInt8 *)p = (OcInt8)re; break;
+      case OcDTypeInt16: *(OcInt16 *)p = (OcInt16)re; break;   case OcDTypeInt32: *(OcInt32 *)p = (OcInt32)re; break;
+      case OcDTypeInt64: *(OcInt64 *)p = (OcInt64)re; break;   case OcDTypeFloat: *(OcFloat *)p = (OcFloat)re; break;
+      case OcDTypeDouble: *(OcDouble *)p = re; break;
+      case OcDTypeCFloat: ((OcCFloat *)p)->real = (OcFloat)re; ((OcCFloat *)p)->imag = (OcFloat)im; break;
+      case OcDTypeCDouble: ((OcCDouble *)p)->real = re; ((OcCDouble *)p)->imag = im; break;
+      default: OcErrorMessage("GEMM scalars of type %s are not supported by this front end", OcDType_name(dtype)); OcDecrefTensor(t); return NULL;
+   }
+   return t;
+}
+/* leading dimension of a matrix operand, flipping the mode when only its rows are contiguous */
+static int gemm_operand(OcTensor **t, char *mode, OcIndex *ld, int complex_type)
+{  OcTensor *x = *t; int es = x->elemsize;
+   if (x->ndims != 2) return OcErrorMessage("This front end multiplies two-dimensional tensors");
+   if ((x->size[0] == 1 || x->strides[0] == es) && (x->size[1] == 1 || (x->strides[1] >= x->size[0] * es && x->strides[1] % es == 0)))
+   {  *ld = (x->size[1] == 1) ? (x->size[0] > 0 ? x->size[0] : 1) : x->strides[1] / es; return 0; }
+   if ((x->size[1] == 1 || x->strides[1] == es) && (x->size[0] == 1 || (x->strides[0] >= x->size[1] * es && x->strides[0] % es == 0)) && !(complex_type && *mode == 'C'))
+   {  /* rows contiguous: the stored matrix is the transpose */
+      OcTensor *v = OcTensor_transpose(x);
+      if (v == NULL) return -1;
+      *ld = (v->size[1] == 1) ? (v->size[0] > 0 ? v->size[0] : 1) : v->strides[1] / es;
+      *mode = (*mode == 'N') ? 'T' : 'N';
+      OcDecrefTensor(x); *t = v;
+      return 0;
+   }
+   {  OcTensor *r = OcTensor_create(2, x->size, NULL, x->dtype, x->device);
+      if (r == NULL) return -1;
+      if (OcTensor_copy(x, r) != 0) { OcDecrefTensor(r); return -1; }
+      OcDecrefTensor(x); *t = r; *ld = r->size[0] > 0 ? r->size[0] : 1;
+      return 0;
+   }
+}
+int OcTensor_gemm(OcScalar *alpha, OcTensor *A, char modeA, OcTensor *B, char modeB, OcScalar *beta, OcTensor **C)
+{  OcTensor *a = OcIncrefTensor(A), *b = OcIncrefTensor(B), *c = NULL, *ta = NULL, *tb = NULL; int result = -1;
+   OcDevice *device = A->device != OcCPU ? A->device : B->device; OcDType dtype = OcDType_getCommonType(A->dtype, B->dtype);
+   OcSize M, N, K, K2, csize[2]; OcIndex ldA, ldB, ldC; OcModuleCore *m = OcModuleCore_forDevice(device);
+   if (*C) dtype = OcDType_getCommonType(dtype, (*C)->dtype);
+   if (m == NULL) { OcErrorMessage("No core module is registered for device %s", device->name); goto final; }
+   if (!m->Tensor_gemmSupportedOn(device, dtype)) { OcErrorMessage("Matrix multiplication is not supported for type %s on %s", OcDType_name(dtype), device->name); goto final; }
+   if (A->ndims != 2 || B->ndims != 2) { OcErrorMessage("This front end multiplies two-dimensional tensors"); goto final; }
+   M = (modeA == 'N') ? A->size[0] : A->size[1]; K = (modeA == 'N') ? A->size[1] : A->size[0];
+   K2 = (modeB == 'N') ? B->size[0] : B->size[1]; N = (modeB == 'N') ? B->size[1] : B->size[0];
+   if (K != K2) { OcErrorMessage("Inner dimensions do not match (%td and %td)", K, K2); goto final; }
+   if (OcTensor_ensure(&a, dtype, device) != 0 || OcTensor_ensure(&b, dtype, device) != 0) goto final;
+   if (gemm_operand(&a, &modeA, &ldA, OcDType_isComplex(dtype)) != 0 || gemm_operand(&b, &modeB, &ldB, OcDType_isComplex(dtype)) != 0) goto final;
+   csize[0] = M; csize[1] = N;
+   if (*C == NULL) { if ((c = OcTensor_create(2, csize, NULL, dtype, device)) == NULL) goto final; }
+   else
+   {  c = OcIncrefTensor(*C);
+      if (c->ndims != 2 || c->size[0] != M || c->size[1] != N) { OcErrorMessage("Destination size does not match the product"); goto final; }
+      if (c->dtype != dtype || c->device != device || OcTensor_isByteswapped(c) || (M > 1 && c->strides[0] != c->elemsize) ||
+          (N > 1 && (c->strides[1] < M * c->elemsize || c->strides[1] % c->elemsize != 0)))
+      {  if (OcTensor_ensure(&c, dtype, device) != 0) goto final;
+         if (c == *C)                                   /* same type but unusable layout: work on a dense copy */
+         {  OcTensor *r = OcTensor_create(2, csize, NULL, dtype, device);
+            if (r == NULL || OcTensor_copy(c, r) != 0) { if (r) OcDecrefTensor(r); goto final; }
+            OcDecrefTensor(c); c = r;
+         }
+      }
+   }
+   ldC = (N > 1) ? c->strides[1] / c->elemsize : (M > 0 ? M : 1);
+   if ((ta = scalar_tensor(alpha, dtype, 1.0)) == NULL || (tb = scalar_tensor(beta, dtype, 0.0)) == NULL) goto final;
+   /* the caller runs the stream protocol around Tensor_gemm (tensor_itf.c:6727-6750) */
+   if (OcTensor_startRead(c, a) != 0 || OcTensor_startRead(c, b) != 0) goto final;
+   result = m->Tensor_gemm(M, N, K, modeA, modeB, ta, a, ldA, b, ldB, tb, c, ldC);
+   if (result == 0 && (OcTensor_update(c) != 0 || OcTensor_finishRead(c, a) != 0 || OcTensor_finishRead(c, b) != 0)) result = -1;
+   if (result == 0 && *C == NULL) { *C = c; c = NULL; }
+   else if (result == 0 && c != *C) result = OcTensor_copy(c, *C);
+final:
+   if (ta) OcDecrefTensor(ta);
+   if (tb) OcDecrefTensor(tb);
+   if (c) OcDecrefTensor(c);
+   OcDecrefTensor(a); OcDecrefTensor(b);
+   return result;
+}
+int OcTensor_mtimes(OcTensor *A, OcTensor *B, OcTensor **C) { return OcTensor_gemm(NULL, A, 'N', B, 'N', NULL, C); }

@@ -1,0 +1,540 @@
+/* The "GPU" device module of Ocean's core module on top of libocean_hip.so.
+ *
+ * Mirrors src/core/gpu: OcInitGPU (ocean_gpu.c:38-58), device / stream / event objects with
+ * free lists (device_gpu.c:81-420), storage (storage_gpu.c:61-302), module registration
+ * (module_core_gpu.c:40-145) and one glue function per table entry (the files under src/core/gpu/op).
+ * Every glue function activates the device, runs the stream protocol the reference runs and makes
+ * ONE call into the device library; function-table lookups by data type become the
+ * (operation, dtype) arguments of that call, and a missing table entry becomes an error from
+ * och_*_supported.
+ */
+#include "ocean_host.h"
+#include "../../include/ocean_hip.h"
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ---- device objects -------------------------------------------------------------- */
+#define OC_GPU_MAX_FREE 64                       /* free-list bound, device_gpu.c:251-370 */
+typedef struct { OcStream HEAD; och_stream handle; } OcStreamGPU;
+typedef struct { OcEvent HEAD; och_event handle; } OcEventGPU;
+typedef struct
+{  OcDevice        HEAD;
+   och_device_prop properties;
+   OcStream       *freeStreams;  int nFreeStreams;
+   OcEvent        *freeEvents;   int nFreeEvents;
+} OcDeviceGPU;
+
+OcDevice **OcGPU = NULL;
+static int oc_gpu_count = 0;
+static int oc_gpu_initialized = 0;
+static OcModuleCore oc_module_core_gpu;          /* the table Ocean copies at registration */
+static OcModuleCore oc_registered_gpu;           /* the registered copy (device_module.c:415) */
+static int oc_registered = 0;
+
+#define OCH_CALL(x) do { if ((x) != 0) return OcErrorMessage("%s", och_last_error()); } while (0)
+#define GPU_STREAM(t) (((OcStreamGPU *)((t)->storage->stream))->handle)
+static int activate(OcDevice *device) { if (och_device_set(device->index) != 0) return OcErrorMessage("%s", och_last_error()); return 0; }
+
+static OcStream *gpu_create_stream(OcDevice *device)
+{  OcDeviceGPU *g = (OcDeviceGPU *)device; OcStreamGPU *s;
+   if (g->freeStreams)
+   {  s = (OcStreamGPU *)g->freeStreams; g->freeStreams = s->HEAD.next; g->nFreeStreams--; }
+   else
+   {  if (activate(device) != 0) return NULL;
+      s = (OcStreamGPU *)calloc(1, sizeof(OcStreamGPU));
+      if (s == NULL) { OcErrorMessage("Insufficient memory to allocate a stream object"); return NULL; }
+      if (och_stream_create(&s->handle) != 0) { OcErrorMessage("%s", och_last_error()); free(s); return NULL; }
+   }
+   s->HEAD.device = device; s->HEAD.next = NULL; s->HEAD.refcount = 1;
+   return &s->HEAD;
+}
+static void gpu_delete_stream(OcStream *stream)
+{  OcDeviceGPU *g;
+   if (stream == NULL || --stream->refcount > 0) return;
+   g = (OcDeviceGPU *)stream->device;
+   if (g->nFreeStreams < OC_GPU_MAX_FREE) { stream->next = g->freeStreams; g->freeStreams = stream; g->nFreeStreams++; }
+   else { och_stream_destroy(((OcStreamGPU *)stream)->handle); free(stream); }
+}
+static int gpu_create_event(OcDevice *device, OcEvent **event)
+{  OcDeviceGPU *g = (OcDeviceGPU *)device; OcEventGPU *e;
+   if (g->freeEvents) { e = (OcEventGPU *)g->freeEvents; g->freeEvents = e->HEAD.next; g->nFreeEvents--; }
+   else
+   {  if (activate(device) != 0) return -1;
+      e = (OcEventGPU *)calloc(1, sizeof(OcEventGPU));
+      if (e == NULL) return OcErrorMessage("Insufficient memory to allocate an event object");
+      if (och_event_create(&e->handle, 0) != 0) { free(e); return OcErrorMessage("%s", och_last_error()); }
+   }
+   e->HEAD.next = NULL; *event = &e->HEAD;
+   return 0;
+}
+static void gpu_delete_event(OcDevice *device, OcEvent *event)
+{  OcDeviceGPU *g = (OcDeviceGPU *)device;
+   if (event == NULL) return;
+   if (g->nFreeEvents < OC_GPU_MAX_FREE) { event->next = g->freeEvents; g->freeEvents = event; g->nFreeEvents++; }
+   else { och_event_destroy(((OcEventGPU *)event)->handle); free(event); }
+}
+static int gpu_sync_stream(OcStream *s)  { OCH_CALL(och_stream_synchronize(((OcStreamGPU *)s)->handle)); return 0; }
+static int gpu_sync_event(OcEvent *e)    { OCH_CALL(och_event_synchronize(((OcEventGPU *)e)->handle)); return 0; }
+static int gpu_record_event(OcEvent *e, OcStream *s) { OCH_CALL(och_event_record(((OcEventGPU *)e)->handle, ((OcStreamGPU *)s)->handle)); return 0; }
+static int gpu_wait_event(OcStream *s, OcEvent *e)   { OCH_CALL(och_stream_wait_event(((OcStreamGPU *)s)->handle, ((OcEventGPU *)e)->handle)); return 0; }
+static void gpu_finalize_device(OcDevice *device)
+{  OcDeviceGPU *g = (OcDeviceGPU *)device;
+   while (g->freeStreams) { OcStream *s = g->freeStreams; g->freeStreams = s->next; och_stream_destroy(((OcStreamGPU *)s)->handle); free(s); }
+   while (g->freeEvents)  { OcEvent *e = g->freeEvents; g->freeEvents = e->next; och_event_destroy(((OcEventGPU *)e)->handle); free(e); }
+}
+
+/* ---- storage ---------------------------------------------------------------------- */
+static void gpu_storage_finalize(OcStorage *storage)
+{  if ((storage->flags & OC_STORAGE_OWNER) && storage->data)
+   {  och_device_set(storage->stream->device->index);
+      och_free_async(storage->data, ((OcStreamGPU *)storage->stream)->handle);
+   }
+}
+static OcStorage *OcStorageGPU_create(OcSize nelem, OcDType dtype, OcDevice *device, OcStream *stream)
+{  OcStorage *s; void *ptr = NULL;
+   if (activate(device) != 0) return NULL;
+   s = (OcStorage *)calloc(1, sizeof(OcStorage));
+   if (s == NULL) { OcErrorMessage("Insufficient memory to allocate the storage object"); return NULL; }
+   s->elemsize = OcDType_size(dtype); s->dtype = dtype; s->nelem = nelem; s->size = s->capacity = nelem * s->elemsize;
+   if (stream == NULL) stream = device->defaultStream;
+   stream->refcount++; s->stream = stream;
+   if (gpu_create_event(device, &s->event) != 0) { gpu_delete_stream(stream); free(s); return NULL; }
+   if (och_malloc_async(&ptr, (size_t)(s->size > 0 ? s->size : 1), ((OcStreamGPU *)stream)->handle) != 0)
+   {  OcErrorMessage("%s", och_last_error()); gpu_delete_event(device, s->event); gpu_delete_stream(stream); free(s); return NULL; }
+   s->data = (char *)ptr; s->flags = OC_STORAGE_OWNER; s->refcount = 1; s->finalize = gpu_storage_finalize;
+   return s;
+}
+static int OcBufferGPU_copy(OcStorage *src, void *srcData, OcStorage *dst, void *dstData, OcDType dtype, OcSize n)
+{  if (src->stream->device != dst->stream->device) return OcErrorMessage("Copies between GPU devices are not part of this build (one device)");
+   if (activate(dst->stream->device) != 0 || OcStorage_startRead(dst, src) != 0) return -1;
+   OCH_CALL(och_memcpy_dtod_async(dstData, srcData, (size_t)(n * OcDType_size(dtype)), ((OcStreamGPU *)dst->stream)->handle));
+   return OcStorage_finishRead(dst, src);
+}
+static int OcBufferGPU_copyFromCPU(OcStorage *src, void *srcData, OcStorage *dst, void *dstData, OcDType dtype, OcSize n)
+{  (void)src;
+   if (activate(dst->stream->device) != 0) return -1;
+   OCH_CALL(och_memcpy_htod(dstData, srcData, (size_t)(n * OcDType_size(dtype)), ((OcStreamGPU *)dst->stream)->handle));   /* blocking, storage_gpu.c:165-189 */
+   return 0;
+}
+static int OcBufferGPU_copyToCPU(OcStorage *src, void *srcData, OcStorage *dst, void *dstData, OcDType dtype, OcSize n)
+{  (void)dst;
+   if (activate(src->stream->device) != 0) return -1;
+   OCH_CALL(och_memcpy_dtoh(dstData, srcData, (size_t)(n * OcDType_size(dtype)), ((OcStreamGPU *)src->stream)->handle));
+   return 0;
+}
+static int OcBufferGPU_copyHostStorage(OcStorage *storage, OcSize offset, OcSize nbytes, void *ptr)
+{  if (activate(storage->stream->device) != 0) return -1;
+   OCH_CALL(och_memcpy_htod(storage->data + offset, ptr, (size_t)nbytes, ((OcStreamGPU *)storage->stream)->handle));
+   return 0;
+}
+static int OcBufferGPU_copyStorageHost(OcStorage *storage, OcSize offset, OcSize nbytes, void *ptr)
+{  if (activate(storage->stream->device) != 0) return -1;
+   OCH_CALL(och_memcpy_dtoh(ptr, storage->data + offset, (size_t)nbytes, ((OcStreamGPU *)storage->stream)->handle));
+   return 0;
+}
+static int OcBufferGPU_zero(OcStorage *storage, void *data, OcDType dtype, OcSize size)
+{  if (activate(storage->stream->device) != 0) return -1;
+   OCH_CALL(och_memset_async(data, 0, (size_t)(size * OcDType_size(dtype)), ((OcStreamGPU *)storage->stream)->handle));
+   return 0;
+}
+static int OcDeviceGPU_formatInfo(OcDevice *device, char **str, const char *header, const char *footer)
+{  OcDeviceGPU *g = (OcDeviceGPU *)device; size_t n = 512 + (header ? strlen(header) : 0) + (footer ? strlen(footer) : 0);
+   if ((*str = (char *)malloc(n)) == NULL) return OcErrorMessage("Insufficient memory for the device description");
+   snprintf(*str, n, "%sDevice %s: %s (%s), %d compute units, %.1f GiB%s", header ? header : "", device->name, g->properties.name,
+            g->properties.arch, g->properties.multiprocessor_count, g->properties.total_global_mem / 1073741824.0, footer ? footer : "");
+   return 0;
+}
+
+/* ---- helpers for the glue ------------------------------------------------------------ */
+static void scalar_value(const OcScalar *s, och_scalar *v) { memset(v, 0, sizeof(*v)); memcpy(v, &s->value, sizeof(*v) < sizeof(s->value) ? sizeof(*v) : sizeof(s->value)); }
+static int same_shape(OcTensor *a, OcTensor *b)
+{  int i; if (a->ndims != b->ndims) return 0;
+   for (i = 0; i < a->ndims; i++) if (a->size[i] != b->size[i]) return 0;
+   return 1;
+}
+#define SZ(t) ((const size_t *)(t)->size)
+
+/* ---- copy ------------------------------------------------------------------------------ */
+static int OcTensorGPU_copy(OcTensor *src, OcTensor *dst)
+{  /* the swapping copy reverses the bytes of the SOURCE elements and then converts; a destination kept in the
+      other byte order is swapped in place after a converting copy (src/core/cpu/op/tensor_copy_cpu.c:140-156) */
+   int differ = (src->dtype != dst->dtype);
+   int swap = differ ? OcTensor_isByteswapped(src) : (OcTensor_isByteswapped(src) != OcTensor_isByteswapped(dst));
+   if (src->device != dst->device) return OcErrorMessage("Copies between GPU devices are not part of this build (one device)");
+   if (src->nelem != dst->nelem) return OcErrorMessage("Mismatch in the number of elements in tensor copy");
+   if (dst->nelem == 0) return 0;
+   if (activate(dst->device) != 0 || OcTensor_startRead(dst, src) != 0) return -1;
+   OCH_CALL((swap ? och_byteswap_copy : och_copy)(src->dtype, dst->dtype, src->ndims, SZ(src), src->strides, OcTensor_data(src),
+                                                    dst->ndims, SZ(dst), dst->strides, OcTensor_data(dst), GPU_STREAM(dst)));
+   if (differ && OcTensor_isByteswapped(dst))
+      OCH_CALL(och_byteswap(dst->dtype, dst->ndims, SZ(dst), dst->strides, OcTensor_data(dst), GPU_STREAM(dst)));
+   if (OcTensor_update(dst) != 0) return -1;
+   return OcTensor_finishRead(dst, src);
+}
+/* Host tensors enter the device as raw bytes of their memory extent and are converted, re-strided and
+   byte-swapped there (tensor_copy_gpu.c:136-161 stages through an intermediate tensor likewise). */
+static int OcTensorGPU_copyFromCPU(OcTensor *src, OcTensor *dst)
+{  OcStorage *stage; OcTensor *view; int result;
+   if (src->nelem != dst->nelem) return OcErrorMessage("Mismatch in the number of elements in tensor copy");
+   if (dst->nelem == 0) return 0;
+   if ((stage = OcStorageGPU_create(src->blockExtent, OcDTypeInt8, dst->device, dst->storage->stream)) == NULL) return -1;
+   if (OcBufferGPU_copyFromCPU(src->storage, OcTensor_data(src) + src->blockOffset, stage, stage->data, OcDTypeInt8, src->blockExtent) != 0)
+   {  OcDecrefStorage(stage); return -1; }
+   view = OcTensor_createFromStorage(stage, src->ndims, src->size, src->strides, -src->blockOffset, src->dtype);
+   OcDecrefStorage(stage);
+   if (view == NULL) return -1;
+   view->flags = src->flags;
+   result = OcTensorGPU_copy(view, dst);
+   OcDecrefTensor(view);
+   return result;
+}
+static int OcTensorGPU_copyToCPU(OcTensor *src, OcTensor *dst)
+{  OcTensor *dense; int result; OcSize i, n = src->nelem; int es = dst->elemsize;
+   char *host;
+   if (src->nelem != dst->nelem) return OcErrorMessage("Mismatch in the number of elements in tensor copy");
+   if (n == 0) return 0;
+   /* convert / gather on the device into a dense tensor of the destination's type and byte order */
+   if ((dense = OcTensor_create(dst->ndims, dst->size, NULL, dst->dtype, src->device)) == NULL) return -1;
+   dense->flags |= (dst->flags & OC_TENSOR_BYTESWAPPED);
+   result = OcTensorGPU_copy(src, dense);
+   if (result == 0 && OcTensor_isContiguous(dst))
+      result = OcBufferGPU_copyToCPU(dense->storage, OcTensor_data(dense), dst->storage, OcTensor_data(dst), dst->dtype, n);
+   else if (result == 0)
+   {  /* strided host destination: download densely, then place element by element */
+      if ((host = (char *)malloc((size_t)(n * es))) == NULL) result = OcErrorMessage("Insufficient memory for the host staging buffer");
+      else
+      {  result = OcBufferGPU_copyToCPU(dense->storage, OcTensor_data(dense), dst->storage, host, dst->dtype, n);
+         if (result == 0)
+         {  OcSize idx[OC_TENSOR_MAX_DIMS] = { 0 }; int d;
+            for (i = 0; i < n; i++)
+            {  OcIndex off = 0;
+               for (d = 0; d < dst->ndims; d++) off += idx[d] * dst->strides[d];
+               memcpy(OcTensor_data(dst) + off, host + i * es, (size_t)es);
+               for (d = 0; d < dst->ndims; d++) { if (++idx[d] < dst->size[d]) break; idx[d] = 0; }
+            }
+         }
+         free(host);
+      }
+   }
+   OcDecrefTensor(dense);
+   return result;
+}
+static int OcTensorGPU_byteswapNoFlag(OcTensor *tensor)
+{  if (tensor->nelem == 0) return 0;
+   if (activate(tensor->device) != 0) return -1;
+   OCH_CALL(och_byteswap(tensor->dtype, tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), GPU_STREAM(tensor)));
+   return OcTensor_update(tensor);
+}
+
+/* ---- fill / steps ------------------------------------------------------------------------ */
+static int OcTensorGPU_fill(OcTensor *tensor, OcScalar *scalar)
+{  och_scalar v; scalar_value(scalar, &v);
+   if (scalar->dtype != tensor->dtype) return OcErrorMessage("Fill value must have the tensor's data type");
+   if (activate(tensor->device) != 0) return -1;
+   OCH_CALL(och_fill(tensor->dtype, tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), v, GPU_STREAM(tensor)));
+   return OcTensor_update(tensor);
+}
+static int OcTensorGPU_fillNaN(OcTensor *tensor, OcScalar *scalar)
+{  och_scalar v; scalar_value(scalar, &v);
+   if (!OcDType_isFloat(tensor->dtype)) return 0;                                    /* integers hold no NaN: nothing to do */
+   if (activate(tensor->device) != 0) return -1;
+   OCH_CALL(och_fill_nan(tensor->dtype, tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), v, GPU_STREAM(tensor)));
+   return OcTensor_update(tensor);
+}
+static int OcTensorGPU_maskedFill(OcTensor *tensor, OcTensor *mask, OcScalar *scalar)
+{  och_scalar v; scalar_value(scalar, &v);
+   if (mask->dtype != OcDTypeBool || !same_shape(tensor, mask)) return OcErrorMessage("Masked fill needs a Boolean mask of the tensor's shape");
+   if (activate(tensor->device) != 0 || OcTensor_startRead(tensor, mask) != 0) return -1;
+   OCH_CALL(och_masked_fill(tensor->dtype, tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), mask->strides, OcTensor_data(mask), v, GPU_STREAM(tensor)));
+   if (OcTensor_update(tensor) != 0) return -1;
+   return OcTensor_finishRead(tensor, mask);
+}
+static int OcTensorGPU_stepsInt64(OcTensor *tensor, OcInt64 offset, OcInt64 step)
+{  if (activate(tensor->device) != 0) return -1;
+   OCH_CALL(och_steps_int64(tensor->dtype, tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), offset, step, GPU_STREAM(tensor)));
+   return OcTensor_update(tensor);
+}
+static int OcTensorGPU_stepsDouble(OcTensor *tensor, OcDouble offset, OcDouble step)
+{  if (activate(tensor->device) != 0) return -1;
+   OCH_CALL(och_steps_double(tensor->dtype, tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), offset, step, GPU_STREAM(tensor)));
+   return OcTensor_update(tensor);
+}
+static int OcTensorGPU_stepsCDouble(OcTensor *tensor, OcCDouble offset, OcCDouble step)
+{  och_cdouble o, s; o.real = offset.real; o.imag = offset.imag; s.real = step.real; s.imag = step.imag;
+   if (activate(tensor->device) != 0) return -1;
+   OCH_CALL(och_steps_cdouble(tensor->dtype, tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), o, s, GPU_STREAM(tensor)));
+   return OcTensor_update(tensor);
+}
+
+/* ---- index operations (op/tensor_index_gpu.c:58-265) -------------------------------------- */
+static int OcTensorGPU_addIfNegative(OcTensor *tensor, OcScalar *scalar)
+{  och_scalar v; scalar_value(scalar, &v);
+   if (activate(tensor->device) != 0) return -1;
+   OCH_CALL(och_add_if_negative(tensor->dtype, tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), v, GPU_STREAM(tensor)));
+   return OcTensor_update(tensor);
+}
+/* tensor: nstrides x nelem indices; offsets: nelem int64 values */
+static int OcTensorGPU_indexToOffset(OcTensor *tensor, OcInt64 *strides, OcTensor *offsets)
+{  int nstrides = (tensor->ndims >= 1) ? (int)tensor->size[0] : 1;
+   OcSize nelem = (tensor->ndims >= 2) ? tensor->size[1] : 1;
+   if (offsets->dtype != OcDTypeInt64) return OcErrorMessage("Offsets must be int64");
+   if (activate(tensor->device) != 0 || OcTensor_startRead(offsets, tensor) != 0) return -1;
+   OCH_CALL(och_index_to_offset(tensor->dtype, nstrides, (const int64_t *)strides, tensor->ndims >= 1 ? tensor->strides[0] : 0, (size_t)nelem,
+                                tensor->ndims >= 2 ? tensor->strides[1] : 0, OcTensor_data(tensor),
+                                offsets->ndims >= 1 ? offsets->strides[0] : 0, OcTensor_data(offsets), GPU_STREAM(offsets)));
+   if (OcTensor_update(offsets) != 0) return -1;
+   return OcTensor_finishRead(offsets, tensor);
+}
+static int index_tables(OcTensorIndexView *view, int64_t **tables)
+{  int d;
+   for (d = 0; d < view->ndims; d++) tables[d] = (view->offsets && view->offsets[d]) ? (int64_t *)OcTensor_data(view->offsets[d]) : NULL;
+   return 0;
+}
+static int OcTensorGPU_getIndex(OcTensorIndexView *view, OcTensor *dst)
+{  int64_t *tables[OC_TENSOR_MAX_DIMS]; OcTensor *v = view->view;
+   index_tables(view, tables);
+   if (activate(dst->device) != 0 || OcTensor_startRead(dst, v) != 0) return -1;
+   OCH_CALL(och_get_index(v->dtype, view->ndims, SZ(v), tables, v->strides, OcTensor_data(v), dst->strides, OcTensor_data(dst), GPU_STREAM(dst)));
+   if (OcTensor_update(dst) != 0) return -1;
+   return OcTensor_finishRead(dst, v);
+}
+static int OcTensorGPU_setIndex(OcTensorIndexView *view, OcTensor *src)
+{  int64_t *tables[OC_TENSOR_MAX_DIMS]; OcTensor *v = view->view;
+   index_tables(view, tables);
+   if (activate(v->device) != 0 || OcTensor_startRead(v, src) != 0) return -1;
+   OCH_CALL(och_set_index(v->dtype, view->ndims, SZ(v), tables, v->strides, OcTensor_data(v), src->strides, OcTensor_data(src), GPU_STREAM(v)));
+   if (OcTensor_update(v) != 0) return -1;
+   return OcTensor_finishRead(v, src);
+}
+static int OcTensorGPU_fillIndex(OcTensorIndexView *view, OcScalar *scalar)
+{  int64_t *tables[OC_TENSOR_MAX_DIMS]; OcTensor *v = view->view; och_scalar val; scalar_value(scalar, &val);
+   index_tables(view, tables);
+   if (activate(v->device) != 0) return -1;
+   OCH_CALL(och_fill_index(v->dtype, view->ndims, SZ(v), tables, v->strides, OcTensor_data(v), val, GPU_STREAM(v)));
+   return OcTensor_update(v);
+}
+
+/* ---- elementwise (op/tensor_unary_gpu.c:59-93, op/tensor_binary_gpu.c:58-97) ------------ */
+static int unary_call(int op, const char *name, OcTensor *src, OcTensor *dst)
+{  if (!och_unary_supported(op, src->dtype)) return OcErrorMessage("Function %s is not supported for type %s on GPU", name, OcDType_name(src->dtype));
+   if ((int)dst->dtype != och_unary_result_dtype(op, src->dtype)) return OcErrorMessage("Invalid destination type in %s", name);
+   if (!same_shape(src, dst)) return OcErrorMessage("Mismatch in tensor sizes in %s", name);
+   if (activate(dst->device) != 0 || OcTensor_startRead(dst, src) != 0) return -1;
+   OCH_CALL(och_unary(op, src->dtype, dst->ndims, SZ(dst), src->strides, OcTensor_data(src), dst->strides, OcTensor_data(dst), GPU_STREAM(dst)));
+   if (OcTensor_update(dst) != 0) return -1;
+   return OcTensor_finishRead(dst, src);
+}
+static int binary_call(int op, const char *name, OcTensor *src1, OcTensor *src2, OcTensor *dst)
+{  if (!och_binary_supported(op, src1->dtype)) return OcErrorMessage("Function %s is not supported for type %s on GPU", name, OcDType_name(src1->dtype));
+   if ((int)src2->dtype != och_binary_operand2_dtype(op, src1->dtype) || (int)dst->dtype != och_binary_result_dtype(op, src1->dtype))
+      return OcErrorMessage("Invalid operand types in %s", name);
+   if (!same_shape(src1, dst) || !same_shape(src2, dst)) return OcErrorMessage("Mismatch in tensor sizes in %s", name);
+   if (activate(dst->device) != 0 || OcTensor_startRead(dst, src1) != 0 || OcTensor_startRead(dst, src2) != 0) return -1;
+   OCH_CALL(och_binary(op, src1->dtype, dst->ndims, SZ(dst), src1->strides, OcTensor_data(src1), src2->strides, OcTensor_data(src2),
+                       dst->strides, OcTensor_data(dst), GPU_STREAM(dst)));
+   if (OcTensor_update(dst) != 0) return -1;
+   if (OcTensor_finishRead(dst, src2) != 0) return -1;
+   return OcTensor_finishRead(dst, src1);
+}
+#define OC_X(NAME, OP) static int OcTensorGPU_##NAME(OcTensor *src, OcTensor *dst) { return unary_call(OP, #NAME, src, dst); }
+OC_UNARY_TABLE(OC_X)
+#undef OC_X
+#define OC_X(NAME, OP) static int OcTensorGPU_##NAME(OcTensor *a, OcTensor *b, OcTensor *c) { return binary_call(OP, #NAME, a, b, c); }
+OC_BINARY_TABLE(OC_X)
+#undef OC_X
+
+/* ---- full reductions (op/tensor_reduce_all_gpu.c:201-444) --------------------------------- */
+static int reduce_call(int op, OcTensor *tensor, OcScalar *lower, OcScalar *upper, double p, void *result)
+{  och_scalar b1, b2;
+   if (!och_reduce_supported(op, tensor->dtype)) return OcErrorMessage("Reduction is not supported for type %s on GPU", OcDType_name(tensor->dtype));
+   if (OcTensor_isByteswapped(tensor)) return OcErrorMessage("Reductions need native byte order");
+   if (lower) scalar_value(lower, &b1);
+   if (upper) scalar_value(upper, &b2);
+   if (activate(tensor->device) != 0) return -1;
+   OCH_CALL(och_reduce_all(op, tensor->dtype, tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor),
+                           lower ? &b1 : NULL, upper ? &b2 : NULL, p, result, NULL, GPU_STREAM(tensor)));
+   return 0;
+}
+#define OC_REDUCE_BOOL(NAME, OP) static int OcTensorGPU_##NAME(OcTensor *t, int *result) \
+   { unsigned char r = 0; if (reduce_call(OP, t, NULL, NULL, 0.0, &r) != 0) return -1; *result = r ? 1 : 0; return 0; }
+OC_REDUCE_BOOL(any, OCH_R_ANY) OC_REDUCE_BOOL(all, OCH_R_ALL)
+static int float_only(int op, OcTensor *t, int ifnot, int *result)
+{  unsigned char r = 0;
+   if (!OcDType_isFloat(t->dtype)) { *result = ifnot; return 0; }            /* integers are always finite */
+   if (reduce_call(op, t, NULL, NULL, 0.0, &r) != 0) return -1;
+   *result = r ? 1 : 0; return 0;
+}
+static int OcTensorGPU_allFinite(OcTensor *t, int *result) { return float_only(OCH_R_ALL_FINITE, t, 1, result); }
+static int OcTensorGPU_anyInf(OcTensor *t, int *result)    { return float_only(OCH_R_ANY_INF, t, 0, result); }
+static int OcTensorGPU_anyNaN(OcTensor *t, int *result)    { return float_only(OCH_R_ANY_NAN, t, 0, result); }
+static int OcTensorGPU_nnz(OcTensor *t, OcUInt64 *result)    { return reduce_call(OCH_R_NNZ, t, NULL, NULL, 0.0, result); }
+static int OcTensorGPU_nnzNaN(OcTensor *t, OcUInt64 *result) { return reduce_call(OCH_R_NNZ_NAN, t, NULL, NULL, 0.0, result); }
+#define OC_REDUCE_RANGE2(NAME, OP) static int OcTensorGPU_##NAME(OcTensor *t, OcScalar *lo, OcScalar *hi, int *result) \
+   { unsigned char r = 0; if (reduce_call(OP, t, lo, hi, 0.0, &r) != 0) return -1; *result = r ? 1 : 0; return 0; }
+#define OC_REDUCE_RANGE1(NAME, OP) static int OcTensorGPU_##NAME(OcTensor *t, OcScalar *bound, int *result) \
+   { unsigned char r = 0; if (reduce_call(OP, t, bound, NULL, 0.0, &r) != 0) return -1; *result = r ? 1 : 0; return 0; }
+OC_REDUCE_RANGE2(allGELE, OCH_R_ALL_GELE) OC_REDUCE_RANGE2(allGELT, OCH_R_ALL_GELT) OC_REDUCE_RANGE2(allGTLE, OCH_R_ALL_GTLE) OC_REDUCE_RANGE2(allGTLT, OCH_R_ALL_GTLT)
+OC_REDUCE_RANGE1(allLE, OCH_R_ALL_LE) OC_REDUCE_RANGE1(allLT, OCH_R_ALL_LT) OC_REDUCE_RANGE1(allGE, OCH_R_ALL_GE) OC_REDUCE_RANGE1(allGT, OCH_R_ALL_GT)
+static int scalar_reduce(int op, OcTensor *t, double p, OcScalar *result)
+{  memset(result, 0, sizeof(*result));
+   if (reduce_call(op, t, NULL, NULL, p, &result->value) != 0) return -1;
+   result->dtype = (OcDType)och_reduce_result_dtype(op, t->dtype);
+   return 0;
+}
+#define OC_REDUCE_SCALAR(NAME, OP) static int OcTensorGPU_##NAME(OcTensor *t, OcScalar *result) { return scalar_reduce(OP, t, 0.0, result); }
+OC_REDUCE_SCALAR(sum, OCH_R_SUM) OC_REDUCE_SCALAR(prod, OCH_R_PROD) OC_REDUCE_SCALAR(sumNaN, OCH_R_SUM_NAN) OC_REDUCE_SCALAR(prodNaN, OCH_R_PROD_NAN)
+OC_REDUCE_SCALAR(sumAbs, OCH_R_SUM_ABS) OC_REDUCE_SCALAR(sumAbsNaN, OCH_R_SUM_ABS_NAN) OC_REDUCE_SCALAR(maximum, OCH_R_MAXIMUM) OC_REDUCE_SCALAR(minimum, OCH_R_MINIMUM)
+OC_REDUCE_SCALAR(maximumAbs, OCH_R_MAXIMUM_ABS) OC_REDUCE_SCALAR(minimumAbs, OCH_R_MINIMUM_ABS) OC_REDUCE_SCALAR(norm2, OCH_R_NORM2) OC_REDUCE_SCALAR(norm2NaN, OCH_R_NORM2_NAN)
+static int OcTensorGPU_norm(OcTensor *t, double p, OcScalar *result)    { return scalar_reduce(OCH_R_NORM, t, p, result); }
+static int OcTensorGPU_normNaN(OcTensor *t, double p, OcScalar *result) { return scalar_reduce(OCH_R_NORM_NAN, t, p, result); }
+
+/* ---- axis reductions (op/tensor_reduce_axis_gpu.c:108-281) --------------------------------- */
+static int axis_call(int op, OcTensor *src, double p, int n, int *axes, OcTensor *dst)
+{  OcSolidReduceAxis a; och_reduce_axis_config c; int i;
+   if (!och_reduce_supported(op, src->dtype)) return OcErrorMessage("Axis reduction is not supported for type %s on GPU", OcDType_name(src->dtype));
+   if ((int)dst->dtype != och_reduce_result_dtype(op, src->dtype)) return OcErrorMessage("Invalid destination type in axis reduction");
+   if (OcTensor_isByteswapped(src) || OcTensor_isByteswapped(dst)) return OcErrorMessage("Axis reductions need native byte order");
+   if (dst->nelem == 0) return 0;
+   if (OcSolid_analyzeReduceAxis(src, n, axes, dst, &a) != 0) return -1;
+   memset(&c, 0, sizeof(c));
+   c.ndims = a.ndims; c.rdims = a.rdims;
+   for (i = 0; i < a.ndims; i++) { c.size[i] = (size_t)a.size[i]; c.strides1[i] = a.strides1[i]; c.strides2[i] = a.strides2[i]; }
+   for (i = 0; i < a.rdims; i++) { c.rsize[i] = (size_t)a.rsize[i]; c.rstrides[i] = a.rstrides[i]; }
+   c.ptr1 = OcTensor_data(src) + a.offset1; c.ptr2 = OcTensor_data(dst) + a.offset2; c.stream = GPU_STREAM(dst);
+   if (activate(dst->device) != 0 || OcTensor_startRead(dst, src) != 0) return -1;
+   OCH_CALL(och_reduce_axis(op, src->dtype, &c, p));
+   if (OcTensor_update(dst) != 0) return -1;
+   return OcTensor_finishRead(dst, src);
+}
+#define OC_X(NAME, OP) static int OcTensorGPU_##NAME(OcTensor *src, int n, int *axes, OcTensor *dst) { return axis_call(OP, src, 0.0, n, axes, dst); }
+OC_AXIS_TABLE(OC_X)
+#undef OC_X
+static int OcTensorGPU_axisNorm(OcTensor *src, double p, int n, int *axes, OcTensor *dst)    { return axis_call(OCH_R_NORM, src, p, n, axes, dst); }
+static int OcTensorGPU_axisNormNaN(OcTensor *src, double p, int n, int *axes, OcTensor *dst) { return axis_call(OCH_R_NORM_NAN, src, p, n, axes, dst); }
+
+/* ---- GEMM (op/tensor_blas_gpu.c:63-286) ------------------------------------------------------ */
+static int OcTensorGPU_gemm(OcSize M, OcSize N, OcSize K, char transA, char transB, OcTensor *alpha, OcTensor *A, OcIndex ldA,
+                            OcTensor *B, OcIndex ldB, OcTensor *beta, OcTensor *C, OcIndex ldC)
+{  OcIndex index[OC_TENSOR_MAX_DIMS] = { 0 }; int i, ndims = A->ndims, host = (alpha->device == OcCPU);
+   char *pa = OcTensor_data(alpha), *pb = OcTensor_data(beta), *pA = OcTensor_data(A), *pB = OcTensor_data(B), *pC = OcTensor_data(C);
+   if (C->nelem == 0) return 0;
+   if (K == 0) { ldA = N; ldB = M; }
+   if (!och_gemm_supported(A->dtype)) return OcErrorMessage("Unsupported data type in function gpu gemm (%s)", OcDType_name(A->dtype));
+   if (activate(A->device) != 0) return -1;
+   for (;;)                                       /* one product per index of the dimensions beyond the second */
+   {  OCH_CALL(och_gemm(A->dtype, transA, transB, (size_t)M, (size_t)N, (size_t)K, pa, pA, ldA > 0 ? ldA : 1, pB, ldB > 0 ? ldB : 1, pb, pC, ldC, host, GPU_STREAM(C)));
+      for (i = 2; i < ndims; i++)
+      {  index[i]++;
+         if (i < alpha->ndims) pa += alpha->strides[i];
+         if (i < beta->ndims)  pb += beta->strides[i];
+         pA += A->strides[i]; pB += B->strides[i]; pC += C->strides[i];
+         if (index[i] < A->size[i]) break;
+         index[i] = 0;
+         if (i < alpha->ndims) pa -= A->size[i] * alpha->strides[i];
+         if (i < beta->ndims)  pb -= A->size[i] * beta->strides[i];
+         pA -= A->size[i] * A->strides[i]; pB -= A->size[i] * B->strides[i]; pC -= A->size[i] * C->strides[i];
+      }
+      if (i >= ndims) break;
+   }
+   return 0;
+}
+static int OcTensorGPU_gemmSupportedOn(OcDevice *device, OcDType dtype) { (void)device; return och_gemm_supported(dtype); }
+
+/* ---- module table and registration ------------------------------------------------------------ */
+static int gpu_initialize_context(OcDevice *device, OcDeviceModule *module, void **context)
+{  OcModuleCore_Context *ctx = (OcModuleCore_Context *)calloc(1, sizeof(OcModuleCore_Context));
+   (void)device; (void)module;
+   if (ctx == NULL) return OcErrorMessage("Insufficient memory for the module context");
+   ctx->scalarCount = 8;
+   *context = ctx;
+   return 0;
+}
+static void gpu_finalize_context(OcDevice *device, OcDeviceModule *module, void *context) { (void)device; (void)module; free(context); }
+static void gpu_finalize_module(OcDeviceModule *module) { (void)module; }
+
+static void fill_table(OcModuleCore *m)
+{  memset(m, 0, sizeof(*m));
+   m->HEAD.available = 1;
+   m->HEAD.initializeContext = gpu_initialize_context; m->HEAD.finalizeContext = gpu_finalize_context; m->HEAD.finalizeModule = gpu_finalize_module;
+   m->Device_formatInfo = OcDeviceGPU_formatInfo;
+   m->Buffer_copy = OcBufferGPU_copy; m->Buffer_copyFromCPU = OcBufferGPU_copyFromCPU; m->Buffer_copyToCPU = OcBufferGPU_copyToCPU;
+   m->Buffer_copyHostStorage = OcBufferGPU_copyHostStorage; m->Buffer_copyStorageHost = OcBufferGPU_copyStorageHost; m->Buffer_zero = OcBufferGPU_zero;
+   m->Storage_create = OcStorageGPU_create; m->Storage_fromObject = NULL;
+   m->Tensor_copy = OcTensorGPU_copy; m->Tensor_copyFromCPU = OcTensorGPU_copyFromCPU; m->Tensor_copyToCPU = OcTensorGPU_copyToCPU;
+   m->Tensor_byteswapNoFlag = OcTensorGPU_byteswapNoFlag;
+   m->Tensor_fill = OcTensorGPU_fill; m->Tensor_fillNaN = OcTensorGPU_fillNaN; m->Tensor_maskedFill = OcTensorGPU_maskedFill;
+   m->Tensor_stepsInt64 = OcTensorGPU_stepsInt64; m->Tensor_stepsDouble = OcTensorGPU_stepsDouble; m->Tensor_stepsCDouble = OcTensorGPU_stepsCDouble;
+   m->Tensor_find = NULL; m->Tensor_maskToOffset = NULL;              /* not available on the GPU in the reference either (docs/future_work.md:33) */
+   m->Tensor_indexToOffset = OcTensorGPU_indexToOffset; m->Tensor_addIfNegative = OcTensorGPU_addIfNegative;
+   m->Tensor_getIndex = OcTensorGPU_getIndex; m->Tensor_setIndex = OcTensorGPU_setIndex; m->Tensor_fillIndex = OcTensorGPU_fillIndex;
+#define OC_X(NAME, OP) m->Tensor_##NAME = OcTensorGPU_##NAME;
+   OC_UNARY_TABLE(OC_X) OC_BINARY_TABLE(OC_X) OC_AXIS_TABLE(OC_X)
+#undef OC_X
+   m->Tensor_allGELE = OcTensorGPU_allGELE; m->Tensor_allGELT = OcTensorGPU_allGELT; m->Tensor_allGTLE = OcTensorGPU_allGTLE; m->Tensor_allGTLT = OcTensorGPU_allGTLT;
+   m->Tensor_allLE = OcTensorGPU_allLE; m->Tensor_allLT = OcTensorGPU_allLT; m->Tensor_allGE = OcTensorGPU_allGE; m->Tensor_allGT = OcTensorGPU_allGT;
+   m->Tensor_any = OcTensorGPU_any; m->Tensor_all = OcTensorGPU_all; m->Tensor_allFinite = OcTensorGPU_allFinite; m->Tensor_anyInf = OcTensorGPU_anyInf;
+   m->Tensor_anyNaN = OcTensorGPU_anyNaN; m->Tensor_nnz = OcTensorGPU_nnz; m->Tensor_nnzNaN = OcTensorGPU_nnzNaN;
+   m->Tensor_sum = OcTensorGPU_sum; m->Tensor_prod = OcTensorGPU_prod; m->Tensor_sumNaN = OcTensorGPU_sumNaN; m->Tensor_prodNaN = OcTensorGPU_prodNaN;
+   m->Tensor_sumAbs = OcTensorGPU_sumAbs; m->Tensor_sumAbsNaN = OcTensorGPU_sumAbsNaN; m->Tensor_maximum = OcTensorGPU_maximum; m->Tensor_minimum = OcTensorGPU_minimum;
+   m->Tensor_maximumAbs = OcTensorGPU_maximumAbs; m->Tensor_minimumAbs = OcTensorGPU_minimumAbs; m->Tensor_norm2 = OcTensorGPU_norm2; m->Tensor_norm2NaN = OcTensorGPU_norm2NaN;
+   m->Tensor_norm = OcTensorGPU_norm; m->Tensor_normNaN = OcTensorGPU_normNaN;
+   m->Tensor_axisNorm = OcTensorGPU_axisNorm; m->Tensor_axisNormNaN = OcTensorGPU_axisNormNaN;
+   m->Tensor_gemm = OcTensorGPU_gemm; m->Tensor_gemmSupportedOn = OcTensorGPU_gemmSupportedOn;
+}
+
+/* device_module.c:313-422: the size must match the interface's view of the table; the table is copied */
+int OcRegisterModule(const char *deviceType, OcDeviceModule *info, size_t size)
+{  if (strcmp(deviceType, "GPU") != 0) return OcErrorMessage("This host registers the GPU device type only (got %s)", deviceType);
+   if (size != sizeof(OcModuleCore)) return OcErrorMessage("Mismatch in device module size (%zu, expected %zu)", size, sizeof(OcModuleCore));
+   memcpy(&oc_registered_gpu, info, size);
+   oc_registered = 1;
+   return 0;
+}
+OcModuleCore *OcModuleCore_forDevice(OcDevice *device)
+{  if (device == NULL || device == OcCPU || !oc_registered) return NULL;
+   return &oc_registered_gpu;
+}
+int OcDeviceGPUCount(void) { return oc_gpu_count; }
+
+int OcInitGPU(void)
+{  int i, count = 0;
+   if (oc_gpu_initialized) return 0;
+   if (och_device_count(&count) != 0) return OcErrorMessage("%s", och_last_error());
+   OcGPU = (OcDevice **)calloc((size_t)(count > 0 ? count : 1), sizeof(OcDevice *));
+   if (OcGPU == NULL) return OcErrorMessage("Insufficient memory for the device list");
+   for (i = 0; i < count; i++)
+   {  OcDeviceGPU *g = (OcDeviceGPU *)calloc(1, sizeof(OcDeviceGPU)); char name[32];
+      if (g == NULL) return OcErrorMessage("Insufficient memory for the device object");
+      snprintf(name, sizeof(name), "gpu%d", i);
+      g->HEAD.index = i; g->HEAD.name = strdup(name); g->HEAD.endianness = 0; g->HEAD.requiresAlignedData = 1; g->HEAD.refcount = 1;
+      g->HEAD.create_stream = gpu_create_stream; g->HEAD.create_event = gpu_create_event; g->HEAD.delete_stream = gpu_delete_stream;
+      g->HEAD.delete_event = gpu_delete_event; g->HEAD.sync_stream = gpu_sync_stream; g->HEAD.sync_event = gpu_sync_event;
+      g->HEAD.record_event = gpu_record_event; g->HEAD.wait_event = gpu_wait_event; g->HEAD.finalize = gpu_finalize_device;
+      if (och_device_properties(i, &g->properties) != 0) return OcErrorMessage("%s", och_last_error());
+      if (och_device_warmup(i) != 0) return OcErrorMessage("%s", och_last_error());          /* device_gpu.c:155-196 */
+      OcGPU[i] = &g->HEAD;
+      if ((g->HEAD.defaultStream = gpu_create_stream(&g->HEAD)) == NULL) return -1;
+      g->HEAD.contextBuffer = (void **)calloc(1, sizeof(void *)); g->HEAD.contextSize = g->HEAD.contextCapacity = 1;
+   }
+   oc_gpu_count = count;
+   fill_table(&oc_module_core_gpu);
+   if (OcRegisterModule("GPU", (OcDeviceModule *)&oc_module_core_gpu, sizeof(OcModuleCore)) != 0) return -1;
+   for (i = 0; i < count; i++)
+      if (oc_registered_gpu.HEAD.initializeContext(OcGPU[i], &oc_registered_gpu.HEAD, &OcGPU[i]->contextBuffer[0]) != 0) return -1;
+   oc_gpu_initialized = 1;
+   return 0;
+}
+void OcFinalizeGPU(void)
+{  int i;
+   if (!oc_gpu_initialized) return;
+   for (i = 0; i < oc_gpu_count; i++)
+   {  OcDevice *d = OcGPU[i];
+      och_device_set(i); och_device_synchronize();
+      oc_registered_gpu.HEAD.finalizeContext(d, &oc_registered_gpu.HEAD, d->contextBuffer[0]);
+      gpu_delete_stream(d->defaultStream);
+      d->finalize(d);
+      free(d->contextBuffer); free(d->name); free(d);
+   }
+   free(OcGPU); OcGPU = NULL; oc_gpu_count = 0; oc_gpu_initialized = 0; oc_registered = 0;
+}

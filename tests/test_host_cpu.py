@@ -1,0 +1,145 @@
+"""CPU checks of the host layer (no GPU): struct layouts against the numbers taken from the
+reference's headers (tests/golden/abi_layout.json), the order of the function table, type
+promotion and the shape routines against the reference's own dtype.c / shape.c (compiled into
+oracle/_ref/libocean_ref_base.so where the reference tree is present), and the axis-reduction
+analysis against brute-force enumeration."""
+import ctypes as C
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+
+import ocean_host as host
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+REF_BASE = os.path.join(ROOT, "oracle", "_ref", "libocean_ref_base.so")
+ref = C.CDLL(REF_BASE) if os.path.exists(REF_BASE) else None
+needs_ref = pytest.mark.skipif(ref is None, reason="oracle/_ref/libocean_ref_base.so not built")
+
+
+def test_struct_layouts_match_reference_headers():
+    golden = json.load(open(os.path.join(ROOT, "tests", "golden", "abi_layout.json")))
+    mine = json.loads(host.lib.OcHost_abiLayout())
+    keys = [k for k in golden if not k.startswith("_")]
+    assert len(keys) > 200
+    assert sorted(keys) == sorted(mine.keys())
+    wrong = {k: (mine[k], golden[k]) for k in keys if mine[k] != golden[k]}
+    assert not wrong, wrong
+    # ctypes mirrors used by the tests agree too
+    assert C.sizeof(host.Tensor) == golden["sizeof(OcTensor)"] and C.sizeof(host.Storage) == golden["sizeof(OcStorage)"]
+    assert C.sizeof(host.Scalar) == golden["sizeof(OcScalar)"]
+
+
+def test_table_order_matches_reference_lists():
+    golden = json.load(open(os.path.join(ROOT, "tests", "golden", "abi_layout.json")))
+    text = open(os.path.join(ROOT, "ocean-tensor-package_amd", "host", "ocean_abi.h")).read()
+    import re
+    def table(name):
+        body = text.split("#define %s(X)" % name)[1].split("\n\n")[0].split("#define")[0]
+        return re.findall(r"X\((\w+), (\d+)\)", body)
+    unary, binary = table("OC_UNARY_TABLE"), table("OC_BINARY_TABLE")
+    assert [n for n, _ in unary] == golden["_unary_order"]
+    assert [n for n, _ in binary] == golden["_binary_order"]
+    assert [int(i) for _, i in unary] == list(range(40)) and [int(i) for _, i in binary] == list(range(27))
+
+
+@needs_ref
+def test_common_type_matches_reference():
+    for a in range(16):
+        for b in range(16):
+            assert host.lib.OcDType_getCommonType(a, b) == ref.OcDType_getCommonType(a, b), (a, b)
+
+
+def test_common_type_examples():
+    # the promotions the benchmark configurations rely on (float64 with int32, float with int16)
+    assert host.lib.OcDType_getCommonType(host.DOUBLE, host.INT32) == host.DOUBLE
+    assert host.lib.OcDType_getCommonType(host.FLOAT, host.INT16) == host.FLOAT
+    assert host.lib.OcDType_getCommonType(host.FLOAT, host.INT32) == host.DOUBLE
+    assert host.lib.OcDType_getCommonType(host.INT8, host.UINT8) == host.INT16
+    assert host.lib.OcDType_getCommonType(host.INT64, host.UINT64) == host.DOUBLE
+    assert host.lib.OcDType_getCommonType(host.CFLOAT, host.DOUBLE) == host.CDOUBLE
+
+
+@needs_ref
+def test_shape_routines_match_reference():
+    rng = np.random.default_rng(8)
+    ss = C.POINTER(C.c_ssize_t)
+    ref.OcShape_sortStrides2.argtypes = [C.c_int, ss, ss, ss]
+    ref.OcShape_mergeBlocks2.argtypes = [C.POINTER(C.c_int), ss, ss, ss]
+    for _ in range(500):
+        nd = int(rng.integers(0, 9))
+        size = rng.integers(1, 6, nd)
+        s1 = rng.choice([0, 4, 8, 16, 32, 64, 128, 256], nd)
+        s2 = rng.choice([0, 4, 8, 16, 32, 64, 128, 256], nd)
+        def run(libx):
+            a, b, c = host._arr(list(size)), host._arr(list(s1)), host._arr(list(s2))
+            libx.OcShape_sortStrides2(nd, a, b, c)
+            n = C.c_int(nd)
+            libx.OcShape_mergeBlocks2(C.byref(n), a, b, c)
+            return n.value, list(a)[:n.value], list(b)[:n.value], list(c)[:n.value]
+        assert run(host.lib) == run(ref), (size, s1, s2)
+
+
+def _offsets(size, strides):
+    tot = np.zeros([int(s) for s in size] or [1], dtype=np.int64)
+    for d, (n, s) in enumerate(zip(size, strides)):
+        shape = [1] * len(size); shape[d] = int(n)
+        tot = tot + (np.arange(int(n), dtype=np.int64) * int(s)).reshape(shape)
+    return tot
+
+
+def test_axis_analysis_enumerates_the_same_elements():
+    """For random strided sources, the (outer, reduced) decomposition must visit, for every destination
+    element, exactly the source elements that the reduction over `axes` assigns to it."""
+    rng = np.random.default_rng(21)
+    cpu = host.cpu_device()
+    for trial in range(200):
+        nd = int(rng.integers(1, 5))
+        shape = [int(x) for x in rng.integers(1, 5, nd)]
+        perm = rng.permutation(nd)
+        strides = [0] * nd; acc = 4
+        for d in perm:
+            sign = -1 if rng.integers(0, 4) == 0 else 1
+            strides[d] = acc * sign; acc *= shape[d] * int(rng.integers(1, 3))
+        src = host.create(shape, host.FLOAT, cpu, strides)
+        k = int(rng.integers(1, nd + 1))
+        axes = sorted(int(a) for a in rng.choice(nd, k, replace=False))
+        keep = bool(rng.integers(0, 2))
+        dshape = [1 if d in axes else shape[d] for d in range(nd)] if keep else [shape[d] for d in range(nd) if d not in axes]
+        dst = host.create(dshape, host.FLOAT, cpu)
+        cfg = host.ReduceAxis()
+        assert host.lib.OcSolid_analyzeReduceAxis(src, k, (C.c_int * k)(*axes), dst, C.byref(cfg)) == 0
+        # expected: map destination offset -> sorted list of source offsets
+        so = _offsets(shape, strides)
+        dstrides = [dst.contents.strides[i] for i in range(dst.contents.ndims)]
+        full_d = [0 if d in axes else dstrides[d if keep else [x for x in range(nd) if x not in axes].index(d)] for d in range(nd)]
+        do = _offsets(shape, full_d)
+        want = {}
+        for s, d in zip(so.reshape(-1), do.reshape(-1)):
+            want.setdefault(int(d), []).append(int(s))
+        # got: enumerate the analysed configuration
+        osz = [cfg.size[i] for i in range(cfg.ndims)]; o1 = [cfg.strides1[i] for i in range(cfg.ndims)]; o2 = [cfg.strides2[i] for i in range(cfg.ndims)]
+        rsz = [cfg.rsize[i] for i in range(cfg.rdims)]; rs = [cfg.rstrides[i] for i in range(cfg.rdims)]
+        outer1 = _offsets(osz, o1).reshape(-1) + cfg.offset1; outer2 = _offsets(osz, o2).reshape(-1) + cfg.offset2
+        inner = _offsets(rsz, rs).reshape(-1)
+        got = {int(d): sorted(int(s + i) for i in inner) for s, d in zip(outer1, outer2)}
+        assert {k2: sorted(v) for k2, v in want.items()} == got, (shape, strides, axes, keep)
+        host.lib.OcDecrefTensor(src); host.lib.OcDecrefTensor(dst)
+
+
+def test_views_and_errors():
+    cpu = host.cpu_device()
+    t = host.create([4, 6], host.DOUBLE, cpu)
+    tt = host.lib.OcTensor_transpose(t)
+    assert host.shape_of(tt) == [6, 4] and [tt.contents.strides[i] for i in range(2)] == [32, 8]
+    sl = host.lib.OcTensor_slice(t, 0, 1, 2, 2)
+    assert host.shape_of(sl) == [2, 6] and sl.contents.offset == t.contents.offset + 8 and sl.contents.strides[0] == 16
+    assert not host.lib.OcTensor_slice(t, 0, 3, 2, 2)            # out of range
+    assert b"out of range" in host.lib.OcError_lastMessage()
+    b = host.lib.OcTensor_broadcastTo(host.create([1, 6], host.DOUBLE, cpu), 2, host._arr([4, 6]))
+    assert [b.contents.strides[i] for i in range(2)] == [0, 8]
+    # without OcInitGPU no device module is registered for a made-up device
+    with pytest.raises(host.OceanError):
+        host.check(host.lib.OcTensor_binary(99, t, t, C.byref(host.TP())))

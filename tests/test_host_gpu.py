@@ -1,0 +1,194 @@
+"""The GPU device module driven through Ocean's module table and a small front end, the way
+Ocean's interface layer drives it (OcInitGPU -> OcModuleCore table -> OcTensorGPU_* -> device
+library). Mirrors examples/python/gpu/tensors/tensor_add_02.py (transposed + broadcast add),
+tensor_dtype_cast_01.py / tensor_copy_0x.py (casting and strided copies between devices),
+ocean_sum_02.py, ocean_axis_reduce_04.py, ocean_gemm_01.py, and BASELINE configuration 2
+end to end: Z = (A.T + r + I) * F with automatic type promotion and a byte-swapped operand.
+
+Expected values come from numpy, which fixes them independently: every step of the float64
+expression is a single correctly rounded IEEE operation or an exact conversion, so the result is
+bit-identical; reductions and GEMM use the tolerances of the other GPU tests.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import ocean_host as host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    return host.gpu_device(0)
+
+
+def binary(op, a, b, out=None):
+    dst = host.TP() if out is None else out
+    host.check(host.lib.OcTensor_binary(op, a, b, C.byref(dst)))
+    return dst
+
+
+ADD, SUB, SCALE, LT, BITSHIFT_LEFT, POWER = 0, 1, 2, 13, 25, 6
+
+
+def test_init_and_table(gpu):
+    assert host.lib.OcInitGPU() == 0 and host.lib.OcInitGPU() == 0           # idempotent
+    assert host.lib.OcDeviceGPUCount() >= 1
+
+
+@pytest.mark.parametrize("n", [96, 4096])
+def test_configuration2_through_the_front_end(gpu, n):
+    rng = np.random.default_rng(2024)
+    A = rng.uniform(-10, 10, (n, n))
+    r = rng.uniform(-10, 10, (n, 1))                                          # Ocean shape (1, n): a row
+    I = rng.integers(-10, 10, (n, n), endpoint=True).astype(np.int32)
+    F = rng.uniform(-10, 10, (n, n)).astype(np.float32)
+    tA = host.from_numpy(A, host.DOUBLE, gpu)
+    tr = host.from_numpy(r, host.DOUBLE, gpu)
+    tI = host.from_numpy(I, host.INT32, gpu)
+    tF = host.from_numpy(F.byteswap(), host.FLOAT, gpu, byteswapped=True)
+    tAt = host.lib.OcTensor_transpose(tA)
+    z = binary(ADD, tAt, tr)                       # transposed view + zero-stride broadcast
+    z2 = binary(ADD, z, tI)                        # int32 operand promoted to float64 by a converting copy
+    z3 = binary(SCALE, z2, tF)                     # byte-swapped float32 operand normalised and widened
+    assert z3.contents.dtype == host.DOUBLE and host.shape_of(z3) == [n, n]
+    want = ((A.T + r) + I.astype(np.float64)) * F.astype(np.float64)
+    got = host.to_numpy(z3)
+    assert got.tobytes() == want.tobytes()
+    # in place: z3 += A.T
+    binary(ADD, z3, tAt, out=z3)
+    assert host.to_numpy(z3).tobytes() == (want + A.T).tobytes()
+    for t in (tA, tr, tI, tF, tAt, z, z2, z3):
+        host.lib.OcDecrefTensor(t)
+
+
+def test_promotion_compare_shift_power(gpu):
+    rng = np.random.default_rng(5)
+    a = rng.integers(-100, 100, (7, 33)).astype(np.int16)
+    b = rng.uniform(-100, 100, (7, 33)).astype(np.float32)
+    ta, tb = host.from_numpy(a, host.INT16, gpu), host.from_numpy(b, host.FLOAT, gpu)
+    s = binary(ADD, ta, tb)
+    assert s.contents.dtype == host.FLOAT
+    assert np.array_equal(host.to_numpy(s), a.astype(np.float32) + b)
+    lt = binary(LT, ta, tb)
+    assert lt.contents.dtype == host.BOOL and np.array_equal(host.to_numpy(lt), (a.astype(np.float32) < b).astype(np.uint8))
+    cnt = rng.integers(0, 8, (7, 33)).astype(np.int32)
+    tc = host.from_numpy(cnt, host.INT32, gpu)
+    sh = binary(BITSHIFT_LEFT, ta, tc)             # counts are converted to int8 on the way in
+    assert sh.contents.dtype == host.INT16 and np.array_equal(host.to_numpy(sh), (a.astype(np.int32) << cnt).astype(np.int16))
+    e = rng.integers(0, 4, (7, 33)).astype(np.int64)
+    te = host.from_numpy(e, host.INT64, gpu)
+    small = host.from_numpy((a % 7).astype(np.int16), host.INT16, gpu)
+    pw = binary(POWER, small, te)
+    assert pw.contents.dtype == host.INT64 and np.array_equal(host.to_numpy(pw), (a % 7).astype(np.int64) ** e)
+    # destination of another type: computed in the common type, then converted
+    out = host.create([33, 7], host.DOUBLE, gpu)
+    binary(ADD, ta, tb, out=out)
+    assert np.array_equal(host.to_numpy(out), (a.astype(np.float32) + b).astype(np.float64))
+    # incompatible shapes are reported, not computed
+    bad = host.from_numpy(np.zeros((7, 5), np.float32), host.FLOAT, gpu)
+    with pytest.raises(host.OceanError, match="not compatible"):
+        binary(ADD, ta, bad)
+
+
+def test_copy_between_devices_with_cast_strides_and_byte_order(gpu):
+    rng = np.random.default_rng(6)
+    cpu = host.cpu_device()
+    src = rng.integers(-32768, 32767, (64, 40, 66), dtype=np.int16, endpoint=True)
+    ts = host.from_numpy(src.byteswap(), host.INT16, None, byteswapped=True)       # host tensor, other byte order
+    view = host.lib.OcTensor_slice(ts, 0, 1, 32, 2)                                  # every second element of dimension 0
+    d = host.create([32, 40, 64], host.FLOAT, gpu)
+    host.check(host.lib.OcTensor_copy(view, d))                                      # upload raw, swap + cast + gather on the device
+    want = src[:, :, 1:65:2].astype(np.float32)
+    assert np.array_equal(host.to_numpy(d), want)
+    # back into a strided, byte-swapped host tensor of another type
+    back = host.create([64, 40, 64], host.DOUBLE, cpu)
+    C.memset(host.data_address(back), 0, back.contents.storage.contents.size)
+    bview = host.lib.OcTensor_slice(back, 0, 0, 32, 2)
+    host.lib.OcTensor_setByteswapped(bview, 1)
+    host.check(host.lib.OcTensor_copy(d, bview))
+    raw = np.empty((64, 40, 64), np.float64)
+    C.memmove(raw.ctypes.data, host.data_address(back), raw.nbytes)
+    assert np.array_equal(raw[:, :, 0::2].byteswap(), want.astype(np.float64))
+    assert not raw[:, :, 1::2].any()                                                 # the gaps were not touched
+
+
+def test_reductions_and_axis_reductions(gpu):
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((50, 70, 90)).astype(np.float32)
+    t = host.from_numpy(x, host.FLOAT, gpu)
+    s = host.Scalar()
+    host.check(host.lib.OcTensor_reduceAll(15, t, 0.0, C.byref(s)))
+    assert s.dtype == host.FLOAT and abs(s.get() - x.astype(np.float64).sum()) <= 1e-5 * np.abs(x).sum()
+    host.check(host.lib.OcTensor_reduceAll(21, t, 0.0, C.byref(s)))
+    assert s.get() == x.max()
+    host.check(host.lib.OcTensor_reduceAll(27, t, 0.0, C.byref(s)))
+    assert abs(s.get() - np.linalg.norm(x.astype(np.float64))) <= 1e-5 * np.linalg.norm(x)
+    xi = rng.integers(-100, 100, (50, 70, 90)).astype(np.int8)
+    ti = host.from_numpy(xi, host.INT8, gpu)
+    host.check(host.lib.OcTensor_reduceAll(15, ti, 0.0, C.byref(s)))
+    assert s.dtype == host.INT64 and s.get() == int(xi.astype(np.int64).sum())
+    # a strided view: every second row, reversed along the last Ocean dimension
+    v = host.lib.OcTensor_slice(t, 1, 1, 30, 2)                 # Ocean dims (90, 70, 50) -> (90, 30, 50)
+    v2 = host.lib.OcTensor_slice(v, 2, 49, 50, -1)
+    xv = x[::-1, 1:61:2, :]
+    for axes, keep in (([0], 0), ([1], 1), ([0, 2], 0), ([2], 0), ([0, 1, 2], 1)):
+        dst = host.TP()
+        host.check(host.lib.OcTensor_axisReduce(15, v2, len(axes), (C.c_int * len(axes))(*axes), keep, 0.0, C.byref(dst)))
+        np_axes = tuple(2 - a for a in axes)
+        want = xv.astype(np.float64).sum(axis=np_axes, keepdims=bool(keep))
+        got = host.to_numpy(dst)
+        assert got.shape == want.shape
+        assert np.allclose(got, want, rtol=0, atol=1e-5 * np.abs(xv).sum(axis=np_axes, keepdims=bool(keep)).max())
+        dmin = host.TP()
+        host.check(host.lib.OcTensor_axisReduce(22, v2, len(axes), (C.c_int * len(axes))(*axes), keep, 0.0, C.byref(dmin)))
+        assert np.array_equal(host.to_numpy(dmin), xv.min(axis=np_axes, keepdims=bool(keep)))
+    with pytest.raises(host.OceanError, match="Repeated axis"):
+        host.check(host.lib.OcTensor_axisReduce(15, t, 2, (C.c_int * 2)(1, 1), 0, 0.0, C.byref(host.TP())))
+
+
+def test_gemm_through_the_front_end(gpu):
+    rng = np.random.default_rng(9)
+    m, n, k = 150, 70, 90
+    A = rng.uniform(-1, 1, (k, m))                 # Ocean (m, k), column-major
+    B = rng.uniform(-1, 1, (n, k))                 # Ocean (k, n)
+    tA, tB = host.from_numpy(A, host.DOUBLE, gpu), host.from_numpy(B, host.DOUBLE, gpu)
+    c = host.TP()
+    host.check(host.lib.OcTensor_mtimes(tA, tB, C.byref(c)))
+    want = (A.T @ B.T).T                           # numpy layout of the Ocean (m, n) result
+    assert host.shape_of(c) == [m, n]
+    assert np.linalg.norm(host.to_numpy(c) - want) <= 1e-13 * np.linalg.norm(np.abs(A.T) @ np.abs(B.T))
+    # transposed views are used through the opposite mode instead of being copied: (A')' * B
+    At = host.from_numpy(np.ascontiguousarray(A.T), host.DOUBLE, gpu)        # Ocean (k, m)
+    v = host.lib.OcTensor_transpose(At)                                      # Ocean (m, k), rows contiguous
+    c2 = host.TP()
+    alpha, beta = host.scalar(host.DOUBLE, 2.0), host.scalar(host.DOUBLE, -1.0)
+    c0 = rng.uniform(-1, 1, (n, m))
+    c2 = host.from_numpy(c0, host.DOUBLE, gpu)
+    host.check(host.lib.OcTensor_gemm(C.byref(alpha), v, b"N", tB, b"N", C.byref(beta), C.byref(c2)))
+    want2 = 2.0 * want - c0
+    assert np.linalg.norm(host.to_numpy(c2) - want2) <= 1e-13 * (2 * np.linalg.norm(np.abs(A.T) @ np.abs(B.T)) + np.linalg.norm(c0))
+    # mixed types promote: int32 x float32 -> double; integer product is exact
+    Ai = rng.integers(-5, 5, (k, m)).astype(np.int32); Bi = rng.integers(-5, 5, (n, k)).astype(np.int32)
+    ci = host.TP()
+    host.check(host.lib.OcTensor_mtimes(host.from_numpy(Ai, host.INT32, gpu), host.from_numpy(Bi, host.INT32, gpu), C.byref(ci)))
+    assert ci.contents.dtype == host.INT32 and np.array_equal(host.to_numpy(ci), (Ai.T @ Bi.T).T)
+    with pytest.raises(host.OceanError, match="Inner dimensions"):
+        host.check(host.lib.OcTensor_mtimes(tA, tA, C.byref(host.TP())))
+
+
+def test_unary_and_fill(gpu):
+    rng = np.random.default_rng(10)
+    x = rng.uniform(0.5, 9, (12, 31))
+    t = host.from_numpy(x, host.DOUBLE, gpu)
+    out = host.TP()
+    host.check(host.lib.OcTensor_unary(17, t, C.byref(out)))               # sqrt
+    assert np.array_equal(host.to_numpy(out), np.sqrt(x))
+    isn = host.TP()
+    host.check(host.lib.OcTensor_unary(36, t, C.byref(isn)))               # isnan -> bool
+    assert isn.contents.dtype == host.BOOL and not host.to_numpy(isn).any()
+    val = host.scalar(host.DOUBLE, 3.25)
+    host.check(host.lib.OcTensor_fill(t, C.byref(val)))
+    assert (host.to_numpy(t) == 3.25).all()
