@@ -103,7 +103,8 @@ class Operand:
         return Operand(parent, view, dtype)
 
     def upload(self, stream):
-        self.dev = oh.to_device(self.parent.view(np.uint8).reshape(-1), stream)
+        # bytes in memory order (the parent is C- or Fortran-contiguous)
+        self.dev = oh.to_device(self.parent.ravel(order="K").view(np.uint8), stream)
         return self
 
     def dptr(self):
@@ -115,7 +116,7 @@ class Operand:
 
     def download(self):
         raw = self.dev.download(np.uint8, self.parent.nbytes)
-        return raw.view(self.parent.dtype).reshape(self.parent.shape)
+        return np.ndarray(shape=self.parent.shape, dtype=self.parent.dtype, buffer=raw, strides=self.parent.strides)
 
     def free(self):
         if self.dev is not None:
