@@ -194,27 +194,47 @@ def main():
 
     # ------------------------------------------------------------------ configuration 1
     n1 = 1 << 24
-    x, y, t, z = [oh.DeviceBuffer(4 * n1, stream) for _ in range(4)]
-    x.upload(rng.uniform(-1, 1, n1).astype(np.float32)); y.upload(rng.uniform(-1, 1, n1).astype(np.float32))
+    # six buffer sets (6 x 256 MB) so that successive launches never find their operands in the 256 MB Infinity Cache
+    c1sets = []
+    for i in range(6):
+        bufs = [oh.DeviceBuffer(4 * n1, stream) for _ in range(4)]
+        bufs[0].upload(rng.uniform(-1, 1, n1).astype(np.float32)); bufs[1].upload(rng.uniform(-1, 1, n1).astype(np.float32))
+        c1sets.append(bufs)
     s1, st1 = oh.sizes([n1]), oh.strides([4])
-    ms_mul = time_launches(lambda: oh.check(lib.och_binary(B["multiply"], F32, 1, s1, st1, x.ptr, st1, y.ptr, st1, t.ptr, h)))
-    ms_add = time_launches(lambda: oh.check(lib.och_binary(B["add"], F32, 1, s1, st1, t.ptr, st1, x.ptr, st1, z.ptr, h)))
+    turn = [0]
+
+    def c1_scale():
+        x, y, t, z = c1sets[turn[0] % 6]; turn[0] += 1
+        oh.check(lib.och_binary(B["multiply"], F32, 1, s1, st1, x.ptr, st1, y.ptr, st1, t.ptr, h))
+
+    def c1_add():
+        x, y, t, z = c1sets[turn[0] % 6]; turn[0] += 1
+        oh.check(lib.och_binary(B["add"], F32, 1, s1, st1, t.ptr, st1, x.ptr, st1, z.ptr, h))
+    ms_mul = time_launches(c1_scale, reps=30)
+    ms_add = time_launches(c1_add, reps=30)
     configs["c1_scale_f32_2^24"] = gbps(12 * n1, ms_mul)
     configs["c1_add_f32_2^24"] = gbps(12 * n1, ms_add)
-    for b in (x, y, t, z):
-        b.free()
+    for bufs in c1sets:
+        for b in bufs:
+            b.free()
 
     # ------------------------------------------------------------------ configuration 3
     n3 = 8192 * 8192
     for dt, es, nm in ((F32, 4, "f32"), (F64, 8, "f64")):
-        buf = oh.DeviceBuffer(es * n3, stream)
+        rbufs = [oh.DeviceBuffer(es * n3, stream) for _ in range(2)]          # alternate: no reuse from the Infinity Cache
         chunk = rng.standard_normal(1 << 22).astype(np.float32 if es == 4 else np.float64)
-        for off in range(0, n3, 1 << 22):
-            buf.upload(chunk, offset=off * es)
+        for buf in rbufs:
+            for off in range(0, n3, 1 << 22):
+                buf.upload(chunk, offset=off * es)
+        rturn = [0]
+
+        def next_buf():
+            rturn[0] += 1
+            return rbufs[rturn[0] % 2]
         dres = oh.DeviceBuffer(64, stream)
         s3, st3 = oh.sizes([n3]), oh.strides([es])
         for opn in ("sum", "norm2", "maximum"):
-            ms = time_launches(lambda: oh.check(lib.och_reduce_all_device(R[opn], dt, 1, s3, st3, buf.ptr, None, None, 0.0, dres.ptr, None, h)), reps=10)
+            ms = time_launches(lambda: oh.check(lib.och_reduce_all_device(R[opn], dt, 1, s3, st3, next_buf().ptr, None, None, 0.0, dres.ptr, None, h)), reps=10)
             configs["c3_%s_%s_8192^2" % (opn, nm)] = gbps(es * n3, ms)
         # axis reductions on a 512 x 512 x 256 view with padded pitches (no two dimensions merge);
         # the view lives in a parent of (512+4) x (512+2) x 256 elements
@@ -244,7 +264,7 @@ def main():
                 ms = time_launches(lambda: oh.check(lib.och_reduce_axis(R[opn], dt, C.byref(cfg), 0.0)), reps=10)
                 configs["c3_axis%d_%s_%s_512x512x256" % (axis, opn, nm)] = gbps(es * (d0 * d1 * d2 + keep[0] * keep[1]), ms)
         abuf.free()
-        for b in (buf, dres, out):
+        for b in rbufs + [dres, out]:
             b.free()
 
     # ------------------------------------------------------------------ configuration 4
@@ -287,6 +307,31 @@ def main():
                     "ms": round(ms, 3), "TFLOPs": round(tf, 2), "frac": round(tf / MFMA_PEAK[nm], 3)}
             for buf in (a, b, c):
                 buf.free()
+        # MGS-QR pattern on a 4096 x 4096 float64 matrix: per (i, j) pair one dot product (gemm M = N = 1, result kept
+        # on the device) and one rank-1 update reading that device scalar; window = the first 64 columns (2016 pairs)
+        m = 4096
+        q = oh.DeviceBuffer(8 * m * m, stream)
+        blockq = rng.uniform(-1, 1, 1 << 22)
+        for off in range(0, 8 * m * m, blockq.nbytes):
+            q.upload(blockq, offset=off)
+        rr = oh.DeviceBuffer(8 * 64 * 64, stream)
+        consts = oh.to_device(np.array([1.0, 0.0, -1.0]), stream)
+        c_one, c_zero, c_minus = [C.c_void_p(consts.address + 8 * i) for i in range(3)]
+        col = lambda j: C.c_void_p(q.address + 8 * m * j)
+        rij = lambda i, j: C.c_void_p(rr.address + 8 * (i + 64 * j))
+
+        def mgs_window():
+            for j in range(64):
+                for i in range(j):
+                    lib.och_gemm(F64, b"T", b"N", 1, 1, m, c_minus, col(i), m, col(j), m, c_zero, rij(i, j), 1, 0, h)
+                    lib.och_gemm(F64, b"N", b"N", m, 1, 1, c_one, col(i), m, rij(i, j), 1, c_one, col(j), m, 0, h)
+        mgs_window(); stream.synchronize()
+        t0 = time.perf_counter(); mgs_window(); stream.synchronize(); dt_s = time.perf_counter() - t0
+        pairs = 64 * 63 // 2
+        configs["c5_mgs_qr_4096_first64cols"] = {"us_per_pair": round(dt_s / pairs * 1e6, 2), "launches_per_pair": 2,
+                                                 "effective_GBps": round(pairs * (2 * 8 * m + 3 * 8 * m) / dt_s / 1e9, 1)}
+        for b in (q, rr, consts):
+            b.free()
     result["configs"] = configs
 
     # ------------------------------------------------------------------ CPU baseline (oracle, Ocean's threading policy)
