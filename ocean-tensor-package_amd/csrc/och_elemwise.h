@@ -56,7 +56,7 @@ template <int NOPS> struct EwParams
    uint64_t group0;                        /* first flat element index (for index-dependent ops) */
    int      ndims;
    int      vecmode[NOPS];
-   int      nt;                            /* streaming launch: wide accesses carry the nontemporal hint */                 /* 1: aligned unit stride, one wide access per group */
+   int      nt;                            /* streaming launch: wide accesses carry the nontemporal hint */
 };
 
 template <class T, int VEC> struct alignas((sizeof(T) * VEC) > 16 ? 16 : (sizeof(T) * VEC)) Pack { T v[VEC]; };
@@ -75,42 +75,43 @@ template <> struct RawVec<4>  { typedef uint32_t type; };
 template <> struct RawVec<8>  { typedef och_u32x2 type; };
 template <> struct RawVec<16> { typedef och_u32x4 type; };
 
-/* nt: nontemporal hint for data that is touched once (large streaming launches); measured on MI355X,
+/* nt (a compile-time constant at every call site: a run-time choice between the two forms is folded into the
+   plain one): nontemporal hint for data that is touched once (large streaming launches); measured on MI355X,
    a float64 add of 3 x 134 MB runs at 6.4 TB/s with the hint and one group per thread, 5.4 TB/s without */
-template <class T, int VEC>
-OCH_D void load_wide(Pack<T, VEC> &p, const char *addr, int nt = 0)
+template <class T, int VEC, bool NT = false>
+OCH_D void load_wide(Pack<T, VEC> &p, const char *addr)
 {
    static_assert(sizeof(Pack<T, VEC>) <= 16, "pack wider than 128 bits");
    typedef typename RawVec<sizeof(Pack<T, VEC>)>::type V;
    V raw;
-   if (nt) raw = __builtin_nontemporal_load(reinterpret_cast<const V *>(addr));
+   if constexpr (NT) raw = __builtin_nontemporal_load(reinterpret_cast<const V *>(addr));
    else    raw = *reinterpret_cast<const V *>(addr);
    __builtin_memcpy(&p, &raw, sizeof(V));
 }
-template <class T, int VEC>
-OCH_D void store_wide(const Pack<T, VEC> &p, char *addr, int nt = 0)
+template <class T, int VEC, bool NT = false>
+OCH_D void store_wide(const Pack<T, VEC> &p, char *addr)
 {
    typedef typename RawVec<sizeof(Pack<T, VEC>)>::type V;
    V raw;
    __builtin_memcpy(&raw, &p, sizeof(V));
-   if (nt) __builtin_nontemporal_store(raw, reinterpret_cast<V *>(addr));
+   if constexpr (NT) __builtin_nontemporal_store(raw, reinterpret_cast<V *>(addr));
    else    *reinterpret_cast<V *>(addr) = raw;
 }
 
-template <class T, int VEC>
-OCH_D void load_pack(Pack<T, VEC> &p, const char *addr, int64_t estride, int vec, int nt = 0)
+template <class T, int VEC, bool NT = false>
+OCH_D void load_pack(Pack<T, VEC> &p, const char *addr, int64_t estride, int vec)
 {
-   if (vec) load_wide<T, VEC>(p, addr, nt);
+   if (vec) load_wide<T, VEC, NT>(p, addr);
    else
    {
 #pragma unroll
       for (int k = 0; k < VEC; k++) p.v[k] = *reinterpret_cast<const T *>(addr + k * estride);
    }
 }
-template <class T, int VEC>
-OCH_D void store_pack(const Pack<T, VEC> &p, char *addr, int64_t estride, int vec, int nt = 0)
+template <class T, int VEC, bool NT = false>
+OCH_D void store_pack(const Pack<T, VEC> &p, char *addr, int64_t estride, int vec)
 {
-   if (vec) store_wide<T, VEC>(p, addr, nt);
+   if (vec) store_wide<T, VEC, NT>(p, addr);
    else
    {
 #pragma unroll
@@ -147,7 +148,7 @@ OCH_D void group_offsets(const EwParams<NOPS> &p, uint32_t g, int64_t (&off)[NOP
 #define OCH_EW_STREAM_BYTES (48ull << 20)
 
 /* z = f(x, y) */
-template <class F, int VEC, int UNR, bool FAST>
+template <class F, int VEC, int UNR, bool FAST, bool NT = false>
 __global__ __launch_bounds__(OCH_EW_BLOCK) void ew3_kernel(const EwParams<3> p)
 {
    typedef typename F::A A; typedef typename F::B B; typedef typename F::R R;
@@ -158,8 +159,8 @@ __global__ __launch_bounds__(OCH_EW_BLOCK) void ew3_kernel(const EwParams<3> p)
    {  uint32_t g = base + u * OCH_EW_BLOCK;
       if (g < p.ngroups)
       {  group_offsets<3>(p, g, off[u]);
-         load_pack<A, VEC>(a[u], p.ptr[0] + off[u][0], p.estride[0], FAST || p.vecmode[0], p.nt);
-         load_pack<B, VEC>(b[u], p.ptr[1] + off[u][1], p.estride[1], FAST || p.vecmode[1], p.nt);
+         load_pack<A, VEC, NT>(a[u], p.ptr[0] + off[u][0], p.estride[0], FAST || p.vecmode[0]);
+         load_pack<B, VEC, NT>(b[u], p.ptr[1] + off[u][1], p.estride[1], FAST || p.vecmode[1]);
       }
    }
 #pragma unroll
@@ -169,13 +170,13 @@ __global__ __launch_bounds__(OCH_EW_BLOCK) void ew3_kernel(const EwParams<3> p)
       {  Pack<R, VEC> r;
 #pragma unroll
          for (int k = 0; k < VEC; k++) r.v[k] = F::f(a[u].v[k], b[u].v[k]);
-         store_pack<R, VEC>(r, p.ptr[2] + off[u][2], p.estride[2], FAST || p.vecmode[2], p.nt);
+         store_pack<R, VEC, NT>(r, p.ptr[2] + off[u][2], p.estride[2], FAST || p.vecmode[2]);
       }
    }
 }
 
 /* y = f(x) */
-template <class F, int VEC, int UNR, bool FAST>
+template <class F, int VEC, int UNR, bool FAST, bool NT = false>
 __global__ __launch_bounds__(OCH_EW_BLOCK) void ew2_kernel(const EwParams<2> p)
 {
    typedef typename F::A A; typedef typename F::R R;
@@ -186,7 +187,7 @@ __global__ __launch_bounds__(OCH_EW_BLOCK) void ew2_kernel(const EwParams<2> p)
    {  uint32_t g = base + u * OCH_EW_BLOCK;
       if (g < p.ngroups)
       {  group_offsets<2>(p, g, off[u]);
-         load_pack<A, VEC>(a[u], p.ptr[0] + off[u][0], p.estride[0], FAST || p.vecmode[0], p.nt);
+         load_pack<A, VEC, NT>(a[u], p.ptr[0] + off[u][0], p.estride[0], FAST || p.vecmode[0]);
       }
    }
 #pragma unroll
@@ -196,7 +197,7 @@ __global__ __launch_bounds__(OCH_EW_BLOCK) void ew2_kernel(const EwParams<2> p)
       {  Pack<R, VEC> r;
 #pragma unroll
          for (int k = 0; k < VEC; k++) r.v[k] = F::f(a[u].v[k]);
-         store_pack<R, VEC>(r, p.ptr[1] + off[u][1], p.estride[1], FAST || p.vecmode[1], p.nt);
+         store_pack<R, VEC, NT>(r, p.ptr[1] + off[u][1], p.estride[1], FAST || p.vecmode[1]);
       }
    }
 }
@@ -204,7 +205,7 @@ __global__ __launch_bounds__(OCH_EW_BLOCK) void ew2_kernel(const EwParams<2> p)
 /* x = f(x, flat index, param): fill, conditional fill, steps. F::RMW tells whether the
    old value is read. The flat index counts elements in the order of the NORMALISED
    dimensions, so index-dependent functors are launched without reordering. */
-template <class F, int VEC, int UNR, bool FAST>
+template <class F, int VEC, int UNR, bool FAST, bool NT = false>
 __global__ __launch_bounds__(OCH_EW_BLOCK) void ew1_kernel(const EwParams<1> p, const typename F::Param prm)
 {
    typedef typename F::R R;
@@ -219,7 +220,7 @@ __global__ __launch_bounds__(OCH_EW_BLOCK) void ew1_kernel(const EwParams<1> p, 
          if constexpr (F::RMW) load_pack<R, VEC>(r, p.ptr[0] + off[0], p.estride[0], FAST || p.vecmode[0]);
 #pragma unroll
          for (int k = 0; k < VEC; k++) r.v[k] = F::f(r.v[k], p.group0 + (uint64_t)g * VEC + k, prm);
-         store_pack<R, VEC>(r, p.ptr[0] + off[0], p.estride[0], FAST || p.vecmode[0], p.nt);
+         store_pack<R, VEC, NT>(r, p.ptr[0] + off[0], p.estride[0], FAST || p.vecmode[0]);
       }
    }
 }
@@ -250,8 +251,8 @@ constexpr int tile_dim(size_t maxsize) { return maxsize >= 16 ? 32 : 64; }
 template <class T> constexpr int tile_pitch(int tile) { return tile + (sizeof(T) >= 4 ? 1 : 4 / (int)sizeof(T)); }
 template <class T> constexpr int tile_bytes(int tile) { return ((tile * tile_pitch<T>(tile) * (int)sizeof(T)) + 15) / 16 * 16; }
 
-template <class T, int TILE>
-OCH_D void tile_stage(T *lds, const char *base, int64_t s0, uint32_t n0, uint32_t n1, int nt)
+template <class T, int TILE, bool NT>
+OCH_D void tile_stage(T *lds, const char *base, int64_t s0, uint32_t n0, uint32_t n1)
 {
    constexpr int VK = vec_for_c<T>();
    constexpr int LPR = TILE / VK;                        /* lanes per row (fixed index along dimension 0) */
@@ -263,7 +264,7 @@ OCH_D void tile_stage(T *lds, const char *base, int64_t s0, uint32_t n0, uint32_
 #pragma unroll
    for (int u = 0; u < PASSES; u++)
    {  uint32_t i0 = row + u * RPP;
-      if (i0 < n0 && i1 < n1) load_wide<T, VK>(v[u], base + (int64_t)i0 * s0 + (int64_t)i1 * (int64_t)sizeof(T), nt);
+      if (i0 < n0 && i1 < n1) load_wide<T, VK, NT>(v[u], base + (int64_t)i0 * s0 + (int64_t)i1 * (int64_t)sizeof(T));
    }
 #pragma unroll
    for (int u = 0; u < PASSES; u++)
@@ -297,7 +298,7 @@ OCH_D void tile_origin(const TileParams<NOPS> &p, int tile, int64_t (&off)[NOPS]
    }
 }
 
-template <class F, int VEC>
+template <class F, int VEC, bool NT>
 __global__ __launch_bounds__(OCH_TILE_THREADS) void ew3_tile_kernel(const TileParams<3> p)
 {
    typedef typename F::A A; typedef typename F::B B; typedef typename F::R R;
@@ -310,8 +311,8 @@ __global__ __launch_bounds__(OCH_TILE_THREADS) void ew3_tile_kernel(const TilePa
    tile_origin<3>(p, TILE, off);
    const uint32_t r0 = p.n0 - blockIdx.x * TILE, r1 = p.n1 - tile_row() * TILE;
    const uint32_t n0 = r0 < (uint32_t)TILE ? r0 : TILE, n1 = r1 < (uint32_t)TILE ? r1 : TILE;
-   if (p.trans[0]) tile_stage<A, TILE>(la, p.ptr[0] + off[0], p.s0[0], n0, n1, p.nt);
-   if (p.trans[1]) tile_stage<B, TILE>(lb, p.ptr[1] + off[1], p.s0[1], n0, n1, p.nt);
+   if (p.trans[0]) tile_stage<A, TILE, NT>(la, p.ptr[0] + off[0], p.s0[0], n0, n1);
+   if (p.trans[1]) tile_stage<B, TILE, NT>(lb, p.ptr[1] + off[1], p.s0[1], n0, n1);
    __syncthreads();
    constexpr int LPC = TILE / VEC, CPP = OCH_TILE_THREADS / LPC, PASSES = (TILE + CPP - 1) / CPP;
    const uint32_t i0 = (threadIdx.x % LPC) * VEC, col = threadIdx.x / LPC;
@@ -325,21 +326,21 @@ __global__ __launch_bounds__(OCH_TILE_THREADS) void ew3_tile_kernel(const TilePa
 #pragma unroll
             for (int k = 0; k < VEC; k++) a.v[k] = la[i1 * tile_pitch<A>(TILE) + i0 + k];
          }
-         else load_pack<A, VEC>(a, p.ptr[0] + off[0] + (int64_t)i0 * p.s0[0] + (int64_t)i1 * p.s1[0], p.s0[0], p.vecmode[0], p.nt);
+         else load_pack<A, VEC, NT>(a, p.ptr[0] + off[0] + (int64_t)i0 * p.s0[0] + (int64_t)i1 * p.s1[0], p.s0[0], p.vecmode[0]);
          if (p.trans[1])
          {
 #pragma unroll
             for (int k = 0; k < VEC; k++) b.v[k] = lb[i1 * tile_pitch<B>(TILE) + i0 + k];
          }
-         else load_pack<B, VEC>(b, p.ptr[1] + off[1] + (int64_t)i0 * p.s0[1] + (int64_t)i1 * p.s1[1], p.s0[1], p.vecmode[1], p.nt);
+         else load_pack<B, VEC, NT>(b, p.ptr[1] + off[1] + (int64_t)i0 * p.s0[1] + (int64_t)i1 * p.s1[1], p.s0[1], p.vecmode[1]);
 #pragma unroll
          for (int k = 0; k < VEC; k++) r.v[k] = F::f(a.v[k], b.v[k]);
-         store_pack<R, VEC>(r, p.ptr[2] + off[2] + (int64_t)i0 * p.s0[2] + (int64_t)i1 * p.s1[2], p.s0[2], p.vecmode[2], p.nt);
+         store_pack<R, VEC, NT>(r, p.ptr[2] + off[2] + (int64_t)i0 * p.s0[2] + (int64_t)i1 * p.s1[2], p.s0[2], p.vecmode[2]);
       }
    }
 }
 
-template <class F, int VEC>
+template <class F, int VEC, bool NT>
 __global__ __launch_bounds__(OCH_TILE_THREADS) void ew2_tile_kernel(const TileParams<2> p)
 {
    typedef typename F::A A; typedef typename F::R R;
@@ -351,7 +352,7 @@ __global__ __launch_bounds__(OCH_TILE_THREADS) void ew2_tile_kernel(const TilePa
    tile_origin<2>(p, TILE, off);
    const uint32_t r0 = p.n0 - blockIdx.x * TILE, r1 = p.n1 - tile_row() * TILE;
    const uint32_t n0 = r0 < (uint32_t)TILE ? r0 : TILE, n1 = r1 < (uint32_t)TILE ? r1 : TILE;
-   tile_stage<A, TILE>(la, p.ptr[0] + off[0], p.s0[0], n0, n1, p.nt);
+   tile_stage<A, TILE, NT>(la, p.ptr[0] + off[0], p.s0[0], n0, n1);
    __syncthreads();
    constexpr int LPC = TILE / VEC, CPP = OCH_TILE_THREADS / LPC, PASSES = (TILE + CPP - 1) / CPP;
    const uint32_t i0 = (threadIdx.x % LPC) * VEC, col = threadIdx.x / LPC;
@@ -362,7 +363,7 @@ __global__ __launch_bounds__(OCH_TILE_THREADS) void ew2_tile_kernel(const TilePa
       {  Pack<R, VEC> r;
 #pragma unroll
          for (int k = 0; k < VEC; k++) r.v[k] = F::f(la[i1 * tile_pitch<A>(TILE) + i0 + k]);
-         store_pack<R, VEC>(r, p.ptr[1] + off[1] + (int64_t)i0 * p.s0[1] + (int64_t)i1 * p.s1[1], p.s0[1], p.vecmode[1], p.nt);
+         store_pack<R, VEC, NT>(r, p.ptr[1] + off[1] + (int64_t)i0 * p.s0[1] + (int64_t)i1 * p.s1[1], p.s0[1], p.vecmode[1]);
       }
    }
 }
@@ -613,13 +614,15 @@ static int launch_ew3(int ndims, const size_t *size,
       const int tb[3] = { tile_bytes<A>(TILE), tile_bytes<B>(TILE), 0 };
       TileParams<3> tp; dim3 grid; size_t lds;
       if (ew_tile_params<3>(tp, s, es, TILE, VEC, grid, lds, tb))
-      {  hipLaunchKernelGGL((ew3_tile_kernel<F, VEC>), grid, dim3(OCH_TILE_THREADS), lds, stream, tp);
+      {  if (tp.nt) hipLaunchKernelGGL((ew3_tile_kernel<F, VEC, true>), grid, dim3(OCH_TILE_THREADS), lds, stream, tp);
+         else       hipLaunchKernelGGL((ew3_tile_kernel<F, VEC, false>), grid, dim3(OCH_TILE_THREADS), lds, stream, tp);
          OCH_CHECK_LAUNCH();
          return 0;
       }
       return ew_dispatch<3>(s, flat0, VEC, es,
          [&](const EwParams<3> &p, uint32_t blocks)
-         {  hipLaunchKernelGGL((ew3_kernel<F, VEC, OCH_EW_UNR, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
+         {  if (p.nt) hipLaunchKernelGGL((ew3_kernel<F, VEC, OCH_EW_UNR, true, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p);
+            else      hipLaunchKernelGGL((ew3_kernel<F, VEC, OCH_EW_UNR, true, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
          [&](const EwParams<3> &p, uint32_t blocks)
          {  hipLaunchKernelGGL((ew3_kernel<F, VEC, 2, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
          [&](const EwParams<3> &p, uint32_t blocks)
@@ -643,13 +646,15 @@ static int launch_ew2(int ndims, const size_t *size,
       const int tb[2] = { tile_bytes<A>(TILE), 0 };
       TileParams<2> tp; dim3 grid; size_t lds;
       if (ew_tile_params<2>(tp, s, es, TILE, VEC, grid, lds, tb))
-      {  hipLaunchKernelGGL((ew2_tile_kernel<F, VEC>), grid, dim3(OCH_TILE_THREADS), lds, stream, tp);
+      {  if (tp.nt) hipLaunchKernelGGL((ew2_tile_kernel<F, VEC, true>), grid, dim3(OCH_TILE_THREADS), lds, stream, tp);
+         else       hipLaunchKernelGGL((ew2_tile_kernel<F, VEC, false>), grid, dim3(OCH_TILE_THREADS), lds, stream, tp);
          OCH_CHECK_LAUNCH();
          return 0;
       }
       return ew_dispatch<2>(s, flat0, VEC, es,
          [&](const EwParams<2> &p, uint32_t blocks)
-         {  hipLaunchKernelGGL((ew2_kernel<F, VEC, OCH_EW_UNR, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
+         {  if (p.nt) hipLaunchKernelGGL((ew2_kernel<F, VEC, OCH_EW_UNR, true, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p);
+            else      hipLaunchKernelGGL((ew2_kernel<F, VEC, OCH_EW_UNR, true, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
          [&](const EwParams<2> &p, uint32_t blocks)
          {  hipLaunchKernelGGL((ew2_kernel<F, VEC, 2, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
          [&](const EwParams<2> &p, uint32_t blocks)
@@ -671,7 +676,8 @@ static int launch_ew1(int ndims, const size_t *size, const ptrdiff_t *st, void *
    return ew_launch_chunked<1>(shape, 0, [&](const EwShape<1> &s, uint64_t flat0) -> int
    {  return ew_dispatch<1>(s, flat0, VEC, es,
          [&](const EwParams<1> &p, uint32_t blocks)
-         {  hipLaunchKernelGGL((ew1_kernel<F, VEC, OCH_EW_UNR, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p, prm); },
+         {  if (p.nt) hipLaunchKernelGGL((ew1_kernel<F, VEC, OCH_EW_UNR, true, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p, prm);
+            else      hipLaunchKernelGGL((ew1_kernel<F, VEC, OCH_EW_UNR, true, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p, prm); },
          [&](const EwParams<1> &p, uint32_t blocks)
          {  hipLaunchKernelGGL((ew1_kernel<F, VEC, 2, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p, prm); },
          [&](const EwParams<1> &p, uint32_t blocks)
