@@ -517,7 +517,7 @@ static int ew_dispatch(const EwShape<NOPS> &s, uint64_t flat0, int vec, const in
 {
    EwParams<NOPS> p;
    auto run = [&](const EwShape<NOPS> &sh, uint64_t f0) -> bool
-   {  if (vec <= 1 || !ew_params<NOPS>(p, sh, vec, es, f0)) return false;
+   {  if (!ew_params<NOPS>(p, sh, vec, es, f0)) return false;      /* vec = 1 (16-byte elements) always fits */
       bool all = true;
       for (int k = 0; k < NOPS; k++) all = all && p.vecmode[k];
       if (all) wide(p, (p.ngroups + OCH_EW_BLOCK * OCH_EW_UNR - 1) / (OCH_EW_BLOCK * OCH_EW_UNR));
@@ -656,7 +656,8 @@ static int launch_ew2(int ndims, const size_t *size,
          {  if (p.nt) hipLaunchKernelGGL((ew2_kernel<F, VEC, OCH_EW_UNR, true, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p);
             else      hipLaunchKernelGGL((ew2_kernel<F, VEC, OCH_EW_UNR, true, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
          [&](const EwParams<2> &p, uint32_t blocks)
-         {  hipLaunchKernelGGL((ew2_kernel<F, VEC, 2, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
+         {  if (p.nt) hipLaunchKernelGGL((ew2_kernel<F, VEC, 2, false, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p);
+            else      hipLaunchKernelGGL((ew2_kernel<F, VEC, 2, false, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
          [&](const EwParams<2> &p, uint32_t blocks)
          {  hipLaunchKernelGGL((ew2_kernel<F, 1, 1, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); });
    });

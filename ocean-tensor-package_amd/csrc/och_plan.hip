@@ -38,7 +38,7 @@ static int analyze(const int *elemsize, int ndims, const size_t *size, const ptr
          tiled = ew_tile_params<NOPS>(tp, s, esr, tile, vec, grid, lds, tbr);
       }
       if (tiled) { kernel = OCH_KERNEL_TILED; v = vec; }
-      else if (vec > 1 && ew_params<NOPS>(p, s, vec, es, flat0))
+      else if (ew_params<NOPS>(p, s, vec, es, flat0))
       {  bool all = true;
          for (int k = 0; k < NOPS; k++) all = all && p.vecmode[k];
          kernel = all ? OCH_KERNEL_WIDE : OCH_KERNEL_MIXED; v = vec;
