@@ -46,6 +46,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-step", action="store_true", help="time the configuration-2 step only (for profiling)")
+    ap.add_argument("--only-gemm", action="store_true", help="run each configuration-5 GEMM twice and exit (for counter collection)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (every figure here is a one-GPU figure)" % args.gpus)
@@ -59,6 +60,23 @@ def main():
     stream = oh.Stream()
     lib = oh.lib
     B, R = oh.B, oh.R
+    if args.only_gemm:
+        rng = np.random.default_rng(5)
+        for dt, es, nm, dim in ((oh.DOUBLE, 8, "double", 8192), (oh.FLOAT, 4, "float", 8192), (oh.CFLOAT, 8, "cfloat", 4096)):
+            a, b, c = [oh.DeviceBuffer(es * dim * dim, stream) for _ in range(3)]
+            block = rng.uniform(-1, 1, 1 << 22).astype(np.float32 if nm != "double" else np.float64)
+            for buf in (a, b):
+                for off in range(0, es * dim * dim, block.nbytes):
+                    buf.upload(block[: (min(block.nbytes, es * dim * dim - off)) // block.itemsize], offset=off)
+            one = np.array([1, 0], dtype=block.dtype); zero = np.zeros(2, dtype=block.dtype)
+            for ta, tb in ((b"N", b"N"), (b"T", b"N"), (b"N", b"T")):
+                for _ in range(2):
+                    oh.check(lib.och_gemm(dt, ta, tb, dim, dim, dim, one.ctypes.data, a.ptr, dim, b.ptr, dim, zero.ctypes.data, c.ptr, dim, 1, stream.handle))
+            stream.synchronize()
+            for buf in (a, b, c):
+                buf.free()
+        print(json.dumps({"mode": "only-gemm"}))
+        return
     F32, F64, I32, I16, CF, CD = oh.FLOAT, oh.DOUBLE, oh.INT32, oh.INT16, oh.CFLOAT, oh.CDOUBLE
 
     def time_launches(fn, reps=20, warm=3):
