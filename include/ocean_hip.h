@@ -305,6 +305,27 @@ int och_fill_index(int dtype, int ndims, const size_t *size, int64_t **offsets,
                    const ptrdiff_t *strides, void *ptr, och_scalar value, och_stream stream);
 
 /* ======================================================================== */
+/* Find / mask-to-offset: positions of the non-zero elements of a bool      */
+/* tensor, in the order of its dimensions with dimension 0 running fastest. */
+/* The reference has these on the CPU only (solid_cpu_find_prepare, _apply, */
+/* _finalize, solid/src/core/cpu/template_index.c:296-500; callers          */
+/* src/core/cpu/op/tensor_index_cpu.c:60-155; the GPU table leaves          */
+/* Tensor_find and Tensor_maskToOffset empty, docs/future_work.md:33).      */
+/*  och_find_count  counts the non-zero elements and fills `workspace`      */
+/*                  (device memory, och_find_workspace_size(nelem) bytes)   */
+/*                  with per-chunk start positions; returns after the count */
+/*                  is known (one stream synchronisation).                  */
+/*  och_find_apply  writes, for the k-th non-zero element, either its ndims */
+/*                  indices to out[k*ndims .. ] (multiplier == NULL) or the */
+/*                  single value sum_d index_d * multiplier[d] to out[k].   */
+/* ======================================================================== */
+size_t och_find_workspace_size(size_t nelem);
+int och_find_count(int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr,
+                   void *workspace, size_t *nnz, och_stream stream);
+int och_find_apply(int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr,
+                   void *workspace, const int64_t *multiplier, int64_t *out, och_stream stream);
+
+/* ======================================================================== */
 /* Launch analysis of an elementwise call, without launching anything.      */
 /* Reports what the library derives from the operands before a launch, the  */
 /* counterpart of solid_gpu_elemwise{1,2,3}_analyze (src/core/gpu/op/       */

@@ -54,6 +54,17 @@ int OcTensor_fill(OcTensor *tensor, OcScalar *value)
    return m->Tensor_fill(tensor, value);
 }
 
+OcTensor *OcTensor_find(OcTensor *mask)
+{  OcModuleCore *m = OcModuleCore_forDevice(mask->device);
+   if (m == NULL || m->Tensor_find == NULL) { OcErrorMessage("Find is not supported on device %s", mask->device->name); return NULL; }
+   return m->Tensor_find(mask);
+}
+OcTensor *OcTensor_maskToOffset(OcTensor *mask, OcIndex *strides)
+{  OcModuleCore *m = OcModuleCore_forDevice(mask->device);
+   if (m == NULL || m->Tensor_maskToOffset == NULL) { OcErrorMessage("Mask-to-offset is not supported on device %s", mask->device->name); return NULL; }
+   return m->Tensor_maskToOffset(mask, strides);
+}
+
 /* ---- elementwise -------------------------------------------------------------------------- */
 typedef int (*oc_binary_fn)(OcTensor *, OcTensor *, OcTensor *);
 typedef int (*oc_unary_fn)(OcTensor *, OcTensor *);

@@ -315,6 +315,33 @@ static int OcTensorGPU_fillIndex(OcTensorIndexView *view, OcScalar *scalar)
    return OcTensor_update(v);
 }
 
+/* Positions of the non-zero elements of a bool tensor (the reference implements these on the CPU only,
+   src/core/cpu/op/tensor_index_cpu.c:60-155; its GPU table leaves the two entries empty). The result lives on
+   the tensor's device: find -> int64 tensor of size ndims x nnz, maskToOffset -> nnz offsets sum(index * stride). */
+static OcTensor *find_common(OcTensor *tensor, OcIndex *multiplier)
+{  OcStorage *work; OcTensor *result = NULL; size_t nnz = 0; OcSize rsize[2]; int64_t mult[OC_TENSOR_MAX_DIMS]; int i;
+   if (tensor->dtype != OcDTypeBool) { OcErrorMessage("Find requires a Boolean tensor"); return NULL; }
+   if (activate(tensor->device) != 0) return NULL;
+   work = OcStorageGPU_create((OcSize)och_find_workspace_size((size_t)tensor->nelem), OcDTypeInt8, tensor->device, tensor->storage->stream);
+   if (work == NULL) return NULL;
+   if (och_find_count(tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), work->data, &nnz, GPU_STREAM(tensor)) != 0)
+   {  OcErrorMessage("%s", och_last_error()); goto final; }
+   if (multiplier) { rsize[0] = (OcSize)nnz; result = OcTensor_create(1, rsize, NULL, OcDTypeInt64, tensor->device); }
+   else { rsize[0] = tensor->ndims; rsize[1] = (OcSize)nnz; result = OcTensor_create(2, rsize, NULL, OcDTypeInt64, tensor->device); }
+   if (result == NULL) goto final;
+   for (i = 0; multiplier && i < tensor->ndims; i++) mult[i] = multiplier[i];
+   if (OcTensor_startRead(result, tensor) != 0 ||
+       och_find_apply(tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), work->data, multiplier ? mult : NULL,
+                      (int64_t *)OcTensor_data(result), GPU_STREAM(result)) != 0)
+   {  OcErrorMessage("%s", och_last_error()); OcDecrefTensor(result); result = NULL; goto final; }
+   OcTensor_update(result); OcTensor_finishRead(result, tensor);
+final:
+   OcDecrefStorage(work);
+   return result;
+}
+static OcTensor *OcTensorGPU_find(OcTensor *tensor) { return find_common(tensor, NULL); }
+static OcTensor *OcTensorGPU_maskToOffset(OcTensor *tensor, OcIndex *strides) { return find_common(tensor, strides); }
+
 /* ---- elementwise (op/tensor_unary_gpu.c:59-93, op/tensor_binary_gpu.c:58-97) ------------ */
 static int unary_call(int op, const char *name, OcTensor *src, OcTensor *dst)
 {  if (!och_unary_supported(op, src->dtype)) return OcErrorMessage("Function %s is not supported for type %s on GPU", name, OcDType_name(src->dtype));
@@ -465,7 +492,7 @@ static void fill_table(OcModuleCore *m)
    m->Tensor_byteswapNoFlag = OcTensorGPU_byteswapNoFlag;
    m->Tensor_fill = OcTensorGPU_fill; m->Tensor_fillNaN = OcTensorGPU_fillNaN; m->Tensor_maskedFill = OcTensorGPU_maskedFill;
    m->Tensor_stepsInt64 = OcTensorGPU_stepsInt64; m->Tensor_stepsDouble = OcTensorGPU_stepsDouble; m->Tensor_stepsCDouble = OcTensorGPU_stepsCDouble;
-   m->Tensor_find = NULL; m->Tensor_maskToOffset = NULL;              /* not available on the GPU in the reference either (docs/future_work.md:33) */
+   m->Tensor_find = OcTensorGPU_find; m->Tensor_maskToOffset = OcTensorGPU_maskToOffset;   /* empty in the reference's GPU table (docs/future_work.md:33) */
    m->Tensor_indexToOffset = OcTensorGPU_indexToOffset; m->Tensor_addIfNegative = OcTensorGPU_addIfNegative;
    m->Tensor_getIndex = OcTensorGPU_getIndex; m->Tensor_setIndex = OcTensorGPU_setIndex; m->Tensor_fillIndex = OcTensorGPU_fillIndex;
 #define OC_X(NAME, OP) m->Tensor_##NAME = OcTensorGPU_##NAME;

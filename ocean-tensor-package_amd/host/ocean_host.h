@@ -68,6 +68,8 @@ int       OcTensor_isContiguous(OcTensor *tensor);
 int OcTensor_copy(OcTensor *src, OcTensor *dst);                                   /* any device, dtype, byte order */
 int OcTensor_ensure(OcTensor **tensor, OcDType dtype, OcDevice *device);           /* replaces *tensor by a converted native-order copy when needed */
 int OcTensor_fill(OcTensor *tensor, OcScalar *value);
+OcTensor *OcTensor_find(OcTensor *mask);                                         /* ndims x nnz indices of the non-zero elements */
+OcTensor *OcTensor_maskToOffset(OcTensor *mask, OcIndex *strides);               /* nnz offsets sum(index * strides) */
 int OcTensor_binary(int op, OcTensor *src1, OcTensor *src2, OcTensor **dst);       /* op: index into the table's binary block */
 int OcTensor_unary(int op, OcTensor *src, OcTensor **dst);
 #define OcTensor_add(a, b, dst)       OcTensor_binary(0, a, b, dst)

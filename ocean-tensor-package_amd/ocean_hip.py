@@ -185,6 +185,9 @@ PROTOTYPES = {
     "och_get_index": (_i, [_i, _i, _sz, C.POINTER(C.POINTER(C.c_int64)), _st, _vp, _st, _vp, _vp]),
     "och_set_index": (_i, [_i, _i, _sz, C.POINTER(C.POINTER(C.c_int64)), _st, _vp, _st, _vp, _vp]),
     "och_fill_index": (_i, [_i, _i, _sz, C.POINTER(C.POINTER(C.c_int64)), _st, _vp, Scalar, _vp]),
+    "och_find_workspace_size": (C.c_size_t, [C.c_size_t]),
+    "och_find_count": (_i, [_i, _sz, _st, _vp, _vp, C.POINTER(C.c_size_t), _vp]),
+    "och_find_apply": (_i, [_i, _sz, _st, _vp, _vp, C.POINTER(C.c_int64), _vp, _vp]),
     "och_elemwise_analyze": (_i, [_i, C.POINTER(_i), _i, _sz, C.POINTER(_st), C.POINTER(_vp), C.c_void_p]),
 }
 

@@ -85,6 +85,10 @@ lib.OcTensor_axisReduce.argtypes = [C.c_int, TP, C.c_int, C.POINTER(C.c_int), C.
 lib.OcTensor_gemm.argtypes = [C.POINTER(Scalar), TP, C.c_char, TP, C.c_char, C.POINTER(Scalar), C.POINTER(TP)]
 lib.OcTensor_mtimes.argtypes = [TP, TP, C.POINTER(TP)]
 lib.OcTensor_fill.argtypes = [TP, C.POINTER(Scalar)]
+lib.OcTensor_find.restype = TP
+lib.OcTensor_find.argtypes = [TP]
+lib.OcTensor_maskToOffset.restype = TP
+lib.OcTensor_maskToOffset.argtypes = [TP, _ss]
 lib.OcSolid_analyzeReduceAxis.argtypes = [TP, C.c_int, C.POINTER(C.c_int), TP, C.POINTER(ReduceAxis)]
 lib.OcShape_sortStrides2.argtypes = [C.c_int, _ss, _ss, _ss]
 lib.OcShape_mergeBlocks2.argtypes = [C.POINTER(C.c_int), _ss, _ss, _ss]

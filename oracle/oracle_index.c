@@ -82,3 +82,24 @@ int oracle_set_index(int dtype, int ndims, const size_t *size, int64_t **offsets
 {  return o_index(1, dtype, ndims, size, offsets, strides1, ptr1, strides2, ptr2, NULL); }
 int oracle_fill_index(int dtype, int ndims, const size_t *size, int64_t **offsets, const ptrdiff_t *strides, void *ptr, och_scalar value)
 {  return o_index(2, dtype, ndims, size, offsets, strides, ptr, NULL, NULL, &value); }
+
+/* find / mask-to-offset (template_index.c:296-500): positions of the non-zero elements of a bool tensor in element
+   order (dimension 0 fastest). multiplier == NULL: ndims indices per hit; otherwise sum of index * multiplier. */
+size_t oracle_find(int ndims, const size_t *size, const ptrdiff_t *strides, const void *ptr, const int64_t *multiplier, int64_t *out)
+{
+   size_t idx[O_MAX_DIMS] = { 0 }, n = 1, e, count = 0; int d;
+   for (d = 0; d < ndims; d++) n *= size[d];
+   for (e = 0; e < n; e++)
+   {  ptrdiff_t off = 0;
+      for (d = 0; d < ndims; d++) off += (ptrdiff_t)idx[d] * strides[d];
+      if (((const char *)ptr)[off] != 0)
+      {  if (out)
+         {  if (multiplier) { int64_t s = 0; for (d = 0; d < ndims; d++) s += (int64_t)idx[d] * multiplier[d]; out[count] = s; }
+            else for (d = 0; d < ndims; d++) out[count * ndims + d] = (int64_t)idx[d];
+         }
+         count++;
+      }
+      for (d = 0; d < ndims; d++) { if (++idx[d] < size[d]) break; idx[d] = 0; }
+   }
+   return count;
+}

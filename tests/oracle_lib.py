@@ -55,6 +55,7 @@ def setup(oh):
         ("oracle_get_index", _i, [_i, _i, _sz, C.POINTER(C.POINTER(C.c_int64)), _st, _vp, _st, _vp]),
         ("oracle_set_index", _i, [_i, _i, _sz, C.POINTER(C.POINTER(C.c_int64)), _st, _vp, _st, _vp]),
         ("oracle_fill_index", _i, [_i, _i, _sz, C.POINTER(C.POINTER(C.c_int64)), _st, _vp, S]),
+        ("oracle_find", C.c_size_t, [_i, _sz, _st, _vp, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     ]:
         if hasattr(lib, name):
             _proto(getattr(lib, name), res, args)

@@ -192,3 +192,19 @@ def test_unary_and_fill(gpu):
     val = host.scalar(host.DOUBLE, 3.25)
     host.check(host.lib.OcTensor_fill(t, C.byref(val)))
     assert (host.to_numpy(t) == 3.25).all()
+
+
+def test_find_and_mask_to_offset_through_the_table(gpu):
+    rng = np.random.default_rng(12)
+    mask = (rng.random((9, 40, 33)) < 0.2).astype(np.uint8)                 # Ocean dims (33, 40, 9)
+    t = host.from_numpy(mask, host.BOOL, gpu)
+    idx = host.lib.OcTensor_find(t)
+    assert idx and idx.contents.dtype == host.INT64
+    got = host.to_numpy(idx)                                                # numpy (nnz, ndims)
+    want = np.stack(np.nonzero(mask), axis=1)[:, ::-1]                      # C-order walk = Ocean dimension 0 fastest
+    assert np.array_equal(got, want)
+    strides = host._arr([8, 8 * 33, 8 * 33 * 40])
+    off = host.lib.OcTensor_maskToOffset(t, strides)
+    assert np.array_equal(host.to_numpy(off), want @ np.array([8, 8 * 33, 8 * 33 * 40]))
+    f = host.from_numpy(np.zeros((3, 3), np.float32), host.FLOAT, gpu)
+    assert not host.lib.OcTensor_find(f) and b"Boolean" in host.lib.OcError_lastMessage()

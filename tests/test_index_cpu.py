@@ -76,3 +76,22 @@ def test_oracle_index_to_offset(dtype):
     es = idx.itemsize
     assert orc.lib.oracle_index_to_offset(dtype, nd, strides.ctypes.data_as(IC.P64), es, n, nd * es, orc.ptr(idx), 8, orc.ptr(out)) == 0
     assert np.array_equal(out, idx.astype(np.int64) @ strides)
+
+
+@pytest.mark.parametrize("shape", [(7,), (5, 9), (4, 3, 6), (2, 3, 2, 5)])
+def test_oracle_find(shape):
+    """Non-zero positions in element order with the first dimension fastest: numpy's nonzero on the
+    transposed (C-ordered) view gives exactly that order."""
+    rng = np.random.default_rng(len(shape))
+    mask = np.asfortranarray(rng.integers(0, 3, shape) == 0).astype(np.uint8)      # Ocean order: mask[i0, i1, ...]
+    nd = len(shape)
+    want = np.stack(np.nonzero(mask.T)[::-1], axis=1)            # rows sorted with the LAST numpy axis of mask.T ... i.e. i0 fastest
+    n = orc.lib.oracle_find(nd, oh.sizes(shape), oh.strides(mask.strides), orc.ptr(mask), None, None)
+    assert n == int(mask.sum())
+    out = np.zeros((n, nd), np.int64)
+    assert orc.lib.oracle_find(nd, oh.sizes(shape), oh.strides(mask.strides), orc.ptr(mask), None, out.ctypes.data_as(IC.P64)) == n
+    assert np.array_equal(out, want)
+    mult = np.array([3, 100, -7, 1000][:nd], np.int64)
+    off = np.zeros(n, np.int64)
+    assert orc.lib.oracle_find(nd, oh.sizes(shape), oh.strides(mask.strides), orc.ptr(mask), mult.ctypes.data_as(IC.P64), off.ctypes.data_as(IC.P64)) == n
+    assert np.array_equal(off, want @ mult)

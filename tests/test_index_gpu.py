@@ -97,3 +97,40 @@ def test_index_to_offset(hip, stream, dtype):
     assert orc.lib.oracle_index_to_offset(dtype, nd, strides.ctypes.data_as(IC.P64), es, n, nd * es, orc.ptr(idx), 8, orc.ptr(want)) == 0
     assert np.array_equal(dout.download(np.int64, n), want)
     didx.free(); dout.free()
+
+
+@pytest.mark.parametrize("shape,density", [((7,), 0.5), ((5, 9), 0.3), ((17, 33, 64), 0.1), ((515, 2048), 0.5), ((3, 4, 5, 6, 7), 0.9),
+                                           ((100000,), 0.0), ((100000,), 1.0), ((4, 0), 0.5), ((3000, 3001), 0.02)])
+def test_find_and_mask_to_offset(hip, stream, shape, density):
+    """och_find_count / och_find_apply against the oracle, on a dense mask and on a strided view (every second
+    element, reversed) of a larger one. Dimensions go to the library fastest first (reversed numpy order)."""
+    import ctypes as C
+    rng = np.random.default_rng(len(shape) * 31 + int(density * 10))
+    nd = len(shape)
+    big = (rng.random(tuple(2 * s + 1 for s in shape)) < density).astype(np.uint8)
+    dbig = oh.to_device(big, stream)
+    dense = tuple(slice(0, s) for s in shape)
+    strided = tuple(slice(2 * s - 1, None, -2) if s else slice(0, 0) for s in shape)
+    for sel in (dense, strided):
+        view = big[sel]
+        assert view.shape == shape
+        sz, st = oh.sizes(shape[::-1]), oh.strides(view.strides[::-1])
+        off = view.ctypes.data - big.ctypes.data if view.size else 0
+        hptr, dptr = C.c_void_p(big.ctypes.data + off), C.c_void_p(dbig.address + off)
+        work = oh.DeviceBuffer(oh.lib.och_find_workspace_size(view.size), stream)
+        nnz = C.c_size_t(12345)
+        oh.check(oh.lib.och_find_count(nd, sz, st, dptr, work.ptr, C.byref(nnz), stream.handle))
+        want_n = orc.lib.oracle_find(nd, sz, st, hptr, None, None)
+        assert nnz.value == want_n == int(view.sum())
+        out = oh.DeviceBuffer(8 * max(1, want_n * nd), stream)
+        oh.check(oh.lib.och_find_apply(nd, sz, st, dptr, work.ptr, None, out.ptr, stream.handle))
+        want = np.zeros(want_n * nd, np.int64)
+        orc.lib.oracle_find(nd, sz, st, hptr, None, want.ctypes.data_as(IC.P64))
+        assert np.array_equal(out.download(np.int64, want_n * nd), want)
+        mult = np.array([8, -800, 12345, 7, 1 << 33][:nd], np.int64)
+        oh.check(oh.lib.och_find_apply(nd, sz, st, dptr, work.ptr, mult.ctypes.data_as(IC.P64), out.ptr, stream.handle))
+        want = np.zeros(want_n, np.int64)
+        orc.lib.oracle_find(nd, sz, st, hptr, mult.ctypes.data_as(IC.P64), want.ctypes.data_as(IC.P64))
+        assert np.array_equal(out.download(np.int64, want_n), want)
+        work.free(); out.free()
+    dbig.free()
