@@ -5,20 +5,22 @@
 #include <string.h>
 
 namespace och {
-red_fn reduce_lookup_a(int op, int dtype);
-red_fn reduce_lookup_b(int op, int dtype);
-red_fn reduce_lookup_c(int op, int dtype);
-red_fn reduce_lookup_d(int op, int dtype);
+/* the instantiations are spread over eight translation units (build time); each knows its own operations */
+#define OCH_RED_PARTS(X) X(a) X(b) X(c) X(d) X(e) X(f) X(g) X(h)
+#define OCH_X(part) red_fn reduce_lookup_##part(int op, int dtype);
+OCH_RED_PARTS(OCH_X)
+#undef OCH_X
 static_assert((int)R_COUNT == (int)OCH_REDUCE_COUNT && (int)R_NORM2_NAN == (int)OCH_R_NORM2_NAN && (int)R_SUM == (int)OCH_R_SUM,
               "operation lists out of step");
 
 static red_fn reduce_lookup(int op, int dtype)
 {
    if (dtype < 0 || dtype >= DT_COUNT || op < 0 || op >= OCH_REDUCE_COUNT) return nullptr;
-   if (op <= 7) return reduce_lookup_a(op, dtype);
-   if (op <= 14) return reduce_lookup_b(op, dtype);
-   if (op <= 20) return reduce_lookup_c(op, dtype);
-   return reduce_lookup_d(op, dtype);
+   red_fn fn = nullptr;
+#define OCH_X(part) if (fn == nullptr) fn = reduce_lookup_##part(op, dtype);
+   OCH_RED_PARTS(OCH_X)
+#undef OCH_X
+   return fn;
 }
 
 #define OCH_MAX_DEVICES 64

@@ -1,17 +1,14 @@
-/* Full-reduction kernels, operations 8..14 of the reduction list. */
+/* Full-reduction kernels, operations: 4 5 6 7 */
 #include "och_reduce_all.h"
 namespace och {
 red_fn reduce_lookup_b(int op, int dtype)
 {
    switch (op)
    {
-      case 8: return RowR<8>::fn[dtype];
-      case 9: return RowR<9>::fn[dtype];
-      case 10: return RowR<10>::fn[dtype];
-      case 11: return RowR<11>::fn[dtype];
-      case 12: return RowR<12>::fn[dtype];
-      case 13: return RowR<13>::fn[dtype];
-      case 14: return RowR<14>::fn[dtype];
+      case 4: return RowR<4>::fn[dtype];
+      case 5: return RowR<5>::fn[dtype];
+      case 6: return RowR<6>::fn[dtype];
+      case 7: return RowR<7>::fn[dtype];
    }
    return nullptr;
 }

@@ -21,6 +21,8 @@ struct AxisParams
    char    *src, *dst;
    int      nd, rd;
    FastDiv  div[OCH_MAX_DIMS], rdiv[OCH_MAX_DIMS];
+   uint32_t glanes;                              /* lanes per output in the wave-cooperative kernel */
+   FastDiv  rgdiv;                               /* 128-bit groups per row of the first reduced dimension (cooperative kernels) */
    int64_t  st1[OCH_MAX_DIMS], st2[OCH_MAX_DIMS], rst[OCH_MAX_DIMS];
    uint32_t nout, relem, rsize0, rrows;          /* relem = rsize0 * rrows */
 };
@@ -46,11 +48,21 @@ OCH_D int64_t axis_row_offset(const AxisParams &p, uint32_t r)
    return off;
 }
 
+/* Workgroups are dealt to the 8 XCDs round-robin, each XCD with its own L2. This permutation of the block index
+   (within runs of 32 blocks) gives every XCD 4 consecutive logical blocks, so that blocks working on neighbouring
+   segments of the same rows -- which share the cache lines at the segment boundaries when the row pitch is not a
+   multiple of the line size -- meet in one L2 instead of fetching those lines from memory twice. */
+OCH_D uint32_t xcd_neighbour_block(uint32_t b, uint32_t nblocks)
+{  const uint32_t chunk = b & ~31u, r = b & 31u;
+   if (chunk + 32 > nblocks) return b;
+   return chunk + (r & 7u) * 4 + (r >> 3);
+}
+
 /* Neighbouring threads own neighbouring outputs: VEC consecutive outputs each (one 128-bit load
    covers them; needs unit source stride along the first outer dimension). SPLIT slices (waves
    when SPLIT is 4) share each output: slice s takes elements s, s + SPLIT, ... of every row of
    the reduced range and the slices are folded through LDS in slice order. */
-template <class RD, class T, int SPLIT, int VEC>
+template <class RD, class T, int SPLIT, int VEC, bool NT = false>
 __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, const typename RD::Param prm)
 {
    typedef typename RD::Acc Acc;
@@ -58,7 +70,7 @@ __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, co
    constexpr int UNR = (VEC > 1) ? 4 : 8;
    __shared__ Acc lds[SPLIT > 1 ? 256 * VEC : 1];
    const uint32_t slice = threadIdx.x / OPB, ol = threadIdx.x % OPB;
-   const uint32_t o = (blockIdx.x * OPB + ol) * VEC;
+   const uint32_t o = (xcd_neighbour_block(blockIdx.x, gridDim.x) * OPB + ol) * VEC;
    const bool active = o < p.nout;
    Acc acc[VEC];
 #pragma unroll
@@ -74,7 +86,7 @@ __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, co
          for (; i + (UNR - 1) * SPLIT < p.rsize0; i += UNR * SPLIT)
          {  Pack<T, VEC> v[UNR];
 #pragma unroll
-            for (int u = 0; u < UNR; u++) load_wide<T, VEC>(v[u], row + (int64_t)(i + u * SPLIT) * s0);
+            for (int u = 0; u < UNR; u++) load_wide<T, VEC, NT>(v[u], row + (int64_t)(i + u * SPLIT) * s0);
 #pragma unroll
             for (int u = 0; u < UNR; u++)
 #pragma unroll
@@ -109,43 +121,62 @@ __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, co
    }
 }
 
-/* GROUP threads cooperate on one output; GROUP is 64 (one wave) or 256 (the whole block) */
-template <class RD, class T, int GROUP>
+/* A group of threads cooperates on one output: GROUP 256 = the whole block, GROUP 64 = p.glanes (8 .. 64, a power
+   of two) lanes of a wave, chosen so that every lane has about four loads in flight on short rows. VEC > 1: the first reduced
+   dimension has unit stride and every row starts 16-byte aligned, so a thread takes VEC neighbouring elements with
+   one 128-bit load (NT: with the nontemporal hint, for sources that are read once from memory). */
+template <class RD, class T, int GROUP, int VEC = 1, bool NT = false>
 __global__ __launch_bounds__(256) void axis_group_kernel(const AxisParams p, const typename RD::Param prm)
 {
    typedef typename RD::Acc Acc;
    __shared__ Acc lds[4];
-   constexpr int PER_BLOCK = 256 / GROUP;
-   const uint32_t lane = threadIdx.x % GROUP;
-   const uint32_t o = blockIdx.x * PER_BLOCK + threadIdx.x / GROUP;
+   const uint32_t G = (GROUP == 256) ? 256u : p.glanes;
+   const uint32_t lane = threadIdx.x % G;
+   const uint32_t o = blockIdx.x * (256 / G) + threadIdx.x / G;
    const bool active = o < p.nout;
    Acc acc = RD::identity();
    int64_t o1 = 0, o2 = 0;
    if (active)
    {  axis_outer_offsets(p, o, o1, o2);
       const char *base = p.src + o1;
-      const int64_t s0 = p.rst[0];
+      const int64_t s0 = (VEC > 1) ? (int64_t)(sizeof(T) * VEC) : p.rst[0];        /* step of one group */
+      const uint32_t n0 = (VEC > 1) ? p.rgdiv.d : p.rsize0;                        /* groups per row */
       if (p.rd <= 1)
       {  uint32_t i = lane;
-         for (; i + 3 * GROUP < p.rsize0; i += 4 * GROUP)
-         {  T v0 = *reinterpret_cast<const T *>(base + (int64_t)i * s0);
-            T v1 = *reinterpret_cast<const T *>(base + (int64_t)(i + GROUP) * s0);
-            T v2 = *reinterpret_cast<const T *>(base + (int64_t)(i + 2 * GROUP) * s0);
-            T v3 = *reinterpret_cast<const T *>(base + (int64_t)(i + 3 * GROUP) * s0);
-            acc = RD::combine(acc, RD::load(v0, prm)); acc = RD::combine(acc, RD::load(v1, prm));
-            acc = RD::combine(acc, RD::load(v2, prm)); acc = RD::combine(acc, RD::load(v3, prm));
+         for (; i + 3 * G < n0; i += 4 * G)
+         {  Pack<T, VEC> v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+            {  if constexpr (VEC > 1) load_wide<T, VEC, NT>(v[u], base + (int64_t)(i + u * G) * s0);
+               else v[u].v[0] = *reinterpret_cast<const T *>(base + (int64_t)(i + u * G) * s0);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+               for (int k = 0; k < VEC; k++) acc = RD::combine(acc, RD::load(v[u].v[k], prm));
          }
-         for (; i < p.rsize0; i += GROUP) acc = RD::combine(acc, RD::load(*reinterpret_cast<const T *>(base + (int64_t)i * s0), prm));
+         for (; i < n0; i += G)
+         {  Pack<T, VEC> v;
+            if constexpr (VEC > 1) load_wide<T, VEC, NT>(v, base + (int64_t)i * s0);
+            else v.v[0] = *reinterpret_cast<const T *>(base + (int64_t)i * s0);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) acc = RD::combine(acc, RD::load(v.v[k], prm));
+         }
       }
       else
-      {  for (uint32_t j = lane; j < p.relem; j += GROUP)
-         {  uint32_t r = fastdiv(j, p.rdiv[0]); uint32_t i = j - r * p.rdiv[0].d;
-            acc = RD::combine(acc, RD::load(*reinterpret_cast<const T *>(base + axis_row_offset(p, r) + (int64_t)i * s0), prm));
+      {  const uint32_t total = (VEC > 1) ? p.relem / VEC : p.relem;
+         for (uint32_t j = lane; j < total; j += G)
+         {  uint32_t r = fastdiv(j, (VEC > 1) ? p.rgdiv : p.rdiv[0]); uint32_t i = j - r * n0;
+            Pack<T, VEC> v;
+            if constexpr (VEC > 1) load_wide<T, VEC, NT>(v, base + axis_row_offset(p, r) + (int64_t)i * s0);
+            else v.v[0] = *reinterpret_cast<const T *>(base + axis_row_offset(p, r) + (int64_t)i * s0);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) acc = RD::combine(acc, RD::load(v.v[k], prm));
          }
       }
    }
 #pragma unroll
-   for (int m = 32; m >= 1; m >>= 1) acc = RD::combine(acc, shfl_xor_any<Acc>(acc, m));
+   for (int m = 32; m >= 1; m >>= 1) if (GROUP == 256 || (uint32_t)m < G) acc = RD::combine(acc, shfl_xor_any<Acc>(acc, m));
    if constexpr (GROUP == 256)
    {  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = acc;
       __syncthreads();
@@ -195,6 +226,8 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
    int64_t outer_fast = (p.nd > 0) ? (p.st1[0] < 0 ? -p.st1[0] : p.st1[0]) : INT64_MAX;
    for (int d = 1; d < p.nd; d++) { int64_t a = p.st1[d] < 0 ? -p.st1[d] : p.st1[d]; if (a < outer_fast) outer_fast = a; }
    int64_t red_fast = (p.rd > 0) ? (p.rst[0] < 0 ? -p.rst[0] : p.rst[0]) : INT64_MAX;
+   /* a source larger than the caches is read once: nontemporal loads (see och_reduce_all.h) */
+   const bool streaming = nout * relem * (uint64_t)sizeof(T) >= OCH_EW_STREAM_BYTES;
    bool cooperative = (p.rd > 0) && ((red_fast < outer_fast) || (nout < 16384 && relem >= 256));
    if (!cooperative)
    {  /* VEC outputs per thread when the first outer dimension has unit source stride and
@@ -205,8 +238,12 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
       for (int d = 0; d < p.rd && wide; d++) if (p.rst[d] % 16 != 0) wide = false;
       const uint64_t groups = wide ? nout / VEC : nout;
       const bool split = groups < (1u << 20) && p.rsize0 >= 16;
-      if (wide && split)
+      if (wide && split && streaming)
+         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 4, VEC, true>), dim3((unsigned)((groups + 63) / 64)), dim3(256), 0, stream, p, prm);
+      else if (wide && split)
          hipLaunchKernelGGL((axis_thread_kernel<RD, T, 4, VEC>), dim3((unsigned)((groups + 63) / 64)), dim3(256), 0, stream, p, prm);
+      else if (wide && streaming)
+         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, VEC, true>), dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, stream, p, prm);
       else if (wide)
          hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, VEC>), dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, stream, p, prm);
       else if (split)
@@ -214,10 +251,32 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
       else
          hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, 1>), dim3((p.nout + 255) / 256), dim3(256), 0, stream, p, prm);
    }
-   else if (relem <= 2048 && nout >= 1024)
-      hipLaunchKernelGGL((axis_group_kernel<RD, T, 64>), dim3((p.nout + 3) / 4), dim3(256), 0, stream, p, prm);
    else
-      hipLaunchKernelGGL((axis_group_kernel<RD, T, 256>), dim3(p.nout), dim3(256), 0, stream, p, prm);
+   {  /* rows of the first reduced dimension are contiguous and 16-byte aligned: 128-bit loads */
+      constexpr int VEC = vec_for<T>();
+      bool wide = (VEC > 1) && p.rst[0] == (int64_t)sizeof(T) && (p.rsize0 % VEC == 0) && (((uintptr_t)p.src) % 16 == 0);
+      for (int d = 0; d < p.nd && wide; d++) if (p.st1[d] % 16 != 0) wide = false;
+      for (int d = 1; d < p.rd && wide; d++) if (p.rst[d] % 16 != 0) wide = false;
+      if (wide) p.rgdiv = make_fastdiv(p.rsize0 / VEC);
+      const bool wave = relem <= 2048 && nout >= 1024;              /* a wave per output, else a block per output */
+      const uint32_t loads = wide ? p.relem / VEC : p.relem;       /* loads per output: about four per lane */
+      p.glanes = 64;
+      while (p.glanes > 8 && (p.glanes / 2) * 4 >= loads) p.glanes /= 2;
+      const uint32_t per_block = 256 / p.glanes;
+      const dim3 grid(wave ? (p.nout + per_block - 1) / per_block : p.nout);
+      if (wide && streaming)
+      {  if (wave) hipLaunchKernelGGL((axis_group_kernel<RD, T, 64, VEC, true>), grid, dim3(256), 0, stream, p, prm);
+         else      hipLaunchKernelGGL((axis_group_kernel<RD, T, 256, VEC, true>), grid, dim3(256), 0, stream, p, prm);
+      }
+      else if (wide)
+      {  if (wave) hipLaunchKernelGGL((axis_group_kernel<RD, T, 64, VEC>), grid, dim3(256), 0, stream, p, prm);
+         else      hipLaunchKernelGGL((axis_group_kernel<RD, T, 256, VEC>), grid, dim3(256), 0, stream, p, prm);
+      }
+      else
+      {  if (wave) hipLaunchKernelGGL((axis_group_kernel<RD, T, 64>), grid, dim3(256), 0, stream, p, prm);
+         else      hipLaunchKernelGGL((axis_group_kernel<RD, T, 256>), grid, dim3(256), 0, stream, p, prm);
+      }
+   }
    OCH_CHECK_LAUNCH();
    return 0;
 }

@@ -3,20 +3,21 @@
  * (all_lt ...) exist as full reductions only. */
 #include "och_reduce_axis.h"
 namespace och {
-axis_fn axis_lookup_a(int op, int dtype);
-axis_fn axis_lookup_b(int op, int dtype);
-axis_fn axis_lookup_c(int op, int dtype);
-axis_fn axis_lookup_d(int op, int dtype);
+/* the instantiations are spread over eight translation units (build time); each knows its own operations */
+#define OCH_AXIS_PARTS(X) X(a) X(b) X(c) X(d) X(e) X(f) X(g) X(h)
+#define OCH_X(part) axis_fn axis_lookup_##part(int op, int dtype);
+OCH_AXIS_PARTS(OCH_X)
+#undef OCH_X
 }
 extern "C" int och_reduce_axis(int op, int dtype, const och_reduce_axis_config *config, double p)
 {
    using namespace och;
    axis_fn fn = nullptr;
    if (dtype >= 0 && dtype < DT_COUNT)
-   {  if (op >= OCH_R_ANY && op <= OCH_R_NNZ_NAN) fn = axis_lookup_a(op, dtype);
-      else if (op >= OCH_R_SUM && op <= OCH_R_PROD_NAN) fn = axis_lookup_b(op, dtype);
-      else if (op >= OCH_R_SUM_ABS && op <= OCH_R_MINIMUM_ABS) fn = axis_lookup_c(op, dtype);
-      else if (op >= OCH_R_NORM && op <= OCH_R_NORM2_NAN) fn = axis_lookup_d(op, dtype);
+   {
+#define OCH_X(part) if (fn == nullptr) fn = axis_lookup_##part(op, dtype);
+      OCH_AXIS_PARTS(OCH_X)
+#undef OCH_X
    }
    if (fn == nullptr) return set_error("axis reduction %d is not available for data type %d", op, dtype);
    return fn(config, p);

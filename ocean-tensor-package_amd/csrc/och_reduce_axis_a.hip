@@ -1,4 +1,4 @@
-/* Axis-reduction kernels, operations: 0 1 2 3 4 5 6 */
+/* Axis-reduction kernels, operations: 0 1 2 */
 #include "och_reduce_axis.h"
 namespace och {
 axis_fn axis_lookup_a(int op, int dtype)
@@ -8,10 +8,6 @@ axis_fn axis_lookup_a(int op, int dtype)
       case 0: return RowA<0>::fn[dtype];
       case 1: return RowA<1>::fn[dtype];
       case 2: return RowA<2>::fn[dtype];
-      case 3: return RowA<3>::fn[dtype];
-      case 4: return RowA<4>::fn[dtype];
-      case 5: return RowA<5>::fn[dtype];
-      case 6: return RowA<6>::fn[dtype];
    }
    return nullptr;
 }

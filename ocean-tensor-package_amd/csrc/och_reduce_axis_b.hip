@@ -1,14 +1,14 @@
-/* Axis-reduction kernels, operations: 15 16 17 18 */
+/* Axis-reduction kernels, operations: 3 4 5 6 */
 #include "och_reduce_axis.h"
 namespace och {
 axis_fn axis_lookup_b(int op, int dtype)
 {
    switch (op)
    {
-      case 15: return RowA<15>::fn[dtype];
-      case 16: return RowA<16>::fn[dtype];
-      case 17: return RowA<17>::fn[dtype];
-      case 18: return RowA<18>::fn[dtype];
+      case 3: return RowA<3>::fn[dtype];
+      case 4: return RowA<4>::fn[dtype];
+      case 5: return RowA<5>::fn[dtype];
+      case 6: return RowA<6>::fn[dtype];
    }
    return nullptr;
 }

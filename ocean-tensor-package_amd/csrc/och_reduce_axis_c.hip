@@ -1,16 +1,12 @@
-/* Axis-reduction kernels, operations: 19 20 21 22 23 24 */
+/* Axis-reduction kernels, operations: 15 16 */
 #include "och_reduce_axis.h"
 namespace och {
 axis_fn axis_lookup_c(int op, int dtype)
 {
    switch (op)
    {
-      case 19: return RowA<19>::fn[dtype];
-      case 20: return RowA<20>::fn[dtype];
-      case 21: return RowA<21>::fn[dtype];
-      case 22: return RowA<22>::fn[dtype];
-      case 23: return RowA<23>::fn[dtype];
-      case 24: return RowA<24>::fn[dtype];
+      case 15: return RowA<15>::fn[dtype];
+      case 16: return RowA<16>::fn[dtype];
    }
    return nullptr;
 }
