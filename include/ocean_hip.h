@@ -286,6 +286,19 @@ int och_gemm(int dtype, char transA, char transB, size_t M, size_t N, size_t K,
              const void *beta, void *C, ptrdiff_t ldC,
              int scalar_mode_host, och_stream stream);
 int och_gemm_supported(int dtype);
+/* The loop over the dimensions beyond the second (tensor_blas_gpu.c:171-252) as one launch: product z of the   */
+/* batch is split into indices over batch_size (first dimension fastest) and every operand -- alpha and beta    */
+/* included, tensor_blas_gpu.c:236-241 -- moves by its own byte stride per index (0: shared by the products;    */
+/* stride_alpha / stride_beta may be NULL for all-zero). nbatch <= 6. The products of a batch must not overlap  */
+/* in C. Host scalars that differ between products fall back to one launch per product.                         */
+int och_gemm_batched(int dtype, char transA, char transB, size_t M, size_t N, size_t K,
+                     const void *alpha, const void *A, ptrdiff_t ldA,
+                     const void *B, ptrdiff_t ldB,
+                     const void *beta, void *C, ptrdiff_t ldC,
+                     int nbatch, const size_t *batch_size,
+                     const ptrdiff_t *stride_alpha, const ptrdiff_t *strideA, const ptrdiff_t *strideB,
+                     const ptrdiff_t *stride_beta, const ptrdiff_t *strideC,
+                     int scalar_mode_host, och_stream stream);
 
 /* ======================================================================== */
 /* Index operations (template_index.cu:37-57, index1.h:182, index2.h:188)   */

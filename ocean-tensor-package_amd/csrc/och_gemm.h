@@ -42,6 +42,28 @@ template <> struct Mfma<float>
    static __device__ __forceinline__ int acc_row(int lane, int r) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
 };
 
+/* Batch of products in one launch (grid z): entry z is split into indices over `size`, and every operand --
+   the scalars included when they live in device memory -- moves by its own byte stride per index (0: shared). */
+#define OCH_GEMM_BATCH_DIMS 6
+struct GemmBatch
+{
+   int      nb;                                   /* 0: a single product */
+   uint32_t z0;                                   /* batch entry of grid z = 0 */
+   uint32_t size[OCH_GEMM_BATCH_DIMS];
+   int64_t  sA[OCH_GEMM_BATCH_DIMS], sB[OCH_GEMM_BATCH_DIMS], sC[OCH_GEMM_BATCH_DIMS];
+   int64_t  sAlpha[OCH_GEMM_BATCH_DIMS], sBeta[OCH_GEMM_BATCH_DIMS];
+};
+__device__ __forceinline__ void gemm_batch_offsets(const GemmBatch &b, int64_t &oA, int64_t &oB, int64_t &oC, int64_t &oAlpha, int64_t &oBeta)
+{  oA = oB = oC = oAlpha = oBeta = 0;
+   if (b.nb == 0) return;
+   uint32_t z = b.z0 + blockIdx.z;
+   for (int d = 0; d < b.nb; d++)
+   {  const uint32_t q = z / b.size[d], i = z - q * b.size[d]; z = q;
+      oA += (int64_t)i * b.sA[d]; oB += (int64_t)i * b.sB[d]; oC += (int64_t)i * b.sC[d];
+      oAlpha += (int64_t)i * b.sAlpha[d]; oBeta += (int64_t)i * b.sBeta[d];
+   }
+}
+
 template <class R> struct GemmParams
 {
    const char *A, *B; char *C;
@@ -52,6 +74,7 @@ template <class R> struct GemmParams
    int      conjA, conjB;
    int      alignedA, alignedB;        /* base pointer and leading dimension allow 128-bit loads */
    uint32_t tiles_m, tiles_n;
+   GemmBatch batch;
 };
 
 #define OCH_GEMM_THREADS 256
@@ -131,6 +154,9 @@ __global__ __launch_bounds__(OCH_GEMM_THREADS, 2) void gemm_mfma_kernel(const Ge
    constexpr int BUF = NPL * KT * (PA + PB);
    __shared__ __align__(16) R lds[2 * BUF];
 
+   int64_t oA, oB, oC, oAlpha, oBeta;
+   gemm_batch_offsets(p.batch, oA, oB, oC, oAlpha, oBeta);
+   const char *pA = p.A + oA, *pB = p.B + oB; char *pC = p.C + oC;
    const uint32_t tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -150,8 +176,8 @@ __global__ __launch_bounds__(OCH_GEMM_THREADS, 2) void gemm_mfma_kernel(const Ge
    SlabLoader<R, CPLX, BKC, EDGE, BN, KT> lb;
    const uint32_t nslabs = (p.K + KT - 1) / KT;
    if (nslabs > 0)
-   {  la.fetch(p.A, p.ldA, m0, 0, p.M, p.K, p.alignedA);
-      lb.fetch(p.B, p.ldB, n0, 0, p.N, p.K, p.alignedB);
+   {  la.fetch(pA, p.ldA, m0, 0, p.M, p.K, p.alignedA);
+      lb.fetch(pB, p.ldB, n0, 0, p.N, p.K, p.alignedB);
       la.stash(lds, PA, p.conjA);
       lb.stash(lds + NPL * KT * PA, PB, p.conjB);
    }
@@ -160,8 +186,8 @@ __global__ __launch_bounds__(OCH_GEMM_THREADS, 2) void gemm_mfma_kernel(const Ge
    {  const R *As = lds + (s & 1) * BUF, *Bs = As + NPL * KT * PA;
       const bool more = s + 1 < nslabs;
       if (more)
-      {  la.fetch(p.A, p.ldA, m0, (s + 1) * KT, p.M, p.K, p.alignedA);
-         lb.fetch(p.B, p.ldB, n0, (s + 1) * KT, p.N, p.K, p.alignedB);
+      {  la.fetch(pA, p.ldA, m0, (s + 1) * KT, p.M, p.K, p.alignedA);
+         lb.fetch(pB, p.ldB, n0, (s + 1) * KT, p.N, p.K, p.alignedB);
       }
 #pragma unroll
       for (int ks = 0; ks < KT / TK; ks++)
@@ -199,8 +225,8 @@ __global__ __launch_bounds__(OCH_GEMM_THREADS, 2) void gemm_mfma_kernel(const Ge
 
    /* epilogue */
    R alr = p.alpha[0], ali = p.alpha[1], ber = p.beta[0], bei = p.beta[1];
-   if (p.alpha_dev) { alr = p.alpha_dev[0]; if (CPLX) ali = p.alpha_dev[1]; }
-   if (p.beta_dev)  { ber = p.beta_dev[0];  if (CPLX) bei = p.beta_dev[1]; }
+   if (p.alpha_dev) { const R *q = reinterpret_cast<const R *>(reinterpret_cast<const char *>(p.alpha_dev) + oAlpha); alr = q[0]; if (CPLX) ali = q[1]; }
+   if (p.beta_dev)  { const R *q = reinterpret_cast<const R *>(reinterpret_cast<const char *>(p.beta_dev) + oBeta);   ber = q[0]; if (CPLX) bei = q[1]; }
    const bool use_c = CPLX ? (ber != 0 || bei != 0) : (ber != 0);
 #pragma unroll
    for (int i = 0; i < TMS; i++)
@@ -211,7 +237,7 @@ __global__ __launch_bounds__(OCH_GEMM_THREADS, 2) void gemm_mfma_kernel(const Ge
          for (int r = 0; r < MM::NACC; r++)
          {  const uint32_t row = m0 + wm + i * T + MM::acc_row(lane, r);
             if (EDGE && (row >= p.M || col >= p.N)) continue;
-            R *c = reinterpret_cast<R *>(p.C + ((int64_t)row + (int64_t)col * p.ldC) * (int64_t)(sizeof(R) * NPL));
+            R *c = reinterpret_cast<R *>(pC + ((int64_t)row + (int64_t)col * p.ldC) * (int64_t)(sizeof(R) * NPL));
             if (!CPLX)
             {  R v = alr * acc[i][j][r];
                if (use_c) v += ber * c[0];
@@ -234,9 +260,11 @@ __global__ __launch_bounds__(256) void gemm_dot_kernel(const GemmParams<R> p, in
 {
    constexpr int NPL = CPLX ? 2 : 1;
    __shared__ double lds[8];
+   int64_t oA, oB, oC, oAlpha, oBeta;
+   gemm_batch_offsets(p.batch, oA, oB, oC, oAlpha, oBeta);
    const uint32_t row = blockIdx.x % p.M, col = blockIdx.x / p.M;
-   const R *a = reinterpret_cast<const R *>(p.A) + (int64_t)row * sAm * NPL;
-   const R *b = reinterpret_cast<const R *>(p.B) + (int64_t)col * sBn * NPL;
+   const R *a = reinterpret_cast<const R *>(p.A + oA) + (int64_t)row * sAm * NPL;
+   const R *b = reinterpret_cast<const R *>(p.B + oB) + (int64_t)col * sBn * NPL;
    double sr = 0, si = 0;
    for (uint32_t k = threadIdx.x; k < p.K; k += 256)
    {  const R *x = a + (int64_t)k * sAk * NPL, *y = b + (int64_t)k * sBk * NPL;
@@ -255,9 +283,9 @@ __global__ __launch_bounds__(256) void gemm_dot_kernel(const GemmParams<R> p, in
    sr = ((lds[0] + lds[2]) + lds[4]) + lds[6];
    si = ((lds[1] + lds[3]) + lds[5]) + lds[7];
    R alr = p.alpha[0], ali = p.alpha[1], ber = p.beta[0], bei = p.beta[1];
-   if (p.alpha_dev) { alr = p.alpha_dev[0]; if (CPLX) ali = p.alpha_dev[1]; }
-   if (p.beta_dev)  { ber = p.beta_dev[0];  if (CPLX) bei = p.beta_dev[1]; }
-   R *c = reinterpret_cast<R *>(p.C) + ((int64_t)row + (int64_t)col * p.ldC) * NPL;
+   if (p.alpha_dev) { const R *q = reinterpret_cast<const R *>(reinterpret_cast<const char *>(p.alpha_dev) + oAlpha); alr = q[0]; if (CPLX) ali = q[1]; }
+   if (p.beta_dev)  { const R *q = reinterpret_cast<const R *>(reinterpret_cast<const char *>(p.beta_dev) + oBeta);   ber = q[0]; if (CPLX) bei = q[1]; }
+   R *c = reinterpret_cast<R *>(p.C + oC) + ((int64_t)row + (int64_t)col * p.ldC) * NPL;
    if (!CPLX)
    {  double v = (double)alr * sr;
       if (ber != 0) v += (double)ber * (double)c[0];
@@ -283,6 +311,8 @@ struct GemmArgs
    ptrdiff_t ldA, ldB, ldC;
    int scalar_mode_host;
    hipStream_t stream;
+   GemmBatch batch;                 /* nb = 0: one product */
+   unsigned  nz;                    /* grid z: batch entries of this launch (1 when nb = 0) */
 };
 
 template <class R, bool CPLX, int WM, int WN, int KT>
@@ -300,23 +330,28 @@ static int launch_gemm_mfma(const GemmArgs &g)
    {  memcpy(p.alpha, g.alpha, ES); memcpy(p.beta, g.beta, ES); }
    else
    {  p.alpha_dev = (const R *)g.alpha; p.beta_dev = (const R *)g.beta; }
+   p.batch = g.batch;
    const bool akc = (g.transA != 'N'), bkc = (g.transB == 'N');
    p.conjA = CPLX && (g.transA == 'C'); p.conjB = CPLX && (g.transB == 'C');
 
    if (g.M * g.N <= 256 && g.K >= 64)
    {  /* op(A)(m,k) = A[m*sAm + k*sAk], op(B)(k,n) = B[k*sBk + n*sBn] */
       const int64_t sAm = akc ? g.ldA : 1, sAk = akc ? 1 : g.ldA, sBk = bkc ? 1 : g.ldB, sBn = bkc ? g.ldB : 1;
-      hipLaunchKernelGGL((gemm_dot_kernel<R, CPLX>), dim3((unsigned)(g.M * g.N)), dim3(256), 0, g.stream, p, sAm, sAk, sBk, sBn);
+      hipLaunchKernelGGL((gemm_dot_kernel<R, CPLX>), dim3((unsigned)(g.M * g.N), 1, g.nz), dim3(256), 0, g.stream, p, sAm, sAk, sBk, sBn);
       OCH_CHECK_LAUNCH();
       return 0;
    }
    p.tiles_m = (uint32_t)((g.M + BM - 1) / BM); p.tiles_n = (uint32_t)((g.N + BN - 1) / BN);
    const uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
    if (blocks > 0x7FFFFFFFull) return set_error("gemm: too many tiles");
-   auto aligned = [&](const void *ptr, ptrdiff_t ld) { return ((uintptr_t)ptr % 16 == 0) && (((int64_t)ld * ES) % 16 == 0); };
-   p.alignedA = aligned(g.A, g.ldA) ? 1 : 0; p.alignedB = aligned(g.B, g.ldB) ? 1 : 0;
-   const bool edge = !(g.M % BM == 0 && g.N % BN == 0 && g.K % KT == 0 && aligned(g.A, g.ldA) && aligned(g.B, g.ldB));
-   const dim3 grid((unsigned)blocks), block(OCH_GEMM_THREADS);
+   auto aligned = [&](const void *ptr, ptrdiff_t ld, const int64_t *bs)
+   {  bool ok = ((uintptr_t)ptr % 16 == 0) && (((int64_t)ld * ES) % 16 == 0);
+      for (int d = 0; d < g.batch.nb; d++) ok = ok && (bs[d] % 16 == 0);                 /* every batch entry */
+      return ok;
+   };
+   p.alignedA = aligned(g.A, g.ldA, g.batch.sA) ? 1 : 0; p.alignedB = aligned(g.B, g.ldB, g.batch.sB) ? 1 : 0;
+   const bool edge = !(g.M % BM == 0 && g.N % BN == 0 && g.K % KT == 0 && p.alignedA && p.alignedB);
+   const dim3 grid((unsigned)blocks, 1, g.nz), block(OCH_GEMM_THREADS);
 #define OCH_GEMM_LAUNCH(AK, BK)                                                                             \
    do { if (edge) hipLaunchKernelGGL((gemm_mfma_kernel<R, CPLX, AK, BK, true, WM, WN, KT>), grid, block, 0, g.stream, p);  \
         else      hipLaunchKernelGGL((gemm_mfma_kernel<R, CPLX, AK, BK, false, WM, WN, KT>), grid, block, 0, g.stream, p); } while (0)

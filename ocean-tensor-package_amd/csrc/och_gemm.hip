@@ -44,9 +44,17 @@ template <> struct GemmElem<half_t>
 template <class T>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(uint32_t M, uint32_t N, uint32_t K,
       T alpha_host, T beta_host, const T *alpha_dev, const T *beta_dev,
-      const T *A, int64_t sAm, int64_t sAk, const T *B, int64_t sBk, int64_t sBn, T *C, int64_t ldC)
+      const T *A, int64_t sAm, int64_t sAk, const T *B, int64_t sBk, int64_t sBn, T *C, int64_t ldC, const GemmBatch batch)
 {
    typedef GemmElem<T> E; typedef typename E::W W;
+   {  int64_t oA, oB, oC, oAlpha, oBeta;
+      gemm_batch_offsets(batch, oA, oB, oC, oAlpha, oBeta);
+      A = reinterpret_cast<const T *>(reinterpret_cast<const char *>(A) + oA);
+      B = reinterpret_cast<const T *>(reinterpret_cast<const char *>(B) + oB);
+      C = reinterpret_cast<T *>(reinterpret_cast<char *>(C) + oC);
+      if (alpha_dev) alpha_dev = reinterpret_cast<const T *>(reinterpret_cast<const char *>(alpha_dev) + oAlpha);
+      if (beta_dev)  beta_dev  = reinterpret_cast<const T *>(reinterpret_cast<const char *>(beta_dev) + oBeta);
+   }
    __shared__ W As[GK][GT + 1], Bs[GK][GT + 1];
    const uint32_t tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
    const uint32_t m0 = blockIdx.x * GT, n0 = blockIdx.y * GT;
@@ -101,9 +109,9 @@ template <class T> static int gemm_generic(const GemmArgs &g)
    const int64_t sAm = ta ? g.ldA : 1, sAk = ta ? 1 : g.ldA, sBk = tb ? g.ldB : 1, sBn = tb ? 1 : g.ldB;
    const uint64_t gx = (g.M + GT - 1) / GT, gy = (g.N + GT - 1) / GT;
    if (gy > 65535) return set_error("gemm: N = %zu is too large for this data type", g.N);
-   hipLaunchKernelGGL((gemm_generic_kernel<T>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, g.stream,
+   hipLaunchKernelGGL((gemm_generic_kernel<T>), dim3((unsigned)gx, (unsigned)gy, g.nz), dim3(256), 0, g.stream,
                       (uint32_t)g.M, (uint32_t)g.N, (uint32_t)g.K, alpha, beta, adev, bdev,
-                      (const T *)g.A, sAm, sAk, (const T *)g.B, sBk, sBn, (T *)g.C, (int64_t)g.ldC);
+                      (const T *)g.A, sAm, sAk, (const T *)g.B, sBk, sBn, (T *)g.C, (int64_t)g.ldC, g.batch);
    OCH_CHECK_LAUNCH();
    return 0;
 }
@@ -122,25 +130,8 @@ using namespace och;
 extern "C" int och_gemm_supported(int dtype)
 {  return (dtype >= 0 && dtype < DT_COUNT && dtype != OCH_CHALF) ? 1 : 0; }
 
-extern "C" int och_gemm(int dtype, char transA, char transB, size_t M, size_t N, size_t K,
-                        const void *alpha, const void *A, ptrdiff_t ldA, const void *B, ptrdiff_t ldB,
-                        const void *beta, void *C, ptrdiff_t ldC, int scalar_mode_host, och_stream stream)
+static int gemm_dispatch(int dtype, const GemmArgs &g)
 {
-   if (!och_gemm_supported(dtype)) return set_error("gemm is not available for data type %d", dtype);
-   GemmArgs g;
-   g.transA = norm_trans(transA); g.transB = norm_trans(transB);
-   if (!g.transA || !g.transB) return set_error("gemm: invalid transposition mode ('%c', '%c')", transA, transB);
-   if (M == 0 || N == 0) return 0;                       /* empty result: tensor_blas_gpu.c:96 */
-   if (M > 0xFFFFFF00ull || N > 0xFFFFFF00ull || K > 0xFFFFFF00ull) return set_error("gemm: dimensions beyond 2^32 are not supported");
-   const size_t rowsA = (g.transA == 'N') ? M : K, rowsB = (g.transB == 'N') ? K : N;
-   if (K > 0 && (ldA < (ptrdiff_t)(rowsA ? rowsA : 1) || ldB < (ptrdiff_t)(rowsB ? rowsB : 1)))
-      return set_error("gemm: leading dimension smaller than the number of rows (ldA = %td, ldB = %td)", ldA, ldB);
-   if (ldC < (ptrdiff_t)M) return set_error("gemm: ldC = %td is smaller than M = %zu", ldC, M);
-   if (!alpha || !beta || !C || (K > 0 && (!A || !B))) return set_error("gemm: null pointer argument");
-   g.M = M; g.N = N; g.K = K; g.alpha = alpha; g.beta = beta; g.A = A; g.B = B; g.C = C;
-   g.ldA = ldA; g.ldB = ldB; g.ldC = ldC; g.scalar_mode_host = scalar_mode_host; g.stream = as_stream(stream);
-   if (dtype < OCH_CHALF && g.transA == 'C') g.transA = 'T';   /* conjugating a real matrix is the identity */
-   if (dtype < OCH_CHALF && g.transB == 'C') g.transB = 'T';
    switch (dtype)
    {  case OCH_BOOL:    return gemm_generic<obool>(g);
       case OCH_UINT8:   return gemm_generic<uint8_t>(g);
@@ -158,4 +149,88 @@ extern "C" int och_gemm(int dtype, char transA, char transB, size_t M, size_t N,
       case OCH_CDOUBLE: return gemm_cdouble(g);
    }
    return set_error("gemm is not available for data type %d", dtype);
+}
+
+/* argument checks shared by the single and the batched entry; returns 1 when there is nothing to do */
+static int gemm_prepare(GemmArgs &g, int dtype, char transA, char transB, size_t M, size_t N, size_t K,
+                        const void *alpha, const void *A, ptrdiff_t ldA, const void *B, ptrdiff_t ldB,
+                        const void *beta, void *C, ptrdiff_t ldC, int scalar_mode_host, och_stream stream)
+{
+   if (!och_gemm_supported(dtype)) return set_error("gemm is not available for data type %d", dtype);
+   g.transA = norm_trans(transA); g.transB = norm_trans(transB);
+   if (!g.transA || !g.transB) return set_error("gemm: invalid transposition mode ('%c', '%c')", transA, transB);
+   if (M == 0 || N == 0) return 1;                       /* empty result: tensor_blas_gpu.c:96 */
+   if (M > 0xFFFFFF00ull || N > 0xFFFFFF00ull || K > 0xFFFFFF00ull) return set_error("gemm: dimensions beyond 2^32 are not supported");
+   const size_t rowsA = (g.transA == 'N') ? M : K, rowsB = (g.transB == 'N') ? K : N;
+   if (K > 0 && (ldA < (ptrdiff_t)(rowsA ? rowsA : 1) || ldB < (ptrdiff_t)(rowsB ? rowsB : 1)))
+      return set_error("gemm: leading dimension smaller than the number of rows (ldA = %td, ldB = %td)", ldA, ldB);
+   if (ldC < (ptrdiff_t)M) return set_error("gemm: ldC = %td is smaller than M = %zu", ldC, M);
+   if (!alpha || !beta || !C || (K > 0 && (!A || !B))) return set_error("gemm: null pointer argument");
+   g.M = M; g.N = N; g.K = K; g.alpha = alpha; g.beta = beta; g.A = A; g.B = B; g.C = C;
+   g.ldA = ldA; g.ldB = ldB; g.ldC = ldC; g.scalar_mode_host = scalar_mode_host; g.stream = as_stream(stream);
+   if (dtype < OCH_CHALF && g.transA == 'C') g.transA = 'T';   /* conjugating a real matrix is the identity */
+   if (dtype < OCH_CHALF && g.transB == 'C') g.transB = 'T';
+   memset(&g.batch, 0, sizeof(g.batch)); g.nz = 1;
+   return 0;
+}
+
+extern "C" int och_gemm(int dtype, char transA, char transB, size_t M, size_t N, size_t K,
+                        const void *alpha, const void *A, ptrdiff_t ldA, const void *B, ptrdiff_t ldB,
+                        const void *beta, void *C, ptrdiff_t ldC, int scalar_mode_host, och_stream stream)
+{
+   GemmArgs g;
+   const int status = gemm_prepare(g, dtype, transA, transB, M, N, K, alpha, A, ldA, B, ldB, beta, C, ldC, scalar_mode_host, stream);
+   if (status != 0) return status < 0 ? -1 : 0;
+   return gemm_dispatch(dtype, g);
+}
+
+extern "C" int och_gemm_batched(int dtype, char transA, char transB, size_t M, size_t N, size_t K,
+                                const void *alpha, const void *A, ptrdiff_t ldA, const void *B, ptrdiff_t ldB,
+                                const void *beta, void *C, ptrdiff_t ldC,
+                                int nbatch, const size_t *batch_size,
+                                const ptrdiff_t *stride_alpha, const ptrdiff_t *strideA, const ptrdiff_t *strideB,
+                                const ptrdiff_t *stride_beta, const ptrdiff_t *strideC,
+                                int scalar_mode_host, och_stream stream)
+{
+   GemmArgs g;
+   if (nbatch < 0 || nbatch > OCH_GEMM_BATCH_DIMS) return set_error("gemm: invalid number of batch dimensions (%d)", nbatch);
+   if (nbatch > 0 && (!batch_size || !strideA || !strideB || !strideC)) return set_error("gemm: null batch argument");
+   const int status = gemm_prepare(g, dtype, transA, transB, M, N, K, alpha, A, ldA, B, ldB, beta, C, ldC, scalar_mode_host, stream);
+   if (status != 0) return status < 0 ? -1 : 0;
+   uint64_t total = 1; bool scalars_move = false;
+   GemmBatch &b = g.batch;
+   for (int d = 0; d < nbatch; d++)
+   {  if (batch_size[d] == 0) return 0;
+      if (batch_size[d] == 1) continue;
+      if (batch_size[d] > 0xFFFFFFFFull || total * batch_size[d] > 0xFFFFFFFFull) return set_error("gemm: too many products in one batch");
+      total *= batch_size[d];
+      b.size[b.nb] = (uint32_t)batch_size[d];
+      b.sA[b.nb] = strideA[d]; b.sB[b.nb] = strideB[d]; b.sC[b.nb] = strideC[d];
+      b.sAlpha[b.nb] = stride_alpha ? stride_alpha[d] : 0; b.sBeta[b.nb] = stride_beta ? stride_beta[d] : 0;
+      if (b.sAlpha[b.nb] != 0 || b.sBeta[b.nb] != 0) scalars_move = true;
+      b.nb++;
+   }
+   if (b.nb == 0) return gemm_dispatch(dtype, g);
+   if (scalar_mode_host && scalars_move)
+   {  /* host scalars that differ between the products are passed by value: one launch per product */
+      const GemmBatch all = b;
+      memset(&b, 0, sizeof(b));
+      for (uint64_t z = 0; z < total; z++)
+      {  uint64_t q = z; int64_t oA = 0, oB = 0, oC = 0, oAl = 0, oBe = 0;
+         for (int d = 0; d < all.nb; d++)
+         {  const uint64_t i = q % all.size[d]; q /= all.size[d];
+            oA += (int64_t)i * all.sA[d]; oB += (int64_t)i * all.sB[d]; oC += (int64_t)i * all.sC[d];
+            oAl += (int64_t)i * all.sAlpha[d]; oBe += (int64_t)i * all.sBeta[d];
+         }
+         g.A = (const char *)A + oA; g.B = (const char *)B + oB; g.C = (char *)C + oC;
+         g.alpha = (const char *)alpha + oAl; g.beta = (const char *)beta + oBe;
+         if (gemm_dispatch(dtype, g) != 0) return -1;
+      }
+      return 0;
+   }
+   for (uint64_t z0 = 0; z0 < total; z0 += 65535)          /* grid z is limited to 65535 */
+   {  b.z0 = (uint32_t)z0; g.nz = (unsigned)((total - z0 < 65535) ? total - z0 : 65535);
+      if (gemm_dispatch(dtype, g) != 0) return -1;
+   }
+   return 0;
 }

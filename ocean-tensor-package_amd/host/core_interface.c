@@ -263,7 +263,7 @@ static OcTensor *scalar_tensor(OcScalar *s, OcDType dtype, double fallback)
 /* leading dimension of a matrix operand, flipping the mode when only its rows are contiguous */
 static int gemm_operand(OcTensor **t, char *mode, OcIndex *ld, int complex_type)
 {  OcTensor *x = *t; int es = x->elemsize;
-   if (x->ndims != 2) return OcErrorMessage("This front end multiplies two-dimensional tensors");
+   if (x->ndims < 2) return OcErrorMessage("Matrix multiplication needs tensors of at least two dimensions");
    if ((x->size[0] == 1 || x->strides[0] == es) && (x->size[1] == 1 || (x->strides[1] >= x->size[0] * es && x->strides[1] % es == 0)))
    {  *ld = (x->size[1] == 1) ? (x->size[0] > 0 ? x->size[0] : 1) : x->strides[1] / es; return 0; }
    if ((x->size[1] == 1 || x->strides[1] == es) && (x->size[0] == 1 || (x->strides[0] >= x->size[1] * es && x->strides[0] % es == 0)) && !(complex_type && *mode == 'C'))
@@ -275,36 +275,54 @@ static int gemm_operand(OcTensor **t, char *mode, OcIndex *ld, int complex_type)
       OcDecrefTensor(x); *t = v;
       return 0;
    }
-   {  OcTensor *r = OcTensor_create(2, x->size, NULL, x->dtype, x->device);
+   {  OcTensor *r = OcTensor_create(x->ndims, x->size, NULL, x->dtype, x->device);
       if (r == NULL) return -1;
       if (OcTensor_copy(x, r) != 0) { OcDecrefTensor(r); return -1; }
       OcDecrefTensor(x); *t = r; *ld = r->size[0] > 0 ? r->size[0] : 1;
       return 0;
    }
 }
+/* C <- alpha * op(A) * op(B) + beta * C on the first two dimensions; the dimensions beyond them index independent
+   products and broadcast between A and B (size 1 or absent: shared), as in Ocean's interface (tensor_itf.c:6433-6750) */
 int OcTensor_gemm(OcScalar *alpha, OcTensor *A, char modeA, OcTensor *B, char modeB, OcScalar *beta, OcTensor **C)
-{  OcTensor *a = OcIncrefTensor(A), *b = OcIncrefTensor(B), *c = NULL, *ta = NULL, *tb = NULL; int result = -1;
+{  OcTensor *a = OcIncrefTensor(A), *b = OcIncrefTensor(B), *c = NULL, *ta = NULL, *tb = NULL, *v; int result = -1, i, nd;
    OcDevice *device = A->device != OcCPU ? A->device : B->device; OcDType dtype = OcDType_getCommonType(A->dtype, B->dtype);
-   OcSize M, N, K, K2, csize[2]; OcIndex ldA, ldB, ldC; OcModuleCore *m = OcModuleCore_forDevice(device);
+   OcSize M, N, K, K2, csize[OC_TENSOR_MAX_DIMS], asize[OC_TENSOR_MAX_DIMS], bsize[OC_TENSOR_MAX_DIMS]; OcIndex ldA, ldB, ldC; OcModuleCore *m = OcModuleCore_forDevice(device);
    if (*C) dtype = OcDType_getCommonType(dtype, (*C)->dtype);
    if (m == NULL) { OcErrorMessage("No core module is registered for device %s", device->name); goto final; }
    if (!m->Tensor_gemmSupportedOn(device, dtype)) { OcErrorMessage("Matrix multiplication is not supported for type %s on %s", OcDType_name(dtype), device->name); goto final; }
-   if (A->ndims != 2 || B->ndims != 2) { OcErrorMessage("This front end multiplies two-dimensional tensors"); goto final; }
+   if (A->ndims < 2 || B->ndims < 2) { OcErrorMessage("Matrix multiplication needs tensors of at least two dimensions"); goto final; }
    M = (modeA == 'N') ? A->size[0] : A->size[1]; K = (modeA == 'N') ? A->size[1] : A->size[0];
    K2 = (modeB == 'N') ? B->size[0] : B->size[1]; N = (modeB == 'N') ? B->size[1] : B->size[0];
    if (K != K2) { OcErrorMessage("Inner dimensions do not match (%td and %td)", K, K2); goto final; }
+   nd = A->ndims > B->ndims ? A->ndims : B->ndims;
+   csize[0] = M; csize[1] = N;
+   for (i = 2; i < nd; i++)
+   {  OcSize sa = i < A->ndims ? A->size[i] : 1, sb = i < B->ndims ? B->size[i] : 1;
+      if (sa != sb && sa != 1 && sb != 1) { OcErrorMessage("Dimension %d of the operands is not compatible (%td and %td)", i, sa, sb); goto final; }
+      csize[i] = (sa == 1) ? sb : sa;
+   }
    if (OcTensor_ensure(&a, dtype, device) != 0 || OcTensor_ensure(&b, dtype, device) != 0) goto final;
    if (gemm_operand(&a, &modeA, &ldA, OcDType_isComplex(dtype)) != 0 || gemm_operand(&b, &modeB, &ldB, OcDType_isComplex(dtype)) != 0) goto final;
-   csize[0] = M; csize[1] = N;
-   if (*C == NULL) { if ((c = OcTensor_create(2, csize, NULL, dtype, device)) == NULL) goto final; }
+   /* all operands get the same number of dimensions; shared ones have stride zero */
+   asize[0] = a->size[0]; asize[1] = a->size[1]; bsize[0] = b->size[0]; bsize[1] = b->size[1];
+   for (i = 2; i < nd; i++) asize[i] = bsize[i] = csize[i];
+   if ((v = OcTensor_broadcastTo(a, nd, asize)) == NULL) goto final;
+   OcDecrefTensor(a); a = v;
+   if ((v = OcTensor_broadcastTo(b, nd, bsize)) == NULL) goto final;
+   OcDecrefTensor(b); b = v;
+   if (*C == NULL) { if ((c = OcTensor_create(nd, csize, NULL, dtype, device)) == NULL) goto final; }
    else
-   {  c = OcIncrefTensor(*C);
-      if (c->ndims != 2 || c->size[0] != M || c->size[1] != N) { OcErrorMessage("Destination size does not match the product"); goto final; }
+   {  int same = ((*C)->ndims == nd);
+      c = OcIncrefTensor(*C);
+      for (i = 0; same && i < nd; i++) if (c->size[i] != csize[i]) same = 0;
+      if (!same) { OcErrorMessage("Destination size does not match the product"); goto final; }
+      for (i = 2; same && i < nd; i++) if (c->size[i] > 1 && c->strides[i] == 0) same = 0;      /* products must not share their destination */
       if (c->dtype != dtype || c->device != device || OcTensor_isByteswapped(c) || (M > 1 && c->strides[0] != c->elemsize) ||
-          (N > 1 && (c->strides[1] < M * c->elemsize || c->strides[1] % c->elemsize != 0)))
+          (N > 1 && (c->strides[1] < M * c->elemsize || c->strides[1] % c->elemsize != 0)) || !same)
       {  if (OcTensor_ensure(&c, dtype, device) != 0) goto final;
          if (c == *C)                                   /* same type but unusable layout: work on a dense copy */
-         {  OcTensor *r = OcTensor_create(2, csize, NULL, dtype, device);
+         {  OcTensor *r = OcTensor_create(nd, csize, NULL, dtype, device);
             if (r == NULL || OcTensor_copy(c, r) != 0) { if (r) OcDecrefTensor(r); goto final; }
             OcDecrefTensor(c); c = r;
          }

@@ -449,20 +449,17 @@ static int OcTensorGPU_gemm(OcSize M, OcSize N, OcSize K, char transA, char tran
    if (K == 0) { ldA = N; ldB = M; }
    if (!och_gemm_supported(A->dtype)) return OcErrorMessage("Unsupported data type in function gpu gemm (%s)", OcDType_name(A->dtype));
    if (activate(A->device) != 0) return -1;
-   for (;;)                                       /* one product per index of the dimensions beyond the second */
-   {  OCH_CALL(och_gemm(A->dtype, transA, transB, (size_t)M, (size_t)N, (size_t)K, pa, pA, ldA > 0 ? ldA : 1, pB, ldB > 0 ? ldB : 1, pb, pC, ldC, host, GPU_STREAM(C)));
-      for (i = 2; i < ndims; i++)
-      {  index[i]++;
-         if (i < alpha->ndims) pa += alpha->strides[i];
-         if (i < beta->ndims)  pb += beta->strides[i];
-         pA += A->strides[i]; pB += B->strides[i]; pC += C->strides[i];
-         if (index[i] < A->size[i]) break;
-         index[i] = 0;
-         if (i < alpha->ndims) pa -= A->size[i] * alpha->strides[i];
-         if (i < beta->ndims)  pb -= A->size[i] * beta->strides[i];
-         pA -= A->size[i] * A->strides[i]; pB -= A->size[i] * B->strides[i]; pC -= A->size[i] * C->strides[i];
+   /* the reference loops over the dimensions beyond the second (tensor_blas_gpu.c:171-252); here they are one batched launch */
+   {  size_t bsize[OC_TENSOR_MAX_DIMS]; ptrdiff_t sa[OC_TENSOR_MAX_DIMS], sb[OC_TENSOR_MAX_DIMS], sA[OC_TENSOR_MAX_DIMS], sB[OC_TENSOR_MAX_DIMS], sC[OC_TENSOR_MAX_DIMS];
+      int nb = 0;
+      for (i = 2; i < ndims; i++, nb++)
+      {  bsize[nb] = (size_t)A->size[i];
+         sa[nb] = (i < alpha->ndims) ? alpha->strides[i] : 0; sb[nb] = (i < beta->ndims) ? beta->strides[i] : 0;
+         sA[nb] = A->strides[i]; sB[nb] = B->strides[i]; sC[nb] = C->strides[i];
       }
-      if (i >= ndims) break;
+      (void)index;
+      OCH_CALL(och_gemm_batched(A->dtype, transA, transB, (size_t)M, (size_t)N, (size_t)K, pa, pA, ldA > 0 ? ldA : 1, pB, ldB > 0 ? ldB : 1, pb, pC, ldC,
+                                nb, bsize, sa, sA, sB, sb, sC, host, GPU_STREAM(C)));
    }
    return 0;
 }

@@ -223,3 +223,70 @@ def test_mgs_qr_pattern(hip, stream):
     assert np.abs(Qg - ref).max() < 1e-11
     off = ~np.eye(n, dtype=bool)
     assert np.abs(Rg[off] - Rref[off]).max() < 1e-11
+
+
+BATCH_CASES = [  # dtype, ta, tb, M, N, K, batch sizes, B shared by the products, scalars on the device / varying per product
+    (H.DOUBLE, "N", "N", 128, 128, 64, (3,), False, False),
+    (H.DOUBLE, "T", "N", 70, 50, 90, (2, 3), True, True),
+    (H.FLOAT, "N", "T", 130, 257, 33, (4,), False, True),
+    (H.FLOAT, "T", "N", 1, 1, 700, (5, 2), False, True),            # dot products
+    (H.CFLOAT, "C", "N", 65, 40, 50, (3,), True, False),
+    (H.CDOUBLE, "N", "C", 33, 31, 17, (2, 2), False, True),
+    (H.INT32, "N", "N", 70, 66, 40, (3,), False, True),
+    (H.BOOL, "T", "T", 20, 30, 10, (2,), False, False),
+    (H.HALF, "N", "N", 64, 64, 64, (3,), False, False),
+    (H.DOUBLE, "N", "N", 16, 16, 16, (1, 7, 1), False, "host"),       # host scalars that differ per product: one launch each
+]
+
+
+@pytest.mark.parametrize("case", BATCH_CASES, ids=lambda c: "%s-%s%s-%dx%dx%d-b%s" % (H.NAMES[c[0]], c[1], c[2], c[3], c[4], c[5], "x".join(map(str, c[6]))))
+def test_gemm_batched_equals_loop(hip, stream, case):
+    """och_gemm_batched (the reference's loop over the dimensions beyond the second, tensor_blas_gpu.c:171-252, as one
+    launch) gives bit for bit what one och_gemm per product gives (those are held to the oracle above); integer
+    results are also compared with the oracle directly."""
+    dtype, ta, tb, M, N, K, bsize, share_b, scalars = case
+    rng = np.random.default_rng(99 + dtype + M)
+    rowsA, colsA = (M, K) if ta == "N" else (K, M)
+    rowsB, colsB = (K, N) if tb == "N" else (N, K)
+    ldA, ldB, ldC = rowsA + 2, rowsB + 1, M + 3
+    total = int(np.prod(bsize))
+    item = np.dtype(H.storage(dtype)).itemsize
+    A = H.random_data(dtype, ldA * colsA * total, rng, "small")
+    B = H.random_data(dtype, ldB * colsB * (1 if share_b else total), rng, "small")
+    C0 = H.random_data(dtype, ldC * N * total, rng, "small")
+    vary = bool(scalars)
+    als = np.concatenate([scalar_of(dtype, v) for v in (rng.integers(1, 3, total) if vary else [2] * total)])
+    bes = np.concatenate([scalar_of(dtype, v) for v in (rng.integers(0, 2, total) if vary else [1] * total)])
+    # byte strides per batch dimension, first dimension fastest
+    mult = [int(np.prod(bsize[:d])) for d in range(len(bsize))]
+    sA = [m * ldA * colsA * item for m in mult]
+    sB = [0 if share_b else m * ldB * colsB * item for m in mult]
+    sC = [m * ldC * N * item for m in mult]
+    sS = [m * item if vary else 0 for m in mult]
+    dA, dB = oh.to_device(A, stream), oh.to_device(B, stream)
+    dC1, dC2 = oh.to_device(C0, stream), oh.to_device(C0, stream)
+    on_host = scalars == "host" or scalars is False
+    if on_host:
+        pal, pbe = als.ctypes.data, bes.ctypes.data
+    else:
+        dal, dbe = oh.to_device(als, stream), oh.to_device(bes, stream)
+        pal, pbe = dal.address, dbe.address
+    oh.check(oh.lib.och_gemm_batched(dtype, ta.encode(), tb.encode(), M, N, K, pal, dA.ptr, ldA, dB.ptr, ldB, pbe, dC1.ptr, ldC,
+                                     len(bsize), oh.sizes(bsize), oh.strides(sS), oh.strides(sA), oh.strides(sB), oh.strides(sS), oh.strides(sC),
+                                     1 if on_host else 0, stream.handle))
+    want = C0.copy()
+    for z in range(total):
+        idx = [(z // m) % n for m, n in zip(mult, bsize)]
+        off = lambda st: sum(i * s for i, s in zip(idx, st))
+        oh.check(oh.lib.och_gemm(dtype, ta.encode(), tb.encode(), M, N, K, pal + off(sS), dA.address + off(sA), ldA, dB.address + off(sB), ldB,
+                                 pbe + off(sS), dC2.address + off(sC), ldC, 1 if on_host else 0, stream.handle))
+        if dtype not in TOL:
+            assert orc.lib.oracle_gemm(dtype, ta.encode(), tb.encode(), M, N, K, als.ctypes.data + off(sS), A.ctypes.data + off(sA), ldA,
+                                       B.ctypes.data + off(sB), ldB, bes.ctypes.data + off(sS), want.ctypes.data + off(sC), ldC, 1) == 0
+    got, loop = dC1.download(C0.dtype, C0.size), dC2.download(C0.dtype, C0.size)
+    H.assert_same_bytes(got, loop, "batched vs loop")
+    if dtype not in TOL:
+        H.assert_same_bytes(got, want, "batched vs oracle")
+    assert not np.array_equal(got, C0)
+    for b in (dA, dB, dC1, dC2):
+        b.free()

@@ -208,3 +208,30 @@ def test_find_and_mask_to_offset_through_the_table(gpu):
     assert np.array_equal(host.to_numpy(off), want @ np.array([8, 8 * 33, 8 * 33 * 40]))
     f = host.from_numpy(np.zeros((3, 3), np.float32), host.FLOAT, gpu)
     assert not host.lib.OcTensor_find(f) and b"Boolean" in host.lib.OcError_lastMessage()
+
+
+def test_batched_gemm_with_broadcast_through_the_front_end(gpu):
+    """Dimensions beyond the second index independent products (tensor_blas_gpu.c:171-252); here one batched launch.
+    A is (m, k, 3, 2), B is (k, n, 1, 2): B is shared along dimension 2."""
+    rng = np.random.default_rng(21)
+    m, n, k = 40, 30, 50
+    A = rng.uniform(-1, 1, (2, 3, k, m))           # numpy axes are Ocean's reversed
+    B = rng.uniform(-1, 1, (2, 1, n, k))
+    tA, tB = host.from_numpy(A, host.DOUBLE, gpu), host.from_numpy(B, host.DOUBLE, gpu)
+    c = host.TP()
+    host.check(host.lib.OcTensor_mtimes(tA, tB, C.byref(c)))
+    assert host.shape_of(c) == [m, n, 3, 2]
+    want = np.einsum("xykm,xznk->xynm", A, np.broadcast_to(B, (2, 1, n, k)))
+    got = host.to_numpy(c)
+    assert got.shape == want.shape
+    assert np.linalg.norm(got - want) <= 1e-13 * np.linalg.norm(np.einsum("xykm,xznk->xynm", np.abs(A), np.abs(B)))
+    # accumulate into an existing destination: C <- 2 * A * B - C, integers, exact
+    Ai = rng.integers(-4, 4, (3, k, m)).astype(np.int64); Bi = rng.integers(-4, 4, (3, n, k)).astype(np.int64)
+    C0 = rng.integers(-9, 9, (3, n, m)).astype(np.int64)
+    tc = host.from_numpy(C0, host.INT64, gpu)
+    alpha, beta = host.scalar(host.INT64, 2), host.scalar(host.INT64, -1)
+    host.check(host.lib.OcTensor_gemm(C.byref(alpha), host.from_numpy(Ai, host.INT64, gpu), b"N", host.from_numpy(Bi, host.INT64, gpu), b"N",
+                                      C.byref(beta), C.byref(tc)))
+    assert np.array_equal(host.to_numpy(tc), 2 * np.einsum("xkm,xnk->xnm", Ai, Bi) - C0)
+    with pytest.raises(host.OceanError, match="not compatible"):
+        host.check(host.lib.OcTensor_mtimes(tA, host.from_numpy(rng.uniform(-1, 1, (2, 2, n, k)), host.DOUBLE, gpu), C.byref(host.TP())))
