@@ -266,11 +266,22 @@ __global__ __launch_bounds__(256) void gemm_dot_kernel(const GemmParams<R> p, in
    const R *a = reinterpret_cast<const R *>(p.A + oA) + (int64_t)row * sAm * NPL;
    const R *b = reinterpret_cast<const R *>(p.B + oB) + (int64_t)col * sBn * NPL;
    double sr = 0, si = 0;
-   for (uint32_t k = threadIdx.x; k < p.K; k += 256)
-   {  const R *x = a + (int64_t)k * sAk * NPL, *y = b + (int64_t)k * sBk * NPL;
-      if (!CPLX) sr += (double)x[0] * (double)y[0];
-      else
-      {  const double xr = x[0], xi = p.conjA ? -(double)x[1] : (double)x[1];
+   if (!CPLX)
+   {  /* four independent loads and partial sums per trip: the block is alone on its compute unit and latency-bound */
+      double s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+      uint32_t k = threadIdx.x;
+      for (; k + 768 < p.K; k += 1024)
+      {  const R x0 = a[(int64_t)k * sAk], x1 = a[(int64_t)(k + 256) * sAk], x2 = a[(int64_t)(k + 512) * sAk], x3 = a[(int64_t)(k + 768) * sAk];
+         const R y0 = b[(int64_t)k * sBk], y1 = b[(int64_t)(k + 256) * sBk], y2 = b[(int64_t)(k + 512) * sBk], y3 = b[(int64_t)(k + 768) * sBk];
+         s0 += (double)x0 * (double)y0; s1 += (double)x1 * (double)y1; s2 += (double)x2 * (double)y2; s3 += (double)x3 * (double)y3;
+      }
+      for (; k < p.K; k += 256) s0 += (double)a[(int64_t)k * sAk] * (double)b[(int64_t)k * sBk];
+      sr = (s0 + s1) + (s2 + s3);
+   }
+   else
+   {  for (uint32_t k = threadIdx.x; k < p.K; k += 256)
+      {  const R *x = a + (int64_t)k * sAk * NPL, *y = b + (int64_t)k * sBk * NPL;
+         const double xr = x[0], xi = p.conjA ? -(double)x[1] : (double)x[1];
          const double yr = y[0], yi = p.conjB ? -(double)y[1] : (double)y[1];
          sr += xr * yr - xi * yi; si += xr * yi + xi * yr;
       }
@@ -282,6 +293,48 @@ __global__ __launch_bounds__(256) void gemm_dot_kernel(const GemmParams<R> p, in
    if (threadIdx.x != 0) return;
    sr = ((lds[0] + lds[2]) + lds[4]) + lds[6];
    si = ((lds[1] + lds[3]) + lds[5]) + lds[7];
+   R alr = p.alpha[0], ali = p.alpha[1], ber = p.beta[0], bei = p.beta[1];
+   if (p.alpha_dev) { const R *q = reinterpret_cast<const R *>(reinterpret_cast<const char *>(p.alpha_dev) + oAlpha); alr = q[0]; if (CPLX) ali = q[1]; }
+   if (p.beta_dev)  { const R *q = reinterpret_cast<const R *>(reinterpret_cast<const char *>(p.beta_dev) + oBeta);   ber = q[0]; if (CPLX) bei = q[1]; }
+   R *c = reinterpret_cast<R *>(p.C + oC) + ((int64_t)row + (int64_t)col * p.ldC) * NPL;
+   if (!CPLX)
+   {  double v = (double)alr * sr;
+      if (ber != 0) v += (double)ber * (double)c[0];
+      c[0] = (R)v;
+   }
+   else
+   {  double vr = (double)alr * sr - (double)ali * si, vi = (double)alr * si + (double)ali * sr;
+      if (ber != 0 || bei != 0)
+      {  const double cr = c[0], ci = c[1];
+         vr += (double)ber * cr - (double)bei * ci; vi += (double)ber * ci + (double)bei * cr;
+      }
+      c[0] = (R)vr; c[1] = (R)vi;
+   }
+}
+
+/* Very short inner dimension (rank-1 updates, K <= 4): one thread per element of C reads its K products directly;
+   the tile machinery of the MFMA kernel would spend its time on padding. Accumulates in double. */
+template <class R, bool CPLX>
+__global__ __launch_bounds__(256) void gemm_outer_kernel(const GemmParams<R> p, int64_t sAm, int64_t sAk, int64_t sBk, int64_t sBn)
+{
+   constexpr int NPL = CPLX ? 2 : 1;
+   int64_t oA, oB, oC, oAlpha, oBeta;
+   gemm_batch_offsets(p.batch, oA, oB, oC, oAlpha, oBeta);
+   const uint64_t e = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+   if (e >= (uint64_t)p.M * p.N) return;
+   const uint32_t col = (uint32_t)(e / p.M), row = (uint32_t)(e - (uint64_t)col * p.M);
+   const R *a = reinterpret_cast<const R *>(p.A + oA) + (int64_t)row * sAm * NPL;
+   const R *b = reinterpret_cast<const R *>(p.B + oB) + (int64_t)col * sBn * NPL;
+   double sr = 0, si = 0;
+   for (uint32_t k = 0; k < p.K; k++)
+   {  const R *x = a + (int64_t)k * sAk * NPL, *y = b + (int64_t)k * sBk * NPL;
+      if (!CPLX) sr += (double)x[0] * (double)y[0];
+      else
+      {  const double xr = x[0], xi = p.conjA ? -(double)x[1] : (double)x[1];
+         const double yr = y[0], yi = p.conjB ? -(double)y[1] : (double)y[1];
+         sr += xr * yr - xi * yi; si += xr * yi + xi * yr;
+      }
+   }
    R alr = p.alpha[0], ali = p.alpha[1], ber = p.beta[0], bei = p.beta[1];
    if (p.alpha_dev) { const R *q = reinterpret_cast<const R *>(reinterpret_cast<const char *>(p.alpha_dev) + oAlpha); alr = q[0]; if (CPLX) ali = q[1]; }
    if (p.beta_dev)  { const R *q = reinterpret_cast<const R *>(reinterpret_cast<const char *>(p.beta_dev) + oBeta);   ber = q[0]; if (CPLX) bei = q[1]; }
@@ -338,6 +391,12 @@ static int launch_gemm_mfma(const GemmArgs &g)
    {  /* op(A)(m,k) = A[m*sAm + k*sAk], op(B)(k,n) = B[k*sBk + n*sBn] */
       const int64_t sAm = akc ? g.ldA : 1, sAk = akc ? 1 : g.ldA, sBk = bkc ? 1 : g.ldB, sBn = bkc ? g.ldB : 1;
       hipLaunchKernelGGL((gemm_dot_kernel<R, CPLX>), dim3((unsigned)(g.M * g.N), 1, g.nz), dim3(256), 0, g.stream, p, sAm, sAk, sBk, sBn);
+      OCH_CHECK_LAUNCH();
+      return 0;
+   }
+   if (g.K <= 4 && (uint64_t)g.M * g.N <= 0x7FFFFFFFull * 256)
+   {  const int64_t sAm = akc ? g.ldA : 1, sAk = akc ? 1 : g.ldA, sBk = bkc ? 1 : g.ldB, sBn = bkc ? g.ldB : 1;
+      hipLaunchKernelGGL((gemm_outer_kernel<R, CPLX>), dim3((unsigned)(((uint64_t)g.M * g.N + 255) / 256), 1, g.nz), dim3(256), 0, g.stream, p, sAm, sAk, sBk, sBn);
       OCH_CHECK_LAUNCH();
       return 0;
    }
