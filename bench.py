@@ -356,6 +356,20 @@ def main():
         pairs = 64 * 63 // 2
         configs["c5_mgs_qr_4096_first64cols"] = {"us_per_pair": round(dt_s / pairs * 1e6, 2), "launches_per_pair": 2,
                                                  "effective_GBps": round(pairs * (2 * 8 * m + 3 * 8 * m) / dt_s / 1e9, 1)}
+        # the same window recorded once and replayed as a graph: no host work per operation
+        if "och_graph_launch" not in oh.MISSING:
+            oh.check(lib.och_stream_begin_capture(h))
+            mgs_window()
+            graph = C.c_void_p()
+            oh.check(lib.och_stream_end_capture(h, C.byref(graph)))
+            oh.check(lib.och_graph_launch(graph, h)); stream.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                oh.check(lib.och_graph_launch(graph, h))
+            stream.synchronize(); dt_g = (time.perf_counter() - t0) / 3
+            oh.check(lib.och_graph_destroy(graph))
+            configs["c5_mgs_qr_4096_first64cols_graph_replay"] = {"us_per_pair": round(dt_g / pairs * 1e6, 2), "launches_per_pair": 2,
+                                                                  "effective_GBps": round(pairs * (2 * 8 * m + 3 * 8 * m) / dt_g / 1e9, 1)}
         for b in (q, rr, consts):
             b.free()
     result["configs"] = configs

@@ -106,6 +106,20 @@ int och_event_record(och_event event, och_stream stream);  /* device_gpu.c:398-4
 int och_event_synchronize(och_event event);                /* device_gpu.c:386-394 */
 int och_event_elapsed_ms(och_event start, och_event stop, float *ms);
 
+/* Launch-bound sequences of small operations (the dot -> scale -> subtract chain of a modified Gram-Schmidt sweep   */
+/* issues millions of them) can be recorded once and replayed as one graph launch. No counterpart in the reference  */
+/* (it launches every operation separately). Between begin and end the stream records instead of executing; calls   */
+/* that synchronise or allocate may not be recorded: och_reduce_all, och_find_count, och_memcpy_htod / dtoh,        */
+/* och_malloc_async / och_free_async, och_copy between tensors of different shape AND type. Everything else in this */
+/* header is recordable; scalars passed in host memory are frozen at their recorded value, scalars in device memory */
+/* are read at every replay. `stream` must be a created stream; call och_device_warmup on the device beforehand     */
+/* (it creates the per-device scratch of the reductions).                                                           */
+typedef void *och_graph;
+int och_stream_begin_capture(och_stream stream);
+int och_stream_end_capture(och_stream stream, och_graph *graph);
+int och_graph_launch(och_graph graph, och_stream stream);
+int och_graph_destroy(och_graph graph);
+
 /* Stream-ordered allocation: the block is usable by work enqueued on `stream`
    after the call and is returned to the device pool in stream order.
    Replaces cudaMalloc/cudaFree of storage_gpu.c:83-95,107-116. */

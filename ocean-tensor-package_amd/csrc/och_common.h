@@ -26,5 +26,9 @@ void clear_error();
    } while (0)
 
 static inline hipStream_t as_stream(och_stream s) { return (hipStream_t)s; }
+/* byte fill by a kernel (och_runtime.hip): unlike a memset node it is safe inside a captured graph */
+int fill_bytes(void *dst, int value, size_t nbytes, hipStream_t stream);
+/* creates the current device's reduction scratch and pinned result slot if they do not exist yet (och_reduce.hip) */
+int red_context_init();
 
 } /* namespace och */

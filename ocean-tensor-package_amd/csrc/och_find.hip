@@ -156,7 +156,7 @@ extern "C" int och_find_count(int ndims, const size_t *size, const ptrdiff_t *st
    if (!workspace || !nnz) return set_error("find: null argument");
    if (find_params(p, ndims, size, strides, ptr) != 0) return -1;
    *nnz = 0;
-   if (p.nelem == 0) { OCH_CHECK_HIP(hipMemsetAsync(workspace, 0, 2 * sizeof(unsigned long long), as_stream(stream))); return 0; }
+   if (p.nelem == 0) return fill_bytes(workspace, 0, 2 * sizeof(unsigned long long), as_stream(stream));
    const uint64_t chunks = (p.nelem + OCH_FIND_CHUNK - 1) / OCH_FIND_CHUNK;
    if (chunks > 0x7FFFFFFFull) return set_error("find: too many elements");
    hipLaunchKernelGGL(find_count_kernel, dim3((unsigned)chunks), dim3(OCH_FIND_THREADS), 0, as_stream(stream), p, (unsigned long long *)workspace);

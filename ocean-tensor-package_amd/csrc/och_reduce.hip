@@ -45,6 +45,7 @@ int red_context(RedContext **out)
    *out = &g_ctx[dev];
    return 0;
 }
+int red_context_init() { RedContext *ctx; return red_context(&ctx); }
 }  /* namespace och */
 
 using namespace och;

@@ -210,7 +210,7 @@ static int launch_reduce_all(int ndims, const size_t *size, const ptrdiff_t *str
    p.partials = scratch;
    p.counter = reinterpret_cast<unsigned int *>(scratch + OCH_RED_MAX_BLOCKS * OCH_RED_SLOT);
    p.result = dresult;
-   if (zero_counter) OCH_CHECK_HIP(hipMemsetAsync(p.counter, 0, sizeof(unsigned int), stream));
+   if (zero_counter && fill_bytes(p.counter, 0, sizeof(unsigned int), stream) != 0) return -1;
    uint64_t want = (p.ngroups + (uint64_t)OCH_RED_BLOCK * OCH_RED_UNR - 1) / ((uint64_t)OCH_RED_BLOCK * OCH_RED_UNR);
    unsigned int blocks = (unsigned int)(want < 1 ? 1 : (want > OCH_RED_MAX_BLOCKS ? OCH_RED_MAX_BLOCKS : want));
    {  const uint64_t step = (uint64_t)OCH_RED_BLOCK * OCH_RED_UNR;

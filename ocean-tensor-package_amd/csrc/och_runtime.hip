@@ -17,6 +17,33 @@ void clear_error() { g_errmsg[0] = 0; }
 __global__ void warmup_kernel(int *p) { if (p) *p = 1; }
 }
 
+namespace och {
+typedef unsigned int fill_u32x4 __attribute__((ext_vector_type(4)));
+/* 16-byte stores over the aligned body (grid-stride), single bytes for the unaligned head and tail (first block) */
+__global__ __launch_bounds__(256) void fill_bytes_kernel(unsigned char *dst, unsigned int pattern, size_t head, size_t body, size_t tail)
+{
+   const fill_u32x4 v = { pattern, pattern, pattern, pattern };
+   fill_u32x4 *b = reinterpret_cast<fill_u32x4 *>(dst + head);
+   for (size_t g = (size_t)blockIdx.x * 256 + threadIdx.x; g < body; g += (size_t)gridDim.x * 256) b[g] = v;
+   if (blockIdx.x == 0)
+   {  if (threadIdx.x < head) dst[threadIdx.x] = (unsigned char)pattern;
+      if (threadIdx.x < tail) dst[head + body * 16 + threadIdx.x] = (unsigned char)pattern;
+   }
+}
+int fill_bytes(void *dst, int value, size_t nbytes, hipStream_t stream)
+{
+   if (nbytes == 0) return 0;
+   if (dst == nullptr) return set_error("memset: null pointer");
+   size_t head = (16 - ((uintptr_t)dst & 15)) & 15; if (head > nbytes) head = nbytes;
+   const size_t body = (nbytes - head) / 16, tail = nbytes - head - body * 16;
+   const unsigned int byte = (unsigned int)value & 0xFFu, pattern = byte * 0x01010101u;
+   size_t blocks = (body + 255) / 256; if (blocks < 1) blocks = 1; if (blocks > 65536) blocks = 65536;
+   hipLaunchKernelGGL(fill_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (unsigned char *)dst, pattern, head, body, tail);
+   OCH_CHECK_LAUNCH();
+   return 0;
+}
+}
+
 extern "C" {
 
 const int och_type_size[OCH_DTYPE_COUNT] = { 1, 1, 2, 4, 8, 1, 2, 4, 8, 2, 4, 8, 4, 8, 16 };
@@ -70,8 +97,9 @@ int och_device_warmup(int device)
    hipLaunchKernelGGL(och::warmup_kernel, dim3(1), dim3(1), 0, 0, (int *)nullptr);
    OCH_CHECK_LAUNCH();
    OCH_CHECK_HIP(hipDeviceSynchronize());
+   const int status = och::red_context_init();      /* the reductions' per-device scratch: allocated here, not in a later (possibly recorded) call */
    OCH_CHECK_HIP(hipSetDevice(prev));
-   return 0;
+   return status;
 }
 int och_device_synchronize(void) { OCH_CHECK_HIP(hipDeviceSynchronize()); return 0; }
 
@@ -98,6 +126,33 @@ int och_event_record(och_event event, och_stream stream)
 int och_event_synchronize(och_event event) { OCH_CHECK_HIP(hipEventSynchronize((hipEvent_t)event)); return 0; }
 int och_event_elapsed_ms(och_event start, och_event stop, float *ms)
 {  OCH_CHECK_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop)); return 0; }
+
+int och_stream_begin_capture(och_stream stream)
+{  if (stream == nullptr) return och::set_error("the default stream cannot record a graph");
+   OCH_CHECK_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+   return 0;
+}
+int och_stream_end_capture(och_stream stream, och_graph *graph)
+{  hipGraph_t g = nullptr; hipGraphExec_t exec = nullptr;
+   if (graph == nullptr) return och::set_error("null graph pointer");
+   *graph = nullptr;
+   OCH_CHECK_HIP(hipStreamEndCapture((hipStream_t)stream, &g));
+   if (g == nullptr) return och::set_error("the stream recorded no graph");
+   hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+   (void)hipGraphDestroy(g);
+   if (e != hipSuccess) return och::set_error("hipGraphInstantiate failed: %s", hipGetErrorString(e));
+   *graph = (och_graph)exec;
+   return 0;
+}
+int och_graph_launch(och_graph graph, och_stream stream)
+{  if (graph == nullptr) return och::set_error("null graph");
+   OCH_CHECK_HIP(hipGraphLaunch((hipGraphExec_t)graph, (hipStream_t)stream));
+   return 0;
+}
+int och_graph_destroy(och_graph graph)
+{  if (graph) OCH_CHECK_HIP(hipGraphExecDestroy((hipGraphExec_t)graph));
+   return 0;
+}
 
 int och_malloc_async(void **ptr, size_t nbytes, och_stream stream)
 {
@@ -138,6 +193,6 @@ int och_memcpy_dtoh(void *dst, const void *src, size_t nbytes, och_stream stream
    return 0;
 }
 int och_memset_async(void *dst, int value, size_t nbytes, och_stream stream)
-{  if (nbytes) OCH_CHECK_HIP(hipMemsetAsync(dst, value, nbytes, (hipStream_t)stream)); return 0; }
+{  return och::fill_bytes(dst, value, nbytes, (hipStream_t)stream); }
 
 } /* extern "C" */

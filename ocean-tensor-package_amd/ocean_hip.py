@@ -155,6 +155,10 @@ PROTOTYPES = {
     "och_memcpy_htod_async": (_i, [_vp, _vp, C.c_size_t, _vp]),
     "och_memcpy_dtoh_async": (_i, [_vp, _vp, C.c_size_t, _vp]),
     "och_memset_async": (_i, [_vp, _i, C.c_size_t, _vp]),
+    "och_stream_begin_capture": (_i, [_vp]),
+    "och_stream_end_capture": (_i, [_vp, C.POINTER(C.c_void_p)]),
+    "och_graph_launch": (_i, [_vp, _vp]),
+    "och_graph_destroy": (_i, [_vp]),
     "och_fill": (_i, [_i, _i, _sz, _st, _vp, Scalar, _vp]),
     "och_fill_nan": (_i, [_i, _i, _sz, _st, _vp, Scalar, _vp]),
     "och_masked_fill": (_i, [_i, _i, _sz, _st, _vp, _st, _vp, Scalar, _vp]),

@@ -197,3 +197,21 @@ def test_config4_cast_byteswap(hip, stream):
     got = y.download()
     x.free(); y.free()
     H.assert_same_bytes(got, z.astype(np.complex128), "config 4b")
+
+
+def test_memset_is_exact_at_any_alignment_and_size(hip, stream):
+    """och_memset_async (Buffer_zero, storage_gpu.c:283-302) fills by a kernel: unaligned head and tail bytes, the
+    16-byte body and a large buffer, with the neighbouring bytes untouched."""
+    rng = np.random.default_rng(77)
+    base = rng.integers(0, 256, 1 << 16, dtype=np.uint8)
+    for off, n, val in ((0, 0, 1), (0, 1, 7), (3, 5, 0), (1, 15, 255), (5, 16, 9), (13, 100, 0x81), (16, 4096, 0), (7, 40001, 3), (0, 1 << 16, 0)):
+        d = oh.to_device(base, stream)
+        oh.check(oh.lib.och_memset_async(C.c_void_p(d.address + off), val, n, stream.handle))
+        want = base.copy(); want[off:off + n] = val & 0xFF
+        assert np.array_equal(d.download(np.uint8), want), (off, n, val)
+        d.free()
+    big = oh.DeviceBuffer((64 << 20) + 3, stream)
+    oh.check(oh.lib.och_memset_async(big.ptr, 0x5A, big.nbytes, stream.handle))
+    got = big.download(np.uint8)
+    assert got.min() == 0x5A and got.max() == 0x5A
+    big.free()

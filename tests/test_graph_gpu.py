@@ -1,0 +1,86 @@
+"""Recording a sequence of library calls into a graph and replaying it (och_stream_begin_capture /
+och_stream_end_capture / och_graph_launch) gives, at every replay, bit for bit what the same calls give when they are
+launched one by one. The sequence is the small-operation pattern of a modified Gram-Schmidt sweep (dot product into a
+device scalar, rank-1 update that reads it) followed by an elementwise operation, a byte fill, a full reduction into
+device memory and an axis reduction. The program's own eager work and synchronisations run between the replays."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import helpers as H
+import ocean_hip as oh
+
+pytestmark = pytest.mark.gpu
+
+
+def test_graph_replays_equal_eager_launches(hip, stream):
+    lib, h = oh.lib, stream.handle
+    rng = np.random.default_rng(31)
+    m, ncol = 1024, 6
+    q0 = rng.uniform(-1, 1, (ncol, m))                     # column-major m x ncol
+    x0 = rng.uniform(-1, 1, (64, 96))
+    dq, dx = oh.to_device(q0, stream), oh.to_device(x0, stream)
+    dr = oh.DeviceBuffer(8 * ncol * ncol, stream)
+    dz, dw = oh.DeviceBuffer(x0.nbytes, stream), oh.DeviceBuffer(1000, stream)
+    dsum, dax = oh.DeviceBuffer(64, stream), oh.DeviceBuffer(8 * 96, stream)
+    consts = oh.to_device(np.array([1.0, 0.0, -1.0]), stream)
+    one, zero, minus = [C.c_void_p(consts.address + 8 * i) for i in range(3)]
+    col = lambda j: C.c_void_p(dq.address + 8 * m * j)
+    rij = lambda i, j: C.c_void_p(dr.address + 8 * (i + ncol * j))
+    shape, st = oh.sizes([96, 64]), oh.strides([8, 8 * 96])
+    cfg = oh.ReduceAxisConfig()
+    cfg.ndims, cfg.rdims = 1, 1
+    cfg.size[0], cfg.strides1[0], cfg.strides2[0] = 96, 8, 8
+    cfg.rsize[0], cfg.rstrides[0] = 64, 8 * 96
+    cfg.ptr1, cfg.ptr2, cfg.stream = dz.ptr.value, dax.ptr.value, h
+
+    def sequence():
+        for j in range(1, ncol):
+            for i in range(j):
+                oh.check(lib.och_gemm(H.DOUBLE, b"T", b"N", 1, 1, m, minus, col(i), m, col(j), m, zero, rij(i, j), 1, 0, h))
+                oh.check(lib.och_gemm(H.DOUBLE, b"N", b"N", m, 1, 1, one, col(i), m, rij(i, j), 1, one, col(j), m, 0, h))
+        oh.check(lib.och_binary(oh.B["add"], H.DOUBLE, 2, shape, st, dx.ptr, st, dx.ptr, st, dz.ptr, h))
+        oh.check(lib.och_binary(oh.B["multiply"], H.DOUBLE, 2, shape, st, dz.ptr, st, dx.ptr, st, dx.ptr, h))      # state that changes per run
+        oh.check(lib.och_memset_async(dw.ptr, 0x3C, 1000, h))
+        oh.check(lib.och_reduce_all_device(oh.R["sum"], H.DOUBLE, 2, shape, st, dz.ptr, None, None, 0.0, dsum.ptr, None, h))
+        oh.check(lib.och_reduce_axis(oh.R["maximum"], H.DOUBLE, C.byref(cfg), 0.0))
+
+    def snapshot():
+        stream.synchronize()
+        return [b.download(np.uint8).copy() for b in (dq, dx, dr, dz, dw, dsum, dax)]
+
+    def reset():
+        dq.upload(q0); dx.upload(x0)
+        for b in (dr, dz, dw, dsum, dax):
+            oh.check(lib.och_memset_async(b.ptr, 0, b.nbytes, h))
+        stream.synchronize()
+
+    reset()
+    eager = []
+    for _ in range(3):
+        sequence()
+        eager.append(snapshot())
+    assert not np.array_equal(eager[0][1], eager[1][1])            # the runs really differ
+
+    reset()
+    oh.check(lib.och_stream_begin_capture(h))
+    sequence()
+    graph = C.c_void_p()
+    oh.check(lib.och_stream_end_capture(h, C.byref(graph)))
+    assert np.array_equal(dx.download(np.float64, x0.size).reshape(x0.shape), x0)       # recording executed nothing
+    scratch = oh.to_device(x0, stream)
+    for k in range(3):
+        oh.check(lib.och_graph_launch(graph, h))
+        got = snapshot()
+        for g, e, name in zip(got, eager[k], ("Q", "x", "R", "z", "w", "sum", "axis")):
+            assert np.array_equal(g, e), "replay %d: %s differs from the eager launches" % (k, name)
+        # unrelated eager work and a synchronisation between the replays
+        oh.check(lib.och_binary(oh.B["add"], H.DOUBLE, 2, shape, st, scratch.ptr, st, scratch.ptr, st, scratch.ptr, h))
+        stream.synchronize()
+    oh.check(lib.och_graph_destroy(graph))
+    # recording on the default stream is refused, as is a second end without a begin
+    with pytest.raises(oh.OceanHipError):
+        oh.check(lib.och_stream_begin_capture(None))
+    for b in (dq, dx, dr, dz, dw, dsum, dax, consts, scratch):
+        b.free()
