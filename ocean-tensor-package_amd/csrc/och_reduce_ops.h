@@ -47,6 +47,10 @@ template <class T> struct red_param
    double phalf, pinv;        /* p/2 and 1/p for the general norm */
 };
 
+/* pow of the general p-norm as one out-of-line function per translation unit: inlined at every load site of every
+   kernel variant it multiplies the code size and the build time of the norm kernels */
+static __device__ __noinline__ double norm_pow(double x, double y) { return pow(x, y); }
+
 template <class T, int OP> struct Reduce
 {
    typedef typename traits<T>::work W;
@@ -230,7 +234,7 @@ template <class T, int OP> struct Reduce
          {  double re = (double)to_work(x.real), im = (double)to_work(x.imag); sq = re * re + im * im; }
          else { double v = (double)raw(x); sq = v * v; }
          if constexpr (OP == R_NORM_NAN || OP == R_NORM2_NAN) { if (isnan(sq)) return 0.0; }
-         if constexpr (OP == R_NORM || OP == R_NORM_NAN) return pow(sq, p.phalf);
+         if constexpr (OP == R_NORM || OP == R_NORM_NAN) return norm_pow(sq, p.phalf);
          else return sq;
       }
    }
@@ -291,7 +295,7 @@ template <class T, int OP> struct Reduce
          else return from_work<ABS>(a);
       }
       else
-      {  double v = (OP == R_NORM || OP == R_NORM_NAN) ? pow(a, p.pinv) : sqrt(a);
+      {  double v = (OP == R_NORM || OP == R_NORM_NAN) ? norm_pow(a, p.pinv) : sqrt(a);
          if constexpr (is_float_v<T> || is_complex_v<T>) return from_work<ABS>((typename traits<ABS>::work)v);
          else return v;
       }
