@@ -10,11 +10,20 @@ import shutil
 SRC = "/root/reference/examples/python/gpu/tensors"
 NAMES = ["tensor_add_02", "ocean_min_01", "ocean_and_01", "ocean_or_01", "ocean_xor_01", "ocean_bitshift_01", "ocean_sign_01",
          "ocean_axis_reduce_04", "ocean_sum_02", "ocean_sumabs_01", "ocean_all_01", "ocean_maximumabs_02", "ocean_gemm_01",
-         "ocean_fabs_01", "ocean_logical_01"]
+         "ocean_fabs_01", "ocean_logical_01",
+         "ocean_bitshift_02", "ocean_fabs_02", "ocean_gemm_10", "ocean_gemm_11", "ocean_linspace_03", "ocean_maximumabs_01", "ocean_not_01",
+         "ocean_cast_01", "ocean_power_01", "ocean_power_02", "ocean_power_03", "ocean_sum_01", "ocean_unary_01", "tensor_add_01",
+         "tensor_axis_norm2_01", "tensor_divide_01", "tensor_multiply_01", "tensor_subtract_01", "tensor_dtype_cast_01", "tensor_fill_01",
+         "tensor_copy_03", "tensor_copy_04", "tensor_copy_06", "tensor_copy_07"]
+# the GPU file of tensor_fillnan_01 records a defect of the reference's GPU kernel (it fills every element,
+# solid/src/core/gpu/template_fill.cu:72-79); the CPU twin holds the defined behaviour (only NaN is replaced)
+CPU_TWINS = ["tensor_fillnan_01"]
 
 if __name__ == "__main__":
     dst = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ref")
     os.makedirs(dst, exist_ok=True)
     for n in NAMES:
         shutil.copyfile(os.path.join(SRC, n + ".ref"), os.path.join(dst, n + ".ref"))
-    print("copied %d files" % len(NAMES))
+    for n in CPU_TWINS:
+        shutil.copyfile(os.path.join(SRC.replace("/gpu/", "/cpu/"), n + ".ref"), os.path.join(dst, n + "_cpu.ref"))
+    print("copied %d files" % (len(NAMES) + len(CPU_TWINS)))

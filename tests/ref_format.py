@@ -13,7 +13,8 @@ TYPE_NAMES = {"bool": H.BOOL, "uint8": H.UINT8, "uint16": H.UINT16, "uint32": H.
               "double": H.DOUBLE, "complex-half": H.CHALF, "complex-float": H.CFLOAT, "complex-double": H.CDOUBLE}
 _NUM = r"(?:-?\d+(?:\.\d+)?(?:e[+-]?\d+)?|-?nan|-?inf)"
 _TOKEN = re.compile(r"(True|False)|(%s)\s*([+-])\s*(%s)j|(%s)" % (_NUM, _NUM, _NUM))
-_TENSOR = re.compile(r"^<tensor\.([\w-]+) of size ([\dx]+) on (\w+)( \(byteswapped\))?>$")
+_TENSOR = re.compile(r"^<(?:empty )?(?:tensor|storage)\.([\w-]+) of size ([\dx]+) on (\w+)( \(byteswapped\))?>$")
+_SCALAR = re.compile(r"^<scalar\.([\w-]+) on (\w+)>$")
 
 
 def parse_values(line):
@@ -32,19 +33,27 @@ def parse_values(line):
 class RefTensor:
     def __init__(self, dtype, shape, values, device, byteswapped):
         self.dtype, self.shape, self.device, self.byteswapped = dtype, shape, device, byteswapped
-        self.values = values            # numpy complex128 / float64 / bool array in Ocean index order A[i0, i1, ...]
+        self.values = values            # numpy complex128 / float64 / bool array in Ocean index order A[i0, i1, ...]; None: printed in part only
 
     def __repr__(self):
         return "RefTensor(%s, %s, %s)" % (H.NAMES[self.dtype], self.shape, self.device)
 
 
 def parse_ref(text):
-    """List of items in file order: RefTensor objects, ('scalars', [values], line) for lines made of values
-    only, and ('text', line) for headings."""
+    """List of items in file order: RefTensor objects (tensors, storages printed as one-dimensional tensors, and
+    "<scalar...>" zero-dimensional tensors with shape []), ('scalars', [values]) for lines made of values only, and
+    ('text', line) for headings."""
     items, rows = [], []
     for line in text.splitlines():
         s = line.strip()
         if not s:
+            continue
+        m = _SCALAR.match(s)
+        if m:                                                        # a zero-dimensional tensor: one value, then this line
+            flat = [v for r in rows for v in r]
+            assert len(flat) == 1, "scalar printed with %d values" % len(flat)
+            items.append(RefTensor(TYPE_NAMES[m.group(1)], [], np.array(flat[0]), m.group(2), False))
+            rows = []
             continue
         m = _TENSOR.match(s)
         if m:
@@ -52,7 +61,10 @@ def parse_ref(text):
             shape = [int(x) for x in m.group(2).split("x")]
             flat = [v for r in rows for v in r]
             n = int(np.prod(shape))
-            assert len(flat) == n, "tensor of size %s printed with %d values" % (shape, len(flat))
+            if len(flat) != n:                                    # large tensors are printed with rows left out
+                items.append(RefTensor(dtype, shape, None, m.group(3), bool(m.group(4))))
+                rows = []
+                continue
             if len(shape) == 1:
                 arr = np.array(flat)
             else:
@@ -139,5 +151,8 @@ def assert_matches(dtype, got_storage, ref, what=""):
     for gp, wp in ((g.real, w.real), (g.imag, w.imag)):
         nan = np.isnan(wp)
         assert np.array_equal(np.isnan(gp), nan), what
+        inf = np.isinf(wp)
+        assert np.array_equal(gp[inf], wp[inf]) and not np.isinf(gp[~inf & ~nan]).any(), what
+        nan = nan | inf
         ok = np.abs(gp[~nan] - wp[~nan]) <= 6e-6 * np.maximum(1.0, np.abs(wp[~nan]))
         assert ok.all(), "%s: got %s want %s" % (what, gp, wp)

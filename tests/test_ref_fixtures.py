@@ -81,6 +81,108 @@ class Engine:
             assert orc.lib.oracle_copy(*args, 1) == 0
         return self._result(c, z)
 
+    def swap_cast(self, ts, td, x):
+        """converting copy that reverses the bytes of every element (real part) on the way: byte-swapped source or destination"""
+        z = np.asfortranarray(np.zeros(x.shape, H.storage(td)))
+        a, c = self._operand(x, ts), self._operand(z, td)
+        nd = x.ndim
+        args = (ts, td, nd, oh.sizes(a.shape), oh.strides(a.strides), self._ptr(a), nd, oh.sizes(c.shape), oh.strides(c.strides), self._ptr(c, z))
+        if self.gpu:
+            oh.check(oh.lib.och_byteswap_copy(*args, self.stream.handle)); a.free()
+        else:
+            assert orc.lib.oracle_byteswap_copy(*args, 1) == 0
+        return self._result(c, z)
+
+    def reshape_copy(self, ts, td, parent, view, dst_shape, swap=False):
+        """copy a (strided / broadcast) view into a dense tensor of another shape with the same number of elements, converting
+        (and reversing the bytes of every element when swap is set); elements are taken in Ocean's order, first index fastest"""
+        z = np.asfortranarray(np.zeros(dst_shape, H.storage(td)))
+        a = H.Operand(parent, view, ts); c = self._operand(z, td)
+        if self.gpu:
+            a.upload(self.stream)
+        args = (ts, td, view.ndim, oh.sizes(a.shape), oh.strides(a.strides), self._ptr(a), z.ndim, oh.sizes(c.shape), oh.strides(c.strides), self._ptr(c, z))
+        fn = (oh.lib.och_byteswap_copy if swap else oh.lib.och_copy) if self.gpu else (orc.lib.oracle_byteswap_copy if swap else orc.lib.oracle_copy)
+        if self.gpu:
+            oh.check(fn(*args, self.stream.handle)); a.free()
+        else:
+            assert fn(*args, 1) == 0
+        return self._result(c, z)
+
+    def byteswap(self, dtype, x):
+        """reverse the bytes of every element in place (a byte-swapped destination of another type is written in native order
+        first and swapped afterwards, tensor_copy_cpu.c:140-156)"""
+        z = x.copy(order="F")
+        c = self._operand(z, dtype)
+        args = (dtype, z.ndim, oh.sizes(z.shape), oh.strides(z.strides), self._ptr(c, z))
+        if self.gpu:
+            oh.check(oh.lib.och_byteswap(*args, self.stream.handle))
+        else:
+            assert orc.lib.oracle_byteswap(*args, 1) == 0
+        return self._result(c, z)
+
+    def binary_inplace(self, name, dtype, parent, view, y):
+        """view (op)= y on a strided view of `parent`; returns the parent afterwards"""
+        op = oh.B[name]
+        work = parent.copy()
+        v = np.lib.stride_tricks.as_strided(work, shape=view.shape, strides=view.strides)
+        a = H.Operand(work, v, dtype); b = self._operand(y, dtype, np.broadcast_to(y, view.shape))
+        if self.gpu:
+            a.upload(self.stream)
+            H.gpu_binary(self.stream, op, dtype, a, b, a)
+            out = a.download(); a.free(); b.free()
+            return out
+        H.cpu_binary(op, dtype, a, b, a, work)
+        return work
+
+    def fill(self, dtype, n, value):
+        z = np.zeros(n, H.storage(dtype))
+        c = self._operand(z, dtype)
+        sc = H.raw_scalar(RF.to_storage(dtype, np.array([value])))
+        args = (dtype, 1, oh.sizes([n]), oh.strides(z.strides), self._ptr(c, z), sc)
+        if self.gpu:
+            oh.check(oh.lib.och_fill(*args, self.stream.handle))
+        else:
+            assert orc.lib.oracle_fill(*args, 1) == 0
+        return self._result(c, z)
+
+    def fill_nan(self, dtype, x, value):
+        z = x.copy()
+        c = self._operand(z, dtype)
+        sc = H.raw_scalar(RF.to_storage(dtype, np.array([value])))
+        args = (dtype, z.ndim, oh.sizes(z.shape), oh.strides(z.strides), self._ptr(c, z), sc)
+        if self.gpu:
+            oh.check(oh.lib.och_fill_nan(*args, self.stream.handle))
+        else:
+            assert orc.lib.oracle_fill_nan(*args, 1) == 0
+        return self._result(c, z)
+
+    def steps_complex(self, dtype, n, offset, step):
+        z = np.zeros(n, H.storage(dtype))
+        c = self._operand(z, dtype)
+        args = (dtype, 1, oh.sizes([n]), oh.strides(z.strides), self._ptr(c, z), oh.CDouble(offset.real, offset.imag), oh.CDouble(step.real, step.imag))
+        if self.gpu:
+            oh.check(oh.lib.och_steps_cdouble(*args, self.stream.handle))
+        else:
+            assert orc.lib.oracle_steps_cdouble(*args, 1) == 0
+        return self._result(c, z)
+
+    def gemm_raw(self, dtype, m, n, k, a, b, c0=None):
+        """C (m x n, column-major, dense) <- A (m x k) * B (k x n); empty operands allowed"""
+        c = np.zeros(m * n, H.storage(dtype)) if c0 is None else c0.copy()
+        al = RF.to_storage(dtype, np.array([1])); be = RF.to_storage(dtype, np.array([0]))
+        lda, ldb, ldc = max(m, 1), max(k, 1), max(m, 1)
+        if self.gpu:
+            da, db, dc = oh.to_device(a, self.stream), oh.to_device(b, self.stream), oh.to_device(c, self.stream)
+            oh.check(oh.lib.och_gemm(dtype, b"N", b"N", m, n, k, orc.ptr(al), da.ptr, lda, db.ptr, ldb, orc.ptr(be), dc.ptr, ldc, 1, self.stream.handle))
+            out = dc.download(c.dtype, m * n)
+            for t in (da, db, dc):
+                t.free()
+            return out
+        keep = np.zeros(1, c.dtype)                      # valid addresses for empty operands
+        assert orc.lib.oracle_gemm(dtype, b"N", b"N", m, n, k, orc.ptr(al), orc.ptr(a if a.size else keep), lda, orc.ptr(b if b.size else keep), ldb,
+                                   orc.ptr(be), orc.ptr(c if c.size else keep), ldc, 1) == 0
+        return c
+
     def reduce(self, name, dtype, x, p=0.0):
         op = oh.R[name]
         rd = oh.lib.och_reduce_result_dtype(op, dtype)
