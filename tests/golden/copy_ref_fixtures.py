@@ -18,6 +18,10 @@ NAMES = ["tensor_add_02", "ocean_min_01", "ocean_and_01", "ocean_or_01", "ocean_
 # the GPU file of tensor_fillnan_01 records a defect of the reference's GPU kernel (it fills every element,
 # solid/src/core/gpu/template_fill.cu:72-79); the CPU twin holds the defined behaviour (only NaN is replaced)
 CPU_TWINS = ["tensor_fillnan_01"]
+# index operations: the GPU index example, and the CPU examples of find (absent from the reference's GPU module)
+OTHER = [("/root/reference/examples/python/gpu/index/index_008.ref", "index_008.ref"),
+         ("/root/reference/examples/python/cpu/tensors/ocean_find_01.ref", "ocean_find_01_cpu.ref"),
+         ("/root/reference/examples/python/cpu/tensors/tensor_find_01.ref", "tensor_find_01_cpu.ref")]
 
 if __name__ == "__main__":
     dst = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ref")
@@ -26,4 +30,6 @@ if __name__ == "__main__":
         shutil.copyfile(os.path.join(SRC, n + ".ref"), os.path.join(dst, n + ".ref"))
     for n in CPU_TWINS:
         shutil.copyfile(os.path.join(SRC.replace("/gpu/", "/cpu/"), n + ".ref"), os.path.join(dst, n + "_cpu.ref"))
-    print("copied %d files" % (len(NAMES) + len(CPU_TWINS)))
+    for src, name in OTHER:
+        shutil.copyfile(src, os.path.join(dst, name))
+    print("copied %d files" % (len(NAMES) + len(CPU_TWINS) + len(OTHER)))
