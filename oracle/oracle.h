@@ -15,7 +15,8 @@
  *   reference tree into oracle/_ref/libocean_ref.so; whole operations additionally against
  *   the expected-output files of the reference's example tests (tests/golden/ref/);
  *   index operations: numpy integer-array indexing and the reference's index_008 output; find: numpy.nonzero and the
- *   reference's ocean_find_01 / tensor_find_01 outputs; integer / bool GEMM: exact arithmetic.
+ *   reference's ocean_find_01 / tensor_find_01 outputs;  integer / bool GEMM: exact arithmetic;
+ *   GEMM transposition / conjugation modes for every floating type: the reference's ocean_gemm_02 ... 09d outputs.
  * PARITY UNPINNED (no golden vector, reference build or closed form fixes the bits; the tests
  * hold these to stated tolerances instead):
  *   oracle_gemm for floating and complex types at large sizes -- the reference's CPU result

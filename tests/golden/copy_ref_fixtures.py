@@ -22,6 +22,10 @@ CPU_TWINS = ["tensor_fillnan_01"]
 OTHER = [("/root/reference/examples/python/gpu/index/index_008.ref", "index_008.ref"),
          ("/root/reference/examples/python/cpu/tensors/ocean_find_01.ref", "ocean_find_01_cpu.ref"),
          ("/root/reference/examples/python/cpu/tensors/tensor_find_01.ref", "tensor_find_01_cpu.ref")]
+# matrix products: transposition / conjugation modes for float, double, complex, int16 and bool (the GPU examples hold three)
+OTHER += [("/root/reference/examples/python/cpu/tensors/%s.ref" % n, "%s_cpu.ref" % n)
+          for n in ("ocean_gemm_02", "ocean_gemm_03", "ocean_gemm_07", "ocean_gemm_08a", "ocean_gemm_09a", "ocean_gemm_09b", "ocean_gemm_09c",
+                    "ocean_gemm_09d", "ocean_multiply_01", "ocean_multiply_02")]
 
 if __name__ == "__main__":
     dst = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ref")
