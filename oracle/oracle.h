@@ -16,7 +16,8 @@
  *   the expected-output files of the reference's example tests (tests/golden/ref/);
  *   index operations: numpy integer-array indexing and the reference's index_008 output; find: numpy.nonzero and the
  *   reference's ocean_find_01 / tensor_find_01 outputs;  integer / bool GEMM: exact arithmetic;
- *   GEMM transposition / conjugation modes for every floating type: the reference's ocean_gemm_02 ... 09d outputs.
+ *   GEMM transposition / conjugation modes for every floating type: the reference's ocean_gemm_02 ... 09d outputs;
+ *   reductions (NaN-skipping variants, any / all / nnz along axes, p-norms): ocean_axis_* and ocean_norm_01 / 02 outputs.
  * PARITY UNPINNED (no golden vector, reference build or closed form fixes the bits; the tests
  * hold these to stated tolerances instead):
  *   oracle_gemm for floating and complex types at large sizes -- the reference's CPU result

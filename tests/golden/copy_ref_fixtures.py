@@ -26,6 +26,9 @@ OTHER = [("/root/reference/examples/python/gpu/index/index_008.ref", "index_008.
 OTHER += [("/root/reference/examples/python/cpu/tensors/%s.ref" % n, "%s_cpu.ref" % n)
           for n in ("ocean_gemm_02", "ocean_gemm_03", "ocean_gemm_07", "ocean_gemm_08a", "ocean_gemm_09a", "ocean_gemm_09b", "ocean_gemm_09c",
                     "ocean_gemm_09d", "ocean_multiply_01", "ocean_multiply_02")]
+# reductions: axis sums / products with NaN variants, all / any / nnz along axes, p-norms
+OTHER += [("/root/reference/examples/python/cpu/tensors/%s.ref" % n, "%s_cpu.ref" % n)
+          for n in ("ocean_axis_reduce_01", "ocean_axis_reduce_02", "ocean_axis_sum_01", "ocean_axis_all_01", "ocean_axis_nnz_01", "ocean_norm_01", "ocean_norm_02")]
 
 if __name__ == "__main__":
     dst = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ref")

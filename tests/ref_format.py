@@ -44,6 +44,7 @@ def parse_ref(text):
     "<scalar...>" zero-dimensional tensors with shape []), ('scalars', [values]) for lines made of values only, and
     ('text', line) for headings."""
     items, rows = [], []
+    in_slices = False
     for line in text.splitlines():
         s = line.strip()
         if not s:
@@ -64,6 +65,7 @@ def parse_ref(text):
             if len(flat) != n:                                    # large tensors are printed with rows left out
                 items.append(RefTensor(dtype, shape, None, m.group(3), bool(m.group(4))))
                 rows = []
+                in_slices = False
                 continue
             if len(shape) == 1:
                 arr = np.array(flat)
@@ -75,8 +77,14 @@ def parse_ref(text):
                 arr = np.moveaxis(a, 0, 2).reshape([d0, d1] + shape[2:], order="F")
             items.append(RefTensor(dtype, shape, arr, m.group(3), bool(m.group(4))))
             rows = []
+            in_slices = False
             continue
         if re.match(r"^\((:|\d+)(,(:|\d+))*\)$", s):
+            if rows and not in_slices:                            # value lines before the first slice header: bare scalars
+                for r in rows:
+                    items.append(("scalars", r))
+                rows = []
+            in_slices = True
             continue
         vals = parse_values(s)
         rest = _TOKEN.sub("", s).replace(">", "").strip()
