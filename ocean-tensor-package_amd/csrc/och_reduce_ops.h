@@ -47,6 +47,19 @@ template <class T> struct red_param
    double phalf, pinv;        /* p/2 and 1/p for the general norm */
 };
 
+/* Complex maximum / minimum keep the FIRST element when every element has a NaN part (reduce_ops.h:912-935: the
+   accumulator starts as the first element and only NaN-free elements replace it). A parallel reduction starts every
+   partial from an identity, so the identity must lose against any element, NaN parts included: it is a quiet NaN with
+   a payload that no arithmetic produces, recognised by its bits. */
+template <class F> OCH_D F extreme_identity()
+{  if constexpr (sizeof(F) == 4) { union { uint32_t u; float f; } c; c.u = 0x7FC0D1CEu; return c.f; }
+   else { union { uint64_t u; double f; } c; c.u = 0x7FF8D1CED1CED1CEull; return c.f; }
+}
+template <class F> OCH_D bool is_extreme_identity(F v)
+{  if constexpr (sizeof(F) == 4) { union { uint32_t u; float f; } c; c.f = v; return c.u == 0x7FC0D1CEu; }
+   else { union { uint64_t u; double f; } c; c.f = v; return c.u == 0x7FF8D1CED1CED1CEull; }
+}
+
 /* pow of the general p-norm as one out-of-line function per translation unit: inlined at every load site of every
    kernel variant it multiplies the code size and the build time of the norm kernels */
 static __device__ __noinline__ double norm_pow(double x, double y) { return pow(x, y); }
@@ -116,7 +129,7 @@ template <class T, int OP> struct Reduce
             return ISMAX ? (T)((U)1 << (sizeof(T) * 8 - 1)) : (T)(((U)1 << (sizeof(T) * 8 - 1)) - 1);
          }
          else if constexpr (is_float_v<T>) return (W)__builtin_nan("");
-         else { cwork<T> a; a.real = (elemwork_t<T>)__builtin_nan(""); a.imag = a.real; return a; }
+         else { cwork<T> a; a.real = extreme_identity<elemwork_t<T>>(); a.imag = a.real; return a; }
       }
       else   /* ABSEXT */
       {  if constexpr (is_bool_v<T>) return ISMAX ? 0 : 1;
@@ -257,7 +270,8 @@ template <class T, int OP> struct Reduce
          else { if constexpr (P) return a * b; else return a + b; }
       }
       else if constexpr (EXTREME && is_complex_v<T>)
-      {  bool take = (!isnan(b.real)) && (!isnan(b.imag)) &&
+      {  if (is_extreme_identity(a.real) && is_extreme_identity(a.imag)) return b;
+         bool take = (!isnan(b.real)) && (!isnan(b.imag)) &&
                      (ISMAX ? ((!(a.real >= b.real)) || ((!(a.real < b.real)) && (!(a.real > b.real)) && (!(a.imag >= b.imag))) || isnan(a.imag))
                             : ((!(a.real <= b.real)) || ((!(a.real < b.real)) && (!(a.real > b.real)) && (!(a.imag <= b.imag))) || isnan(a.imag)));
          return take ? b : a;

@@ -29,6 +29,13 @@ OTHER += [("/root/reference/examples/python/cpu/tensors/%s.ref" % n, "%s_cpu.ref
 # reductions: axis sums / products with NaN variants, all / any / nnz along axes, p-norms
 OTHER += [("/root/reference/examples/python/cpu/tensors/%s.ref" % n, "%s_cpu.ref" % n)
           for n in ("ocean_axis_reduce_01", "ocean_axis_reduce_02", "ocean_axis_sum_01", "ocean_axis_all_01", "ocean_axis_nnz_01", "ocean_norm_01", "ocean_norm_02")]
+# division family on operands of either sign
+OTHER += [("/root/reference/examples/python/cpu/tensors/%s.ref" % n, "%s_cpu.ref" % n)
+          for n in ("ocean_divide_01", "ocean_floordivide_01", "ocean_truedivide_01", "ocean_fmod_01")]
+# extremes with NaN and complex ordering; square root and negation over the types; integer power with a negative exponent
+OTHER += [("/root/reference/examples/python/cpu/tensors/%s.ref" % n, "%s_cpu.ref" % n)
+          for n in ("ocean_maximum_01", "ocean_minimum_01", "ocean_maximum_abs_01", "ocean_minimum_abs_01", "tensor_sqrt_01", "ocean_sqrt",
+                    "tensor_negative_01", "tensor_negative_02", "ocean_power_04")]
 
 if __name__ == "__main__":
     dst = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ref")

@@ -136,8 +136,10 @@ def from_storage(dtype, arr):
         return arr != 0
     if dtype == H.HALF:
         return half_bits_to_float(arr)
-    if dtype == H.CHALF:
-        return half_bits_to_float(arr["real"]) + 1j * half_bits_to_float(arr["imag"])
+    if dtype == H.CHALF:                                              # not real + 1j * imag: that turns a NaN imaginary part into NaN + NaNj
+        out = np.empty(np.shape(arr), np.complex128)
+        out.real, out.imag = half_bits_to_float(arr["real"]), half_bits_to_float(arr["imag"])
+        return out
     if dtype in H.COMPLEX_TYPES:
         return arr.astype(np.complex128)
     return arr.astype(np.float64)

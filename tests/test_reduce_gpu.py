@@ -201,3 +201,45 @@ def test_config3_full_reductions(hip, stream, dtype):
     _, s2 = gpu_reduce(stream, oh.R["sum"], dtype, x)
     x.free()
     H.assert_same_bytes(s, s2, "repeatability")
+
+
+@pytest.mark.parametrize("dtype", [H.CFLOAT, H.CDOUBLE, H.CHALF], ids=lambda d: H.NAMES[d])
+def test_complex_extremes_when_every_element_has_a_nan_part(hip, stream, dtype):
+    """The reference starts from the first element and lets only NaN-free elements replace it (reduce_ops.h:912-968):
+    when every element has a NaN part the result is the first element, whatever the size and the layout of the
+    reduction (many blocks, axis reductions of both kinds); one NaN-free element anywhere wins."""
+    rng = np.random.default_rng(5 + dtype)
+    n = 300001
+    re, im = rng.uniform(-5, 5, n), rng.uniform(-5, 5, n)
+    pick = rng.random(n) < 0.5
+    re[pick] = np.nan; im[~pick] = np.nan
+    def as_storage(re, im):
+        if dtype == H.CHALF:
+            out = np.empty(n, H.storage(dtype)); out["real"] = H.f32_to_half_bits(re.astype(np.float32)); out["imag"] = H.f32_to_half_bits(im.astype(np.float32))
+            return out
+        out = np.empty(n, H.storage(dtype)); out.real, out.imag = re, im
+        return out
+    for clean_at in (None, 123457):
+        r2, i2 = re.copy(), im.copy()
+        if clean_at is not None:
+            r2[clean_at], i2[clean_at] = -4.0, 2.0
+        data = as_storage(r2, i2)
+        x = H.Operand.contiguous(data, dtype).upload(stream)
+        for name in ("maximum", "minimum"):
+            _, got = gpu_reduce(stream, oh.R[name], dtype, x)
+            _, want = cpu_reduce(oh.R[name], dtype, x)
+            assert got.tobytes() == want.tobytes() == data[0 if clean_at is None else clean_at].tobytes(), (name, clean_at)
+        x.free()
+        # the same through the axis kernels: 3 rows of 100000 (cooperative kernel), 100000 columns of 3 (per-thread kernel)
+        mat = data[:300000].reshape(3, 100000)
+        for view, axes in ((mat, [1]), (mat.T, [0])):
+            src = H.Operand(mat, view, dtype).upload(stream)
+            kept = [view.shape[d] for d in range(view.ndim) if d not in axes]
+            z = np.zeros(kept, data.dtype)
+            dst = H.Operand(z, z, dtype).upload(stream)
+            zc = z.copy(); cdst = H.Operand(zc, zc, dtype)
+            for name in ("maximum", "minimum"):
+                oh.check(oh.lib.och_reduce_axis(oh.R[name], dtype, H.axis_config(src, dst, axes, stream), 0.0))
+                assert orc.lib.oracle_reduce_axis(oh.R[name], dtype, H.axis_config(src, cdst, axes, device=False), 0.0) == 0
+                assert dst.download().tobytes() == zc.tobytes(), (name, axes, clean_at)
+            src.free(); dst.free()

@@ -298,3 +298,58 @@ def test_gemm_with_empty_operands(engine):
     want = tensors(load("ocean_gemm_11"))[0]            # (5 x 0) * (0 x 5) -> 5 x 5 zeros, whatever C held before
     got = engine.gemm_raw(H.FLOAT, 5, 5, 0, np.zeros(0, np.float32), np.zeros(0, np.float32), c0=np.full(25, 7, np.float32))
     RF.assert_matches(H.FLOAT, got.reshape((5, 5), order="F"), want, "product over an empty inner dimension")
+
+
+PAIRS = [(4, 3), (4, -3), (-4, 3), (-4, -3), (-2, -3), (2, -3), (10, 5), (10, -5)]
+
+
+@pytest.mark.parametrize("name,op", [("ocean_divide_01_cpu", "divide"), ("ocean_floordivide_01_cpu", "floor_divide"), ("ocean_truedivide_01_cpu", "true_divide")])
+def test_division_of_either_sign(engine, name, op):
+    """a (op) b for the eight sign combinations the CPU example prints, in int8, half, float and double: integer `divide`
+    and `floorDivide` round towards minus infinity, integer `trueDivide` truncates (binary_ops.h:154-235)."""
+    ts = tensors(load(name))
+    assert len(ts) == 32
+    for g, (a, b) in enumerate(PAIRS):
+        for k, dt in enumerate((H.INT8, H.HALF, H.FLOAT, H.DOUBLE)):
+            rd, got = engine.binary(op, dt, RF.to_storage(dt, np.array([a])), RF.to_storage(dt, np.array([b])))
+            RF.assert_matches(rd, got, ts[4 * g + k], "%d %s %d (%s)" % (a, op, b, H.NAMES[dt]))
+
+
+def test_mod_and_fmod(engine):
+    ts = tensors(load("ocean_fmod_01_cpu"))
+    a, b = [-20, 20, -20, 20], [3, 3, -3, -3]
+    for base, op in ((0, "mod"), (4, "fmod")):           # mod takes the sign of the divisor, fmod that of the dividend
+        for k, dt in enumerate((H.INT64, H.FLOAT, H.DOUBLE)):
+            rd, got = engine.binary(op, dt, RF.to_storage(dt, np.array(a)), RF.to_storage(dt, np.array(b)))
+            RF.assert_matches(rd, got, ts[base + k], "%s %s" % (op, H.NAMES[dt]))
+            RF.assert_matches(rd, got, ts[base + 3].values, "%s: the values the example expects" % op)
+
+
+def test_sqrt_and_negative_over_types(engine):
+    ts = tensors(load("tensor_sqrt_01_cpu"))
+    assert len(ts) == 6
+    # sqrt of an integer tensor is computed in double (the interface converts first); negative reals give NaN, complex
+    # numbers their principal root; the last case stores the int8 -> double result into uint8 (NaN and fractions truncate)
+    u8 = RF.to_storage(H.UINT8, np.arange(5))
+    RF.assert_matches(H.DOUBLE, engine.unary("sqrt", H.DOUBLE, engine.cast(H.UINT8, H.DOUBLE, u8))[1], ts[0], "sqrt(uint8)")
+    lin = np.linspace(-5, 5, 11)
+    RF.assert_matches(H.DOUBLE, engine.unary("sqrt", H.DOUBLE, RF.to_storage(H.DOUBLE, lin))[1], ts[1], "sqrt(int16) in double")
+    for want, dt in zip(ts[2:5], (H.HALF, H.FLOAT, H.CDOUBLE)):
+        rd, got = engine.unary("sqrt", dt, RF.to_storage(dt, lin))
+        RF.assert_matches(rd, got, want, "sqrt %s" % H.NAMES[dt])
+    ts2 = tensors(load("ocean_sqrt_cpu"))               # arange(10) double, byte-swapped source and destination: values as above
+    rd, got = engine.unary("sqrt", H.DOUBLE, RF.to_storage(H.DOUBLE, np.arange(10.0)))
+    RF.assert_matches(rd, got, ts2[1], "sqrt(arange(10))"); RF.assert_matches(rd, got, ts2[2], "in place")
+    ts = tensors(load("tensor_negative_01_cpu"))
+    assert len(ts) == 6
+    RF.assert_matches(H.BOOL, engine.unary("negative", H.BOOL, RF.to_storage(H.BOOL, np.array([1, 0, 0])))[1], ts[0], "-bool")
+    # -uint8 is computed in int16 (the interface converts to the signed type that holds the range)
+    RF.assert_matches(H.INT16, engine.unary("negative", H.INT16, RF.to_storage(H.INT16, np.arange(5)))[1], ts[1], "-uint8 as int16")
+    for want, dt in zip(ts[2:], (H.INT16, H.HALF, H.FLOAT, H.CDOUBLE)):
+        rd, got = engine.unary("negative", dt, RF.to_storage(dt, lin))
+        RF.assert_matches(rd, got, want, "negative %s" % H.NAMES[dt])
+    want = tensors(load("tensor_negative_02_cpu"))[0]   # -(-128) wraps to -128 in int8
+    RF.assert_matches(H.INT8, engine.unary("negative", H.INT8, RF.to_storage(H.INT8, np.array([-128, -1, 0, 1, 127])))[1], want, "negative int8 extremes")
+    want = tensors(load("ocean_power_04_cpu"))[0]       # integer power with a negative exponent is 0 (binary_ops.h:238-248)
+    rd, got = power(engine, H.INT64, RF.to_storage(H.INT64, np.array([2, 3, 4])), H.INT64, RF.to_storage(H.INT64, np.array([-1])), H.INT64)
+    RF.assert_matches(rd, got, want, "[2, 3, 4] ** -1")

@@ -122,3 +122,31 @@ def test_norm_02(engine):
     assert tail == [5.0, 5.0] or len(tail) == 2
     rd, got = engine.reduce("nnz", H.DOUBLE, a); assert got[0] == tail[0]
     rd, got = engine.reduce("nnz_nan", H.DOUBLE, a); assert got[0] == tail[1]
+
+
+NAN = float("nan")
+
+
+@pytest.mark.parametrize("name,op,y,cases", [
+    ("ocean_maximum_01_cpu", "maximum", complex(3, NAN),
+     [[NAN, 2], [1, NAN, 2], [2, NAN, 1], ["x", 2 + 1j], ["y", 1 + 2j], ["y", 1 + 3j], ["y", 1 + 4j], ["x", "y"], ["y", "x"],
+      [1 + 1j, 2 + 0j], [1 + 1j, 2 + 1j], [1 + 1j, 2 + 2j], [1 + 1j, 1 + 0j], [1 + 2j, 1 + 2j], [1 + 2j, 1 + 3j]]),
+    ("ocean_minimum_01_cpu", "minimum", complex(1, NAN),
+     [[NAN, 2], [1, NAN, 2], [2, NAN, 1], ["x", 2 + 1j], ["y", 0 + 2j], ["y", 1 + 3j], ["y", 2 + 4j], ["x", "y"], ["y", "x"],
+      [2 + 1j, 1 + 0j], [2 + 1j, 1 + 1j], [2 + 1j, 1 + 2j], [1 + 1j, 1 + 2j], [1 + 2j, 1 + 2j], [1 + 4j, 1 + 3j]]),
+    ("ocean_maximum_abs_01_cpu", "maximum_abs", complex(1, NAN),
+     [[NAN, 2], [1, NAN, 2], [-2, NAN, 1], ["x", 3 + 4j], ["y", 0 + 2j], ["x", "y"], [3 + 4j, 1 + 0j], [1 + 0j, 3 + 4j]]),
+    ("ocean_minimum_abs_01_cpu", "minimum_abs", complex(1, NAN),
+     [[NAN, 2], [1, NAN, 2], [-2, NAN, 1], ["x", 3 + 4j], ["y", 0 + 2j], ["x", "y"], [3 + 4j, 1 + 0j], [1 + 0j, 3 + 4j]])])
+def test_extremes_with_nan_and_complex_order(engine, name, op, y, cases):
+    """maximum / minimum (and of absolute values) over half vectors with NaN (NaN is skipped) and over complex-half vectors
+    (ordered by real part, then imaginary part; an element with a NaN part never wins unless nothing else is there).
+    x = NaN + 1j, y as given; the first three cases of each file are real (half), the others complex-half."""
+    vals = scalars(load(name))
+    assert len(vals) == len(cases)
+    x = complex(NAN, 1)
+    for k, (case, want) in enumerate(zip(cases, vals)):
+        dt = H.HALF if k < 3 else H.CHALF
+        data = np.array([x if v == "x" else y if v == "y" else v for v in case], dtype=np.complex128)
+        rd, got = engine.reduce(op, dt, RF.to_storage(dt, data))
+        RF.assert_matches(rd, got, np.array([want]), "%s %s" % (op, case))
