@@ -112,8 +112,7 @@ int och_event_elapsed_ms(och_event start, och_event stop, float *ms);
 /* that synchronise or allocate may not be recorded: och_reduce_all, och_find_count, och_memcpy_htod / dtoh,        */
 /* och_malloc_async / och_free_async, och_copy between tensors of different shape AND type. Everything else in this */
 /* header is recordable; scalars passed in host memory are frozen at their recorded value, scalars in device memory */
-/* are read at every replay. `stream` must be a created stream; call och_device_warmup on the device beforehand     */
-/* (it creates the per-device scratch of the reductions).                                                           */
+/* are read at every replay. `stream` must be a created stream.                                                     */
 typedef void *och_graph;
 int och_stream_begin_capture(och_stream stream);
 int och_stream_end_capture(och_stream stream, och_graph *graph);

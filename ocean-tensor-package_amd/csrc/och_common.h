@@ -28,7 +28,22 @@ void clear_error();
 static inline hipStream_t as_stream(och_stream s) { return (hipStream_t)s; }
 /* byte fill by a kernel (och_runtime.hip): unlike a memset node it is safe inside a captured graph */
 int fill_bytes(void *dst, int value, size_t nbytes, hipStream_t stream);
-/* creates the current device's reduction scratch and pinned result slot if they do not exist yet (och_reduce.hip) */
-int red_context_init();
+
+/* Scratch memory that kernels of one stream share: work on one stream is ordered, work on different streams is not
+   (Ocean gives every storage its own stream), so every (device, stream) pair owns its scratch. It is created on the
+   first use of the stream -- or by och_device_warmup / och_stream_begin_capture, so that no allocation happens while
+   a stream records -- and released when the stream is destroyed. */
+#define OCH_RED_MAX_BLOCKS 512
+#define OCH_RED_SLOT 16                               /* bytes per partial of a full reduction */
+#define OCH_RED_SCRATCH (OCH_RED_MAX_BLOCKS * OCH_RED_SLOT + 256)
+#define OCH_GEMM_WORKSPACE (16u << 20)                /* partial products of the split-K matrix-vector kernels */
+struct StreamContext
+{  char *red_scratch;          /* OCH_RED_SCRATCH bytes, partial slots + ticket counter (zero between launches) */
+   void *host_result;          /* 64 bytes of pinned host memory: result of a full reduction */
+   char *gemm_workspace;       /* OCH_GEMM_WORKSPACE bytes, created by stream_gemm_workspace */
+};
+int stream_context(hipStream_t stream, StreamContext **ctx);
+int stream_gemm_workspace(hipStream_t stream, char **workspace);
+void stream_context_release(hipStream_t stream);
 
 } /* namespace och */

@@ -18,6 +18,7 @@
 #pragma once
 #include "och_common.h"
 #include "och_dtypes.h"
+#include "och_gemv.h"
 #include <string.h>
 
 namespace och {
@@ -399,6 +400,25 @@ static int launch_gemm_mfma(const GemmArgs &g)
       hipLaunchKernelGGL((gemm_outer_kernel<R, CPLX>), dim3((unsigned)(((uint64_t)g.M * g.N + 255) / 256), 1, g.nz), dim3(256), 0, g.stream, p, sAm, sAk, sBk, sBn);
       OCH_CHECK_LAUNCH();
       return 0;
+   }
+   if (g.batch.nb == 0 && (g.N <= OCH_GEMV_MAX_S || g.M <= OCH_GEMV_MAX_S) && (g.M >= 64 || g.N >= 64))
+   {  /* one very small dimension: stream the large operand once (och_gemv.h) */
+      const int64_t sAm = akc ? g.ldA : 1, sAk = akc ? 1 : g.ldA, sBk = bkc ? 1 : g.ldB, sBn = bkc ? g.ldB : 1;
+      GemvParams<R> v;
+      memset(&v, 0, sizeof(v));
+      if (g.N <= g.M)
+      {  v.X = (const R *)g.A; v.sXr = sAm; v.sXk = sAk; v.conjX = p.conjA; v.Y = (const R *)g.B; v.sYk = sBk; v.sYs = sBn; v.conjY = p.conjB;
+         v.O = (R *)g.C; v.sOr = 1; v.sOs = g.ldC; v.rows = (uint32_t)g.M; v.S = (uint32_t)g.N;
+      }
+      else
+      {  v.X = (const R *)g.B; v.sXr = sBn; v.sXk = sBk; v.conjX = p.conjB; v.Y = (const R *)g.A; v.sYk = sAk; v.sYs = sAm; v.conjY = p.conjA;
+         v.O = (R *)g.C; v.sOr = g.ldC; v.sOs = 1; v.rows = (uint32_t)g.N; v.S = (uint32_t)g.M;
+      }
+      v.K = (uint32_t)g.K;
+      memcpy(v.alpha, p.alpha, sizeof(v.alpha)); memcpy(v.beta, p.beta, sizeof(v.beta));
+      v.alpha_dev = p.alpha_dev; v.beta_dev = p.beta_dev;
+      const int status = launch_gemv<R, CPLX>(v, g.stream);
+      if (status != 0) return status < 0 ? -1 : 0;
    }
    p.tiles_m = (uint32_t)((g.M + BM - 1) / BM); p.tiles_n = (uint32_t)((g.N + BN - 1) / BN);
    const uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;

@@ -1,7 +1,6 @@
-/* C ABI of the full reductions (och_reduce_all and its queries) and the per-device
- * scratch they use when the caller supplies none. */
+/* C ABI of the full reductions (och_reduce_all and its queries). Without a caller's buffer they use the scratch of
+ * the stream they run on. */
 #include "och_reduce_all.h"
-#include <mutex>
 #include <string.h>
 
 namespace och {
@@ -23,29 +22,6 @@ static red_fn reduce_lookup(int op, int dtype)
    return fn;
 }
 
-#define OCH_MAX_DEVICES 64
-static RedContext g_ctx[OCH_MAX_DEVICES];
-static bool g_ctx_ready[OCH_MAX_DEVICES];
-static std::mutex g_ctx_mutex;
-
-int red_context(RedContext **out)
-{
-   int dev;
-   OCH_CHECK_HIP(hipGetDevice(&dev));
-   if (dev < 0 || dev >= OCH_MAX_DEVICES) return set_error("device index %d out of range", dev);
-   std::lock_guard<std::mutex> lock(g_ctx_mutex);
-   if (!g_ctx_ready[dev])
-   {  void *scratch = nullptr, *host = nullptr;
-      OCH_CHECK_HIP(hipMalloc(&scratch, OCH_RED_SCRATCH));
-      OCH_CHECK_HIP(hipMemset(scratch, 0, OCH_RED_SCRATCH));
-      OCH_CHECK_HIP(hipHostMalloc(&host, 64, hipHostMallocDefault));
-      g_ctx[dev].scratch = (char *)scratch; g_ctx[dev].host_result = host;
-      g_ctx_ready[dev] = true;
-   }
-   *out = &g_ctx[dev];
-   return 0;
-}
-int red_context_init() { RedContext *ctx; return red_context(&ctx); }
 }  /* namespace och */
 
 using namespace och;
@@ -76,9 +52,9 @@ extern "C" int och_reduce_all_device(int op, int dtype, int ndims, const size_t 
    if (fn == nullptr) return set_error("reduction %d is not available for data type %d", op, dtype);
    char *scratch = (char *)buffer;
    if (scratch == nullptr)
-   {  RedContext *ctx;
-      if (red_context(&ctx) != 0) return -1;
-      scratch = ctx->scratch;
+   {  StreamContext *ctx;
+      if (stream_context(as_stream(stream), &ctx) != 0) return -1;
+      scratch = ctx->red_scratch;
    }
    return fn(ndims, size, strides, ptr, param1, param2, p, dresult, scratch, buffer != nullptr, as_stream(stream));
 }
@@ -87,8 +63,8 @@ extern "C" int och_reduce_all(int op, int dtype, int ndims, const size_t *size, 
                    void *ptr, const och_scalar *param1, const och_scalar *param2, double p,
                    void *result, void *buffer, och_stream stream)
 {
-   RedContext *ctx;
-   if (red_context(&ctx) != 0) return -1;
+   StreamContext *ctx;
+   if (stream_context(as_stream(stream), &ctx) != 0) return -1;
    /* the kernel writes the scalar straight into pinned host memory; one synchronisation */
    if (och_reduce_all_device(op, dtype, ndims, size, strides, ptr, param1, param2, p, ctx->host_result, buffer, stream) != 0) return -1;
    OCH_CHECK_HIP(hipStreamSynchronize(as_stream(stream)));

@@ -25,9 +25,6 @@ namespace och {
 
 #define OCH_RED_BLOCK 256
 #define OCH_RED_UNR 4
-#define OCH_RED_MAX_BLOCKS 512
-#define OCH_RED_SLOT 16                               /* bytes per partial */
-#define OCH_RED_SCRATCH (OCH_RED_MAX_BLOCKS * OCH_RED_SLOT + 256)
 
 template <class A> OCH_D A shfl_xor_any(A v, int mask)
 {
@@ -158,9 +155,6 @@ __global__ __launch_bounds__(OCH_RED_BLOCK) void reduce_all_kernel(const RedPara
    }
 }
 
-/* per-device scratch and pinned result slot used when the caller passes no buffer */
-struct RedContext { char *scratch; void *host_result; };
-int red_context(RedContext **ctx);
 
 typedef int (*red_fn)(int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr,
                       const och_scalar *b1, const och_scalar *b2, double pnorm,

@@ -5,6 +5,9 @@
  * stream-ordered allocation from the device's default memory pool. */
 #include "och_common.h"
 #include <string.h>
+#include <map>
+#include <mutex>
+#include <utility>
 
 namespace och {
 static thread_local char g_errmsg[512] = "";
@@ -18,6 +21,54 @@ __global__ void warmup_kernel(int *p) { if (p) *p = 1; }
 }
 
 namespace och {
+static std::map<std::pair<int, hipStream_t>, StreamContext> g_stream_ctx;
+static std::mutex g_stream_ctx_mutex;
+
+int stream_context(hipStream_t stream, StreamContext **out)
+{
+   int dev;
+   OCH_CHECK_HIP(hipGetDevice(&dev));
+   std::lock_guard<std::mutex> lock(g_stream_ctx_mutex);
+   auto key = std::make_pair(dev, stream);
+   auto it = g_stream_ctx.find(key);
+   if (it == g_stream_ctx.end())
+   {  StreamContext c = { nullptr, nullptr, nullptr };
+      void *scratch = nullptr, *host = nullptr;
+      OCH_CHECK_HIP(hipMalloc(&scratch, OCH_RED_SCRATCH));
+      hipError_t e = hipMemset(scratch, 0, OCH_RED_SCRATCH);
+      if (e == hipSuccess) e = hipHostMalloc(&host, 64, hipHostMallocDefault);
+      if (e != hipSuccess) { (void)hipFree(scratch); return set_error("stream scratch: %s", hipGetErrorString(e)); }
+      c.red_scratch = (char *)scratch; c.host_result = host;
+      it = g_stream_ctx.insert(std::make_pair(key, c)).first;
+   }
+   *out = &it->second;                 /* std::map nodes stay where they are when other streams are added */
+   return 0;
+}
+int stream_gemm_workspace(hipStream_t stream, char **workspace)
+{
+   StreamContext *c;
+   if (stream_context(stream, &c) != 0) return -1;
+   std::lock_guard<std::mutex> lock(g_stream_ctx_mutex);
+   if (c->gemm_workspace == nullptr)
+   {  void *w = nullptr;
+      OCH_CHECK_HIP(hipMalloc(&w, OCH_GEMM_WORKSPACE));
+      c->gemm_workspace = (char *)w;
+   }
+   *workspace = c->gemm_workspace;
+   return 0;
+}
+void stream_context_release(hipStream_t stream)
+{
+   int dev;
+   if (hipGetDevice(&dev) != hipSuccess) return;
+   std::lock_guard<std::mutex> lock(g_stream_ctx_mutex);
+   auto it = g_stream_ctx.find(std::make_pair(dev, stream));
+   if (it == g_stream_ctx.end()) return;
+   (void)hipFree(it->second.red_scratch); (void)hipHostFree(it->second.host_result);
+   if (it->second.gemm_workspace) (void)hipFree(it->second.gemm_workspace);
+   g_stream_ctx.erase(it);
+}
+
 typedef unsigned int fill_u32x4 __attribute__((ext_vector_type(4)));
 /* 16-byte stores over the aligned body (grid-stride), single bytes for the unaligned head and tail (first block) */
 __global__ __launch_bounds__(256) void fill_bytes_kernel(unsigned char *dst, unsigned int pattern, size_t head, size_t body, size_t tail)
@@ -97,7 +148,8 @@ int och_device_warmup(int device)
    hipLaunchKernelGGL(och::warmup_kernel, dim3(1), dim3(1), 0, 0, (int *)nullptr);
    OCH_CHECK_LAUNCH();
    OCH_CHECK_HIP(hipDeviceSynchronize());
-   const int status = och::red_context_init();      /* the reductions' per-device scratch: allocated here, not in a later (possibly recorded) call */
+   och::StreamContext *ctx;
+   const int status = och::stream_context(nullptr, &ctx);        /* scratch of the default stream */
    OCH_CHECK_HIP(hipSetDevice(prev));
    return status;
 }
@@ -109,7 +161,12 @@ int och_stream_create(och_stream *stream)
    OCH_CHECK_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
    *stream = (och_stream)s; return 0;
 }
-int och_stream_destroy(och_stream stream) { OCH_CHECK_HIP(hipStreamDestroy((hipStream_t)stream)); return 0; }
+int och_stream_destroy(och_stream stream)
+{  OCH_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));      /* its scratch may still be in use */
+   och::stream_context_release((hipStream_t)stream);
+   OCH_CHECK_HIP(hipStreamDestroy((hipStream_t)stream));
+   return 0;
+}
 int och_stream_synchronize(och_stream stream) { OCH_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream)); return 0; }
 int och_stream_wait_event(och_stream stream, och_event event)
 {  OCH_CHECK_HIP(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0)); return 0; }
@@ -129,6 +186,8 @@ int och_event_elapsed_ms(och_event start, och_event stop, float *ms)
 
 int och_stream_begin_capture(och_stream stream)
 {  if (stream == nullptr) return och::set_error("the default stream cannot record a graph");
+   char *workspace;                                    /* allocate the stream's scratch now: nothing may be allocated while it records */
+   if (och::stream_gemm_workspace((hipStream_t)stream, &workspace) != 0) return -1;
    OCH_CHECK_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
    return 0;
 }

@@ -290,3 +290,21 @@ def test_gemm_batched_equals_loop(hip, stream, case):
     assert not np.array_equal(got, C0)
     for b in (dA, dB, dC1, dC2):
         b.free()
+
+
+SKINNY = [(300, 1, 500), (1, 300, 500), (1000, 3, 70), (5, 2000, 33), (4100, 8, 129), (2050, 1, 4099), (8, 4097, 513), (66, 7, 5), (4096, 2, 64)]
+
+
+@pytest.mark.parametrize("dtype", [H.FLOAT, H.DOUBLE, H.CFLOAT, H.CDOUBLE], ids=lambda d: H.NAMES[d])
+def test_gemm_with_one_small_dimension(hip, stream, dtype):
+    """Matrix x vector and matrix x few-columns products (and their transposes) take the streaming kernels: rows
+    contiguous (split over K, partial results in the stream's workspace) or K contiguous (lanes share a row). Every mode
+    pair, unaligned leading dimensions (pad = 3) and aligned ones, host and device scalars, beta != 0."""
+    rng = np.random.default_rng(700 + dtype)
+    cplx = dtype in H.COMPLEX_TYPES
+    modes = ["N", "T"] + (["C"] if cplx else [])
+    for (M, N, K) in SKINNY:
+        for ta in modes:
+            for tb in modes:
+                alpha, beta = ((2 - 1j, -1 + 0.5j) if cplx else (2, -1)) if (M + K + len(ta)) % 2 else (1, 0)
+                run_case(stream, dtype, ta, tb, M, N, K, alpha, beta, rng, device_scalars=(N % 2 == 0), pad=3 if (K % 2) else 0)

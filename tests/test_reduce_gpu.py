@@ -243,3 +243,30 @@ def test_complex_extremes_when_every_element_has_a_nan_part(hip, stream, dtype):
                 assert orc.lib.oracle_reduce_axis(oh.R[name], dtype, H.axis_config(src, cdst, axes, device=False), 0.0) == 0
                 assert dst.download().tobytes() == zc.tobytes(), (name, axes, clean_at)
             src.free(); dst.free()
+
+
+def test_reductions_on_two_streams_do_not_share_scratch(hip, stream):
+    """Ocean gives every storage its own stream, so full reductions of different tensors run concurrently; the partial
+    results and the ticket counter they use belong to the stream. Two streams reduce different data back to back, many
+    times, without synchronisation in between; every result must equal the one computed alone."""
+    rng = np.random.default_rng(77)
+    other = oh.Stream()
+    n = 1 << 21
+    xs = [rng.integers(-1000, 1000, n).astype(np.int64), rng.integers(-1000, 1000, n).astype(np.int64)]
+    streams = [stream, other]
+    bufs = [oh.to_device(x, s) for x, s in zip(xs, streams)]
+    reps = 40
+    outs = [oh.DeviceBuffer(8 * reps, s) for s in streams]
+    for s in streams:
+        s.synchronize()
+    for r in range(reps):
+        for k in (0, 1):
+            oh.check(oh.lib.och_reduce_all_device(oh.R["sum"], H.INT64, 1, oh.sizes([n - r]), oh.strides([8]), bufs[k].ptr, None, None, 0.0,
+                                                  C.c_void_p(outs[k].address + 8 * r), None, streams[k].handle))
+    for k in (0, 1):
+        got = outs[k].download(np.int64, reps)
+        want = np.array([xs[k][:n - r].sum() for r in range(reps)])
+        assert np.array_equal(got, want), "stream %d" % k
+    for b in bufs + outs:
+        b.free()
+    other.synchronize(); other.destroy()
