@@ -76,6 +76,11 @@ template <class R> struct GemmParams
    int      alignedA, alignedB;        /* base pointer and leading dimension allow 128-bit loads */
    uint32_t tiles_m, tiles_n;
    GemmBatch batch;
+   /* split K (few tiles, long K; only without a batch): grid z is the slice, every slice covers split_slabs slabs of K and
+      leaves its raw sums in partial[z] (dense M x N planes, complex: real plane then imaginary plane); gemm_split_finish
+      adds the slices in order and applies alpha / beta */
+   uint32_t split_slabs;
+   R       *partial;
 };
 
 #define OCH_GEMM_THREADS 256
@@ -175,10 +180,14 @@ __global__ __launch_bounds__(OCH_GEMM_THREADS, 2) void gemm_mfma_kernel(const Ge
 
    SlabLoader<R, CPLX, AKC, EDGE, BM, KT> la;
    SlabLoader<R, CPLX, BKC, EDGE, BN, KT> lb;
-   const uint32_t nslabs = (p.K + KT - 1) / KT;
+   uint32_t slab0 = 0, nslabs = (p.K + KT - 1) / KT;
+   if (p.split_slabs)
+   {  slab0 = blockIdx.z * p.split_slabs;
+      nslabs = (slab0 + p.split_slabs < nslabs) ? p.split_slabs : (slab0 < nslabs ? nslabs - slab0 : 0);
+   }
    if (nslabs > 0)
-   {  la.fetch(pA, p.ldA, m0, 0, p.M, p.K, p.alignedA);
-      lb.fetch(pB, p.ldB, n0, 0, p.N, p.K, p.alignedB);
+   {  la.fetch(pA, p.ldA, m0, slab0 * KT, p.M, p.K, p.alignedA);
+      lb.fetch(pB, p.ldB, n0, slab0 * KT, p.N, p.K, p.alignedB);
       la.stash(lds, PA, p.conjA);
       lb.stash(lds + NPL * KT * PA, PB, p.conjB);
    }
@@ -187,8 +196,8 @@ __global__ __launch_bounds__(OCH_GEMM_THREADS, 2) void gemm_mfma_kernel(const Ge
    {  const R *As = lds + (s & 1) * BUF, *Bs = As + NPL * KT * PA;
       const bool more = s + 1 < nslabs;
       if (more)
-      {  la.fetch(pA, p.ldA, m0, (s + 1) * KT, p.M, p.K, p.alignedA);
-         lb.fetch(pB, p.ldB, n0, (s + 1) * KT, p.N, p.K, p.alignedB);
+      {  la.fetch(pA, p.ldA, m0, (slab0 + s + 1) * KT, p.M, p.K, p.alignedA);
+         lb.fetch(pB, p.ldB, n0, (slab0 + s + 1) * KT, p.N, p.K, p.alignedB);
       }
 #pragma unroll
       for (int ks = 0; ks < KT / TK; ks++)
@@ -224,6 +233,25 @@ __global__ __launch_bounds__(OCH_GEMM_THREADS, 2) void gemm_mfma_kernel(const Ge
       __syncthreads();
    }
 
+   if (p.split_slabs)
+   {  /* raw sums of this K slice */
+      R *plane = p.partial + (size_t)blockIdx.z * NPL * p.M * p.N;
+#pragma unroll
+      for (int i = 0; i < TMS; i++)
+#pragma unroll
+         for (int j = 0; j < TNS; j++)
+         {  const uint32_t col = n0 + wn + j * T + lane % T;
+#pragma unroll
+            for (int r = 0; r < MM::NACC; r++)
+            {  const uint32_t row = m0 + wm + i * T + MM::acc_row(lane, r);
+               if (row >= p.M || col >= p.N) continue;
+               plane[(size_t)col * p.M + row] = acc[i][j][r];
+               if (CPLX) plane[(size_t)p.M * p.N + (size_t)col * p.M + row] = acci[i][j][r];
+            }
+         }
+      return;
+   }
+
    /* epilogue */
    R alr = p.alpha[0], ali = p.alpha[1], ber = p.beta[0], bei = p.beta[1];
    if (p.alpha_dev) { const R *q = reinterpret_cast<const R *>(reinterpret_cast<const char *>(p.alpha_dev) + oAlpha); alr = q[0]; if (CPLX) ali = q[1]; }
@@ -252,6 +280,40 @@ __global__ __launch_bounds__(OCH_GEMM_THREADS, 2) void gemm_mfma_kernel(const Ge
             }
          }
       }
+}
+
+/* adds the K slices of a split product in slice order and applies alpha / beta: one thread per element of C */
+template <class R, bool CPLX>
+__global__ __launch_bounds__(256) void gemm_split_finish_kernel(const GemmParams<R> p, uint32_t slices)
+{
+   constexpr int NPL = CPLX ? 2 : 1;
+   const uint64_t e = (uint64_t)blockIdx.x * 256 + threadIdx.x, mn = (uint64_t)p.M * p.N;
+   if (e >= mn) return;
+   const uint32_t col = (uint32_t)(e / p.M), row = (uint32_t)(e - (uint64_t)col * p.M);
+   R sr = 0, si = 0;
+   uint32_t t = 0;
+   for (; t + 7 < slices; t += 8)
+   {  R vr[8], vi[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) { vr[u] = p.partial[(size_t)(t + u) * NPL * mn + e]; if (CPLX) vi[u] = p.partial[(size_t)(t + u) * NPL * mn + mn + e]; }
+#pragma unroll
+      for (int u = 0; u < 8; u++) { sr += vr[u]; if (CPLX) si += vi[u]; }
+   }
+   for (; t < slices; t++) { sr += p.partial[(size_t)t * NPL * mn + e]; if (CPLX) si += p.partial[(size_t)t * NPL * mn + mn + e]; }
+   R alr = p.alpha[0], ali = p.alpha[1], ber = p.beta[0], bei = p.beta[1];
+   if (p.alpha_dev) { alr = p.alpha_dev[0]; if (CPLX) ali = p.alpha_dev[1]; }
+   if (p.beta_dev)  { ber = p.beta_dev[0];  if (CPLX) bei = p.beta_dev[1]; }
+   R *c = reinterpret_cast<R *>(p.C) + ((int64_t)row + (int64_t)col * p.ldC) * NPL;
+   if (!CPLX)
+   {  R v = alr * sr;
+      if (ber != 0) v += ber * c[0];
+      c[0] = v;
+   }
+   else
+   {  R vr = alr * sr - ali * si, vi = alr * si + ali * sr;
+      if (ber != 0 || bei != 0) { const R cr = c[0], ci = c[1]; vr += ber * cr - bei * ci; vi += ber * ci + bei * cr; }
+      c[0] = vr; c[1] = vi;
+   }
 }
 
 /* Few outputs (dot products, tiny C): one block per element of C strides over K. Accumulates
@@ -430,7 +492,26 @@ static int launch_gemm_mfma(const GemmArgs &g)
    };
    p.alignedA = aligned(g.A, g.ldA, g.batch.sA) ? 1 : 0; p.alignedB = aligned(g.B, g.ldB, g.batch.sB) ? 1 : 0;
    const bool edge = !(g.M % BM == 0 && g.N % BN == 0 && g.K % KT == 0 && p.alignedA && p.alignedB);
-   const dim3 grid((unsigned)blocks, 1, g.nz), block(OCH_GEMM_THREADS);
+   /* few tiles and a long K: slices of K in grid z, at least 16 slabs each, about 512 blocks in all, partial sums within the workspace */
+   uint32_t slices = 1;
+   {  const uint64_t nslabs = (g.K + KT - 1) / KT;
+      if (g.batch.nb == 0 && blocks < 128 && nslabs >= 64)
+      {  uint64_t want = (512 + blocks - 1) / blocks;
+         if (want > nslabs / 16) want = nslabs / 16;
+         const uint64_t fit = OCH_GEMM_WORKSPACE / ((uint64_t)g.M * g.N * ES);
+         if (want > fit) want = fit;
+         if (want > 65535) want = 65535;
+         if (want >= 2)
+         {  char *ws;
+            if (stream_gemm_workspace(g.stream, &ws) != 0) return -1;
+            p.split_slabs = (uint32_t)((nslabs + want - 1) / want);
+            slices = (uint32_t)((nslabs + p.split_slabs - 1) / p.split_slabs);
+            p.partial = reinterpret_cast<R *>(ws);
+            if (slices < 2) { slices = 1; p.split_slabs = 0; p.partial = nullptr; }
+         }
+      }
+   }
+   const dim3 grid((unsigned)blocks, 1, slices > 1 ? slices : g.nz), block(OCH_GEMM_THREADS);
 #define OCH_GEMM_LAUNCH(AK, BK)                                                                             \
    do { if (edge) hipLaunchKernelGGL((gemm_mfma_kernel<R, CPLX, AK, BK, true, WM, WN, KT>), grid, block, 0, g.stream, p);  \
         else      hipLaunchKernelGGL((gemm_mfma_kernel<R, CPLX, AK, BK, false, WM, WN, KT>), grid, block, 0, g.stream, p); } while (0)
@@ -439,8 +520,17 @@ static int launch_gemm_mfma(const GemmArgs &g)
    else if (!bkc)    OCH_GEMM_LAUNCH(true, false);
    else              OCH_GEMM_LAUNCH(true, true);
 #undef OCH_GEMM_LAUNCH
+   if (slices > 1)
+      hipLaunchKernelGGL((gemm_split_finish_kernel<R, CPLX>), dim3((unsigned)(((uint64_t)g.M * g.N + 255) / 256)), dim3(256), 0, g.stream, p, slices);
    OCH_CHECK_LAUNCH();
    return 0;
+}
+
+/* fewer block tiles than one and a half per compute unit of an MI355X (256 CUs): the large tile would leave most of
+   the device idle (1024^3 double: 64 tiles, 13.8 TFLOP/s) */
+static inline bool gemm_few_tiles(const GemmArgs &g, int bm, int bn)
+{  const uint64_t tiles = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * (uint64_t)g.nz;
+   return tiles < 384;
 }
 
 int gemm_float(const GemmArgs &g);

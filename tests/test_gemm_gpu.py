@@ -308,3 +308,18 @@ def test_gemm_with_one_small_dimension(hip, stream, dtype):
             for tb in modes:
                 alpha, beta = ((2 - 1j, -1 + 0.5j) if cplx else (2, -1)) if (M + K + len(ta)) % 2 else (1, 0)
                 run_case(stream, dtype, ta, tb, M, N, K, alpha, beta, rng, device_scalars=(N % 2 == 0), pad=3 if (K % 2) else 0)
+
+
+LONG_K = [(128, 128, 20000), (100, 70, 5003), (64, 200, 9000), (9, 9, 70000), (256, 130, 4096)]
+
+
+@pytest.mark.parametrize("dtype", [H.FLOAT, H.DOUBLE, H.CFLOAT, H.CDOUBLE], ids=lambda d: H.NAMES[d])
+def test_gemm_with_few_tiles_and_long_k(hip, stream, dtype):
+    """Products with few output tiles and a long inner dimension are split over K: every slice leaves raw sums in the
+    stream's workspace and a second kernel adds them in slice order and applies alpha / beta (beta != 0 included)."""
+    rng = np.random.default_rng(800 + dtype)
+    cplx = dtype in H.COMPLEX_TYPES
+    for (M, N, K) in LONG_K:
+        for ta, tb in (("N", "N"), ("T", "N"), ("N", "T"), ("C" if cplx else "T", "C" if cplx else "T")):
+            alpha, beta = ((2 - 1j, -1 + 0.5j) if cplx else (2, -1)) if (M + len(ta)) % 2 else (1, 0)
+            run_case(stream, dtype, ta, tb, M, N, K, alpha, beta, rng, device_scalars=(K % 2 == 0), pad=3 if (K % 2) else 0)
