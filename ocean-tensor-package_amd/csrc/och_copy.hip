@@ -98,6 +98,12 @@ static int copy_impl(int ts, int td, int swap,
                      int nd2, const size_t *size2, const ptrdiff_t *st2, void *p2, hipStream_t stream)
 {
    if (!dtype_ok(ts) || !dtype_ok(td)) return set_error("invalid data type (%d, %d)", ts, td);
+   {  /* equal shapes: the elementwise engine merges the dimensions of both sides together (merging each side on its own
+         would give a transposed source and a dense destination different shapes and send them down the reshape path) */
+      bool same = (nd1 == nd2) && nd1 >= 0 && nd1 <= OCH_MAX_DIMS;
+      for (int d = 0; d < nd1 && same; d++) same = (size1[d] == size2[d]);
+      if (same) return copy_lookup(ts, td, swap)(nd1, size1, st1, p1, st2, p2, stream);
+   }
    Side a, b;
    if (side_normalize(a, nd1, size1, st1) != 0 || side_normalize(b, nd2, size2, st2) != 0) return -1;
    if (a.nelem != b.nelem) return set_error("copy: element counts differ (%llu, %llu)", (unsigned long long)a.nelem, (unsigned long long)b.nelem);
