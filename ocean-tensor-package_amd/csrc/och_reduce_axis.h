@@ -22,6 +22,13 @@ struct AxisParams
    int      nd, rd;
    FastDiv  div[OCH_MAX_DIMS], rdiv[OCH_MAX_DIMS];
    uint32_t glanes;                              /* lanes per output in the wave-cooperative kernel */
+   uint32_t opb;                                 /* output groups per block in the sharing per-thread kernel */
+   /* few outputs, long reduced range: grid y cuts the reduced range into `slices` pieces of slice_len (rows of the
+      reduced range when slice_rows is set, else positions along its first dimension; the cooperative kernels count in
+      loads); every piece leaves its accumulator in partials[slice][output] (16-byte slots) and axis_finish_kernel
+      folds the pieces in order */
+   uint32_t slices, slice_len; int slice_rows;
+   char    *partials;
    FastDiv  rgdiv;                               /* 128-bit groups per row of the first reduced dimension (cooperative kernels) */
    int64_t  st1[OCH_MAX_DIMS], st2[OCH_MAX_DIMS], rst[OCH_MAX_DIMS];
    uint32_t nout, relem, rsize0, rrows;          /* relem = rsize0 * rrows */
@@ -66,7 +73,10 @@ template <class RD, class T, int SPLIT, int VEC, bool NT = false>
 __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, const typename RD::Param prm)
 {
    typedef typename RD::Acc Acc;
-   constexpr int OPB = 256 / SPLIT;                 /* output groups per block */
+   /* output groups per block: 256 without sharing; with sharing p.opb (a power of two, at most 64: fewer when there are
+      fewer groups, so that the lanes of a wave still read neighbouring memory), the other 256 / p.opb threads of a group
+      being its slices */
+   const uint32_t OPB = (SPLIT > 1) ? p.opb : 256u, NSL = 256u / OPB;
    constexpr int UNR = (VEC > 1) ? 4 : 8;
    __shared__ Acc lds[SPLIT > 1 ? 256 * VEC : 1];
    const uint32_t slice = threadIdx.x / OPB, ol = threadIdx.x % OPB;
@@ -80,19 +90,25 @@ __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, co
    {  axis_outer_offsets(p, o, o1, o2);
       const char *base = p.src + o1;
       const int64_t s0 = p.rst[0];
-      for (uint32_t r = 0; r < p.rrows; r++)
+      uint32_t r_lo = 0, r_hi = p.rrows, i_lo = 0, i_hi = p.rsize0;
+      if (p.slices > 1)
+      {  const uint32_t a = blockIdx.y * p.slice_len;
+         if (p.slice_rows) { r_lo = a; r_hi = (a + p.slice_len < p.rrows) ? a + p.slice_len : p.rrows; }
+         else { i_lo = a; i_hi = (a + p.slice_len < p.rsize0) ? a + p.slice_len : p.rsize0; }
+      }
+      for (uint32_t r = r_lo; r < r_hi; r++)
       {  const char *row = base + ((p.rd > 1) ? axis_row_offset(p, r) : 0);
-         uint32_t i = slice;
-         for (; i + (UNR - 1) * SPLIT < p.rsize0; i += UNR * SPLIT)
+         uint32_t i = i_lo + slice;
+         for (; i + (UNR - 1) * NSL < i_hi; i += UNR * NSL)
          {  Pack<T, VEC> v[UNR];
 #pragma unroll
-            for (int u = 0; u < UNR; u++) load_wide<T, VEC, NT>(v[u], row + (int64_t)(i + u * SPLIT) * s0);
+            for (int u = 0; u < UNR; u++) load_wide<T, VEC, NT>(v[u], row + (int64_t)(i + u * NSL) * s0);
 #pragma unroll
             for (int u = 0; u < UNR; u++)
 #pragma unroll
                for (int k = 0; k < VEC; k++) acc[k] = RD::combine(acc[k], RD::load(v[u].v[k], prm));
          }
-         for (; i < p.rsize0; i += SPLIT)
+         for (; i < i_hi; i += NSL)
          {  Pack<T, VEC> v;
             load_wide<T, VEC>(v, row + (int64_t)i * s0);
 #pragma unroll
@@ -107,8 +123,7 @@ __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, co
       __syncthreads();
       if (slice == 0)
       {
-#pragma unroll
-         for (int s2 = 1; s2 < SPLIT; s2++)
+         for (uint32_t s2 = 1; s2 < NSL; s2++)
 #pragma unroll
             for (int k = 0; k < VEC; k++) acc[k] = RD::combine(acc[k], lds[k * 256 + s2 * OPB + ol]);
       }
@@ -117,12 +132,28 @@ __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, co
    {
 #pragma unroll
       for (int k = 0; k < VEC; k++)
-         *reinterpret_cast<typename RD::Res *>(p.dst + o2 + (int64_t)k * p.st2[0]) = RD::finalize(acc[k], prm);
+      {  if (p.slices > 1) *reinterpret_cast<Acc *>(p.partials + ((size_t)blockIdx.y * p.nout + o + k) * 16) = acc[k];
+         else *reinterpret_cast<typename RD::Res *>(p.dst + o2 + (int64_t)k * p.st2[0]) = RD::finalize(acc[k], prm);
+      }
    }
 }
 
+/* folds the pieces of a sliced reduction in slice order: one thread per output */
+template <class RD, class T>
+__global__ __launch_bounds__(256) void axis_finish_kernel(const AxisParams p, const typename RD::Param prm)
+{
+   typedef typename RD::Acc Acc;
+   const uint32_t o = blockIdx.x * 256 + threadIdx.x;
+   if (o >= p.nout) return;
+   int64_t o1, o2;
+   axis_outer_offsets(p, o, o1, o2);
+   Acc acc = *reinterpret_cast<const Acc *>(p.partials + (size_t)o * 16);
+   for (uint32_t t = 1; t < p.slices; t++) acc = RD::combine(acc, *reinterpret_cast<const Acc *>(p.partials + ((size_t)t * p.nout + o) * 16));
+   *reinterpret_cast<typename RD::Res *>(p.dst + o2) = RD::finalize(acc, prm);
+}
+
 /* A group of threads cooperates on one output: GROUP 256 = the whole block, GROUP 64 = p.glanes (8 .. 64, a power
-   of two) lanes of a wave, chosen so that every lane has about four loads in flight on short rows. VEC > 1: the first reduced
+   of two) lanes of a wave (1 .. 64), chosen so that every lane has about four loads in flight on short rows. VEC > 1: the first reduced
    dimension has unit stride and every row starts 16-byte aligned, so a thread takes VEC neighbouring elements with
    one 128-bit load (NT: with the nontemporal hint, for sources that are read once from memory). */
 template <class RD, class T, int GROUP, int VEC = 1, bool NT = false>
@@ -141,9 +172,13 @@ __global__ __launch_bounds__(256) void axis_group_kernel(const AxisParams p, con
       const char *base = p.src + o1;
       const int64_t s0 = (VEC > 1) ? (int64_t)(sizeof(T) * VEC) : p.rst[0];        /* step of one group */
       const uint32_t n0 = (VEC > 1) ? p.rgdiv.d : p.rsize0;                        /* groups per row */
+      /* range of loads of this piece of the reduced range */
+      const uint32_t total = (p.rd <= 1) ? n0 : ((VEC > 1) ? p.relem / VEC : p.relem);
+      uint32_t lo = 0, hi = total;
+      if (p.slices > 1) { lo = blockIdx.y * p.slice_len; hi = (lo + p.slice_len < total) ? lo + p.slice_len : total; }
       if (p.rd <= 1)
-      {  uint32_t i = lane;
-         for (; i + 3 * G < n0; i += 4 * G)
+      {  uint32_t i = lo + lane;
+         for (; i + 3 * G < hi; i += 4 * G)
          {  Pack<T, VEC> v[4];
 #pragma unroll
             for (int u = 0; u < 4; u++)
@@ -155,7 +190,7 @@ __global__ __launch_bounds__(256) void axis_group_kernel(const AxisParams p, con
 #pragma unroll
                for (int k = 0; k < VEC; k++) acc = RD::combine(acc, RD::load(v[u].v[k], prm));
          }
-         for (; i < n0; i += G)
+         for (; i < hi; i += G)
          {  Pack<T, VEC> v;
             if constexpr (VEC > 1) load_wide<T, VEC, NT>(v, base + (int64_t)i * s0);
             else v.v[0] = *reinterpret_cast<const T *>(base + (int64_t)i * s0);
@@ -164,8 +199,7 @@ __global__ __launch_bounds__(256) void axis_group_kernel(const AxisParams p, con
          }
       }
       else
-      {  const uint32_t total = (VEC > 1) ? p.relem / VEC : p.relem;
-         for (uint32_t j = lane; j < total; j += G)
+      {  for (uint32_t j = lo + lane; j < hi; j += G)
          {  uint32_t r = fastdiv(j, (VEC > 1) ? p.rgdiv : p.rdiv[0]); uint32_t i = j - r * n0;
             Pack<T, VEC> v;
             if constexpr (VEC > 1) load_wide<T, VEC, NT>(v, base + axis_row_offset(p, r) + (int64_t)i * s0);
@@ -182,7 +216,10 @@ __global__ __launch_bounds__(256) void axis_group_kernel(const AxisParams p, con
       __syncthreads();
       if (threadIdx.x == 0) { acc = RD::combine(RD::combine(lds[0], lds[1]), RD::combine(lds[2], lds[3])); }
    }
-   if (active && lane == 0) *reinterpret_cast<typename RD::Res *>(p.dst + o2) = RD::finalize(acc, prm);
+   if (active && lane == 0)
+   {  if (p.slices > 1) *reinterpret_cast<Acc *>(p.partials + ((size_t)blockIdx.y * p.nout + o) * 16) = acc;
+      else *reinterpret_cast<typename RD::Res *>(p.dst + o2) = RD::finalize(acc, prm);
+   }
 }
 
 typedef int (*axis_fn)(const och_reduce_axis_config *c, double pnorm);
@@ -228,7 +265,25 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
    int64_t red_fast = (p.rd > 0) ? (p.rst[0] < 0 ? -p.rst[0] : p.rst[0]) : INT64_MAX;
    /* a source larger than the caches is read once: nontemporal loads (see och_reduce_all.h) */
    const bool streaming = nout * relem * (uint64_t)sizeof(T) >= OCH_EW_STREAM_BYTES;
-   bool cooperative = (p.rd > 0) && ((red_fast < outer_fast) || (nout < 16384 && relem >= 256));
+   /* cooperate on an output when the reduced range is the faster one in memory (or there is a single output); otherwise
+      neighbouring threads take neighbouring outputs, and a long reduced range is cut into pieces below */
+   bool cooperative = (p.rd > 0) && ((red_fast < outer_fast) || p.nd == 0);
+   /* too few blocks for the device and a long reduced range: cut the range into pieces (grid y), about 1024 blocks in all,
+      every piece at least min_len long, the partial accumulators within the stream's workspace */
+   auto plan_slices = [&](uint64_t blocks, uint64_t range, uint64_t min_len) -> int
+   {  p.slices = 1; p.slice_len = 0; p.partials = nullptr;
+      if (blocks >= 512 || range < 2 * min_len) return 0;
+      uint64_t want = (1024 + blocks - 1) / blocks;
+      if (want > range / min_len) want = range / min_len;
+      const uint64_t fit = OCH_GEMM_WORKSPACE / ((uint64_t)p.nout * 16);
+      if (want > fit) want = fit;
+      if (want > 65535) want = 65535;
+      if (want < 2) return 0;
+      p.slice_len = (uint32_t)((range + want - 1) / want);
+      p.slices = (uint32_t)((range + p.slice_len - 1) / p.slice_len);
+      if (p.slices < 2) { p.slices = 1; return 0; }
+      return stream_gemm_workspace(stream, &p.partials);
+   };
    if (!cooperative)
    {  /* VEC outputs per thread when the first outer dimension has unit source stride and
          everything is 16-byte aligned; four waves per output group while there are few groups */
@@ -238,18 +293,19 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
       for (int d = 0; d < p.rd && wide; d++) if (p.rst[d] % 16 != 0) wide = false;
       const uint64_t groups = wide ? nout / VEC : nout;
       const bool split = groups < (1u << 20) && p.rsize0 >= 16;
-      if (wide && split && streaming)
-         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 4, VEC, true>), dim3((unsigned)((groups + 63) / 64)), dim3(256), 0, stream, p, prm);
-      else if (wide && split)
-         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 4, VEC>), dim3((unsigned)((groups + 63) / 64)), dim3(256), 0, stream, p, prm);
-      else if (wide && streaming)
-         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, VEC, true>), dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, stream, p, prm);
-      else if (wide)
-         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, VEC>), dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, stream, p, prm);
-      else if (split)
-         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 4, 1>), dim3((p.nout + 63) / 64), dim3(256), 0, stream, p, prm);
-      else
-         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, 1>), dim3((p.nout + 255) / 256), dim3(256), 0, stream, p, prm);
+      p.opb = 64;
+      while (p.opb > 1 && p.opb / 2 >= groups) p.opb /= 2;
+      const unsigned blocks = (unsigned)(split ? (groups + p.opb - 1) / p.opb : (groups + 255) / 256);
+      /* pieces of the reduced range: whole rows of it when there are several, else positions along its first dimension */
+      p.slice_rows = (p.rd > 1 && p.rrows >= 8) ? 1 : 0;
+      if (plan_slices(blocks, p.slice_rows ? p.rrows : p.rsize0, p.slice_rows ? 4 : (split ? 16 * (256 / p.opb) : 16)) != 0) return -1;
+      const dim3 grid(blocks, p.slices);
+      if (wide && split && streaming) hipLaunchKernelGGL((axis_thread_kernel<RD, T, 4, VEC, true>), grid, dim3(256), 0, stream, p, prm);
+      else if (wide && split)         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 4, VEC>), grid, dim3(256), 0, stream, p, prm);
+      else if (wide && streaming)     hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, VEC, true>), grid, dim3(256), 0, stream, p, prm);
+      else if (wide)                  hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, VEC>), grid, dim3(256), 0, stream, p, prm);
+      else if (split)                 hipLaunchKernelGGL((axis_thread_kernel<RD, T, 4, 1>), grid, dim3(256), 0, stream, p, prm);
+      else                            hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, 1>), grid, dim3(256), 0, stream, p, prm);
    }
    else
    {  /* rows of the first reduced dimension are contiguous and 16-byte aligned: 128-bit loads */
@@ -261,9 +317,14 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
       const bool wave = relem <= 2048 && nout >= 1024;              /* a wave per output, else a block per output */
       const uint32_t loads = wide ? p.relem / VEC : p.relem;       /* loads per output: about four per lane */
       p.glanes = 64;
-      while (p.glanes > 8 && (p.glanes / 2) * 4 >= loads) p.glanes /= 2;
+      while (p.glanes > 1 && (p.glanes / 2) * 4 >= loads) p.glanes /= 2;
       const uint32_t per_block = 256 / p.glanes;
-      const dim3 grid(wave ? (p.nout + per_block - 1) / per_block : p.nout);
+      const unsigned blocks = wave ? (p.nout + per_block - 1) / per_block : p.nout;
+      p.slice_rows = 0;
+      {  const uint64_t range = (p.rd <= 1) ? (wide ? p.rsize0 / VEC : p.rsize0) : loads;
+         if (plan_slices(blocks, range, (uint64_t)(wave ? p.glanes : 256) * 8) != 0) return -1;
+      }
+      const dim3 grid(blocks, p.slices);
       if (wide && streaming)
       {  if (wave) hipLaunchKernelGGL((axis_group_kernel<RD, T, 64, VEC, true>), grid, dim3(256), 0, stream, p, prm);
          else      hipLaunchKernelGGL((axis_group_kernel<RD, T, 256, VEC, true>), grid, dim3(256), 0, stream, p, prm);
@@ -277,6 +338,7 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
          else      hipLaunchKernelGGL((axis_group_kernel<RD, T, 256>), grid, dim3(256), 0, stream, p, prm);
       }
    }
+   if (p.slices > 1) hipLaunchKernelGGL((axis_finish_kernel<RD, T>), dim3((p.nout + 255) / 256), dim3(256), 0, stream, p, prm);
    OCH_CHECK_LAUNCH();
    return 0;
 }

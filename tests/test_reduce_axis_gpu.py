@@ -131,3 +131,42 @@ def test_config3_axis_reductions(hip, stream, dtype):
         rd, got, want = run_case(stream, "minimum", dtype, parent, view, [axis])
         H.assert_same_bytes(got, want, "axis %d min" % axis)
         H.assert_same_bytes(got, view.min(axis=axis).T.copy(), "axis %d min vs numpy" % axis)
+
+
+SLICED = [  # Ocean shape (dimension 0 fastest), reduced axes: few outputs (or output groups) and a long reduced range
+    ((1024, 3000), [1]),          # row sums of a column-major matrix: per-thread kernel, pieces along the reduced dimension
+    ((200, 300, 64), [1, 2]),     # per-thread kernel, pieces of whole rows of the reduced range
+    ((200, 300, 64), [0, 1]),     # a block per output, two reduced dimensions
+    ((300000, 8), [0]),           # eight outputs, each a long contiguous row
+    ((8, 300000), [1]),           # eight outputs, reduced dimension strided
+    ((64, 5, 4000), [0, 2]),
+    ((70001,), [0]),
+]
+
+
+@pytest.mark.parametrize("dtype", [H.INT32, H.FLOAT, H.DOUBLE, H.CFLOAT], ids=lambda d: H.NAMES[d])
+def test_axis_reductions_cut_into_pieces(hip, stream, dtype):
+    """Too few outputs to occupy the device: the reduced range is cut into pieces (grid y), every piece leaves its
+    accumulator in the stream's workspace and a second kernel folds the pieces in order. Integers and extremes are exact,
+    floating sums / norms within the usual bounds of the float64 result."""
+    rng = np.random.default_rng(900 + dtype)
+    for shape, axes in SLICED:
+        parent = H.random_data(dtype, int(np.prod(shape)), rng, "general").reshape(shape[::-1])
+        view = parent.T
+        v = to_f64(dtype, view)
+        for name in ("sum", "maximum", "nnz", "norm2", "sum_abs"):
+            if not oh.lib.och_reduce_supported(oh.R[name], dtype):
+                continue
+            rd, got, want = run_case(stream, name, dtype, parent, view, axes)
+            what = "%s %s %s axes=%s" % (name, H.NAMES[dtype], shape, axes)
+            if dtype == H.INT32 and name != "norm2" or name in ("maximum", "nnz"):
+                H.assert_same_bytes(got, want, what)
+                continue
+            # floating sums: against the float64 evaluation (the oracle adds in the element type, serially, and is the
+            # less accurate side on ranges this long)
+            g = to_f64(rd, got)
+            ax = tuple(axes)
+            truth = {"sum": v.sum(axis=ax), "sum_abs": np.abs(v).sum(axis=ax), "norm2": np.sqrt((np.abs(v) ** 2).sum(axis=ax))}[name].T
+            scale = np.abs(v).sum(axis=ax).T if name == "sum" else np.abs(truth)
+            tol = 1e-12 if dtype == H.DOUBLE else 1e-5
+            assert np.all(np.abs(g - truth) <= tol * np.maximum(np.asarray(scale), 1e-6)), what
