@@ -88,7 +88,7 @@ struct RedParams
    int   ntail;
 };
 
-/* WIDE: flat, unit-stride, aligned source read with VEC-wide loads (compile-time, so that the
+/* WIDE: the first dimension is contiguous, divisible by VEC and aligned: VEC-wide loads (compile-time, so that the
    loads stay single 128-bit instructions); otherwise VEC is 1 and any layout is accepted. */
 template <class RD, class T, int VEC, bool WIDE, bool NT = false>
 __global__ __launch_bounds__(OCH_RED_BLOCK) void reduce_all_kernel(const RedParams p, const typename RD::Param prm)
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(OCH_RED_BLOCK) void reduce_all_kernel(const RedPara
    uint64_t g = (uint64_t)blockIdx.x * p.per_block + threadIdx.x;
    uint64_t end = (uint64_t)blockIdx.x * p.per_block + p.per_block;
    if (end > p.ngroups) end = p.ngroups;
-   const bool flat = WIDE || (p.ew.ndims == 1);
+   const bool flat = (p.ew.ndims == 1);
    /* main loop: OCH_RED_UNR independent groups per trip, loads first, one accumulator per group */
    for (; g + (OCH_RED_UNR - 1) * stride < end; g += OCH_RED_UNR * stride)
    {  Pack<T, VEC> v[OCH_RED_UNR];
@@ -197,7 +197,9 @@ static int launch_reduce_all(int ndims, const size_t *size, const ptrdiff_t *str
          p.tail = shape.ptr[0] + (int64_t)(n - n % vec) * shape.stride[0][0];
       }
       else
-      {  ew_params<1>(p.ew, shape, 1, es, 0);
+      {  /* several dimensions: 128-bit loads along the first one when it is contiguous, divisible and aligned */
+         wide_launch = (VEC > 1) && ew_params<1>(p.ew, shape, VEC, es, 0) && p.ew.vecmode[0];
+         if (!wide_launch) ew_params<1>(p.ew, shape, 1, es, 0);
          p.ngroups = p.ew.ngroups;
       }
    }
