@@ -83,6 +83,10 @@ OCH_HD float half_to_float(half_t hh)
    h &= 0x7FFFu;
    if (h == 0) return 0.f;                       /* both zeros map to +0 */
    uint32_t e = h & 0x7C00u;
+#if defined(__HIP_DEVICE_COMPILE__)
+   /* finite non-zero values: the hardware conversion is exact, as is the normalisation loop below (subnormals included) */
+   if (e != 0x7C00u) { _Float16 x; __builtin_memcpy(&x, &hh.v, 2); return (float)x; }
+#endif
    if (e == 0)
    {  /* subnormal: normalise the mantissa */
       uint32_t shift = 1; h <<= 1;
