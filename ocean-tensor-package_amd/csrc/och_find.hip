@@ -6,7 +6,8 @@
  *   scan  : one block turns the counts into start positions in place (exclusive prefix sum), the total goes to
  *           workspace[0], which the host reads back
  *   apply : every block recomputes its chunk, ranks its non-zero elements with a block-wide prefix sum
- *           (wave scan + LDS) and writes indices or offsets at start[chunk] + rank
+ *           (wave scan + LDS), compacts their positions in LDS and writes indices or offsets from start[chunk] on
+ * A thread looks at 16 consecutive elements; where these are 16 aligned consecutive bytes it takes them in one load.
  * The output order is deterministic: the order of the elements themselves.
  */
 #include "och_elemwise.h"
@@ -14,7 +15,7 @@
 namespace och {
 
 #define OCH_FIND_THREADS 256
-#define OCH_FIND_PER_THREAD 8
+#define OCH_FIND_PER_THREAD 16
 #define OCH_FIND_CHUNK (OCH_FIND_THREADS * OCH_FIND_PER_THREAD)
 
 struct FindParams
@@ -26,6 +27,7 @@ struct FindParams
    int64_t     strides[OCH_MAX_DIMS];
    int64_t     mult[OCH_MAX_DIMS];
    int         offsets;             /* 1: write sum of index * mult; 0: write the indices */
+   int         wide;                /* 1: every aligned run of 16 elements is 16 consecutive, 16-byte aligned bytes */
 };
 
 /* flat element number -> indices (dimension 0 fastest); returns the byte offset. Element counts below 2^32 use the
@@ -56,11 +58,20 @@ OCH_D void find_step(const FindParams &p, uint32_t (&idx)[OCH_MAX_DIMS], int64_t
       off -= (int64_t)p.div[d].d * p.strides[d]; idx[d] = 0;
    }
 }
+/* four bytes -> four bits: bit k set iff byte k is non-zero */
+OCH_D unsigned int find_nibble(uint32_t w)
+{  const uint32_t t = ((((w & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | w) & 0x80808080u) >> 7;   /* bits 0, 8, 16, 24 */
+   return (t * 0x01020408u) >> 24;                /* the four products that land in bits 24..27 do not collide */
+}
 /* bit k of the result: element base + k exists and is non-zero */
 OCH_D unsigned int find_flags(const FindParams &p, uint64_t base)
 {  unsigned int flags = 0; uint32_t idx[OCH_MAX_DIMS];
    if (base >= p.nelem) return 0;
    int64_t off = find_decompose(p, base, idx);
+   if (p.wide)
+   {  const uint4 w = *(const uint4 *)(p.ptr + off);
+      return find_nibble(w.x) | (find_nibble(w.y) << 4) | (find_nibble(w.z) << 8) | (find_nibble(w.w) << 12);
+   }
    for (int k = 0; k < OCH_FIND_PER_THREAD && base + k < p.nelem; k++)
    {  if (p.ptr[off] != 0) flags |= 1u << k;
       find_step(p, idx, off);
@@ -98,34 +109,37 @@ __global__ __launch_bounds__(1024) void find_scan_kernel(unsigned long long *wor
    for (uint64_t i = lo; i < hi; i++) { unsigned long long v = workspace[1 + i]; workspace[1 + i] = run; run += v; }
 }
 
+/* The non-zero elements of the chunk are first compacted in LDS (their position within the chunk, in element order);
+   the threads then write the results side by side, so that the stores of a wave cover consecutive output entries. */
 __global__ __launch_bounds__(OCH_FIND_THREADS) void find_apply_kernel(const FindParams p, const unsigned long long *workspace, int64_t *out)
 {
    __shared__ unsigned int lds[OCH_FIND_THREADS / 64];
-   const uint64_t base = (uint64_t)blockIdx.x * OCH_FIND_CHUNK + (uint64_t)threadIdx.x * OCH_FIND_PER_THREAD;
-   const unsigned int flags = find_flags(p, base), c = __popc(flags);
-   /* exclusive rank of this thread's first hit within the block */
+   __shared__ unsigned short where[OCH_FIND_CHUNK];
+   const uint64_t chunk = (uint64_t)blockIdx.x * OCH_FIND_CHUNK;
+   const unsigned int flags = find_flags(p, chunk + (uint64_t)threadIdx.x * OCH_FIND_PER_THREAD), c = __popc(flags);
    unsigned int incl = c;
    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
    for (int d = 1; d < 64; d <<= 1) { unsigned int v = __shfl_up(incl, d, 64); if (lane >= d) incl += v; }
    if (lane == 63) lds[wave] = incl;
    __syncthreads();
-   unsigned int before = 0;
-   for (int w = 0; w < wave; w++) before += lds[w];
-   uint64_t pos = workspace[1 + blockIdx.x] + before + (incl - c);
-   if (c == 0) return;
-   uint32_t idx[OCH_MAX_DIMS];
-   int64_t off = find_decompose(p, base, idx);
-   for (int k = 0; k < OCH_FIND_PER_THREAD; k++)
-   {  if (flags & (1u << k))
-      {  if (p.offsets)
-         {  int64_t s = 0;
-            for (int d = 0; d < p.ndims; d++) s += (int64_t)idx[d] * p.mult[d];
-            out[pos] = s;
-         }
-         else for (int d = 0; d < p.ndims; d++) out[pos * p.ndims + d] = idx[d];
-         pos++;
+   unsigned int before = 0, total = 0;
+   for (int w = 0; w < OCH_FIND_THREADS / 64; w++) { if (w < wave) before += lds[w]; total += lds[w]; }
+   unsigned int rank = before + (incl - c);
+   for (unsigned int f = flags; f; f &= f - 1)
+      where[rank++] = (unsigned short)(threadIdx.x * OCH_FIND_PER_THREAD + (__ffs(f) - 1));
+   __syncthreads();
+   const uint64_t start = workspace[1 + blockIdx.x];
+   for (unsigned int j = threadIdx.x; j < total; j += OCH_FIND_THREADS)
+   {  const uint64_t e = chunk + where[j];
+      if (p.ndims == 1) { out[start + j] = p.offsets ? (int64_t)e * p.mult[0] : (int64_t)e; continue; }
+      uint32_t idx[OCH_MAX_DIMS];
+      find_decompose(p, e, idx);
+      if (p.offsets)
+      {  int64_t s = 0;
+         for (int d = 0; d < p.ndims; d++) s += (int64_t)idx[d] * p.mult[d];
+         out[start + j] = s;
       }
-      find_step(p, idx, off);
+      else for (int d = 0; d < p.ndims; d++) out[(start + j) * p.ndims + d] = idx[d];
    }
 }
 
@@ -140,6 +154,9 @@ static int find_params(FindParams &p, int ndims, const size_t *size, const ptrdi
       p.nelem *= size[d]; p.div[d] = make_fastdiv((uint32_t)(size[d] ? size[d] : 1)); p.strides[d] = strides[d];
    }
    if (p.nelem > 0 && ptr == nullptr) return set_error("find: null data pointer");
+   /* runs of 16 elements are 16 aligned bytes when dimension 0 is dense, a multiple of 16 long, and every row starts aligned */
+   p.wide = (ndims >= 1 && p.nelem > 0 && strides[0] == 1 && size[0] % 16 == 0 && ((uintptr_t)ptr & 15) == 0);
+   for (int d = 1; d < ndims && p.wide; d++) if (size[d] > 1 && (strides[d] & 15) != 0) p.wide = 0;
    return 0;
 }
 

@@ -134,3 +134,32 @@ def test_find_and_mask_to_offset(hip, stream, shape, density):
         assert np.array_equal(out.download(np.int64, want_n), want)
         work.free(); out.free()
     dbig.free()
+
+
+@pytest.mark.parametrize("shape,shift", [((1 << 20,), 0), ((1 << 20,), 16), ((1 << 20,), 3), ((37, 4096), 0), ((5, 7, 48), 0),
+                                         ((5, 7, 48), 32), ((33, 40), 0), ((3, 16), 0)])
+def test_find_contiguous_mask(hip, stream, shape, shift):
+    """Dense masks whose fastest dimension is a multiple of 16 (the 16-byte load path when the base is aligned too; `shift`
+    bytes into the allocation) against numpy.nonzero and numpy.ravel_multi_index."""
+    import ctypes as C
+    rng = np.random.default_rng(sum(shape) + shift)
+    mask = (rng.random(shape) < 0.3).astype(np.uint8) * rng.integers(1, 255, shape).astype(np.uint8)
+    n, nd = mask.size, len(shape)
+    raw = np.zeros(n + 64, np.uint8); raw[shift:shift + n] = mask.ravel()
+    draw = oh.to_device(raw, stream)
+    sz, st = oh.sizes(shape[::-1]), oh.strides(mask.strides[::-1])
+    work = oh.DeviceBuffer(oh.lib.och_find_workspace_size(n), stream)
+    nnz = C.c_size_t(0)
+    dptr = C.c_void_p(draw.address + shift)
+    oh.check(oh.lib.och_find_count(nd, sz, st, dptr, work.ptr, C.byref(nnz), stream.handle))
+    hits = np.nonzero(mask)
+    assert nnz.value == len(hits[0])
+    out = oh.DeviceBuffer(8 * max(1, nnz.value * nd), stream)
+    oh.check(oh.lib.och_find_apply(nd, sz, st, dptr, work.ptr, None, out.ptr, stream.handle))
+    # numpy order (last numpy axis fastest) is the library's order (its dimension 0 fastest); indices come fastest first
+    want = np.stack(hits[::-1], axis=1).astype(np.int64)
+    assert np.array_equal(out.download(np.int64, nnz.value * nd).reshape(-1, nd), want)
+    mult = np.array([3, -1000, 1 << 35][:nd], np.int64)
+    oh.check(oh.lib.och_find_apply(nd, sz, st, dptr, work.ptr, mult.ctypes.data_as(IC.P64), out.ptr, stream.handle))
+    assert np.array_equal(out.download(np.int64, nnz.value), want @ mult)
+    draw.free(); work.free(); out.free()
