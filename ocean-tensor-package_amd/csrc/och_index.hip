@@ -20,6 +20,7 @@ template <class T> static T idx_scalar_as(const och_scalar &s) { T v; memcpy(&v,
 struct IndexParams
 {
    uint64_t       size[OCH_MAX_DIMS];
+   FastDiv        div[OCH_MAX_DIMS];           /* used when nelem < 2^32 */
    const int64_t *offsets[OCH_MAX_DIMS];
    int64_t        strides1[OCH_MAX_DIMS], strides2[OCH_MAX_DIMS];
    char          *ptr1, *ptr2;
@@ -40,21 +41,45 @@ __global__ __launch_bounds__(256) void index_to_offset_kernel(uint64_t nelem, in
    *reinterpret_cast<int64_t *>(dst + (int64_t)j * stride2) = s;
 }
 
-/* MODE 0: gather  *ptr2 = *ptr1(indexed);  1: scatter  *ptr1(indexed) = *ptr2;  2: fill  *ptr1(indexed) = value */
-template <class E, int MODE>
+/* MODE 0: gather  *ptr2 = *ptr1(indexed);  1: scatter  *ptr1(indexed) = *ptr2;  2: fill  *ptr1(indexed) = value.
+   V > 1: a work item is a run of V elements (16 bytes) along a dense dimension 0 that has no offset table; the host has
+   divided size[0] by V and set both strides of dimension 0 to 16. Offset tables are device data, so whether a run is
+   16-byte aligned is only known here: aligned runs move in one access, others element by element. */
+template <class E, int MODE, int V>
 __global__ __launch_bounds__(256) void index_kernel(const IndexParams p, const E value)
 {
+   const bool small = p.nelem <= 0xFFFFFFFFull;
    for (uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x; idx < p.nelem; idx += (uint64_t)gridDim.x * 256)
-   {  uint64_t q = idx; int64_t o1 = 0, o2 = 0;
-      for (int d = 0; d < p.ndims; d++)
-      {  uint64_t s = q % p.size[d]; q /= p.size[d];
-         o1 += p.offsets[d] ? p.offsets[d][s] : (int64_t)s * p.strides1[d];
-         if (MODE != 2) o2 += (int64_t)s * p.strides2[d];
+   {  int64_t o1 = 0, o2 = 0;
+      if (small)
+      {  uint32_t q = (uint32_t)idx;
+         for (int d = 0; d < p.ndims; d++)
+         {  const uint32_t q2 = fastdiv(q, p.div[d]), s = q - q2 * p.div[d].d; q = q2;
+            o1 += p.offsets[d] ? p.offsets[d][s] : (int64_t)s * p.strides1[d];
+            if (MODE != 2) o2 += (int64_t)s * p.strides2[d];
+         }
       }
-      E *a = reinterpret_cast<E *>(p.ptr1 + o1);
-      if (MODE == 0) *reinterpret_cast<E *>(p.ptr2 + o2) = *a;
-      else if (MODE == 1) *a = *reinterpret_cast<const E *>(p.ptr2 + o2);
-      else *a = value;
+      else
+      {  uint64_t q = idx;
+         for (int d = 0; d < p.ndims; d++)
+         {  uint64_t s = q % p.size[d]; q /= p.size[d];
+            o1 += p.offsets[d] ? p.offsets[d][s] : (int64_t)s * p.strides1[d];
+            if (MODE != 2) o2 += (int64_t)s * p.strides2[d];
+         }
+      }
+      char *a = p.ptr1 + o1, *b = p.ptr2 + o2;
+      if (V > 1 && ((((uintptr_t)a) | (MODE != 2 ? (uintptr_t)b : 0)) & 15) == 0)
+      {  if (MODE == 0) *reinterpret_cast<uint4 *>(b) = *reinterpret_cast<const uint4 *>(a);
+         else if (MODE == 1) *reinterpret_cast<uint4 *>(a) = *reinterpret_cast<const uint4 *>(b);
+         else { union { uint4 w; E e[V]; } u; for (int k = 0; k < V; k++) u.e[k] = value; *reinterpret_cast<uint4 *>(a) = u.w; }
+         continue;
+      }
+      for (int k = 0; k < V; k++)
+      {  E *x = reinterpret_cast<E *>(a) + k;
+         if (MODE == 0) reinterpret_cast<E *>(b)[k] = *x;
+         else if (MODE == 1) *x = reinterpret_cast<const E *>(b)[k];
+         else *x = value;
+      }
    }
 }
 
@@ -65,10 +90,17 @@ struct alignas(2) E2 { unsigned char b[2]; };
 struct E1 { unsigned char b[1]; };
 
 template <class E, int MODE>
-static int launch_index(const IndexParams &p, const och_scalar &value, hipStream_t stream)
+static int launch_index(IndexParams &p, const och_scalar &value, hipStream_t stream)
 {  E v; memcpy(&v, &value, sizeof(E));
-   uint64_t blocks = (p.nelem + 255) / 256; if (blocks > 65536) blocks = 65536;
-   hipLaunchKernelGGL((index_kernel<E, MODE>), dim3((unsigned)blocks), dim3(256), 0, stream, p, v);
+   constexpr int V = 16 / (int)sizeof(E);
+   const bool runs = p.ndims >= 1 && p.offsets[0] == nullptr && p.size[0] % V == 0 && p.strides1[0] == (int64_t)sizeof(E) &&
+                     (MODE == 2 || p.strides2[0] == (int64_t)sizeof(E));
+   if (runs) { p.size[0] /= V; p.nelem /= V; p.strides1[0] = 16; if (MODE != 2) p.strides2[0] = 16; }
+   if (p.nelem <= 0xFFFFFFFFull)
+      for (int d = 0; d < p.ndims; d++) p.div[d] = make_fastdiv((uint32_t)p.size[d]);
+   uint64_t blocks = (p.nelem + 255) / 256; if (blocks > (1u << 20)) blocks = 1u << 20;
+   if (runs) hipLaunchKernelGGL((index_kernel<E, MODE, V>), dim3((unsigned)blocks), dim3(256), 0, stream, p, v);
+   else      hipLaunchKernelGGL((index_kernel<E, MODE, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, p, v);
    OCH_CHECK_LAUNCH();
    return 0;
 }

@@ -68,6 +68,45 @@ def test_gather_large_and_empty(hip, stream):
         b.free()
 
 
+@pytest.mark.parametrize("dtype", [H.INT8, H.HALF, H.FLOAT, H.DOUBLE, H.CDOUBLE], ids=lambda d: H.NAMES[d])
+@pytest.mark.parametrize("shift", [0, 1])
+def test_row_gather_scatter_fill(hip, stream, dtype, shift):
+    """Whole rows through an offset table on the slow dimension (rows move as 16-byte runs where both ends are aligned);
+    `shift` elements into the allocations makes the rows unaligned for element sizes below 16. Against numpy indexing."""
+    rng = np.random.default_rng(7 + dtype + shift)
+    n, m, k = 352, 130, 77
+    flat = H.random_data(dtype, m * n + shift, rng)
+    es = flat.itemsize
+    parent = flat[shift:].reshape(m, n)
+    rows = rng.permutation(m)[:k].astype(np.int64)
+    dtab_buf = oh.to_device(rows * (n * es), stream)
+    dtab = IC.pointer_table([None, dtab_buf], lambda b: b.address)
+    dflat = oh.to_device(flat, stream)
+    dout = oh.to_device(np.zeros(k * n + shift, flat.dtype), stream)
+    import ctypes as C
+    pp, po = C.c_void_p(dflat.address + shift * es), C.c_void_p(dout.address + shift * es)
+    sz = oh.sizes([n, k])
+    oh.check(oh.lib.och_get_index(dtype, 2, sz, dtab, oh.strides([es, 0]), pp, oh.strides([es, es * n]), po, stream.handle))
+    H.assert_same_bytes(dout.download(flat.dtype, k * n + shift)[shift:].reshape(k, n), parent[rows], "row gather")
+    src = H.random_data(dtype, k * n + shift, rng)
+    dsrc = oh.to_device(src, stream)
+    ps = C.c_void_p(dsrc.address + shift * es)
+    oh.check(oh.lib.och_set_index(dtype, 2, sz, dtab, oh.strides([es, 0]), pp, oh.strides([es, es * n]), ps, stream.handle))
+    want = parent.copy(); want[rows] = src[shift:].reshape(k, n)
+    H.assert_same_bytes(dflat.download(flat.dtype, m * n + shift)[shift:].reshape(m, n), want, "row scatter")
+    val = H.random_data(dtype, 1, rng)
+    half = rows[: k // 2]
+    dtab2_buf = oh.to_device(half * (n * es), stream)
+    dtab2 = IC.pointer_table([None, dtab2_buf], lambda b: b.address)
+    oh.check(oh.lib.och_fill_index(dtype, 2, oh.sizes([n, half.size]), dtab2, oh.strides([es, 0]), pp, H.raw_scalar(val), stream.handle))
+    want[half] = val[0]
+    got = dflat.download(flat.dtype, m * n + shift)
+    H.assert_same_bytes(got[shift:].reshape(m, n), want, "row fill")
+    H.assert_same_bytes(got[:shift], flat[:shift], "bytes before the parent")
+    for b in (dtab_buf, dtab2_buf, dflat, dout, dsrc):
+        b.free()
+
+
 @pytest.mark.parametrize("dtype", [H.INT8, H.INT16, H.INT32, H.INT64], ids=lambda d: H.NAMES[d])
 def test_add_if_negative(hip, stream, dtype):
     rng = np.random.default_rng(dtype)
