@@ -537,5 +537,6 @@ int gemm_float(const GemmArgs &g);
 int gemm_double(const GemmArgs &g);
 int gemm_cfloat(const GemmArgs &g);
 int gemm_cdouble(const GemmArgs &g);
+int gemm_half(const GemmArgs &g);      /* 1: not taken, use the generic kernel */
 
 } /* namespace och */

@@ -142,7 +142,7 @@ static int gemm_dispatch(int dtype, const GemmArgs &g)
       case OCH_INT16:   return gemm_generic<int16_t>(g);
       case OCH_INT32:   return gemm_generic<int32_t>(g);
       case OCH_INT64:   return gemm_generic<int64_t>(g);
-      case OCH_HALF:    return gemm_generic<half_t>(g);
+      case OCH_HALF:    { const int status = gemm_half(g); return (status == 1) ? gemm_generic<half_t>(g) : status; }
       case OCH_FLOAT:   return gemm_float(g);
       case OCH_DOUBLE:  return gemm_double(g);
       case OCH_CFLOAT:  return gemm_cfloat(g);
