@@ -133,11 +133,12 @@ def test_gemm_scalars(hip, stream, dtype):
 @pytest.mark.parametrize("tb", ["N", "T"])
 def test_gemm_half_matrix_cores(hip, stream, ta, tb):
     """Half products large enough for the MFMA kernel: whole tiles with aligned operands (128-bit loads), ragged edges,
-    leading dimensions that rule out wide loads, both tile sizes, a long K, scalars in device memory."""
+    leading dimensions that rule out wide loads, all three tile sizes, a long K, scalars in device memory."""
     rng = np.random.default_rng(900 + ord(ta) + 2 * ord(tb))
     for (M, N, K, pad, alpha, beta, dev) in [(128, 128, 64, 0, 1, 0, False), (256, 384, 96, 8, 2, -1, False), (200, 136, 100, 3, 1, 1, True),
                                               (64, 64, 32, 0, -1, 0.5, False), (96, 160, 2048, 0, 0.5, 0, True), (33, 47, 17, 5, 1, 0, False),
-                                              (2560, 2304, 48, 0, 1, 1, False), (2500, 2300, 40, 4, 1, 0, False)]:
+                                              (2560, 2304, 48, 0, 1, 1, False), (2500, 2300, 40, 4, 1, 0, False), (4096, 3072, 64, 0, 1, 0, False),
+                                              (4000, 3100, 70, 0, -1, 1, True)]:
         run_case(stream, H.HALF, ta, tb, M, N, K, alpha, beta, rng, device_scalars=dev, pad=pad)
 
 
