@@ -9,10 +9,9 @@
  * A block of NWM x NWN waves owns a (NWM*WM) x (NWN*WN) tile of C, each wave WM x WN of it as 32 x 32 MFMA tiles. Per K
  * step of KT = 64 the block stages slabs of op(A) and op(B) through LDS, loading slab s+1 from memory into registers before the
  * MFMAs of slab s and writing it to the other LDS buffer afterwards. An MFMA operand is eight consecutive k of one row
- * (column) per lane, so both operands are kept [row][k] in LDS (row pitch KT + 8 halves: the 16-byte reads of 16
- * neighbouring rows fall into distinct banks) and a fragment is one 16-byte LDS read. An operand that is contiguous
- * along k in memory ('T' for A, 'N' for B) arrives in that shape; one that is contiguous along m / n is transposed in
- * registers on its way to LDS. Which k a lane holds does not matter as long as A and B agree, and they do by construction.
+ * (column) per lane, so LDS holds both operands as 16-byte chunks of 8 k and a fragment is one 16-byte LDS read per lane.
+ * An operand that is contiguous along k in memory ('T' for A, 'N' for B) arrives in that shape; one that is contiguous
+ * along m / n is transposed in registers on its way to LDS. Which k a lane holds does not matter as long as A and B agree, and they do by construction.
  */
 #include "och_gemm.h"
 
@@ -27,30 +26,34 @@ struct HalfGemmParams
    uint32_t M, N, K;
    half_t   alpha, beta;                /* when the scalars live in host memory */
    const half_t *alpha_dev, *beta_dev;  /* non-null: read the scalar from device memory */
-   int      alignedA, alignedB;         /* base pointer, leading dimension and batch strides allow 128-bit loads */
+   int      alignedA, alignedB, alignedC; /* base pointer, leading dimension and batch strides allow 128-bit accesses */
    uint32_t tiles_m, tiles_n;
    GemmBatch batch;
 };
 
-/* Moves a BMN x KT slab of an operand (2-byte elements) from memory to registers and on to LDS, where it is kept
-   [row][k] with a row pitch of KT + 8 halves; the 16-byte chunk c of row r sits at chunk position c ^ ((r / 16) mod 8).
-   KC (contiguous along k in memory): a thread loads 16 bytes = 8 k of one row and stores them as they are.
+/* Moves a BMN x KT slab of an operand (2-byte elements) from memory to registers and on to LDS.
+   LDS layout: [chunk of 8 k][slot][8 halves], 32 bytes of padding after every chunk plane. A fragment read takes one
+   chunk of 32 neighbouring slots: 512 consecutive bytes.
+   KC (contiguous along k in memory): a thread loads 16 bytes = one chunk of one row; row r sits in slot r. Eight
+   neighbouring lanes store the eight chunks of a row; the padding moves each plane on by eight banks.
    !KC (contiguous along the row index): a thread loads NV consecutive k for 8 neighbouring rows (16 bytes each),
    transposes the 8 x NV block in registers and stores NV k for each of the 8 rows. Neighbouring lanes hold rows that are
-   8 apart; the chunk permutation spreads them over the banks (without it 16 lanes share a bank), and it leaves the
-   fragment reads of 16 neighbouring rows, which the row pitch already keeps apart, as they are. */
+   8 apart, so row r sits in slot (r mod 8) * (BMN / 8) + r / 8: the stores of a wave cover consecutive slots. Which row
+   of the tile an MFMA lane works on is then a matter of bookkeeping when C is written (row_of_slot). */
 template <bool KC, bool EDGE, int BMN, int KT, int THREADS>
 struct HalfSlab
 {
    static constexpr int NV = BMN * KT / 8 / THREADS;                   /* 16-byte loads per thread */
-   static constexpr int PITCH = KT + 8;                                /* LDS row pitch in halves */
-   static constexpr int SIZE = BMN * PITCH;                            /* halves per LDS buffer */
+   static constexpr int PLANE = BMN * 8 + 16;                          /* halves per chunk plane */
+   static constexpr int SIZE = (KT / 8) * PLANE;                       /* halves per LDS buffer */
    static_assert(NV >= 1 && (BMN * KT) % (8 * THREADS) == 0, "slab does not divide among the threads");
    static_assert(KC || NV == 2 || NV == 4 || NV == 8, "the transposing loader needs 2, 4 or 8 k per thread");
-   static_assert(KT == 64, "the chunk permutation assumes 8 chunks per row");
-   static __device__ __forceinline__ uint32_t chunk_at(uint32_t row, uint32_t chunk) { return chunk ^ ((row >> 4) & 7); }
    och_gu32x4 reg[NV];
 
+   static __device__ __forceinline__ uint32_t row_of_slot(uint32_t slot)
+   {  return KC ? slot : (slot % (BMN / 8)) * 8 + slot / (BMN / 8); }
+   /* row_of_slot(s + o) - row_of_slot(s) for offsets o whose sum with s does not carry out of s mod (BMN / 8) */
+   static constexpr uint32_t row_step(uint32_t o) { return KC ? o : (o % (BMN / 8)) * 8 + o / (BMN / 8); }
    static __device__ __forceinline__ void where(int v, uint32_t &mn, uint32_t &k)
    {  if (!KC) { mn = (threadIdx.x % (BMN / 8)) * 8; k = (threadIdx.x / (BMN / 8)) * NV + v; }
       else     { const uint32_t q = threadIdx.x + THREADS * v; k = (q % (KT / 8)) * 8; mn = q / (KT / 8); }
@@ -76,20 +79,20 @@ struct HalfSlab
          }
       }
    }
-   __device__ __forceinline__ void stash(uint16_t *plane) const
+   __device__ __forceinline__ void stash(uint16_t *buffer) const
    {
       if (KC)
       {
 #pragma unroll
          for (int v = 0; v < NV; v++)
          {  uint32_t mn, k; where(v, mn, k);
-            *reinterpret_cast<och_gu32x4 *>(plane + mn * PITCH + chunk_at(mn, k / 8) * 8) = reg[v];
+            *reinterpret_cast<och_gu32x4 *>(buffer + (k / 8) * PLANE + mn * 8) = reg[v];
          }
       }
       else
       {  constexpr int WD = NV / 2;                     /* 32-bit words per row: k pairs */
          uint32_t mn, k; where(0, mn, k);
-         uint16_t *dst = plane + mn * PITCH + chunk_at(mn, k / 8) * 8 + k % 8;      /* mn is a multiple of 8: one chunk position for the 8 rows */
+         uint16_t *dst = buffer + (k / 8) * PLANE + (mn / 8) * 8 + k % 8;          /* row mn + i: slot i * (BMN / 8) + mn / 8 */
 #pragma unroll
          for (int i = 0; i < 8; i++)
          {  uint32_t out[WD];
@@ -98,16 +101,17 @@ struct HalfSlab
             {  const uint32_t x = reg[2 * w][i >> 1], y = reg[2 * w + 1][i >> 1];
                out[w] = (i & 1) ? ((x >> 16) | (y & 0xFFFF0000u)) : ((x & 0xFFFFu) | (y << 16));
             }
-            if (WD == 1) *reinterpret_cast<uint32_t *>(dst + i * PITCH) = out[0];
-            else if (WD == 2) { uint2 t; t.x = out[0]; t.y = out[WD > 1 ? 1 : 0]; *reinterpret_cast<uint2 *>(dst + i * PITCH) = t; }
-            else { och_gu32x4 t; t.x = out[0]; t.y = out[WD > 1 ? 1 : 0]; t.z = out[WD > 2 ? 2 : 0]; t.w = out[WD > 3 ? 3 : 0]; *reinterpret_cast<och_gu32x4 *>(dst + i * PITCH) = t; }
+            uint16_t *at = dst + i * BMN;                /* BMN / 8 slots of 8 halves */
+            if (WD == 1) *reinterpret_cast<uint32_t *>(at) = out[0];
+            else if (WD == 2) { uint2 t; t.x = out[0]; t.y = out[WD > 1 ? 1 : 0]; *reinterpret_cast<uint2 *>(at) = t; }
+            else { och_gu32x4 t; t.x = out[0]; t.y = out[WD > 1 ? 1 : 0]; t.z = out[WD > 2 ? 2 : 0]; t.w = out[WD > 3 ? 3 : 0]; *reinterpret_cast<och_gu32x4 *>(at) = t; }
          }
       }
    }
-   /* the eight k of row `row` that lane group `kg` (0 or 1) feeds to MFMA step `ks` (16 k per step) */
-   static __device__ __forceinline__ och_h8 fragment(const uint16_t *plane, int row, int ks, int kg)
+   /* the eight k of slot `slot` that lane group `kg` (0 or 1) feeds to MFMA step `ks` (16 k per step) */
+   static __device__ __forceinline__ och_h8 fragment(const uint16_t *buffer, int slot, int ks, int kg)
    {  och_h8 f;
-      const och_gu32x4 raw = *reinterpret_cast<const och_gu32x4 *>(plane + row * PITCH + chunk_at(row, ks * 2 + kg) * 8);
+      const och_gu32x4 raw = *reinterpret_cast<const och_gu32x4 *>(buffer + (ks * 2 + kg) * PLANE + slot * 8);
       __builtin_memcpy(&f, &raw, 16);
       return f;
    }
@@ -126,6 +130,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
    int64_t oA, oB, oC, oAlpha, oBeta;
    gemm_batch_offsets(p.batch, oA, oB, oC, oAlpha, oBeta);
    const char *pA = p.A + oA, *pB = p.B + oB; char *pC = p.C + oC;
+   /* (numbering the tiles so that every XCD owns a run of consecutive ones was measured and is slower: 8192^3 TN 958 -> 908 TFLOP/s) */
    const uint32_t tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -173,26 +178,67 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
       __syncthreads();
    }
 
-   /* epilogue: accumulator register r of lane l is C(8 * (r / 4) + 4 * (l / 32) + r % 4, l % 32) of its 32 x 32 tile */
+   /* epilogue: accumulator register r of lane l belongs to slot 8 * (r / 4) + 4 * (l / 32) + r % 4 of A and slot l % 32 of B
+      within its 32 x 32 tile */
    half_t al = p.alpha, be = p.beta;
    if (p.alpha_dev) al = *reinterpret_cast<const half_t *>(reinterpret_cast<const char *>(p.alpha_dev) + oAlpha);
    if (p.beta_dev)  be = *reinterpret_cast<const half_t *>(reinterpret_cast<const char *>(p.beta_dev) + oBeta);
    const float alpha = half_to_float(al), beta = half_to_float(be);
+   /* this lane's part of tile (i, j): rows row0 + row_step(32 i + 8 (r / 4) + r % 4), column col0 + row_step(32 j); the
+      slot offsets added here never carry out of a group of BM / 8 (BN / 8) slots, so the steps are compile-time numbers */
+   const uint32_t row0 = LA::row_of_slot(wm + 4 * (lane >> 5)), col0 = LB::row_of_slot(wn + lane % T);
+   if (beta == 0)
+   {  /* C is only written: the rounded tile goes through LDS (the slab buffers are free after the last barrier), column
+         by column with a pitch of BM + 8 halves, and leaves in 16-byte pieces that follow the columns of C */
+      constexpr int CP = BM + 8;
+      constexpr int PASSES = (BN * CP <= 2 * BUF) ? 1 : ((BN / 2) * CP <= 2 * BUF) ? 2 : 4;
+      constexpr int CPASS = BN / PASSES;
+      static_assert(CPASS * CP <= 2 * BUF, "the staged tile does not fit into the slab buffers");
+      for (int h = 0; h < PASSES; h++)
+      {  uint16_t *mine = lds + ((int)col0 - h * CPASS) * CP + row0;
 #pragma unroll
-   for (int i = 0; i < TMS; i++)
+         for (int j = 0; j < TNS; j++)
+         {  if (PASSES > 1 && (col0 + LB::row_step(j * T)) / CPASS != (uint32_t)h) continue;
 #pragma unroll
-      for (int j = 0; j < TNS; j++)
-      {  const uint32_t col = n0 + wn + j * T + lane % T;
+            for (int i = 0; i < TMS; i++)
+#pragma unroll
+               for (int r = 0; r < 16; r++)
+                  mine[LB::row_step(j * T) * CP + LA::row_step(i * T + 8 * (r >> 2) + (r & 3))] = float_to_half(alpha * acc[i][j][r]).v;
+         }
+         __syncthreads();
+         const uint32_t c0 = n0 + h * CPASS;
+         const bool whole = !EDGE || (p.alignedC && (uint64_t)m0 + BM <= p.M && (uint64_t)c0 + CPASS <= p.N);
+         for (uint32_t q = threadIdx.x; q < CPASS * (BM / 8); q += THREADS)
+         {  const uint32_t c = q / (BM / 8), r8 = (q % (BM / 8)) * 8;
+            const uint16_t *src = lds + c * CP + r8;
+            char *dst = pC + ((int64_t)(m0 + r8) + (int64_t)(c0 + c) * p.ldC) * 2;
+            if (whole) *reinterpret_cast<och_gu32x4 *>(dst) = *reinterpret_cast<const och_gu32x4 *>(src);
+            else if (c0 + c < p.N)
+            {
+#pragma unroll
+               for (int e = 0; e < 8; e++)
+                  if (m0 + r8 + e < p.M) reinterpret_cast<uint16_t *>(dst)[e] = src[e];
+            }
+         }
+         if (h + 1 < PASSES) __syncthreads();
+      }
+      return;
+   }
+   char *mine = pC + ((int64_t)(m0 + row0) + (int64_t)(n0 + col0) * p.ldC) * 2;
+#pragma unroll
+   for (int j = 0; j < TNS; j++)
+   {  if (EDGE && n0 + col0 + LB::row_step(j * T) >= p.N) continue;
+#pragma unroll
+      for (int i = 0; i < TMS; i++)
 #pragma unroll
          for (int r = 0; r < 16; r++)
-         {  const uint32_t row = m0 + wm + i * T + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            if (EDGE && (row >= p.M || col >= p.N)) continue;
-            half_t *c = reinterpret_cast<half_t *>(pC + ((int64_t)row + (int64_t)col * p.ldC) * 2);
-            float v = alpha * acc[i][j][r];
-            if (beta != 0) v += beta * half_to_float(*c);
-            *c = float_to_half(v);
+         {
+            const uint32_t dr = LA::row_step(i * T + 8 * (r >> 2) + (r & 3));
+            if (EDGE && m0 + row0 + dr >= p.M) continue;
+            half_t *c = reinterpret_cast<half_t *>(mine + ((int64_t)dr + (int64_t)LB::row_step(j * T) * p.ldC) * 2);
+            *c = float_to_half(alpha * acc[i][j][r] + beta * half_to_float(*c));
          }
-      }
+   }
 }
 
 template <int WM, int WN, int NWM, int NWN, int KT>
@@ -217,7 +263,8 @@ static int launch_gemm_half(const GemmArgs &g)
       return ok;
    };
    p.alignedA = aligned(g.A, g.ldA, g.batch.sA) ? 1 : 0; p.alignedB = aligned(g.B, g.ldB, g.batch.sB) ? 1 : 0;
-   const bool edge = !(g.M % BM == 0 && g.N % BN == 0 && g.K % KT == 0 && p.alignedA && p.alignedB);
+   p.alignedC = aligned(g.C, g.ldC, g.batch.sC) ? 1 : 0;
+   const bool edge = !(g.M % BM == 0 && g.N % BN == 0 && g.K % KT == 0 && p.alignedA && p.alignedB && p.alignedC);
    const dim3 grid((unsigned)blocks, 1, g.nz), block(THREADS);
    /* both LDS buffers; above 64 KB the kernel has to be told */
 #define OCH_HGEMM_LAUNCH(AK, BK, EDGE)                                                                                   \
@@ -237,9 +284,9 @@ static int launch_gemm_half(const GemmArgs &g)
 }
 
 /* returns 1 when the product is left to the generic kernel (very small results or K).
-   Measured at 8192^3 (NN / NT / TN / TT, TFLOP/s): 256 x 256 tiles with eight waves 711 / 758 / 904 / 846,
-   128 x 128 tiles with four waves 610 / 608 / 791 / 737; at 4096^3 (256 tiles of 256 x 256) 661 / 556 / 650 / 621
-   against 617 / 473 / 594 / 585. */
+   Measured at 8192^3 (NN / NT / TN / TT, TFLOP/s): 256 x 256 tiles with eight waves 763 / 841 / 958 / 947; with
+   128 x 128 tiles and four waves the same kernel stays 15 - 25 % below that. 4096^3 (256 tiles of 256 x 256):
+   793 / 653 / 720 / 696. */
 int gemm_half(const GemmArgs &g)
 {
    if (g.M < 32 || g.N < 32 || g.K < 16) return 1;
