@@ -86,12 +86,27 @@ typedef struct {
    int      pci_bus_id, pci_device_id, pci_domain_id;
    int      concurrent_kernels;
    int      ecc_enabled;
+   /* the remaining fields of OcDevicePropGPU (include/ocean/core/gpu/device_gpu.h:31-75) that HIP reports */
+   size_t   free_global_mem;          /* at the time of the query; och_device_mem_info refreshes it */
+   size_t   total_const_mem;
+   size_t   mem_pitch;
+   int      regs_per_block;
+   int      max_threads_dim[3];
+   int      max_grid_size[3];
+   int      major, minor;             /* gfx950 reports 9.5 */
+   int      async_engine_count;       /* > 0: copies overlap kernels (deviceOverlap) */
+   int      kernel_exec_timeout_enabled;
+   int      integrated;
+   int      can_map_host_memory;
+   int      compute_mode;
+   int      tcc_driver;               /* always 0 */
 } och_device_prop;
 
 int och_device_count(int *count);                          /* device_gpu.c:184 cudaGetDeviceCount */
 int och_device_set(int device);                            /* cuda.c:67 OcCuda_setDevice */
 int och_device_get(int *device);
-int och_device_properties(int device, och_device_prop *p); /* device_gpu.c:471-637 */
+int och_device_properties(int device, och_device_prop *p); /* device_gpu.c:471-616 */
+int och_device_mem_info(int device, size_t *free_bytes, size_t *total_bytes); /* device_gpu.c:620-637 updateProperties */
 int och_device_can_access_peer(int device, int peer, int *result); /* device_gpu.c:447-454 */
 int och_device_warmup(int device);                         /* device_gpu.c:155-172 + template_dummy.cu:21-37 */
 int och_device_synchronize(void);

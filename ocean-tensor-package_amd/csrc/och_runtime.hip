@@ -131,6 +131,26 @@ int och_device_properties(int device, och_device_prop *p)
    p->pci_bus_id = d.pciBusID; p->pci_device_id = d.pciDeviceID; p->pci_domain_id = d.pciDomainID;
    p->concurrent_kernels = d.concurrentKernels;
    p->ecc_enabled = d.ECCEnabled;
+   p->total_const_mem = d.totalConstMem; p->mem_pitch = d.memPitch; p->regs_per_block = d.regsPerBlock;
+   for (int i = 0; i < 3; i++) { p->max_threads_dim[i] = d.maxThreadsDim[i]; p->max_grid_size[i] = d.maxGridSize[i]; }
+   p->major = d.major; p->minor = d.minor;
+   p->async_engine_count = d.asyncEngineCount;
+   p->kernel_exec_timeout_enabled = d.kernelExecTimeoutEnabled;
+   p->integrated = d.integrated; p->can_map_host_memory = d.canMapHostMemory; p->compute_mode = d.computeMode;
+   p->tcc_driver = 0;
+   size_t total = 0;
+   return och_device_mem_info(device, &p->free_global_mem, &total);
+}
+
+int och_device_mem_info(int device, size_t *free_bytes, size_t *total_bytes)
+{
+   int prev;
+   if (!free_bytes || !total_bytes) return och::set_error("och_device_mem_info: null argument");
+   OCH_CHECK_HIP(hipGetDevice(&prev));
+   OCH_CHECK_HIP(hipSetDevice(device));
+   const hipError_t e = hipMemGetInfo(free_bytes, total_bytes);
+   OCH_CHECK_HIP(hipSetDevice(prev));
+   OCH_CHECK_HIP(e);
    return 0;
 }
 

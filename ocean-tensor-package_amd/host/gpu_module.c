@@ -520,6 +520,25 @@ OcModuleCore *OcModuleCore_forDevice(OcDevice *device)
    return &oc_registered_gpu;
 }
 int OcDeviceGPUCount(void) { return oc_gpu_count; }
+OcDevice *OcDeviceGPUByIndex(int index) { return (index >= 0 && index < oc_gpu_count) ? OcGPU[index] : NULL; }
+int OcDeviceGPU_isInstance(OcDevice *device)
+{  int i;
+   for (i = 0; i < oc_gpu_count; i++) if (OcGPU[i] == device) return 1;
+   return 0;
+}
+int OcDeviceGPU_peerAccess(int device1, int device2)
+{  int result = 0;
+   if (device1 == device2) return 1;
+   if (och_device_can_access_peer(device1, device2, &result) != 0) return 0;
+   return result;
+}
+int OcDeviceGPU_properties(OcDevice *device, void *och_device_prop_out)
+{  OcDeviceGPU *g = (OcDeviceGPU *)device; size_t total = 0;
+   if (!OcDeviceGPU_isInstance(device) || och_device_prop_out == NULL) return OcErrorMessage("Device properties: not a GPU device");
+   OCH_CALL(och_device_mem_info(device->index, &g->properties.free_global_mem, &total));
+   memcpy(och_device_prop_out, &g->properties, sizeof(g->properties));
+   return 0;
+}
 
 int OcInitGPU(void)
 {  int i, count = 0;

@@ -37,6 +37,11 @@ extern OcDevice **OcGPU;                    /* OcGPU[i], i < OcDeviceGPUCount() 
 int  OcInitGPU(void);                       /* ocean_gpu.c:38-58: idempotent; creates devices, fills and registers the table */
 void OcFinalizeGPU(void);
 int  OcDeviceGPUCount(void);
+OcDevice *OcDeviceGPUByIndex(int index);   /* device_gpu.c:437-443: NULL when out of range */
+int  OcDeviceGPU_isInstance(OcDevice *device);                       /* device_gpu.c:458-462 */
+int  OcDeviceGPU_peerAccess(int device1, int device2);               /* device_gpu.c:447-454 */
+/* device_gpu.c:471-637: the cached properties of a GPU device, with the amount of free memory refreshed (updateProperties) */
+int  OcDeviceGPU_properties(OcDevice *device, void *och_device_prop_out);
 OcModuleCore *OcModuleCore_forDevice(OcDevice *device);   /* what OC_GET_CORE_FUNCTION resolves against */
 int  OcRegisterModule(const char *deviceType, OcDeviceModule *info, size_t size);
 

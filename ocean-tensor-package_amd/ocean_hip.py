@@ -110,7 +110,12 @@ class DeviceProp(C.Structure):
                 ("max_threads_per_block", C.c_int), ("max_threads_per_multiprocessor", C.c_int),
                 ("clock_rate_khz", C.c_int), ("memory_clock_rate_khz", C.c_int), ("memory_bus_width", C.c_int),
                 ("l2_cache_size", C.c_int), ("pci_bus_id", C.c_int), ("pci_device_id", C.c_int),
-                ("pci_domain_id", C.c_int), ("concurrent_kernels", C.c_int), ("ecc_enabled", C.c_int)]
+                ("pci_domain_id", C.c_int), ("concurrent_kernels", C.c_int), ("ecc_enabled", C.c_int),
+                ("free_global_mem", C.c_size_t), ("total_const_mem", C.c_size_t), ("mem_pitch", C.c_size_t),
+                ("regs_per_block", C.c_int), ("max_threads_dim", C.c_int * 3), ("max_grid_size", C.c_int * 3),
+                ("major", C.c_int), ("minor", C.c_int), ("async_engine_count", C.c_int),
+                ("kernel_exec_timeout_enabled", C.c_int), ("integrated", C.c_int), ("can_map_host_memory", C.c_int),
+                ("compute_mode", C.c_int), ("tcc_driver", C.c_int)]
 
 
 class ReduceAxisConfig(C.Structure):
@@ -132,6 +137,7 @@ PROTOTYPES = {
     "och_device_set": (_i, [_i]),
     "och_device_get": (_i, [C.POINTER(_i)]),
     "och_device_properties": (_i, [_i, C.POINTER(DeviceProp)]),
+    "och_device_mem_info": (_i, [_i, _sz, _sz]),
     "och_device_can_access_peer": (_i, [_i, _i, C.POINTER(_i)]),
     "och_device_warmup": (_i, [_i]),
     "och_device_synchronize": (_i, []),

@@ -109,6 +109,19 @@ def _need(ptr):
     return ptr
 
 
+def dtype_of(numpy_dtype):
+    """Ocean data type of a numpy dtype (bool -> bool, float16 -> half; anything else by item type)."""
+    dt = np.dtype(numpy_dtype)
+    if dt == np.bool_:
+        return BOOL
+    if dt == np.float16:
+        return HALF
+    for code in (UINT8, UINT16, UINT32, UINT64, INT8, INT16, INT32, INT64, FLOAT, DOUBLE, CFLOAT, CDOUBLE):
+        if np.dtype(NUMPY[code]) == dt:
+            return code
+    raise OceanError("no Ocean data type for numpy dtype %s" % dt)
+
+
 def cpu_device():
     return C.c_void_p.in_dll(lib, "OcCPU")
 
