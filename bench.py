@@ -371,6 +371,18 @@ def main():
             oh.check(lib.och_graph_destroy(graph))
             configs["c5_mgs_qr_4096_first64cols_graph_replay"] = {"us_per_pair": round(dt_g / pairs * 1e6, 2), "launches_per_pair": 2,
                                                                   "effective_GBps": round(pairs * (2 * 8 * m + 3 * 8 * m) / dt_g / 1e9, 1)}
+        # the same window through the fused projection: one launch per column instead of two per pair
+        if "och_mgs_project" not in oh.MISSING:
+            def mgs_fused():
+                for j in range(1, 64):
+                    lib.och_mgs_project(F64, m, j, q.ptr, m, col(j), C.c_void_p(rr.address + 8 * 64 * j), h)
+            mgs_fused(); stream.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                mgs_fused()
+            stream.synchronize(); dt_f = (time.perf_counter() - t0) / 3
+            configs["c5_mgs_qr_4096_first64cols_fused_projection"] = {"us_per_pair": round(dt_f / pairs * 1e6, 3), "launches_per_pair": round(63 / pairs, 4),
+                                                                      "effective_GBps": round(pairs * (2 * 8 * m + 3 * 8 * m) / dt_f / 1e9, 1)}
         for b in (q, rr, consts):
             b.free()
     result["configs"] = configs

@@ -328,6 +328,15 @@ int och_gemm_batched(int dtype, char transA, char transB, size_t M, size_t N, si
                      const ptrdiff_t *stride_beta, const ptrdiff_t *strideC,
                      int scalar_mode_host, och_stream stream);
 
+/* Fused projection step of a modified Gram-Schmidt sweep. No counterpart in the reference, whose callers issue one    */
+/* dot product (gemm with M = N = 1) and one rank-1 update per pair of columns, i.e. 2 k launches for this:             */
+/*    for i = 0 .. k-1 (in this order):  r[i] = q_i^H v;   v <- v - r[i] q_i                                            */
+/* q_i = Q + i * ldq (ldq in elements) and v are dense vectors of n elements in device memory; r (k elements, device   */
+/* memory) receives the coefficients and may be NULL. dtype: OCH_FLOAT, OCH_DOUBLE, OCH_CFLOAT, OCH_CDOUBLE. One launch */
+/* for n <= 16384 (the vector stays in the registers of one workgroup); longer vectors run the two gemm launches per    */
+/* column and need r. Dot products accumulate in double, as och_gemm's do.                                               */
+int och_mgs_project(int dtype, size_t n, size_t k, const void *Q, ptrdiff_t ldq, void *v, void *r, och_stream stream);
+
 /* ======================================================================== */
 /* Index operations (template_index.cu:37-57, index1.h:182, index2.h:188)   */
 /* ======================================================================== */

@@ -465,6 +465,32 @@ static int OcTensorGPU_gemm(OcSize M, OcSize N, OcSize K, char transA, char tran
 }
 static int OcTensorGPU_gemmSupportedOn(OcDevice *device, OcDType dtype) { (void)device; return och_gemm_supported(dtype); }
 
+/* ---- beside the table: fused Gram-Schmidt projection (no slot in OcModuleCore, no counterpart in the reference) -------- */
+/* v <- v - sum_i q_i (q_i^H v), one column of Q after the other; Q is n x k with dense columns, v a dense vector of n
+   elements, r NULL or a dense vector of k elements that receives the coefficients; all on the same GPU, same type */
+int OcTensorGPU_projectColumns(OcTensor *Q, OcTensor *v, OcTensor *r)
+{  OcSize n, k; OcIndex es;
+   if (Q == NULL || v == NULL) return OcErrorMessage("projectColumns: missing operand");
+   es = OcDType_size(Q->dtype);
+   if (!OcDeviceGPU_isInstance(Q->device) || v->device != Q->device || (r && r->device != Q->device))
+      return OcErrorMessage("projectColumns: all tensors must be on the same GPU device");
+   if (v->dtype != Q->dtype || (r && r->dtype != Q->dtype)) return OcErrorMessage("projectColumns: mismatch in data types");
+   if (Q->ndims < 1 || Q->ndims > 2 || v->ndims != 1) return OcErrorMessage("projectColumns: Q must be a matrix and v a vector");
+   n = Q->size[0]; k = (Q->ndims == 2) ? Q->size[1] : 1;
+   if (v->size[0] != n || (r && (r->ndims != 1 || r->size[0] != k))) return OcErrorMessage("projectColumns: mismatch in tensor sizes");
+   if ((n > 1 && (Q->strides[0] != es || v->strides[0] != es)) || (r && k > 1 && r->strides[0] != es) ||
+       (Q->ndims == 2 && k > 1 && (Q->strides[1] % es != 0 || Q->strides[1] < (OcIndex)(n * es))))
+      return OcErrorMessage("projectColumns: columns and vectors must be dense");
+   if (n == 0 || k == 0) return 0;
+   if (activate(v->device) != 0 || OcTensor_startRead(v, Q) != 0) return -1;
+   if (r && OcTensor_startRead(v, r) != 0) return -1;             /* r is written on v's stream: order it behind r's own work */
+   OCH_CALL(och_mgs_project(Q->dtype, (size_t)n, (size_t)k, OcTensor_data(Q), (Q->ndims == 2 && k > 1) ? Q->strides[1] / es : (OcIndex)n,
+                            OcTensor_data(v), r ? OcTensor_data(r) : NULL, GPU_STREAM(v)));
+   if (OcTensor_update(v) != 0) return -1;
+   if (r && OcTensor_finishRead(v, r) != 0) return -1;
+   return OcTensor_finishRead(v, Q);
+}
+
 /* ---- module table and registration ------------------------------------------------------------ */
 static int gpu_initialize_context(OcDevice *device, OcDeviceModule *module, void **context)
 {  OcModuleCore_Context *ctx = (OcModuleCore_Context *)calloc(1, sizeof(OcModuleCore_Context));

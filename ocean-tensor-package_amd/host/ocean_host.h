@@ -42,6 +42,8 @@ int  OcDeviceGPU_isInstance(OcDevice *device);                       /* device_g
 int  OcDeviceGPU_peerAccess(int device1, int device2);               /* device_gpu.c:447-454 */
 /* device_gpu.c:471-637: the cached properties of a GPU device, with the amount of free memory refreshed (updateProperties) */
 int  OcDeviceGPU_properties(OcDevice *device, void *och_device_prop_out);
+/* beside the module table (no counterpart in the reference): v <- v - sum_i q_i (q_i^H v), columns in order; r may be NULL */
+int  OcTensorGPU_projectColumns(OcTensor *Q, OcTensor *v, OcTensor *r);
 OcModuleCore *OcModuleCore_forDevice(OcDevice *device);   /* what OC_GET_CORE_FUNCTION resolves against */
 int  OcRegisterModule(const char *deviceType, OcDeviceModule *info, size_t size);
 

@@ -192,6 +192,7 @@ PROTOTYPES = {
     "och_gemm_supported": (_i, [_i]),
     "och_gemm_batched": (_i, [_i, C.c_char, C.c_char, C.c_size_t, C.c_size_t, C.c_size_t, _vp, _vp, C.c_ssize_t, _vp, C.c_ssize_t,
                               _vp, _vp, C.c_ssize_t, _i, _sz, _st, _st, _st, _st, _st, _i, _vp]),
+    "och_mgs_project": (_i, [_i, C.c_size_t, C.c_size_t, _vp, C.c_ssize_t, _vp, _vp, _vp]),
     "och_add_if_negative": (_i, [_i, _i, _sz, _st, _vp, Scalar, _vp]),
     "och_index_to_offset": (_i, [_i, _i, C.POINTER(C.c_int64), C.c_ssize_t, C.c_size_t, C.c_ssize_t, _vp, C.c_ssize_t, _vp, _vp]),
     "och_get_index": (_i, [_i, _i, _sz, C.POINTER(C.POINTER(C.c_int64)), _st, _vp, _st, _vp, _vp]),

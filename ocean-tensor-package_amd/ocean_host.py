@@ -85,6 +85,7 @@ lib.OcTensor_axisReduce.argtypes = [C.c_int, TP, C.c_int, C.POINTER(C.c_int), C.
 lib.OcTensor_gemm.argtypes = [C.POINTER(Scalar), TP, C.c_char, TP, C.c_char, C.POINTER(Scalar), C.POINTER(TP)]
 lib.OcTensor_mtimes.argtypes = [TP, TP, C.POINTER(TP)]
 lib.OcTensor_fill.argtypes = [TP, C.POINTER(Scalar)]
+lib.OcTensorGPU_projectColumns.argtypes = [TP, TP, TP]
 lib.OcTensor_find.restype = TP
 lib.OcTensor_find.argtypes = [TP]
 lib.OcTensor_maskToOffset.restype = TP

@@ -235,3 +235,46 @@ def test_batched_gemm_with_broadcast_through_the_front_end(gpu):
     assert np.array_equal(host.to_numpy(tc), 2 * np.einsum("xkm,xnk->xnm", Ai, Bi) - C0)
     with pytest.raises(host.OceanError, match="not compatible"):
         host.check(host.lib.OcTensor_mtimes(tA, host.from_numpy(rng.uniform(-1, 1, (2, 2, n, k)), host.DOUBLE, gpu), C.byref(host.TP())))
+
+
+def test_gram_schmidt_with_the_fused_projection(gpu):
+    """A modified Gram-Schmidt factorisation A = Q R through the front end: every column is made orthogonal to the finished
+    ones by OcTensorGPU_projectColumns (one launch; the reference's example issues a dot product and an update per pair),
+    normalised with norm2 and a scale. Checked through what a QR factorisation must satisfy: Q'Q = I, Q R = A, R upper
+    triangular with the norms on its diagonal; and against numpy's QR up to the signs of the columns."""
+    rng = np.random.default_rng(21)
+    n, k = 300, 24
+    A = rng.uniform(-1, 1, (k, n))                      # numpy (k, n) = Ocean (n, k): columns contiguous
+    tA = host.from_numpy(A, host.DOUBLE, gpu)
+    tR = host.from_numpy(np.zeros((k, k)), host.DOUBLE, gpu)
+    NORM2, DIVIDE = 27, 3
+    for j in range(k):
+        colj = host.lib.OcTensor_slice(tA, 1, j, 1, 1)               # Ocean (n, 1)
+        vj = host.lib.OcTensor_slice(tA, 1, j, 1, 1)
+        vj.contents.ndims = 1                                        # the column as a vector
+        if j > 0:
+            Qj = host.lib.OcTensor_slice(tA, 1, 0, j, 1)
+            rj = host.lib.OcTensor_slice(tR, 1, j, 1, 1); rj.contents.ndims = 1; rj.contents.size[0] = j; rj.contents.nelem = j
+            host.check(host.lib.OcTensorGPU_projectColumns(Qj, vj, rj))
+        nrm = host.Scalar()
+        host.check(host.lib.OcTensor_reduceAll(NORM2, vj, 0.0, C.byref(nrm)))
+        d = nrm.get()
+        host.check(host.lib.OcTensor_fill(host.lib.OcTensor_slice(host.lib.OcTensor_slice(tR, 1, j, 1, 1), 0, j, 1, 1), C.byref(host.scalar(host.DOUBLE, d))))
+        inv = host.from_numpy(np.array([1.0 / d]), host.DOUBLE, gpu)
+        out = vj
+        host.check(host.lib.OcTensor_binary(SCALE, vj, host.lib.OcTensor_broadcastTo(inv, 1, host._arr([n])), C.byref(out)))
+    Q = host.to_numpy(tA).T                              # (n, k)
+    R = host.to_numpy(tR).T                              # (k, k): column j holds the coefficients of column j
+    assert np.allclose(np.tril(R, -1), 0)
+    assert np.linalg.norm(Q.T @ Q - np.eye(k)) < 1e-12
+    assert np.linalg.norm(Q @ R - A.T) < 1e-12 * np.linalg.norm(A)
+    qn, rn = np.linalg.qr(A.T)
+    sign = np.sign(np.diag(rn))
+    assert np.linalg.norm(Q - qn * sign) < 1e-10 and np.linalg.norm(R - (rn.T * sign).T) < 1e-10
+    # argument checks
+    with pytest.raises(host.OceanError, match="same GPU"):
+        host.check(host.lib.OcTensorGPU_projectColumns(tA, host.from_numpy(np.zeros(n), host.DOUBLE), None))
+    with pytest.raises(host.OceanError, match="data types"):
+        host.check(host.lib.OcTensorGPU_projectColumns(tA, host.from_numpy(np.zeros(n, np.float32), host.FLOAT, gpu), None))
+    with pytest.raises(host.OceanError, match="sizes"):
+        host.check(host.lib.OcTensorGPU_projectColumns(tA, host.from_numpy(np.zeros(n + 1), host.DOUBLE, gpu), None))
