@@ -29,6 +29,10 @@ struct HalfGemmParams
    int      alignedA, alignedB, alignedC; /* base pointer, leading dimension and batch strides allow 128-bit accesses */
    uint32_t tiles_m, tiles_n;
    GemmBatch batch;
+   /* split K (few tiles, long K; only without a batch): grid z is the slice, every slice covers split_slabs slabs of K and
+      leaves its raw float sums in partial[z] (dense M x N planes); gemm_half_finish_kernel adds the slices in order */
+   uint32_t split_slabs;
+   float   *partial;
 };
 
 /* Moves a BMN x KT slab of an operand (2-byte elements) from memory to registers and on to LDS.
@@ -61,19 +65,26 @@ struct HalfSlab
    /* element (mn, k) of op(.) lives at mn + k * ld (!KC) or k + mn * ld (KC) */
    __device__ __forceinline__ void fetch(const char *mat, int64_t ld, uint32_t mn0, uint32_t k0, uint32_t MN, uint32_t K, int aligned)
    {
-      const bool wide = !EDGE || (aligned && (uint64_t)mn0 + BMN <= MN && (uint64_t)k0 + KT <= K);
 #pragma unroll
       for (int v = 0; v < NV; v++)
       {  uint32_t mn, k; where(v, mn, k);
          const int64_t gm = (int64_t)mn0 + mn, gk = (int64_t)k0 + k;
-         if (wide) reg[v] = *reinterpret_cast<const och_gu32x4 *>(mat + (KC ? (gk + gm * ld) : (gm + gk * ld)) * 2);
+         const char *at = mat + (KC ? (gk + gm * ld) : (gm + gk * ld)) * 2;
+         if (!EDGE) { reg[v] = *reinterpret_cast<const och_gu32x4 *>(at); continue; }
+         /* edge tiles: a vector that lies inside the matrix (and is aligned) is still one load, one that lies outside is
+            zero without touching memory; element-wise loads remain for vectors that straddle the border or are unaligned */
+         const bool some = KC ? (gm < (int64_t)MN && gk < (int64_t)K) : (gk < (int64_t)K && gm < (int64_t)MN);
+         const bool all  = KC ? (gm < (int64_t)MN && gk + 8 <= (int64_t)K) : (gk < (int64_t)K && gm + 8 <= (int64_t)MN);
+         if (all && aligned) reg[v] = *reinterpret_cast<const och_gu32x4 *>(at);
          else
          {  uint32_t w[4] = { 0, 0, 0, 0 };
+            if (some)
+            {
 #pragma unroll
-            for (int e = 0; e < 8; e++)
-            {  const int64_t em = gm + (KC ? 0 : e), ek = gk + (KC ? e : 0);
-               if (em < (int64_t)MN && ek < (int64_t)K)
-                  w[e >> 1] |= (uint32_t)*reinterpret_cast<const uint16_t *>(mat + (KC ? (ek + em * ld) : (em + ek * ld)) * 2) << (16 * (e & 1));
+               for (int e = 0; e < 8; e++)
+               {  const bool ok = KC ? (gk + e < (int64_t)K) : (gm + e < (int64_t)MN);
+                  if (ok) w[e >> 1] |= (uint32_t)*reinterpret_cast<const uint16_t *>(at + 2 * e) << (16 * (e & 1));
+               }
             }
             reg[v].x = w[0]; reg[v].y = w[1]; reg[v].z = w[2]; reg[v].w = w[3];
          }
@@ -145,10 +156,14 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
          for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
 
    LA la; LB lb;
-   const uint32_t nslabs = (p.K + KT - 1) / KT;
+   uint32_t slab0 = 0, nslabs = (p.K + KT - 1) / KT;
+   if (p.split_slabs)
+   {  slab0 = blockIdx.z * p.split_slabs;
+      nslabs = (slab0 + p.split_slabs < nslabs) ? p.split_slabs : (slab0 < nslabs ? nslabs - slab0 : 0);
+   }
    if (nslabs > 0)
-   {  la.fetch(pA, p.ldA, m0, 0, p.M, p.K, p.alignedA);
-      lb.fetch(pB, p.ldB, n0, 0, p.N, p.K, p.alignedB);
+   {  la.fetch(pA, p.ldA, m0, slab0 * KT, p.M, p.K, p.alignedA);
+      lb.fetch(pB, p.ldB, n0, slab0 * KT, p.N, p.K, p.alignedB);
       la.stash(lds); lb.stash(lds + LA::SIZE);
    }
    __syncthreads();
@@ -156,8 +171,8 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
    {  const uint16_t *As = lds + (s & 1) * BUF, *Bs = As + LA::SIZE;
       const bool more = s + 1 < nslabs;
       if (more)
-      {  la.fetch(pA, p.ldA, m0, (s + 1) * KT, p.M, p.K, p.alignedA);
-         lb.fetch(pB, p.ldB, n0, (s + 1) * KT, p.N, p.K, p.alignedB);
+      {  la.fetch(pA, p.ldA, m0, (slab0 + s + 1) * KT, p.M, p.K, p.alignedA);
+         lb.fetch(pB, p.ldB, n0, (slab0 + s + 1) * KT, p.N, p.K, p.alignedB);
       }
 #pragma unroll
       for (int ks = 0; ks < KT / 16; ks++)
@@ -178,6 +193,25 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
       __syncthreads();
    }
 
+   const uint32_t row0 = LA::row_of_slot(wm + 4 * (lane >> 5)), col0 = LB::row_of_slot(wn + lane % T);
+   if (p.split_slabs)
+   {  /* raw sums of this K slice */
+      float *plane = p.partial + (size_t)blockIdx.z * p.M * p.N;
+#pragma unroll
+      for (int j = 0; j < TNS; j++)
+      {  const uint32_t col = n0 + col0 + LB::row_step(j * T);
+         if (col >= p.N) continue;
+#pragma unroll
+         for (int i = 0; i < TMS; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+            {  const uint32_t row = m0 + row0 + LA::row_step(i * T + 8 * (r >> 2) + (r & 3));
+               if (row < p.M) plane[(size_t)col * p.M + row] = acc[i][j][r];
+            }
+      }
+      return;
+   }
+
    /* epilogue: accumulator register r of lane l belongs to slot 8 * (r / 4) + 4 * (l / 32) + r % 4 of A and slot l % 32 of B
       within its 32 x 32 tile */
    half_t al = p.alpha, be = p.beta;
@@ -186,7 +220,6 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
    const float alpha = half_to_float(al), beta = half_to_float(be);
    /* this lane's part of tile (i, j): rows row0 + row_step(32 i + 8 (r / 4) + r % 4), column col0 + row_step(32 j); the
       slot offsets added here never carry out of a group of BM / 8 (BN / 8) slots, so the steps are compile-time numbers */
-   const uint32_t row0 = LA::row_of_slot(wm + 4 * (lane >> 5)), col0 = LB::row_of_slot(wn + lane % T);
    if (beta == 0)
    {  /* C is only written: the rounded tile goes through LDS (the slab buffers are free after the last barrier), column
          by column with a pitch of BM + 8 halves, and leaves in 16-byte pieces that follow the columns of C */
@@ -241,6 +274,29 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
    }
 }
 
+/* adds the K slices of a split product in slice order, applies alpha / beta and rounds: one thread per element of C */
+__global__ __launch_bounds__(256) void gemm_half_finish_kernel(const HalfGemmParams p, uint32_t slices)
+{
+   const uint64_t e = (uint64_t)blockIdx.x * 256 + threadIdx.x, mn = (uint64_t)p.M * p.N;
+   if (e >= mn) return;
+   const uint32_t col = (uint32_t)(e / p.M), row = (uint32_t)(e - (uint64_t)col * p.M);
+   float s = 0;
+   uint32_t t = 0;
+   for (; t + 7 < slices; t += 8)
+   {  float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) v[u] = p.partial[(size_t)(t + u) * mn + e];
+#pragma unroll
+      for (int u = 0; u < 8; u++) s += v[u];
+   }
+   for (; t < slices; t++) s += p.partial[(size_t)t * mn + e];
+   const float alpha = half_to_float(p.alpha_dev ? *p.alpha_dev : p.alpha), beta = half_to_float(p.beta_dev ? *p.beta_dev : p.beta);
+   half_t *c = reinterpret_cast<half_t *>(p.C) + ((int64_t)row + (int64_t)col * p.ldC);
+   float v = alpha * s;
+   if (beta != 0) v += beta * half_to_float(*c);
+   *c = float_to_half(v);
+}
+
 template <int WM, int WN, int NWM, int NWN, int KT>
 static int launch_gemm_half(const GemmArgs &g)
 {
@@ -265,7 +321,26 @@ static int launch_gemm_half(const GemmArgs &g)
    p.alignedA = aligned(g.A, g.ldA, g.batch.sA) ? 1 : 0; p.alignedB = aligned(g.B, g.ldB, g.batch.sB) ? 1 : 0;
    p.alignedC = aligned(g.C, g.ldC, g.batch.sC) ? 1 : 0;
    const bool edge = !(g.M % BM == 0 && g.N % BN == 0 && g.K % KT == 0 && p.alignedA && p.alignedB && p.alignedC);
-   const dim3 grid((unsigned)blocks, 1, g.nz), block(THREADS);
+   /* few tiles and a long K: slices of K in grid z, at least 8 slabs each, about 512 blocks in all, partial sums within the workspace */
+   uint32_t slices = 1;
+   {  const uint64_t nslabs = (g.K + KT - 1) / KT;
+      if (g.batch.nb == 0 && blocks < 128 && nslabs >= 32)
+      {  uint64_t want = (512 + blocks - 1) / blocks;
+         if (want > nslabs / 8) want = nslabs / 8;
+         const uint64_t fit = OCH_GEMM_WORKSPACE / ((uint64_t)g.M * g.N * sizeof(float));
+         if (want > fit) want = fit;
+         if (want > 65535) want = 65535;
+         if (want >= 2)
+         {  char *ws;
+            if (stream_gemm_workspace(g.stream, &ws) != 0) return -1;
+            p.split_slabs = (uint32_t)((nslabs + want - 1) / want);
+            slices = (uint32_t)((nslabs + p.split_slabs - 1) / p.split_slabs);
+            p.partial = reinterpret_cast<float *>(ws);
+            if (slices < 2) { slices = 1; p.split_slabs = 0; p.partial = nullptr; }
+         }
+      }
+   }
+   const dim3 grid((unsigned)blocks, 1, slices > 1 ? slices : g.nz), block(THREADS);
    /* both LDS buffers; above 64 KB the kernel has to be told */
 #define OCH_HGEMM_LAUNCH(AK, BK, EDGE)                                                                                   \
    do { auto kernel = gemm_half_kernel<AK, BK, EDGE, WM, WN, NWM, NWN, KT>;                                              \
@@ -279,17 +354,21 @@ static int launch_gemm_half(const GemmArgs &g)
    else              OCH_HGEMM_PICK(true, true);
 #undef OCH_HGEMM_PICK
 #undef OCH_HGEMM_LAUNCH
+   if (slices > 1)
+      hipLaunchKernelGGL(gemm_half_finish_kernel, dim3((unsigned)(((uint64_t)g.M * g.N + 255) / 256)), dim3(256), 0, g.stream, p, slices);
    OCH_CHECK_LAUNCH();
    return 0;
 }
 
-/* returns 1 when the product is left to the generic kernel (very small results or K).
+/* returns 1 when the product is left to the generic kernel (K < 16). Small results run on the 64 x 64 tile with the part
+   outside the matrices read as zero -- the matrix cores are fast enough for that to beat a scalar kernel -- and products
+   with few tiles and a long K are cut along K.
    Measured at 8192^3 (NN / NT / TN / TT, TFLOP/s): 256 x 256 tiles with eight waves 763 / 841 / 958 / 947; with
    128 x 128 tiles and four waves the same kernel stays 15 - 25 % below that. 4096^3 (256 tiles of 256 x 256):
    793 / 653 / 720 / 696. */
 int gemm_half(const GemmArgs &g)
 {
-   if (g.M < 32 || g.N < 32 || g.K < 16) return 1;
+   if (g.K < 16) return 1;                      /* C <- beta C, and updates of so low a rank that writing C is all there is */
    const uint64_t big = ((g.M + 255) / 256) * ((g.N + 255) / 256) * (uint64_t)g.nz;
    if (big >= 192) return launch_gemm_half<64, 128, 4, 2, 64>(g);
    if (!gemm_few_tiles(g, 128, 128)) return launch_gemm_half<64, 64, 2, 2, 64>(g);

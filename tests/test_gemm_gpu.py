@@ -138,7 +138,11 @@ def test_gemm_half_matrix_cores(hip, stream, ta, tb):
     for (M, N, K, pad, alpha, beta, dev) in [(128, 128, 64, 0, 1, 0, False), (256, 384, 96, 8, 2, -1, False), (200, 136, 100, 3, 1, 1, True),
                                               (64, 64, 32, 0, -1, 0.5, False), (96, 160, 2048, 0, 0.5, 0, True), (33, 47, 17, 5, 1, 0, False),
                                               (2560, 2304, 48, 0, 1, 1, False), (2500, 2300, 40, 4, 1, 0, False), (4096, 3072, 64, 0, 1, 0, False),
-                                              (4000, 3100, 70, 0, -1, 1, True)]:
+                                              (4000, 3100, 70, 0, -1, 1, True),
+                                              # results narrower than a tile, vectors, K below one MFMA step, K not a multiple of 8
+                                              (2000, 1, 1000, 0, 1, 0, False), (1, 1500, 999, 0, 1, 1, False), (700, 9, 3, 1, 2, 0, False), (31, 31, 15, 0, 1, 0, False),
+                                              # few tiles and a long K: cut along K, float partial sums added in order
+                                              (128, 64, 8192, 0, 1, 0, False), (1, 1, 70000, 0, 1, -1, True), (100, 130, 5000, 4, -1, 1, False)]:
         run_case(stream, H.HALF, ta, tb, M, N, K, alpha, beta, rng, device_scalars=dev, pad=pad)
 
 
