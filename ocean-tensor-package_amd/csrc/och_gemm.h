@@ -105,17 +105,18 @@ struct SlabLoader
    /* mat: operand origin; element (mn, k) of op(.) lives at mn + k * ld (!KC) or k + mn * ld (KC) */
    __device__ __forceinline__ void fetch(const char *mat, int64_t ld, uint32_t mn0, uint32_t k0, uint32_t MN, uint32_t K, int aligned)
    {
-      /* 4-byte reals: slabs that lie inside the matrix and are aligned take 128-bit loads also in the
-         edge-handling kernel (uniform over the block). Measured at 8000^3, ld 8192: float 94 -> 113 TFLOP/s;
-         for double the two-way code was slower than the checked 8-byte loads (57 -> 49), so it is left out. */
-      const bool wide = !EDGE || (sizeof(R) == 4 && aligned && (uint64_t)mn0 + BMN <= MN && (uint64_t)k0 + KT <= K);
+      /* Edge-handling kernel: a 128-bit vector that lies inside the matrix and is aligned is still one load (most vectors
+         of most tiles), one that lies outside is zero without touching memory; only vectors that straddle the border, and
+         all of them when the operand is not aligned, are loaded element by element. */
 #pragma unroll
       for (int v = 0; v < NV; v++)
       {  uint32_t mn, k; where(v, mn, k);
          const int64_t gm = (int64_t)mn0 + mn, gk = (int64_t)k0 + k;
-         if (wide)
-         {  const char *addr = mat + (KC ? (gk + gm * ld) : (gm + gk * ld)) * ES;
-            och_gu32x4 raw = *reinterpret_cast<const och_gu32x4 *>(addr);
+         const char *addr = mat + (KC ? (gk + gm * ld) : (gm + gk * ld)) * ES;
+         bool whole = true;
+         if (EDGE) whole = aligned && (KC ? (gm < (int64_t)MN && gk + VE <= (int64_t)K) : (gk < (int64_t)K && gm + VE <= (int64_t)MN));
+         if (whole)
+         {  och_gu32x4 raw = *reinterpret_cast<const och_gu32x4 *>(addr);
             __builtin_memcpy(&reg[v][0], &raw, 16);
          }
          else
@@ -124,7 +125,7 @@ struct SlabLoader
             for (int e = 0; e < VE; e++)
             {  const int64_t em = gm + (KC ? 0 : e), ek = gk + (KC ? e : 0);
                const bool ok = (em < (int64_t)MN) && (ek < (int64_t)K);
-               const R *src = reinterpret_cast<const R *>(mat + (KC ? (ek + em * ld) : (em + ek * ld)) * ES);
+               const R *src = reinterpret_cast<const R *>(addr + (int64_t)e * ES);
 #pragma unroll
                for (int c = 0; c < NPL; c++) reg[v][e * NPL + c] = ok ? src[c] : (R)0;
             }
@@ -526,11 +527,25 @@ static int launch_gemm_mfma(const GemmArgs &g)
    return 0;
 }
 
-/* fewer block tiles than one and a half per compute unit of an MI355X (256 CUs): the large tile would leave most of
-   the device idle (1024^3 double: 64 tiles, 13.8 TFLOP/s) */
-static inline bool gemm_few_tiles(const GemmArgs &g, int bm, int bn)
-{  const uint64_t tiles = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * (uint64_t)g.nz;
-   return tiles < 384;
+/* Compute units of the current device (cached per device). */
+int gemm_compute_units(void);
+
+/* Which block tile to use. The compute units work through the tiles in rounds, and the last round is as long as the others
+   however few tiles it holds: 3000^3 double is 576 tiles of 128 x 128, i.e. 2.25 rounds on 256 units, and ran at 39
+   TFLOP/s where 4000^3 (exactly 4 rounds) reached 56. A candidate's score is its efficiency on large products (measured,
+   relative to the largest tile) times the share of the rounds that does useful work; the best score wins, ties go to the
+   larger tile (first in the list). */
+struct GemmTileChoice { int bm, bn; double efficiency; };
+static inline int gemm_pick_tile(const GemmArgs &g, const GemmTileChoice *choice, int n)
+{  const uint64_t units = (uint64_t)gemm_compute_units();
+   int best = 0; double best_score = -1;
+   for (int c = 0; c < n; c++)
+   {  const uint64_t tiles = ((g.M + choice[c].bm - 1) / choice[c].bm) * ((g.N + choice[c].bn - 1) / choice[c].bn) * (uint64_t)g.nz;
+      const uint64_t rounds = (tiles + units - 1) / units;
+      const double score = choice[c].efficiency * (double)tiles / (double)(rounds * units);
+      if (score > best_score * 1.02) { best = c; best_score = score; }
+   }
+   return best;
 }
 
 int gemm_float(const GemmArgs &g);

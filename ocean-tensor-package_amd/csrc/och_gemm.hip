@@ -116,6 +116,18 @@ template <class T> static int gemm_generic(const GemmArgs &g)
    return 0;
 }
 
+int gemm_compute_units(void)
+{  static int cached[64];
+   int device = 0;
+   if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
+   if (cached[device] == 0)
+   {  int n = 0;
+      if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0) n = 256;
+      cached[device] = n;
+   }
+   return cached[device];
+}
+
 static char norm_trans(char t)
 {  if (t == 'N' || t == 'n') return 'N';
    if (t == 'T' || t == 't') return 'T';

@@ -1,9 +1,13 @@
-/* cfloat GEMM: 128 x 128 block tile, 64 x 64 per wave, real and imaginary planes, K slab 8.
-   Products with too few of those tiles to occupy the device use 64 x 64 block tiles instead. */
+/* cfloat GEMM: as float, with real and imaginary planes (four real MFMAs per tile), K slab 8. */
 #include "och_gemm.h"
 namespace och {
 int gemm_cfloat(const GemmArgs &g)
-{  if (gemm_few_tiles(g, 128, 128)) return launch_gemm_mfma<float, true, 32, 32, 8>(g);
-   return launch_gemm_mfma<float, true, 64, 64, 8>(g);
+{  static const GemmTileChoice choice[4] = { { 128, 128, 1.0 }, { 128, 64, 0.94 }, { 64, 128, 0.94 }, { 64, 64, 0.86 } };
+   switch (gemm_pick_tile(g, choice, 4))
+   {  case 0:  return launch_gemm_mfma<float, true, 64, 64, 8>(g);
+      case 1:  return launch_gemm_mfma<float, true, 64, 32, 8>(g);
+      case 2:  return launch_gemm_mfma<float, true, 32, 64, 8>(g);
+      default: return launch_gemm_mfma<float, true, 32, 32, 8>(g);
+   }
 }
 }

@@ -369,10 +369,12 @@ static int launch_gemm_half(const GemmArgs &g)
 int gemm_half(const GemmArgs &g)
 {
    if (g.K < 16) return 1;                      /* C <- beta C, and updates of so low a rank that writing C is all there is */
-   const uint64_t big = ((g.M + 255) / 256) * ((g.N + 255) / 256) * (uint64_t)g.nz;
-   if (big >= 192) return launch_gemm_half<64, 128, 4, 2, 64>(g);
-   if (!gemm_few_tiles(g, 128, 128)) return launch_gemm_half<64, 64, 2, 2, 64>(g);
-   return launch_gemm_half<32, 32, 2, 2, 64>(g);
+   static const GemmTileChoice choice[3] = { { 256, 256, 1.0 }, { 128, 128, 0.8 }, { 64, 64, 0.55 } };
+   switch (gemm_pick_tile(g, choice, 3))
+   {  case 0:  return launch_gemm_half<64, 128, 4, 2, 64>(g);
+      case 1:  return launch_gemm_half<64, 64, 2, 2, 64>(g);
+      default: return launch_gemm_half<32, 32, 2, 2, 64>(g);
+   }
 }
 
 } /* namespace och */
