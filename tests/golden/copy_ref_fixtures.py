@@ -14,7 +14,9 @@ NAMES = ["tensor_add_02", "ocean_min_01", "ocean_and_01", "ocean_or_01", "ocean_
          "ocean_bitshift_02", "ocean_fabs_02", "ocean_gemm_10", "ocean_gemm_11", "ocean_linspace_03", "ocean_maximumabs_01", "ocean_not_01",
          "ocean_cast_01", "ocean_power_01", "ocean_power_02", "ocean_power_03", "ocean_sum_01", "ocean_unary_01", "tensor_add_01",
          "tensor_axis_norm2_01", "tensor_divide_01", "tensor_multiply_01", "tensor_subtract_01", "tensor_dtype_cast_01", "tensor_fill_01",
-         "tensor_copy_03", "tensor_copy_04", "tensor_copy_06", "tensor_copy_07"]
+         "tensor_copy_03", "tensor_copy_04", "tensor_copy_06", "tensor_copy_07",
+         "tensor_copy_01", "tensor_copy_02", "tensor_copy_05", "tensor_copy_09", "tensor_clone_01", "tensor_clone_02", "tensor_clone_03",
+         "tensor_device_cast_01", "tensor_split_01"]
 # the GPU file of tensor_fillnan_01 records a defect of the reference's GPU kernel (it fills every element,
 # solid/src/core/gpu/template_fill.cu:72-79); the CPU twin holds the defined behaviour (only NaN is replaced)
 CPU_TWINS = ["tensor_fillnan_01"]

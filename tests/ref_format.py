@@ -67,7 +67,9 @@ def parse_ref(text):
                 rows = []
                 in_slices = False
                 continue
-            if len(shape) == 1:
+            if n == 0:
+                arr = np.zeros(shape)
+            elif len(shape) == 1:
                 arr = np.array(flat)
             else:
                 # slices follow in order of the higher dimensions (first of them fastest); each slice lists rows of dimension 0

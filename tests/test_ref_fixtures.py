@@ -108,6 +108,22 @@ class Engine:
             assert fn(*args, 1) == 0
         return self._result(c, z)
 
+    def strided_copy(self, ts, td, src_parent, src_view, dst_parent, dst_view):
+        """dst_view <- src_view, converting; both are views (any strides: zero, negative) into their parent arrays. Returns
+        the destination parent afterwards."""
+        z = dst_parent.copy(order="K")
+        zview = np.ndarray(shape=dst_view.shape, dtype=z.dtype, buffer=z, strides=dst_view.strides,
+                           offset=dst_view.__array_interface__["data"][0] - dst_parent.__array_interface__["data"][0]) if dst_view.size else z
+        a = H.Operand(src_parent, src_view, ts); c = H.Operand(z, zview, td)
+        if self.gpu:
+            a.upload(self.stream); c.upload(self.stream)
+        args = (ts, td, src_view.ndim, oh.sizes(a.shape), oh.strides(a.strides), self._ptr(a), dst_view.ndim, oh.sizes(c.shape), oh.strides(c.strides), self._ptr(c, z))
+        if self.gpu:
+            oh.check(oh.lib.och_copy(*args, self.stream.handle)); a.free()
+        else:
+            assert orc.lib.oracle_copy(*args, 1) == 0
+        return self._result(c, z)
+
     def byteswap(self, dtype, x):
         """reverse the bytes of every element in place (a byte-swapped destination of another type is written in native order
         first and swapped afterwards, tensor_copy_cpu.c:140-156)"""
