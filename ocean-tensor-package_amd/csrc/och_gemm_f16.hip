@@ -365,7 +365,10 @@ static int launch_gemm_half(const GemmArgs &g)
    with few tiles and a long K are cut along K.
    Measured at 8192^3 (NN / NT / TN / TT, TFLOP/s): 256 x 256 tiles with eight waves 763 / 841 / 958 / 947; with
    128 x 128 tiles and four waves the same kernel stays 15 - 25 % below that. 4096^3 (256 tiles of 256 x 256):
-   793 / 653 / 720 / 696. */
+   793 / 653 / 720 / 696. A 256 x 256 tile with four waves of 128 x 128 (a third less LDS traffic per MFMA) measures the
+   same. With the loads from memory, the LDS stores, the fragment reads and the barriers taken out one by one the TN
+   product rises from 850 to 1017, 1169, 1366 and, with the bare MFMA loop left, 1495 TFLOP/s: that, not the nominal
+   2500, is what the matrix cores sustain here, and the kernel runs at about two thirds of it. */
 int gemm_half(const GemmArgs &g)
 {
    if (g.K < 16) return 1;                      /* C <- beta C, and updates of so low a rank that writing C is all there is */
