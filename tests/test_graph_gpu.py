@@ -84,3 +84,60 @@ def test_graph_replays_equal_eager_launches(hip, stream):
         oh.check(lib.och_stream_begin_capture(None))
     for b in (dq, dx, dr, dz, dw, dsum, dax, consts, scratch):
         b.free()
+
+
+def test_graph_with_half_gemm_split_k_projection_and_gather(hip, stream):
+    """The entries added after the first recording test are recordable too: the half-precision MFMA product (a kernel with
+    more than 64 KB of LDS), a product cut along K (partial sums in the stream's workspace, which begin_capture creates),
+    the fused Gram-Schmidt projection and a gather through an offset table. Every replay must equal the eager run."""
+    lib, h = oh.lib, stream.handle
+    rng = np.random.default_rng(32)
+    M = N = 512; K = 128
+    a16 = rng.standard_normal(M * K).astype(np.float16); b16 = rng.standard_normal(K * N).astype(np.float16)
+    dA, dB, dC = oh.to_device(a16, stream), oh.to_device(b16, stream), oh.DeviceBuffer(2 * M * N, stream)
+    long_a = rng.uniform(-1, 1, 64 * 16384); long_b = rng.uniform(-1, 1, 16384 * 64)
+    dLA, dLB, dLC = oh.to_device(long_a, stream), oh.to_device(long_b, stream), oh.DeviceBuffer(8 * 64 * 64, stream)
+    n, k = 2000, 5
+    q = rng.uniform(-1, 1, n * (k + 1)) / 40
+    dQ, dR = oh.to_device(q, stream), oh.DeviceBuffer(8 * k, stream)
+    rows = rng.permutation(64)[:20].astype(np.int64) * (8 * 64)
+    dtab = oh.to_device(rows, stream)
+    import index_cases as IC
+    table = IC.pointer_table([None, dtab], lambda b: b.address)
+    dG = oh.DeviceBuffer(8 * 64 * 20, stream)
+    one16, zero16 = np.array([0x3C00], np.uint16), np.array([0], np.uint16)
+    one, zero = np.array([1.0]), np.array([0.0])
+
+    def sequence():
+        oh.check(lib.och_gemm(H.HALF, b"N", b"T", M, N, K, one16.ctypes.data_as(C.c_void_p), dA.ptr, M, dB.ptr, N, zero16.ctypes.data_as(C.c_void_p), dC.ptr, M, 1, h))
+        oh.check(lib.och_gemm(H.DOUBLE, b"N", b"N", 64, 64, 16384, one.ctypes.data_as(C.c_void_p), dLA.ptr, 64, dLB.ptr, 16384, zero.ctypes.data_as(C.c_void_p), dLC.ptr, 64, 1, h))
+        oh.check(lib.och_mgs_project(H.DOUBLE, n, k, dQ.ptr, n, C.c_void_p(dQ.address + 8 * n * k), dR.ptr, h))        # the last column changes per run
+        oh.check(lib.och_get_index(H.DOUBLE, 2, oh.sizes([64, 20]), table, oh.strides([8, 0]), dLC.ptr, oh.strides([8, 8 * 64]), dG.ptr, h))
+
+    outputs = (dC, dLC, dQ, dR, dG)
+    def snapshot():
+        stream.synchronize()
+        return [b.download(np.uint8).copy() for b in outputs]
+    def reset():
+        dQ.upload(q)
+        for b in (dC, dLC, dR, dG):
+            oh.check(lib.och_memset_async(b.ptr, 0, b.nbytes, h))
+        stream.synchronize()
+
+    reset()
+    eager = []
+    for _ in range(3):
+        sequence(); eager.append(snapshot())
+    assert not np.array_equal(eager[0][2], eager[1][2])
+    reset()
+    oh.check(lib.och_stream_begin_capture(h))
+    sequence()
+    graph = C.c_void_p()
+    oh.check(lib.och_stream_end_capture(h, C.byref(graph)))
+    for r in range(3):
+        oh.check(lib.och_graph_launch(graph, h))
+        for g, e, name in zip(snapshot(), eager[r], ("half product", "split product", "Q", "r", "gather")):
+            assert np.array_equal(g, e), "replay %d: %s differs from the eager launches" % (r, name)
+    oh.check(lib.och_graph_destroy(graph))
+    for b in (dA, dB, dC, dLA, dLB, dLC, dQ, dR, dtab, dG):
+        b.free()
