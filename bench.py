@@ -334,6 +334,23 @@ def main():
                     "ms": round(ms, 3), "TFLOPs": round(tf, 2), "frac": round(tf / MFMA_PEAK[nm], 3)}
             for buf in (a, b, c):
                 buf.free()
+        # beyond the named configurations: the half-precision product of the same size (float accumulation, one rounding)
+        if lib.och_gemm_supported(oh.HALF):
+            dim = 8192
+            a, b, c = [oh.DeviceBuffer(2 * dim * dim, stream) for _ in range(3)]
+            block = rng.uniform(-1, 1, 1 << 22).astype(np.float16)
+            for buf in (a, b):
+                for off in range(0, 2 * dim * dim, block.nbytes):
+                    buf.upload(block, offset=off)
+            one16 = np.array([0x3C00, 0], np.uint16); zero16 = np.zeros(2, np.uint16)
+            for ta, tb in ((b"N", b"N"), (b"T", b"N"), (b"N", b"T")):
+                fn = lambda: oh.check(lib.och_gemm(oh.HALF, ta, tb, dim, dim, dim, one16.ctypes.data, a.ptr, dim, b.ptr, dim,
+                                                   zero16.ctypes.data, c.ptr, dim, 1, h))
+                ms = time_launches(fn, reps=3, warm=1)
+                tf = 2 * dim ** 3 / ms / 1e9
+                configs["extra_gemm_half_%d_%s%s" % (dim, ta.decode(), tb.decode())] = {"ms": round(ms, 3), "TFLOPs": round(tf, 2), "frac": round(tf / 2500.0, 3)}
+            for buf in (a, b, c):
+                buf.free()
         # MGS-QR pattern on a 4096 x 4096 float64 matrix: per (i, j) pair one dot product (gemm M = N = 1, result kept
         # on the device) and one rank-1 update reading that device scalar; window = the first 64 columns (2016 pairs)
         m = 4096
