@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Benchmark of the MI355X device module on BASELINE.json's configurations (one GPU).
+"""Benchmark of the MI355X device module on the five reference workload configurations (one GPU).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only-step]
 

@@ -168,7 +168,7 @@ def test_binary_in_place_and_empty(hip, stream):
 
 
 def test_config1_scale_add_fp32(hip, stream):
-    """BASELINE config 1: z = x*y + x on contiguous float32 vectors of 2^24 elements, U(-1,1),
+    """benchmark configuration 1: z = x*y + x on contiguous float32 vectors of 2^24 elements, U(-1,1),
     as two table calls (scale, then add); bit-exact against the CPU path."""
     n = 1 << 24
     rng = np.random.default_rng(1234)

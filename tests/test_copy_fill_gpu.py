@@ -168,7 +168,7 @@ def test_steps(hip, stream, dtype):
 
 
 def test_config4_cast_byteswap(hip, stream):
-    """BASELINE config 4 at reduced size plus the full-size round-trip property:
+    """benchmark configuration 4 at reduced size plus the full-size round-trip property:
     int16 3-D tensor (full int16 range, stored byteswapped, step-2 slice) -> contiguous float32, and
     complex64 -> complex128."""
     rng = np.random.default_rng(4)

@@ -2,7 +2,7 @@
 Ocean's interface layer drives it (OcInitGPU -> OcModuleCore table -> OcTensorGPU_* -> device
 library). Mirrors examples/python/gpu/tensors/tensor_add_02.py (transposed + broadcast add),
 tensor_dtype_cast_01.py / tensor_copy_0x.py (casting and strided copies between devices),
-ocean_sum_02.py, ocean_axis_reduce_04.py, ocean_gemm_01.py, and BASELINE configuration 2
+ocean_sum_02.py, ocean_axis_reduce_04.py, ocean_gemm_01.py, and benchmark configuration 2
 end to end: Z = (A.T + r + I) * F with automatic type promotion and a byte-swapped operand.
 
 Expected values come from numpy, which fixes them independently: every step of the float64

@@ -113,7 +113,7 @@ def test_axis_layouts(hip, stream):
 
 @pytest.mark.parametrize("dtype", [H.FLOAT, H.DOUBLE], ids=lambda d: H.NAMES[d])
 def test_config3_axis_reductions(hip, stream, dtype):
-    """BASELINE config 3, axis part: sum and min along axis 0 and axis 1 of a 3-D 512 x 512 x 256
+    """benchmark configuration 3, axis part: sum and min along axis 0 and axis 1 of a 3-D 512 x 512 x 256
     non-contiguous view (cut from a larger parent so that no two dimensions merge), N(0,1) data.
     min is exact; sum within 1e-5 / 1e-12 of the float64 result relative to the sum of magnitudes."""
     rng = np.random.default_rng(303)

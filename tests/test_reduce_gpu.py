@@ -178,7 +178,7 @@ def test_reduce_strided_and_empty(hip, stream):
 
 @pytest.mark.parametrize("dtype", [H.FLOAT, H.DOUBLE], ids=lambda d: H.NAMES[d])
 def test_config3_full_reductions(hip, stream, dtype):
-    """BASELINE config 3, full reductions: sum, 2-norm and max of an 8192 x 8192 N(0,1) tensor.
+    """benchmark configuration 3, full reductions: sum, 2-norm and max of an 8192 x 8192 N(0,1) tensor.
     max is exact; sum within 1e-5 (float) / 1e-12 (double) of the exact sum relative to sum|x|, and also
     relative to |sum| itself thanks to double accumulation; norm2 within the same relative tolerance."""
     n = 8192 * 8192
