@@ -161,19 +161,21 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
    {  slab0 = blockIdx.z * p.split_slabs;
       nslabs = (slab0 + p.split_slabs < nslabs) ? p.split_slabs : (slab0 < nslabs ? nslabs - slab0 : 0);
    }
+   /* registers hold the slab after the one in LDS: slab s + 1 is stored half way through the MFMAs of slab s (its stores
+      run under the remaining MFMAs instead of in front of the barrier) and the loads of slab s + 2 are issued right after,
+      a slab and a half before their data is needed */
    if (nslabs > 0)
    {  la.fetch(pA, p.ldA, m0, slab0 * KT, p.M, p.K, p.alignedA);
       lb.fetch(pB, p.ldB, n0, slab0 * KT, p.N, p.K, p.alignedB);
       la.stash(lds); lb.stash(lds + LA::SIZE);
+      if (nslabs > 1)
+      {  la.fetch(pA, p.ldA, m0, (slab0 + 1) * KT, p.M, p.K, p.alignedA);
+         lb.fetch(pB, p.ldB, n0, (slab0 + 1) * KT, p.N, p.K, p.alignedB);
+      }
    }
    __syncthreads();
    for (uint32_t s = 0; s < nslabs; s++)
    {  const uint16_t *As = lds + (s & 1) * BUF, *Bs = As + LA::SIZE;
-      const bool more = s + 1 < nslabs;
-      if (more)
-      {  la.fetch(pA, p.ldA, m0, (slab0 + s + 1) * KT, p.M, p.K, p.alignedA);
-         lb.fetch(pB, p.ldB, n0, (slab0 + s + 1) * KT, p.N, p.K, p.alignedB);
-      }
 #pragma unroll
       for (int ks = 0; ks < KT / 16; ks++)
       {  och_h8 a[TMS], b[TNS];
@@ -185,10 +187,14 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
          for (int i = 0; i < TMS; i++)
 #pragma unroll
             for (int j = 0; j < TNS; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
-      }
-      if (more)
-      {  uint16_t *An = lds + ((s + 1) & 1) * BUF;
-         la.stash(An); lb.stash(An + LA::SIZE);
+         if (ks == KT / 32 - 1 && s + 1 < nslabs)
+         {  uint16_t *An = lds + ((s + 1) & 1) * BUF;
+            la.stash(An); lb.stash(An + LA::SIZE);
+            if (s + 2 < nslabs)
+            {  la.fetch(pA, p.ldA, m0, (slab0 + s + 2) * KT, p.M, p.K, p.alignedA);
+               lb.fetch(pB, p.ldB, n0, (slab0 + s + 2) * KT, p.N, p.K, p.alignedB);
+            }
+         }
       }
       __syncthreads();
    }
