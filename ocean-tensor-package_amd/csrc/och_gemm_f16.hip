@@ -369,11 +369,11 @@ static int launch_gemm_half(const GemmArgs &g)
 /* returns 1 when the product is left to the generic kernel (K < 16). Small results run on the 64 x 64 tile with the part
    outside the matrices read as zero -- the matrix cores are fast enough for that to beat a scalar kernel -- and products
    with few tiles and a long K are cut along K.
-   Measured at 8192^3 (NN / NT / TN / TT, TFLOP/s): 256 x 256 tiles with eight waves 763 / 841 / 958 / 947; with
+   Measured at 8192^3 (NN / NT / TN / TT, TFLOP/s): 256 x 256 tiles with eight waves 798 / 908 / 1021 / 1005; with
    128 x 128 tiles and four waves the same kernel stays 15 - 25 % below that. 4096^3 (256 tiles of 256 x 256):
    793 / 653 / 720 / 696. A 256 x 256 tile with four waves of 128 x 128 (a third less LDS traffic per MFMA) measures the
    same. With the loads from memory, the LDS stores, the fragment reads and the barriers taken out one by one the TN
-   product rises from 850 to 1017, 1169, 1366 and, with the bare MFMA loop left, 1495 TFLOP/s: that, not the nominal
+   product (850 before the loads were moved a slab and a half ahead) rises to 1017, 1169, 1366 and, with the bare MFMA loop left, 1495 TFLOP/s: that, not the nominal
    2500, is what the matrix cores sustain here, and the kernel runs at about two thirds of it. */
 int gemm_half(const GemmArgs &g)
 {
