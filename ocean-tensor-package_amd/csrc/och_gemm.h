@@ -85,6 +85,19 @@ template <class R> struct GemmParams
 
 #define OCH_GEMM_THREADS 256
 
+/* Column twist of the k-major LDS planes. The row pitch moves every k on by 8 banks (of 32), so rows k and k + 4 start in
+   the same bank; an operand that is contiguous along k in memory is stored by lanes that hold different k for the same
+   column, and those stores collided (SQ_LDS_BANK_CONFLICT was a third to a half of the LDS cycles with such an operand,
+   zero without). Element (k, c) therefore sits in column c ^ twist(k), twist = ((k / 4) mod 4) * (columns that the lanes of
+   one LDS cycle cover): a multiple of the vector length and smaller than an MFMA tile, so vector stores along the row and
+   the fragment reads of an aligned tile keep their shape. */
+template <class R, bool CPLX, int KT> __device__ __forceinline__ uint32_t lds_twist(uint32_t k)
+{  constexpr int VE = 16 / ((int)sizeof(R) * (CPLX ? 2 : 1));          /* elements per 128-bit load */
+   constexpr int LANES = (sizeof(R) == 4) ? 32 : 16;                    /* lanes served per LDS cycle (128 bytes) */
+   constexpr int COLS = LANES / (KT / VE);                              /* columns they cover when k varies fastest */
+   return ((k >> 2) & 3u) * COLS;
+}
+
 /* Moves a BMN x KT slab of an operand from global memory to registers (fetch) and from there
    to its k-major LDS planes (stash). KC: the operand is contiguous along k in memory. */
 template <class R, bool CPLX, bool KC, bool EDGE, int BMN, int KT>
@@ -140,7 +153,7 @@ struct SlabLoader
       {  uint32_t mn, k; where(v, mn, k);
 #pragma unroll
          for (int e = 0; e < VE; e++)
-         {  const uint32_t em = mn + (KC ? 0 : e), ek = k + (KC ? e : 0);
+         {  const uint32_t ek = k + (KC ? e : 0), em = (mn ^ lds_twist<R, CPLX, KT>(ek)) + (KC ? 0 : e);
             planes[ek * pitch + em] = reg[v][e * NPL];
             if (CPLX) planes[(KT + ek) * pitch + em] = conj ? -reg[v][e * NPL + 1] : reg[v][e * NPL + 1];
          }
@@ -214,13 +227,13 @@ __global__ __launch_bounds__(OCH_GEMM_THREADS, 2) void gemm_mfma_kernel(const Ge
          R a[TMS], b[TNS], ai[CPLX ? TMS : 1], bi[CPLX ? TNS : 1];
 #pragma unroll
          for (int i = 0; i < TMS; i++)
-         {  a[i] = As[k * PA + wm + i * T + lane % T];
-            if (CPLX) ai[i] = As[(KT + k) * PA + wm + i * T + lane % T];
+         {  a[i] = As[k * PA + ((wm + i * T + lane % T) ^ lds_twist<R, CPLX, KT>(k))];
+            if (CPLX) ai[i] = As[(KT + k) * PA + ((wm + i * T + lane % T) ^ lds_twist<R, CPLX, KT>(k))];
          }
 #pragma unroll
          for (int j = 0; j < TNS; j++)
-         {  b[j] = Bs[k * PB + wn + j * T + lane % T];
-            if (CPLX) bi[j] = Bs[(KT + k) * PB + wn + j * T + lane % T];
+         {  b[j] = Bs[k * PB + ((wn + j * T + lane % T) ^ lds_twist<R, CPLX, KT>(k))];
+            if (CPLX) bi[j] = Bs[(KT + k) * PB + ((wn + j * T + lane % T) ^ lds_twist<R, CPLX, KT>(k))];
          }
 #pragma unroll
          for (int i = 0; i < TMS; i++)
