@@ -632,7 +632,9 @@ static int launch_ew3(int ndims, const size_t *size,
          {  if (p.nt) hipLaunchKernelGGL((ew3_kernel<F, VEC, OCH_EW_UNR, true, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p);
             else      hipLaunchKernelGGL((ew3_kernel<F, VEC, OCH_EW_UNR, true, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
          [&](const EwParams<3> &p, uint32_t blocks)
-         {  hipLaunchKernelGGL((ew3_kernel<F, VEC, 2, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
+         {  /* nontemporal accesses reach only the operands that take the wide path; a broadcast operand keeps its cached loads */
+            if (p.nt) hipLaunchKernelGGL((ew3_kernel<F, VEC, 2, false, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p);
+            else      hipLaunchKernelGGL((ew3_kernel<F, VEC, 2, false, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
          [&](const EwParams<3> &p, uint32_t blocks)
          {  hipLaunchKernelGGL((ew3_kernel<F, 1, 1, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); });
    });
