@@ -102,6 +102,12 @@ template <class T, int VEC, bool NT = false>
 OCH_D void load_pack(Pack<T, VEC> &p, const char *addr, int64_t estride, int vec)
 {
    if (vec) load_wide<T, VEC, NT>(p, addr);
+   else if (estride == 0)
+   {  /* broadcast along the vector: one load serves all elements */
+      const T x = *reinterpret_cast<const T *>(addr);
+#pragma unroll
+      for (int k = 0; k < VEC; k++) p.v[k] = x;
+   }
    else
    {
 #pragma unroll
