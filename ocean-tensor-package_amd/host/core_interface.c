@@ -227,6 +227,18 @@ final:
 }
 
 /* ---- GEMM ---------------------------------------------------------------------------------------- */
+/* float -> half as Ocean converts it (solid/src/base/generic/half.c): values below 2^-15 become zero, ties round away from
+   zero, NaN becomes 0x7F00 */
+static OcUInt16 half_bits(float f)
+{  unsigned int raw, d, s, ex; memcpy(&raw, &f, 4);
+   d = raw & 0x007FFFFFu; s = (raw >> 16) & 0x8000u; ex = (raw >> 23) & 0xFFu;
+   if (ex < 112u) return 0;
+   if (ex > 143u) return (OcUInt16)((ex == 255u && d != 0) ? 0x7F00u : (s | 0x7C00u));
+   {  unsigned int v = (((ex - 112u) << 10) | (d >> 13) | s) & 0xFFFFu;
+      if ((d & 0x1FFFu) >= 0x1000u) v++;
+      return (OcUInt16)v;
+   }
+}
 /* C <- alpha op(A) op(B) + beta C. Operands are brought to one type; an operand whose columns are not
    contiguous is either used through the opposite transposition (when its rows are contiguous) or copied
    (tensor_itf.c:6137-6778); alpha and beta become one-element host tensors of that type (:5951-5992). */
@@ -256,6 +268,7 @@ static OcTensor *scalar_tensor(OcScalar *s, OcDType dtype, double fallback)
       case OcDTypeDouble: *(OcDouble *)p = re; break;
       case OcDTypeCFloat: ((OcCFloat *)p)->real = (OcFloat)re; ((OcCFloat *)p)->imag = (OcFloat)im; break;
       case OcDTypeCDouble: ((OcCDouble *)p)->real = re; ((OcCDouble *)p)->imag = im; break;
+      case OcDTypeHalf: *(OcUInt16 *)p = half_bits((float)re); break;
       default: OcErrorMessage("GEMM scalars of type %s are not supported by this front end", OcDType_name(dtype)); OcDecrefTensor(t); return NULL;
    }
    return t;
@@ -286,10 +299,13 @@ static int gemm_operand(OcTensor **t, char *mode, OcIndex *ld, int complex_type)
    products and broadcast between A and B (size 1 or absent: shared), as in Ocean's interface (tensor_itf.c:6433-6750) */
 int OcTensor_gemm(OcScalar *alpha, OcTensor *A, char modeA, OcTensor *B, char modeB, OcScalar *beta, OcTensor **C)
 {  OcTensor *a = OcIncrefTensor(A), *b = OcIncrefTensor(B), *c = NULL, *ta = NULL, *tb = NULL, *v; int result = -1, i, nd;
-   OcDevice *device = A->device != OcCPU ? A->device : B->device; OcDType dtype = OcDType_getCommonType(A->dtype, B->dtype);
+   OcDevice *device = A->device != OcCPU ? A->device : B->device; OcDType dtype = OcDType_getCommonType(A->dtype, B->dtype), halftype = OcDTypeNone;
    OcSize M, N, K, K2, csize[OC_TENSOR_MAX_DIMS], asize[OC_TENSOR_MAX_DIMS], bsize[OC_TENSOR_MAX_DIMS]; OcIndex ldA, ldB, ldC; OcModuleCore *m = OcModuleCore_forDevice(device);
    if (*C) dtype = OcDType_getCommonType(dtype, (*C)->dtype);
    if (m == NULL) { OcErrorMessage("No core module is registered for device %s", device->name); goto final; }
+   /* half types the device cannot multiply are computed in float and converted back (tensor_itf.c:6388-6400, 6756-6758) */
+   if ((dtype == OcDTypeHalf || dtype == OcDTypeCHalf) && !m->Tensor_gemmSupportedOn(device, dtype))
+   {  halftype = dtype; dtype = (dtype == OcDTypeHalf) ? OcDTypeFloat : OcDTypeCFloat; }
    if (!m->Tensor_gemmSupportedOn(device, dtype)) { OcErrorMessage("Matrix multiplication is not supported for type %s on %s", OcDType_name(dtype), device->name); goto final; }
    if (A->ndims < 2 || B->ndims < 2) { OcErrorMessage("Matrix multiplication needs tensors of at least two dimensions"); goto final; }
    M = (modeA == 'N') ? A->size[0] : A->size[1]; K = (modeA == 'N') ? A->size[1] : A->size[0];
@@ -334,6 +350,7 @@ int OcTensor_gemm(OcScalar *alpha, OcTensor *A, char modeA, OcTensor *B, char mo
    if (OcTensor_startRead(c, a) != 0 || OcTensor_startRead(c, b) != 0) goto final;
    result = m->Tensor_gemm(M, N, K, modeA, modeB, ta, a, ldA, b, ldB, tb, c, ldC);
    if (result == 0 && (OcTensor_update(c) != 0 || OcTensor_finishRead(c, a) != 0 || OcTensor_finishRead(c, b) != 0)) result = -1;
+   if (result == 0 && *C == NULL && halftype != OcDTypeNone) result = OcTensor_ensure(&c, halftype, device);
    if (result == 0 && *C == NULL) { *C = c; c = NULL; }
    else if (result == 0 && c != *C) result = OcTensor_copy(c, *C);
 final:

@@ -278,3 +278,31 @@ def test_gram_schmidt_with_the_fused_projection(gpu):
         host.check(host.lib.OcTensorGPU_projectColumns(tA, host.from_numpy(np.zeros(n, np.float32), host.FLOAT, gpu), None))
     with pytest.raises(host.OceanError, match="sizes"):
         host.check(host.lib.OcTensorGPU_projectColumns(tA, host.from_numpy(np.zeros(n + 1), host.DOUBLE, gpu), None))
+
+
+def test_complex_half_product_falls_back_to_complex_float(gpu):
+    """The device module multiplies half but not complex-half matrices (Tensor_gemmSupportedOn); for complex-half the front
+    end computes in complex-float and converts the result back, as tensor_itf.c:6388-6400 and 6756-6758 do."""
+    rng = np.random.default_rng(17)
+    m, n, k = 40, 24, 56
+    A = (rng.integers(-4, 5, (k, m)) + 1j * rng.integers(-4, 5, (k, m))).astype(np.complex64)       # Ocean (m, k)
+    B = (rng.integers(-4, 5, (n, k)) + 1j * rng.integers(-4, 5, (n, k))).astype(np.complex64)       # Ocean (k, n)
+    host.lib.OcTensor_ensure.argtypes = [C.POINTER(host.TP), C.c_int, C.c_void_p]
+    tA, tB = host.from_numpy(A, host.CFLOAT, gpu), host.from_numpy(B, host.CFLOAT, gpu)
+    host.check(host.lib.OcTensor_ensure(C.byref(tA), host.CHALF, gpu)); host.check(host.lib.OcTensor_ensure(C.byref(tB), host.CHALF, gpu))
+    assert tA.contents.dtype == host.CHALF
+    c = host.TP()
+    host.check(host.lib.OcTensor_mtimes(tA, tB, C.byref(c)))
+    assert c.contents.dtype == host.CHALF and host.shape_of(c) == [m, n]
+    host.check(host.lib.OcTensor_ensure(C.byref(c), host.CFLOAT, gpu))
+    want = (A.T @ B.T).T                                   # small integers: every partial sum is exact in float, results below 2048 exact in half
+    got = host.to_numpy(c)
+    assert np.abs(want).max() < 2048 and np.array_equal(got, want)
+    # half itself runs on the device module directly
+    hA, hB = host.from_numpy(A.real.copy(), host.FLOAT, gpu), host.from_numpy(B.real.copy(), host.FLOAT, gpu)
+    host.check(host.lib.OcTensor_ensure(C.byref(hA), host.HALF, gpu)); host.check(host.lib.OcTensor_ensure(C.byref(hB), host.HALF, gpu))
+    ch = host.TP()
+    host.check(host.lib.OcTensor_mtimes(hA, hB, C.byref(ch)))
+    assert ch.contents.dtype == host.HALF
+    host.check(host.lib.OcTensor_ensure(C.byref(ch), host.FLOAT, gpu))
+    assert np.array_equal(host.to_numpy(ch), (A.real.T @ B.real.T).T)
