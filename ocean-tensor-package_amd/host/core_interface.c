@@ -138,7 +138,12 @@ int OcTensor_unary(int op, OcTensor *src, OcTensor **dst)
       if (fn == NULL) return OcErrorMessage("Tensor operation is not supported on device %s", src->device->name);
    }
    a = OcIncrefTensor(src);
-   if (OcTensor_ensure(&a, a->dtype, a->device) != 0) goto final;
+   {  /* the negative of an unsigned tensor is taken in its signed type (tensor_itf.c:3637-3651, signed types of src/base/dtype.c:57-61) */
+      static const OcDType signed_of[5] = { OcDTypeInt16, OcDTypeInt16, OcDTypeInt32, OcDTypeInt64, OcDTypeDouble };
+      OcDType work = a->dtype;
+      if (op == 0 && work >= OcDTypeUInt8 && work <= OcDTypeUInt64) work = signed_of[work];
+      if (OcTensor_ensure(&a, work, a->device) != 0) goto final;
+   }
    rtype = a->dtype;
    if (op >= 35) rtype = OcDTypeBool;                                       /* isinf ... isneginf */
    if (op == 28 && OcDType_isComplex(a->dtype)) rtype = OcDType_getBaseType(a->dtype);   /* absolute of complex is real */

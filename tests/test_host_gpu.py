@@ -306,3 +306,17 @@ def test_complex_half_product_falls_back_to_complex_float(gpu):
     assert ch.contents.dtype == host.HALF
     host.check(host.lib.OcTensor_ensure(C.byref(ch), host.FLOAT, gpu))
     assert np.array_equal(host.to_numpy(ch), (A.real.T @ B.real.T).T)
+
+
+def test_negative_of_unsigned_takes_the_signed_type(gpu):
+    """-arange(5, uint8) is an int16 tensor 0 -1 -2 -3 -4 (examples/python/cpu/tensors/tensor_negative_01.ref; the
+    interface casts to the signed type before it calls the module, tensor_itf.c:3637-3651); uint64 goes to double."""
+    import ocean_hip as oh
+    for dt, np_t, want_dt, want_np in ((host.UINT8, np.uint8, host.INT16, np.int16), (host.UINT16, np.uint16, host.INT32, np.int32),
+                                       (host.UINT32, np.uint32, host.INT64, np.int64), (host.UINT64, np.uint64, host.DOUBLE, np.float64),
+                                       (host.INT8, np.int8, host.INT8, np.int8)):
+        t = host.from_numpy(np.arange(5, dtype=np_t), dt, gpu)
+        out = host.TP()
+        host.check(host.lib.OcTensor_unary(oh.U["negative"], t, C.byref(out)))
+        assert out.contents.dtype == want_dt
+        assert np.array_equal(host.to_numpy(out), -np.arange(5).astype(want_np))
