@@ -351,6 +351,22 @@ def main():
                 configs["extra_gemm_half_%d_%s%s" % (dim, ta.decode(), tb.decode())] = {"ms": round(ms, 3), "TFLOPs": round(tf, 2), "frac": round(tf / 2500.0, 3)}
             for buf in (a, b, c):
                 buf.free()
+        if lib.och_gemm_supported(oh.INT8):
+            dim = 8192
+            a, b, c = [oh.DeviceBuffer(dim * dim, stream) for _ in range(3)]
+            block = rng.integers(-128, 127, 1 << 22, endpoint=True).astype(np.int8)
+            for buf in (a, b):
+                for off in range(0, dim * dim, block.nbytes):
+                    buf.upload(block, offset=off)
+            one8 = np.array([1, 0], np.int8); zero8 = np.zeros(2, np.int8)
+            for ta, tb in ((b"N", b"N"), (b"T", b"N")):
+                fn = lambda: oh.check(lib.och_gemm(oh.INT8, ta, tb, dim, dim, dim, one8.ctypes.data, a.ptr, dim, b.ptr, dim,
+                                                   zero8.ctypes.data, c.ptr, dim, 1, h))
+                ms = time_launches(fn, reps=3, warm=1)
+                tf = 2 * dim ** 3 / ms / 1e9
+                configs["extra_gemm_int8_%d_%s%s" % (dim, ta.decode(), tb.decode())] = {"ms": round(ms, 3), "TOPs": round(tf, 2), "frac": round(tf / 5000.0, 3)}
+            for buf in (a, b, c):
+                buf.free()
         # MGS-QR pattern on a 4096 x 4096 float64 matrix: per (i, j) pair one dot product (gemm M = N = 1, result kept
         # on the device) and one rank-1 update reading that device scalar; window = the first 64 columns (2016 pairs)
         m = 4096

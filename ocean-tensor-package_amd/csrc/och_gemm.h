@@ -583,5 +583,7 @@ int gemm_double(const GemmArgs &g);
 int gemm_cfloat(const GemmArgs &g);
 int gemm_cdouble(const GemmArgs &g);
 int gemm_half(const GemmArgs &g);      /* 1: not taken, use the generic kernel */
+int gemm_int8(const GemmArgs &g);      /* int8 and uint8; 1: not taken */
+int gemm_bool(const GemmArgs &g);      /* 1: not taken */
 
 } /* namespace och */

@@ -145,12 +145,12 @@ extern "C" int och_gemm_supported(int dtype)
 static int gemm_dispatch(int dtype, const GemmArgs &g)
 {
    switch (dtype)
-   {  case OCH_BOOL:    return gemm_generic<obool>(g);
-      case OCH_UINT8:   return gemm_generic<uint8_t>(g);
+   {  case OCH_BOOL:    { const int status = gemm_bool(g); return (status == 1) ? gemm_generic<obool>(g) : status; }
+      case OCH_UINT8:   { const int status = gemm_int8(g); return (status == 1) ? gemm_generic<uint8_t>(g) : status; }
       case OCH_UINT16:  return gemm_generic<uint16_t>(g);
       case OCH_UINT32:  return gemm_generic<uint32_t>(g);
       case OCH_UINT64:  return gemm_generic<uint64_t>(g);
-      case OCH_INT8:    return gemm_generic<int8_t>(g);
+      case OCH_INT8:    { const int status = gemm_int8(g); return (status == 1) ? gemm_generic<int8_t>(g) : status; }
       case OCH_INT16:   return gemm_generic<int16_t>(g);
       case OCH_INT32:   return gemm_generic<int32_t>(g);
       case OCH_INT64:   return gemm_generic<int64_t>(g);

@@ -33,10 +33,11 @@ def as_float(dtype, a):
     return a
 
 
-def matrix(dtype, rows, cols, ld, rng):
+def matrix(dtype, rows, cols, ld, rng, kind="small"):
     """Column-major rows x cols matrix inside an ld x cols parent; the padding rows hold junk
     that must never be read into the result."""
-    flat = H.random_data(dtype, ld * max(cols, 1), rng, "small")
+    flat = H.random_data(dtype, ld * max(cols, 1), rng, kind)
+    # bool tensors hold 0 / 1 only (solid/src/core/cpu/template_blas.c:186); the 8-bit integer types use their whole range
     return flat
 
 
@@ -49,13 +50,13 @@ def scalar_of(dtype, value):
     return np.array([value]).astype(st)
 
 
-def run_case(stream, dtype, ta, tb, M, N, K, alpha, beta, rng, device_scalars=False, pad=3):
+def run_case(stream, dtype, ta, tb, M, N, K, alpha, beta, rng, device_scalars=False, pad=3, kind="small"):
     rowsA, colsA = (M, K) if ta == "N" else (K, M)
     rowsB, colsB = (K, N) if tb == "N" else (N, K)
     ldA, ldB, ldC = max(rowsA, 1) + pad, max(rowsB, 1) + pad, max(M, 1) + pad
-    A = matrix(dtype, rowsA, colsA, ldA, rng)
-    B = matrix(dtype, rowsB, colsB, ldB, rng)
-    C0 = matrix(dtype, M, N, ldC, rng)
+    A = matrix(dtype, rowsA, colsA, ldA, rng, kind)
+    B = matrix(dtype, rowsB, colsB, ldB, rng, kind)
+    C0 = matrix(dtype, M, N, ldC, rng, kind)
     al, be = scalar_of(dtype, alpha), scalar_of(dtype, beta)
     dA, dB, dC = oh.to_device(A, stream), oh.to_device(B, stream), oh.to_device(C0, stream)
     if device_scalars:
@@ -144,6 +145,23 @@ def test_gemm_half_matrix_cores(hip, stream, ta, tb):
                                               # few tiles and a long K: cut along K, float partial sums added in order
                                               (128, 64, 8192, 0, 1, 0, False), (1, 1, 70000, 0, 1, -1, True), (100, 130, 5000, 4, -1, 1, False)]:
         run_case(stream, H.HALF, ta, tb, M, N, K, alpha, beta, rng, device_scalars=dev, pad=pad)
+
+
+@pytest.mark.parametrize("dtype", [H.INT8, H.UINT8, H.BOOL], ids=lambda d: H.NAMES[d])
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+def test_gemm_bytes_matrix_cores(hip, stream, dtype, ta, tb):
+    """8-bit integer and bool products on the MFMA kernel (K >= 32), bit-exact against the oracle's wrap-around / OR-AND
+    arithmetic: whole tiles with aligned operands, ragged edges, unaligned leading dimensions, all three tile sizes, a
+    long K cut into slices, scalars in device memory, beta != 0."""
+    rng = np.random.default_rng(950 + dtype + ord(ta) + 2 * ord(tb))
+    neg = 3 if dtype == H.UINT8 else -1
+    for (M, N, K, pad, alpha, beta, dev) in [(128, 128, 128, 0, 1, 0, False), (256, 384, 160, 16, 2, neg, False), (200, 136, 100, 3, 1, 1, True),
+                                              (64, 64, 32, 0, neg, 1, False), (96, 160, 2048, 0, 3, 0, True), (33, 47, 37, 5, 1, 0, False),
+                                              (2560, 2304, 256, 0, 1, 1, False), (2500, 2300, 130, 4, 1, 0, False), (4096, 3072, 128, 0, 1, 0, False),
+                                              (1, 1500, 999, 0, 1, 1, False), (128, 64, 8192, 0, 1, 0, False), (1, 1, 70000, 0, 1, neg, True)]:
+        if dtype == H.BOOL:
+            alpha, beta = (1 if alpha else 0), (1 if beta else 0)
+        run_case(stream, dtype, ta, tb, M, N, K, alpha, beta, rng, device_scalars=dev, pad=pad, kind="full")
 
 
 def test_gemm_errors_and_empty(hip, stream):
