@@ -270,6 +270,9 @@ BATCH_CASES = [  # dtype, ta, tb, M, N, K, batch sizes, B shared by the products
     (H.INT32, "N", "N", 70, 66, 40, (3,), False, True),
     (H.BOOL, "T", "T", 20, 30, 10, (2,), False, False),
     (H.HALF, "N", "N", 64, 64, 64, (3,), False, False),
+    (H.INT8, "N", "T", 70, 66, 96, (3, 2), False, True),              # 8-bit MFMA kernel with batch offsets and per-product scalars
+    (H.UINT8, "T", "N", 129, 64, 40, (2,), True, False),
+    (H.BOOL, "N", "N", 64, 40, 64, (4,), False, True),
     (H.DOUBLE, "N", "N", 16, 16, 16, (1, 7, 1), False, "host"),       # host scalars that differ per product: one launch each
 ]
 
