@@ -562,18 +562,19 @@ int gemm_compute_units(void);
 
 /* Which block tile to use. The compute units work through the tiles in rounds, and the last round is as long as the others
    however few tiles it holds: 3000^3 double is 576 tiles of 128 x 128, i.e. 2.25 rounds on 256 units, and ran at 39
-   TFLOP/s where 4000^3 (exactly 4 rounds) reached 56. A candidate's score is its efficiency on large products (measured,
-   relative to the largest tile) times the share of the rounds that does useful work; the best score wins, ties go to the
-   larger tile (first in the list). */
+   TFLOP/s where 4000^3 (exactly 4 rounds) reached 56. A candidate's cost is rounds x tile area / efficiency (its measured
+   efficiency on large products, relative to the largest tile): the time the product takes in units of one element of C
+   per compute unit. It also charges the part of edge tiles that lies outside C, so a dot product does not get the
+   largest tile. The cheapest candidate wins; within 2 % the larger tile (earlier in the list) is kept. */
 struct GemmTileChoice { int bm, bn; double efficiency; };
 static inline int gemm_pick_tile(const GemmArgs &g, const GemmTileChoice *choice, int n)
 {  const uint64_t units = (uint64_t)gemm_compute_units();
-   int best = 0; double best_score = -1;
+   int best = 0; double best_cost = 0;
    for (int c = 0; c < n; c++)
    {  const uint64_t tiles = ((g.M + choice[c].bm - 1) / choice[c].bm) * ((g.N + choice[c].bn - 1) / choice[c].bn) * (uint64_t)g.nz;
       const uint64_t rounds = (tiles + units - 1) / units;
-      const double score = choice[c].efficiency * (double)tiles / (double)(rounds * units);
-      if (score > best_score * 1.02) { best = c; best_score = score; }
+      const double cost = (double)rounds * choice[c].bm * choice[c].bn / choice[c].efficiency;
+      if (c == 0 || cost < best_cost * 0.98) { best = c; best_cost = cost; }
    }
    return best;
 }

@@ -308,7 +308,7 @@ static int launch_gemm_byte(const GemmArgs &g)
    /* few tiles and a long K: slices of K in grid z, at least 8 slabs each, about 512 blocks in all, partial sums within the workspace */
    uint32_t slices = 1;
    {  const uint64_t nslabs = (g.K + KT - 1) / KT;
-      if (g.batch.nb == 0 && blocks < 128 && nslabs >= 32)
+      if (g.batch.nb == 0 && blocks < (uint64_t)gemm_compute_units() && nslabs >= 32)
       {  uint64_t want = (512 + blocks - 1) / blocks;
          if (want > nslabs / 8) want = nslabs / 8;
          const uint64_t fit = OCH_GEMM_WORKSPACE / ((uint64_t)g.M * g.N * sizeof(int));
