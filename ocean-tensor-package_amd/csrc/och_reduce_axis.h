@@ -28,6 +28,7 @@ struct AxisParams
       loads); every piece leaves its accumulator in partials[slice][output] (16-byte slots) and axis_finish_kernel
       folds the pieces in order */
    uint32_t slices, slice_len; int slice_rows;
+   int      dst_wide;                            /* per-thread kernel: the VEC results of a thread are neighbours in memory and 16-byte aligned */
    char    *partials;
    FastDiv  rgdiv;                               /* 128-bit groups per row of the first reduced dimension (cooperative kernels) */
    int64_t  st1[OCH_MAX_DIMS], st2[OCH_MAX_DIMS], rst[OCH_MAX_DIMS];
@@ -129,27 +130,62 @@ __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, co
       }
    }
    if (active && slice == 0)
-   {
+   {  typedef typename RD::Res Res;
+      /* results per store instruction: up to 16 bytes. Element-wise stores of a thread's VEC results put the lanes of
+         one store instruction VEC results apart (sums of 2 x 2^25 int8 into int64: 1.8 TB/s). */
+      constexpr int PV = (VEC > 1) ? ((sizeof(Res) * VEC >= 16) ? (int)(16 / sizeof(Res)) : VEC) : 1;
+      if (VEC > 1 && p.dst_wide && p.slices <= 1)
+      {
 #pragma unroll
-      for (int k = 0; k < VEC; k++)
-      {  if (p.slices > 1) *reinterpret_cast<Acc *>(p.partials + ((size_t)blockIdx.y * p.nout + o + k) * 16) = acc[k];
-         else *reinterpret_cast<typename RD::Res *>(p.dst + o2 + (int64_t)k * p.st2[0]) = RD::finalize(acc[k], prm);
+         for (int q = 0; q < VEC / PV; q++)
+         {  Pack<Res, PV> out;
+#pragma unroll
+            for (int k = 0; k < PV; k++) out.v[k] = RD::finalize(acc[q * PV + k], prm);
+            store_wide<Res, PV>(out, p.dst + o2 + (int64_t)(q * PV) * (int64_t)sizeof(Res));
+         }
+      }
+      else
+      {
+#pragma unroll
+         for (int k = 0; k < VEC; k++)
+         {  if (p.slices > 1) *reinterpret_cast<Acc *>(p.partials + ((size_t)blockIdx.y * p.nout + o + k) * 16) = acc[k];
+            else *reinterpret_cast<Res *>(p.dst + o2 + (int64_t)k * p.st2[0]) = RD::finalize(acc[k], prm);
+         }
       }
    }
 }
 
-/* folds the pieces of a sliced reduction in slice order: one thread per output */
+/* folds the pieces of a sliced reduction: `lanes` threads (a power of two, at most 64) per output. A lane takes pieces
+   lane, lane + lanes, ... in that order, four loads in flight, and the lanes are combined by a butterfly: a fixed order
+   for a given number of pieces, so the result is reproducible. With one thread per output the fold of a thousand pieces
+   was a chain of a thousand dependent memory latencies and took longer than the reduction itself. */
 template <class RD, class T>
-__global__ __launch_bounds__(256) void axis_finish_kernel(const AxisParams p, const typename RD::Param prm)
+__global__ __launch_bounds__(256) void axis_finish_kernel(const AxisParams p, const typename RD::Param prm, const uint32_t lanes)
 {
    typedef typename RD::Acc Acc;
-   const uint32_t o = blockIdx.x * 256 + threadIdx.x;
-   if (o >= p.nout) return;
-   int64_t o1, o2;
-   axis_outer_offsets(p, o, o1, o2);
-   Acc acc = *reinterpret_cast<const Acc *>(p.partials + (size_t)o * 16);
-   for (uint32_t t = 1; t < p.slices; t++) acc = RD::combine(acc, *reinterpret_cast<const Acc *>(p.partials + ((size_t)t * p.nout + o) * 16));
-   *reinterpret_cast<typename RD::Res *>(p.dst + o2) = RD::finalize(acc, prm);
+   const uint32_t o = (blockIdx.x * 256 + threadIdx.x) / lanes, lane = threadIdx.x % lanes;
+   const bool active = o < p.nout;
+   Acc acc = RD::identity();
+   if (active)
+   {  const char *slot = p.partials + (size_t)o * 16;
+      const size_t pitch = (size_t)p.nout * 16;
+      uint32_t t = lane;
+      for (; t + 3 * lanes < p.slices; t += 4 * lanes)
+      {  Acc v[4];
+#pragma unroll
+         for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const Acc *>(slot + (size_t)(t + u * lanes) * pitch);
+#pragma unroll
+         for (int u = 0; u < 4; u++) acc = RD::combine(acc, v[u]);
+      }
+      for (; t < p.slices; t += lanes) acc = RD::combine(acc, *reinterpret_cast<const Acc *>(slot + (size_t)t * pitch));
+   }
+#pragma unroll
+   for (int m = 32; m >= 1; m >>= 1) if ((uint32_t)m < lanes) acc = RD::combine(acc, shfl_xor_any<Acc>(acc, m));
+   if (active && lane == 0)
+   {  int64_t o1, o2;
+      axis_outer_offsets(p, o, o1, o2);
+      *reinterpret_cast<typename RD::Res *>(p.dst + o2) = RD::finalize(acc, prm);
+   }
 }
 
 /* A group of threads cooperates on one output: GROUP 256 = the whole block, GROUP 64 = p.glanes (8 .. 64, a power
@@ -291,6 +327,8 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
       bool wide = (VEC > 1) && p.nd > 0 && p.st1[0] == (int64_t)sizeof(T) && (p.div[0].d % VEC == 0) && (((uintptr_t)p.src) % 16 == 0);
       for (int d = 1; d < p.nd && wide; d++) if (p.st1[d] % 16 != 0) wide = false;
       for (int d = 0; d < p.rd && wide; d++) if (p.rst[d] % 16 != 0) wide = false;
+      p.dst_wide = (wide && p.st2[0] == (int64_t)sizeof(typename RD::Res) && (((uintptr_t)p.dst) % 16 == 0)) ? 1 : 0;
+      for (int d = 1; d < p.nd && p.dst_wide; d++) if (p.st2[d] % 16 != 0) p.dst_wide = 0;
       const uint64_t groups = wide ? nout / VEC : nout;
       const bool split = groups < (1u << 20) && p.rsize0 >= 16;
       p.opb = 64;
@@ -325,7 +363,10 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
          if (plan_slices(blocks, range, (uint64_t)(wave ? p.glanes : 256) * 8) != 0) return -1;
       }
       const dim3 grid(blocks, p.slices);
-      if (wide && streaming)
+      /* the nontemporal hint only where one load instruction of a wave covers whole cache lines: with fewer than eight
+         lanes per output the four loads of a lane share their lines with its neighbours' loads, and lines that are not
+         kept came from memory twice (8 floats per output: 3.8 TB/s with the hint) */
+      if (wide && streaming && (!wave || p.glanes >= 8))
       {  if (wave) hipLaunchKernelGGL((axis_group_kernel<RD, T, 64, VEC, true>), grid, dim3(256), 0, stream, p, prm);
          else      hipLaunchKernelGGL((axis_group_kernel<RD, T, 256, VEC, true>), grid, dim3(256), 0, stream, p, prm);
       }
@@ -338,7 +379,11 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
          else      hipLaunchKernelGGL((axis_group_kernel<RD, T, 256>), grid, dim3(256), 0, stream, p, prm);
       }
    }
-   if (p.slices > 1) hipLaunchKernelGGL((axis_finish_kernel<RD, T>), dim3((p.nout + 255) / 256), dim3(256), 0, stream, p, prm);
+   if (p.slices > 1)
+   {  uint32_t lanes = 1;                        /* at least eight pieces per lane, at most 2^20 threads */
+      while (lanes < 64 && lanes * 16 <= p.slices && (uint64_t)p.nout * lanes * 2 <= (1u << 20)) lanes *= 2;
+      hipLaunchKernelGGL((axis_finish_kernel<RD, T>), dim3((unsigned)(((uint64_t)p.nout * lanes + 255) / 256)), dim3(256), 0, stream, p, prm, lanes);
+   }
    OCH_CHECK_LAUNCH();
    return 0;
 }
