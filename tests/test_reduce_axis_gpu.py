@@ -30,10 +30,24 @@ def to_f64(dtype, a):
     return a.astype(np.complex128 if dtype >= H.CFLOAT else np.float64)
 
 
-def run_case(stream, name, dtype, parent, view, axes, p=3.0):
+def run_case(stream, name, dtype, parent, view, axes, p=3.0, shift=0):
+    """shift: the destination starts that many elements into its allocation (not 16-byte aligned any more)."""
     op = oh.R[name]
     rd = oh.lib.och_reduce_result_dtype(op, dtype)
     kept_shape = [n for d, n in enumerate(view.shape) if d not in axes]
+    if shift:
+        flat = np.zeros(int(np.prod(kept_shape)) + shift, H.storage(rd))
+        out_parent, out_view = flat, flat[shift:].reshape(kept_shape[::-1]).T
+        src = H.Operand(parent, view, dtype).upload(stream)
+        dst = H.Operand(out_parent, out_view, rd).upload(stream)
+        cfg = H.axis_config(src, dst, axes, stream)
+        oh.check(oh.lib.och_reduce_axis(op, dtype, cfg, p))
+        got = dst.download()
+        want = out_parent.copy()
+        dsth = H.Operand(want, want[shift:].reshape(kept_shape[::-1]).T, rd)
+        assert orc.lib.oracle_reduce_axis(op, dtype, H.axis_config(src, dsth, axes, device=False), p) == 0
+        src.free(); dst.free()
+        return rd, got, want
     out_parent = np.zeros(kept_shape[::-1] if kept_shape else (1,), H.storage(rd))     # column-major destination
     out_view = out_parent.T if kept_shape else out_parent.reshape(())
     src = H.Operand(parent, view, dtype).upload(stream)
@@ -147,7 +161,7 @@ SLICED = [  # Ocean shape (dimension 0 fastest), reduced axes: few outputs (or o
 @pytest.mark.parametrize("dtype", [H.INT32, H.FLOAT, H.DOUBLE, H.CFLOAT], ids=lambda d: H.NAMES[d])
 def test_axis_reductions_cut_into_pieces(hip, stream, dtype):
     """Too few outputs to occupy the device: the reduced range is cut into pieces (grid y), every piece leaves its
-    accumulator in the stream's workspace and a second kernel folds the pieces in order. Integers and extremes are exact,
+    accumulator in the stream's workspace and a second kernel folds the pieces in a fixed order. Integers and extremes are exact,
     floating sums / norms within the usual bounds of the float64 result."""
     rng = np.random.default_rng(900 + dtype)
     for shape, axes in SLICED:
@@ -170,3 +184,24 @@ def test_axis_reductions_cut_into_pieces(hip, stream, dtype):
             scale = np.abs(v).sum(axis=ax).T if name == "sum" else np.abs(truth)
             tol = 1e-12 if dtype == H.DOUBLE else 1e-5
             assert np.all(np.abs(g - truth) <= tol * np.maximum(np.asarray(scale), 1e-6)), what
+
+
+VECTOR_STORES = [(H.BOOL, "any"), (H.BOOL, "sum"), (H.INT8, "sum"), (H.UINT8, "maximum"), (H.INT16, "sum"), (H.INT16, "nnz"),
+                 (H.INT32, "minimum"), (H.HALF, "maximum"), (H.FLOAT, "any"), (H.FLOAT, "maximum"), (H.FLOAT, "nnz"),
+                 (H.DOUBLE, "all"), (H.DOUBLE, "minimum"), (H.CFLOAT, "nnz"), (H.CFLOAT, "any")]
+
+
+@pytest.mark.parametrize("dtype,name", VECTOR_STORES, ids=["%s-%s" % (H.NAMES[d], n) for d, n in VECTOR_STORES])
+def test_axis_results_stored_as_vectors(hip, stream, dtype, name):
+    """Neighbouring threads own neighbouring outputs and a thread's results (16 bytes of input wide: 2 to 16 of them) are
+    neighbours in the destination: they leave in stores of up to 16 bytes -- 1-byte logical results, 2- and 4-byte
+    extremes, 8-byte sums and counts in several stores per thread. Every result is exact. The same reduction into a
+    destination that starts one element into its allocation takes the element-wise stores and gives the same values,
+    and nothing is written in front of it."""
+    rng = np.random.default_rng(1200 + 16 * dtype + len(name))
+    for shape, axes in (((192, 37), [1]), ((64, 9, 5), [1]), ((4096, 3), [1])):
+        parent = H.random_data(dtype, int(np.prod(shape)), rng, "general").reshape(shape[::-1])
+        rd, got, want = run_case(stream, name, dtype, parent, parent.T, axes)
+        H.assert_same_bytes(got, want, "%s %s %s aligned" % (name, H.NAMES[dtype], shape))
+        rd, got1, want1 = run_case(stream, name, dtype, parent, parent.T, axes, shift=1)
+        H.assert_same_bytes(got1, want1, "%s %s %s shifted by one element" % (name, H.NAMES[dtype], shape))
