@@ -255,6 +255,28 @@ def main():
         for opn in ("sum", "norm2", "maximum"):
             ms = time_launches(lambda: oh.check(lib.och_reduce_all_device(R[opn], dt, 1, s3, st3, next_buf().ptr, None, None, 0.0, dres.ptr, None, h)), reps=10)
             configs["c3_%s_%s_8192^2" % (opn, nm)] = gbps(es * n3, ms)
+        # two more axis reductions over the same dense 2^26 elements, outside the named configurations: few outputs with
+        # a long strided reduced range (cut into pieces and folded by a second kernel), and many outputs of 8 elements each
+        few = oh.DeviceBuffer(es * 64, stream); many = oh.DeviceBuffer(es * (1 << 23), stream)
+        for label, osize, ostride, rsize, rstride, dest in (("64x2^20_axis1_few_outputs", 64, es, 1 << 20, 64 * es, few),
+                                                            ("8x2^23_axis0_short_rows", 1 << 23, 8 * es, 8, es, many)):
+            assert (osize - 1) * ostride + (rsize - 1) * rstride + es <= es * n3 and osize * es <= dest.nbytes
+            ecfgs = []
+            for buf in rbufs:
+                cfg = oh.ReduceAxisConfig()
+                cfg.ndims, cfg.rdims = 1, 1
+                cfg.size[0], cfg.strides1[0], cfg.strides2[0] = osize, ostride, es
+                cfg.rsize[0], cfg.rstrides[0] = rsize, rstride
+                cfg.ptr1, cfg.ptr2, cfg.stream = buf.ptr.value, dest.ptr.value, h
+                ecfgs.append(cfg)
+            eturn = [0]
+
+            def next_ecfg():
+                eturn[0] += 1
+                return ecfgs[eturn[0] % 2]
+            ms = time_launches(lambda: oh.check(lib.och_reduce_axis(R["sum"], dt, C.byref(next_ecfg()), 0.0)), reps=10)
+            configs["extra_axis_sum_%s_%s" % (nm, label)] = gbps(es * (n3 + osize), ms)
+        few.free(); many.free()
         # axis reductions on a 512 x 512 x 256 view with padded pitches (no two dimensions merge);
         # the view lives in a parent of (512+4) x (512+2) x 256 elements
         d0, d1, d2 = 512, 512, 256
