@@ -86,11 +86,38 @@ struct RedParams
    void *result;
    char *tail;                 /* flat layout only: elements left over after the last full group */
    int   ntail;
+   int64_t rowbytes;           /* row mode: bytes of one row of the first dimension */
 };
 
-/* WIDE: the first dimension is contiguous, divisible by VEC and aligned: VEC-wide loads (compile-time, so that the
-   loads stay single 128-bit instructions); otherwise VEC is 1 and any layout is accepted. */
-template <class RD, class T, int VEC, bool WIDE, bool NT = false>
+/* Row mode: the first dimension is contiguous but its rows are not whole aligned 16-byte groups (a width that is not a
+   multiple of VEC, a pitch or a start that is not a multiple of 16 bytes: sub-matrices of 1- and 2-byte types mostly).
+   Group g is chunk i of row r: the ALIGNED 16 bytes at (row start rounded down to 16) + 16 i. The first and the last
+   chunk of a row hold elements in front of / behind the row; [lo, hi) are the elements of the pack that belong to it.
+   A chunk is loaded only when it holds at least one element of the row, so every load stays inside a 16-byte unit that
+   the tensor owns part of. One load instruction per 16 bytes instead of one per element: 1000-byte rows of int8 at a
+   pitch of 1024 are summed at 0.67 TB/s element by element. */
+template <class T, int VEC>
+OCH_D void rows_load(const RedParams &p, uint32_t g, Pack<T, VEC> &v, int &lo, int &hi)
+{
+   const uint32_t r = fastdiv(g, p.ew.div[0]), i = g - r * p.ew.div[0].d;
+   int64_t rowoff = 0;
+   uint32_t q = r;
+   for (int d = 1; d < p.ew.ndims - 1; d++)
+   {  const uint32_t q2 = fastdiv(q, p.ew.div[d]);
+      rowoff += (int64_t)(q - q2 * p.ew.div[d].d) * p.ew.stride[0][d]; q = q2;
+   }
+   if (p.ew.ndims > 1) rowoff += (int64_t)q * p.ew.stride[0][p.ew.ndims - 1];
+   const char *row = p.ew.ptr[0] + rowoff;
+   const int64_t first = (int64_t)i * 16 - (int64_t)((uintptr_t)row & 15);       /* byte position of the chunk within the row */
+   const int64_t left = p.rowbytes - first;                                       /* bytes of the row from the chunk's start on */
+   lo = (first < 0) ? (int)((-first) / (int64_t)sizeof(T)) : 0;
+   hi = (left <= 0) ? 0 : ((left >= 16) ? VEC : (int)(left / (int64_t)sizeof(T)));
+   if (hi > lo) load_wide<T, VEC>(v, row + first);
+}
+
+/* MODE 1 (wide): the first dimension is contiguous, divisible by VEC and aligned: VEC-wide loads (compile-time, so that
+   the loads stay single 128-bit instructions); MODE 2: row mode (see rows_load); MODE 0: VEC is 1 and any layout is accepted. */
+template <class RD, class T, int VEC, int MODE, bool NT = false>
 __global__ __launch_bounds__(OCH_RED_BLOCK) void reduce_all_kernel(const RedParams p, const typename RD::Param prm)
 {
    typedef typename RD::Acc Acc;
@@ -110,25 +137,47 @@ __global__ __launch_bounds__(OCH_RED_BLOCK) void reduce_all_kernel(const RedPara
    /* main loop: OCH_RED_UNR independent groups per trip, loads first, one accumulator per group */
    for (; g + (OCH_RED_UNR - 1) * stride < end; g += OCH_RED_UNR * stride)
    {  Pack<T, VEC> v[OCH_RED_UNR];
+      if constexpr (MODE == 2)
+      {  int lo[OCH_RED_UNR], hi[OCH_RED_UNR];
 #pragma unroll
-      for (int u = 0; u < OCH_RED_UNR; u++)
-      {  int64_t off[1];
-         if (flat) off[0] = (int64_t)(g + u * stride) * p.ew.gstride[0];
-         else group_offsets<1>(p.ew, (uint32_t)(g + u * stride), off);
-         load_pack<T, VEC, NT>(v[u], p.ew.ptr[0] + off[0], p.ew.estride[0], WIDE);
+         for (int u = 0; u < OCH_RED_UNR; u++) { v[u] = Pack<T, VEC>{}; rows_load<T, VEC>(p, (uint32_t)(g + u * stride), v[u], lo[u], hi[u]); }
+#pragma unroll
+         for (int k = 0; k < VEC; k++)
+#pragma unroll
+            for (int u = 0; u < OCH_RED_UNR; u++) if (k >= lo[u] && k < hi[u]) part[u] = RD::combine(part[u], RD::load(v[u].v[k], prm));
       }
+      else
+      {
 #pragma unroll
-      for (int k = 0; k < VEC; k++)
+         for (int u = 0; u < OCH_RED_UNR; u++)
+         {  int64_t off[1];
+            if (flat) off[0] = (int64_t)(g + u * stride) * p.ew.gstride[0];
+            else group_offsets<1>(p.ew, (uint32_t)(g + u * stride), off);
+            load_pack<T, VEC, NT>(v[u], p.ew.ptr[0] + off[0], p.ew.estride[0], MODE == 1);
+         }
 #pragma unroll
-         for (int u = 0; u < OCH_RED_UNR; u++) part[u] = RD::combine(part[u], RD::load(v[u].v[k], prm));
+         for (int k = 0; k < VEC; k++)
+#pragma unroll
+            for (int u = 0; u < OCH_RED_UNR; u++) part[u] = RD::combine(part[u], RD::load(v[u].v[k], prm));
+      }
    }
    for (; g < end; g += stride)
-   {  Pack<T, VEC> v; int64_t off[1];
-      if (flat) off[0] = (int64_t)g * p.ew.gstride[0];
-      else group_offsets<1>(p.ew, (uint32_t)g, off);
-      load_pack<T, VEC>(v, p.ew.ptr[0] + off[0], p.ew.estride[0], WIDE);
+   {  Pack<T, VEC> v;
+      if constexpr (MODE == 2)
+      {  int lo, hi;
+         v = Pack<T, VEC>{};
+         rows_load<T, VEC>(p, (uint32_t)g, v, lo, hi);
 #pragma unroll
-      for (int k = 0; k < VEC; k++) part[0] = RD::combine(part[0], RD::load(v.v[k], prm));
+         for (int k = 0; k < VEC; k++) if (k >= lo && k < hi) part[0] = RD::combine(part[0], RD::load(v.v[k], prm));
+      }
+      else
+      {  int64_t off[1];
+         if (flat) off[0] = (int64_t)g * p.ew.gstride[0];
+         else group_offsets<1>(p.ew, (uint32_t)g, off);
+         load_pack<T, VEC>(v, p.ew.ptr[0] + off[0], p.ew.estride[0], MODE == 1);
+#pragma unroll
+         for (int k = 0; k < VEC; k++) part[0] = RD::combine(part[0], RD::load(v.v[k], prm));
+      }
    }
    Acc acc = part[0];
 #pragma unroll
@@ -203,6 +252,26 @@ static int launch_reduce_all(int ndims, const size_t *size, const ptrdiff_t *str
          p.ngroups = p.ew.ngroups;
       }
    }
+   /* row mode: contiguous rows of at least 24 bytes that the wide path cannot take (shorter rows would load about as
+      many chunks as they hold elements) */
+   bool rows_launch = false;
+   if constexpr (VEC > 1)
+   {  if (shape.nelem > 0 && !wide_launch && shape.stride[0][0] == (int64_t)sizeof(T) && ((uintptr_t)shape.ptr[0]) % sizeof(T) == 0
+          && shape.size[0] * sizeof(T) >= 24)
+      {  bool ok = true;
+         for (int d = 1; d < shape.ndims; d++) if (shape.stride[0][d] % (int64_t)sizeof(T) != 0) ok = false;
+         const uint64_t rowbytes = shape.size[0] * sizeof(T);
+         const uint64_t chunks = (16 - sizeof(T) + rowbytes + 15) / 16;            /* of the worst-placed row */
+         const uint64_t rows = shape.nelem / shape.size[0];
+         if (ok && chunks <= 0xFFFFFFFFull && rows * chunks <= 0xFFFF0000ull)
+         {  ew_params<1>(p.ew, shape, 1, es, 0);
+            p.ew.div[0] = make_fastdiv((uint32_t)chunks);
+            p.rowbytes = (int64_t)rowbytes;
+            p.ngroups = rows * chunks; p.ntail = 0; p.tail = nullptr;
+            rows_launch = true;
+         }
+      }
+   }
    p.partials = scratch;
    p.counter = reinterpret_cast<unsigned int *>(scratch + OCH_RED_MAX_BLOCKS * OCH_RED_SLOT);
    p.result = dresult;
@@ -216,9 +285,11 @@ static int launch_reduce_all(int ndims, const size_t *size, const ptrdiff_t *str
    /* sources that are read once from memory (larger than the caches) carry the nontemporal hint: measured on
       MI355X, 268 MB of float32 are summed at 6.3 TB/s with the hint and at 5.5 TB/s without */
    const bool streaming = wide_launch && p.ngroups * (uint64_t)(sizeof(T) * VEC) >= OCH_EW_STREAM_BYTES;
-   if (streaming)        hipLaunchKernelGGL((reduce_all_kernel<RD, T, VEC, true, true>), dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
-   else if (wide_launch) hipLaunchKernelGGL((reduce_all_kernel<RD, T, VEC, true>), dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
-   else             hipLaunchKernelGGL((reduce_all_kernel<RD, T, 1, false>),  dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
+   if (streaming)        hipLaunchKernelGGL((reduce_all_kernel<RD, T, VEC, 1, true>), dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
+   else if (wide_launch) hipLaunchKernelGGL((reduce_all_kernel<RD, T, VEC, 1>), dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
+   else if (rows_launch)
+   {  if constexpr (VEC > 1) hipLaunchKernelGGL((reduce_all_kernel<RD, T, VEC, 2>), dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm); }
+   else             hipLaunchKernelGGL((reduce_all_kernel<RD, T, 1, 0>),  dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
    OCH_CHECK_LAUNCH();
    return 0;
 }

@@ -270,3 +270,47 @@ def test_reductions_on_two_streams_do_not_share_scratch(hip, stream):
     for b in bufs + outs:
         b.free()
     other.synchronize(); other.destroy()
+
+
+ROW_TYPES = [H.BOOL, H.INT8, H.UINT8, H.INT16, H.UINT16, H.HALF, H.INT32, H.FLOAT, H.INT64, H.DOUBLE, H.CHALF, H.CFLOAT]
+
+
+@pytest.mark.parametrize("dtype", ROW_TYPES, ids=lambda d: H.NAMES[d])
+def test_reduce_rows_that_are_not_whole_vectors(hip, stream, dtype):
+    """Contiguous rows that the 16-byte path cannot take as they are -- a width that is not a multiple of the vector
+    length, a row pitch that is not a multiple of 16 bytes, a view that starts inside a 16-byte unit, a single misaligned
+    run -- are read in aligned 16-byte chunks whose elements outside the row are left out. The elements next to every
+    row (the rest of the parent) hold values that would change every result if one of them were counted. Counts,
+    extremes and integer sums are exact; floating sums are within the usual bound of the float64 value."""
+    rng = np.random.default_rng(3100 + dtype)
+    es = np.dtype(H.storage(dtype)).itemsize
+    layouts = []            # (parent shape, view builder)
+    layouts.append(((37, 1024), lambda p: p[:, 3:1003].T))                 # 1000 wide, starts 3 elements in, aligned pitch
+    layouts.append(((29, 1001), lambda p: p[:, 0:999].T))                  # odd width, odd pitch: every row placed differently
+    layouts.append(((5000,), lambda p: p[1:4998]))                         # one run that starts one element in
+    layouts.append(((5, 7, 130), lambda p: p[:, :, 1:101].transpose(2, 1, 0)))
+    layouts.append(((300, 70), lambda p: p[:, 1:70].T))                    # rows a little over 64 bytes for 1-byte types
+    layouts.append(((400, 33), lambda p: p[:, 1:32].T))                    # 31 elements: two or three chunks per row of bytes
+    for shape, build in layouts:
+        n = int(np.prod(shape))
+        kind = "small" if dtype in (H.HALF, H.CHALF) else "general"
+        parent = H.random_data(dtype, n, rng, kind).reshape(shape)
+        view = build(parent)
+        inside = np.zeros(shape, bool); build(inside)[...] = True
+        # poison what lies outside the view: large values (and a non-zero count) that no result may reflect
+        flat = parent.reshape(-1); mask = ~inside.reshape(-1)
+        poison = H.random_data(dtype, n, rng, "positive" if dtype != H.BOOL else "general")
+        flat[mask] = poison[mask]
+        x = H.Operand(parent, view, dtype).upload(stream)
+        for name in ("sum", "maximum", "minimum", "nnz", "any", "all"):
+            op = oh.R[name]
+            if not oh.lib.och_reduce_supported(op, dtype):
+                continue
+            rd, got = gpu_reduce(stream, op, dtype, x)
+            _, want = cpu_reduce(op, dtype, x)
+            what = "%s %s parent %s" % (name, H.NAMES[dtype], shape)
+            if name != "sum" or dtype <= H.INT64:
+                H.assert_same_bytes(got, want, what)
+            else:
+                check_against_truth(name, dtype, rd, got, np.ascontiguousarray(view))
+        x.free()
