@@ -28,6 +28,7 @@ struct AxisParams
       loads); every piece leaves its accumulator in partials[slice][output] (16-byte slots) and axis_finish_kernel
       folds the pieces in order */
    uint32_t slices, slice_len; int slice_rows;
+   int64_t  rowbytes;                            /* row mode of the cooperative kernels: bytes of one row of the first reduced dimension */
    int      dst_wide;                            /* per-thread kernel: the VEC results of a thread are neighbours in memory and 16-byte aligned */
    char    *partials;
    FastDiv  rgdiv;                               /* 128-bit groups per row of the first reduced dimension (cooperative kernels) */
@@ -188,11 +189,29 @@ __global__ __launch_bounds__(256) void axis_finish_kernel(const AxisParams p, co
    }
 }
 
+/* One load of the cooperative kernels: element (VEC 1), aligned 16-byte group i of the row (VEC > 1), or -- row mode,
+   for contiguous rows that are not whole aligned groups: odd width, odd pitch, a start inside a 16-byte unit -- the
+   aligned 16-byte chunk i counted from the row start rounded down to 16, of which only the elements [lo, hi) belong
+   to the row. A chunk is loaded only when it holds an element of the row. */
+template <class T, int VEC, bool ROWS, bool NT>
+OCH_D void axis_fetch(Pack<T, VEC> &v, const char *rowbase, uint32_t i, int64_t s0, int64_t rowbytes, int &lo, int &hi)
+{
+   if constexpr (VEC > 1 && ROWS)
+   {  const int64_t first = (int64_t)i * 16 - (int64_t)((uintptr_t)rowbase & 15);
+      const int64_t left = rowbytes - first;
+      lo = (first < 0) ? (int)((-first) / (int64_t)sizeof(T)) : 0;
+      hi = (left <= 0) ? 0 : ((left >= 16) ? VEC : (int)(left / (int64_t)sizeof(T)));
+      if (hi > lo) load_wide<T, VEC>(v, rowbase + first);
+   }
+   else if constexpr (VEC > 1) { lo = 0; hi = VEC; load_wide<T, VEC, NT>(v, rowbase + (int64_t)i * s0); }
+   else { lo = 0; hi = 1; v.v[0] = *reinterpret_cast<const T *>(rowbase + (int64_t)i * s0); }
+}
+
 /* A group of threads cooperates on one output: GROUP 256 = the whole block, GROUP 64 = p.glanes (8 .. 64, a power
    of two) lanes of a wave (1 .. 64), chosen so that every lane has about four loads in flight on short rows. VEC > 1: the first reduced
    dimension has unit stride and every row starts 16-byte aligned, so a thread takes VEC neighbouring elements with
-   one 128-bit load (NT: with the nontemporal hint, for sources that are read once from memory). */
-template <class RD, class T, int GROUP, int VEC = 1, bool NT = false>
+   one 128-bit load (NT: with the nontemporal hint, for sources that are read once from memory); ROWS: see axis_fetch. */
+template <class RD, class T, int GROUP, int VEC = 1, bool NT = false, bool ROWS = false>
 __global__ __launch_bounds__(256) void axis_group_kernel(const AxisParams p, const typename RD::Param prm)
 {
    typedef typename RD::Acc Acc;
@@ -207,41 +226,41 @@ __global__ __launch_bounds__(256) void axis_group_kernel(const AxisParams p, con
    {  axis_outer_offsets(p, o, o1, o2);
       const char *base = p.src + o1;
       const int64_t s0 = (VEC > 1) ? (int64_t)(sizeof(T) * VEC) : p.rst[0];        /* step of one group */
-      const uint32_t n0 = (VEC > 1) ? p.rgdiv.d : p.rsize0;                        /* groups per row */
+      const uint32_t n0 = (VEC > 1) ? p.rgdiv.d : p.rsize0;                        /* groups (chunks) per row */
       /* range of loads of this piece of the reduced range */
-      const uint32_t total = (p.rd <= 1) ? n0 : ((VEC > 1) ? p.relem / VEC : p.relem);
+      const uint32_t total = (p.rd <= 1) ? n0 : ((VEC > 1) ? p.rrows * n0 : p.relem);
       uint32_t lo = 0, hi = total;
       if (p.slices > 1) { lo = blockIdx.y * p.slice_len; hi = (lo + p.slice_len < total) ? lo + p.slice_len : total; }
       if (p.rd <= 1)
       {  uint32_t i = lo + lane;
          for (; i + 3 * G < hi; i += 4 * G)
-         {  Pack<T, VEC> v[4];
+         {  Pack<T, VEC> v[4]; int klo[4], khi[4];
 #pragma unroll
             for (int u = 0; u < 4; u++)
-            {  if constexpr (VEC > 1) load_wide<T, VEC, NT>(v[u], base + (int64_t)(i + u * G) * s0);
-               else v[u].v[0] = *reinterpret_cast<const T *>(base + (int64_t)(i + u * G) * s0);
+            {  if constexpr (ROWS) v[u] = Pack<T, VEC>{};
+               axis_fetch<T, VEC, ROWS, NT>(v[u], base, i + u * G, s0, p.rowbytes, klo[u], khi[u]);
             }
 #pragma unroll
             for (int u = 0; u < 4; u++)
 #pragma unroll
-               for (int k = 0; k < VEC; k++) acc = RD::combine(acc, RD::load(v[u].v[k], prm));
+               for (int k = 0; k < VEC; k++) if (k >= klo[u] && k < khi[u]) acc = RD::combine(acc, RD::load(v[u].v[k], prm));
          }
          for (; i < hi; i += G)
-         {  Pack<T, VEC> v;
-            if constexpr (VEC > 1) load_wide<T, VEC, NT>(v, base + (int64_t)i * s0);
-            else v.v[0] = *reinterpret_cast<const T *>(base + (int64_t)i * s0);
+         {  Pack<T, VEC> v; int klo, khi;
+            if constexpr (ROWS) v = Pack<T, VEC>{};
+            axis_fetch<T, VEC, ROWS, NT>(v, base, i, s0, p.rowbytes, klo, khi);
 #pragma unroll
-            for (int k = 0; k < VEC; k++) acc = RD::combine(acc, RD::load(v.v[k], prm));
+            for (int k = 0; k < VEC; k++) if (k >= klo && k < khi) acc = RD::combine(acc, RD::load(v.v[k], prm));
          }
       }
       else
       {  for (uint32_t j = lo + lane; j < hi; j += G)
          {  uint32_t r = fastdiv(j, (VEC > 1) ? p.rgdiv : p.rdiv[0]); uint32_t i = j - r * n0;
-            Pack<T, VEC> v;
-            if constexpr (VEC > 1) load_wide<T, VEC, NT>(v, base + axis_row_offset(p, r) + (int64_t)i * s0);
-            else v.v[0] = *reinterpret_cast<const T *>(base + axis_row_offset(p, r) + (int64_t)i * s0);
+            Pack<T, VEC> v; int klo, khi;
+            if constexpr (ROWS) v = Pack<T, VEC>{};
+            axis_fetch<T, VEC, ROWS, NT>(v, base + axis_row_offset(p, r), i, s0, p.rowbytes, klo, khi);
 #pragma unroll
-            for (int k = 0; k < VEC; k++) acc = RD::combine(acc, RD::load(v.v[k], prm));
+            for (int k = 0; k < VEC; k++) if (k >= klo && k < khi) acc = RD::combine(acc, RD::load(v.v[k], prm));
          }
       }
    }
@@ -352,14 +371,25 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
       for (int d = 0; d < p.nd && wide; d++) if (p.st1[d] % 16 != 0) wide = false;
       for (int d = 1; d < p.rd && wide; d++) if (p.rst[d] % 16 != 0) wide = false;
       if (wide) p.rgdiv = make_fastdiv(p.rsize0 / VEC);
+      /* row mode: contiguous rows of at least 24 bytes that are not whole aligned groups */
+      bool rows = false;
+      if (VEC > 1 && !wide && p.rst[0] == (int64_t)sizeof(T) && ((uintptr_t)p.src) % sizeof(T) == 0 && (uint64_t)p.rsize0 * sizeof(T) >= 24)
+      {  rows = true;
+         for (int d = 0; d < p.nd; d++) if (p.st1[d] % (int64_t)sizeof(T) != 0) rows = false;
+         for (int d = 1; d < p.rd; d++) if (p.rst[d] % (int64_t)sizeof(T) != 0) rows = false;
+         const uint64_t rowbytes = (uint64_t)p.rsize0 * sizeof(T);
+         const uint64_t chunks = (16 - sizeof(T) + rowbytes + 15) / 16;             /* of the worst-placed row */
+         if (chunks * p.rrows > 0xFFFFFF00ull) rows = false;
+         if (rows) { p.rgdiv = make_fastdiv((uint32_t)chunks); p.rowbytes = (int64_t)rowbytes; }
+      }
       const bool wave = relem <= 2048 && nout >= 1024;              /* a wave per output, else a block per output */
-      const uint32_t loads = wide ? p.relem / VEC : p.relem;       /* loads per output: about four per lane */
+      const uint32_t loads = wide ? p.relem / VEC : (rows ? p.rrows * p.rgdiv.d : p.relem);       /* loads per output: about four per lane */
       p.glanes = 64;
       while (p.glanes > 1 && (p.glanes / 2) * 4 >= loads) p.glanes /= 2;
       const uint32_t per_block = 256 / p.glanes;
       const unsigned blocks = wave ? (p.nout + per_block - 1) / per_block : p.nout;
       p.slice_rows = 0;
-      {  const uint64_t range = (p.rd <= 1) ? (wide ? p.rsize0 / VEC : p.rsize0) : loads;
+      {  const uint64_t range = (p.rd <= 1) ? (wide ? p.rsize0 / VEC : (rows ? p.rgdiv.d : p.rsize0)) : loads;
          if (plan_slices(blocks, range, (uint64_t)(wave ? p.glanes : 256) * 8) != 0) return -1;
       }
       const dim3 grid(blocks, p.slices);
@@ -373,6 +403,12 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
       else if (wide)
       {  if (wave) hipLaunchKernelGGL((axis_group_kernel<RD, T, 64, VEC>), grid, dim3(256), 0, stream, p, prm);
          else      hipLaunchKernelGGL((axis_group_kernel<RD, T, 256, VEC>), grid, dim3(256), 0, stream, p, prm);
+      }
+      else if (rows)
+      {  if constexpr (VEC > 1)
+         {  if (wave) hipLaunchKernelGGL((axis_group_kernel<RD, T, 64, VEC, false, true>), grid, dim3(256), 0, stream, p, prm);
+            else      hipLaunchKernelGGL((axis_group_kernel<RD, T, 256, VEC, false, true>), grid, dim3(256), 0, stream, p, prm);
+         }
       }
       else
       {  if (wave) hipLaunchKernelGGL((axis_group_kernel<RD, T, 64>), grid, dim3(256), 0, stream, p, prm);

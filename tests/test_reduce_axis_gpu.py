@@ -205,3 +205,41 @@ def test_axis_results_stored_as_vectors(hip, stream, dtype, name):
         H.assert_same_bytes(got, want, "%s %s %s aligned" % (name, H.NAMES[dtype], shape))
         rd, got1, want1 = run_case(stream, name, dtype, parent, parent.T, axes, shift=1)
         H.assert_same_bytes(got1, want1, "%s %s %s shifted by one element" % (name, H.NAMES[dtype], shape))
+
+
+ROW_MODE_TYPES = [H.BOOL, H.INT8, H.INT16, H.HALF, H.INT32, H.FLOAT, H.CFLOAT]
+
+
+@pytest.mark.parametrize("dtype", ROW_MODE_TYPES, ids=lambda d: H.NAMES[d])
+def test_axis_rows_that_are_not_whole_vectors(hip, stream, dtype):
+    """Reductions along a contiguous dimension whose rows are not whole aligned 16-byte groups (odd width, odd pitch, a
+    view that starts inside a 16-byte unit): the rows are read in aligned 16-byte chunks and the elements of the first
+    and last chunk outside the row are left out. A block per output, a few lanes per output, two reduced dimensions and
+    a reduced range cut into pieces; what lies next to the rows in the parent would change every result if counted."""
+    rng = np.random.default_rng(4100 + dtype)
+    layouts = [((37, 1024), lambda p: p[:, 3:1003].T, [0]),                      # 37 outputs, a block each
+               ((1500, 70), lambda p: p[:, 1:70].T, [0]),                        # 1500 outputs, a few lanes each
+               ((29, 1001), lambda p: p[:, 0:999].T, [0]),                       # every row placed differently
+               ((6, 40, 130), lambda p: p[:, :, 1:101].transpose(2, 1, 0), [0, 2]),
+               ((3, 300001), lambda p: p[:, 1:300000].T, [0])]                   # three outputs, rows cut into pieces
+    for shape, build, axes in layouts:
+        n = int(np.prod(shape))
+        parent = H.random_data(dtype, n, rng, "small" if dtype == H.HALF else "general").reshape(shape)
+        inside = np.zeros(shape, bool); build(inside)[...] = True
+        poison = H.random_data(dtype, n, rng, "positive" if dtype != H.BOOL else "general")
+        flat, mask = parent.reshape(-1), ~inside.reshape(-1)
+        flat[mask] = poison[mask]
+        view = build(parent)
+        v = to_f64(dtype, view)
+        for name in ("sum", "maximum", "nnz"):
+            if not oh.lib.och_reduce_supported(oh.R[name], dtype):
+                continue
+            rd, got, want = run_case(stream, name, dtype, parent, view, axes)
+            what = "%s %s parent %s" % (name, H.NAMES[dtype], shape)
+            if name != "sum" or dtype <= H.INT64:
+                H.assert_same_bytes(got, want, what)
+                continue
+            g, ax = to_f64(rd, got), tuple(axes)
+            truth, scale = v.sum(axis=ax).T, np.abs(v).sum(axis=ax).T
+            tol = 4e-3 if dtype == H.HALF else 1e-5
+            assert np.all(np.abs(g - truth) <= tol * np.maximum(np.asarray(scale), 1e-6)), what
