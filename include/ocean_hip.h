@@ -254,6 +254,11 @@ int och_binary_result_dtype(int op, int dtype);
 /* `buffer` may be NULL (the library then uses a per-device scratch block); */
 /* otherwise it must hold och_reduce_all_buffer_size() bytes.               */
 /* bound/lower/upper are given in the tensor's own dtype.                   */
+/* Reductions (full and along axes) read a contiguous row that is not made  */
+/* of whole 16-byte groups in ALIGNED 16-byte loads: of the first and last  */
+/* 16-byte unit that a row touches, bytes next to the row are loaded too    */
+/* (never used, never written). No load leaves a 16-byte unit of which the  */
+/* tensor owns at least one byte.                                           */
 /* ======================================================================== */
 typedef enum {
    OCH_R_ANY = 0, OCH_R_ALL, OCH_R_ALL_FINITE, OCH_R_ANY_INF, OCH_R_ANY_NAN,
