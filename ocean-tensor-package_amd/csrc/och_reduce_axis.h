@@ -29,6 +29,10 @@ struct AxisParams
       folds the pieces in order */
    uint32_t slices, slice_len; int slice_rows;
    int64_t  rowbytes;                            /* row mode of the cooperative kernels: bytes of one row of the first reduced dimension */
+   /* row mode of the per-thread kernel: the rows of the first outer dimension are not whole aligned groups, but every row
+      starts at the same position row_m within a 16-byte unit; a thread owns the aligned chunk c of a row, i.e. the
+      outputs c * VEC - row_m / sizeof(T) + k that lie inside the row (rgdiv: chunks per row) */
+   uint32_t row_groups, row_n0; int row_m;
    int      dst_wide;                            /* per-thread kernel: the VEC results of a thread are neighbours in memory and 16-byte aligned */
    char    *partials;
    FastDiv  rgdiv;                               /* 128-bit groups per row of the first reduced dimension (cooperative kernels) */
@@ -71,7 +75,7 @@ OCH_D uint32_t xcd_neighbour_block(uint32_t b, uint32_t nblocks)
    covers them; needs unit source stride along the first outer dimension). SPLIT slices (waves
    when SPLIT is 4) share each output: slice s takes elements s, s + SPLIT, ... of every row of
    the reduced range and the slices are folded through LDS in slice order. */
-template <class RD, class T, int SPLIT, int VEC, bool NT = false>
+template <class RD, class T, int SPLIT, int VEC, bool NT = false, bool ROWS = false>
 __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, const typename RD::Param prm)
 {
    typedef typename RD::Acc Acc;
@@ -82,15 +86,24 @@ __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, co
    constexpr int UNR = (VEC > 1) ? 4 : 8;
    __shared__ Acc lds[SPLIT > 1 ? 256 * VEC : 1];
    const uint32_t slice = threadIdx.x / OPB, ol = threadIdx.x % OPB;
-   const uint32_t o = (xcd_neighbour_block(blockIdx.x, gridDim.x) * OPB + ol) * VEC;
-   const bool active = o < p.nout;
+   const uint32_t group = xcd_neighbour_block(blockIdx.x, gridDim.x) * OPB + ol;
+   /* first output of the thread; row mode: first output of the thread's row, and the position of pack element 0 in it */
+   uint32_t o = group * VEC; int first = 0; int64_t chunk = 0;
+   bool active = o < p.nout;
+   if constexpr (ROWS)
+   {  active = group < p.row_groups;
+      const uint32_t q = fastdiv(group, p.rgdiv), c = group - q * p.rgdiv.d;
+      o = q * p.row_n0;
+      first = (int)(c * VEC) - p.row_m / (int)sizeof(T);
+      chunk = (int64_t)c * 16 - p.row_m;
+   }
    Acc acc[VEC];
 #pragma unroll
    for (int k = 0; k < VEC; k++) acc[k] = RD::identity();
    int64_t o1 = 0, o2 = 0;
    if (active)
    {  axis_outer_offsets(p, o, o1, o2);
-      const char *base = p.src + o1;
+      const char *base = p.src + o1 + chunk;
       const int64_t s0 = p.rst[0];
       uint32_t r_lo = 0, r_hi = p.rrows, i_lo = 0, i_hi = p.rsize0;
       if (p.slices > 1)
@@ -135,7 +148,18 @@ __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, co
       /* results per store instruction: up to 16 bytes. Element-wise stores of a thread's VEC results put the lanes of
          one store instruction VEC results apart (sums of 2 x 2^25 int8 into int64: 1.8 TB/s). */
       constexpr int PV = (VEC > 1) ? ((sizeof(Res) * VEC >= 16) ? (int)(16 / sizeof(Res)) : VEC) : 1;
-      if (VEC > 1 && p.dst_wide && p.slices <= 1)
+      if constexpr (ROWS)
+      {
+#pragma unroll
+         for (int k = 0; k < VEC; k++)
+         {  const int i = first + k;                   /* position in the row; elements of the chunk outside the row are dropped */
+            if (i >= 0 && (uint32_t)i < p.row_n0)
+            {  if (p.slices > 1) *reinterpret_cast<Acc *>(p.partials + ((size_t)blockIdx.y * p.nout + o + (uint32_t)i) * 16) = acc[k];
+               else *reinterpret_cast<Res *>(p.dst + o2 + (int64_t)i * p.st2[0]) = RD::finalize(acc[k], prm);
+            }
+         }
+      }
+      else if (VEC > 1 && p.dst_wide && p.slices <= 1)
       {
 #pragma unroll
          for (int q = 0; q < VEC / PV; q++)
@@ -348,7 +372,22 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
       for (int d = 0; d < p.rd && wide; d++) if (p.rst[d] % 16 != 0) wide = false;
       p.dst_wide = (wide && p.st2[0] == (int64_t)sizeof(typename RD::Res) && (((uintptr_t)p.dst) % 16 == 0)) ? 1 : 0;
       for (int d = 1; d < p.nd && p.dst_wide; d++) if (p.st2[d] % 16 != 0) p.dst_wide = 0;
-      const uint64_t groups = wide ? nout / VEC : nout;
+      /* row mode: unit stride along the first outer dimension, every other stride a multiple of 16 bytes (so all rows
+         start at the same position within a 16-byte unit), rows of at least 24 bytes, but not whole aligned groups */
+      bool rows = false;
+      if (VEC > 1 && !wide && p.nd > 0 && p.st1[0] == (int64_t)sizeof(T) && ((uintptr_t)p.src) % sizeof(T) == 0 && (uint64_t)p.div[0].d * sizeof(T) >= 24)
+      {  rows = true;
+         for (int d = 1; d < p.nd; d++) if (p.st1[d] % 16 != 0) rows = false;
+         for (int d = 0; d < p.rd; d++) if (p.rst[d] % 16 != 0) rows = false;
+         if (rows)
+         {  p.row_m = (int)(((uintptr_t)p.src) % 16); p.row_n0 = p.div[0].d;
+            const uint64_t chunks = ((uint64_t)p.row_m + (uint64_t)p.row_n0 * sizeof(T) + 15) / 16;
+            const uint64_t total = chunks * (nout / p.row_n0);
+            if (total > 0xFFFFFF00ull) rows = false;
+            else { p.rgdiv = make_fastdiv((uint32_t)chunks); p.row_groups = (uint32_t)total; }
+         }
+      }
+      const uint64_t groups = wide ? nout / VEC : (rows ? (uint64_t)p.row_groups : nout);
       const bool split = groups < (1u << 20) && p.rsize0 >= 16;
       p.opb = 64;
       while (p.opb > 1 && p.opb / 2 >= groups) p.opb /= 2;
@@ -361,6 +400,12 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
       else if (wide && split)         hipLaunchKernelGGL((axis_thread_kernel<RD, T, 4, VEC>), grid, dim3(256), 0, stream, p, prm);
       else if (wide && streaming)     hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, VEC, true>), grid, dim3(256), 0, stream, p, prm);
       else if (wide)                  hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, VEC>), grid, dim3(256), 0, stream, p, prm);
+      else if (rows)
+      {  if constexpr (VEC > 1)
+         {  if (split) hipLaunchKernelGGL((axis_thread_kernel<RD, T, 4, VEC, false, true>), grid, dim3(256), 0, stream, p, prm);
+            else       hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, VEC, false, true>), grid, dim3(256), 0, stream, p, prm);
+         }
+      }
       else if (split)                 hipLaunchKernelGGL((axis_thread_kernel<RD, T, 4, 1>), grid, dim3(256), 0, stream, p, prm);
       else                            hipLaunchKernelGGL((axis_thread_kernel<RD, T, 1, 1>), grid, dim3(256), 0, stream, p, prm);
    }

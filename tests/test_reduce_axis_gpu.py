@@ -221,7 +221,12 @@ def test_axis_rows_that_are_not_whole_vectors(hip, stream, dtype):
                ((1500, 70), lambda p: p[:, 1:70].T, [0]),                        # 1500 outputs, a few lanes each
                ((29, 1001), lambda p: p[:, 0:999].T, [0]),                       # every row placed differently
                ((6, 40, 130), lambda p: p[:, :, 1:101].transpose(2, 1, 0), [0, 2]),
-               ((3, 300001), lambda p: p[:, 1:300000].T, [0])]                   # three outputs, rows cut into pieces
+               ((3, 300001), lambda p: p[:, 1:300000].T, [0]),                   # three outputs, rows cut into pieces
+               # the kept dimension is the contiguous one: a thread owns an aligned chunk of neighbouring outputs
+               ((37, 1024), lambda p: p[:, 3:1003].T, [1]),
+               ((9, 50, 48), lambda p: p[:, :, 1:44].transpose(2, 1, 0), [1]),
+               ((9, 50, 48), lambda p: p[:, :, 1:44].transpose(2, 1, 0), [1, 2]),
+               ((300000, 48), lambda p: p[:, 1:40].T, [1])]                      # 39 outputs, a long range cut into pieces
     for shape, build, axes in layouts:
         n = int(np.prod(shape))
         parent = H.random_data(dtype, n, rng, "small" if dtype == H.HALF else "general").reshape(shape)
