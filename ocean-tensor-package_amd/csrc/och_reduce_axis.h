@@ -391,6 +391,9 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
       const bool split = groups < (1u << 20) && p.rsize0 >= 16;
       p.opb = 64;
       while (p.opb > 1 && p.opb / 2 >= groups) p.opb /= 2;
+      /* fewer blocks than compute units: narrower blocks (down to 32 groups = 512 contiguous bytes per row) before the
+         reduced range is cut into pieces, which costs a second kernel */
+      if (split && wide) while (p.opb > 32 && (groups + p.opb - 1) / p.opb < 256 && p.rsize0 >= 32 * (256 / (p.opb / 2))) p.opb /= 2;
       const unsigned blocks = (unsigned)(split ? (groups + p.opb - 1) / p.opb : (groups + 255) / 256);
       /* pieces of the reduced range: whole rows of it when there are several, else positions along its first dimension */
       p.slice_rows = (p.rd > 1 && p.rrows >= 8) ? 1 : 0;
