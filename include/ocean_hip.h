@@ -282,6 +282,17 @@ int och_reduce_all(int op, int dtype, int ndims, const size_t *size, const ptrdi
 int och_reduce_all_device(int op, int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
                    void *ptr, const och_scalar *param1, const och_scalar *param2, double p,
                    void *dresult, void *buffer, och_stream stream);
+/* The same reduction for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses */
+/* that forbid hipMalloc). No counterpart in the reference. It calls no allocating routine: the partial slots and the */
+/* ticket counter live in a fixed array of och_reduce_all_buffer_size() bytes (8448) inside the library's device code, */
+/* one copy per device, held until the process ends; its address is looked up by och_device_warmup (or by the first   */
+/* call on a device). Tensors of more than och_reduce_all_noalloc_max_elements() (2^40) elements are refused with an  */
+/* error. All calls on one device share the array: calls that overlap (different streams, different host threads) on  */
+/* one device race and give wrong results; calls on one stream are ordered and safe. */
+int och_reduce_all_device_noalloc(int op, int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+                   void *ptr, const och_scalar *param1, const och_scalar *param2, double p,
+                   void *dresult, och_stream stream);
+size_t och_reduce_all_noalloc_max_elements(void);
 
 /* ======================================================================== */
 /* Axis reductions (template_reduce_axis.cu:54-80; reduce_axis.h:563-597)   */

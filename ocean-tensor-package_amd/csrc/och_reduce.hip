@@ -2,6 +2,7 @@
  * the stream they run on. */
 #include "och_reduce_all.h"
 #include <string.h>
+#include <mutex>
 
 namespace och {
 /* the instantiations are spread over eight translation units (build time); each knows its own operations */
@@ -57,6 +58,58 @@ extern "C" int och_reduce_all_device(int op, int dtype, int ndims, const size_t 
       scratch = ctx->red_scratch;
    }
    return fn(ndims, size, strides, ptr, param1, param2, p, dresult, scratch, buffer != nullptr, as_stream(stream));
+}
+
+/* ---- the entry point that allocates nothing ------------------------------------------------
+   Same kernels as och_reduce_all_device; the partial slots and the ticket counter live in a
+   file-scope device array instead of memory that the library or the caller allocates. The array's
+   name is only a host-side handle: its device address is asked for once per device (each device
+   holds its own copy at its own address) and only that address is ever handed to a kernel. */
+#define OCH_RED_STATIC_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[OCH_RED_SCRATCH];
+static char *g_static_scratch[OCH_RED_STATIC_DEVICES];
+static std::mutex g_static_scratch_mutex;
+
+namespace och {
+int reduce_static_scratch(char **out)
+{
+   int dev;
+   OCH_CHECK_HIP(hipGetDevice(&dev));
+   if (dev < 0 || dev >= OCH_RED_STATIC_DEVICES) return set_error("device index %d is beyond the %d devices the static scratch covers", dev, OCH_RED_STATIC_DEVICES);
+   std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+   if (g_static_scratch[dev] == nullptr)
+   {  void *ptr = nullptr;
+      OCH_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+      if (ptr == nullptr) return set_error("the static reduction scratch has no address on device %d", dev);
+      g_static_scratch[dev] = (char *)ptr;
+   }
+   *out = g_static_scratch[dev];
+   return 0;
+}
+}
+
+extern "C" size_t och_reduce_all_noalloc_max_elements(void) { return (size_t)OCH_RED_NOALLOC_MAX_ELEMENTS; }
+
+extern "C" int och_reduce_all_device_noalloc(int op, int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,
+                   void *ptr, const och_scalar *param1, const och_scalar *param2, double p,
+                   void *dresult, och_stream stream)
+{
+   red_fn fn = reduce_lookup(op, dtype);
+   if (fn == nullptr) return set_error("reduction %d is not available for data type %d", op, dtype);
+   if (ndims < 0 || ndims > OCH_MAX_DIMS) return set_error("invalid number of dimensions (%d)", ndims);
+   if (dresult == nullptr) return set_error("och_reduce_all_device_noalloc: null result pointer");
+   unsigned long long nelem = 1;
+   for (int d = 0; d < ndims; d++)
+   {  if (size[d] != 0 && nelem > OCH_RED_NOALLOC_MAX_ELEMENTS / size[d])
+         return set_error("och_reduce_all_device_noalloc: more than %llu elements; use och_reduce_all_device", (unsigned long long)OCH_RED_NOALLOC_MAX_ELEMENTS);
+      nelem *= size[d];
+   }
+   char *dscratch;
+   if (reduce_static_scratch(&dscratch) != 0) return -1;
+   /* the array keeps what the last call (or a failed launch) left: the counter is cleared by a small fill kernel on
+      this stream in front of every reduction; the partial slots need no clearing (every slot that is read was written
+      by this launch) */
+   return fn(ndims, size, strides, ptr, param1, param2, p, dresult, dscratch, true, as_stream(stream));
 }
 
 extern "C" int och_reduce_all(int op, int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,

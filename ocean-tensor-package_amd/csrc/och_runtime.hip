@@ -169,7 +169,9 @@ int och_device_warmup(int device)
    OCH_CHECK_LAUNCH();
    OCH_CHECK_HIP(hipDeviceSynchronize());
    och::StreamContext *ctx;
-   const int status = och::stream_context(nullptr, &ctx);        /* scratch of the default stream */
+   int status = och::stream_context(nullptr, &ctx);              /* scratch of the default stream */
+   char *fixed;
+   if (status == 0) status = och::reduce_static_scratch(&fixed); /* this device's address of the scratch that needs no allocation */
    OCH_CHECK_HIP(hipSetDevice(prev));
    return status;
 }

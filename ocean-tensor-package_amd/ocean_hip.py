@@ -186,6 +186,8 @@ PROTOTYPES = {
     "och_reduce_result_dtype": (_i, [_i, _i]),
     "och_reduce_all": (_i, [_i, _i, _i, _sz, _st, _vp, C.POINTER(Scalar), C.POINTER(Scalar), C.c_double, _vp, _vp, _vp]),
     "och_reduce_all_device": (_i, [_i, _i, _i, _sz, _st, _vp, C.POINTER(Scalar), C.POINTER(Scalar), C.c_double, _vp, _vp, _vp]),
+    "och_reduce_all_device_noalloc": (_i, [_i, _i, _i, _sz, _st, _vp, C.POINTER(Scalar), C.POINTER(Scalar), C.c_double, _vp, _vp]),
+    "och_reduce_all_noalloc_max_elements": (C.c_size_t, []),
     "och_reduce_axis": (_i, [_i, _i, C.POINTER(ReduceAxisConfig), C.c_double]),
     "och_gemm": (_i, [_i, C.c_char, C.c_char, C.c_size_t, C.c_size_t, C.c_size_t, _vp, _vp, C.c_ssize_t, _vp, C.c_ssize_t,
                       _vp, _vp, C.c_ssize_t, _i, _vp]),
