@@ -57,6 +57,8 @@ template <int NOPS> struct EwParams
    int      ndims;
    int      vecmode[NOPS];
    int      nt;                            /* streaming launch: wide accesses carry the nontemporal hint */
+   uint32_t unr;                           /* groups per thread of this launch (at most the kernel's UNR) */
+   uint32_t block;                         /* threads per workgroup of this launch */
 };
 
 template <class T, int VEC> struct alignas((sizeof(T) * VEC) > 16 ? 16 : (sizeof(T) * VEC)) Pack { T v[VEC]; };
@@ -98,10 +100,37 @@ OCH_D void store_wide(const Pack<T, VEC> &p, char *addr)
    else    *reinterpret_cast<V *>(addr) = raw;
 }
 
+/* Source elements one apart (a step-2 slice along the first dimension): the 2 VEC consecutive elements that hold the
+   group are read with one or two <=128-bit loads and every second one is kept. The element behind the last one kept
+   lies in the same aligned 16-byte unit as an element of the tensor, so no load leaves such a unit. Measured on MI355X
+   for int16 (step 2) -> float32: 4.8 TB/s of the bytes asked for against 4.6 with one 2-byte load per element (the
+   memory system moves the skipped elements either way: 8 bytes of traffic for 6 bytes asked for). */
+template <class T, int VEC, bool NT = false>
+OCH_D void load_even(Pack<T, VEC> &p, const char *addr)
+{
+   constexpr int SPAN = 2 * VEC * (int)sizeof(T);
+   constexpr int W = SPAN > 16 ? 16 : SPAN, NL = SPAN / W;
+   typedef typename RawVec<W>::type V;
+   V raw[NL];
+#pragma unroll
+   for (int l = 0; l < NL; l++)
+   {  if constexpr (NT) raw[l] = __builtin_nontemporal_load(reinterpret_cast<const V *>(addr) + l);
+      else    raw[l] = reinterpret_cast<const V *>(addr)[l];
+   }
+   T e[2 * VEC];
+   __builtin_memcpy(e, raw, SPAN);
+#pragma unroll
+   for (int k = 0; k < VEC; k++) p.v[k] = e[2 * k];
+}
+template <class T, int VEC> constexpr bool even_loads_pay() { return VEC > 1 && sizeof(T) <= 4; }
+
+/* vec: 1 = one wide access, 2 = every second of 2 VEC consecutive elements (inputs only), 0 = element accesses */
 template <class T, int VEC, bool NT = false>
 OCH_D void load_pack(Pack<T, VEC> &p, const char *addr, int64_t estride, int vec)
 {
-   if (vec) load_wide<T, VEC, NT>(p, addr);
+   if (vec == 1) load_wide<T, VEC, NT>(p, addr);
+   else if (even_loads_pay<T, VEC>() && vec == 2)
+   {  if constexpr (even_loads_pay<T, VEC>()) load_even<T, VEC, NT>(p, addr); }
    else if (estride == 0)
    {  /* broadcast along the vector: one load serves all elements */
       const T x = *reinterpret_cast<const T *>(addr);
@@ -149,61 +178,80 @@ OCH_D void group_offsets(const EwParams<NOPS> &p, uint32_t g, int64_t (&off)[NOP
    }
 }
 
+/* A wave of these kernels lives for one or two memory round trips, so what it does before its first load counts. Left
+   to itself the compiler fetches every kernel argument where it is first used: four dependent scalar-load round trips
+   before the first global load of the one-dimensional path. Naming the fields that every path needs in an empty asm at
+   the top of the kernel makes it fetch them together, one round trip (float64 <- int32 cast of 2^24 elements on
+   MI355X: 5.97 -> 6.3 TB/s). */
+template <int NOPS>
+OCH_D void ew_fetch_arguments(const EwParams<NOPS> &p)
+{
+#pragma unroll
+   for (int k = 0; k < NOPS; k++) asm volatile("" :: "s"(p.ptr[k]), "s"(p.gstride[k]));
+   asm volatile("" :: "s"(p.ngroups), "s"(p.ndims), "s"(p.unr), "s"(p.block));
+}
+
 #define OCH_EW_BLOCK 256
+/* workgroup size of streaming launches of the all-wide kernels: on MI355X a float64 add of 3 x 134 MB runs at 6.43 TB/s
+   with 512 threads per workgroup and at 6.38 with 256, a float32 -> float64 cast at 6.28 against 6.18 */
+#define OCH_EW_BLOCK_STREAM 512
+#define OCH_EW_MAX_BLOCK 512
 /* launches that move at least this many bytes are treated as streaming (larger than the L2 of all XCDs) */
 #define OCH_EW_STREAM_BYTES (48ull << 20)
 
 /* z = f(x, y) */
 template <class F, int VEC, int UNR, bool FAST, bool NT = false>
-__global__ __launch_bounds__(OCH_EW_BLOCK) void ew3_kernel(const EwParams<3> p)
+__global__ __launch_bounds__(OCH_EW_MAX_BLOCK) void ew3_kernel(const EwParams<3> p)
 {
    typedef typename F::A A; typedef typename F::B B; typedef typename F::R R;
-   const uint32_t base = blockIdx.x * (OCH_EW_BLOCK * UNR) + threadIdx.x;
+   ew_fetch_arguments<3>(p);
+   const uint32_t base = blockIdx.x * (p.block * p.unr) + threadIdx.x;
    Pack<A, VEC> a[UNR]; Pack<B, VEC> b[UNR]; int64_t off[UNR][3];
 #pragma unroll
    for (int u = 0; u < UNR; u++)
-   {  uint32_t g = base + u * OCH_EW_BLOCK;
-      if (g < p.ngroups)
+   {  uint32_t g = base + u * p.block;
+      if ((uint32_t)u < p.unr && g < p.ngroups)
       {  group_offsets<3>(p, g, off[u]);
-         load_pack<A, VEC, NT>(a[u], p.ptr[0] + off[u][0], p.estride[0], FAST || p.vecmode[0]);
-         load_pack<B, VEC, NT>(b[u], p.ptr[1] + off[u][1], p.estride[1], FAST || p.vecmode[1]);
+         load_pack<A, VEC, NT>(a[u], p.ptr[0] + off[u][0], p.estride[0], FAST ? 1 : p.vecmode[0]);
+         load_pack<B, VEC, NT>(b[u], p.ptr[1] + off[u][1], p.estride[1], FAST ? 1 : p.vecmode[1]);
       }
    }
 #pragma unroll
    for (int u = 0; u < UNR; u++)
-   {  uint32_t g = base + u * OCH_EW_BLOCK;
-      if (g < p.ngroups)
+   {  uint32_t g = base + u * p.block;
+      if ((uint32_t)u < p.unr && g < p.ngroups)
       {  Pack<R, VEC> r;
 #pragma unroll
          for (int k = 0; k < VEC; k++) r.v[k] = F::f(a[u].v[k], b[u].v[k]);
-         store_pack<R, VEC, NT>(r, p.ptr[2] + off[u][2], p.estride[2], FAST || p.vecmode[2]);
+         store_pack<R, VEC, NT>(r, p.ptr[2] + off[u][2], p.estride[2], FAST ? 1 : p.vecmode[2]);
       }
    }
 }
 
 /* y = f(x) */
 template <class F, int VEC, int UNR, bool FAST, bool NT = false>
-__global__ __launch_bounds__(OCH_EW_BLOCK) void ew2_kernel(const EwParams<2> p)
+__global__ __launch_bounds__(OCH_EW_MAX_BLOCK) void ew2_kernel(const EwParams<2> p)
 {
    typedef typename F::A A; typedef typename F::R R;
-   const uint32_t base = blockIdx.x * (OCH_EW_BLOCK * UNR) + threadIdx.x;
+   ew_fetch_arguments<2>(p);
+   const uint32_t base = blockIdx.x * (p.block * p.unr) + threadIdx.x;
    Pack<A, VEC> a[UNR]; int64_t off[UNR][2];
 #pragma unroll
    for (int u = 0; u < UNR; u++)
-   {  uint32_t g = base + u * OCH_EW_BLOCK;
-      if (g < p.ngroups)
+   {  uint32_t g = base + u * p.block;
+      if ((uint32_t)u < p.unr && g < p.ngroups)
       {  group_offsets<2>(p, g, off[u]);
-         load_pack<A, VEC, NT>(a[u], p.ptr[0] + off[u][0], p.estride[0], FAST || p.vecmode[0]);
+         load_pack<A, VEC, NT>(a[u], p.ptr[0] + off[u][0], p.estride[0], FAST ? 1 : p.vecmode[0]);
       }
    }
 #pragma unroll
    for (int u = 0; u < UNR; u++)
-   {  uint32_t g = base + u * OCH_EW_BLOCK;
-      if (g < p.ngroups)
+   {  uint32_t g = base + u * p.block;
+      if ((uint32_t)u < p.unr && g < p.ngroups)
       {  Pack<R, VEC> r;
 #pragma unroll
          for (int k = 0; k < VEC; k++) r.v[k] = F::f(a[u].v[k]);
-         store_pack<R, VEC, NT>(r, p.ptr[1] + off[u][1], p.estride[1], FAST || p.vecmode[1]);
+         store_pack<R, VEC, NT>(r, p.ptr[1] + off[u][1], p.estride[1], FAST ? 1 : p.vecmode[1]);
       }
    }
 }
@@ -212,21 +260,22 @@ __global__ __launch_bounds__(OCH_EW_BLOCK) void ew2_kernel(const EwParams<2> p)
    old value is read. The flat index counts elements in the order of the NORMALISED
    dimensions, so index-dependent functors are launched without reordering. */
 template <class F, int VEC, int UNR, bool FAST, bool NT = false>
-__global__ __launch_bounds__(OCH_EW_BLOCK) void ew1_kernel(const EwParams<1> p, const typename F::Param prm)
+__global__ __launch_bounds__(OCH_EW_MAX_BLOCK) void ew1_kernel(const EwParams<1> p, const typename F::Param prm)
 {
    typedef typename F::R R;
-   const uint32_t base = blockIdx.x * (OCH_EW_BLOCK * UNR) + threadIdx.x;
+   ew_fetch_arguments<1>(p);
+   const uint32_t base = blockIdx.x * (p.block * p.unr) + threadIdx.x;
 #pragma unroll
    for (int u = 0; u < UNR; u++)
-   {  uint32_t g = base + u * OCH_EW_BLOCK;
-      if (g < p.ngroups)
+   {  uint32_t g = base + u * p.block;
+      if ((uint32_t)u < p.unr && g < p.ngroups)
       {  int64_t off[1];
          group_offsets<1>(p, g, off);
          Pack<R, VEC> r;
-         if constexpr (F::RMW) load_pack<R, VEC>(r, p.ptr[0] + off[0], p.estride[0], FAST || p.vecmode[0]);
+         if constexpr (F::RMW) load_pack<R, VEC>(r, p.ptr[0] + off[0], p.estride[0], FAST ? 1 : p.vecmode[0]);
 #pragma unroll
          for (int k = 0; k < VEC; k++) r.v[k] = F::f(r.v[k], p.group0 + (uint64_t)g * VEC + k, prm);
-         store_pack<R, VEC, NT>(r, p.ptr[0] + off[0], p.estride[0], FAST || p.vecmode[0]);
+         store_pack<R, VEC, NT>(r, p.ptr[0] + off[0], p.estride[0], FAST ? 1 : p.vecmode[0]);
       }
    }
 }
@@ -238,13 +287,15 @@ __global__ __launch_bounds__(OCH_EW_BLOCK) void ew1_kernel(const EwParams<1> p, 
    kernels work on TILE x TILE blocks of (dimension 0, dimension d1): such an input is read
    with 128-bit loads along d1, parked transposed in LDS, and then consumed in output order;
    the other operands are accessed directly along dimension 0. */
-#define OCH_TILE_THREADS 256
+/* threads per tile: a 64 x 64 tile of 8-byte elements takes 33 KB of LDS, so workgroups of 256 threads leave a compute
+   unit with 16 waves; 1024 threads per tile (two 16-byte loads in flight per thread instead of eight) fill it with 32
+   (transposed float64 add, 4096 x 4096, on MI355X: 5.9 -> 6.2 TB/s). The smaller tiles of the other types fit eight times
+   with 256 threads. */
+constexpr int tile_threads(size_t maxsize) { return maxsize == 8 ? 1024 : 256; }
 template <int NOPS> struct TileParams
-{
+{  /* the fields every workgroup reads come first, so that one scalar load brings them in (see tile_fetch_arguments) */
    char    *ptr[NOPS];
    int64_t  s0[NOPS], s1[NOPS];             /* byte strides along dimension 0 and along d1 */
-   int64_t  so[NOPS][OCH_MAX_DIMS];         /* byte strides of the remaining (outer) dimensions */
-   FastDiv  odiv[OCH_MAX_DIMS];
    uint32_t n0, n1;                         /* extents of dimension 0 and d1 */
    int      nouter;
    int      trans[NOPS];                    /* read through LDS */
@@ -252,31 +303,46 @@ template <int NOPS> struct TileParams
    int      lds_off[NOPS];                  /* byte offset of the operand's LDS tile */
    int      nt;                             /* streaming launch: nontemporal hint on global accesses */
    int      diagonal;                       /* walk the tile grid along diagonals (see tile_row) */
+   int64_t  so[NOPS][OCH_MAX_DIMS];         /* byte strides of the remaining (outer) dimensions */
+   FastDiv  odiv[OCH_MAX_DIMS];
 };
+
+/* one scalar-load round trip for the arguments instead of one per first use (see ew_fetch_arguments) */
+template <int NOPS>
+OCH_D void tile_fetch_arguments(const TileParams<NOPS> &p)
+{
+#pragma unroll
+   for (int k = 0; k < NOPS; k++) asm volatile("" :: "s"(p.ptr[k]), "s"(p.s0[k]), "s"(p.s1[k]), "s"(p.trans[k]), "s"(p.vecmode[k]), "s"(p.lds_off[k]));
+   asm volatile("" :: "s"(p.n0), "s"(p.n1), "s"(p.nouter), "s"(p.diagonal));
+}
 
 constexpr int tile_dim(size_t maxsize) { return maxsize >= 16 ? 32 : 64; }
 template <class T> constexpr int tile_pitch(int tile) { return tile + (sizeof(T) >= 4 ? 1 : 4 / (int)sizeof(T)); }
 template <class T> constexpr int tile_bytes(int tile) { return ((tile * tile_pitch<T>(tile) * (int)sizeof(T)) + 15) / 16 * 16; }
 
-template <class T, int TILE, bool NT>
+/* Loads of positions outside an edge tile are not skipped but redirected to a position inside it (and what they
+   bring is never used): without a branch around them the compiler issues all loads of a thread back to back before
+   the first one is waited for. n1 is a multiple of the vector length (the host checks it), n0 >= 1. */
+template <class T, int TILE, bool NT, int THREADS>
 OCH_D void tile_stage(T *lds, const char *base, int64_t s0, uint32_t n0, uint32_t n1)
 {
    constexpr int VK = vec_for_c<T>();
    constexpr int LPR = TILE / VK;                        /* lanes per row (fixed index along dimension 0) */
-   constexpr int RPP = OCH_TILE_THREADS / LPR;           /* rows per pass */
+   constexpr int RPP = THREADS / LPR;                    /* rows per pass */
    constexpr int PASSES = (TILE + RPP - 1) / RPP;
    constexpr int PITCH = tile_pitch<T>(TILE);
    const uint32_t i1 = (threadIdx.x % LPR) * VK, row = threadIdx.x / LPR;
+   const uint32_t i1c = (i1 < n1) ? i1 : 0;
    Pack<T, VK> v[PASSES];
 #pragma unroll
    for (int u = 0; u < PASSES; u++)
-   {  uint32_t i0 = row + u * RPP;
-      if (i0 < n0 && i1 < n1) load_wide<T, VK, NT>(v[u], base + (int64_t)i0 * s0 + (int64_t)i1 * (int64_t)sizeof(T));
+   {  const uint32_t i0 = row + u * RPP, i0c = (i0 < n0) ? i0 : n0 - 1;
+      load_wide<T, VK, NT>(v[u], base + (int64_t)i0c * s0 + (int64_t)i1c * (int64_t)sizeof(T));
    }
 #pragma unroll
    for (int u = 0; u < PASSES; u++)
-   {  uint32_t i0 = row + u * RPP;
-      if (i0 < n0 && i1 < n1)
+   {  const uint32_t i0 = row + u * RPP;
+      if (PASSES * RPP <= TILE || i0 < (uint32_t)TILE)
       {
 #pragma unroll
          for (int j = 0; j < VK; j++) lds[(i1 + j) * PITCH + i0] = v[u].v[j];
@@ -287,18 +353,19 @@ OCH_D void tile_stage(T *lds, const char *base, int64_t s0, uint32_t n0, uint32_
 /* Tile row of a block. Blocks that run together have neighbouring blockIdx.x. When the pitch of the transposed operand
    is a power of two between 16 KB and 64 KB (4096 x 4096 or 8192 x 8192 float64), the straight order makes them all read
    the same 512-byte column of that operand at a pitch of one matrix row, i.e. the same few memory channels; shifting
-   the tile row by the tile column walks the grid along diagonals and spreads both the reads and the writes (measured
-   on MI355X: 6.0 against 4.9 TB/s at 4096 x 4096). For every other pitch the straight order is the faster one by
+   the tile row by (three times) the tile column walks the grid along diagonals and spreads both the reads and the writes
+   (measured on MI355X: 6.2 against 5.6 TB/s at 4096 x 4096; a shift of one tile row per column gives 6.15, square
+   super-tiles of 4 to 32 tiles 5.7 - 5.9). For every other pitch the straight order is the faster one by
    10 - 25 % (5.5 against 4.4 TB/s at 4224 x 4224), so the host chooses per launch. */
-OCH_D uint32_t tile_row(int diagonal) { return diagonal ? (blockIdx.y + blockIdx.x) % gridDim.y : blockIdx.y; }
+OCH_D uint32_t tile_row(int diagonal) { return diagonal ? (blockIdx.y + 3 * blockIdx.x) % gridDim.y : blockIdx.y; }
 
 template <int NOPS>
-OCH_D void tile_origin(const TileParams<NOPS> &p, int tile, int64_t (&off)[NOPS])
+OCH_D void tile_origin(const TileParams<NOPS> &p, int tile, uint32_t trow, int64_t (&off)[NOPS])
 {
    uint32_t q = blockIdx.z;
 #pragma unroll
    for (int k = 0; k < NOPS; k++)
-      off[k] = (int64_t)blockIdx.x * tile * p.s0[k] + (int64_t)tile_row(p.diagonal) * tile * p.s1[k];
+      off[k] = (int64_t)blockIdx.x * tile * p.s0[k] + (int64_t)trow * tile * p.s1[k];
    for (int d = 0; d < p.nouter; d++)
    {  uint32_t q2 = fastdiv(q, p.odiv[d]);
       uint32_t i = q - q2 * p.odiv[d].d; q = q2;
@@ -307,73 +374,88 @@ OCH_D void tile_origin(const TileParams<NOPS> &p, int tile, int64_t (&off)[NOPS]
    }
 }
 
+/* operand k of a tiled kernel in output order: from its LDS tile, or straight from memory (position clamped into the tile) */
+template <class T, int VEC, int TILE, bool NT>
+OCH_D void tile_fetch(Pack<T, VEC> &v, const T *lds, int trans, const char *base, int64_t s0, int64_t s1, int vecmode, uint32_t i0c, uint32_t i1c)
+{
+   if (trans)
+   {
+#pragma unroll
+      for (int k = 0; k < VEC; k++) v.v[k] = lds[i1c * tile_pitch<T>(TILE) + i0c + k];
+   }
+   else load_pack<T, VEC, NT>(v, base + (int64_t)i0c * s0 + (int64_t)i1c * s1, s0, vecmode);
+}
+
+template <class A, class B, class R> constexpr size_t max_size3()
+{  return sizeof(A) > sizeof(B) ? (sizeof(A) > sizeof(R) ? sizeof(A) : sizeof(R)) : (sizeof(B) > sizeof(R) ? sizeof(B) : sizeof(R)); }
+
 template <class F, int VEC, bool NT>
-__global__ __launch_bounds__(OCH_TILE_THREADS) void ew3_tile_kernel(const TileParams<3> p)
+__global__ __launch_bounds__(tile_threads(max_size3<typename F::A, typename F::B, typename F::R>())) void ew3_tile_kernel(const TileParams<3> p)
 {
    typedef typename F::A A; typedef typename F::B B; typedef typename F::R R;
-   constexpr size_t MAXS = sizeof(A) > sizeof(B) ? (sizeof(A) > sizeof(R) ? sizeof(A) : sizeof(R)) : (sizeof(B) > sizeof(R) ? sizeof(B) : sizeof(R));
-   constexpr int TILE = tile_dim(MAXS);
+   constexpr size_t MAXS = max_size3<A, B, R>();
+   constexpr int TILE = tile_dim(MAXS), THREADS = tile_threads(MAXS);
    extern __shared__ __align__(16) char och_tile_lds[];
+   tile_fetch_arguments<3>(p);
    A *la = reinterpret_cast<A *>(och_tile_lds + p.lds_off[0]);
    B *lb = reinterpret_cast<B *>(och_tile_lds + p.lds_off[1]);
    int64_t off[3];
-   tile_origin<3>(p, TILE, off);
-   const uint32_t r0 = p.n0 - blockIdx.x * TILE, r1 = p.n1 - tile_row(p.diagonal) * TILE;
+   const uint32_t trow = tile_row(p.diagonal);
+   tile_origin<3>(p, TILE, trow, off);
+   const uint32_t r0 = p.n0 - blockIdx.x * TILE, r1 = p.n1 - trow * TILE;
    const uint32_t n0 = r0 < (uint32_t)TILE ? r0 : TILE, n1 = r1 < (uint32_t)TILE ? r1 : TILE;
-   if (p.trans[0]) tile_stage<A, TILE, NT>(la, p.ptr[0] + off[0], p.s0[0], n0, n1);
-   if (p.trans[1]) tile_stage<B, TILE, NT>(lb, p.ptr[1] + off[1], p.s0[1], n0, n1);
+   if (p.trans[0]) tile_stage<A, TILE, NT, THREADS>(la, p.ptr[0] + off[0], p.s0[0], n0, n1);
+   if (p.trans[1]) tile_stage<B, TILE, NT, THREADS>(lb, p.ptr[1] + off[1], p.s0[1], n0, n1);
    __syncthreads();
-   constexpr int LPC = TILE / VEC, CPP = OCH_TILE_THREADS / LPC, PASSES = (TILE + CPP - 1) / CPP;
+   constexpr int LPC = TILE / VEC, CPP = THREADS / LPC, PASSES = (TILE + CPP - 1) / CPP;
    const uint32_t i0 = (threadIdx.x % LPC) * VEC, col = threadIdx.x / LPC;
+   const uint32_t i0c = (i0 < n0) ? i0 : 0;                  /* n0 is a multiple of VEC */
+   Pack<A, VEC> a[PASSES]; Pack<B, VEC> b[PASSES];
 #pragma unroll
    for (int u = 0; u < PASSES; u++)
-   {  uint32_t i1 = col + u * CPP;
+   {  const uint32_t i1 = col + u * CPP, i1c = (i1 < n1) ? i1 : n1 - 1;
+      tile_fetch<A, VEC, TILE, NT>(a[u], la, p.trans[0], p.ptr[0] + off[0], p.s0[0], p.s1[0], p.vecmode[0], i0c, i1c);
+      tile_fetch<B, VEC, TILE, NT>(b[u], lb, p.trans[1], p.ptr[1] + off[1], p.s0[1], p.s1[1], p.vecmode[1], i0c, i1c);
+   }
+#pragma unroll
+   for (int u = 0; u < PASSES; u++)
+   {  const uint32_t i1 = col + u * CPP;
       if (i0 < n0 && i1 < n1)
-      {  Pack<A, VEC> a; Pack<B, VEC> b; Pack<R, VEC> r;
-         if (p.trans[0])
-         {
+      {  Pack<R, VEC> r;
 #pragma unroll
-            for (int k = 0; k < VEC; k++) a.v[k] = la[i1 * tile_pitch<A>(TILE) + i0 + k];
-         }
-         else load_pack<A, VEC, NT>(a, p.ptr[0] + off[0] + (int64_t)i0 * p.s0[0] + (int64_t)i1 * p.s1[0], p.s0[0], p.vecmode[0]);
-         if (p.trans[1])
-         {
-#pragma unroll
-            for (int k = 0; k < VEC; k++) b.v[k] = lb[i1 * tile_pitch<B>(TILE) + i0 + k];
-         }
-         else load_pack<B, VEC, NT>(b, p.ptr[1] + off[1] + (int64_t)i0 * p.s0[1] + (int64_t)i1 * p.s1[1], p.s0[1], p.vecmode[1]);
-#pragma unroll
-         for (int k = 0; k < VEC; k++) r.v[k] = F::f(a.v[k], b.v[k]);
+         for (int k = 0; k < VEC; k++) r.v[k] = F::f(a[u].v[k], b[u].v[k]);
          store_pack<R, VEC, NT>(r, p.ptr[2] + off[2] + (int64_t)i0 * p.s0[2] + (int64_t)i1 * p.s1[2], p.s0[2], p.vecmode[2]);
       }
    }
 }
 
 template <class F, int VEC, bool NT>
-__global__ __launch_bounds__(OCH_TILE_THREADS) void ew2_tile_kernel(const TileParams<2> p)
+__global__ __launch_bounds__(tile_threads(max_size3<typename F::A, typename F::A, typename F::R>())) void ew2_tile_kernel(const TileParams<2> p)
 {
    typedef typename F::A A; typedef typename F::R R;
    constexpr size_t MAXS = sizeof(A) > sizeof(R) ? sizeof(A) : sizeof(R);
-   constexpr int TILE = tile_dim(MAXS);
+   constexpr int TILE = tile_dim(MAXS), THREADS = tile_threads(MAXS);
    extern __shared__ __align__(16) char och_tile_lds[];
+   tile_fetch_arguments<2>(p);
    A *la = reinterpret_cast<A *>(och_tile_lds);
    int64_t off[2];
-   tile_origin<2>(p, TILE, off);
-   const uint32_t r0 = p.n0 - blockIdx.x * TILE, r1 = p.n1 - tile_row(p.diagonal) * TILE;
+   const uint32_t trow = tile_row(p.diagonal);
+   tile_origin<2>(p, TILE, trow, off);
+   const uint32_t r0 = p.n0 - blockIdx.x * TILE, r1 = p.n1 - trow * TILE;
    const uint32_t n0 = r0 < (uint32_t)TILE ? r0 : TILE, n1 = r1 < (uint32_t)TILE ? r1 : TILE;
-   tile_stage<A, TILE, NT>(la, p.ptr[0] + off[0], p.s0[0], n0, n1);
+   tile_stage<A, TILE, NT, THREADS>(la, p.ptr[0] + off[0], p.s0[0], n0, n1);
    __syncthreads();
-   constexpr int LPC = TILE / VEC, CPP = OCH_TILE_THREADS / LPC, PASSES = (TILE + CPP - 1) / CPP;
+   constexpr int LPC = TILE / VEC, CPP = THREADS / LPC, PASSES = (TILE + CPP - 1) / CPP;
    const uint32_t i0 = (threadIdx.x % LPC) * VEC, col = threadIdx.x / LPC;
+   const uint32_t i0c = (i0 < n0) ? i0 : 0;
 #pragma unroll
    for (int u = 0; u < PASSES; u++)
-   {  uint32_t i1 = col + u * CPP;
-      if (i0 < n0 && i1 < n1)
-      {  Pack<R, VEC> r;
+   {  const uint32_t i1 = col + u * CPP, i1c = (i1 < n1) ? i1 : n1 - 1;
+      Pack<R, VEC> r;
 #pragma unroll
-         for (int k = 0; k < VEC; k++) r.v[k] = F::f(la[i1 * tile_pitch<A>(TILE) + i0 + k]);
+      for (int k = 0; k < VEC; k++) r.v[k] = F::f(la[i1c * tile_pitch<A>(TILE) + i0c + k]);
+      if (i0 < n0 && i1 < n1)
          store_pack<R, VEC, NT>(r, p.ptr[1] + off[1] + (int64_t)i0 * p.s0[1] + (int64_t)i1 * p.s1[1], p.s0[1], p.vecmode[1]);
-      }
    }
 }
 
@@ -481,11 +563,14 @@ static int ew_launch_chunked(EwShape<NOPS> s, uint64_t flat0, L &&launch)
 }
 
 /* Fill kernel parameters for a VEC-wide launch; returns false when VEC does not fit */
+/* even_inputs: the first `even_inputs` operands are inputs whose kernel can read a step-2 first dimension with wide
+   loads (vecmode 2, see load_even) */
 template <int NOPS>
-static bool ew_params(EwParams<NOPS> &p, const EwShape<NOPS> &s, int vec, const int elemsize[NOPS], uint64_t flat0)
+static bool ew_params(EwParams<NOPS> &p, const EwShape<NOPS> &s, int vec, const int elemsize[NOPS], uint64_t flat0, int even_inputs = 0)
 {
    if (s.size[0] % vec != 0) return false;
    p.ndims = s.ndims;
+   p.unr = 1; p.block = OCH_EW_BLOCK;
    p.ngroups = (uint32_t)(s.nelem / vec);
    p.group0 = flat0;
    {  uint64_t bytes = 0;
@@ -503,6 +588,12 @@ static bool ew_params(EwParams<NOPS> &p, const EwShape<NOPS> &s, int vec, const 
       bool v = (s.stride[k][0] == elemsize[k]) && (((uintptr_t)s.ptr[k]) % width == 0);
       for (int d = 1; d < s.ndims && v; d++) if (s.stride[k][d] % width != 0) v = false;
       p.vecmode[k] = v ? 1 : 0;
+      if (!v && k < even_inputs && vec > 1 && elemsize[k] <= 4 && s.stride[k][0] == 2 * elemsize[k])
+      {  int span = 2 * elemsize[k] * vec; if (span > 16) span = 16;
+         bool e = (((uintptr_t)s.ptr[k]) % span == 0);
+         for (int d = 1; d < s.ndims && e; d++) if (s.stride[k][d] % span != 0) e = false;
+         if (e) p.vecmode[k] = 2;
+      }
    }
    return true;
 }
@@ -520,17 +611,27 @@ template <class A, class B, class C> constexpr int vec_for3()
      wide  : every operand has aligned unit stride along dim 0 -> VEC-wide accesses only
      mixed : dim 0 divisible by VEC, some operands strided or broadcast
      single: one element per thread (odd sizes); for 1-D shapes only the tail uses it   */
+/* Launcher signature: (parameters, workgroups, threads per workgroup) */
 template <int NOPS, class LW, class LM, class LS>
 static int ew_dispatch(const EwShape<NOPS> &s, uint64_t flat0, int vec, const int (&es)[NOPS],
                        LW &&wide, LM &&mixed, LS &&single)
 {
    EwParams<NOPS> p;
    auto run = [&](const EwShape<NOPS> &sh, uint64_t f0) -> bool
-   {  if (!ew_params<NOPS>(p, sh, vec, es, f0)) return false;      /* vec = 1 (16-byte elements) always fits */
+   {  if (!ew_params<NOPS>(p, sh, vec, es, f0, NOPS - 1)) return false;      /* vec = 1 (16-byte elements) always fits */
       bool all = true;
-      for (int k = 0; k < NOPS; k++) all = all && p.vecmode[k];
-      if (all) wide(p, (p.ngroups + OCH_EW_BLOCK * OCH_EW_UNR - 1) / (OCH_EW_BLOCK * OCH_EW_UNR));
-      else     mixed(p, (p.ngroups + OCH_EW_BLOCK * 2 - 1) / (OCH_EW_BLOCK * 2));
+      for (int k = 0; k < NOPS; k++) all = all && (p.vecmode[k] == 1);
+      const uint32_t block = p.nt ? OCH_EW_BLOCK_STREAM : OCH_EW_BLOCK;
+      p.block = block;
+      if (all) wide(p, (p.ngroups + block * OCH_EW_UNR - 1) / (block * OCH_EW_UNR), block);
+      else
+      {  /* operands with element accesses want two groups in flight per thread; when every operand is read or written
+            in wide accesses (or is a broadcast) one group per thread and the larger workgroup stream faster */
+         bool elementwise = false;
+         for (int k = 0; k < NOPS; k++) if (p.vecmode[k] == 0 && p.estride[k] != 0) elementwise = true;
+         if (elementwise) { p.unr = 2; p.block = OCH_EW_BLOCK; mixed(p, (p.ngroups + OCH_EW_BLOCK * 2 - 1) / (OCH_EW_BLOCK * 2), (uint32_t)OCH_EW_BLOCK); }
+         else             { p.unr = 1; mixed(p, (p.ngroups + block - 1) / block, block); }
+      }
       return true;
    };
    if (!run(s, flat0))
@@ -541,11 +642,11 @@ static int ew_dispatch(const EwShape<NOPS> &s, uint64_t flat0, int vec, const in
          for (int k = 0; k < NOPS; k++) tail.ptr[k] = s.ptr[k] + (int64_t)body.size[0] * s.stride[k][0];
          run(body, flat0);
          ew_params<NOPS>(p, tail, 1, es, flat0 + body.nelem);
-         single(p, 1u);
+         single(p, 1u, (uint32_t)OCH_EW_BLOCK);
       }
       else
       {  ew_params<NOPS>(p, s, 1, es, flat0);
-         single(p, (p.ngroups + OCH_EW_BLOCK - 1) / OCH_EW_BLOCK);
+         single(p, (p.ngroups + OCH_EW_BLOCK - 1) / OCH_EW_BLOCK, (uint32_t)OCH_EW_BLOCK);
       }
    }
    OCH_CHECK_LAUNCH();
@@ -628,21 +729,21 @@ static int launch_ew3(int ndims, const size_t *size,
       const int tb[3] = { tile_bytes<A>(TILE), tile_bytes<B>(TILE), 0 };
       TileParams<3> tp; dim3 grid; size_t lds;
       if (ew_tile_params<3>(tp, s, es, TILE, VEC, grid, lds, tb))
-      {  if (tp.nt) hipLaunchKernelGGL((ew3_tile_kernel<F, VEC, true>), grid, dim3(OCH_TILE_THREADS), lds, stream, tp);
-         else       hipLaunchKernelGGL((ew3_tile_kernel<F, VEC, false>), grid, dim3(OCH_TILE_THREADS), lds, stream, tp);
+      {  if (tp.nt) hipLaunchKernelGGL((ew3_tile_kernel<F, VEC, true>), grid, dim3(tile_threads(MAXS)), lds, stream, tp);
+         else       hipLaunchKernelGGL((ew3_tile_kernel<F, VEC, false>), grid, dim3(tile_threads(MAXS)), lds, stream, tp);
          OCH_CHECK_LAUNCH();
          return 0;
       }
       return ew_dispatch<3>(s, flat0, VEC, es,
-         [&](const EwParams<3> &p, uint32_t blocks)
-         {  if (p.nt) hipLaunchKernelGGL((ew3_kernel<F, VEC, OCH_EW_UNR, true, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p);
-            else      hipLaunchKernelGGL((ew3_kernel<F, VEC, OCH_EW_UNR, true, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
-         [&](const EwParams<3> &p, uint32_t blocks)
+         [&](const EwParams<3> &p, uint32_t blocks, uint32_t threads)
+         {  if (p.nt) hipLaunchKernelGGL((ew3_kernel<F, VEC, OCH_EW_UNR, true, true>), dim3(blocks), dim3(threads), 0, stream, p);
+            else      hipLaunchKernelGGL((ew3_kernel<F, VEC, OCH_EW_UNR, true, false>), dim3(blocks), dim3(threads), 0, stream, p); },
+         [&](const EwParams<3> &p, uint32_t blocks, uint32_t threads)
          {  /* nontemporal accesses reach only the operands that take the wide path; a broadcast operand keeps its cached loads */
-            if (p.nt) hipLaunchKernelGGL((ew3_kernel<F, VEC, 2, false, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p);
-            else      hipLaunchKernelGGL((ew3_kernel<F, VEC, 2, false, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
-         [&](const EwParams<3> &p, uint32_t blocks)
-         {  hipLaunchKernelGGL((ew3_kernel<F, 1, 1, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); });
+            if (p.nt) hipLaunchKernelGGL((ew3_kernel<F, VEC, 2, false, true>), dim3(blocks), dim3(threads), 0, stream, p);
+            else      hipLaunchKernelGGL((ew3_kernel<F, VEC, 2, false, false>), dim3(blocks), dim3(threads), 0, stream, p); },
+         [&](const EwParams<3> &p, uint32_t blocks, uint32_t threads)
+         {  hipLaunchKernelGGL((ew3_kernel<F, 1, 1, false>), dim3(blocks), dim3(threads), 0, stream, p); });
    });
 }
 
@@ -662,20 +763,20 @@ static int launch_ew2(int ndims, const size_t *size,
       const int tb[2] = { tile_bytes<A>(TILE), 0 };
       TileParams<2> tp; dim3 grid; size_t lds;
       if (ew_tile_params<2>(tp, s, es, TILE, VEC, grid, lds, tb))
-      {  if (tp.nt) hipLaunchKernelGGL((ew2_tile_kernel<F, VEC, true>), grid, dim3(OCH_TILE_THREADS), lds, stream, tp);
-         else       hipLaunchKernelGGL((ew2_tile_kernel<F, VEC, false>), grid, dim3(OCH_TILE_THREADS), lds, stream, tp);
+      {  if (tp.nt) hipLaunchKernelGGL((ew2_tile_kernel<F, VEC, true>), grid, dim3(tile_threads(MAXS)), lds, stream, tp);
+         else       hipLaunchKernelGGL((ew2_tile_kernel<F, VEC, false>), grid, dim3(tile_threads(MAXS)), lds, stream, tp);
          OCH_CHECK_LAUNCH();
          return 0;
       }
       return ew_dispatch<2>(s, flat0, VEC, es,
-         [&](const EwParams<2> &p, uint32_t blocks)
-         {  if (p.nt) hipLaunchKernelGGL((ew2_kernel<F, VEC, OCH_EW_UNR, true, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p);
-            else      hipLaunchKernelGGL((ew2_kernel<F, VEC, OCH_EW_UNR, true, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
-         [&](const EwParams<2> &p, uint32_t blocks)
-         {  if (p.nt) hipLaunchKernelGGL((ew2_kernel<F, VEC, 2, false, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p);
-            else      hipLaunchKernelGGL((ew2_kernel<F, VEC, 2, false, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); },
-         [&](const EwParams<2> &p, uint32_t blocks)
-         {  hipLaunchKernelGGL((ew2_kernel<F, 1, 1, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p); });
+         [&](const EwParams<2> &p, uint32_t blocks, uint32_t threads)
+         {  if (p.nt) hipLaunchKernelGGL((ew2_kernel<F, VEC, OCH_EW_UNR, true, true>), dim3(blocks), dim3(threads), 0, stream, p);
+            else      hipLaunchKernelGGL((ew2_kernel<F, VEC, OCH_EW_UNR, true, false>), dim3(blocks), dim3(threads), 0, stream, p); },
+         [&](const EwParams<2> &p, uint32_t blocks, uint32_t threads)
+         {  if (p.nt) hipLaunchKernelGGL((ew2_kernel<F, VEC, 2, false, true>), dim3(blocks), dim3(threads), 0, stream, p);
+            else      hipLaunchKernelGGL((ew2_kernel<F, VEC, 2, false, false>), dim3(blocks), dim3(threads), 0, stream, p); },
+         [&](const EwParams<2> &p, uint32_t blocks, uint32_t threads)
+         {  hipLaunchKernelGGL((ew2_kernel<F, 1, 1, false>), dim3(blocks), dim3(threads), 0, stream, p); });
    });
 }
 
@@ -692,13 +793,13 @@ static int launch_ew1(int ndims, const size_t *size, const ptrdiff_t *st, void *
    const int es[1] = { (int)sizeof(R) };
    return ew_launch_chunked<1>(shape, 0, [&](const EwShape<1> &s, uint64_t flat0) -> int
    {  return ew_dispatch<1>(s, flat0, VEC, es,
-         [&](const EwParams<1> &p, uint32_t blocks)
-         {  if (p.nt) hipLaunchKernelGGL((ew1_kernel<F, VEC, OCH_EW_UNR, true, true>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p, prm);
-            else      hipLaunchKernelGGL((ew1_kernel<F, VEC, OCH_EW_UNR, true, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p, prm); },
-         [&](const EwParams<1> &p, uint32_t blocks)
-         {  hipLaunchKernelGGL((ew1_kernel<F, VEC, 2, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p, prm); },
-         [&](const EwParams<1> &p, uint32_t blocks)
-         {  hipLaunchKernelGGL((ew1_kernel<F, 1, 1, false>), dim3(blocks), dim3(OCH_EW_BLOCK), 0, stream, p, prm); });
+         [&](const EwParams<1> &p, uint32_t blocks, uint32_t threads)
+         {  if (p.nt) hipLaunchKernelGGL((ew1_kernel<F, VEC, OCH_EW_UNR, true, true>), dim3(blocks), dim3(threads), 0, stream, p, prm);
+            else      hipLaunchKernelGGL((ew1_kernel<F, VEC, OCH_EW_UNR, true, false>), dim3(blocks), dim3(threads), 0, stream, p, prm); },
+         [&](const EwParams<1> &p, uint32_t blocks, uint32_t threads)
+         {  hipLaunchKernelGGL((ew1_kernel<F, VEC, 2, false>), dim3(blocks), dim3(threads), 0, stream, p, prm); },
+         [&](const EwParams<1> &p, uint32_t blocks, uint32_t threads)
+         {  hipLaunchKernelGGL((ew1_kernel<F, 1, 1, false>), dim3(blocks), dim3(threads), 0, stream, p, prm); });
    });
 }
 

@@ -40,7 +40,7 @@ static int analyze(const int *elemsize, int ndims, const size_t *size, const ptr
       if (tiled) { kernel = OCH_KERNEL_TILED; v = vec; }
       else if (ew_params<NOPS>(p, s, vec, es, flat0))
       {  bool all = true;
-         for (int k = 0; k < NOPS; k++) all = all && p.vecmode[k];
+         for (int k = 0; k < NOPS; k++) all = all && (p.vecmode[k] == 1);
          kernel = all ? OCH_KERNEL_WIDE : OCH_KERNEL_MIXED; v = vec;
       }
       else if (vec > 1 && s.ndims == 1 && s.size[0] > (uint64_t)vec)
@@ -48,7 +48,7 @@ static int analyze(const int *elemsize, int ndims, const size_t *size, const ptr
          body.size[0] = s.size[0] - s.size[0] % vec; body.nelem = body.size[0];
          ew_params<NOPS>(p, body, vec, es, flat0);
          bool all = true;
-         for (int k = 0; k < NOPS; k++) all = all && p.vecmode[k];
+         for (int k = 0; k < NOPS; k++) all = all && (p.vecmode[k] == 1);
          kernel = all ? OCH_KERNEL_WIDE : OCH_KERNEL_MIXED; v = vec; n = 2;      /* body + tail */
       }
       else ew_params<NOPS>(p, s, 1, es, flat0);

@@ -247,7 +247,7 @@ static int launch_reduce_all(int ndims, const size_t *size, const ptrdiff_t *str
       }
       else
       {  /* several dimensions: 128-bit loads along the first one when it is contiguous, divisible and aligned */
-         wide_launch = (VEC > 1) && ew_params<1>(p.ew, shape, VEC, es, 0) && p.ew.vecmode[0];
+         wide_launch = (VEC > 1) && ew_params<1>(p.ew, shape, VEC, es, 0) && p.ew.vecmode[0] == 1;
          if (!wide_launch) ew_params<1>(p.ew, shape, 1, es, 0);
          p.ngroups = p.ew.ngroups;
       }

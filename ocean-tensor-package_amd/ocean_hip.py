@@ -204,6 +204,7 @@ PROTOTYPES = {
     "och_find_count": (_i, [_i, _sz, _st, _vp, _vp, C.POINTER(C.c_size_t), _vp]),
     "och_find_apply": (_i, [_i, _sz, _st, _vp, _vp, C.POINTER(C.c_int64), _vp, _vp]),
     "och_elemwise_analyze": (_i, [_i, C.POINTER(_i), _i, _sz, C.POINTER(_st), C.POINTER(_vp), C.c_void_p]),
+    "och_membench": (_i, [_i, _i, _i, _i, _i, _i, C.c_size_t, _i, _i, C.POINTER(C.c_float), C.POINTER(C.c_float), C.POINTER(C.c_size_t), _vp]),
 }
 
 

@@ -80,6 +80,8 @@ int oracle_reduce_supported(int op, int dtype);
 int oracle_reduce_result_dtype(int op, int dtype);
 /* Axis reduction; configuration as och_reduce_axis_config (stream ignored). Serial. */
 int oracle_reduce_axis(int op, int dtype, const och_reduce_axis_config *config, double p);
+/* The same with the outputs split over threads as the CPU module does for many outputs (same bits as the serial form). */
+int oracle_reduce_axis_threads(int op, int dtype, const och_reduce_axis_config *config, double p, int nthreads);
 
 /* Column-major GEMM, textbook triple loop; accumulation in the element type. */
 int oracle_gemm(int dtype, char transA, char transB, size_t M, size_t N, size_t K,

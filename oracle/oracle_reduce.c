@@ -136,3 +136,42 @@ int oracle_reduce_axis(int op, int dtype, const och_reduce_axis_config *c, doubl
    }
    return 0;
 }
+
+/* The same axis reduction with the CPU module's multi-thread split for many outputs (reduce_axis.h:65-104, 300-400,
+   variant "omp1"): the outputs are dealt to the threads in contiguous ranges of the flat output index and every
+   thread reduces its outputs on its own, so the result equals the serial one bit for bit. Fewer than 4 outputs per
+   thread, or 256 operations or fewer, run serially here (the reference's cooperative variant "omp2" reorders the
+   additions of one output; it is not restated). */
+int oracle_reduce_axis_threads(int op, int dtype, const och_reduce_axis_config *c, double p, int nthreads)
+{
+   const o_red_desc *d;
+   o_red_param prm;
+   size_t nout, relem;
+   const ptrdiff_t *st[2] = { c->strides1, c->strides2 };
+   void *pp[2] = { c->ptr1, c->ptr2 };
+   if (!oracle_reduce_supported(op, dtype)) return -1;
+   nout = o_nelem(c->ndims, c->size);
+   relem = o_nelem(c->rdims, c->rsize);
+   if (nthreads <= 1 || nout * relem <= 256 || nout < 4 * (size_t)nthreads) return oracle_reduce_axis(op, dtype, c, p);
+   d = o_red_table[op][dtype];
+   memset(&prm, 0, sizeof(prm));
+   prm.p = p;
+   #pragma omp parallel num_threads(nthreads)
+   {  size_t a, b, i; int rank = 0, nt = 1;
+      o_iter it;
+#ifdef _OPENMP
+      rank = omp_get_thread_num(); nt = omp_get_num_threads();
+#endif
+      o_thread_range(nout, rank, nt, &a, &b);
+      if (a < b)
+      {  o_iter_init(&it, 2, c->ndims, c->size, st, pp, a);
+         for (i = a; i < b; i++)
+         {  char acc[32];
+            d->accumulate(c->rdims, c->rsize, c->rstrides, it.p[0], 0, relem, &prm, acc);
+            d->finalize(acc, &prm, it.p[1]);
+            o_iter_carry(&it, 1);
+         }
+      }
+   }
+   return 0;
+}

@@ -48,6 +48,7 @@ def setup(oh):
         ("oracle_reduce_supported", _i, [_i, _i]),
         ("oracle_reduce_result_dtype", _i, [_i, _i]),
         ("oracle_reduce_axis", _i, [_i, _i, C.POINTER(oh.ReduceAxisConfig), C.c_double]),
+        ("oracle_reduce_axis_threads", _i, [_i, _i, C.POINTER(oh.ReduceAxisConfig), C.c_double, _i]),
         ("oracle_gemm", _i, [_i, C.c_char, C.c_char, C.c_size_t, C.c_size_t, C.c_size_t, _vp, _vp, C.c_ssize_t, _vp,
                             C.c_ssize_t, _vp, _vp, C.c_ssize_t, _i]),
         ("oracle_add_if_negative", _i, [_i, _i, _sz, _st, _vp, S]),
