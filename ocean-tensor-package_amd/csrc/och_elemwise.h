@@ -143,6 +143,25 @@ OCH_D void load_pack(Pack<T, VEC> &p, const char *addr, int64_t estride, int vec
       for (int k = 0; k < VEC; k++) p.v[k] = *reinterpret_cast<const T *>(addr + k * estride);
    }
 }
+/* load_pack in two steps for kernels that issue their loads long before they use them: a broadcast along the vector is
+   one load into the first element, and copying it to the others -- which has to wait for the load, and with it for
+   every load issued before -- is left to load_pack_finish at the point of use */
+template <class T, int VEC, bool NT = false>
+OCH_D void load_pack_issue(Pack<T, VEC> &p, const char *addr, int64_t estride, int vec)
+{
+   if (vec == 0 && estride == 0) p.v[0] = *reinterpret_cast<const T *>(addr);
+   else load_pack<T, VEC, NT>(p, addr, estride, vec);
+}
+template <class T, int VEC>
+OCH_D void load_pack_finish(Pack<T, VEC> &p, int64_t estride, int vec)
+{
+   if (vec == 0 && estride == 0)
+   {
+#pragma unroll
+      for (int k = 1; k < VEC; k++) p.v[k] = p.v[0];
+   }
+}
+
 template <class T, int VEC, bool NT = false>
 OCH_D void store_pack(const Pack<T, VEC> &p, char *addr, int64_t estride, int vec)
 {
@@ -303,6 +322,7 @@ template <int NOPS> struct TileParams
    int      lds_off[NOPS];                  /* byte offset of the operand's LDS tile */
    int      nt;                             /* streaming launch: nontemporal hint on global accesses */
    int      diagonal;                       /* walk the tile grid along diagonals (see tile_row) */
+   FastDiv  rowdiv;                         /* division by the number of tile rows (gridDim.y) */
    int64_t  so[NOPS][OCH_MAX_DIMS];         /* byte strides of the remaining (outer) dimensions */
    FastDiv  odiv[OCH_MAX_DIMS];
 };
@@ -313,42 +333,53 @@ OCH_D void tile_fetch_arguments(const TileParams<NOPS> &p)
 {
 #pragma unroll
    for (int k = 0; k < NOPS; k++) asm volatile("" :: "s"(p.ptr[k]), "s"(p.s0[k]), "s"(p.s1[k]), "s"(p.trans[k]), "s"(p.vecmode[k]), "s"(p.lds_off[k]));
-   asm volatile("" :: "s"(p.n0), "s"(p.n1), "s"(p.nouter), "s"(p.diagonal));
+   asm volatile("" :: "s"(p.n0), "s"(p.n1), "s"(p.nouter), "s"(p.diagonal), "s"(p.rowdiv.d), "s"(p.rowdiv.m), "s"(p.rowdiv.s1), "s"(p.rowdiv.s2));
 }
 
 constexpr int tile_dim(size_t maxsize) { return maxsize >= 16 ? 32 : 64; }
 template <class T> constexpr int tile_pitch(int tile) { return tile + (sizeof(T) >= 4 ? 1 : 4 / (int)sizeof(T)); }
 template <class T> constexpr int tile_bytes(int tile) { return ((tile * tile_pitch<T>(tile) * (int)sizeof(T)) + 15) / 16 * 16; }
 
+/* Byte offset of position (i0, i1) within a tile. The host takes the tiled kernels only when every stride along the two
+   tile dimensions is below 2^23 bytes in magnitude, so 24-bit multiplies and 32-bit sums are exact: a handful of
+   full-rate instructions per address where 64-bit products cost several quarter-rate ones (with 32 waves per compute
+   unit that arithmetic was a fifth of a tile's time). */
+OCH_D int64_t tile_offset(uint32_t i0, int s0, uint32_t i1, int s1) { return (int64_t)(__mul24((int)i0, s0) + __mul24((int)i1, s1)); }
+
 /* Loads of positions outside an edge tile are not skipped but redirected to a position inside it (and what they
    bring is never used): without a branch around them the compiler issues all loads of a thread back to back before
-   the first one is waited for. n1 is a multiple of the vector length (the host checks it), n0 >= 1. */
-template <class T, int TILE, bool NT, int THREADS>
-OCH_D void tile_stage(T *lds, const char *base, int64_t s0, uint32_t n0, uint32_t n1)
+   the first one is waited for. n1 is a multiple of the vector length (the host checks it), n0 >= 1.
+   tile_load issues the loads of one thread, tile_park writes what they brought into the LDS tile, transposed. */
+template <class T, int TILE, int THREADS> struct TileStage
 {
-   constexpr int VK = vec_for_c<T>();
-   constexpr int LPR = TILE / VK;                        /* lanes per row (fixed index along dimension 0) */
-   constexpr int RPP = THREADS / LPR;                    /* rows per pass */
-   constexpr int PASSES = (TILE + RPP - 1) / RPP;
-   constexpr int PITCH = tile_pitch<T>(TILE);
-   const uint32_t i1 = (threadIdx.x % LPR) * VK, row = threadIdx.x / LPR;
-   const uint32_t i1c = (i1 < n1) ? i1 : 0;
+   static constexpr int VK = vec_for_c<T>();
+   static constexpr int LPR = TILE / VK;                        /* lanes per row (fixed index along dimension 0) */
+   static constexpr int RPP = THREADS / LPR;                    /* rows per pass */
+   static constexpr int PASSES = (TILE + RPP - 1) / RPP;
+   static constexpr int PITCH = tile_pitch<T>(TILE);
    Pack<T, VK> v[PASSES];
+   template <bool NT> OCH_D void load(const char *base, int s0, uint32_t n0, uint32_t n1)
+   {  const uint32_t i1 = (threadIdx.x % LPR) * VK, row = threadIdx.x / LPR;
+      const uint32_t i1c = (i1 < n1) ? i1 : 0;
 #pragma unroll
-   for (int u = 0; u < PASSES; u++)
-   {  const uint32_t i0 = row + u * RPP, i0c = (i0 < n0) ? i0 : n0 - 1;
-      load_wide<T, VK, NT>(v[u], base + (int64_t)i0c * s0 + (int64_t)i1c * (int64_t)sizeof(T));
-   }
-#pragma unroll
-   for (int u = 0; u < PASSES; u++)
-   {  const uint32_t i0 = row + u * RPP;
-      if (PASSES * RPP <= TILE || i0 < (uint32_t)TILE)
-      {
-#pragma unroll
-         for (int j = 0; j < VK; j++) lds[(i1 + j) * PITCH + i0] = v[u].v[j];
+      for (int u = 0; u < PASSES; u++)
+      {  const uint32_t i0 = row + u * RPP, i0c = (i0 < n0) ? i0 : n0 - 1;
+         load_wide<T, VK, NT>(v[u], base + tile_offset(i0c, s0, i1c, (int)sizeof(T)));
       }
    }
-}
+   OCH_D void park(T *lds) const
+   {  const uint32_t i1 = (threadIdx.x % LPR) * VK, row = threadIdx.x / LPR;
+#pragma unroll
+      for (int u = 0; u < PASSES; u++)
+      {  const uint32_t i0 = row + u * RPP;
+         if (PASSES * RPP <= TILE || i0 < (uint32_t)TILE)
+         {
+#pragma unroll
+            for (int j = 0; j < VK; j++) lds[(i1 + j) * PITCH + i0] = v[u].v[j];
+         }
+      }
+   }
+};
 
 /* Tile row of a block. Blocks that run together have neighbouring blockIdx.x. When the pitch of the transposed operand
    is a power of two between 16 KB and 64 KB (4096 x 4096 or 8192 x 8192 float64), the straight order makes them all read
@@ -356,8 +387,16 @@ OCH_D void tile_stage(T *lds, const char *base, int64_t s0, uint32_t n0, uint32_
    the tile row by (three times) the tile column walks the grid along diagonals and spreads both the reads and the writes
    (measured on MI355X: 6.2 against 5.6 TB/s at 4096 x 4096; a shift of one tile row per column gives 6.15, square
    super-tiles of 4 to 32 tiles 5.7 - 5.9). For every other pitch the straight order is the faster one by
-   10 - 25 % (5.5 against 4.4 TB/s at 4224 x 4224), so the host chooses per launch. */
-OCH_D uint32_t tile_row(int diagonal) { return diagonal ? (blockIdx.y + 3 * blockIdx.x) % gridDim.y : blockIdx.y; }
+   10 - 25 % (5.5 against 4.4 TB/s at 4224 x 4224), so the host chooses per launch.
+   What a wave computes before its first load is scalar work that the waves of a SIMD do one after the other, so it
+   is kept short: the remainder comes from a multiply-shift division prepared on the host, the tile origins from
+   32 x 32 -> 64-bit products (the host keeps tile coordinates below 2^31 and strides below 2^23). */
+template <int NOPS>
+OCH_D uint32_t tile_row(const TileParams<NOPS> &p)
+{  if (!p.diagonal) return blockIdx.y;
+   const uint32_t t = blockIdx.y + 3 * blockIdx.x;
+   return t - fastdiv(t, p.rowdiv) * p.rowdiv.d;
+}
 
 template <int NOPS>
 OCH_D void tile_origin(const TileParams<NOPS> &p, int tile, uint32_t trow, int64_t (&off)[NOPS])
@@ -365,25 +404,13 @@ OCH_D void tile_origin(const TileParams<NOPS> &p, int tile, uint32_t trow, int64
    uint32_t q = blockIdx.z;
 #pragma unroll
    for (int k = 0; k < NOPS; k++)
-      off[k] = (int64_t)blockIdx.x * tile * p.s0[k] + (int64_t)trow * tile * p.s1[k];
+      off[k] = (int64_t)(int)(blockIdx.x * tile) * (int64_t)(int)p.s0[k] + (int64_t)(int)(trow * tile) * (int64_t)(int)p.s1[k];
    for (int d = 0; d < p.nouter; d++)
    {  uint32_t q2 = fastdiv(q, p.odiv[d]);
       uint32_t i = q - q2 * p.odiv[d].d; q = q2;
 #pragma unroll
       for (int k = 0; k < NOPS; k++) off[k] += (int64_t)i * p.so[k][d];
    }
-}
-
-/* operand k of a tiled kernel in output order: from its LDS tile, or straight from memory (position clamped into the tile) */
-template <class T, int VEC, int TILE, bool NT>
-OCH_D void tile_fetch(Pack<T, VEC> &v, const T *lds, int trans, const char *base, int64_t s0, int64_t s1, int vecmode, uint32_t i0c, uint32_t i1c)
-{
-   if (trans)
-   {
-#pragma unroll
-      for (int k = 0; k < VEC; k++) v.v[k] = lds[i1c * tile_pitch<T>(TILE) + i0c + k];
-   }
-   else load_pack<T, VEC, NT>(v, base + (int64_t)i0c * s0 + (int64_t)i1c * s1, s0, vecmode);
 }
 
 template <class A, class B, class R> constexpr size_t max_size3()
@@ -400,22 +427,49 @@ __global__ __launch_bounds__(tile_threads(max_size3<typename F::A, typename F::B
    A *la = reinterpret_cast<A *>(och_tile_lds + p.lds_off[0]);
    B *lb = reinterpret_cast<B *>(och_tile_lds + p.lds_off[1]);
    int64_t off[3];
-   const uint32_t trow = tile_row(p.diagonal);
+   const uint32_t trow = tile_row(p);
    tile_origin<3>(p, TILE, trow, off);
    const uint32_t r0 = p.n0 - blockIdx.x * TILE, r1 = p.n1 - trow * TILE;
    const uint32_t n0 = r0 < (uint32_t)TILE ? r0 : TILE, n1 = r1 < (uint32_t)TILE ? r1 : TILE;
-   if (p.trans[0]) tile_stage<A, TILE, NT, THREADS>(la, p.ptr[0] + off[0], p.s0[0], n0, n1);
-   if (p.trans[1]) tile_stage<B, TILE, NT, THREADS>(lb, p.ptr[1] + off[1], p.s0[1], n0, n1);
-   __syncthreads();
+   /* order of a workgroup: loads of the transposed operands, loads of the operands that are read straight from memory
+      (their latency runs in parallel instead of starting behind the barrier), LDS, barrier, LDS */
    constexpr int LPC = TILE / VEC, CPP = THREADS / LPC, PASSES = (TILE + CPP - 1) / CPP;
    const uint32_t i0 = (threadIdx.x % LPC) * VEC, col = threadIdx.x / LPC;
    const uint32_t i0c = (i0 < n0) ? i0 : 0;                  /* n0 is a multiple of VEC */
+   TileStage<A, TILE, THREADS> sa; TileStage<B, TILE, THREADS> sb;
    Pack<A, VEC> a[PASSES]; Pack<B, VEC> b[PASSES];
+   if (p.trans[0]) sa.template load<NT>(p.ptr[0] + off[0], (int)p.s0[0], n0, n1);
+   if (p.trans[1]) sb.template load<NT>(p.ptr[1] + off[1], (int)p.s0[1], n0, n1);
 #pragma unroll
    for (int u = 0; u < PASSES; u++)
    {  const uint32_t i1 = col + u * CPP, i1c = (i1 < n1) ? i1 : n1 - 1;
-      tile_fetch<A, VEC, TILE, NT>(a[u], la, p.trans[0], p.ptr[0] + off[0], p.s0[0], p.s1[0], p.vecmode[0], i0c, i1c);
-      tile_fetch<B, VEC, TILE, NT>(b[u], lb, p.trans[1], p.ptr[1] + off[1], p.s0[1], p.s1[1], p.vecmode[1], i0c, i1c);
+      if (!p.trans[0]) load_pack_issue<A, VEC, NT>(a[u], p.ptr[0] + off[0] + tile_offset(i0c, (int)p.s0[0], i1c, (int)p.s1[0]), p.s0[0], p.vecmode[0]);
+      if (!p.trans[1]) load_pack_issue<B, VEC, NT>(b[u], p.ptr[1] + off[1] + tile_offset(i0c, (int)p.s0[1], i1c, (int)p.s1[1]), p.s0[1], p.vecmode[1]);
+   }
+   if (p.trans[0]) sa.park(la);
+   if (p.trans[1]) sb.park(lb);
+   __syncthreads();
+   /* every load of this thread was issued before the barrier; waiting for all of them here, in one place that every
+      path runs through, lets the compiler see that nothing is outstanding afterwards. Otherwise the paths through
+      the run-time operand modes merge with different numbers of loads in flight, it falls back to waiting for
+      everything -- stores included -- in front of each later pass, and a thread's second store waits for its first
+      to be acknowledged (transposed float64 add 4096 x 4096: 5.85 -> 6.2 TB/s) */
+   __builtin_amdgcn_s_waitcnt(0x0F70);          /* vmcnt(0); expcnt and lgkmcnt left alone */
+#pragma unroll
+   for (int u = 0; u < PASSES; u++)
+   {  const uint32_t i1 = col + u * CPP, i1c = (i1 < n1) ? i1 : n1 - 1;
+      if (p.trans[0])
+      {
+#pragma unroll
+         for (int k = 0; k < VEC; k++) a[u].v[k] = la[i1c * tile_pitch<A>(TILE) + i0c + k];
+      }
+      else load_pack_finish<A, VEC>(a[u], p.s0[0], p.vecmode[0]);
+      if (p.trans[1])
+      {
+#pragma unroll
+         for (int k = 0; k < VEC; k++) b[u].v[k] = lb[i1c * tile_pitch<B>(TILE) + i0c + k];
+      }
+      else load_pack_finish<B, VEC>(b[u], p.s0[1], p.vecmode[1]);
    }
 #pragma unroll
    for (int u = 0; u < PASSES; u++)
@@ -424,7 +478,7 @@ __global__ __launch_bounds__(tile_threads(max_size3<typename F::A, typename F::B
       {  Pack<R, VEC> r;
 #pragma unroll
          for (int k = 0; k < VEC; k++) r.v[k] = F::f(a[u].v[k], b[u].v[k]);
-         store_pack<R, VEC, NT>(r, p.ptr[2] + off[2] + (int64_t)i0 * p.s0[2] + (int64_t)i1 * p.s1[2], p.s0[2], p.vecmode[2]);
+         store_pack<R, VEC, NT>(r, p.ptr[2] + off[2] + tile_offset(i0, (int)p.s0[2], i1, (int)p.s1[2]), p.s0[2], p.vecmode[2]);
       }
    }
 }
@@ -439,11 +493,13 @@ __global__ __launch_bounds__(tile_threads(max_size3<typename F::A, typename F::A
    tile_fetch_arguments<2>(p);
    A *la = reinterpret_cast<A *>(och_tile_lds);
    int64_t off[2];
-   const uint32_t trow = tile_row(p.diagonal);
+   const uint32_t trow = tile_row(p);
    tile_origin<2>(p, TILE, trow, off);
    const uint32_t r0 = p.n0 - blockIdx.x * TILE, r1 = p.n1 - trow * TILE;
    const uint32_t n0 = r0 < (uint32_t)TILE ? r0 : TILE, n1 = r1 < (uint32_t)TILE ? r1 : TILE;
-   tile_stage<A, TILE, NT, THREADS>(la, p.ptr[0] + off[0], p.s0[0], n0, n1);
+   TileStage<A, TILE, THREADS> sa;
+   sa.template load<NT>(p.ptr[0] + off[0], (int)p.s0[0], n0, n1);
+   sa.park(la);
    __syncthreads();
    constexpr int LPC = TILE / VEC, CPP = THREADS / LPC, PASSES = (TILE + CPP - 1) / CPP;
    const uint32_t i0 = (threadIdx.x % LPC) * VEC, col = threadIdx.x / LPC;
@@ -455,7 +511,7 @@ __global__ __launch_bounds__(tile_threads(max_size3<typename F::A, typename F::A
 #pragma unroll
       for (int k = 0; k < VEC; k++) r.v[k] = F::f(la[i1c * tile_pitch<A>(TILE) + i0c + k]);
       if (i0 < n0 && i1 < n1)
-         store_pack<R, VEC, NT>(r, p.ptr[1] + off[1] + (int64_t)i0 * p.s0[1] + (int64_t)i1 * p.s1[1], p.s0[1], p.vecmode[1]);
+         store_pack<R, VEC, NT>(r, p.ptr[1] + off[1] + tile_offset(i0, (int)p.s0[1], i1, (int)p.s1[1]), p.s0[1], p.vecmode[1]);
    }
 }
 
@@ -670,6 +726,10 @@ static bool ew_tile_params(TileParams<NOPS> &t, const EwShape<NOPS> &s, const in
    for (int d = 1; d < s.ndims && d1 < 0; d++)
       for (int k = 0; k < out; k++) if (is_trans(k, d)) { d1 = d; break; }
    if (d1 < 0 || s.size[d1] < 16) return false;
+   for (int k = 0; k < NOPS; k++)            /* in-tile offsets are computed with 24-bit multiplies (tile_offset) */
+   {  const int64_t lim = (int64_t)1 << 23;
+      if (s.stride[k][0] >= lim || s.stride[k][0] <= -lim || s.stride[k][d1] >= lim || s.stride[k][d1] <= -lim) return false;
+   }
    memset(&t, 0, sizeof(t));
    bool any = false; size_t lds = 0;
    for (int k = 0; k < NOPS; k++)
@@ -696,7 +756,8 @@ static bool ew_tile_params(TileParams<NOPS> &t, const EwShape<NOPS> &s, const in
       t.nouter++; outer *= s.size[d];
    }
    uint64_t tiles0 = (s.size[0] + tile - 1) / tile, tiles1 = (s.size[d1] + tile - 1) / tile;
-   if (outer > 65535 || tiles1 > 65535 || tiles0 > 0x7FFFFFFFull) return false;
+   if (outer > 65535 || tiles1 > 65535 || s.size[0] >= 0x40000000ull || s.size[d1] >= 0x40000000ull) return false;
+   t.rowdiv = make_fastdiv((uint32_t)tiles1);
    t.n0 = (uint32_t)s.size[0]; t.n1 = (uint32_t)s.size[d1];
    {  uint64_t bytes = 0;
       for (int k = 0; k < NOPS; k++) bytes += s.nelem * (uint64_t)es[k];
