@@ -168,7 +168,7 @@ def test_steps(hip, stream, dtype):
 
 
 def test_config4_cast_byteswap(hip, stream):
-    """benchmark configuration 4 at reduced size plus the full-size round-trip property:
+    """benchmark configuration 4 at reduced size (the full size is test_config4_full_size):
     int16 3-D tensor (full int16 range, stored byteswapped, step-2 slice) -> contiguous float32, and
     complex64 -> complex128."""
     rng = np.random.default_rng(4)
@@ -197,6 +197,89 @@ def test_config4_cast_byteswap(hip, stream):
     got = y.download()
     x.free(); y.free()
     H.assert_same_bytes(got, z.astype(np.complex128), "config 4b")
+
+
+def test_config4_full_size(hip, stream):
+    """benchmark configuration 4 at its full size, bit for bit against the closed form (every int16 is exactly
+    representable in float32 and every float32 in float64, so numpy's astype is the exact answer) and against the
+    oracle: int16 1024 x 1024 x 64, uniform over the whole range, stored byte-swapped, every second element of the
+    first dimension -> contiguous float32; complex64 -> complex128, 2^26 elements with parts from U(-1, 1)."""
+    rng = np.random.default_rng(404)
+    d0, d1, d2 = 1024, 1024, 64
+    parent = rng.integers(-32768, 32767, size=(d2, d1, 2 * d0), dtype=np.int16, endpoint=True)
+    swapped = parent.byteswap()
+    view = swapped.transpose(2, 1, 0)[::2]
+    assert view.shape == (d0, d1, d2)
+    x = H.Operand(swapped, view, H.INT16).upload(stream)
+    out = np.zeros((d2, d1, d0), np.float32)
+    y = H.Operand(out, out.transpose(2, 1, 0), H.FLOAT).upload(stream)
+    oh.check(oh.lib.och_byteswap_copy(H.INT16, H.FLOAT, 3, oh.sizes(x.shape), oh.strides(x.strides), x.dptr(),
+                                      3, oh.sizes(y.shape), oh.strides(y.strides), y.dptr(), stream.handle))
+    got = y.download()
+    want = out
+    assert orc.lib.oracle_byteswap_copy(H.INT16, H.FLOAT, 3, oh.sizes(x.shape), oh.strides(x.strides), x.hptr(),
+                                        3, oh.sizes(y.shape), oh.strides(y.strides), y.hptr(want), 16) == 0
+    x.free(); y.free()
+    assert got.tobytes() == want.tobytes(), "config 4a, full size, against the oracle"
+    assert np.array_equal(got, parent[:, :, ::2].astype(np.float32)), "config 4a, full size, against the closed form"
+    del parent, swapped, got, want, out
+    n = 1 << 26
+    z = np.empty(n, np.complex64)
+    z.real = rng.uniform(-1, 1, n).astype(np.float32); z.imag = rng.uniform(-1, 1, n).astype(np.float32)
+    x = H.Operand.contiguous(z, H.CFLOAT).upload(stream)
+    dst = oh.DeviceBuffer(16 * n, stream)
+    oh.check(oh.lib.och_copy(H.CFLOAT, H.CDOUBLE, 1, oh.sizes([n]), oh.strides([8]), x.dptr(), 1, oh.sizes([n]), oh.strides([16]), dst.ptr, stream.handle))
+    got = dst.download(np.complex128, n)
+    x.free(); dst.free()
+    want = np.empty(n, np.complex128)
+    assert orc.lib.oracle_copy(H.CFLOAT, H.CDOUBLE, 1, oh.sizes([n]), oh.strides([8]), orc.ptr(z), 1, oh.sizes([n]), oh.strides([16]), orc.ptr(want), 16) == 0
+    assert got.tobytes() == want.tobytes(), "config 4b, full size, against the oracle"
+    assert np.array_equal(got, z.astype(np.complex128)), "config 4b, full size, against the closed form"
+
+
+STEP2_TYPES = [H.BOOL, H.INT8, H.UINT8, H.INT16, H.HALF, H.INT32, H.FLOAT, H.INT64, H.DOUBLE, H.CFLOAT]
+
+
+@pytest.mark.parametrize("dtype", STEP2_TYPES, ids=lambda d: H.NAMES[d])
+def test_step2_sources(hip, stream, dtype):
+    """Sources that are every second element of their first dimension (x[::2]) are read in wide loads of which the odd
+    elements are dropped, when alignment allows, and element by element otherwise; both must give the oracle's bytes.
+    Cases: aligned and misaligned starts, lengths that are and are not multiples of the vector length, a second
+    dimension with an aligned and with an odd pitch, the last element of the view being the last of its buffer (the
+    dropped element behind it would lie outside), same-type copies and widening casts, with and without byte swap."""
+    rng = np.random.default_rng(900 + dtype)
+    dst_types = [dtype, H.FLOAT if dtype not in (H.FLOAT, H.CFLOAT) else H.DOUBLE]
+    if dtype == H.CFLOAT:
+        dst_types = [H.CFLOAT, H.CDOUBLE]
+    cases = []      # (parent elements, start, count, rows, pitch in elements)
+    for start in (0, 1, 2, 8):
+        for count in (1, 5, 64, 257, 1024):
+            cases.append((start, count, 1, 0))
+    cases += [(0, 128, 7, 256), (0, 128, 7, 258), (4, 100, 5, 301), (0, 64, 3, 128)]
+    for start, count, rows, pitch in cases:
+        nparent = start + 2 * count - 1 if rows == 1 else start + (rows - 1) * pitch + 2 * count - 1
+        parent = H.random_data(dtype, nparent, rng, "full")
+        if rows == 1:
+            view = parent[start:start + 2 * count - 1:2]
+        else:
+            view = np.lib.stride_tricks.as_strided(parent[start:], shape=(rows, count), strides=(pitch * parent.itemsize, 2 * parent.itemsize)).T
+        for dt2 in dst_types:
+            for swap in (0, 1):
+                if swap and dtype in (H.BOOL, H.INT8, H.UINT8):
+                    continue
+                x = H.Operand(parent, view, dtype).upload(stream)
+                out = np.zeros(view.size + 3, H.storage(dt2))
+                o = 1 if (start + count) % 2 else 0                    # destinations that wide stores can and cannot take
+                oview = out[o:o + view.size] if rows == 1 else out[o:o + view.size].reshape(rows, count).T
+                y = H.Operand(out, oview, dt2).upload(stream)
+                gfn, cfn = (oh.lib.och_byteswap_copy, orc.lib.oracle_byteswap_copy) if swap else (oh.lib.och_copy, orc.lib.oracle_copy)
+                nd = len(x.shape)
+                oh.check(gfn(dtype, dt2, nd, oh.sizes(x.shape), oh.strides(x.strides), x.dptr(), nd, oh.sizes(y.shape), oh.strides(y.strides), y.dptr(), stream.handle))
+                want = out.copy()
+                assert cfn(dtype, dt2, nd, oh.sizes(x.shape), oh.strides(x.strides), x.hptr(), nd, oh.sizes(y.shape), oh.strides(y.strides), y.hptr(want), 1) == 0
+                got = y.download()
+                x.free(); y.free()
+                H.assert_same_bytes(got.view(np.uint8), want.view(np.uint8), "step-2 %s -> %s swap %d case %s" % (H.NAMES[dtype], H.NAMES[dt2], swap, (start, count, rows, pitch)))
 
 
 def test_memset_is_exact_at_any_alignment_and_size(hip, stream):

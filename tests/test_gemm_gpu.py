@@ -260,6 +260,67 @@ def test_mgs_qr_pattern(hip, stream):
     assert np.abs(Rg[off] - Rref[off]).max() < 1e-11
 
 
+def test_mgs_qr_window_on_the_4096_matrix(hip, stream):
+    """The benchmark's modified Gram-Schmidt workload at its real shape: the first 64 columns of a 4096 x 4096 float64
+    matrix with entries from U(-1, 1), per pair one dot product (gemm, M = N = 1, K = 4096, result kept on the device)
+    and one rank-1 update (gemm, K = 1) reading that device scalar, per column a norm (full reduction into a device
+    scalar) and a division by it -- 2016 pairs, 4160 launches, nothing read back in between. Run launch by launch
+    and again recorded once and replayed as a graph, from the same start; both against the same recurrence evaluated
+    in float64 on the host (dot products in extended precision). Bound: the GEMM bound of 1e-13 times the 64
+    operations a column receives (columns have unit norm, so the bound is absolute)."""
+    rng = np.random.default_rng(4096)
+    m, ncol = 4096, 64
+    A = rng.uniform(-1, 1, (m, m))                       # column j = A[j, :]
+    pairs = [(i, j) for j in range(ncol) for i in range(j)]
+    ref = A[:ncol].copy(); Rref = np.zeros((ncol, ncol))
+    for j in range(ncol):
+        for i in range(j):
+            r = float(np.dot(ref[i].astype(np.longdouble), ref[j].astype(np.longdouble)))
+            Rref[j, i] = r; ref[j] -= r * ref[i]
+        nr = float(np.sqrt(np.dot(ref[j].astype(np.longdouble), ref[j].astype(np.longdouble))))
+        Rref[j, j] = nr; ref[j] /= nr
+    consts = oh.to_device(np.array([1.0, 0.0, -1.0]), stream)
+    c_one, c_zero, c_minus = [C.c_void_p(consts.address + 8 * k) for k in range(3)]
+    results = {}
+    for mode in ("eager", "graph"):
+        Q = oh.to_device(A, stream)
+        R = oh.to_device(np.zeros((ncol, ncol)), stream)
+        col = lambda j: C.c_void_p(Q.address + 8 * m * j)
+        rij = lambda i, j: C.c_void_p(R.address + 8 * (i + ncol * j))
+
+        def window():
+            for j in range(ncol):
+                for i in range(j):
+                    oh.check(oh.lib.och_gemm(H.DOUBLE, b"T", b"N", 1, 1, m, c_minus, col(i), m, col(j), m, c_zero, rij(i, j), 1, 0, stream.handle))
+                    oh.check(oh.lib.och_gemm(H.DOUBLE, b"N", b"N", m, 1, 1, c_one, col(i), m, rij(i, j), 1, c_one, col(j), m, 0, stream.handle))
+                oh.check(oh.lib.och_reduce_all_device(oh.R["norm2"], H.DOUBLE, 1, oh.sizes([m]), oh.strides([8]), col(j), None, None, 0.0, rij(j, j), None, stream.handle))
+                oh.check(oh.lib.och_binary(oh.B["divide"], H.DOUBLE, 1, oh.sizes([m]), oh.strides([8]), col(j), oh.strides([0]), rij(j, j), oh.strides([8]), col(j), stream.handle))
+        if mode == "eager":
+            window()
+        else:
+            oh.check(oh.lib.och_stream_begin_capture(stream.handle))
+            window()
+            graph = C.c_void_p()
+            oh.check(oh.lib.och_stream_end_capture(stream.handle, C.byref(graph)))
+            oh.check(oh.lib.och_graph_launch(graph, stream.handle))
+            stream.synchronize()
+            oh.check(oh.lib.och_graph_destroy(graph))
+        Qg = Q.download(np.float64, ncol * m).reshape(ncol, m)
+        Rg = R.download(np.float64, ncol * ncol).reshape(ncol, ncol)
+        Rg[np.tril(np.ones((ncol, ncol), bool), -1)] *= -1                 # alpha = -1: the dot products are stored negated
+        rest = Q.download(np.float64, m, offset=8 * m * ncol)
+        Q.free(); R.free()
+        assert np.array_equal(rest, A[ncol]), "a column outside the window was touched"
+        assert np.abs(Qg @ Qg.T - np.eye(ncol)).max() < 1e-12, mode
+        assert np.abs(Qg - ref).max() <= 1e-13 * ncol, (mode, np.abs(Qg - ref).max())
+        low = np.tril(np.ones((ncol, ncol), bool))
+        assert np.abs(Rg[low] - Rref[low]).max() <= 1e-13 * ncol * np.abs(Rref).max(), (mode, np.abs(Rg[low] - Rref[low]).max())
+        results[mode] = (Qg, Rg)
+    # the replayed graph runs the same kernels on the same data in the same order
+    assert results["eager"][0].tobytes() == results["graph"][0].tobytes() and results["eager"][1].tobytes() == results["graph"][1].tobytes()
+    consts.free()
+
+
 BATCH_CASES = [  # dtype, ta, tb, M, N, K, batch sizes, B shared by the products, scalars on the device / varying per product
     (H.DOUBLE, "N", "N", 128, 128, 64, (3,), False, False),
     (H.DOUBLE, "T", "N", 70, 50, 90, (2, 3), True, True),
