@@ -4,12 +4,13 @@
  * binary :3983-4133, reductions :5299-5514, axis reductions :5522-5766, gemm :5951-6778) and
  * src/core/generic/tensor_op.c:141-423 (common type, automatic casts, broadcasting, allocation).
  */
-#include "ocean_host.h"
+#include "core_interface.h"
+#include "../../include/ocean_gpu_module.h"
 #include <stdlib.h>
 #include <string.h>
 
 #define MODULE_OR_FAIL(m, device) OcModuleCore *m = OcModuleCore_forDevice(device); \
-   if (m == NULL) return OcErrorMessage("No core module is registered for device %s", (device) ? (device)->name : "(null)")
+   if (m == NULL) OcError(-1, "No core module is registered for device %s", (device) ? (device)->name : "(null)")
 
 /* ---- copy between any two tensors ------------------------------------------------------- */
 static int host_copy_same_type(OcTensor *src, OcTensor *dst)
@@ -25,10 +26,10 @@ static int host_copy_same_type(OcTensor *src, OcTensor *dst)
    return 0;
 }
 int OcTensor_copy(OcTensor *src, OcTensor *dst)
-{  if (src->nelem != dst->nelem) return OcErrorMessage("Mismatch in the number of elements in tensor copy");
+{  if (src->nelem != dst->nelem) OcError(-1, "Mismatch in the number of elements in tensor copy");
    if (src->device == OcCPU && dst->device == OcCPU)
    {  if (src->dtype != dst->dtype || OcTensor_isByteswapped(src) != OcTensor_isByteswapped(dst))
-         return OcErrorMessage("Converting copies between host tensors need the CPU device module, which is not part of this build");
+         OcError(-1, "Converting copies between host tensors need the CPU device module, which is not part of this build");
       return host_copy_same_type(src, dst);
    }
    if (src->device == OcCPU) { MODULE_OR_FAIL(m, dst->device); return m->Tensor_copyFromCPU(src, dst); }
@@ -38,17 +39,19 @@ int OcTensor_copy(OcTensor *src, OcTensor *dst)
 
 /* Replace *tensor by a native-order tensor of the requested type on the requested device when it is not one
    already (tensor_itf.c:1226-1304). The replacement is a new column-major tensor; the old reference is released. */
-int OcTensor_ensure(OcTensor **tensor, OcDType dtype, OcDevice *device)
+static int tensor_ensure(OcTensor **tensor, OcDType dtype, OcDevice *device, int temporary)
 {  OcTensor *t = *tensor, *r;
    if (dtype == OcDTypeNone) dtype = t->dtype;
    if (device == NULL) device = t->device;
    if (t->dtype == dtype && t->device == device && !OcTensor_isByteswapped(t)) return 0;
-   if ((r = OcTensor_create(t->ndims, t->size, NULL, dtype, device)) == NULL) return -1;
+   r = temporary ? OcTensor_createTemporary(t->ndims, t->size, NULL, dtype, device) : OcTensor_create(t->ndims, t->size, NULL, dtype, device);
+   if (r == NULL) return -1;
    if (OcTensor_copy(t, r) != 0) { OcDecrefTensor(r); return -1; }
    OcDecrefTensor(t);
    *tensor = r;
    return 0;
 }
+int OcTensor_ensure(OcTensor **tensor, OcDType dtype, OcDevice *device) { return tensor_ensure(tensor, dtype, device, 0); }
 int OcTensor_fill(OcTensor *tensor, OcScalar *value)
 {  MODULE_OR_FAIL(m, tensor->device);
    return m->Tensor_fill(tensor, value);
@@ -76,7 +79,7 @@ static int broadcast_shape(OcTensor *a, OcTensor *b, int *ndims, OcSize *size)
 {  int i, n = a->ndims > b->ndims ? a->ndims : b->ndims;
    for (i = 0; i < n; i++)
    {  OcSize sa = i < a->ndims ? a->size[i] : 1, sb = i < b->ndims ? b->size[i] : 1;
-      if (sa != sb && sa != 1 && sb != 1) return OcErrorMessage("Tensor dimensions are not compatible (dimension %d: %td and %td)", i, sa, sb);
+      if (sa != sb && sa != 1 && sb != 1) OcError(-1, "Tensor dimensions are not compatible (dimension %d: %td and %td)", i, sa, sb);
       size[i] = (sa == 1) ? sb : sa;
    }
    *ndims = n;
@@ -86,10 +89,10 @@ int OcTensor_binary(int op, OcTensor *src1, OcTensor *src2, OcTensor **dst)
 {  OcTensor *a = NULL, *b = NULL, *va = NULL, *vb = NULL, *out = NULL; OcSize size[OC_TENSOR_MAX_DIMS]; int ndims = 0, result = -1;
    OcDevice *device = src1->device != OcCPU ? src1->device : (src2->device != OcCPU ? src2->device : ((*dst) ? (*dst)->device : OcCPU));
    OcDType dtype, dtype2, rtype; oc_binary_fn fn; int is_compare = (op >= 13 && op <= 18), is_shift = (op >= 25), is_logical = (op >= 22 && op <= 24);
-   if (op < 0 || op >= OC_NBINARY) return OcErrorMessage("Invalid binary operation index (%d)", op);
+   if (op < 0 || op >= OC_NBINARY) OcError(-1, "Invalid binary operation index (%d)", op);
    {  MODULE_OR_FAIL(m, device);
       fn = ((oc_binary_fn *)&m->Tensor_add)[op];
-      if (fn == NULL) return OcErrorMessage("Tensor operation is not supported on device %s", device->name);
+      if (fn == NULL) OcError(-1, "Tensor operation is not supported on device %s", device->name);
    }
    /* common type of the operands; shifts keep the type of the first operand and take int8 counts,
       integer powers take int16 exponents, logical operations work on bool */
@@ -100,7 +103,8 @@ int OcTensor_binary(int op, OcTensor *src1, OcTensor *src2, OcTensor **dst)
    if (op == 6 && !OcDType_isFloat(dtype)) dtype2 = OcDTypeInt16;
    rtype = is_compare ? OcDTypeBool : dtype;
    a = OcIncrefTensor(src1); b = OcIncrefTensor(src2);
-   if (OcTensor_ensure(&a, dtype, device) != 0 || OcTensor_ensure(&b, dtype2, device) != 0) goto final;
+   /* converted operands live in the device's ring of temporary storages: releasing them does not wait for the device */
+   if (tensor_ensure(&a, dtype, device, 1) != 0 || tensor_ensure(&b, dtype2, device, 1) != 0) goto final;
    if (broadcast_shape(a, b, &ndims, size) != 0) goto final;
    if ((va = OcTensor_broadcastTo(a, ndims, size)) == NULL || (vb = OcTensor_broadcastTo(b, ndims, size)) == NULL) goto final;
    if (*dst == NULL)
@@ -132,10 +136,10 @@ final:
 }
 int OcTensor_unary(int op, OcTensor *src, OcTensor **dst)
 {  OcTensor *a = NULL, *out = NULL; oc_unary_fn fn; int result = -1; OcDType rtype;
-   if (op < 0 || op >= OC_NUNARY) return OcErrorMessage("Invalid unary operation index (%d)", op);
+   if (op < 0 || op >= OC_NUNARY) OcError(-1, "Invalid unary operation index (%d)", op);
    {  MODULE_OR_FAIL(m, src->device);
       fn = ((oc_unary_fn *)&m->Tensor_negative)[op];
-      if (fn == NULL) return OcErrorMessage("Tensor operation is not supported on device %s", src->device->name);
+      if (fn == NULL) OcError(-1, "Tensor operation is not supported on device %s", src->device->name);
    }
    a = OcIncrefTensor(src);
    {  /* the negative of an unsigned tensor is taken in its signed type (tensor_itf.c:3637-3651, signed types of src/base/dtype.c:57-61) */
@@ -202,8 +206,8 @@ int OcTensor_axisReduce(int which, OcTensor *src, int n, int *axes, int keepdims
    static const int order[] = { 0, 1, 2, 3, 4, 5, 6, 15, 17, 16, 18, 19, 20, 22, 21, 24, 23, 27, 28 };   /* table order of the axis block */
    for (i = 0, j = 0; i < n; i++)
    {  int k = axes[i] < 0 ? axes[i] + src->ndims : axes[i];
-      if (k < 0 || k >= src->ndims) return OcErrorMessage("Axis index %d out of range", axes[i]);
-      if (flag[k]) return OcErrorMessage("Repeated axis index %d", axes[i]);
+      if (k < 0 || k >= src->ndims) OcError(-1, "Axis index %d out of range", axes[i]);
+      if (flag[k]) OcError(-1, "Repeated axis index %d", axes[i]);
       flag[k] = 1; ax[j++] = k;
    }
    for (i = 0; i < src->ndims; i++) { if (!flag[i]) size[nd++] = src->size[i]; else if (keepdims) size[nd++] = 1; }
@@ -281,7 +285,7 @@ static OcTensor *scalar_tensor(OcScalar *s, OcDType dtype, double fallback)
 /* leading dimension of a matrix operand, flipping the mode when only its rows are contiguous */
 static int gemm_operand(OcTensor **t, char *mode, OcIndex *ld, int complex_type)
 {  OcTensor *x = *t; int es = x->elemsize;
-   if (x->ndims < 2) return OcErrorMessage("Matrix multiplication needs tensors of at least two dimensions");
+   if (x->ndims < 2) OcError(-1, "Matrix multiplication needs tensors of at least two dimensions");
    if ((x->size[0] == 1 || x->strides[0] == es) && (x->size[1] == 1 || (x->strides[1] >= x->size[0] * es && x->strides[1] % es == 0)))
    {  *ld = (x->size[1] == 1) ? (x->size[0] > 0 ? x->size[0] : 1) : x->strides[1] / es; return 0; }
    if ((x->size[1] == 1 || x->strides[1] == es) && (x->size[0] == 1 || (x->strides[0] >= x->size[1] * es && x->strides[0] % es == 0)) && !(complex_type && *mode == 'C'))
@@ -366,3 +370,67 @@ final:
    return result;
 }
 int OcTensor_mtimes(OcTensor *A, OcTensor *B, OcTensor **C) { return OcTensor_gemm(NULL, A, 'N', B, 'N', NULL, C); }
+
+/* ---- index operations through the table (src/core/interface/index_itf.c, tensor_itf.c:2359-2700) ----------------- */
+/* indices: int64 tensor [k, n] on the tensor's device: n index tuples for the first k dimensions of `tensor` (negative
+   values count from the end). Builds the view the interface builds -- one offset table per indexed dimension, made by
+   Tensor_addIfNegative + Tensor_indexToOffset on storages (and streams) of their own -- and hands it to the module. */
+static int index_view(OcTensor *tensor, OcTensor *indices, OcTensorIndexView *view, OcTensor **work, OcSize *vsize, OcIndex *vstrides, int *vnd)
+{  OcModuleCore *m = OcModuleCore_forDevice(tensor->device); int k, d; OcSize n;
+   if (m == NULL) OcError(-1, "No core module is registered for device %s", tensor->device->name);
+   if (indices->dtype != OcDTypeInt64 || indices->ndims != 2 || indices->device != tensor->device) OcError(-1, "Indices must be an int64 tensor [k, n] on the tensor's device");
+   k = (int)indices->size[0]; n = indices->size[1];
+   if (k < 1 || k > tensor->ndims) OcError(-1, "Number of index dimensions out of range");
+   memset(view, 0, sizeof(*view));
+   /* view dimensions: one of size n for the tuples, then the dimensions of the tensor that are not indexed; every
+      indexed dimension but the first becomes a dimension of size 1 whose table is broadcast -- here the k tables are
+      folded into ONE table of byte offsets (indexToOffset multiplies by the strides and sums over the k rows) */
+   *vnd = 1 + tensor->ndims - k;
+   vsize[0] = n; vstrides[0] = 0;
+   for (d = k; d < tensor->ndims; d++) { vsize[1 + d - k] = tensor->size[d]; vstrides[1 + d - k] = tensor->strides[d]; }
+   {  OcTensor *idx = OcTensor_create(2, indices->size, NULL, OcDTypeInt64, tensor->device), *off; OcInt64 strides[OC_TENSOR_MAX_DIMS]; OcScalar s;
+      OcSize one = n;
+      if (idx == NULL) return -1;
+      if (OcTensor_copy(indices, idx) != 0) { OcDecrefTensor(idx); return -1; }
+      for (d = 0; d < k; d++)              /* negative indices: add the dimension's size, row by row */
+      {  OcTensor *row = OcTensor_slice(idx, 0, d, 1, 1);
+         s.dtype = OcDTypeInt64; s.value.sInt64 = tensor->size[d];
+         if (row == NULL || m->Tensor_addIfNegative(row, &s) != 0) { if (row) OcDecrefTensor(row); OcDecrefTensor(idx); return -1; }
+         OcDecrefTensor(row);
+         strides[d] = tensor->strides[d];
+      }
+      if ((off = OcTensor_create(1, &one, NULL, OcDTypeInt64, tensor->device)) == NULL) { OcDecrefTensor(idx); return -1; }
+      if (m->Tensor_indexToOffset(idx, strides, off) != 0) { OcDecrefTensor(idx); OcDecrefTensor(off); return -1; }
+      OcDecrefTensor(idx);
+      *work = off;
+   }
+   return 0;
+}
+int OcTensor_getIndexed(OcTensor *tensor, OcTensor *indices, OcTensor **dst)
+{  OcTensorIndexView view; OcTensor *off = NULL, *v = NULL, *out = NULL, *offsets[OC_TENSOR_MAX_DIMS] = { 0 }; OcSize vsize[OC_TENSOR_MAX_DIMS]; OcIndex vstrides[OC_TENSOR_MAX_DIMS];
+   int vnd, result = -1; OcModuleCore *m = OcModuleCore_forDevice(tensor->device);
+   if (index_view(tensor, indices, &view, &off, vsize, vstrides, &vnd) != 0) return -1;
+   if ((v = OcTensor_createFromStorage(tensor->storage, vnd, vsize, vstrides, tensor->offset, tensor->dtype)) == NULL) goto final;
+   offsets[0] = off; view.ndims = vnd; view.view = v; view.offsets = offsets;
+   if ((out = OcTensor_create(vnd, vsize, NULL, tensor->dtype, tensor->device)) == NULL) goto final;
+   if ((result = m->Tensor_getIndex(&view, out)) == 0) { *dst = out; out = NULL; }
+final:
+   if (out) OcDecrefTensor(out);
+   if (v) OcDecrefTensor(v);
+   if (off) OcDecrefTensor(off);
+   return result;
+}
+int OcTensor_setIndexed(OcTensor *tensor, OcTensor *indices, OcTensor *src)
+{  OcTensorIndexView view; OcTensor *off = NULL, *v = NULL, *offsets[OC_TENSOR_MAX_DIMS] = { 0 }; OcSize vsize[OC_TENSOR_MAX_DIMS]; OcIndex vstrides[OC_TENSOR_MAX_DIMS];
+   int vnd, d, result = -1; OcModuleCore *m = OcModuleCore_forDevice(tensor->device);
+   if (index_view(tensor, indices, &view, &off, vsize, vstrides, &vnd) != 0) return -1;
+   if ((v = OcTensor_createFromStorage(tensor->storage, vnd, vsize, vstrides, tensor->offset, tensor->dtype)) == NULL) goto final;
+   offsets[0] = off; view.ndims = vnd; view.view = v; view.offsets = offsets;
+   if (src->ndims != vnd || src->dtype != tensor->dtype || src->device != tensor->device) { OcErrorMessage("Source of an indexed assignment must match the view"); goto final; }
+   for (d = 0; d < vnd; d++) if (src->size[d] != vsize[d]) { OcErrorMessage("Source size mismatch in dimension %d", d); goto final; }
+   result = m->Tensor_setIndex(&view, src);
+final:
+   if (v) OcDecrefTensor(v);
+   if (off) OcDecrefTensor(off);
+   return result;
+}

@@ -14,133 +14,171 @@
 #include <stdlib.h>
 #include <string.h>
 
-/* ---- device objects -------------------------------------------------------------- */
+/* ---- device objects (device_gpu.c:81-122, 251-420) ------------------------------------ */
 #define OC_GPU_MAX_FREE 64                       /* free-list bound, device_gpu.c:251-370 */
 typedef struct { OcStream HEAD; och_stream handle; } OcStreamGPU;
 typedef struct { OcEvent HEAD; och_event handle; } OcEventGPU;
+typedef struct { OcStorage HEAD; } OcStorageGPU;
 typedef struct
 {  OcDevice        HEAD;
    och_device_prop properties;
    OcStream       *freeStreams;  int nFreeStreams;
    OcEvent        *freeEvents;   int nFreeEvents;
+   long            eventsRecorded, eventsWaited, streamsCreated;      /* activity counters (OcDeviceGPU_activity) */
 } OcDeviceGPU;
+/* the context of the core module on a GPU device: the interface's part first (module_core_gpu.h:28-32 has the BLAS
+   handle behind it; the MFMA GEMM kernels need none) */
+typedef struct { OcModuleCore_Context HEAD; int deviceIndex; } OcModuleCoreGPU_Context;
 
 OcDevice **OcGPU = NULL;
 static int oc_gpu_count = 0;
 static int oc_gpu_initialized = 0;
-static OcModuleCore oc_module_core_gpu;          /* the table Ocean copies at registration */
-static OcModuleCore oc_registered_gpu;           /* the registered copy (device_module.c:415) */
-static int oc_registered = 0;
+static OcDeviceType *oc_device_type_gpu = NULL;
+static OcModuleCore oc_module_core_gpu;          /* the table that registration copies (device_module.c:415) */
 
-#define OCH_CALL(x) do { if ((x) != 0) return OcErrorMessage("%s", och_last_error()); } while (0)
+#define OCH_CALL(x) do { if ((x) != 0) OcError(-1, "%s", och_last_error()); } while (0)
 #define GPU_STREAM(t) (((OcStreamGPU *)((t)->storage->stream))->handle)
-static int activate(OcDevice *device) { if (och_device_set(device->index) != 0) return OcErrorMessage("%s", och_last_error()); return 0; }
+static int activate(OcDevice *device) { if (och_device_set(device->index) != 0) OcError(-1, "%s", och_last_error()); return 0; }
 
-static OcStream *gpu_create_stream(OcDevice *device)
+static OcStream *OcDeviceGPU_createStream(OcDevice *device)
 {  OcDeviceGPU *g = (OcDeviceGPU *)device; OcStreamGPU *s;
    if (g->freeStreams)
    {  s = (OcStreamGPU *)g->freeStreams; g->freeStreams = s->HEAD.next; g->nFreeStreams--; }
    else
    {  if (activate(device) != 0) return NULL;
-      s = (OcStreamGPU *)calloc(1, sizeof(OcStreamGPU));
-      if (s == NULL) { OcErrorMessage("Insufficient memory to allocate a stream object"); return NULL; }
-      if (och_stream_create(&s->handle) != 0) { OcErrorMessage("%s", och_last_error()); free(s); return NULL; }
+      s = (OcStreamGPU *)OcMalloc(sizeof(OcStreamGPU));
+      if (s == NULL) OcError(NULL, "Insufficient memory to allocate a stream object");
+      if (och_stream_create(&s->handle) != 0) { OcErrorMessage("%s", och_last_error()); OcFree(s); return NULL; }
+      g->streamsCreated++;
    }
    s->HEAD.device = device; s->HEAD.next = NULL; s->HEAD.refcount = 1;
    return &s->HEAD;
 }
-static void gpu_delete_stream(OcStream *stream)
+/* called by OcDecrefStream when the last reference goes (device.c:225-236, after synchronising the stream) */
+static void OcDeviceGPU_deleteStream(OcStream *stream)
 {  OcDeviceGPU *g;
-   if (stream == NULL || --stream->refcount > 0) return;
+   if (stream == NULL) return;
    g = (OcDeviceGPU *)stream->device;
    if (g->nFreeStreams < OC_GPU_MAX_FREE) { stream->next = g->freeStreams; g->freeStreams = stream; g->nFreeStreams++; }
-   else { och_stream_destroy(((OcStreamGPU *)stream)->handle); free(stream); }
+   else { och_stream_destroy(((OcStreamGPU *)stream)->handle); OcFree(stream); }
 }
-static int gpu_create_event(OcDevice *device, OcEvent **event)
+static int OcDeviceGPU_createEvent(OcDevice *device, OcEvent **event)
 {  OcDeviceGPU *g = (OcDeviceGPU *)device; OcEventGPU *e;
    if (g->freeEvents) { e = (OcEventGPU *)g->freeEvents; g->freeEvents = e->HEAD.next; g->nFreeEvents--; }
    else
    {  if (activate(device) != 0) return -1;
-      e = (OcEventGPU *)calloc(1, sizeof(OcEventGPU));
-      if (e == NULL) return OcErrorMessage("Insufficient memory to allocate an event object");
-      if (och_event_create(&e->handle, 0) != 0) { free(e); return OcErrorMessage("%s", och_last_error()); }
+      e = (OcEventGPU *)OcMalloc(sizeof(OcEventGPU));
+      if (e == NULL) OcError(-1, "Insufficient memory to allocate an event object");
+      if (och_event_create(&e->handle, 0) != 0) { OcFree(e); OcError(-1, "%s", och_last_error()); }
    }
    e->HEAD.next = NULL; *event = &e->HEAD;
    return 0;
 }
-static void gpu_delete_event(OcDevice *device, OcEvent *event)
+static void OcDeviceGPU_deleteEvent(OcDevice *device, OcEvent *event)
 {  OcDeviceGPU *g = (OcDeviceGPU *)device;
    if (event == NULL) return;
    if (g->nFreeEvents < OC_GPU_MAX_FREE) { event->next = g->freeEvents; g->freeEvents = event; g->nFreeEvents++; }
-   else { och_event_destroy(((OcEventGPU *)event)->handle); free(event); }
+   else { och_event_destroy(((OcEventGPU *)event)->handle); OcFree(event); }
 }
-static int gpu_sync_stream(OcStream *s)  { OCH_CALL(och_stream_synchronize(((OcStreamGPU *)s)->handle)); return 0; }
-static int gpu_sync_event(OcEvent *e)    { OCH_CALL(och_event_synchronize(((OcEventGPU *)e)->handle)); return 0; }
-static int gpu_record_event(OcEvent *e, OcStream *s) { OCH_CALL(och_event_record(((OcEventGPU *)e)->handle, ((OcStreamGPU *)s)->handle)); return 0; }
-static int gpu_wait_event(OcStream *s, OcEvent *e)   { OCH_CALL(och_stream_wait_event(((OcStreamGPU *)s)->handle, ((OcEventGPU *)e)->handle)); return 0; }
-static void gpu_finalize_device(OcDevice *device)
+static int OcStreamGPU_synchronize(OcStream *s)  { OCH_CALL(och_stream_synchronize(((OcStreamGPU *)s)->handle)); return 0; }
+static int OcEventGPU_synchronize(OcEvent *e)    { OCH_CALL(och_event_synchronize(((OcEventGPU *)e)->handle)); return 0; }
+static int OcEventGPU_record(OcEvent *e, OcStream *s)
+{  ((OcDeviceGPU *)s->device)->eventsRecorded++;
+   OCH_CALL(och_event_record(((OcEventGPU *)e)->handle, ((OcStreamGPU *)s)->handle)); return 0;
+}
+static int OcStreamGPU_waitEvent(OcStream *s, OcEvent *e)
+{  ((OcDeviceGPU *)s->device)->eventsWaited++;
+   OCH_CALL(och_stream_wait_event(((OcStreamGPU *)s)->handle, ((OcEventGPU *)e)->handle)); return 0;
+}
+static void OcFreeDeviceGPU(OcDevice *device)
 {  OcDeviceGPU *g = (OcDeviceGPU *)device;
-   while (g->freeStreams) { OcStream *s = g->freeStreams; g->freeStreams = s->next; och_stream_destroy(((OcStreamGPU *)s)->handle); free(s); }
-   while (g->freeEvents)  { OcEvent *e = g->freeEvents; g->freeEvents = e->next; och_event_destroy(((OcEventGPU *)e)->handle); free(e); }
+   och_device_set(device->index);
+   while (g->freeStreams) { OcStream *s = g->freeStreams; g->freeStreams = s->next; och_stream_destroy(((OcStreamGPU *)s)->handle); OcFree(s); }
+   while (g->freeEvents)  { OcEvent *e = g->freeEvents; g->freeEvents = e->next; och_event_destroy(((OcEventGPU *)e)->handle); OcFree(e); }
+}
+/* device_gpu.c:81-122. A GPU device has NO default stream: every storage gets a stream of its own (storage.c:94-103),
+   so that operations on different tensors overlap and are ordered by the read / write protocol only. */
+static OcDevice *OcCreateDeviceGPU(OcDeviceType *type, int index, const char *name)
+{  OcDevice *device = OcCreateDevice(type, index, name, sizeof(OcDeviceGPU)); OcDeviceGPU *g = (OcDeviceGPU *)device;
+   if (device == NULL) return NULL;
+   device->finalize = OcFreeDeviceGPU; device->endianness = 0; device->requiresAlignedData = 1;
+   device->create_stream = OcDeviceGPU_createStream; device->create_event = OcDeviceGPU_createEvent;
+   device->delete_stream = OcDeviceGPU_deleteStream; device->delete_event = OcDeviceGPU_deleteEvent;
+   device->sync_stream = OcStreamGPU_synchronize;    device->sync_event = OcEventGPU_synchronize;
+   device->record_event = OcEventGPU_record;          device->wait_event = OcStreamGPU_waitEvent;
+   g->freeStreams = NULL; g->nFreeStreams = 0; g->freeEvents = NULL; g->nFreeEvents = 0;
+   g->eventsRecorded = g->eventsWaited = g->streamsCreated = 0;
+   if (och_device_properties(index, &g->properties) != 0 || och_device_warmup(index) != 0)          /* device_gpu.c:155-196, 471-616 */
+   {  OcErrorMessage("%s", och_last_error()); OcDecrefDevice(device); return NULL; }
+   return device;
 }
 
-/* ---- storage ---------------------------------------------------------------------- */
-static void gpu_storage_finalize(OcStorage *storage)
-{  if ((storage->flags & OC_STORAGE_OWNER) && storage->data)
+/* ---- storage (storage_gpu.c:61-302) ------------------------------------------------- */
+static void OcStorageGPU_finalize(OcStorage *storage)
+{  if (storage->data && OcStorage_isOwner(storage))
    {  och_device_set(storage->stream->device->index);
-      och_free_async(storage->data, ((OcStreamGPU *)storage->stream)->handle);
+      och_free_async(storage->data, ((OcStreamGPU *)storage->stream)->handle);       /* stream-ordered: behind the storage's last work */
    }
 }
 static OcStorage *OcStorageGPU_create(OcSize nelem, OcDType dtype, OcDevice *device, OcStream *stream)
-{  OcStorage *s; void *ptr = NULL;
-   if (activate(device) != 0) return NULL;
-   s = (OcStorage *)calloc(1, sizeof(OcStorage));
-   if (s == NULL) { OcErrorMessage("Insufficient memory to allocate the storage object"); return NULL; }
-   s->elemsize = OcDType_size(dtype); s->dtype = dtype; s->nelem = nelem; s->size = s->capacity = nelem * s->elemsize;
-   if (stream == NULL) stream = device->defaultStream;
-   stream->refcount++; s->stream = stream;
-   if (gpu_create_event(device, &s->event) != 0) { gpu_delete_stream(stream); free(s); return NULL; }
-   if (och_malloc_async(&ptr, (size_t)(s->size > 0 ? s->size : 1), ((OcStreamGPU *)stream)->handle) != 0)
-   {  OcErrorMessage("%s", och_last_error()); gpu_delete_event(device, s->event); gpu_delete_stream(stream); free(s); return NULL; }
-   s->data = (char *)ptr; s->flags = OC_STORAGE_OWNER; s->refcount = 1; s->finalize = gpu_storage_finalize;
-   return s;
+{  OcStorage *storage = OcAllocateStorage(device, dtype, stream, sizeof(OcStorageGPU)); void *ptr = NULL; OcSize size;
+   if (storage == NULL) return NULL;
+   storage->flags |= OC_STORAGE_OWNER; storage->finalize = OcStorageGPU_finalize; storage->data = NULL;
+   size = nelem * storage->elemsize;
+   storage->size = size; storage->capacity = size; storage->nelem = nelem;
+   if (nelem > 0)
+   {  if (activate(device) != 0) goto error;
+      if (och_malloc_async(&ptr, (size_t)size, ((OcStreamGPU *)storage->stream)->handle) != 0)
+      {  OcErrorMessage("Error allocating %s storage of size %lu on %s: %s", OcDType_name(dtype), (unsigned long)nelem, device->name, och_last_error());
+         goto error;
+      }
+      storage->data = (char *)ptr;
+   }
+   return storage;
+error:
+   OcDecrefStorage(storage);
+   return NULL;
 }
 static int OcBufferGPU_copy(OcStorage *src, void *srcData, OcStorage *dst, void *dstData, OcDType dtype, OcSize n)
-{  if (src->stream->device != dst->stream->device) return OcErrorMessage("Copies between GPU devices are not part of this build (one device)");
-   if (activate(dst->stream->device) != 0 || OcStorage_startRead(dst, src) != 0) return -1;
+{  if (n == 0) return 0;
+   if (src->stream->device != dst->stream->device) OcError(-1, "Copies between GPU devices are not part of this build (one device)");
+   if (OcStorage_startRead(dst, src) != 0 || activate(dst->stream->device) != 0) return -1;
    OCH_CALL(och_memcpy_dtod_async(dstData, srcData, (size_t)(n * OcDType_size(dtype)), ((OcStreamGPU *)dst->stream)->handle));
+   if (OcStorage_update(dst) != 0) return -1;
    return OcStorage_finishRead(dst, src);
 }
+/* the transfers between host and device block, as the reference's do (storage_gpu.c:165-250): wait for the storage's
+   outstanding work, copy, record */
 static int OcBufferGPU_copyFromCPU(OcStorage *src, void *srcData, OcStorage *dst, void *dstData, OcDType dtype, OcSize n)
 {  (void)src;
-   if (activate(dst->stream->device) != 0) return -1;
-   OCH_CALL(och_memcpy_htod(dstData, srcData, (size_t)(n * OcDType_size(dtype)), ((OcStreamGPU *)dst->stream)->handle));   /* blocking, storage_gpu.c:165-189 */
-   return 0;
+   if (OcStorage_synchronize(dst) != 0 || activate(dst->stream->device) != 0) return -1;
+   OCH_CALL(och_memcpy_htod(dstData, srcData, (size_t)(n * OcDType_size(dtype)), ((OcStreamGPU *)dst->stream)->handle));
+   return OcStorage_update(dst);
 }
 static int OcBufferGPU_copyToCPU(OcStorage *src, void *srcData, OcStorage *dst, void *dstData, OcDType dtype, OcSize n)
-{  (void)dst;
-   if (activate(src->stream->device) != 0) return -1;
+{  if (OcStorage_synchronize(src) != 0 || activate(src->stream->device) != 0) return -1;
    OCH_CALL(och_memcpy_dtoh(dstData, srcData, (size_t)(n * OcDType_size(dtype)), ((OcStreamGPU *)src->stream)->handle));
-   return 0;
+   if (OcStorage_update(dst) != 0) return -1;
+   return OcStorage_finishRead(src, src);                              /* updates the read event */
 }
 static int OcBufferGPU_copyHostStorage(OcStorage *storage, OcSize offset, OcSize nbytes, void *ptr)
-{  if (activate(storage->stream->device) != 0) return -1;
+{  if (OcStorage_synchronize(storage) != 0 || activate(storage->stream->device) != 0) return -1;
    OCH_CALL(och_memcpy_htod(storage->data + offset, ptr, (size_t)nbytes, ((OcStreamGPU *)storage->stream)->handle));
-   return 0;
+   return OcStorage_update(storage);
 }
 static int OcBufferGPU_copyStorageHost(OcStorage *storage, OcSize offset, OcSize nbytes, void *ptr)
-{  if (activate(storage->stream->device) != 0) return -1;
+{  if (OcStorage_synchronize(storage) != 0 || activate(storage->stream->device) != 0) return -1;
    OCH_CALL(och_memcpy_dtoh(ptr, storage->data + offset, (size_t)nbytes, ((OcStreamGPU *)storage->stream)->handle));
-   return 0;
+   return OcStorage_finishRead(storage, storage);
 }
 static int OcBufferGPU_zero(OcStorage *storage, void *data, OcDType dtype, OcSize size)
 {  if (activate(storage->stream->device) != 0) return -1;
    OCH_CALL(och_memset_async(data, 0, (size_t)(size * OcDType_size(dtype)), ((OcStreamGPU *)storage->stream)->handle));
-   return 0;
+   return OcStorage_update(storage);
 }
 static int OcDeviceGPU_formatInfo(OcDevice *device, char **str, const char *header, const char *footer)
 {  OcDeviceGPU *g = (OcDeviceGPU *)device; size_t n = 512 + (header ? strlen(header) : 0) + (footer ? strlen(footer) : 0);
-   if ((*str = (char *)malloc(n)) == NULL) return OcErrorMessage("Insufficient memory for the device description");
+   if ((*str = (char *)OcMalloc(n)) == NULL) OcError(-1, "Insufficient memory for the device description");
    snprintf(*str, n, "%sDevice %s: %s (%s), %d compute units, %.1f GiB%s", header ? header : "", device->name, g->properties.name,
             g->properties.arch, g->properties.multiprocessor_count, g->properties.total_global_mem / 1073741824.0, footer ? footer : "");
    return 0;
@@ -161,8 +199,8 @@ static int OcTensorGPU_copy(OcTensor *src, OcTensor *dst)
       other byte order is swapped in place after a converting copy (src/core/cpu/op/tensor_copy_cpu.c:140-156) */
    int differ = (src->dtype != dst->dtype);
    int swap = differ ? OcTensor_isByteswapped(src) : (OcTensor_isByteswapped(src) != OcTensor_isByteswapped(dst));
-   if (src->device != dst->device) return OcErrorMessage("Copies between GPU devices are not part of this build (one device)");
-   if (src->nelem != dst->nelem) return OcErrorMessage("Mismatch in the number of elements in tensor copy");
+   if (src->device != dst->device) OcError(-1, "Copies between GPU devices are not part of this build (one device)");
+   if (src->nelem != dst->nelem) OcError(-1, "Mismatch in the number of elements in tensor copy");
    if (dst->nelem == 0) return 0;
    if (activate(dst->device) != 0 || OcTensor_startRead(dst, src) != 0) return -1;
    OCH_CALL((swap ? och_byteswap_copy : och_copy)(src->dtype, dst->dtype, src->ndims, SZ(src), src->strides, OcTensor_data(src),
@@ -172,19 +210,21 @@ static int OcTensorGPU_copy(OcTensor *src, OcTensor *dst)
    if (OcTensor_update(dst) != 0) return -1;
    return OcTensor_finishRead(dst, src);
 }
-/* Host tensors enter the device as raw bytes of their memory extent and are converted, re-strided and
-   byte-swapped there (tensor_copy_gpu.c:136-161 stages through an intermediate tensor likewise). */
+/* Host tensors enter the device as the raw bytes of their memory extent and are converted, re-strided and byte-swapped
+   there. The extent follows Ocean's convention (shape.c:82-125, used by tensor_copy_gpu.c:141-153): `offset` is the
+   number of bytes in FRONT of the data pointer (negative strides), so the window starts at data - offset. */
 static int OcTensorGPU_copyFromCPU(OcTensor *src, OcTensor *dst)
-{  OcStorage *stage; OcTensor *view; int result;
-   if (src->nelem != dst->nelem) return OcErrorMessage("Mismatch in the number of elements in tensor copy");
+{  OcStorage *stage; OcTensor *view; OcSize offset, extent; int result;
+   if (src->nelem != dst->nelem) OcError(-1, "Mismatch in the number of elements in tensor copy");
    if (dst->nelem == 0) return 0;
-   if ((stage = OcStorageGPU_create(src->blockExtent, OcDTypeInt8, dst->device, dst->storage->stream)) == NULL) return -1;
-   if (OcBufferGPU_copyFromCPU(src->storage, OcTensor_data(src) + src->blockOffset, stage, stage->data, OcDTypeInt8, src->blockExtent) != 0)
+   if (OcShape_extent(src->ndims, src->size, src->strides, src->elemsize, &offset, &extent) != 0) return -1;
+   if ((stage = OcStorage_createTemporary(extent, OcDTypeInt8, dst->device)) == NULL) return -1;
+   if (OcBufferGPU_copyFromCPU(src->storage, OcTensor_data(src) - offset, stage, stage->data, OcDTypeInt8, extent) != 0)
    {  OcDecrefStorage(stage); return -1; }
-   view = OcTensor_createFromStorage(stage, src->ndims, src->size, src->strides, -src->blockOffset, src->dtype);
+   view = OcTensor_createFromStorage(stage, src->ndims, src->size, src->strides, offset, src->dtype);
    OcDecrefStorage(stage);
    if (view == NULL) return -1;
-   view->flags = src->flags;
+   OcTensor_setByteswapped(view, OcTensor_isByteswapped(src));
    result = OcTensorGPU_copy(view, dst);
    OcDecrefTensor(view);
    return result;
@@ -192,17 +232,17 @@ static int OcTensorGPU_copyFromCPU(OcTensor *src, OcTensor *dst)
 static int OcTensorGPU_copyToCPU(OcTensor *src, OcTensor *dst)
 {  OcTensor *dense; int result; OcSize i, n = src->nelem; int es = dst->elemsize;
    char *host;
-   if (src->nelem != dst->nelem) return OcErrorMessage("Mismatch in the number of elements in tensor copy");
+   if (src->nelem != dst->nelem) OcError(-1, "Mismatch in the number of elements in tensor copy");
    if (n == 0) return 0;
    /* convert / gather on the device into a dense tensor of the destination's type and byte order */
-   if ((dense = OcTensor_create(dst->ndims, dst->size, NULL, dst->dtype, src->device)) == NULL) return -1;
-   dense->flags |= (dst->flags & OC_TENSOR_BYTESWAPPED);
+   if ((dense = OcTensor_createTemporary(dst->ndims, dst->size, NULL, dst->dtype, src->device)) == NULL) return -1;
+   OcTensor_setByteswapped(dense, OcTensor_isByteswapped(dst));
    result = OcTensorGPU_copy(src, dense);
    if (result == 0 && OcTensor_isContiguous(dst))
       result = OcBufferGPU_copyToCPU(dense->storage, OcTensor_data(dense), dst->storage, OcTensor_data(dst), dst->dtype, n);
    else if (result == 0)
    {  /* strided host destination: download densely, then place element by element */
-      if ((host = (char *)malloc((size_t)(n * es))) == NULL) result = OcErrorMessage("Insufficient memory for the host staging buffer");
+      if ((host = (char *)OcMalloc((size_t)(n * es))) == NULL) { OcErrorMessage("Insufficient memory for the host staging buffer"); result = -1; }
       else
       {  result = OcBufferGPU_copyToCPU(dense->storage, OcTensor_data(dense), dst->storage, host, dst->dtype, n);
          if (result == 0)
@@ -214,7 +254,7 @@ static int OcTensorGPU_copyToCPU(OcTensor *src, OcTensor *dst)
                for (d = 0; d < dst->ndims; d++) { if (++idx[d] < dst->size[d]) break; idx[d] = 0; }
             }
          }
-         free(host);
+         OcFree(host);
       }
    }
    OcDecrefTensor(dense);
@@ -230,7 +270,7 @@ static int OcTensorGPU_byteswapNoFlag(OcTensor *tensor)
 /* ---- fill / steps ------------------------------------------------------------------------ */
 static int OcTensorGPU_fill(OcTensor *tensor, OcScalar *scalar)
 {  och_scalar v; scalar_value(scalar, &v);
-   if (scalar->dtype != tensor->dtype) return OcErrorMessage("Fill value must have the tensor's data type");
+   if (scalar->dtype != tensor->dtype) OcError(-1, "Fill value must have the tensor's data type");
    if (activate(tensor->device) != 0) return -1;
    OCH_CALL(och_fill(tensor->dtype, tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), v, GPU_STREAM(tensor)));
    return OcTensor_update(tensor);
@@ -244,7 +284,7 @@ static int OcTensorGPU_fillNaN(OcTensor *tensor, OcScalar *scalar)
 }
 static int OcTensorGPU_maskedFill(OcTensor *tensor, OcTensor *mask, OcScalar *scalar)
 {  och_scalar v; scalar_value(scalar, &v);
-   if (mask->dtype != OcDTypeBool || !same_shape(tensor, mask)) return OcErrorMessage("Masked fill needs a Boolean mask of the tensor's shape");
+   if (mask->dtype != OcDTypeBool || !same_shape(tensor, mask)) OcError(-1, "Masked fill needs a Boolean mask of the tensor's shape");
    if (activate(tensor->device) != 0 || OcTensor_startRead(tensor, mask) != 0) return -1;
    OCH_CALL(och_masked_fill(tensor->dtype, tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), mask->strides, OcTensor_data(mask), v, GPU_STREAM(tensor)));
    if (OcTensor_update(tensor) != 0) return -1;
@@ -276,13 +316,13 @@ static int OcTensorGPU_addIfNegative(OcTensor *tensor, OcScalar *scalar)
 }
 /* tensor: nstrides x nelem indices; offsets: nelem int64 values */
 static int OcTensorGPU_indexToOffset(OcTensor *tensor, OcInt64 *strides, OcTensor *offsets)
-{  int nstrides = (tensor->ndims >= 1) ? (int)tensor->size[0] : 1;
-   OcSize nelem = (tensor->ndims >= 2) ? tensor->size[1] : 1;
-   if (offsets->dtype != OcDTypeInt64) return OcErrorMessage("Offsets must be int64");
+{  OcIndex stride1, strideReduce; OcSize nelem; int nstrides;
+   if (offsets->dtype != OcDTypeInt64) OcError(-1, "Offsets must be int64");
+   if (tensor->ndims == 1) { stride1 = tensor->strides[0]; strideReduce = 0; nstrides = 1; nelem = tensor->size[0]; }      /* one index per element */
+   else { stride1 = tensor->strides[1]; strideReduce = tensor->strides[0]; nstrides = (int)tensor->size[0]; nelem = tensor->size[1]; }
    if (activate(tensor->device) != 0 || OcTensor_startRead(offsets, tensor) != 0) return -1;
-   OCH_CALL(och_index_to_offset(tensor->dtype, nstrides, (const int64_t *)strides, tensor->ndims >= 1 ? tensor->strides[0] : 0, (size_t)nelem,
-                                tensor->ndims >= 2 ? tensor->strides[1] : 0, OcTensor_data(tensor),
-                                offsets->ndims >= 1 ? offsets->strides[0] : 0, OcTensor_data(offsets), GPU_STREAM(offsets)));
+   OCH_CALL(och_index_to_offset(tensor->dtype, nstrides, (const int64_t *)strides, strideReduce, (size_t)nelem, stride1, OcTensor_data(tensor),
+                                offsets->strides[0], OcTensor_data(offsets), GPU_STREAM(offsets)));
    if (OcTensor_update(offsets) != 0) return -1;
    return OcTensor_finishRead(offsets, tensor);
 }
@@ -291,28 +331,41 @@ static int index_tables(OcTensorIndexView *view, int64_t **tables)
    for (d = 0; d < view->ndims; d++) tables[d] = (view->offsets && view->offsets[d]) ? (int64_t *)OcTensor_data(view->offsets[d]) : NULL;
    return 0;
 }
+/* the offset tables are tensors with storages (and streams) of their own, written by indexToOffset: the launch is
+   ordered behind their writers and they are released to later writers afterwards (tensor_index_gpu.c:155-172, 199-216, 248-260) */
+static int index_start(OcTensorIndexView *view, OcTensor *target)
+{  int d;
+   for (d = 0; d < view->ndims; d++) if (view->offsets && view->offsets[d] && OcTensor_startRead(target, view->offsets[d]) != 0) return -1;
+   return 0;
+}
+static int index_finish(OcTensorIndexView *view, OcTensor *target)
+{  int d;
+   for (d = 0; d < view->ndims; d++) if (view->offsets && view->offsets[d] && OcTensor_finishRead(target, view->offsets[d]) != 0) return -1;
+   return 0;
+}
 static int OcTensorGPU_getIndex(OcTensorIndexView *view, OcTensor *dst)
 {  int64_t *tables[OC_TENSOR_MAX_DIMS]; OcTensor *v = view->view;
    index_tables(view, tables);
-   if (activate(dst->device) != 0 || OcTensor_startRead(dst, v) != 0) return -1;
+   if (activate(dst->device) != 0 || OcTensor_startRead(dst, v) != 0 || index_start(view, dst) != 0) return -1;
    OCH_CALL(och_get_index(v->dtype, view->ndims, SZ(v), tables, v->strides, OcTensor_data(v), dst->strides, OcTensor_data(dst), GPU_STREAM(dst)));
-   if (OcTensor_update(dst) != 0) return -1;
-   return OcTensor_finishRead(dst, v);
+   if (OcTensor_update(dst) != 0 || OcTensor_finishRead(dst, v) != 0) return -1;
+   return index_finish(view, dst);
 }
 static int OcTensorGPU_setIndex(OcTensorIndexView *view, OcTensor *src)
 {  int64_t *tables[OC_TENSOR_MAX_DIMS]; OcTensor *v = view->view;
    index_tables(view, tables);
-   if (activate(v->device) != 0 || OcTensor_startRead(v, src) != 0) return -1;
+   if (activate(v->device) != 0 || OcTensor_startRead(v, src) != 0 || index_start(view, v) != 0) return -1;
    OCH_CALL(och_set_index(v->dtype, view->ndims, SZ(v), tables, v->strides, OcTensor_data(v), src->strides, OcTensor_data(src), GPU_STREAM(v)));
-   if (OcTensor_update(v) != 0) return -1;
-   return OcTensor_finishRead(v, src);
+   if (OcTensor_update(v) != 0 || OcTensor_finishRead(v, src) != 0) return -1;
+   return index_finish(view, v);
 }
 static int OcTensorGPU_fillIndex(OcTensorIndexView *view, OcScalar *scalar)
 {  int64_t *tables[OC_TENSOR_MAX_DIMS]; OcTensor *v = view->view; och_scalar val; scalar_value(scalar, &val);
    index_tables(view, tables);
-   if (activate(v->device) != 0) return -1;
+   if (activate(v->device) != 0 || index_start(view, v) != 0) return -1;
    OCH_CALL(och_fill_index(v->dtype, view->ndims, SZ(v), tables, v->strides, OcTensor_data(v), val, GPU_STREAM(v)));
-   return OcTensor_update(v);
+   if (OcTensor_update(v) != 0) return -1;
+   return index_finish(view, v);
 }
 
 /* Positions of the non-zero elements of a bool tensor (the reference implements these on the CPU only,
@@ -322,19 +375,22 @@ static OcTensor *find_common(OcTensor *tensor, OcIndex *multiplier)
 {  OcStorage *work; OcTensor *result = NULL; size_t nnz = 0; OcSize rsize[2]; int64_t mult[OC_TENSOR_MAX_DIMS]; int i;
    if (tensor->dtype != OcDTypeBool) { OcErrorMessage("Find requires a Boolean tensor"); return NULL; }
    if (activate(tensor->device) != 0) return NULL;
-   work = OcStorageGPU_create((OcSize)och_find_workspace_size((size_t)tensor->nelem), OcDTypeInt8, tensor->device, tensor->storage->stream);
+   /* the counts are produced and read on the tensor's stream */
+   work = OcStorage_createWithStream((OcSize)och_find_workspace_size((size_t)tensor->nelem), OcDTypeInt8, tensor->storage->stream);
    if (work == NULL) return NULL;
    if (och_find_count(tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), work->data, &nnz, GPU_STREAM(tensor)) != 0)
    {  OcErrorMessage("%s", och_last_error()); goto final; }
+   if (OcStorage_update(work) != 0) goto final;
    if (multiplier) { rsize[0] = (OcSize)nnz; result = OcTensor_create(1, rsize, NULL, OcDTypeInt64, tensor->device); }
    else { rsize[0] = tensor->ndims; rsize[1] = (OcSize)nnz; result = OcTensor_create(2, rsize, NULL, OcDTypeInt64, tensor->device); }
    if (result == NULL) goto final;
    for (i = 0; multiplier && i < tensor->ndims; i++) mult[i] = multiplier[i];
-   if (OcTensor_startRead(result, tensor) != 0 ||
-       och_find_apply(tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), work->data, multiplier ? mult : NULL,
+   if (OcTensor_startRead(result, tensor) != 0 || OcStorage_startRead(result->storage, work) != 0) { OcDecrefTensor(result); result = NULL; goto final; }
+   if (och_find_apply(tensor->ndims, SZ(tensor), tensor->strides, OcTensor_data(tensor), work->data, multiplier ? mult : NULL,
                       (int64_t *)OcTensor_data(result), GPU_STREAM(result)) != 0)
    {  OcErrorMessage("%s", och_last_error()); OcDecrefTensor(result); result = NULL; goto final; }
-   OcTensor_update(result); OcTensor_finishRead(result, tensor);
+   if (OcTensor_update(result) != 0 || OcTensor_finishRead(result, tensor) != 0 || OcStorage_finishRead(result->storage, work) != 0)
+   {  OcDecrefTensor(result); result = NULL; }
 final:
    OcDecrefStorage(work);
    return result;
@@ -344,19 +400,19 @@ static OcTensor *OcTensorGPU_maskToOffset(OcTensor *tensor, OcIndex *strides) { 
 
 /* ---- elementwise (op/tensor_unary_gpu.c:59-93, op/tensor_binary_gpu.c:58-97) ------------ */
 static int unary_call(int op, const char *name, OcTensor *src, OcTensor *dst)
-{  if (!och_unary_supported(op, src->dtype)) return OcErrorMessage("Function %s is not supported for type %s on GPU", name, OcDType_name(src->dtype));
-   if ((int)dst->dtype != och_unary_result_dtype(op, src->dtype)) return OcErrorMessage("Invalid destination type in %s", name);
-   if (!same_shape(src, dst)) return OcErrorMessage("Mismatch in tensor sizes in %s", name);
+{  if (!och_unary_supported(op, src->dtype)) OcError(-1, "Function %s is not supported for type %s on GPU", name, OcDType_name(src->dtype));
+   if ((int)dst->dtype != och_unary_result_dtype(op, src->dtype)) OcError(-1, "Invalid destination type in %s", name);
+   if (!same_shape(src, dst)) OcError(-1, "Mismatch in tensor sizes in %s", name);
    if (activate(dst->device) != 0 || OcTensor_startRead(dst, src) != 0) return -1;
    OCH_CALL(och_unary(op, src->dtype, dst->ndims, SZ(dst), src->strides, OcTensor_data(src), dst->strides, OcTensor_data(dst), GPU_STREAM(dst)));
    if (OcTensor_update(dst) != 0) return -1;
    return OcTensor_finishRead(dst, src);
 }
 static int binary_call(int op, const char *name, OcTensor *src1, OcTensor *src2, OcTensor *dst)
-{  if (!och_binary_supported(op, src1->dtype)) return OcErrorMessage("Function %s is not supported for type %s on GPU", name, OcDType_name(src1->dtype));
+{  if (!och_binary_supported(op, src1->dtype)) OcError(-1, "Function %s is not supported for type %s on GPU", name, OcDType_name(src1->dtype));
    if ((int)src2->dtype != och_binary_operand2_dtype(op, src1->dtype) || (int)dst->dtype != och_binary_result_dtype(op, src1->dtype))
-      return OcErrorMessage("Invalid operand types in %s", name);
-   if (!same_shape(src1, dst) || !same_shape(src2, dst)) return OcErrorMessage("Mismatch in tensor sizes in %s", name);
+      OcError(-1, "Invalid operand types in %s", name);
+   if (!same_shape(src1, dst) || !same_shape(src2, dst)) OcError(-1, "Mismatch in tensor sizes in %s", name);
    if (activate(dst->device) != 0 || OcTensor_startRead(dst, src1) != 0 || OcTensor_startRead(dst, src2) != 0) return -1;
    OCH_CALL(och_binary(op, src1->dtype, dst->ndims, SZ(dst), src1->strides, OcTensor_data(src1), src2->strides, OcTensor_data(src2),
                        dst->strides, OcTensor_data(dst), GPU_STREAM(dst)));
@@ -374,8 +430,8 @@ OC_BINARY_TABLE(OC_X)
 /* ---- full reductions (op/tensor_reduce_all_gpu.c:201-444) --------------------------------- */
 static int reduce_call(int op, OcTensor *tensor, OcScalar *lower, OcScalar *upper, double p, void *result)
 {  och_scalar b1, b2;
-   if (!och_reduce_supported(op, tensor->dtype)) return OcErrorMessage("Reduction is not supported for type %s on GPU", OcDType_name(tensor->dtype));
-   if (OcTensor_isByteswapped(tensor)) return OcErrorMessage("Reductions need native byte order");
+   if (!och_reduce_supported(op, tensor->dtype)) OcError(-1, "Reduction is not supported for type %s on GPU", OcDType_name(tensor->dtype));
+   if (OcTensor_isByteswapped(tensor)) OcError(-1, "Reductions need native byte order");
    if (lower) scalar_value(lower, &b1);
    if (upper) scalar_value(upper, &b2);
    if (activate(tensor->device) != 0) return -1;
@@ -419,16 +475,17 @@ static int OcTensorGPU_normNaN(OcTensor *t, double p, OcScalar *result) { return
 /* ---- axis reductions (op/tensor_reduce_axis_gpu.c:108-281) --------------------------------- */
 static int axis_call(int op, OcTensor *src, double p, int n, int *axes, OcTensor *dst)
 {  OcSolidReduceAxis a; och_reduce_axis_config c; int i;
-   if (!och_reduce_supported(op, src->dtype)) return OcErrorMessage("Axis reduction is not supported for type %s on GPU", OcDType_name(src->dtype));
-   if ((int)dst->dtype != och_reduce_result_dtype(op, src->dtype)) return OcErrorMessage("Invalid destination type in axis reduction");
-   if (OcTensor_isByteswapped(src) || OcTensor_isByteswapped(dst)) return OcErrorMessage("Axis reductions need native byte order");
+   memset(&a, 0, sizeof(a));
+   if (!och_reduce_supported(op, src->dtype)) OcError(-1, "Axis reduction is not supported for type %s on GPU", OcDType_name(src->dtype));
+   if ((int)dst->dtype != och_reduce_result_dtype(op, src->dtype)) OcError(-1, "Invalid destination type in axis reduction");
+   if (OcTensor_isByteswapped(src) || OcTensor_isByteswapped(dst)) OcError(-1, "Axis reductions need native byte order");
    if (dst->nelem == 0) return 0;
-   if (OcSolid_analyzeReduceAxis(src, n, axes, dst, &a) != 0) return -1;
+   OcSolid_analyzeReduceAxis(&a, src, dst, n, axes, 0);
    memset(&c, 0, sizeof(c));
    c.ndims = a.ndims; c.rdims = a.rdims;
    for (i = 0; i < a.ndims; i++) { c.size[i] = (size_t)a.size[i]; c.strides1[i] = a.strides1[i]; c.strides2[i] = a.strides2[i]; }
    for (i = 0; i < a.rdims; i++) { c.rsize[i] = (size_t)a.rsize[i]; c.rstrides[i] = a.rstrides[i]; }
-   c.ptr1 = OcTensor_data(src) + a.offset1; c.ptr2 = OcTensor_data(dst) + a.offset2; c.stream = GPU_STREAM(dst);
+   c.ptr1 = a.ptr1; c.ptr2 = a.ptr2; c.stream = GPU_STREAM(dst);
    if (activate(dst->device) != 0 || OcTensor_startRead(dst, src) != 0) return -1;
    OCH_CALL(och_reduce_axis(op, src->dtype, &c, p));
    if (OcTensor_update(dst) != 0) return -1;
@@ -447,7 +504,7 @@ static int OcTensorGPU_gemm(OcSize M, OcSize N, OcSize K, char transA, char tran
    char *pa = OcTensor_data(alpha), *pb = OcTensor_data(beta), *pA = OcTensor_data(A), *pB = OcTensor_data(B), *pC = OcTensor_data(C);
    if (C->nelem == 0) return 0;
    if (K == 0) { ldA = N; ldB = M; }
-   if (!och_gemm_supported(A->dtype)) return OcErrorMessage("Unsupported data type in function gpu gemm (%s)", OcDType_name(A->dtype));
+   if (!och_gemm_supported(A->dtype)) OcError(-1, "Unsupported data type in function gpu gemm (%s)", OcDType_name(A->dtype));
    if (activate(A->device) != 0) return -1;
    /* the reference loops over the dimensions beyond the second (tensor_blas_gpu.c:171-252); here they are one batched launch */
    {  size_t bsize[OC_TENSOR_MAX_DIMS]; ptrdiff_t sa[OC_TENSOR_MAX_DIMS], sb[OC_TENSOR_MAX_DIMS], sA[OC_TENSOR_MAX_DIMS], sB[OC_TENSOR_MAX_DIMS], sC[OC_TENSOR_MAX_DIMS];
@@ -470,17 +527,17 @@ static int OcTensorGPU_gemmSupportedOn(OcDevice *device, OcDType dtype) { (void)
    elements, r NULL or a dense vector of k elements that receives the coefficients; all on the same GPU, same type */
 int OcTensorGPU_projectColumns(OcTensor *Q, OcTensor *v, OcTensor *r)
 {  OcSize n, k; OcIndex es;
-   if (Q == NULL || v == NULL) return OcErrorMessage("projectColumns: missing operand");
+   if (Q == NULL || v == NULL) OcError(-1, "projectColumns: missing operand");
    es = OcDType_size(Q->dtype);
    if (!OcDeviceGPU_isInstance(Q->device) || v->device != Q->device || (r && r->device != Q->device))
-      return OcErrorMessage("projectColumns: all tensors must be on the same GPU device");
-   if (v->dtype != Q->dtype || (r && r->dtype != Q->dtype)) return OcErrorMessage("projectColumns: mismatch in data types");
-   if (Q->ndims < 1 || Q->ndims > 2 || v->ndims != 1) return OcErrorMessage("projectColumns: Q must be a matrix and v a vector");
+      OcError(-1, "projectColumns: all tensors must be on the same GPU device");
+   if (v->dtype != Q->dtype || (r && r->dtype != Q->dtype)) OcError(-1, "projectColumns: mismatch in data types");
+   if (Q->ndims < 1 || Q->ndims > 2 || v->ndims != 1) OcError(-1, "projectColumns: Q must be a matrix and v a vector");
    n = Q->size[0]; k = (Q->ndims == 2) ? Q->size[1] : 1;
-   if (v->size[0] != n || (r && (r->ndims != 1 || r->size[0] != k))) return OcErrorMessage("projectColumns: mismatch in tensor sizes");
+   if (v->size[0] != n || (r && (r->ndims != 1 || r->size[0] != k))) OcError(-1, "projectColumns: mismatch in tensor sizes");
    if ((n > 1 && (Q->strides[0] != es || v->strides[0] != es)) || (r && k > 1 && r->strides[0] != es) ||
        (Q->ndims == 2 && k > 1 && (Q->strides[1] % es != 0 || Q->strides[1] < (OcIndex)(n * es))))
-      return OcErrorMessage("projectColumns: columns and vectors must be dense");
+      OcError(-1, "projectColumns: columns and vectors must be dense");
    if (n == 0 || k == 0) return 0;
    if (activate(v->device) != 0 || OcTensor_startRead(v, Q) != 0) return -1;
    if (r && OcTensor_startRead(v, r) != 0) return -1;             /* r is written on v's stream: order it behind r's own work */
@@ -491,22 +548,29 @@ int OcTensorGPU_projectColumns(OcTensor *Q, OcTensor *v, OcTensor *r)
    return OcTensor_finishRead(v, Q);
 }
 
-/* ---- module table and registration ------------------------------------------------------------ */
-static int gpu_initialize_context(OcDevice *device, OcDeviceModule *module, void **context)
-{  OcModuleCore_Context *ctx = (OcModuleCore_Context *)calloc(1, sizeof(OcModuleCore_Context));
-   (void)device; (void)module;
-   if (ctx == NULL) return OcErrorMessage("Insufficient memory for the module context");
-   ctx->scalarCount = 8;
-   *context = ctx;
-   return 0;
+/* ---- module table and registration (module_core_gpu.c:40-145) ------------------------------------ */
+static int initializeContext(OcDevice *device, OcDeviceModule *deviceModule, void **context)
+{  OcModuleCoreGPU_Context *ctx;
+   (void)deviceModule;
+   /* assigned first, so that a partial initialisation is cleaned up by finalizeContext; the interface's part of the
+      context holds the ring of temporary storages and the scalar slots (module_core.c:52-79) */
+   *context = (void *)OcModuleCore_createContext(device, sizeof(OcModuleCoreGPU_Context));
+   if ((ctx = (OcModuleCoreGPU_Context *)(*context)) == NULL) return -1;
+   ctx->deviceIndex = device->index;
+   return activate(device);
 }
-static void gpu_finalize_context(OcDevice *device, OcDeviceModule *module, void *context) { (void)device; (void)module; free(context); }
-static void gpu_finalize_module(OcDeviceModule *module) { (void)module; }
+static void finalizeContext(OcDevice *device, OcDeviceModule *deviceModule, void *context)
+{  (void)deviceModule;
+   if (context == NULL) return;
+   och_device_set(device->index); och_device_synchronize();        /* the temporaries may still be in use */
+   OcModuleCore_freeContext((OcModuleCore_Context *)context);
+}
+static void finalizeModule(OcDeviceModule *deviceModule) { (void)deviceModule; }
 
-static void fill_table(OcModuleCore *m)
+static void initializeFunctions(OcModuleCore *m)
 {  memset(m, 0, sizeof(*m));
-   m->HEAD.available = 1;
-   m->HEAD.initializeContext = gpu_initialize_context; m->HEAD.finalizeContext = gpu_finalize_context; m->HEAD.finalizeModule = gpu_finalize_module;
+   m->HEAD.module = &oc_module_core;               /* registration increments its reference count */
+   m->HEAD.initializeContext = initializeContext; m->HEAD.finalizeContext = finalizeContext; m->HEAD.finalizeModule = finalizeModule;
    m->Device_formatInfo = OcDeviceGPU_formatInfo;
    m->Buffer_copy = OcBufferGPU_copy; m->Buffer_copyFromCPU = OcBufferGPU_copyFromCPU; m->Buffer_copyToCPU = OcBufferGPU_copyToCPU;
    m->Buffer_copyHostStorage = OcBufferGPU_copyHostStorage; m->Buffer_copyStorageHost = OcBufferGPU_copyStorageHost; m->Buffer_zero = OcBufferGPU_zero;
@@ -533,25 +597,9 @@ static void fill_table(OcModuleCore *m)
    m->Tensor_gemm = OcTensorGPU_gemm; m->Tensor_gemmSupportedOn = OcTensorGPU_gemmSupportedOn;
 }
 
-/* device_module.c:313-422: the size must match the interface's view of the table; the table is copied */
-int OcRegisterModule(const char *deviceType, OcDeviceModule *info, size_t size)
-{  if (strcmp(deviceType, "GPU") != 0) return OcErrorMessage("This host registers the GPU device type only (got %s)", deviceType);
-   if (size != sizeof(OcModuleCore)) return OcErrorMessage("Mismatch in device module size (%zu, expected %zu)", size, sizeof(OcModuleCore));
-   memcpy(&oc_registered_gpu, info, size);
-   oc_registered = 1;
-   return 0;
-}
-OcModuleCore *OcModuleCore_forDevice(OcDevice *device)
-{  if (device == NULL || device == OcCPU || !oc_registered) return NULL;
-   return &oc_registered_gpu;
-}
 int OcDeviceGPUCount(void) { return oc_gpu_count; }
 OcDevice *OcDeviceGPUByIndex(int index) { return (index >= 0 && index < oc_gpu_count) ? OcGPU[index] : NULL; }
-int OcDeviceGPU_isInstance(OcDevice *device)
-{  int i;
-   for (i = 0; i < oc_gpu_count; i++) if (OcGPU[i] == device) return 1;
-   return 0;
-}
+int OcDeviceGPU_isInstance(OcDevice *device) { return (device != NULL && oc_device_type_gpu != NULL && device->type == oc_device_type_gpu); }
 int OcDeviceGPU_peerAccess(int device1, int device2)
 {  int result = 0;
    if (device1 == device2) return 1;
@@ -560,50 +608,68 @@ int OcDeviceGPU_peerAccess(int device1, int device2)
 }
 int OcDeviceGPU_properties(OcDevice *device, void *och_device_prop_out)
 {  OcDeviceGPU *g = (OcDeviceGPU *)device; size_t total = 0;
-   if (!OcDeviceGPU_isInstance(device) || och_device_prop_out == NULL) return OcErrorMessage("Device properties: not a GPU device");
+   if (!OcDeviceGPU_isInstance(device) || och_device_prop_out == NULL) OcError(-1, "Device properties: not a GPU device");
    OCH_CALL(och_device_mem_info(device->index, &g->properties.free_global_mem, &total));
    memcpy(och_device_prop_out, &g->properties, sizeof(g->properties));
    return 0;
 }
-
-int OcInitGPU(void)
-{  int i, count = 0;
-   if (oc_gpu_initialized) return 0;
-   if (och_device_count(&count) != 0) return OcErrorMessage("%s", och_last_error());
-   OcGPU = (OcDevice **)calloc((size_t)(count > 0 ? count : 1), sizeof(OcDevice *));
-   if (OcGPU == NULL) return OcErrorMessage("Insufficient memory for the device list");
-   for (i = 0; i < count; i++)
-   {  OcDeviceGPU *g = (OcDeviceGPU *)calloc(1, sizeof(OcDeviceGPU)); char name[32];
-      if (g == NULL) return OcErrorMessage("Insufficient memory for the device object");
-      snprintf(name, sizeof(name), "gpu%d", i);
-      g->HEAD.index = i; g->HEAD.name = strdup(name); g->HEAD.endianness = 0; g->HEAD.requiresAlignedData = 1; g->HEAD.refcount = 1;
-      g->HEAD.create_stream = gpu_create_stream; g->HEAD.create_event = gpu_create_event; g->HEAD.delete_stream = gpu_delete_stream;
-      g->HEAD.delete_event = gpu_delete_event; g->HEAD.sync_stream = gpu_sync_stream; g->HEAD.sync_event = gpu_sync_event;
-      g->HEAD.record_event = gpu_record_event; g->HEAD.wait_event = gpu_wait_event; g->HEAD.finalize = gpu_finalize_device;
-      if (och_device_properties(i, &g->properties) != 0) return OcErrorMessage("%s", och_last_error());
-      if (och_device_warmup(i) != 0) return OcErrorMessage("%s", och_last_error());          /* device_gpu.c:155-196 */
-      OcGPU[i] = &g->HEAD;
-      if ((g->HEAD.defaultStream = gpu_create_stream(&g->HEAD)) == NULL) return -1;
-      g->HEAD.contextBuffer = (void **)calloc(1, sizeof(void *)); g->HEAD.contextSize = g->HEAD.contextCapacity = 1;
-   }
-   oc_gpu_count = count;
-   fill_table(&oc_module_core_gpu);
-   if (OcRegisterModule("GPU", (OcDeviceModule *)&oc_module_core_gpu, sizeof(OcModuleCore)) != 0) return -1;
-   for (i = 0; i < count; i++)
-      if (oc_registered_gpu.HEAD.initializeContext(OcGPU[i], &oc_registered_gpu.HEAD, &OcGPU[i]->contextBuffer[0]) != 0) return -1;
-   oc_gpu_initialized = 1;
+/* events recorded, stream waits issued and streams created on a GPU device since it was created (no counterpart in the
+   reference): what a test needs to see that operands on different streams really go through the event protocol */
+int OcDeviceGPU_activity(OcDevice *device, long *eventsRecorded, long *eventsWaited, long *streamsCreated)
+{  OcDeviceGPU *g = (OcDeviceGPU *)device;
+   if (!OcDeviceGPU_isInstance(device)) OcError(-1, "Device activity: not a GPU device");
+   if (eventsRecorded) *eventsRecorded = g->eventsRecorded;
+   if (eventsWaited) *eventsWaited = g->eventsWaited;
+   if (streamsCreated) *streamsCreated = g->streamsCreated;
    return 0;
 }
-void OcFinalizeGPU(void)
+
+/* device_gpu.c:196-250 */
+static void OcFinalizeDevicesGPU(void)
 {  int i;
-   if (!oc_gpu_initialized) return;
-   for (i = 0; i < oc_gpu_count; i++)
-   {  OcDevice *d = OcGPU[i];
-      och_device_set(i); och_device_synchronize();
-      oc_registered_gpu.HEAD.finalizeContext(d, &oc_registered_gpu.HEAD, d->contextBuffer[0]);
-      gpu_delete_stream(d->defaultStream);
-      d->finalize(d);
-      free(d->contextBuffer); free(d->name); free(d);
+   if (oc_device_type_gpu) { OcDecrefDeviceType(oc_device_type_gpu); oc_device_type_gpu = NULL; }
+   if (OcGPU != NULL)
+   {  for (i = 0; i < oc_gpu_count; i++)
+         if (OcGPU[i] != NULL) { och_device_set(i); och_device_synchronize(); OcDecrefDevice(OcGPU[i]); OcGPU[i] = NULL; }
+      OcFree(OcGPU); OcGPU = NULL;
    }
-   free(OcGPU); OcGPU = NULL; oc_gpu_count = 0; oc_gpu_initialized = 0; oc_registered = 0;
+   oc_gpu_count = 0;
+}
+static int OcInitDevicesGPU(void)
+{  OcDeviceType *type; OcDevice *device; char name[16]; int count = 0, index;
+   if (och_device_count(&count) != 0) count = 0;
+   if ((type = OcCreateDeviceType("GPU")) == NULL) return -1;
+   oc_device_type_gpu = OcIncrefDeviceType(type);
+   if (count > 0)
+   {  if ((OcGPU = (OcDevice **)OcMalloc(sizeof(OcDevice *) * (size_t)count)) == NULL) OcError(-1, "Error allocating GPU device buffer");
+      for (index = 0; index < count; index++) OcGPU[index] = NULL;
+   }
+   oc_gpu_count = count;
+   for (index = 0; index < count; index++)
+   {  snprintf(name, sizeof(name), "gpu%d", index);
+      device = OcCreateDeviceGPU(type, index, name);
+      if (device != NULL && OcRegisterDevice(device) == 0) OcGPU[index] = device;       /* the creation reference is the list's */
+      else { if (device) OcDecrefDevice(device); OcFinalizeDevicesGPU(); return -1; }
+   }
+   return 0;
+}
+/* module_core_gpu.c:127-145 */
+static int OcInitModuleCore_GPU(void)
+{  if (OcModuleCore_initialize() != 0) return -1;
+   initializeFunctions(&oc_module_core_gpu);
+   return OcRegisterModule("GPU", (OcDeviceModule *)&oc_module_core_gpu, sizeof(oc_module_core_gpu));
+}
+void OcFinalizeGPU(void)
+{  if (!oc_gpu_initialized) return;
+   oc_gpu_initialized = 0;
+   OcFinalizeDevicesGPU();
+}
+/* ocean_gpu.c:38-58: the devices first, then the module (registration creates the module's context on every
+   device of the type that exists, device_module.c:388-405) */
+int OcInitGPU(void)
+{  if (oc_gpu_initialized) return 0;
+   if (OcInitDevicesGPU() != 0) return -1;
+   if (OcInitModuleCore_GPU() != 0) { OcFinalizeDevicesGPU(); return -1; }
+   oc_gpu_initialized = 1;
+   return OcFinalizeAddHandler(OcFinalizeGPU, "Finalize Ocean GPU");
 }

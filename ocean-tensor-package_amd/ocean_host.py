@@ -57,8 +57,9 @@ def scalar(dtype, value):
 
 
 class ReduceAxis(C.Structure):
-    _fields_ = [("ndims", C.c_int), ("size", C.c_ssize_t * 8), ("strides1", C.c_ssize_t * 8), ("strides2", C.c_ssize_t * 8),
-                ("rdims", C.c_int), ("rsize", C.c_ssize_t * 8), ("rstrides", C.c_ssize_t * 8), ("offset1", C.c_ssize_t), ("offset2", C.c_ssize_t)]
+    """OcSolidReduceAxis (include/ocean/external/ocean-solid/ocean_solid.h:73-83)."""
+    _fields_ = [("ndims", C.c_int), ("rdims", C.c_int), ("size", C.c_size_t * 8), ("rsize", C.c_size_t * 8), ("strides1", C.c_ssize_t * 8),
+                ("strides2", C.c_ssize_t * 8), ("rstrides", C.c_ssize_t * 8), ("ptr1", C.c_void_p), ("ptr2", C.c_void_p)]
 
 
 TP = C.POINTER(Tensor)
@@ -90,7 +91,13 @@ lib.OcTensor_find.restype = TP
 lib.OcTensor_find.argtypes = [TP]
 lib.OcTensor_maskToOffset.restype = TP
 lib.OcTensor_maskToOffset.argtypes = [TP, _ss]
-lib.OcSolid_analyzeReduceAxis.argtypes = [TP, C.c_int, C.POINTER(C.c_int), TP, C.POINTER(ReduceAxis)]
+lib.OcSolid_analyzeReduceAxis.restype = None
+lib.OcSolid_analyzeReduceAxis.argtypes = [C.POINTER(ReduceAxis), TP, TP, C.c_int, C.POINTER(C.c_int), C.c_int]
+lib.OcShape_extent.argtypes = [C.c_int, _ss, _ss, C.c_ssize_t, _ss, _ss]
+lib.OcDeviceGPU_activity.argtypes = [C.c_void_p, C.POINTER(C.c_long), C.POINTER(C.c_long), C.POINTER(C.c_long)]
+lib.OcFinalize.restype = None
+lib.OcShape_sortStrides2.restype = None
+lib.OcShape_mergeBlocks2.restype = None
 lib.OcShape_sortStrides2.argtypes = [C.c_int, _ss, _ss, _ss]
 lib.OcShape_mergeBlocks2.argtypes = [C.POINTER(C.c_int), _ss, _ss, _ss]
 

@@ -320,3 +320,115 @@ def test_negative_of_unsigned_takes_the_signed_type(gpu):
         host.check(host.lib.OcTensor_unary(oh.U["negative"], t, C.byref(out)))
         assert out.contents.dtype == want_dt
         assert np.array_equal(host.to_numpy(out), -np.arange(5).astype(want_np))
+
+
+def _activity(gpu):
+    rec, wait, streams = C.c_long(), C.c_long(), C.c_long()
+    host.check(host.lib.OcDeviceGPU_activity(gpu, C.byref(rec), C.byref(wait), C.byref(streams)))
+    return rec.value, wait.value, streams.value
+
+
+def test_every_storage_has_its_own_stream_and_operations_are_ordered_by_events(gpu):
+    """The reference gives every GPU storage a stream of its own (no default stream on GPU devices, storage.c:94-103)
+    and orders operations by the read / write protocol alone (storage.c:141-222). Here the operands of a binary
+    operation, a copy, an axis reduction and a GEMM all live on different streams, and every step is followed at once
+    by an operation on ANOTHER stream that overwrites one of its inputs: without the event protocol (startRead /
+    update / finishRead) the overwrite overtakes the reader and the results below are wrong. Sizes are large enough
+    (64 MB per tensor) that the readers are still running when the overwrites are issued."""
+    rng = np.random.default_rng(31)
+    n = 2896                                                                    # n * n doubles = 64 MB
+    X, Y = rng.uniform(-1, 1, (n, n)), rng.uniform(-1, 1, (n, n))
+    rec0, wait0, _ = _activity(gpu)
+    tx, ty = host.from_numpy(X, host.DOUBLE, gpu), host.from_numpy(Y, host.DOUBLE, gpu)
+    streams = {tx.contents.storage.contents.stream, ty.contents.storage.contents.stream}
+    assert None not in streams and len(streams) == 2
+    seven, three = host.scalar(host.DOUBLE, 7.0), host.scalar(host.DOUBLE, 3.0)
+    for rep in range(3):
+        # binary operation on z's stream, then its first input overwritten on that input's own stream
+        z = binary(ADD, tx, ty)
+        assert z.contents.storage.contents.stream not in streams
+        host.check(host.lib.OcTensor_fill(tx, C.byref(seven)))
+        # copy (with a cast) out of z on the copy's stream, then z overwritten
+        c = host.create([n, n], host.FLOAT, gpu)
+        host.check(host.lib.OcTensor_copy(z, c))
+        host.check(host.lib.OcTensor_fill(z, C.byref(three)))
+        # axis reduction of the copy into a tensor on yet another stream, then the copy overwritten
+        r = host.TP()
+        host.check(host.lib.OcTensor_axisReduce(15, c, 1, (C.c_int * 1)(0), 0, 0.0, C.byref(r)))
+        host.check(host.lib.OcTensor_fill(c, C.byref(host.scalar(host.FLOAT, 1.0))))
+        z32 = (X + Y).astype(np.float32)                                         # the cast is exact arithmetic: one rounding
+        ref = z32.sum(axis=1, dtype=np.float64)
+        assert np.abs(host.to_numpy(r) - ref).max() <= 1e-5 * np.abs(z32).sum(axis=1, dtype=np.float64).max()
+        assert host.to_numpy(z).min() == 3.0 and host.to_numpy(tx).max() == 7.0 and host.to_numpy(c).max() == 1.0
+        # restore x for the next round (upload waits for the storage's outstanding work)
+        host.lib.OcDecrefTensor(tx)
+        tx = host.from_numpy(X, host.DOUBLE, gpu)
+        for t in (z, c, r):
+            host.lib.OcDecrefTensor(t)
+    # GEMM: C on its own stream reads A and B, which are overwritten right after the call
+    m = 1024
+    A, B = rng.uniform(-1, 1, (m, m)), rng.uniform(-1, 1, (m, m))
+    ta, tb = host.from_numpy(A, host.DOUBLE, gpu), host.from_numpy(B, host.DOUBLE, gpu)
+    c = host.TP()
+    host.check(host.lib.OcTensor_mtimes(ta, tb, C.byref(c)))
+    host.check(host.lib.OcTensor_fill(ta, C.byref(seven))); host.check(host.lib.OcTensor_fill(tb, C.byref(seven)))
+    want = (A.T @ B.T).T
+    assert np.linalg.norm(host.to_numpy(c) - want) <= 1e-13 * m * np.linalg.norm(want)
+    rec1, wait1, _ = _activity(gpu)
+    assert rec1 - rec0 >= 30 and wait1 - wait0 >= 30                            # the protocol really ran
+    for t in (tx, ty, ta, tb, c):
+        host.lib.OcDecrefTensor(t)
+
+
+def test_index_tables_on_their_own_streams(gpu):
+    """Gather and scatter through offset tables that were written just before, on storages (and streams) of their own,
+    by addIfNegative + indexToOffset: the gather must wait for the tables (tensor_index_gpu.c:155-172, 199-216)."""
+    rng = np.random.default_rng(32)
+    rows, cols, picks = 4096, 2048, 1 << 15
+    T = rng.uniform(-1, 1, (cols, rows))                                        # Ocean shape (rows, cols): dimension 0 fastest
+    idx = np.stack([rng.integers(-rows, rows, picks), rng.integers(-cols, cols, picks)], axis=1).astype(np.int64)   # Ocean [2, picks]
+    host.lib.OcTensor_getIndexed.argtypes = [host.TP, host.TP, C.POINTER(host.TP)]
+    host.lib.OcTensor_setIndexed.argtypes = [host.TP, host.TP, host.TP]
+    t, ti = host.from_numpy(T, host.DOUBLE, gpu), host.from_numpy(idx, host.INT64, gpu)
+    out = host.TP()
+    host.check(host.lib.OcTensor_getIndexed(t, ti, C.byref(out)))
+    got = host.to_numpy(out)
+    assert got.shape == (picks,) and np.array_equal(got, T[idx[:, 1], idx[:, 0]])
+    # scatter: distinct positions, so the result does not depend on the order of the writes
+    flat = rng.choice(rows * cols, picks, replace=False)
+    idx2 = np.stack([flat % rows, flat // rows], axis=1).astype(np.int64)
+    vals = rng.uniform(5, 6, picks)
+    ti2, tv = host.from_numpy(idx2, host.INT64, gpu), host.from_numpy(vals, host.DOUBLE, gpu)
+    host.check(host.lib.OcTensor_setIndexed(t, ti2, tv))
+    want = T.copy(); want[idx2[:, 1], idx2[:, 0]] = vals
+    assert np.array_equal(host.to_numpy(t), want)
+    # one indexed dimension, the rest of the tensor whole: rows of a matrix picked by (negative) column numbers
+    pick = np.array([[-1], [0], [5], [-cols]], dtype=np.int64)                  # Ocean [1, 4] ... indexes dimension 0
+    tp = host.from_numpy(pick, host.INT64, gpu)
+    out2 = host.TP()
+    host.check(host.lib.OcTensor_getIndexed(t, tp, C.byref(out2)))
+    sel = [rows - 1, 0, 5, rows - cols]
+    assert np.array_equal(host.to_numpy(out2), want[:, sel])
+    for x in (t, ti, out, ti2, tv, tp, out2):
+        host.lib.OcDecrefTensor(x)
+
+
+def test_temporaries_come_from_the_ring(gpu):
+    """Converted operands of a binary operation live in the device's ring of three temporary storages
+    (storage_itf.c:61-121): a long sequence of promoting operations creates no new streams once the ring is warm."""
+    rng = np.random.default_rng(33)
+    a = rng.integers(-100, 100, (512, 512)).astype(np.int32)
+    b = rng.uniform(-1, 1, (512, 512))
+    ta, tb = host.from_numpy(a, host.INT32, gpu), host.from_numpy(b, host.DOUBLE, gpu)
+    z = binary(ADD, ta, tb)
+    host.lib.OcDecrefTensor(z)
+    for _ in range(4):                                                         # warm the three slots
+        z = binary(ADD, ta, tb); host.lib.OcDecrefTensor(z)
+    _, _, streams0 = _activity(gpu)
+    for _ in range(60):
+        z = binary(ADD, ta, tb)
+        assert np.array_equal(host.to_numpy(z), a + b)
+        host.lib.OcDecrefTensor(z)
+    _, _, streams1 = _activity(gpu)
+    assert streams1 == streams0                                                # streams come back from the free list, temporaries from the ring
+    host.lib.OcDecrefTensor(ta); host.lib.OcDecrefTensor(tb)
