@@ -306,7 +306,9 @@ static int gemm_operand(OcTensor **t, char *mode, OcIndex *ld, int complex_type)
 }
 /* C <- alpha * op(A) * op(B) + beta * C on the first two dimensions; the dimensions beyond them index independent
    products and broadcast between A and B (size 1 or absent: shared), as in Ocean's interface (tensor_itf.c:6433-6750) */
-int OcTensor_gemm(OcScalar *alpha, OcTensor *A, char modeA, OcTensor *B, char modeB, OcScalar *beta, OcTensor **C)
+/* alphaT / betaT: NULL (then the OcScalar, or 1 and 0), or tensors of one element per product: dimensions 0 and 1 of
+   size 1, the dimensions beyond them broadcast with those of A and B (tensor_itf.c:6433-6470) */
+static int gemm_core(OcScalar *alpha, OcTensor *alphaT, OcTensor *A, char modeA, OcTensor *B, char modeB, OcScalar *beta, OcTensor *betaT, OcTensor **C)
 {  OcTensor *a = OcIncrefTensor(A), *b = OcIncrefTensor(B), *c = NULL, *ta = NULL, *tb = NULL, *v; int result = -1, i, nd;
    OcDevice *device = A->device != OcCPU ? A->device : B->device; OcDType dtype = OcDType_getCommonType(A->dtype, B->dtype), halftype = OcDTypeNone;
    OcSize M, N, K, K2, csize[OC_TENSOR_MAX_DIMS], asize[OC_TENSOR_MAX_DIMS], bsize[OC_TENSOR_MAX_DIMS]; OcIndex ldA, ldB, ldC; OcModuleCore *m = OcModuleCore_forDevice(device);
@@ -321,12 +323,21 @@ int OcTensor_gemm(OcScalar *alpha, OcTensor *A, char modeA, OcTensor *B, char mo
    K2 = (modeB == 'N') ? B->size[0] : B->size[1]; N = (modeB == 'N') ? B->size[1] : B->size[0];
    if (K != K2) { OcErrorMessage("Inner dimensions do not match (%td and %td)", K, K2); goto final; }
    nd = A->ndims > B->ndims ? A->ndims : B->ndims;
+   if (alphaT && alphaT->ndims > nd) nd = alphaT->ndims;
+   if (betaT && betaT->ndims > nd) nd = betaT->ndims;
    csize[0] = M; csize[1] = N;
    for (i = 2; i < nd; i++)
-   {  OcSize sa = i < A->ndims ? A->size[i] : 1, sb = i < B->ndims ? B->size[i] : 1;
-      if (sa != sb && sa != 1 && sb != 1) { OcErrorMessage("Dimension %d of the operands is not compatible (%td and %td)", i, sa, sb); goto final; }
-      csize[i] = (sa == 1) ? sb : sa;
+   {  OcTensor *ops[4] = { A, B, alphaT, betaT }; int k;
+      csize[i] = 1;
+      for (k = 0; k < 4; k++)
+      {  OcSize sk = (ops[k] && i < ops[k]->ndims) ? ops[k]->size[i] : 1;
+         if (sk != 1 && csize[i] != 1 && sk != csize[i]) { OcErrorMessage("Dimension %d of the operands is not compatible (%td and %td)", i, csize[i], sk); goto final; }
+         if (sk != 1) csize[i] = sk;
+      }
    }
+   for (i = 0; i < 2; i++)
+      if ((alphaT && i < alphaT->ndims && alphaT->size[i] != 1) || (betaT && i < betaT->ndims && betaT->size[i] != 1))
+      {  OcErrorMessage("The scalars of a matrix product must have size one in the first two dimensions"); goto final; }
    if (OcTensor_ensure(&a, dtype, device) != 0 || OcTensor_ensure(&b, dtype, device) != 0) goto final;
    if (gemm_operand(&a, &modeA, &ldA, OcDType_isComplex(dtype)) != 0 || gemm_operand(&b, &modeB, &ldB, OcDType_isComplex(dtype)) != 0) goto final;
    /* all operands get the same number of dimensions; shared ones have stride zero */
@@ -354,11 +365,25 @@ int OcTensor_gemm(OcScalar *alpha, OcTensor *A, char modeA, OcTensor *B, char mo
       }
    }
    ldC = (N > 1) ? c->strides[1] / c->elemsize : (M > 0 ? M : 1);
-   if ((ta = scalar_tensor(alpha, dtype, 1.0)) == NULL || (tb = scalar_tensor(beta, dtype, 0.0)) == NULL) goto final;
+   /* scalars: both on the host or both on the device (the module reads the flag from alpha, tensor_blas_gpu.c:108-120) */
+   {  OcDevice *sdev = (alphaT && alphaT->device != OcCPU) || (betaT && betaT->device != OcCPU) ? device : OcCPU;
+      OcSize ssize[OC_TENSOR_MAX_DIMS]; int k;
+      ssize[0] = ssize[1] = 1; for (k = 2; k < nd; k++) ssize[k] = csize[k];
+      ta = alphaT ? OcIncrefTensor(alphaT) : scalar_tensor(alpha, dtype, 1.0);
+      tb = betaT ? OcIncrefTensor(betaT) : scalar_tensor(beta, dtype, 0.0);
+      if (ta == NULL || tb == NULL) goto final;
+      if (OcTensor_ensure(&ta, dtype, sdev) != 0 || OcTensor_ensure(&tb, dtype, sdev) != 0) goto final;
+      if ((v = OcTensor_broadcastTo(ta, nd, ssize)) == NULL) goto final;
+      OcDecrefTensor(ta); ta = v;
+      if ((v = OcTensor_broadcastTo(tb, nd, ssize)) == NULL) goto final;
+      OcDecrefTensor(tb); tb = v;
+      if (sdev != OcCPU && (OcTensor_startRead(c, ta) != 0 || OcTensor_startRead(c, tb) != 0)) goto final;
+   }
    /* the caller runs the stream protocol around Tensor_gemm (tensor_itf.c:6727-6750) */
    if (OcTensor_startRead(c, a) != 0 || OcTensor_startRead(c, b) != 0) goto final;
    result = m->Tensor_gemm(M, N, K, modeA, modeB, ta, a, ldA, b, ldB, tb, c, ldC);
    if (result == 0 && (OcTensor_update(c) != 0 || OcTensor_finishRead(c, a) != 0 || OcTensor_finishRead(c, b) != 0)) result = -1;
+   if (result == 0 && ta->device != OcCPU && (OcTensor_finishRead(c, ta) != 0 || OcTensor_finishRead(c, tb) != 0)) result = -1;
    if (result == 0 && *C == NULL && halftype != OcDTypeNone) result = OcTensor_ensure(&c, halftype, device);
    if (result == 0 && *C == NULL) { *C = c; c = NULL; }
    else if (result == 0 && c != *C) result = OcTensor_copy(c, *C);
@@ -371,6 +396,10 @@ final:
 }
 int OcTensor_mtimes(OcTensor *A, OcTensor *B, OcTensor **C) { return OcTensor_gemm(NULL, A, 'N', B, 'N', NULL, C); }
 
+int OcTensor_gemm(OcScalar *alpha, OcTensor *A, char modeA, OcTensor *B, char modeB, OcScalar *beta, OcTensor **C)
+{  return gemm_core(alpha, NULL, A, modeA, B, modeB, beta, NULL, C); }
+int OcTensor_gemmTensors(OcTensor *alpha, OcTensor *A, char modeA, OcTensor *B, char modeB, OcTensor *beta, OcTensor **C)
+{  return gemm_core(NULL, alpha, A, modeA, B, modeB, NULL, beta, C); }
 /* ---- index operations through the table (src/core/interface/index_itf.c, tensor_itf.c:2359-2700) ----------------- */
 /* indices: int64 tensor [k, n] on the tensor's device: n index tuples for the first k dimensions of `tensor` (negative
    values count from the end). Builds the view the interface builds -- one offset table per indexed dimension, made by

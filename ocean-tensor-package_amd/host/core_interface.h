@@ -31,6 +31,7 @@ int OcTensor_unary(int op, OcTensor *src, OcTensor **dst);
 int OcTensor_reduceAll(int which, OcTensor *tensor, double p, OcScalar *result);    /* which: och reduction index of an OcScalar-valued reduction */
 int OcTensor_axisReduce(int which, OcTensor *src, int n, int *axes, int keepdims, double p, OcTensor **dst);
 int OcTensor_gemm(OcScalar *alpha, OcTensor *A, char modeA, OcTensor *B, char modeB, OcScalar *beta, OcTensor **C);
+int OcTensor_gemmTensors(OcTensor *alpha, OcTensor *A, char modeA, OcTensor *B, char modeB, OcTensor *beta, OcTensor **C);   /* scalars as tensors (one per product), NULL: 1 and 0 */
 int OcTensor_mtimes(OcTensor *A, OcTensor *B, OcTensor **C);
 /* index operations through the table: indices is an int64 tensor of shape [nindexed dims, n]; view dimensions beyond it stay whole */
 int OcTensor_getIndexed(OcTensor *tensor, OcTensor *indices, OcTensor **dst);
