@@ -1,5 +1,6 @@
-"""ctypes binding of the CPU oracle (oracle/liboracle.so) and, when it was built, of the
-reference's own operation macros (oracle/_ref/libocean_ref.so). Test infrastructure only."""
+"""ctypes binding of the CPU oracle (oracle/liboracle.so). The library of the reference's own operation macros
+(oracle/_ref/libocean_ref.so) is mapped only when load_ref() is called, which the CPU tests that pin the oracle
+against it do; nothing that runs on a GPU machine calls it. Test infrastructure only."""
 import ctypes as C
 import os
 
@@ -12,7 +13,23 @@ REF_PATH = os.path.join(ROOT, "oracle", "_ref", "libocean_ref.so")
 if not os.path.exists(ORACLE_PATH):
     raise ImportError("oracle/liboracle.so is missing: run `make -C oracle`")
 lib = C.CDLL(ORACLE_PATH)
-ref = C.CDLL(REF_PATH) if os.path.exists(REF_PATH) else None
+_ref = None
+
+
+def ref_built():
+    return os.path.exists(REF_PATH)
+
+
+def load_ref():
+    """The reference-macro library, mapped on first use."""
+    global _ref
+    if _ref is None:
+        _ref = C.CDLL(REF_PATH)
+        for name in ("ref_binary", "ref_unary", "ref_reduce", "ref_assign", "ref_swap_assign"):
+            getattr(_ref, name).restype = C.c_void_p
+        _proto(_ref.ref_half_to_float, C.c_float, [C.c_uint16])
+        _proto(_ref.ref_float_to_half, C.c_uint16, [C.c_float])
+    return _ref
 
 _sz = C.POINTER(C.c_size_t)
 _st = C.POINTER(C.c_ssize_t)
@@ -60,11 +77,6 @@ def setup(oh):
     ]:
         if hasattr(lib, name):
             _proto(getattr(lib, name), res, args)
-    if ref is not None:
-        for name in ("ref_binary", "ref_unary", "ref_reduce", "ref_assign", "ref_swap_assign"):
-            getattr(ref, name).restype = C.c_void_p
-        _proto(ref.ref_half_to_float, C.c_float, [C.c_uint16])
-        _proto(ref.ref_float_to_half, C.c_uint16, [C.c_float])
 
 
 def ptr(a):

@@ -20,7 +20,7 @@ import helpers as H
 import ocean_hip as oh
 
 orc = H.orc
-pytestmark = pytest.mark.skipif(orc.ref is None, reason="oracle/_ref was not built (reference tree absent)")
+pytestmark = pytest.mark.skipif(not orc.ref_built(), reason="oracle/_ref was not built (reference tree absent)")
 
 REF_BIN = ["add", "subtract", "multiply", "divide", "true_divide", "floor_divide", "power", "mod", "fmod",
            "min", "max", "fmin", "fmax", "lt", "le", "eq", "ne", "ge", "gt",
@@ -91,7 +91,7 @@ PAIRS = [(op, dt) for op in range(len(oh.BINARY_OPS)) for dt in H.ALL_TYPES]
 
 @pytest.mark.parametrize("op,dtype", PAIRS, ids=["%s-%s" % (oh.BINARY_OPS[o], H.NAMES[d]) for o, d in PAIRS])
 def test_binary_matches_reference(op, dtype):
-    fn = orc.ref.ref_binary(op, dtype)
+    fn = orc.load_ref().ref_binary(op, dtype)
     sup = bool(orc.lib.oracle_binary_supported(op, dtype))
     name = oh.BINARY_OPS[op]
     if not fn:
@@ -127,7 +127,7 @@ UPAIRS = [(op, dt) for op in range(len(oh.UNARY_OPS)) for dt in H.ALL_TYPES]
 
 @pytest.mark.parametrize("op,dtype", UPAIRS, ids=["%s-%s" % (oh.UNARY_OPS[o], H.NAMES[d]) for o, d in UPAIRS])
 def test_unary_matches_reference(op, dtype):
-    fn = orc.ref.ref_unary(op, dtype)
+    fn = orc.load_ref().ref_unary(op, dtype)
     name = oh.UNARY_OPS[op]
     sup = bool(orc.lib.oracle_unary_supported(op, dtype))
     assert sup == bool(fn), "support differs for %s %s" % (name, H.NAMES[dtype])
@@ -169,7 +169,7 @@ def test_half_conversion_exhaustive():
     """All 65536 half patterns to float, and a float sweep (every exponent, ties, boundaries) to half."""
     for h in range(0x10000):
         a = orc.lib.oracle_half_to_float(h)
-        b = orc.ref.ref_half_to_float(h)
+        b = orc.load_ref().ref_half_to_float(h)
         assert np.float32(a).view(np.uint32) == np.float32(b).view(np.uint32) or (a != a and b != b), hex(h)
     rng = np.random.default_rng(3)
     bits = np.concatenate([
@@ -180,7 +180,7 @@ def test_half_conversion_exhaustive():
     bits = np.concatenate([bits, bits | np.uint32(0x80000000)])
     floats = bits.view(np.float32)
     for f in floats[:: 7]:
-        assert orc.lib.oracle_float_to_half(float(f)) == orc.ref.ref_float_to_half(float(f)), float(f)
+        assert orc.lib.oracle_float_to_half(float(f)) == orc.load_ref().ref_float_to_half(float(f)), float(f)
 
 
 CPAIRS = [(s, d) for s in H.ALL_TYPES for d in H.ALL_TYPES]
@@ -206,7 +206,7 @@ def test_conversions_match_reference(ts, td):
             x.real, x.imag = v, rng.uniform(-5, 5, n)
         else:
             x = v.astype(x.dtype)
-    for swap, getter, orfn in ((0, orc.ref.ref_assign, orc.lib.oracle_copy), (1, orc.ref.ref_swap_assign, orc.lib.oracle_byteswap_copy)):
+    for swap, getter, orfn in ((0, orc.load_ref().ref_assign, orc.lib.oracle_copy), (1, orc.load_ref().ref_swap_assign, orc.lib.oracle_byteswap_copy)):
         fn = getter(ts, td)
         assert fn
         src = x.copy()
@@ -237,7 +237,7 @@ RPAIRS = [(op, dt) for op in range(len(oh.REDUCE_OPS)) for dt in H.ALL_TYPES]
 def test_reductions_match_reference(op, dtype):
     """Serial fold of a contiguous vector: init / accumulate / finalize code of reduce_ops.h."""
     name = oh.REDUCE_OPS[op]
-    fn = orc.ref.ref_reduce(op, dtype)
+    fn = orc.load_ref().ref_reduce(op, dtype)
     sup = bool(orc.lib.oracle_reduce_supported(op, dtype))
     if not fn:
         # *_nan variants of integer types forward to the plain operation in the CPU sources
