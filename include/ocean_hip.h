@@ -63,6 +63,16 @@ extern const int och_type_size[OCH_DTYPE_COUNT];
 /* Message of the most recent failure in the calling thread. */
 const char *och_last_error(void);
 
+/* The first runtime error since the last check (OcCuda_setStatus / OcCuda_checkStatus / OcCuda_clearStatus,            */
+/* src/core/gpu/cuda.c:84-120). Work is asynchronous: an error raised by a kernel or a copy while it runs is seen by   */
+/* whichever call looks next, and calls after it may fail in its wake. Every failing call of this library notes its    */
+/* error code; the first one is kept. och_stream_synchronize, och_event_synchronize and och_device_synchronize also    */
+/* ask the runtime, once the wait is over, for an error raised meanwhile, note it and return -1 with a message that    */
+/* says where it was found. och_status_check returns 0 when nothing was noted; otherwise -1 with "HIP error: ..." as   */
+/* the message, and forgets the error. och_status_clear forgets it without reporting.                                  */
+int  och_status_check(void);
+void och_status_clear(void);
+
 /* ======================================================================== */
 /* Device, stream, event and memory glue                                    */
 /* Replaces: src/core/gpu/device_gpu.c:155-420 (warm-up, streams, events),  */
@@ -139,7 +149,9 @@ int och_membench(int kind, int unr, int nt, int map, int block, int blocks, size
 /* that synchronise or allocate may not be recorded: och_reduce_all, och_find_count, och_memcpy_htod / dtoh,        */
 /* och_malloc_async / och_free_async, och_copy between tensors of different shape AND type. Everything else in this */
 /* header is recordable; scalars passed in host memory are frozen at their recorded value, scalars in device memory */
-/* are read at every replay. `stream` must be a created stream.                                                     */
+/* are read at every replay. `stream` must be a created stream. A graph replays on the stream that recorded it and on */
+/* no other (och_graph_launch returns an error): its reductions and split products use that stream's scratch memory,  */
+/* which a replay elsewhere would share, unordered, with the work of the recording stream.                           */
 typedef void *och_graph;
 int och_stream_begin_capture(och_stream stream);
 int och_stream_end_capture(och_stream stream, och_graph *graph);
@@ -305,6 +317,16 @@ int och_reduce_all_device_noalloc(int op, int dtype, int ndims, const size_t *si
                    void *ptr, const och_scalar *param1, const och_scalar *param2, double p,
                    void *dresult, och_stream stream);
 size_t och_reduce_all_noalloc_max_elements(void);
+/* A full reduction over a layout of several dimensions indexes at most 0xFFFF0000 elements per launch (the reference  */
+/* switches to 64-bit indices instead, solid/src/core/gpu/op/apply_elemwise.c:68-99). Larger tensors are cut along     */
+/* their outer dimensions into boxes that are launched one after the other; the launches share the partial slots and  */
+/* the ticket counter, and the last block of the last launch folds. och_reduce_cut_parts is that cutting, on the host */
+/* alone: first index and extent per dimension of every box (ndims values per box, at most max_boxes boxes written),   */
+/* returns the number of boxes, or -1 when dimension 0 alone exceeds the limit (it is never cut). Test hook:           */
+/* och_reduce_set_part_limit lowers the number of elements per launch (0 restores the default) so that small tensors  */
+/* take this path.                                                                                                    */
+long long och_reduce_cut_parts(int ndims, const size_t *size, size_t limit, long long max_boxes, size_t *starts, size_t *counts);
+void och_reduce_set_part_limit(size_t nelem);
 
 /* ======================================================================== */
 /* Axis reductions (template_reduce_axis.cu:54-80; reduce_axis.h:563-597)   */

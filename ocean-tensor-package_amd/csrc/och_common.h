@@ -12,17 +12,34 @@ namespace och {
 
 int  set_error(const char *fmt, ...);        /* stores the message, returns -1 */
 void clear_error();
+void note_status(int hip_error);             /* keeps the first error until och_status_check clears it */
 
+/* Every failing runtime call is also noted in a process-wide status that keeps the FIRST error until
+   och_status_check reports and clears it (the protocol of src/core/gpu/cuda.c:84-120): work is asynchronous, so the
+   call that returns an error is often not the one that caused it, and later calls may fail in its wake. */
 #define OCH_CHECK_HIP(CALL)                                                          \
    do { hipError_t _e = (CALL);                                                      \
         if (_e != hipSuccess)                                                        \
+        {  och::note_status((int)_e);                                                \
            return och::set_error("%s failed: %s (%s:%d)", #CALL, hipGetErrorString(_e), __FILE__, __LINE__); \
+        }                                                                            \
    } while (0)
 
 #define OCH_CHECK_LAUNCH()                                                           \
    do { hipError_t _e = hipGetLastError();                                           \
         if (_e != hipSuccess)                                                        \
+        {  och::note_status((int)_e);                                                \
            return och::set_error("kernel launch failed: %s (%s:%d)", hipGetErrorString(_e), __FILE__, __LINE__); \
+        }                                                                            \
+   } while (0)
+
+/* After a wait has returned: an error that a kernel or copy raised while it ran shows up as the runtime's last error */
+#define OCH_CHECK_AFTER_WAIT(WHAT)                                                   \
+   do { hipError_t _e = hipGetLastError();                                           \
+        if (_e != hipSuccess)                                                        \
+        {  och::note_status((int)_e);                                                \
+           return och::set_error("asynchronous error found when %s finished waiting: %s", WHAT, hipGetErrorString(_e)); \
+        }                                                                            \
    } while (0)
 
 static inline hipStream_t as_stream(och_stream s) { return (hipStream_t)s; }

@@ -154,18 +154,25 @@ extern "C" int och_index_to_offset(int dtype, int nstrides, const int64_t *strid
    if (nelem == 0) return 0;
    ToOffsetStrides st; memset(&st, 0, sizeof(st));
    for (int i = 0; i < nstrides; i++) st.s[i] = strides[i];
-   const dim3 grid((unsigned)((nelem + 255) / 256)), block(256);
-   if (nelem > 0xFFFFFF00ull * 256ull) return set_error("index_to_offset: too many elements");
-   switch (dtype)
-   {
-#define OCH_CASE(T, ID) case ID: hipLaunchKernelGGL((index_to_offset_kernel<T>), grid, block, 0, as_stream(stream), (uint64_t)nelem, nstrides, st, \
-                           (int64_t)stride_reduce, (const char *)ptr1, (int64_t)stride1, (char *)ptr2, (int64_t)stride2); break;
-      OCH_CASE(uint8_t, OCH_UINT8) OCH_CASE(uint16_t, OCH_UINT16) OCH_CASE(uint32_t, OCH_UINT32) OCH_CASE(uint64_t, OCH_UINT64)
-      OCH_CASE(int8_t, OCH_INT8) OCH_CASE(int16_t, OCH_INT16) OCH_CASE(int32_t, OCH_INT32) OCH_CASE(int64_t, OCH_INT64)
+   /* launches of at most 2^31 elements each (the grid of one launch is 32 bits of blocks wide, and the runtime accepts
+      far fewer blocks than that) */
+   const size_t per_launch = (size_t)1 << 31;
+   for (size_t first = 0; first < nelem; first += per_launch)
+   {  const size_t n = (nelem - first < per_launch) ? nelem - first : per_launch;
+      const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+      const char *src = (const char *)ptr1 + (int64_t)first * (int64_t)stride1;
+      char *dst = (char *)ptr2 + (int64_t)first * (int64_t)stride2;
+      switch (dtype)
+      {
+#define OCH_CASE(T, ID) case ID: hipLaunchKernelGGL((index_to_offset_kernel<T>), grid, block, 0, as_stream(stream), (uint64_t)n, nstrides, st, \
+                           (int64_t)stride_reduce, src, (int64_t)stride1, dst, (int64_t)stride2); break;
+         OCH_CASE(uint8_t, OCH_UINT8) OCH_CASE(uint16_t, OCH_UINT16) OCH_CASE(uint32_t, OCH_UINT32) OCH_CASE(uint64_t, OCH_UINT64)
+         OCH_CASE(int8_t, OCH_INT8) OCH_CASE(int16_t, OCH_INT16) OCH_CASE(int32_t, OCH_INT32) OCH_CASE(int64_t, OCH_INT64)
 #undef OCH_CASE
-      default: return set_error("index_to_offset is available for integer types only (got %d)", dtype);
+         default: return set_error("index_to_offset is available for integer types only (got %d)", dtype);
+      }
+      OCH_CHECK_LAUNCH();
    }
-   OCH_CHECK_LAUNCH();
    return 0;
 }
 

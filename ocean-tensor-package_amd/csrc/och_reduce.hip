@@ -2,6 +2,7 @@
  * the stream they run on. */
 #include "och_reduce_all.h"
 #include <string.h>
+#include <atomic>
 #include <mutex>
 
 namespace och {
@@ -43,6 +44,25 @@ extern "C" int och_reduce_result_dtype(int op, int dtype)
    if (op == OCH_R_MAXIMUM || op == OCH_R_MINIMUM) return dtype;
    if (op == OCH_R_MAXIMUM_ABS || op == OCH_R_MINIMUM_ABS) return abstype;
    return (isbool || isuint || issint) ? OCH_DOUBLE : abstype;      /* norms */
+}
+
+namespace och {
+static std::atomic<uint64_t> g_part_limit(OCH_RED_PART_LIMIT);
+uint64_t reduce_part_limit() { return g_part_limit.load(); }
+}
+extern "C" void och_reduce_set_part_limit(size_t nelem)
+{  och::g_part_limit.store((nelem == 0 || nelem > OCH_RED_PART_LIMIT) ? OCH_RED_PART_LIMIT : (uint64_t)nelem); }
+extern "C" long long och_reduce_cut_parts(int ndims, const size_t *size, size_t limit, long long max_boxes, size_t *starts, size_t *counts)
+{
+   if (ndims < 1 || ndims > OCH_MAX_DIMS) return -1;
+   uint64_t sz[OCH_MAX_DIMS]; long long kept = 0;
+   for (int d = 0; d < ndims; d++) sz[d] = size[d];
+   return (long long)och::reduce_cut_parts(ndims, sz, (uint64_t)limit, [&](const uint64_t *start, const uint64_t *count)
+          {  if (kept < max_boxes)
+             {  for (int d = 0; d < ndims; d++) { starts[kept * ndims + d] = start[d]; counts[kept * ndims + d] = count[d]; }
+                kept++;
+             }
+          });
 }
 
 extern "C" int och_reduce_all_device(int op, int dtype, int ndims, const size_t *size, const ptrdiff_t *strides,

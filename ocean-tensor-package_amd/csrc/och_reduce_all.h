@@ -87,7 +87,45 @@ struct RedParams
    char *tail;                 /* flat layout only: elements left over after the last full group */
    int   ntail;
    int64_t rowbytes;           /* row mode: bytes of one row of the first dimension */
+   unsigned int slot_base;     /* partial slot of block 0 of this launch */
+   unsigned int total_blocks;  /* blocks of all launches that share the counter: the block that draws the last ticket folds */
 };
+
+/* Number of elements one launch of a layout with several dimensions indexes (its group index is 32 bits wide). Larger
+   tensors are cut along their outer dimensions into parts that are launched one after the other on the same stream:
+   every part writes its blocks' partial results into its own range of slots and the block that draws the last ticket
+   of the last part folds them all. och_reduce_set_part_limit lowers the number so that small tensors exercise this. */
+#define OCH_RED_PART_LIMIT 0xFFFF0000ull
+uint64_t reduce_part_limit();
+
+/* Cuts `size` (ndims > 1, product above `limit`) into boxes of at most `limit` elements: whole runs of the outermost
+   dimension where one index of it fits, otherwise index by index with the next dimension cut in turn. Calls
+   visit(start, count) with the first index and the extent of every box in every dimension; returns the number of boxes,
+   or -1 when the first dimension alone exceeds the limit (it is never cut: rows stay whole). */
+template <class Visit>
+static int64_t reduce_cut_parts(int ndims, const uint64_t *size, uint64_t limit, Visit visit)
+{
+   uint64_t start[OCH_MAX_DIMS] = { 0 }, count[OCH_MAX_DIMS], inner[OCH_MAX_DIMS + 1];
+   inner[0] = 1;
+   for (int d = 0; d < ndims; d++) { inner[d + 1] = inner[d] * size[d]; count[d] = size[d]; }   /* inner[d]: elements below dimension d */
+   if (ndims < 1 || size[0] > limit) return -1;
+   int top = ndims - 1;
+   while (top > 0 && inner[top] > limit) top--;         /* dimensions above `top` are walked index by index */
+   /* dimension `top` is cut into runs of `run` indices (inner[top] <= limit, so run >= 1); top == 0 keeps whole rows */
+   const uint64_t run = (top == 0) ? size[0] : limit / inner[top];
+   int64_t boxes = 0;
+   for (int d = top + 1; d < ndims; d++) { count[d] = 1; start[d] = 0; }
+   for (;;)
+   {  for (uint64_t at = 0; at < size[top]; at += run)
+      {  start[top] = at; count[top] = (size[top] - at < run) ? size[top] - at : run;
+         visit(start, count); boxes++;
+      }
+      int d = top + 1;
+      for (; d < ndims; d++) { if (++start[d] < size[d]) break; start[d] = 0; }
+      if (d >= ndims) break;
+   }
+   return boxes;
+}
 
 /* Row mode: the first dimension is contiguous but its rows are not whole aligned 16-byte groups (a width that is not a
    multiple of VEC, a pitch or a start that is not a multiple of 16 bytes: sub-matrices of 1- and 2-byte types mostly).
@@ -186,15 +224,15 @@ __global__ __launch_bounds__(OCH_RED_BLOCK) void reduce_all_kernel(const RedPara
       acc = RD::combine(acc, RD::load(*reinterpret_cast<const T *>(p.tail + (int64_t)threadIdx.x * p.ew.estride[0]), prm));
    acc = block_reduce<RD>(acc, lds);
    if (threadIdx.x == 0)
-   {  store_shared_global<Acc>(p.partials + (size_t)blockIdx.x * OCH_RED_SLOT, acc);
+   {  store_shared_global<Acc>(p.partials + (size_t)(p.slot_base + blockIdx.x) * OCH_RED_SLOT, acc);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");            /* the write-through stores above have completed */
       ticket = __hip_atomic_fetch_add(p.counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
    }
    __syncthreads();
-   if (ticket != gridDim.x - 1) return;
+   if (ticket != p.total_blocks - 1) return;
    /* last block: every partial is in memory; fold them in index order */
    acc = RD::identity();
-   for (unsigned int b = threadIdx.x; b < gridDim.x; b += OCH_RED_BLOCK)
+   for (unsigned int b = threadIdx.x; b < p.total_blocks; b += OCH_RED_BLOCK)
       acc = RD::combine(acc, load_shared_global<Acc>(p.partials + (size_t)b * OCH_RED_SLOT));
    __syncthreads();
    acc = block_reduce<RD>(acc, lds);
@@ -209,25 +247,14 @@ typedef int (*red_fn)(int ndims, const size_t *size, const ptrdiff_t *strides, v
                       const och_scalar *b1, const och_scalar *b2, double pnorm,
                       void *dresult, char *scratch, bool zero_counter, hipStream_t stream);
 
+/* One launch: `shape` is normalised and holds at most reduce_part_limit() elements unless it is one-dimensional.
+   blocks == 0: the launch stands alone and picks its own number of blocks; otherwise it is one of several that share
+   the partial slots (its blocks write slots slot_base ...) and the counter (total blocks of all launches). */
 template <class T, int OP>
-static int launch_reduce_all(int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr,
-                             const och_scalar *b1, const och_scalar *b2, double pnorm,
-                             void *dresult, char *scratch, bool zero_counter, hipStream_t stream)
+static int launch_reduce_part(const EwShape<1> &shape, const typename Reduce<T, OP>::Param &prm, void *dresult, char *scratch,
+                              unsigned int slot_base, unsigned int nblocks, unsigned int total, hipStream_t stream)
 {
    typedef Reduce<T, OP> RD;
-   static_assert(sizeof(typename RD::Acc) <= OCH_RED_SLOT, "accumulator does not fit a partial slot");
-   typename RD::Param prm;
-   memset(&prm, 0, sizeof(prm));
-   if (b1) memcpy(&prm.bound1, b1, sizeof(T));
-   if (b2) memcpy(&prm.bound2, b2, sizeof(T));
-   prm.phalf = pnorm / 2; prm.pinv = (pnorm != 0) ? 1.0 / pnorm : 0.0;
-
-   const ptrdiff_t *st[1] = { strides }; void *pp[1] = { ptr };
-   EwShape<1> shape;
-   if (ew_normalize<1>(shape, ndims, size, st, pp, 0, true) != 0) return -1;
-   if (shape.nelem == 0 && RD::NEEDS_DATA) return set_error("reduction of an empty tensor is undefined for this operation");
-   if (shape.ndims > 1 && shape.nelem > 0xFFFF0000ull) return set_error("strided reduction of more than 2^32 elements is not supported");
-
    RedParams p;
    memset(&p, 0, sizeof(p));
    constexpr int VEC = vec_for<T>();
@@ -275,9 +302,10 @@ static int launch_reduce_all(int ndims, const size_t *size, const ptrdiff_t *str
    p.partials = scratch;
    p.counter = reinterpret_cast<unsigned int *>(scratch + OCH_RED_MAX_BLOCKS * OCH_RED_SLOT);
    p.result = dresult;
-   if (zero_counter && fill_bytes(p.counter, 0, sizeof(unsigned int), stream) != 0) return -1;
    uint64_t want = (p.ngroups + (uint64_t)OCH_RED_BLOCK * OCH_RED_UNR - 1) / ((uint64_t)OCH_RED_BLOCK * OCH_RED_UNR);
    unsigned int blocks = (unsigned int)(want < 1 ? 1 : (want > OCH_RED_MAX_BLOCKS ? OCH_RED_MAX_BLOCKS : want));
+   if (nblocks != 0) blocks = nblocks;                        /* blocks beyond the data fold the identity */
+   p.slot_base = slot_base; p.total_blocks = (nblocks != 0) ? total : blocks;
    {  const uint64_t step = (uint64_t)OCH_RED_BLOCK * OCH_RED_UNR;
       uint64_t per = (p.ngroups + blocks - 1) / blocks;
       p.per_block = (per + step - 1) / step * step;
@@ -292,6 +320,61 @@ static int launch_reduce_all(int ndims, const size_t *size, const ptrdiff_t *str
    else             hipLaunchKernelGGL((reduce_all_kernel<RD, T, 1, 0>),  dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
    OCH_CHECK_LAUNCH();
    return 0;
+}
+
+template <class T, int OP>
+static int launch_reduce_all(int ndims, const size_t *size, const ptrdiff_t *strides, void *ptr,
+                             const och_scalar *b1, const och_scalar *b2, double pnorm,
+                             void *dresult, char *scratch, bool zero_counter, hipStream_t stream)
+{
+   typedef Reduce<T, OP> RD;
+   static_assert(sizeof(typename RD::Acc) <= OCH_RED_SLOT, "accumulator does not fit a partial slot");
+   typename RD::Param prm;
+   memset(&prm, 0, sizeof(prm));
+   if (b1) memcpy(&prm.bound1, b1, sizeof(T));
+   if (b2) memcpy(&prm.bound2, b2, sizeof(T));
+   prm.phalf = pnorm / 2; prm.pinv = (pnorm != 0) ? 1.0 / pnorm : 0.0;
+
+   const ptrdiff_t *st[1] = { strides }; void *pp[1] = { ptr };
+   EwShape<1> shape;
+   if (ew_normalize<1>(shape, ndims, size, st, pp, 0, true) != 0) return -1;
+   if (shape.nelem == 0 && RD::NEEDS_DATA) return set_error("reduction of an empty tensor is undefined for this operation");
+   unsigned int *counter = reinterpret_cast<unsigned int *>(scratch + OCH_RED_MAX_BLOCKS * OCH_RED_SLOT);
+   if (zero_counter && fill_bytes(counter, 0, sizeof(unsigned int), stream) != 0) return -1;
+   const uint64_t limit = reduce_part_limit();
+   if (shape.ndims > 1 && shape.nelem > limit)
+   {  /* more elements than one launch indexes: one launch per box, all of them sharing the slots and the counter */
+      struct Box { uint64_t start[OCH_MAX_DIMS], count[OCH_MAX_DIMS]; };
+      Box boxes[OCH_RED_MAX_BLOCKS];                         /* on the stack: this path allocates nothing, on the host either */
+      int64_t kept = 0;
+      const int64_t n = reduce_cut_parts(shape.ndims, shape.size, limit, [&](const uint64_t *start, const uint64_t *count)
+                        {  if (kept < OCH_RED_MAX_BLOCKS)
+                           {  Box &b = boxes[kept++]; for (int d = 0; d < shape.ndims; d++) { b.start[d] = start[d]; b.count[d] = count[d]; } }
+                        });
+      if (n < 0) return set_error("reduction: the first dimension of a strided tensor exceeds %llu elements", (unsigned long long)limit);
+      if (n > OCH_RED_MAX_BLOCKS) return set_error("reduction: the tensor needs %lld launches, more than the %d that share the partial results", (long long)n, OCH_RED_MAX_BLOCKS);
+      const unsigned int each = (unsigned int)(OCH_RED_MAX_BLOCKS / n), total = each * (unsigned int)n;
+      unsigned int base = 0;
+      for (int64_t k = 0; k < n; k++)
+      {  const Box &b = boxes[k];
+         EwShape<1> part = shape;
+         int nd = 0;
+         part.nelem = 1;
+         for (int d = 0; d < shape.ndims; d++)
+         {  part.ptr[0] += (int64_t)b.start[d] * shape.stride[0][d]; part.nelem *= b.count[d];
+            if (d == 0 || b.count[d] != 1) { part.size[nd] = b.count[d]; part.stride[0][nd] = shape.stride[0][d]; nd++; }
+         }
+         part.ndims = nd;
+         if (launch_reduce_part<T, OP>(part, prm, dresult, scratch, base, each, total, stream) != 0)
+         {  /* the launches so far have drawn tickets that no later block will complete: start the next call from zero */
+            (void)fill_bytes(counter, 0, sizeof(unsigned int), stream);
+            return -1;
+         }
+         base += each;
+      }
+      return 0;
+   }
+   return launch_reduce_part<T, OP>(shape, prm, dresult, scratch, 0, 0, 0, stream);
 }
 
 template <class T, int OP, bool OK> struct PickR { static constexpr red_fn fn = nullptr; };

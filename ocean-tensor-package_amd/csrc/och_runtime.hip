@@ -5,6 +5,7 @@
  * stream-ordered allocation from the device's default memory pool. */
 #include "och_common.h"
 #include <string.h>
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -17,6 +18,11 @@ int set_error(const char *fmt, ...)
    return -1;
 }
 void clear_error() { g_errmsg[0] = 0; }
+static std::atomic<int> g_status(0);              /* hipSuccess, or the first error since the last check */
+void note_status(int hip_error)
+{  int none = 0;
+   if (hip_error != 0) g_status.compare_exchange_strong(none, hip_error);
+}
 __global__ void warmup_kernel(int *p) { if (p) *p = 1; }
 }
 
@@ -34,8 +40,16 @@ int stream_context(hipStream_t stream, StreamContext **out)
    if (it == g_stream_ctx.end())
    {  StreamContext c = { nullptr, nullptr, nullptr };
       void *scratch = nullptr, *host = nullptr;
+      /* the scratch cannot be created while the stream records a graph: allocation is not a graph node, and the
+         zeroing below would become one and run again at every replay, in the middle of the recorded reductions */
+      hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+      if (stream != nullptr) OCH_CHECK_HIP(hipStreamIsCapturing(stream, &capturing));
+      if (capturing != hipStreamCaptureStatusNone)
+         return set_error("a stream must be used once, or recording must start with och_stream_begin_capture, before library calls are recorded on it");
       OCH_CHECK_HIP(hipMalloc(&scratch, OCH_RED_SCRATCH));
-      hipError_t e = hipMemset(scratch, 0, OCH_RED_SCRATCH);
+      /* zeroed by a kernel on the owning stream itself: ordered before the stream's first reduction by the stream,
+         whatever its blocking mode with respect to the null stream */
+      hipError_t e = (fill_bytes(scratch, 0, OCH_RED_SCRATCH, stream) == 0) ? hipSuccess : hipErrorLaunchFailure;
       if (e == hipSuccess) e = hipHostMalloc(&host, 64, hipHostMallocDefault);
       if (e != hipSuccess) { (void)hipFree(scratch); return set_error("stream scratch: %s", hipGetErrorString(e)); }
       c.red_scratch = (char *)scratch; c.host_result = host;
@@ -100,6 +114,14 @@ extern "C" {
 const int och_type_size[OCH_DTYPE_COUNT] = { 1, 1, 2, 4, 8, 1, 2, 4, 8, 2, 4, 8, 4, 8, 16 };
 
 const char *och_last_error(void) { return och::g_errmsg; }
+
+int och_status_check(void)
+{  int e = och::g_status.exchange(0);
+   if (e == 0) return 0;
+   (void)hipGetLastError();
+   return och::set_error("HIP error: %s", hipGetErrorString((hipError_t)e));
+}
+void och_status_clear(void) { och::g_status.store(0); }
 
 int och_device_count(int *count)
 {
@@ -175,7 +197,7 @@ int och_device_warmup(int device)
    OCH_CHECK_HIP(hipSetDevice(prev));
    return status;
 }
-int och_device_synchronize(void) { OCH_CHECK_HIP(hipDeviceSynchronize()); return 0; }
+int och_device_synchronize(void) { OCH_CHECK_HIP(hipDeviceSynchronize()); OCH_CHECK_AFTER_WAIT("the device"); return 0; }
 
 int och_stream_create(och_stream *stream)
 {
@@ -189,7 +211,7 @@ int och_stream_destroy(och_stream stream)
    OCH_CHECK_HIP(hipStreamDestroy((hipStream_t)stream));
    return 0;
 }
-int och_stream_synchronize(och_stream stream) { OCH_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream)); return 0; }
+int och_stream_synchronize(och_stream stream) { OCH_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream)); OCH_CHECK_AFTER_WAIT("a stream"); return 0; }
 int och_stream_wait_event(och_stream stream, och_event event)
 {  OCH_CHECK_HIP(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0)); return 0; }
 
@@ -202,7 +224,7 @@ int och_event_create(och_event *event, int timing)
 int och_event_destroy(och_event event) { OCH_CHECK_HIP(hipEventDestroy((hipEvent_t)event)); return 0; }
 int och_event_record(och_event event, och_stream stream)
 {  OCH_CHECK_HIP(hipEventRecord((hipEvent_t)event, (hipStream_t)stream)); return 0; }
-int och_event_synchronize(och_event event) { OCH_CHECK_HIP(hipEventSynchronize((hipEvent_t)event)); return 0; }
+int och_event_synchronize(och_event event) { OCH_CHECK_HIP(hipEventSynchronize((hipEvent_t)event)); OCH_CHECK_AFTER_WAIT("an event"); return 0; }
 int och_event_elapsed_ms(och_event start, och_event stop, float *ms)
 {  OCH_CHECK_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop)); return 0; }
 
@@ -213,8 +235,13 @@ int och_stream_begin_capture(och_stream stream)
    OCH_CHECK_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
    return 0;
 }
+/* A recorded graph keeps the stream it was recorded on: its reductions and split products address that stream's
+   scratch (partial results, ticket counter, workspace), so a replay on another stream would share them with whatever
+   runs on the recording stream at the same time. */
+struct och_graph_record { hipGraphExec_t exec; hipStream_t stream; int device; };
+
 int och_stream_end_capture(och_stream stream, och_graph *graph)
-{  hipGraph_t g = nullptr; hipGraphExec_t exec = nullptr;
+{  hipGraph_t g = nullptr; hipGraphExec_t exec = nullptr; int device = 0;
    if (graph == nullptr) return och::set_error("null graph pointer");
    *graph = nullptr;
    OCH_CHECK_HIP(hipStreamEndCapture((hipStream_t)stream, &g));
@@ -222,16 +249,25 @@ int och_stream_end_capture(och_stream stream, och_graph *graph)
    hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
    (void)hipGraphDestroy(g);
    if (e != hipSuccess) return och::set_error("hipGraphInstantiate failed: %s", hipGetErrorString(e));
-   *graph = (och_graph)exec;
+   if ((e = hipGetDevice(&device)) != hipSuccess) { (void)hipGraphExecDestroy(exec); return och::set_error("hipGetDevice failed: %s", hipGetErrorString(e)); }
+   och_graph_record *r = new och_graph_record{ exec, (hipStream_t)stream, device };
+   *graph = (och_graph)r;
    return 0;
 }
 int och_graph_launch(och_graph graph, och_stream stream)
 {  if (graph == nullptr) return och::set_error("null graph");
-   OCH_CHECK_HIP(hipGraphLaunch((hipGraphExec_t)graph, (hipStream_t)stream));
+   och_graph_record *r = (och_graph_record *)graph;
+   if ((hipStream_t)stream != r->stream)
+      return och::set_error("a graph replays on the stream that recorded it: its kernels use that stream's scratch memory");
+   OCH_CHECK_HIP(hipGraphLaunch(r->exec, r->stream));
    return 0;
 }
 int och_graph_destroy(och_graph graph)
-{  if (graph) OCH_CHECK_HIP(hipGraphExecDestroy((hipGraphExec_t)graph));
+{  if (graph == nullptr) return 0;
+   och_graph_record *r = (och_graph_record *)graph;
+   hipError_t e = hipGraphExecDestroy(r->exec);
+   delete r;
+   OCH_CHECK_HIP(e);
    return 0;
 }
 

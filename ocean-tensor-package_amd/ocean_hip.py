@@ -133,6 +133,10 @@ _i = C.c_int
 # every symbol that include/ocean_hip.h declares, with its argument types
 PROTOTYPES = {
     "och_last_error": (C.c_char_p, []),
+    "och_status_check": (_i, []),
+    "och_status_clear": (None, []),
+    "och_reduce_cut_parts": (C.c_longlong, [_i, C.POINTER(C.c_size_t), C.c_size_t, C.c_longlong, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "och_reduce_set_part_limit": (None, [C.c_size_t]),
     "och_device_count": (_i, [C.POINTER(_i)]),
     "och_device_set": (_i, [_i]),
     "och_device_get": (_i, [C.POINTER(_i)]),

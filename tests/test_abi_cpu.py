@@ -192,3 +192,43 @@ def test_kernel_choice():
     # first dimension equal to the vector width (one group per row: divisor 1)
     p = oh.elemwise_analyze([4, 4], [4, 5], [[4, 32], [4, 16]], [a, a])
     assert p.div_d[0] == 1 and fastdiv(12345, 1, p.div_m[0], p.div_s1[0], p.div_s2[0]) == 12345
+
+
+def test_cutting_a_large_reduction_into_launches():
+    """och_reduce_cut_parts (host arithmetic only): the boxes are disjoint, cover the tensor, hold at most `limit` elements
+    each, and never cut dimension 0; a dimension 0 beyond the limit is refused."""
+    import ocean_hip as oh
+    rng = np.random.default_rng(12)
+    cases = [([64, 20, 12, 9], 2304), ([64, 20, 12, 9], 997), ([63, 280], 64), ([5, 3, 2, 2, 3], 7), ([7], 7), ([4, 1, 6], 4),
+             ([1 << 20, 1 << 13, 1 << 5], 0xFFFF0000), ([1 << 31, 3, 40], 0xFFFF0000), ([3, 1 << 33], 0xFFFF0000)]
+    cases += [([int(v) for v in rng.integers(1, 9, rng.integers(2, 6))], int(rng.integers(8, 200))) for _ in range(200)]
+    for size, limit in cases:
+        nd, cap = len(size), 4096
+        starts, counts = (C.c_size_t * (cap * nd))(), (C.c_size_t * (cap * nd))()
+        n = oh.lib.och_reduce_cut_parts(nd, oh.sizes(size), limit, cap, starts, counts)
+        if size[0] > limit:
+            assert n == -1
+            continue
+        assert 1 <= n <= cap, (size, limit, n)
+        total = 0
+        small = int(np.prod(size, dtype=np.float64)) <= 1 << 20
+        seen = np.zeros(size[::-1], np.int32) if small else None
+        for k in range(n):
+            st, ct = [starts[k * nd + d] for d in range(nd)], [counts[k * nd + d] for d in range(nd)]
+            assert st[0] == 0 and ct[0] == size[0], "dimension 0 is never cut"
+            assert all(ct[d] >= 1 and st[d] + ct[d] <= size[d] for d in range(nd))
+            vol = 1
+            for c in ct:
+                vol *= c
+            assert vol <= limit, (size, limit, st, ct)
+            total += vol
+            if small:
+                seen[tuple(slice(st[d], st[d] + ct[d]) for d in range(nd - 1, -1, -1))] += 1
+        want = 1
+        for v in size:
+            want *= v
+        assert total == want, (size, limit)
+        if small:
+            assert (seen == 1).all(), (size, limit)
+        # a full run holds more than half the limit and at most one run per outer index is partial: under four times the minimum
+        assert n <= 4 * -(-want // limit), (size, limit, n)

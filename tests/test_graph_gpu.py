@@ -11,6 +11,8 @@ import pytest
 import helpers as H
 import ocean_hip as oh
 
+orc = H.orc
+
 pytestmark = pytest.mark.gpu
 
 
@@ -78,6 +80,11 @@ def test_graph_replays_equal_eager_launches(hip, stream):
         # unrelated eager work and a synchronisation between the replays
         oh.check(lib.och_binary(oh.B["add"], H.DOUBLE, 2, shape, st, scratch.ptr, st, scratch.ptr, st, scratch.ptr, h))
         stream.synchronize()
+    # a graph replays on its recording stream only: its reductions use that stream's partial slots and counter
+    other = oh.Stream()
+    assert lib.och_graph_launch(graph, other.handle) == -1 and "stream that recorded it" in lib.och_last_error().decode()
+    assert lib.och_graph_launch(graph, None) == -1
+    other.destroy()
     oh.check(lib.och_graph_destroy(graph))
     # recording on the default stream is refused, as is a second end without a begin
     with pytest.raises(oh.OceanHipError):
@@ -141,3 +148,30 @@ def test_graph_with_half_gemm_split_k_projection_and_gather(hip, stream):
     oh.check(lib.och_graph_destroy(graph))
     for b in (dA, dB, dC, dLA, dLB, dLC, dQ, dR, dtab, dG):
         b.free()
+
+
+def test_first_error_is_kept_until_it_is_checked(hip, stream):
+    """The status protocol of src/core/gpu/cuda.c:84-120: the first failing runtime call is remembered, later ones do not
+    replace it, och_status_check reports it once and forgets it. The failures are host-side argument errors."""
+    lib = oh.lib
+    lib.och_status_clear()
+    assert lib.och_status_check() == 0
+    stream.synchronize()
+    assert lib.och_status_check() == 0                              # waiting on healthy work notes nothing
+    count = C.c_int()
+    oh.check(lib.och_device_count(C.byref(count)))
+    assert lib.och_device_set(count.value + 100) == -1               # hipErrorInvalidDevice
+    first = lib.och_last_error().decode()
+    graph = C.c_void_p()
+    assert lib.och_stream_end_capture(stream.handle, C.byref(graph)) == -1     # a different error: the stream records nothing
+    assert lib.och_status_check() == -1
+    msg = lib.och_last_error().decode()
+    assert msg.startswith("HIP error: ") and msg[len("HIP error: "):] in first
+    assert lib.och_status_check() == 0
+    oh.check(lib.och_device_set(0))
+    # the stream still works
+    x = oh.to_device(np.arange(8, dtype=np.float64), stream)
+    out = np.zeros(1)
+    oh.check(lib.och_reduce_all(oh.R["sum"], H.DOUBLE, 1, oh.sizes([8]), oh.strides([8]), x.ptr, None, None, 0.0, orc.ptr(out), None, stream.handle))
+    assert out[0] == 28.0
+    x.free()

@@ -314,3 +314,52 @@ def test_reduce_rows_that_are_not_whole_vectors(hip, stream, dtype):
             else:
                 check_against_truth(name, dtype, rd, got, np.ascontiguousarray(view))
         x.free()
+
+
+def test_strided_reductions_in_several_launches(hip, stream):
+    """A layout of several dimensions with more elements than one launch indexes is cut along its outer dimensions; the
+    launches share the partial slots and the ticket counter. The limit is lowered so that small tensors take this path:
+    integer results must equal the one-launch results bit for bit, the float64 sum is within the usual bound, and the
+    counter is left at zero (the ordinary reduction that follows is right)."""
+    rng = np.random.default_rng(77)
+    parent = rng.integers(-100, 100, size=(9, 14, 40, 66), dtype=np.int32)
+    views = [parent[:, 1:13, ::2, 1:65].transpose(3, 2, 1, 0),         # every dimension strided: 64 x 20 x 12 x 9 in Ocean order
+             parent[::2, :, 3:39, 2:50],                               # numpy order: the last axis is Ocean's first dimension
+             parent[3, 2:9, :, 1:64]]
+    try:
+        for view in views:
+            x = H.Operand(parent, view, H.INT32).upload(stream)
+            want = {}
+            for name in ("sum", "maximum", "minimum", "nnz", "sum_abs"):
+                oh.lib.och_reduce_set_part_limit(0)
+                _, want[name] = gpu_reduce(stream, oh.R[name], H.INT32, x)
+                _, cpu = cpu_reduce(oh.R[name], H.INT32, x)
+                H.assert_same_bytes(want[name], cpu, "one launch " + name)
+            # every limit keeps the number of launches within the 512 that share the slots
+            for limit in (view.size // 2 + 1, 5000, 997) + ((200, 64) if view.ndim == 3 else ()):
+                oh.lib.och_reduce_set_part_limit(limit)
+                for name in want:
+                    _, got = gpu_reduce(stream, oh.R[name], H.INT32, x)
+                    H.assert_same_bytes(got, want[name], "%s with at most %d elements per launch, view %s" % (name, limit, view.shape))
+            x.free()
+        # floating point: order of the fold differs between the cuts, the bound does not
+        pf = rng.standard_normal((40, 50, 30))
+        vf = pf[1:39, ::2, 2:29].transpose(1, 2, 0)
+        x = H.Operand(pf, vf, H.DOUBLE).upload(stream)
+        for limit in (0, 4096, 333):
+            oh.lib.och_reduce_set_part_limit(limit)
+            for name in ("sum", "norm2"):
+                rd, got = gpu_reduce(stream, oh.R[name], H.DOUBLE, x)
+                check_against_truth(name, H.DOUBLE, rd, got, np.ascontiguousarray(vf))
+        # a first dimension that alone exceeds the limit is refused, and the refusal leaves the counter usable
+        oh.lib.och_reduce_set_part_limit(8)
+        out = np.zeros(1, np.float64)
+        assert oh.lib.och_reduce_all(oh.R["sum"], H.DOUBLE, len(x.shape), oh.sizes(x.shape), oh.strides(x.strides), x.dptr(), None, None, 0.0,
+                                     orc.ptr(out), None, stream.handle) == -1
+        assert "first dimension" in oh.lib.och_last_error().decode()
+        oh.lib.och_reduce_set_part_limit(0)
+        rd, got = gpu_reduce(stream, oh.R["sum"], H.DOUBLE, x)
+        check_against_truth("sum", H.DOUBLE, rd, got, np.ascontiguousarray(vf))
+        x.free()
+    finally:
+        oh.lib.och_reduce_set_part_limit(0)
