@@ -12,6 +12,7 @@ namespace och {
 
 int  set_error(const char *fmt, ...);        /* stores the message, returns -1 */
 void clear_error();
+int  gemm_compute_units(void);               /* compute units of the current device (cached per device) */
 void note_status(int hip_error);             /* keeps the first error until och_status_check clears it */
 
 /* Every failing runtime call is also noted in a process-wide status that keeps the FIRST error until

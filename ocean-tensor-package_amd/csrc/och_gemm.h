@@ -568,7 +568,8 @@ int gemm_compute_units(void);
    largest tile. The cheapest candidate wins; within 2 % the larger tile (earlier in the list) is kept. */
 struct GemmTileChoice { int bm, bn; double efficiency; };
 static inline int gemm_pick_tile(const GemmArgs &g, const GemmTileChoice *choice, int n)
-{  const uint64_t units = (uint64_t)gemm_compute_units();
+{  if ((g.M * g.N <= 256 && g.K >= 64) || g.K <= 4) return n - 1;       /* dot and outer products have kernels of their own: no tile to choose */
+   const uint64_t units = (uint64_t)gemm_compute_units();
    int best = 0; double best_cost = 0;
    for (int c = 0; c < n; c++)
    {  const uint64_t tiles = ((g.M + choice[c].bm - 1) / choice[c].bm) * ((g.N + choice[c].bn - 1) / choice[c].bn) * (uint64_t)g.nz;

@@ -25,6 +25,7 @@ namespace och {
 
 #define OCH_RED_BLOCK 256
 #define OCH_RED_UNR 4
+#define OCH_RED_BLOCK_STREAM 512             /* threads of the workgroups that stream a large contiguous source */
 
 template <class A> OCH_D A shfl_xor_any(A v, int mask)
 {
@@ -60,7 +61,7 @@ template <class A> OCH_D void store_shared_global(char *addr, const A &a)
 }
 
 /* reduce across the 256 threads of a block; the result is valid in thread 0 */
-template <class RD> OCH_D typename RD::Acc block_reduce(typename RD::Acc a, typename RD::Acc *lds)
+template <class RD, int BLOCK = OCH_RED_BLOCK> OCH_D typename RD::Acc block_reduce(typename RD::Acc a, typename RD::Acc *lds)
 {
    typedef typename RD::Acc Acc;
 #pragma unroll
@@ -71,7 +72,7 @@ template <class RD> OCH_D typename RD::Acc block_reduce(typename RD::Acc a, type
    if (threadIdx.x == 0)
    {
 #pragma unroll
-      for (int w = 1; w < OCH_RED_BLOCK / 64; w++) a = RD::combine(a, lds[w]);
+      for (int w = 1; w < BLOCK / 64; w++) a = RD::combine(a, lds[w]);
    }
    return a;
 }
@@ -96,6 +97,7 @@ struct RedParams
    every part writes its blocks' partial results into its own range of slots and the block that draws the last ticket
    of the last part folds them all. och_reduce_set_part_limit lowers the number so that small tensors exercise this. */
 #define OCH_RED_PART_LIMIT 0xFFFF0000ull
+#define OCH_RED_MAX_PARTS 512
 uint64_t reduce_part_limit();
 
 /* Cuts `size` (ndims > 1, product above `limit`) into boxes of at most `limit` elements: whole runs of the outermost
@@ -155,39 +157,39 @@ OCH_D void rows_load(const RedParams &p, uint32_t g, Pack<T, VEC> &v, int &lo, i
 
 /* MODE 1 (wide): the first dimension is contiguous, divisible by VEC and aligned: VEC-wide loads (compile-time, so that
    the loads stay single 128-bit instructions); MODE 2: row mode (see rows_load); MODE 0: VEC is 1 and any layout is accepted. */
-template <class RD, class T, int VEC, int MODE, bool NT = false>
-__global__ __launch_bounds__(OCH_RED_BLOCK) void reduce_all_kernel(const RedParams p, const typename RD::Param prm)
+template <class RD, class T, int VEC, int MODE, bool NT = false, int BLOCK = OCH_RED_BLOCK, int UNR = OCH_RED_UNR>
+__global__ __launch_bounds__(BLOCK) void reduce_all_kernel(const RedParams p, const typename RD::Param prm)
 {
    typedef typename RD::Acc Acc;
-   __shared__ Acc lds[OCH_RED_BLOCK / 64];
+   __shared__ Acc lds[BLOCK / 64];
    __shared__ unsigned int ticket;
-   Acc part[OCH_RED_UNR];
+   Acc part[UNR];
 #pragma unroll
-   for (int u = 0; u < OCH_RED_UNR; u++) part[u] = RD::identity();
+   for (int u = 0; u < UNR; u++) part[u] = RD::identity();
    /* every block walks one contiguous range of groups, OCH_RED_BLOCK groups per step, so that
       the loads in flight stay close together in memory (a grid-wide stride is a large power of
       two and lands the concurrent loads on the same memory channels) */
-   const uint64_t stride = OCH_RED_BLOCK;
+   const uint64_t stride = BLOCK;
    uint64_t g = (uint64_t)blockIdx.x * p.per_block + threadIdx.x;
    uint64_t end = (uint64_t)blockIdx.x * p.per_block + p.per_block;
    if (end > p.ngroups) end = p.ngroups;
    const bool flat = (p.ew.ndims == 1);
-   /* main loop: OCH_RED_UNR independent groups per trip, loads first, one accumulator per group */
-   for (; g + (OCH_RED_UNR - 1) * stride < end; g += OCH_RED_UNR * stride)
-   {  Pack<T, VEC> v[OCH_RED_UNR];
+   /* main loop: UNR independent groups per trip, loads first, one accumulator per group */
+   for (; g + (UNR - 1) * stride < end; g += UNR * stride)
+   {  Pack<T, VEC> v[UNR];
       if constexpr (MODE == 2)
-      {  int lo[OCH_RED_UNR], hi[OCH_RED_UNR];
+      {  int lo[UNR], hi[UNR];
 #pragma unroll
-         for (int u = 0; u < OCH_RED_UNR; u++) { v[u] = Pack<T, VEC>{}; rows_load<T, VEC>(p, (uint32_t)(g + u * stride), v[u], lo[u], hi[u]); }
+         for (int u = 0; u < UNR; u++) { v[u] = Pack<T, VEC>{}; rows_load<T, VEC>(p, (uint32_t)(g + u * stride), v[u], lo[u], hi[u]); }
 #pragma unroll
          for (int k = 0; k < VEC; k++)
 #pragma unroll
-            for (int u = 0; u < OCH_RED_UNR; u++) if (k >= lo[u] && k < hi[u]) part[u] = RD::combine(part[u], RD::load(v[u].v[k], prm));
+            for (int u = 0; u < UNR; u++) if (k >= lo[u] && k < hi[u]) part[u] = RD::combine(part[u], RD::load(v[u].v[k], prm));
       }
       else
       {
 #pragma unroll
-         for (int u = 0; u < OCH_RED_UNR; u++)
+         for (int u = 0; u < UNR; u++)
          {  int64_t off[1];
             if (flat) off[0] = (int64_t)(g + u * stride) * p.ew.gstride[0];
             else group_offsets<1>(p.ew, (uint32_t)(g + u * stride), off);
@@ -196,7 +198,7 @@ __global__ __launch_bounds__(OCH_RED_BLOCK) void reduce_all_kernel(const RedPara
 #pragma unroll
          for (int k = 0; k < VEC; k++)
 #pragma unroll
-            for (int u = 0; u < OCH_RED_UNR; u++) part[u] = RD::combine(part[u], RD::load(v[u].v[k], prm));
+            for (int u = 0; u < UNR; u++) part[u] = RD::combine(part[u], RD::load(v[u].v[k], prm));
       }
    }
    for (; g < end; g += stride)
@@ -219,10 +221,10 @@ __global__ __launch_bounds__(OCH_RED_BLOCK) void reduce_all_kernel(const RedPara
    }
    Acc acc = part[0];
 #pragma unroll
-   for (int u = 1; u < OCH_RED_UNR; u++) acc = RD::combine(acc, part[u]);
+   for (int u = 1; u < UNR; u++) acc = RD::combine(acc, part[u]);
    if (blockIdx.x == 0 && (int)threadIdx.x < p.ntail)
       acc = RD::combine(acc, RD::load(*reinterpret_cast<const T *>(p.tail + (int64_t)threadIdx.x * p.ew.estride[0]), prm));
-   acc = block_reduce<RD>(acc, lds);
+   acc = block_reduce<RD, BLOCK>(acc, lds);
    if (threadIdx.x == 0)
    {  store_shared_global<Acc>(p.partials + (size_t)(p.slot_base + blockIdx.x) * OCH_RED_SLOT, acc);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");            /* the write-through stores above have completed */
@@ -232,10 +234,10 @@ __global__ __launch_bounds__(OCH_RED_BLOCK) void reduce_all_kernel(const RedPara
    if (ticket != p.total_blocks - 1) return;
    /* last block: every partial is in memory; fold them in index order */
    acc = RD::identity();
-   for (unsigned int b = threadIdx.x; b < p.total_blocks; b += OCH_RED_BLOCK)
+   for (unsigned int b = threadIdx.x; b < p.total_blocks; b += BLOCK)
       acc = RD::combine(acc, load_shared_global<Acc>(p.partials + (size_t)b * OCH_RED_SLOT));
    __syncthreads();
-   acc = block_reduce<RD>(acc, lds);
+   acc = block_reduce<RD, BLOCK>(acc, lds);
    if (threadIdx.x == 0)
    {  *reinterpret_cast<typename RD::Res *>(p.result) = RD::finalize(acc, prm);
       *p.counter = 0;
@@ -302,18 +304,25 @@ static int launch_reduce_part(const EwShape<1> &shape, const typename Reduce<T, 
    p.partials = scratch;
    p.counter = reinterpret_cast<unsigned int *>(scratch + OCH_RED_MAX_BLOCKS * OCH_RED_SLOT);
    p.result = dresult;
-   uint64_t want = (p.ngroups + (uint64_t)OCH_RED_BLOCK * OCH_RED_UNR - 1) / ((uint64_t)OCH_RED_BLOCK * OCH_RED_UNR);
-   unsigned int blocks = (unsigned int)(want < 1 ? 1 : (want > OCH_RED_MAX_BLOCKS ? OCH_RED_MAX_BLOCKS : want));
+   const bool streaming = wide_launch && p.ngroups * (uint64_t)(sizeof(T) * VEC) >= OCH_EW_STREAM_BYTES;
+   /* Sources that are read once from memory (larger than the caches) carry the nontemporal hint (268 MB of float32
+      are summed at 6.3 TB/s with it and at 5.5 TB/s without) and run as one workgroup of 512 threads per compute
+      unit: every unit starts at once, works through one contiguous range with 2048 loads of 16 bytes in flight and
+      hands in one partial result. Measured on 268 MB of float32 / 537 MB of float64 (GB/s): 256 x 512 threads
+      6530 / 6920; 512 x 256 threads 6190 / 6800; 1024 x 256 5550 / 6450; 4096 x 256 3820 / 5540; 256 x 1024 6160 / 6580;
+      eight or two loads per thread in flight instead of four 6190 / 6660 and 5080 / 5400. */
+   const unsigned int threads = streaming ? OCH_RED_BLOCK_STREAM : OCH_RED_BLOCK;
+   const unsigned int cap = streaming ? (unsigned int)gemm_compute_units() : OCH_RED_MAX_BLOCKS;
+   uint64_t want = (p.ngroups + (uint64_t)threads * OCH_RED_UNR - 1) / ((uint64_t)threads * OCH_RED_UNR);
+   unsigned int blocks = (unsigned int)(want < 1 ? 1 : (want > cap ? cap : want));
+   if (blocks > OCH_RED_MAX_BLOCKS) blocks = OCH_RED_MAX_BLOCKS;
    if (nblocks != 0) blocks = nblocks;                        /* blocks beyond the data fold the identity */
    p.slot_base = slot_base; p.total_blocks = (nblocks != 0) ? total : blocks;
-   {  const uint64_t step = (uint64_t)OCH_RED_BLOCK * OCH_RED_UNR;
+   {  const uint64_t step = (uint64_t)threads * OCH_RED_UNR;
       uint64_t per = (p.ngroups + blocks - 1) / blocks;
       p.per_block = (per + step - 1) / step * step;
    }
-   /* sources that are read once from memory (larger than the caches) carry the nontemporal hint: measured on
-      MI355X, 268 MB of float32 are summed at 6.3 TB/s with the hint and at 5.5 TB/s without */
-   const bool streaming = wide_launch && p.ngroups * (uint64_t)(sizeof(T) * VEC) >= OCH_EW_STREAM_BYTES;
-   if (streaming)        hipLaunchKernelGGL((reduce_all_kernel<RD, T, VEC, 1, true>), dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
+   if (streaming)        hipLaunchKernelGGL((reduce_all_kernel<RD, T, VEC, 1, true, OCH_RED_BLOCK_STREAM>), dim3(blocks), dim3(OCH_RED_BLOCK_STREAM), 0, stream, p, prm);
    else if (wide_launch) hipLaunchKernelGGL((reduce_all_kernel<RD, T, VEC, 1>), dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm);
    else if (rows_launch)
    {  if constexpr (VEC > 1) hipLaunchKernelGGL((reduce_all_kernel<RD, T, VEC, 2>), dim3(blocks), dim3(OCH_RED_BLOCK), 0, stream, p, prm); }
@@ -345,15 +354,15 @@ static int launch_reduce_all(int ndims, const size_t *size, const ptrdiff_t *str
    if (shape.ndims > 1 && shape.nelem > limit)
    {  /* more elements than one launch indexes: one launch per box, all of them sharing the slots and the counter */
       struct Box { uint64_t start[OCH_MAX_DIMS], count[OCH_MAX_DIMS]; };
-      Box boxes[OCH_RED_MAX_BLOCKS];                         /* on the stack: this path allocates nothing, on the host either */
+      Box boxes[OCH_RED_MAX_PARTS];                         /* on the stack: this path allocates nothing, on the host either */
       int64_t kept = 0;
       const int64_t n = reduce_cut_parts(shape.ndims, shape.size, limit, [&](const uint64_t *start, const uint64_t *count)
-                        {  if (kept < OCH_RED_MAX_BLOCKS)
+                        {  if (kept < OCH_RED_MAX_PARTS)
                            {  Box &b = boxes[kept++]; for (int d = 0; d < shape.ndims; d++) { b.start[d] = start[d]; b.count[d] = count[d]; } }
                         });
       if (n < 0) return set_error("reduction: the first dimension of a strided tensor exceeds %llu elements", (unsigned long long)limit);
-      if (n > OCH_RED_MAX_BLOCKS) return set_error("reduction: the tensor needs %lld launches, more than the %d that share the partial results", (long long)n, OCH_RED_MAX_BLOCKS);
-      const unsigned int each = (unsigned int)(OCH_RED_MAX_BLOCKS / n), total = each * (unsigned int)n;
+      if (n > OCH_RED_MAX_PARTS) return set_error("reduction: the tensor needs %lld launches, more than the %d that share the partial results", (long long)n, OCH_RED_MAX_PARTS);
+      const unsigned int each = (unsigned int)(OCH_RED_MAX_PARTS / n), total = each * (unsigned int)n;
       unsigned int base = 0;
       for (int64_t k = 0; k < n; k++)
       {  const Box &b = boxes[k];
