@@ -438,7 +438,7 @@ int och_find_apply(int ndims, const size_t *size, const ptrdiff_t *strides, void
 /* each dimension in the kernels. The last operand is the destination.      */
 /* Needs no GPU.                                                            */
 /* ======================================================================== */
-enum { OCH_KERNEL_WIDE = 0, OCH_KERNEL_MIXED = 1, OCH_KERNEL_SINGLE = 2, OCH_KERNEL_TILED = 3 };
+enum { OCH_KERNEL_WIDE = 0, OCH_KERNEL_MIXED = 1, OCH_KERNEL_SINGLE = 2, OCH_KERNEL_TILED = 3, OCH_KERNEL_ROWS = 4 };
 typedef struct {
    int        ndims;
    size_t     size[OCH_MAX_DIMS];
@@ -448,9 +448,20 @@ typedef struct {
    int        vec;                        /* elements per access in that launch */
    int        launches;                   /* kernel launches for the whole call */
    unsigned   div_d[OCH_MAX_DIMS], div_m[OCH_MAX_DIMS], div_s1[OCH_MAX_DIMS], div_s2[OCH_MAX_DIMS];
+   unsigned   row_units;                  /* OCH_KERNEL_ROWS: work items per row of dimension 0 */
+   size_t     row_elements;               /* OCH_KERNEL_ROWS: elements in such a row */
 } och_elemwise_plan;
 int och_elemwise_analyze(int noperands, const int *elemsize, int ndims, const size_t *size,
                          const ptrdiff_t *const *strides, void *const *ptrs, och_elemwise_plan *plan);
+/* OCH_KERNEL_ROWS (unit-stride rows that are not whole aligned vectors: an odd width, a start or a pitch that is not  */
+/* a multiple of the vector width): a work item is one aligned unit of `vec` elements of a destination row. For unit   */
+/* number `unit` of a row of row_elements elements of elemsize bytes that starts `misalignment` bytes into such a unit: */
+/* *first = row position of the unit's element 0 (negative in a first unit that begins in front of the row), [lo, hi)  */
+/* = its elements inside the row; returns 1 when there are any, else 0. Units with lo = 0 and hi = vec move with one   */
+/* access per operand, the others element by element. och_elemwise_row_units: units given to every row.                */
+int och_elemwise_row_unit(unsigned unit, int misalignment, int elemsize, int vec, size_t row_elements,
+                          long long *first, int *lo, int *hi);
+size_t och_elemwise_row_units(size_t row_elements, int elemsize, int vec);
 
 #ifdef __cplusplus
 }

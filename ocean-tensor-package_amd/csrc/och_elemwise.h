@@ -59,6 +59,7 @@ template <int NOPS> struct EwParams
    int      nt;                            /* streaming launch: wide accesses carry the nontemporal hint */
    uint32_t unr;                           /* groups per thread of this launch (at most the kernel's UNR) */
    uint32_t block;                         /* threads per workgroup of this launch */
+   uint64_t row_n0;                        /* row kernels: elements in a row of dimension 0 (div[0] then divides by the chunks of a row) */
 };
 
 template <class T, int VEC> struct alignas((sizeof(T) * VEC) > 16 ? 16 : (sizeof(T) * VEC)) Pack { T v[VEC]; };
@@ -98,6 +99,19 @@ OCH_D void store_wide(const Pack<T, VEC> &p, char *addr)
    __builtin_memcpy(&raw, &p, sizeof(V));
    if constexpr (NT) __builtin_nontemporal_store(raw, reinterpret_cast<V *>(addr));
    else    *reinterpret_cast<V *>(addr) = raw;
+}
+
+/* A pack read from an address that is only aligned to its element: one load instruction all the same (the device runs
+   with unaligned access enabled; the under-aligned vector type tells the compiler not to assume more). */
+template <class T, int VEC, bool NT = false>
+OCH_D void load_unaligned(Pack<T, VEC> &p, const char *addr)
+{
+   typedef typename RawVec<sizeof(Pack<T, VEC>)>::type V;
+   typedef V __attribute__((aligned(alignof(T) < sizeof(V) ? alignof(T) : sizeof(V)))) VU;
+   V raw;
+   if constexpr (NT) raw = __builtin_nontemporal_load(reinterpret_cast<const VU *>(addr));
+   else    raw = *reinterpret_cast<const VU *>(addr);
+   __builtin_memcpy(&p, &raw, sizeof(V));
 }
 
 /* Source elements one apart (a step-2 slice along the first dimension): the 2 VEC consecutive elements that hold the
@@ -295,6 +309,130 @@ __global__ __launch_bounds__(OCH_EW_MAX_BLOCK) void ew1_kernel(const EwParams<1>
 #pragma unroll
          for (int k = 0; k < VEC; k++) r.v[k] = F::f(r.v[k], p.group0 + (uint64_t)g * VEC + k, prm);
          store_pack<R, VEC, NT>(r, p.ptr[0] + off[0], p.estride[0], FAST ? 1 : p.vecmode[0]);
+      }
+   }
+}
+
+
+/* ---- row kernels: unit-stride rows that are not whole aligned vectors ----------
+   A sub-matrix whose width is not a multiple of VEC, whose rows start inside a 16-byte unit or whose pitch is not a
+   multiple of 16 bytes cannot take the all-wide kernels, and with one element per thread 1- and 2-byte types move a
+   byte or two per lane and instruction. Here a work item is one ALIGNED unit of a destination row (VEC elements,
+   WD = VEC * sizeof(R) <= 16 bytes): units that lie inside the row are written with one wide store, and their inputs are
+   read with one load each from wherever the same elements lie in the input rows (aligned to the element only); the
+   units at the two ends of a row hold fewer elements and move them one by one, so no byte outside a row is ever
+   written, nor read. Every row gets the number of units of the worst-placed row; units left over do nothing.
+   Inputs that are not unit-stride along the row (a broadcast, a stepped or transposed view) are read element by
+   element (vecmode 0). */
+/* Unit c of a destination row of n0 elements of esr bytes that starts m bytes into an aligned unit of `vec` elements:
+   row position e0 of the unit's element 0 (negative in the first unit when m > 0) and the range [lo, hi) of its
+   elements that lie inside the row; false when there are none. */
+__host__ __device__ inline bool row_unit_range(uint32_t c, int m, int esr, int vec, uint64_t n0, int64_t &e0, int &lo, int &hi)
+{
+   e0 = (int64_t)c * vec - m / esr;
+   const int64_t left = (int64_t)n0 - e0;
+   lo = (e0 < 0) ? (int)(-e0) : 0;
+   hi = (left >= vec) ? vec : (left > 0 ? (int)left : 0);
+   return hi > lo;
+}
+/* units every row is given: those of a row that starts on the last element of an aligned unit */
+static inline uint64_t row_units(uint64_t n0, int esr, int vec)
+{  const uint64_t wd = (uint64_t)vec * esr;
+   return (wd - esr + n0 * esr + wd - 1) / wd;
+}
+
+template <int NOPS>
+OCH_D bool row_unit(const EwParams<NOPS> &p, uint32_t g, int wd, int esr, int vec, int64_t (&off)[NOPS], int64_t &e0, int &lo, int &hi)
+{
+   const uint32_t r = fastdiv(g, p.div[0]), c = g - r * p.div[0].d;
+#pragma unroll
+   for (int k = 0; k < NOPS; k++) off[k] = 0;
+   uint32_t q = r;
+   for (int d = 1; d < p.ndims - 1; d++)
+   {  const uint32_t q2 = fastdiv(q, p.div[d]), i = q - q2 * p.div[d].d; q = q2;
+#pragma unroll
+      for (int k = 0; k < NOPS; k++) off[k] += (int64_t)i * p.stride[k][d];
+   }
+   if (p.ndims > 1)
+   {
+#pragma unroll
+      for (int k = 0; k < NOPS; k++) off[k] += (int64_t)q * p.stride[k][p.ndims - 1];
+   }
+   const int m = (int)((uintptr_t)(p.ptr[NOPS - 1] + off[NOPS - 1]) & (uintptr_t)(wd - 1));    /* bytes of the first unit in front of the row */
+   return row_unit_range(c, m, esr, vec, p.row_n0, e0, lo, hi);
+}
+
+template <class F, int VEC, bool NT = false>
+__global__ __launch_bounds__(OCH_EW_BLOCK) void ew3_rows_kernel(const EwParams<3> p)
+{
+   typedef typename F::A A; typedef typename F::B B; typedef typename F::R R;
+   const uint32_t g = blockIdx.x * OCH_EW_BLOCK + threadIdx.x;
+   if (g >= p.ngroups) return;
+   int64_t off[3], e0; int lo, hi;
+   if (!row_unit<3>(p, g, VEC * (int)sizeof(R), (int)sizeof(R), VEC, off, e0, lo, hi)) return;
+   const char *pa = p.ptr[0] + off[0] + e0 * p.estride[0], *pb = p.ptr[1] + off[1] + e0 * p.estride[1];
+   char *pr = p.ptr[2] + off[2] + e0 * (int64_t)sizeof(R);
+   if (lo == 0 && hi == VEC)
+   {  Pack<A, VEC> a; Pack<B, VEC> b; Pack<R, VEC> r;
+      if (p.vecmode[0]) load_unaligned<A, VEC, NT>(a, pa); else load_pack<A, VEC>(a, pa, p.estride[0], 0);
+      if (p.vecmode[1]) load_unaligned<B, VEC, NT>(b, pb); else load_pack<B, VEC>(b, pb, p.estride[1], 0);
+#pragma unroll
+      for (int k = 0; k < VEC; k++) r.v[k] = F::f(a.v[k], b.v[k]);
+      store_wide<R, VEC, NT>(r, pr);
+   }
+   else
+   {  for (int k = lo; k < hi; k++)
+         *reinterpret_cast<R *>(pr + k * (int64_t)sizeof(R)) =
+            F::f(*reinterpret_cast<const A *>(pa + k * p.estride[0]), *reinterpret_cast<const B *>(pb + k * p.estride[1]));
+   }
+}
+
+template <class F, int VEC, bool NT = false>
+__global__ __launch_bounds__(OCH_EW_BLOCK) void ew2_rows_kernel(const EwParams<2> p)
+{
+   typedef typename F::A A; typedef typename F::R R;
+   const uint32_t g = blockIdx.x * OCH_EW_BLOCK + threadIdx.x;
+   if (g >= p.ngroups) return;
+   int64_t off[2], e0; int lo, hi;
+   if (!row_unit<2>(p, g, VEC * (int)sizeof(R), (int)sizeof(R), VEC, off, e0, lo, hi)) return;
+   const char *pa = p.ptr[0] + off[0] + e0 * p.estride[0];
+   char *pr = p.ptr[1] + off[1] + e0 * (int64_t)sizeof(R);
+   if (lo == 0 && hi == VEC)
+   {  Pack<A, VEC> a; Pack<R, VEC> r;
+      if (p.vecmode[0]) load_unaligned<A, VEC, NT>(a, pa); else load_pack<A, VEC>(a, pa, p.estride[0], 0);
+#pragma unroll
+      for (int k = 0; k < VEC; k++) r.v[k] = F::f(a.v[k]);
+      store_wide<R, VEC, NT>(r, pr);
+   }
+   else
+   {  for (int k = lo; k < hi; k++)
+         *reinterpret_cast<R *>(pr + k * (int64_t)sizeof(R)) = F::f(*reinterpret_cast<const A *>(pa + k * p.estride[0]));
+   }
+}
+
+/* x = f(x, flat index, param) on rows: the flat index of an element is its row times the row length plus its position */
+template <class F, int VEC, bool NT = false>
+__global__ __launch_bounds__(OCH_EW_BLOCK) void ew1_rows_kernel(const EwParams<1> p, const typename F::Param prm)
+{
+   typedef typename F::R R;
+   const uint32_t g = blockIdx.x * OCH_EW_BLOCK + threadIdx.x;
+   if (g >= p.ngroups) return;
+   int64_t off[1], e0; int lo, hi;
+   if (!row_unit<1>(p, g, VEC * (int)sizeof(R), (int)sizeof(R), VEC, off, e0, lo, hi)) return;
+   char *pr = p.ptr[0] + off[0] + e0 * (int64_t)sizeof(R);
+   const uint64_t flat = p.group0 + (uint64_t)fastdiv(g, p.div[0]) * p.row_n0 + (uint64_t)e0;     /* of element 0 of the unit (wraps back for k >= lo) */
+   if (lo == 0 && hi == VEC)
+   {  Pack<R, VEC> r;
+      if constexpr (F::RMW) load_wide<R, VEC>(r, pr);
+#pragma unroll
+      for (int k = 0; k < VEC; k++) r.v[k] = F::f(r.v[k], flat + k, prm);
+      store_wide<R, VEC, NT>(r, pr);
+   }
+   else
+   {  for (int k = lo; k < hi; k++)
+      {  R x{};
+         if constexpr (F::RMW) x = *reinterpret_cast<const R *>(pr + k * (int64_t)sizeof(R));
+         *reinterpret_cast<R *>(pr + k * (int64_t)sizeof(R)) = F::f(x, flat + k, prm);
       }
    }
 }
@@ -654,6 +792,58 @@ static bool ew_params(EwParams<NOPS> &p, const EwShape<NOPS> &s, int vec, const 
    return true;
 }
 
+/* Parameters of the row kernels, or false when they do not apply: the destination (last operand) must have unit stride
+   along dimension 0 and rows of at least 24 bytes, every operand must be aligned to its element, and the units of all
+   rows must be countable in 32 bits. */
+template <int NOPS>
+static bool ew_rows_params(EwParams<NOPS> &p, const EwShape<NOPS> &s, int vec, const int elemsize[NOPS], uint64_t flat0)
+{
+   const int out = NOPS - 1;
+   if (vec <= 1 || s.nelem == 0 || s.stride[out][0] != elemsize[out]) return false;
+   const uint64_t n0 = s.size[0];
+   if (n0 * elemsize[out] < 24) return false;
+   for (int k = 0; k < NOPS; k++)
+   {  if (((uintptr_t)s.ptr[k]) % elemsize[k] != 0) return false;
+      for (int d = 0; d < s.ndims; d++) if (s.stride[k][d] % elemsize[k] != 0) return false;
+   }
+   const uint64_t chunks = row_units(n0, elemsize[out], vec);
+   const uint64_t rows = s.nelem / n0;
+   if (chunks > 0xFFFFFFFFull || rows * chunks > 0xFFFF0000ull) return false;
+   p.ndims = s.ndims;
+   p.unr = 1; p.block = OCH_EW_BLOCK;
+   p.ngroups = (uint32_t)(rows * chunks);
+   p.group0 = flat0;
+   p.row_n0 = n0;
+   {  uint64_t bytes = 0;
+      for (int k = 0; k < NOPS; k++) bytes += s.nelem * (uint64_t)elemsize[k];
+      p.nt = (bytes >= OCH_EW_STREAM_BYTES) ? 1 : 0;
+   }
+   p.div[0] = make_fastdiv((uint32_t)chunks);
+   for (int d = 1; d < s.ndims; d++) p.div[d] = make_fastdiv((uint32_t)s.size[d]);
+   for (int k = 0; k < NOPS; k++)
+   {  p.ptr[k] = s.ptr[k];
+      p.estride[k] = s.stride[k][0];
+      p.gstride[k] = s.stride[k][0] * vec;
+      for (int d = 0; d < OCH_MAX_DIMS; d++) p.stride[k][d] = (d < s.ndims) ? s.stride[k][d] : 0;
+      p.vecmode[k] = (s.stride[k][0] == elemsize[k]) ? 1 : 0;
+   }
+   return true;
+}
+
+template <int NOPS>
+static bool ew_rows_wanted(const EwShape<NOPS> &s, int vec, const int elemsize[NOPS])
+{
+   if (vec <= 1) return false;
+   bool misfit = (s.ndims > 1 && s.size[0] % vec != 0);
+   for (int k = 0; k < NOPS; k++)
+   {  if (s.stride[k][0] != elemsize[k]) continue;
+      int width = elemsize[k] * vec; if (width > 16) width = 16;
+      if (((uintptr_t)s.ptr[k]) % width != 0) misfit = true;
+      for (int d = 1; d < s.ndims; d++) if (s.stride[k][d] % width != 0) misfit = true;
+   }
+   return misfit;
+}
+
 template <class T> constexpr int vec_for() { return (16 / (int)sizeof(T)) > 0 ? (16 / (int)sizeof(T)) : 1; }
 template <class A, class B, class C> constexpr int vec_for3()
 {  constexpr int m = sizeof(A) > sizeof(B) ? (sizeof(A) > sizeof(C) ? sizeof(A) : sizeof(C)) : (sizeof(B) > sizeof(C) ? sizeof(B) : sizeof(C));
@@ -668,11 +858,20 @@ template <class A, class B, class C> constexpr int vec_for3()
      mixed : dim 0 divisible by VEC, some operands strided or broadcast
      single: one element per thread (odd sizes); for 1-D shapes only the tail uses it   */
 /* Launcher signature: (parameters, workgroups, threads per workgroup) */
-template <int NOPS, class LW, class LM, class LS>
+template <int NOPS, class LW, class LM, class LS, class LR>
 static int ew_dispatch(const EwShape<NOPS> &s, uint64_t flat0, int vec, const int (&es)[NOPS],
-                       LW &&wide, LM &&mixed, LS &&single)
+                       LW &&wide, LM &&mixed, LS &&single, LR &&rows)
 {
    EwParams<NOPS> p;
+   /* unit-stride rows that are not whole aligned vectors (see the row kernels): a width that VEC does not divide (a
+      one-dimensional shape of such a length is cut into body and tail below instead), or a unit-stride operand whose
+      start or pitch is not a multiple of its vector width */
+   {  if (ew_rows_wanted<NOPS>(s, vec, es) && ew_rows_params<NOPS>(p, s, vec, es, flat0))
+      {  rows(p, (p.ngroups + OCH_EW_BLOCK - 1) / OCH_EW_BLOCK, (uint32_t)OCH_EW_BLOCK);
+         OCH_CHECK_LAUNCH();
+         return 0;
+      }
+   }
    auto run = [&](const EwShape<NOPS> &sh, uint64_t f0) -> bool
    {  if (!ew_params<NOPS>(p, sh, vec, es, f0, NOPS - 1)) return false;      /* vec = 1 (16-byte elements) always fits */
       bool all = true;
@@ -804,7 +1003,12 @@ static int launch_ew3(int ndims, const size_t *size,
             if (p.nt) hipLaunchKernelGGL((ew3_kernel<F, VEC, 2, false, true>), dim3(blocks), dim3(threads), 0, stream, p);
             else      hipLaunchKernelGGL((ew3_kernel<F, VEC, 2, false, false>), dim3(blocks), dim3(threads), 0, stream, p); },
          [&](const EwParams<3> &p, uint32_t blocks, uint32_t threads)
-         {  hipLaunchKernelGGL((ew3_kernel<F, 1, 1, false>), dim3(blocks), dim3(threads), 0, stream, p); });
+         {  hipLaunchKernelGGL((ew3_kernel<F, 1, 1, false>), dim3(blocks), dim3(threads), 0, stream, p); },
+         [&](const EwParams<3> &p, uint32_t blocks, uint32_t threads)
+         {  if constexpr (VEC > 1)
+            {  if (p.nt) hipLaunchKernelGGL((ew3_rows_kernel<F, VEC, true>), dim3(blocks), dim3(threads), 0, stream, p);
+               else      hipLaunchKernelGGL((ew3_rows_kernel<F, VEC, false>), dim3(blocks), dim3(threads), 0, stream, p);
+            } });
    });
 }
 
@@ -837,7 +1041,12 @@ static int launch_ew2(int ndims, const size_t *size,
          {  if (p.nt) hipLaunchKernelGGL((ew2_kernel<F, VEC, 2, false, true>), dim3(blocks), dim3(threads), 0, stream, p);
             else      hipLaunchKernelGGL((ew2_kernel<F, VEC, 2, false, false>), dim3(blocks), dim3(threads), 0, stream, p); },
          [&](const EwParams<2> &p, uint32_t blocks, uint32_t threads)
-         {  hipLaunchKernelGGL((ew2_kernel<F, 1, 1, false>), dim3(blocks), dim3(threads), 0, stream, p); });
+         {  hipLaunchKernelGGL((ew2_kernel<F, 1, 1, false>), dim3(blocks), dim3(threads), 0, stream, p); },
+         [&](const EwParams<2> &p, uint32_t blocks, uint32_t threads)
+         {  if constexpr (VEC > 1)
+            {  if (p.nt) hipLaunchKernelGGL((ew2_rows_kernel<F, VEC, true>), dim3(blocks), dim3(threads), 0, stream, p);
+               else      hipLaunchKernelGGL((ew2_rows_kernel<F, VEC, false>), dim3(blocks), dim3(threads), 0, stream, p);
+            } });
    });
 }
 
@@ -860,7 +1069,12 @@ static int launch_ew1(int ndims, const size_t *size, const ptrdiff_t *st, void *
          [&](const EwParams<1> &p, uint32_t blocks, uint32_t threads)
          {  hipLaunchKernelGGL((ew1_kernel<F, VEC, 2, false>), dim3(blocks), dim3(threads), 0, stream, p, prm); },
          [&](const EwParams<1> &p, uint32_t blocks, uint32_t threads)
-         {  hipLaunchKernelGGL((ew1_kernel<F, 1, 1, false>), dim3(blocks), dim3(threads), 0, stream, p, prm); });
+         {  hipLaunchKernelGGL((ew1_kernel<F, 1, 1, false>), dim3(blocks), dim3(threads), 0, stream, p, prm); },
+         [&](const EwParams<1> &p, uint32_t blocks, uint32_t threads)
+         {  if constexpr (VEC > 1)
+            {  if (p.nt) hipLaunchKernelGGL((ew1_rows_kernel<F, VEC, true>), dim3(blocks), dim3(threads), 0, stream, p, prm);
+               else      hipLaunchKernelGGL((ew1_rows_kernel<F, VEC, false>), dim3(blocks), dim3(threads), 0, stream, p, prm);
+            } });
    });
 }
 

@@ -38,6 +38,10 @@ static int analyze(const int *elemsize, int ndims, const size_t *size, const ptr
          tiled = ew_tile_params<NOPS>(tp, s, esr, tile, vec, grid, lds, tbr);
       }
       if (tiled) { kernel = OCH_KERNEL_TILED; v = vec; }
+      else if (ew_rows_wanted<NOPS>(s, vec, es) && ew_rows_params<NOPS>(p, s, vec, es, flat0))
+      {  kernel = OCH_KERNEL_ROWS; v = vec;
+         if (first) { plan->row_units = p.div[0].d; plan->row_elements = (size_t)p.row_n0; }
+      }
       else if (ew_params<NOPS>(p, s, vec, es, flat0))
       {  bool all = true;
          for (int k = 0; k < NOPS; k++) all = all && (p.vecmode[k] == 1);
@@ -68,6 +72,14 @@ static int analyze(const int *elemsize, int ndims, const size_t *size, const ptr
 } /* namespace och */
 
 using namespace och;
+
+extern "C" int och_elemwise_row_unit(unsigned unit, int misalignment, int elemsize, int vec, size_t row_elements,
+                                     long long *first, int *lo, int *hi)
+{  int64_t e0; const bool any = row_unit_range(unit, misalignment, elemsize, vec, row_elements, e0, *lo, *hi);
+   *first = e0;
+   return any ? 1 : 0;
+}
+extern "C" size_t och_elemwise_row_units(size_t row_elements, int elemsize, int vec) { return (size_t)row_units(row_elements, elemsize, vec); }
 
 extern "C" int och_elemwise_analyze(int noperands, const int *elemsize, int ndims, const size_t *size,
                                     const ptrdiff_t *const *strides, void *const *ptrs, och_elemwise_plan *plan)

@@ -87,10 +87,11 @@ def make_scalar(dtype, value):
 class ElemwisePlan(C.Structure):
     _fields_ = [("ndims", C.c_int), ("size", C.c_size_t * 8), ("strides", (C.c_ssize_t * 8) * 3), ("offset", C.c_ssize_t * 3),
                 ("kernel", C.c_int), ("vec", C.c_int), ("launches", C.c_int),
-                ("div_d", C.c_uint * 8), ("div_m", C.c_uint * 8), ("div_s1", C.c_uint * 8), ("div_s2", C.c_uint * 8)]
+                ("div_d", C.c_uint * 8), ("div_m", C.c_uint * 8), ("div_s1", C.c_uint * 8), ("div_s2", C.c_uint * 8),
+                ("row_units", C.c_uint), ("row_elements", C.c_size_t)]
 
 
-KERNEL_WIDE, KERNEL_MIXED, KERNEL_SINGLE, KERNEL_TILED = 0, 1, 2, 3
+KERNEL_WIDE, KERNEL_MIXED, KERNEL_SINGLE, KERNEL_TILED, KERNEL_ROWS = 0, 1, 2, 3, 4
 
 
 def elemwise_analyze(elemsizes, size, strides_per_operand, addresses):
@@ -208,6 +209,8 @@ PROTOTYPES = {
     "och_find_count": (_i, [_i, _sz, _st, _vp, _vp, C.POINTER(C.c_size_t), _vp]),
     "och_find_apply": (_i, [_i, _sz, _st, _vp, _vp, C.POINTER(C.c_int64), _vp, _vp]),
     "och_elemwise_analyze": (_i, [_i, C.POINTER(_i), _i, _sz, C.POINTER(_st), C.POINTER(_vp), C.c_void_p]),
+    "och_elemwise_row_unit": (_i, [C.c_uint, _i, _i, _i, C.c_size_t, C.POINTER(C.c_longlong), C.POINTER(_i), C.POINTER(_i)]),
+    "och_elemwise_row_units": (C.c_size_t, [C.c_size_t, _i, _i]),
     "och_membench": (_i, [_i, _i, _i, _i, _i, _i, C.c_size_t, _i, _i, C.POINTER(C.c_float), C.POINTER(C.c_float), C.POINTER(C.c_size_t), _vp]),
 }
 

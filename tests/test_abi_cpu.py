@@ -163,8 +163,11 @@ def test_normalisation_preserves_offsets(case):
     # no two neighbouring dimensions are still mergeable
     for d in range(plan.ndims - 1):
         assert not all(nstr[k][d + 1] == nstr[k][d] * nsize[d] for k in range(len(es)))
-    assert plan.kernel in (oh.KERNEL_WIDE, oh.KERNEL_MIXED, oh.KERNEL_SINGLE, oh.KERNEL_TILED)
-    if plan.kernel != oh.KERNEL_SINGLE:
+    assert plan.kernel in (oh.KERNEL_WIDE, oh.KERNEL_MIXED, oh.KERNEL_SINGLE, oh.KERNEL_TILED, oh.KERNEL_ROWS)
+    if plan.kernel == oh.KERNEL_ROWS:
+        assert nstr[-1][0] == es[-1] and nsize[0] * es[-1] >= 24 and plan.row_elements == nsize[0]
+        assert plan.row_units == oh.lib.och_elemwise_row_units(nsize[0], es[-1], plan.vec)
+    elif plan.kernel != oh.KERNEL_SINGLE:
         assert nsize[0] % plan.vec == 0 or plan.ndims == 1
 
 
@@ -183,8 +186,19 @@ def test_kernel_choice():
     # odd length: vector body + scalar tail
     p = oh.elemwise_analyze([4, 4, 4], [4099], [[4]] * 3, [a, a, a])
     assert (p.kernel, p.launches) == (oh.KERNEL_WIDE, 2)
-    # misaligned pointer: cannot use wide accesses
+    # misaligned pointer of a unit-stride operand: aligned units of the destination, inputs read where they lie
     p = oh.elemwise_analyze([4, 4, 4], [4096], [[4]] * 3, [a + 4, a, a])
+    assert p.kernel == oh.KERNEL_ROWS and p.vec == 4 and p.row_units == (12 + 4096 * 4 + 15) // 16
+    # odd width of a sub-matrix, odd pitch, start inside a unit: rows
+    p = oh.elemwise_analyze([1, 1], [999, 37], [[1, 1001], [1, 1001]], [a + 3, a + 5])
+    assert p.kernel == oh.KERNEL_ROWS and p.vec == 16 and p.row_elements == 999 and p.row_units == (15 + 999 + 15) // 16
+    # rows shorter than 24 bytes stay with one element per thread; a destination that is not unit-stride too
+    p = oh.elemwise_analyze([1, 1], [21, 37], [[1, 64], [1, 64]], [a, a])
+    assert p.kernel == oh.KERNEL_SINGLE
+    p = oh.elemwise_analyze([2, 2], [999, 37], [[2, 2048], [4, 4096]], [a, a])
+    assert p.kernel == oh.KERNEL_SINGLE
+    # a broadcast input next to aligned operands is no reason for rows
+    p = oh.elemwise_analyze([4, 4, 4], [4096, 8], [[4, 16384], [0, 4], [4, 16384]], [a, a, a])
     assert p.kernel == oh.KERNEL_MIXED
     # more than 2^32 elements: several launches
     p = oh.elemwise_analyze([1], [1 << 33], [[1]], [a])
@@ -232,3 +246,30 @@ def test_cutting_a_large_reduction_into_launches():
             assert (seen == 1).all(), (size, limit)
         # a full run holds more than half the limit and at most one run per outer index is partial: under four times the minimum
         assert n <= 4 * -(-want // limit), (size, limit, n)
+
+
+def test_units_of_a_row_partition_it():
+    """The row kernels' work items: for every width, element size and placement of a row the ranges [lo, hi) of its units
+    cover the row exactly once; units that take the one-access path (lo = 0, hi = vec) start on an aligned address; no
+    unit reaches outside the row; the number of units given to every row is enough for the worst placement."""
+    first, lo, hi = C.c_longlong(), C.c_int(), C.c_int()
+    for es in (1, 2, 4, 8):
+        for vec in {16 // es, max(1, 8 // es), max(1, 4 // es)} - {1}:
+            wd = vec * es
+            for n0 in list(range(1, 70)) + [255, 256, 257, 1000, 1001, 4097]:
+                units = oh.lib.och_elemwise_row_units(n0, es, vec)
+                for m in range(0, wd, es):
+                    covered = np.zeros(n0, np.int32)
+                    for c in range(units + 2):
+                        any_ = oh.lib.och_elemwise_row_unit(c, m, es, vec, n0, C.byref(first), C.byref(lo), C.byref(hi))
+                        if not any_:
+                            assert hi.value <= lo.value
+                            continue
+                        assert c < units, (es, vec, n0, m, c)
+                        assert 0 <= lo.value < hi.value <= vec
+                        a, b = first.value + lo.value, first.value + hi.value
+                        assert 0 <= a and b <= n0
+                        covered[a:b] += 1
+                        if lo.value == 0 and hi.value == vec:
+                            assert (m + first.value * es) % wd == 0
+                    assert (covered == 1).all(), (es, vec, n0, m)
