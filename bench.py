@@ -31,7 +31,10 @@ Printed: ONE JSON line with the driver's fields plus
                   this host: the full-size step, and bounded samples of the other configurations
 
 --only NAME runs one configuration with few samples and then a plain float64 copy of known size
-(the yardstick that scales the FETCH_SIZE / WRITE_SIZE counters of a profiling run).
+(the yardstick that scales the FETCH_SIZE / WRITE_SIZE counters of a profiling run). In such a run a
+one-byte fill (a single workgroup of fill_bytes_kernel) precedes every measured kernel, and the JSON
+line lists the measured kernels in that order under "segments", so that the dispatches of a counter
+run can be told apart.
 --ceiling prints the whole sweep of the streaming micro-benchmark as a table.
 """
 import argparse
@@ -137,6 +140,10 @@ def main():
         two events on the launch stream (so the events' own cost is spread; at least ~0.6 ms per sample)"""
         samples = samples or SAMPLES
         e0, e1 = oh.Event(), oh.Event()
+        if profiling:
+            # a one-byte fill in front of every measured kernel: in a counter run the dispatches between two of these
+            # single-workgroup fills belong to one entry of "segments"
+            oh.check(lib.och_memset_async(separator.ptr, 0, 1, h))
         for _ in range(warm):
             fn()
         e0.record(stream); fn(); fn(); e1.record(stream); e1.synchronize()
@@ -169,6 +176,8 @@ def main():
             m = min(block.nbytes, nbytes - off) // block.itemsize
             buf.upload(block[:m], offset=off)
 
+    segments = []                      # names of the measured kernels in launch order (profiling runs)
+    separator = oh.DeviceBuffer(256, stream)
     traffic_table = {}
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
@@ -176,6 +185,7 @@ def main():
             traffic_table = json.load(f)
 
     def with_traffic(entry, name):
+        segments.append(name)
         t = traffic_table.get(name)
         if t:
             entry["traffic_MB"] = round((t["fetch_bytes"] + t["write_bytes"]) / 1e6, 1)
@@ -288,7 +298,7 @@ def main():
         result["roofline"] = {"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                               "frac": round(dom["GBps"] / HBM_PEAK_GBS, 3),
                               "traffic": dom.get("traffic_GBps"),
-                              "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --only c2`, scaled by a float64 copy of known size)" if t else None,
+                              "traffic_source": "profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --only c1|c2|c3|c4`, scaled by a float64 copy of known size)" if t else None,
                               "algorithmic_bytes_per_launch": next(b for nm, _, b, _ in step_kernels if nm == dom["kernel"]),
                               "traffic_bytes_per_launch": (t["fetch_bytes"] + t["write_bytes"]) if t else None,
                               "launch_ms": dom["ms"], "best_launch_ms": dom["best_ms"], "samples": SAMPLES,
@@ -561,6 +571,7 @@ def main():
         oh.check(lib.och_copy(F64, F64, 2, shape, st_f64, ya.ptr, 2, shape, st_f64, yb.ptr, h))
         stream.synchronize()
         result["mode"] = "only " + args.only
+        result["segments"] = segments
         print(json.dumps(result))
         return
 
