@@ -119,6 +119,44 @@ struct HalfSlab
          }
       }
    }
+   /* the same in single instructions, for loops that place every one of them by hand: load number v (whole tiles only),
+      and store number `piece` of the NV = 8 that move the registers to LDS */
+   /* address of load v = the slab's first element (the same for all threads: mat + element (mn0, k0)) + a step per v that is
+      the same for all threads + the thread's own offset, which does not change from slab to slab: a scalar base and a
+      32-bit vector offset, no 64-bit vector arithmetic in the loop */
+   static __device__ __forceinline__ uint32_t thread_offset(int64_t ld)
+   {  uint32_t mn, k; where(0, mn, k);
+      return (uint32_t)((KC ? ((int64_t)k + (int64_t)mn * ld) : ((int64_t)mn + (int64_t)k * ld)) * 2);
+   }
+   static __device__ __forceinline__ const char *slab_base(const char *mat, int64_t ld, uint32_t mn0, uint32_t k0)
+   {  return mat + (KC ? ((int64_t)k0 + (int64_t)mn0 * ld) : ((int64_t)mn0 + (int64_t)k0 * ld)) * 2; }
+   __device__ __forceinline__ void fetch_one(int v, const char *base, int64_t ld, uint32_t toff)
+   {  /* where(v) - where(0): KC rows THREADS / (KT / 8) * v further on, !KC k further on by v */
+      const int64_t step = KC ? (int64_t)(THREADS / (KT / 8)) * v * ld * 2 : (int64_t)v * ld * 2;
+      reg[v] = *reinterpret_cast<const och_gu32x4 *>(base + step + toff);
+   }
+   static constexpr int PIECES = KC ? NV : 8;                           /* stores that move the registers to LDS */
+   __device__ __forceinline__ void stash_one(uint16_t *buffer, int piece) const
+   {  static_assert(KC || NV == 8 || NV == 4, "a transposed piece is a store of 16 or 8 bytes");
+      if (KC)
+      {  uint32_t mn, k; where(piece, mn, k);
+         *reinterpret_cast<och_gu32x4 *>(buffer + (k / 8) * PLANE + mn * 8) = reg[piece];
+      }
+      else
+      {  constexpr int WD = NV / 2;
+         uint32_t mn, k; where(0, mn, k);
+         uint16_t *at = buffer + (k / 8) * PLANE + (mn / 8) * 8 + k % 8 + piece * BMN;
+         uint32_t out[WD];
+#pragma unroll
+         for (int w = 0; w < WD; w++)
+         {  /* the low (even piece) or high (odd piece) halves of two words, side by side: one byte permutation */
+            const uint32_t x = reg[2 * w][piece >> 1], y = reg[2 * w + 1][piece >> 1];
+            out[w] = __builtin_amdgcn_perm(y, x, (piece & 1) ? 0x07060302u : 0x05040100u);
+         }
+         if (WD == 2) { uint2 t; t.x = out[0]; t.y = out[1]; *reinterpret_cast<uint2 *>(at) = t; }
+         else { och_gu32x4 t; t.x = out[0]; t.y = out[1]; t.z = out[WD > 2 ? 2 : 0]; t.w = out[WD > 3 ? 3 : 0]; *reinterpret_cast<och_gu32x4 *>(at) = t; }
+      }
+   }
    /* the eight k of slot `slot` that lane group `kg` (0 or 1) feeds to MFMA step `ks` (16 k per step) */
    static __device__ __forceinline__ och_h8 fragment(const uint16_t *buffer, int slot, int ks, int kg)
    {  och_h8 f;
@@ -128,7 +166,14 @@ struct HalfSlab
    }
 };
 
-template <bool AKC, bool BKC, bool EDGE, int WM, int WN, int NWM, int NWN, int KT>
+/* PIPE: the main loop of the large tile with one wave per SIMD (four waves of 128 x 128): nothing hides a wave's memory
+   and LDS latencies but the wave itself, so the loop is software-pipelined by hand. The fragments of MFMA step ks + 1 are
+   read from LDS while the MFMAs of step ks run (two sets of fragment registers), the registers that hold slab s + 1 go
+   to the other LDS buffer during steps 0 and 1 and the loads of slab s + 2 leave during step 2, and the one barrier of a
+   slab stands in front of the last step's MFMAs, with the first fragment reads of the next slab right behind it. The
+   loop body has no branches (slab numbers past the end are clamped to the last slab: its data is loaded and stored once
+   more and never read), so the whole slab is one scheduling region. Only for tiles that lie inside the matrices. */
+template <bool AKC, bool BKC, bool EDGE, int WM, int WN, int NWM, int NWN, int KT, bool PIPE = false>
 __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGemmParams p)
 {
    constexpr int T = 32, THREADS = 64 * NWM * NWN;
@@ -161,6 +206,83 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
    {  slab0 = blockIdx.z * p.split_slabs;
       nslabs = (slab0 + p.split_slabs < nslabs) ? p.split_slabs : (slab0 < nslabs ? nslabs - slab0 : 0);
    }
+   if constexpr (PIPE)
+   {  static_assert(!EDGE && KT == 64, "the pipelined loop is for whole tiles and slabs of 64");
+      och_h8 fa[2][TMS], fb[2][TNS];
+      const int arow = wm + lane % T, brow = wn + lane % T, kg = lane / T;
+      const uint32_t toffA = LA::thread_offset(p.ldA), toffB = LB::thread_offset(p.ldB);
+#define OCH_FRAGS(SET, AS, BS, KS)                                                                        \
+      do { _Pragma("unroll") for (int i = 0; i < TMS; i++) fa[SET][i] = LA::fragment(AS, arow + i * T, KS, kg);      \
+           _Pragma("unroll") for (int j = 0; j < TNS; j++) fb[SET][j] = LB::fragment(BS, brow + j * T, KS, kg); } while (0)
+#define OCH_MFMAS(SET)                                                                                    \
+      do { _Pragma("unroll") for (int i = 0; i < TMS; i++)                                                \
+           _Pragma("unroll") for (int j = 0; j < TNS; j++)                                                \
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[SET][i], fb[SET][j], acc[i][j], 0, 0, 0); } while (0)
+      /* a step = CH chunks of two MFMAs; chunk q also reads its share of the TMS + TNS fragments of the next step and runs
+         FIRST and SECOND (a share of the step's stores to LDS and loads from memory); a scheduling fence closes the chunk */
+      constexpr int CH = TMS * TNS / 2, NF = TMS + TNS;
+      static_assert(TNS % 2 == 0, "a chunk is two MFMAs of one row of tiles");
+#define OCH_SHARE(q, N, I) for (int I = (q) * (N) / CH; I < ((q) + 1) * (N) / CH; I++)
+#define OCH_STEP(CUR, NXT, AS, BS, KS, FIRST, SECOND)                                                                  \
+      do { _Pragma("unroll") for (int q = 0; q < CH; q++)                                                             \
+           {  _Pragma("unroll") OCH_SHARE(q, NF, f)                                                                    \
+              {  if (f < TMS) fa[NXT][f < TMS ? f : 0] = LA::fragment(AS, arow + f * T, KS, kg);                       \
+                 else fb[NXT][f >= TMS ? f - TMS : 0] = LB::fragment(BS, brow + (f - TMS) * T, KS, kg);                \
+              }                                                                                                        \
+              FIRST; SECOND;                                                                                           \
+              acc[(2 * q) / TNS][(2 * q) % TNS] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[CUR][(2 * q) / TNS], fb[CUR][(2 * q) % TNS], acc[(2 * q) / TNS][(2 * q) % TNS], 0, 0, 0); \
+              acc[(2 * q) / TNS][(2 * q) % TNS + 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[CUR][(2 * q) / TNS], fb[CUR][(2 * q) % TNS + 1], acc[(2 * q) / TNS][(2 * q) % TNS + 1], 0, 0, 0); \
+              __builtin_amdgcn_sched_barrier(0);                                                                       \
+           } } while (0)
+      if (nslabs > 0)
+      {  const uint32_t last = slab0 + nslabs - 1;
+         la.fetch(pA, p.ldA, m0, slab0 * KT, p.M, p.K, p.alignedA);
+         lb.fetch(pB, p.ldB, n0, slab0 * KT, p.N, p.K, p.alignedB);
+         la.stash(lds); lb.stash(lds + LA::SIZE);
+         {  /* the loads of the second slab leave in the order in which the loop issues them (A then B, pair by pair): the
+               compiler's count of loads that may still be in flight at a store of the loop is the worse of the two ways
+               into the loop, and with the loads here in any order every store of the loop waited for nearly all of them */
+            const uint32_t s1 = (slab0 + 1 < last) ? slab0 + 1 : last;
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int v = 0; v < LA::NV; v++)
+            {  la.fetch_one(v, LA::slab_base(pA, p.ldA, m0, s1 * KT), p.ldA, toffA);
+               __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int v = 0; v < LB::NV; v++)
+            {  lb.fetch_one(v, LB::slab_base(pB, p.ldB, n0, s1 * KT), p.ldB, toffB);
+               __builtin_amdgcn_sched_barrier(0);
+            }
+         }
+         __syncthreads();
+         OCH_FRAGS(0, lds, lds + LA::SIZE, 0);
+         for (uint32_t s = 0; s < nslabs; s++)
+         {  const uint16_t *As = lds + (s & 1) * BUF, *Bs = As + LA::SIZE;
+            uint16_t *An = lds + ((s + 1) & 1) * BUF, *Bn = An + LA::SIZE;
+            const uint32_t s2 = (slab0 + s + 2 < last) ? slab0 + s + 2 : last;
+            const char *nextA = LA::slab_base(pA, p.ldA, m0, s2 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, s2 * KT);
+            /* Every step is eight chunks of two MFMAs; a chunk also issues one fragment read for the next step and two of the
+               step's other memory instructions, and a scheduling fence closes it, so the instructions leave in this order.
+               Step 0: slab s + 1 of A goes from its registers to LDS (chunks 0-3) and slab s + 2 of A is asked for (chunks
+               4-7), a slab ahead of its own store; step 1: the same for B; step 2: fragment reads only; then the barrier;
+               step 3 reads the first fragments of the next slab. */
+            OCH_STEP(0, 1, As, Bs, 1, _Pragma("unroll") OCH_SHARE(q, LA::PIECES, e) la.stash_one(An, e), (void)0);
+            OCH_STEP(1, 0, As, Bs, 2, _Pragma("unroll") OCH_SHARE(q, LB::PIECES, e) lb.stash_one(Bn, e),
+                                      _Pragma("unroll") OCH_SHARE(q, LA::NV, v) la.fetch_one(v, nextA, p.ldA, toffA));
+            OCH_STEP(0, 1, As, Bs, 3, _Pragma("unroll") OCH_SHARE(q, LB::NV, v) lb.fetch_one(v, nextB, p.ldB, toffB), (void)0);
+            __syncthreads();
+            OCH_STEP(1, 0, An, Bn, 0, (void)0, (void)0);
+         }
+         __syncthreads();
+      }
+#undef OCH_FRAGS
+#undef OCH_MFMAS
+#undef OCH_STEP
+#undef OCH_SHARE
+   }
+   else
+   {
    /* registers hold the slab after the one in LDS: slab s + 1 is stored half way through the MFMAs of slab s (its stores
       run under the remaining MFMAs instead of in front of the barrier) and the loads of slab s + 2 are issued right after,
       a slab and a half before their data is needed */
@@ -199,6 +321,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
       __syncthreads();
    }
 
+   }
    const uint32_t row0 = LA::row_of_slot(wm + 4 * (lane >> 5)), col0 = LB::row_of_slot(wn + lane % T);
    if (p.split_slabs)
    {  /* raw sums of this K slice */
@@ -303,7 +426,7 @@ __global__ __launch_bounds__(256) void gemm_half_finish_kernel(const HalfGemmPar
    *c = float_to_half(v);
 }
 
-template <int WM, int WN, int NWM, int NWN, int KT>
+template <int WM, int WN, int NWM, int NWN, int KT, bool PIPE = false>
 static int launch_gemm_half(const GemmArgs &g)
 {
    constexpr int BM = NWM * WM, BN = NWN * WN, THREADS = 64 * NWM * NWN;
@@ -349,7 +472,7 @@ static int launch_gemm_half(const GemmArgs &g)
    const dim3 grid((unsigned)blocks, 1, slices > 1 ? slices : g.nz), block(THREADS);
    /* both LDS buffers; above 64 KB the kernel has to be told */
 #define OCH_HGEMM_LAUNCH(AK, BK, EDGE)                                                                                   \
-   do { auto kernel = gemm_half_kernel<AK, BK, EDGE, WM, WN, NWM, NWN, KT>;                                              \
+   do { auto kernel = gemm_half_kernel<AK, BK, EDGE, WM, WN, NWM, NWN, KT, PIPE && !(EDGE)>;                             \
         const size_t lds = 2 * 2 * (size_t)(HalfSlab<AK, EDGE, BM, KT, THREADS>::SIZE + HalfSlab<BK, EDGE, BN, KT, THREADS>::SIZE); \
         if (lds > 65536) OCH_CHECK_HIP(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
         hipLaunchKernelGGL(kernel, grid, block, lds, g.stream, p); } while (0)
@@ -380,7 +503,10 @@ int gemm_half(const GemmArgs &g)
    if (g.K < 16) return 1;                      /* C <- beta C, and updates of so low a rank that writing C is all there is */
    static const GemmTileChoice choice[3] = { { 256, 256, 1.0 }, { 128, 128, 0.8 }, { 64, 64, 0.55 } };
    switch (gemm_pick_tile(g, choice, 3))
-   {  case 0:  return launch_gemm_half<64, 128, 4, 2, 64>(g);
+   {  case 0:
+         /* whole aligned tiles: four waves of 128 x 128 with the hand-pipelined loop; otherwise eight waves of 64 x 128 */
+         if (g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0) return launch_gemm_half<128, 128, 2, 2, 64, true>(g);
+         return launch_gemm_half<64, 128, 4, 2, 64>(g);
       case 1:  return launch_gemm_half<64, 64, 2, 2, 64>(g);
       default: return launch_gemm_half<32, 32, 2, 2, 64>(g);
    }

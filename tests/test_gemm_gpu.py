@@ -140,6 +140,10 @@ def test_gemm_half_matrix_cores(hip, stream, ta, tb):
                                               (64, 64, 32, 0, -1, 0.5, False), (96, 160, 2048, 0, 0.5, 0, True), (33, 47, 17, 5, 1, 0, False),
                                               (2560, 2304, 48, 0, 1, 1, False), (2500, 2300, 40, 4, 1, 0, False), (4096, 3072, 64, 0, 1, 0, False),
                                               (4000, 3100, 70, 0, -1, 1, True),
+                                              # whole aligned tiles of 256 x 256 with K a multiple of 64: the hand-pipelined loop, and for
+                                              # 'T' x 'N' the kernel that loads straight into LDS (one to five slabs of 64: start-up, clamped
+                                              # loads past the end, every LDS stage reused)
+                                              (4096, 3072, 128, 0, 2, -1, True), (3072, 4096, 192, 0, 1, 0, False), (4096, 3072, 320, 0, -1, 1, False),
                                               # results narrower than a tile, vectors, K below one MFMA step, K not a multiple of 8
                                               (2000, 1, 1000, 0, 1, 0, False), (1, 1500, 999, 0, 1, 1, False), (700, 9, 3, 1, 2, 0, False), (31, 31, 15, 0, 1, 0, False),
                                               # few tiles and a long K: cut along K, float partial sums added in order
