@@ -51,7 +51,7 @@ struct ByteSlab
    static constexpr int PLANE = BMN * 16 + 32;                         /* bytes per chunk plane */
    static constexpr int SIZE = (KT / 16) * PLANE;                      /* bytes per LDS buffer */
    static_assert(NV >= 1 && (BMN * KT) % (16 * THREADS) == 0, "slab does not divide among the threads");
-   static_assert(KC || NV == 2 || NV == 4, "the transposing loader needs 2 or 4 k per thread");
+   static_assert(KC || NV == 2 || NV == 4 || NV == 8, "the transposing loader needs 2, 4 or 8 k per thread");
    och_gu32x4 reg[NV];
 
    static __device__ __forceinline__ uint32_t row_of_slot(uint32_t slot) { return KC ? slot : (slot % G) * 16 + slot / G; }
@@ -108,9 +108,47 @@ struct ByteSlab
             if (NV == 2) *reinterpret_cast<uint16_t *>(dst + i * (G * 16)) = (uint16_t)lo;
             else
             {  const uint32_t hi = __builtin_amdgcn_perm(reg[NV > 2 ? 3 : 1][i >> 2], reg[NV > 2 ? 2 : 0][i >> 2], sel);
-               *reinterpret_cast<uint32_t *>(dst + i * (G * 16)) = (lo & 0xFFFFu) | (hi << 16);
+               const uint32_t w0 = (lo & 0xFFFFu) | (hi << 16);
+               if (NV == 4) *reinterpret_cast<uint32_t *>(dst + i * (G * 16)) = w0;
+               else
+               {  const uint32_t lo2 = __builtin_amdgcn_perm(reg[NV > 4 ? 5 : 1][i >> 2], reg[NV > 4 ? 4 : 0][i >> 2], sel);
+                  const uint32_t hi2 = __builtin_amdgcn_perm(reg[NV > 4 ? 7 : 1][i >> 2], reg[NV > 4 ? 6 : 0][i >> 2], sel);
+                  uint2 t; t.x = w0; t.y = (lo2 & 0xFFFFu) | (hi2 << 16);
+                  *reinterpret_cast<uint2 *>(dst + i * (G * 16)) = t;
+               }
             }
          }
+      }
+   }
+   /* The same in single instructions, for the loop that places every one of them by hand (whole tiles, no bool): load
+      number v as a scalar base (the slab's first element, the same for all threads) + a step per v + the thread's own
+      offset, which does not change from slab to slab; and store number `piece` of the PIECES that move the registers to LDS */
+   static constexpr int PIECES = KC ? NV : 16;
+   static __device__ __forceinline__ uint32_t thread_offset(int64_t ld)
+   {  uint32_t mn, k; where(0, mn, k);
+      return (uint32_t)(KC ? ((int64_t)k + (int64_t)mn * ld) : ((int64_t)mn + (int64_t)k * ld));
+   }
+   static __device__ __forceinline__ const char *slab_base(const char *mat, int64_t ld, uint32_t mn0, uint32_t k0)
+   {  return mat + (KC ? ((int64_t)k0 + (int64_t)mn0 * ld) : ((int64_t)mn0 + (int64_t)k0 * ld)); }
+   __device__ __forceinline__ void fetch_one(int v, const char *base, int64_t ld, uint32_t toff)
+   {  const int64_t step = KC ? (int64_t)(THREADS / (KT / 16)) * v * ld : (int64_t)v * ld;
+      reg[v] = *reinterpret_cast<const och_gu32x4 *>(base + step + toff);
+   }
+   __device__ __forceinline__ void stash_one(char *buffer, int piece) const
+   {  static_assert(KC || NV == 8, "a transposed piece is a store of 8 bytes");
+      if (KC)
+      {  uint32_t mn, k; where(piece, mn, k);
+         *reinterpret_cast<och_gu32x4 *>(buffer + (k / 16) * PLANE + mn * 16) = reg[piece];
+      }
+      else
+      {  uint32_t mn, k; where(0, mn, k);
+         char *at = buffer + (k / 16) * PLANE + (mn / 16) * 16 + k % 16 + piece * (G * 16);
+         const uint32_t sel = 0x0C0C0400u + (uint32_t)(piece & 3) * 0x0101u;
+         uint32_t pair[4];
+#pragma unroll
+         for (int w = 0; w < 4; w++) pair[w] = __builtin_amdgcn_perm(reg[NV > 2 * w + 1 ? 2 * w + 1 : 1][piece >> 2], reg[NV > 2 * w ? 2 * w : 0][piece >> 2], sel);
+         uint2 t; t.x = (pair[0] & 0xFFFFu) | (pair[1] << 16); t.y = (pair[2] & 0xFFFFu) | (pair[3] << 16);
+         *reinterpret_cast<uint2 *>(at) = t;
       }
    }
    /* the sixteen k of slot `slot` that lane group `kg` (0 or 1) feeds to MFMA step `ks` (32 k per step) */
@@ -128,7 +166,11 @@ template <bool BOOL> __device__ __forceinline__ uint8_t byte_finish(int s, uint8
    return (uint8_t)((uint32_t)alpha * (uint32_t)s + (use_c ? (uint32_t)beta * (uint32_t)c : 0u));
 }
 
-template <bool AKC, bool BKC, bool EDGE, bool BOOL, int WM, int WN, int NWM, int NWN, int KT>
+/* PIPE: the hand-scheduled main loop of the half-precision kernel (gemm_half_kernel), for whole 256 x 256 tiles of int8 /
+   uint8 with four waves of 128 x 128: fragments one MFMA step ahead in a second set of registers, the stores of slab s + 1
+   to LDS and the loads of slab s + 2 spread one per chunk of two MFMAs over steps 0 to 2, one barrier per slab in front of
+   the last step, no branches in the loop body (slab numbers past the end are clamped). */
+template <bool AKC, bool BKC, bool EDGE, bool BOOL, int WM, int WN, int NWM, int NWN, int KT, bool PIPE = false>
 __global__ __launch_bounds__(64 * NWM * NWN) void gemm_byte_kernel(const ByteGemmParams p)
 {
    constexpr int T = 32, THREADS = 64 * NWM * NWN;
@@ -161,6 +203,68 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_byte_kernel(const ByteGem
    {  slab0 = blockIdx.z * p.split_slabs;
       nslabs = (slab0 + p.split_slabs < nslabs) ? p.split_slabs : (slab0 < nslabs ? nslabs - slab0 : 0);
    }
+   if constexpr (PIPE)
+   {  static_assert(!EDGE && !BOOL && KT == 128, "the pipelined loop is for whole tiles of 8-bit integers and slabs of 128");
+      och_i32x4 fa[2][TMS], fb[2][TNS];
+      const int arow = wm + lane % T, brow = wn + lane % T, kg = lane / T;
+      const uint32_t toffA = LA::thread_offset(p.ldA), toffB = LB::thread_offset(p.ldB);
+      constexpr int CH = TMS * TNS / 2, NF = TMS + TNS;
+      static_assert(TNS % 2 == 0, "a chunk is two MFMAs of one row of tiles");
+#define OCH_SHARE(q, N, I) for (int I = (q) * (N) / CH; I < ((q) + 1) * (N) / CH; I++)
+#define OCH_STEP(CUR, NXT, AS, BS, KS, FIRST, SECOND)                                                                  \
+      do { _Pragma("unroll") for (int q = 0; q < CH; q++)                                                             \
+           {  _Pragma("unroll") OCH_SHARE(q, NF, f)                                                                    \
+              {  if (f < TMS) fa[NXT][f < TMS ? f : 0] = LA::fragment(AS, arow + f * T, KS, kg);                       \
+                 else fb[NXT][f >= TMS ? f - TMS : 0] = LB::fragment(BS, brow + (f - TMS) * T, KS, kg);                \
+              }                                                                                                        \
+              FIRST; SECOND;                                                                                           \
+              acc[(2 * q) / TNS][(2 * q) % TNS] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[CUR][(2 * q) / TNS], fb[CUR][(2 * q) % TNS], acc[(2 * q) / TNS][(2 * q) % TNS], 0, 0, 0); \
+              acc[(2 * q) / TNS][(2 * q) % TNS + 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[CUR][(2 * q) / TNS], fb[CUR][(2 * q) % TNS + 1], acc[(2 * q) / TNS][(2 * q) % TNS + 1], 0, 0, 0); \
+              __builtin_amdgcn_sched_barrier(0);                                                                       \
+           } } while (0)
+      if (nslabs > 0)
+      {  const uint32_t last = slab0 + nslabs - 1;
+         la.fetch(pA, p.ldA, m0, slab0 * KT, p.M, p.K, p.alignedA);
+         lb.fetch(pB, p.ldB, n0, slab0 * KT, p.N, p.K, p.alignedB);
+         la.stash(lds); lb.stash(lds + LA::SIZE);
+         {  /* in the order of the loop, so that the compiler's count of loads in flight at the loop's stores is exact */
+            const uint32_t s1 = (slab0 + 1 < last) ? slab0 + 1 : last;
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int v = 0; v < LA::NV; v++)
+            {  la.fetch_one(v, LA::slab_base(pA, p.ldA, m0, s1 * KT), p.ldA, toffA);
+               __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int v = 0; v < LB::NV; v++)
+            {  lb.fetch_one(v, LB::slab_base(pB, p.ldB, n0, s1 * KT), p.ldB, toffB);
+               __builtin_amdgcn_sched_barrier(0);
+            }
+         }
+         __syncthreads();
+#pragma unroll
+         for (int i = 0; i < TMS; i++) fa[0][i] = LA::fragment(lds, arow + i * T, 0, kg);
+#pragma unroll
+         for (int j = 0; j < TNS; j++) fb[0][j] = LB::fragment(lds + LA::SIZE, brow + j * T, 0, kg);
+         for (uint32_t s = 0; s < nslabs; s++)
+         {  const char *As = lds + (s & 1) * BUF, *Bs = As + LA::SIZE;
+            char *An = lds + ((s + 1) & 1) * BUF, *Bn = An + LA::SIZE;
+            const uint32_t s2 = (slab0 + s + 2 < last) ? slab0 + s + 2 : last;
+            const char *nextA = LA::slab_base(pA, p.ldA, m0, s2 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, s2 * KT);
+            OCH_STEP(0, 1, As, Bs, 1, _Pragma("unroll") OCH_SHARE(q, LA::PIECES, e) la.stash_one(An, e), (void)0);
+            OCH_STEP(1, 0, As, Bs, 2, _Pragma("unroll") OCH_SHARE(q, LB::PIECES, e) lb.stash_one(Bn, e),
+                                      _Pragma("unroll") OCH_SHARE(q, LA::NV, v) la.fetch_one(v, nextA, p.ldA, toffA));
+            OCH_STEP(0, 1, As, Bs, 3, _Pragma("unroll") OCH_SHARE(q, LB::NV, v) lb.fetch_one(v, nextB, p.ldB, toffB), (void)0);
+            __syncthreads();
+            OCH_STEP(1, 0, An, Bn, 0, (void)0, (void)0);
+         }
+         __syncthreads();
+      }
+#undef OCH_STEP
+#undef OCH_SHARE
+   }
+   else
+   {
    if (nslabs > 0)
    {  la.fetch(pA, p.ldA, m0, slab0 * KT, p.M, p.K, p.alignedA);
       lb.fetch(pB, p.ldB, n0, slab0 * KT, p.N, p.K, p.alignedB);
@@ -196,6 +300,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_byte_kernel(const ByteGem
       __syncthreads();
    }
 
+   }
    /* accumulator register r of lane l belongs to slot 8 * (r / 4) + 4 * (l / 32) + r % 4 of A and slot l % 32 of B within
       its 32 x 32 tile; the slot offsets added below never carry out of a group of BM / 16 (BN / 16) slots */
    const uint32_t row0 = LA::row_of_slot(wm + 4 * (lane >> 5)), col0 = LB::row_of_slot(wn + lane % T);
@@ -281,7 +386,7 @@ __global__ __launch_bounds__(256) void gemm_byte_finish_kernel(const ByteGemmPar
    *c = byte_finish<BOOL>(s, alpha, beta, beta ? *c : (uint8_t)0, beta != 0);
 }
 
-template <bool BOOL, int WM, int WN, int NWM, int NWN, int KT>
+template <bool BOOL, int WM, int WN, int NWM, int NWN, int KT, bool PIPE = false>
 static int launch_gemm_byte(const GemmArgs &g)
 {
    constexpr int BM = NWM * WM, BN = NWN * WN, THREADS = 64 * NWM * NWN;
@@ -326,7 +431,7 @@ static int launch_gemm_byte(const GemmArgs &g)
    }
    const dim3 grid((unsigned)blocks, 1, slices > 1 ? slices : g.nz), block(THREADS);
 #define OCH_BGEMM_LAUNCH(AK, BK, EDGE)                                                                                    \
-   do { auto kernel = gemm_byte_kernel<AK, BK, EDGE, BOOL, WM, WN, NWM, NWN, KT>;                                         \
+   do { auto kernel = gemm_byte_kernel<AK, BK, EDGE, BOOL, WM, WN, NWM, NWN, KT, PIPE && !(EDGE) && !BOOL>;               \
         const size_t lds = 2 * (size_t)(ByteSlab<AK, EDGE, BOOL, BM, KT, THREADS>::SIZE + ByteSlab<BK, EDGE, BOOL, BN, KT, THREADS>::SIZE); \
         if (lds > 65536) OCH_CHECK_HIP(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
         hipLaunchKernelGGL(kernel, grid, block, lds, g.stream, p); } while (0)
@@ -349,7 +454,10 @@ template <bool BOOL> static int gemm_byte_pick(const GemmArgs &g)
    if (g.K < 32) return 1;
    static const GemmTileChoice choice[3] = { { 256, 256, 1.0 }, { 128, 128, 0.8 }, { 64, 64, 0.55 } };
    switch (gemm_pick_tile(g, choice, 3))
-   {  case 0:  return launch_gemm_byte<BOOL, 64, 128, 4, 2, 128>(g);
+   {  case 0:
+         /* whole tiles of 8-bit integers: four waves of 128 x 128 with the hand-pipelined loop; otherwise eight waves of 64 x 128 */
+         if (!BOOL && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 128 == 0) return launch_gemm_byte<BOOL, 128, 128, 2, 2, 128, true>(g);
+         return launch_gemm_byte<BOOL, 64, 128, 4, 2, 128>(g);
       case 1:  return launch_gemm_byte<BOOL, 64, 64, 2, 2, 128>(g);
       default: return launch_gemm_byte<BOOL, 32, 32, 2, 2, 128>(g);
    }

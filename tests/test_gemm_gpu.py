@@ -140,10 +140,6 @@ def test_gemm_half_matrix_cores(hip, stream, ta, tb):
                                               (64, 64, 32, 0, -1, 0.5, False), (96, 160, 2048, 0, 0.5, 0, True), (33, 47, 17, 5, 1, 0, False),
                                               (2560, 2304, 48, 0, 1, 1, False), (2500, 2300, 40, 4, 1, 0, False), (4096, 3072, 64, 0, 1, 0, False),
                                               (4000, 3100, 70, 0, -1, 1, True),
-                                              # whole aligned tiles of 256 x 256 with K a multiple of 64: the hand-pipelined loop, and for
-                                              # 'T' x 'N' the kernel that loads straight into LDS (one to five slabs of 64: start-up, clamped
-                                              # loads past the end, every LDS stage reused)
-                                              (4096, 3072, 128, 0, 2, -1, True), (3072, 4096, 192, 0, 1, 0, False), (4096, 3072, 320, 0, -1, 1, False),
                                               # results narrower than a tile, vectors, K below one MFMA step, K not a multiple of 8
                                               (2000, 1, 1000, 0, 1, 0, False), (1, 1500, 999, 0, 1, 1, False), (700, 9, 3, 1, 2, 0, False), (31, 31, 15, 0, 1, 0, False),
                                               # few tiles and a long K: cut along K, float partial sums added in order
@@ -166,6 +162,62 @@ def test_gemm_bytes_matrix_cores(hip, stream, dtype, ta, tb):
         if dtype == H.BOOL:
             alpha, beta = (1 if alpha else 0), (1 if beta else 0)
         run_case(stream, dtype, ta, tb, M, N, K, alpha, beta, rng, device_scalars=dev, pad=pad, kind="full")
+
+
+@pytest.mark.parametrize("dtype", [H.HALF, H.INT8, H.UINT8], ids=lambda d: H.NAMES[d])
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+def test_gemm_pipelined_whole_tiles(hip, stream, dtype, ta, tb):
+    """Products that the tile choice gives to the 256 x 256 tile (256 tiles or more) and that consist of whole aligned
+    tiles run on the hand-pipelined loop: one slab (start-up only), three and five slabs (clamped loads past the end, both
+    LDS buffers reused), with and without beta, scalars in host and in device memory. Checked without O(n^3) host work:
+    eight complete rows and columns of C computed directly, and C times probe vectors against op(A) (op(B) x) -- in exact
+    arithmetic modulo 256 for the 8-bit types, to the half-precision bound for half."""
+    rng = np.random.default_rng(1200 + dtype + ord(ta) + 2 * ord(tb))
+    n = 4096
+    kt = 64 if dtype == H.HALF else 128
+    exact = dtype != H.HALF
+    for slabs, alpha, beta, dev in ((1, 1, 0, False), (3, 2, -1 if dtype != H.UINT8 else 3, True), (5, -1 if dtype != H.UINT8 else 5, 1, False)):
+        K = slabs * kt
+        rowsA, colsA = (n, K) if ta == "N" else (K, n)
+        rowsB, colsB = (K, n) if tb == "N" else (n, K)
+        A, B, C0 = matrix(dtype, rowsA, colsA, rowsA, rng, "full" if exact else "small"), matrix(dtype, rowsB, colsB, rowsB, rng, "full" if exact else "small"), \
+            matrix(dtype, n, n, n, rng, "full" if exact else "small")
+        al, be = scalar_of(dtype, alpha), scalar_of(dtype, beta)
+        dA, dB, dC = oh.to_device(A, stream), oh.to_device(B, stream), oh.to_device(C0, stream)
+        if dev:
+            dal, dbe = oh.to_device(al, stream), oh.to_device(be, stream)
+            pal, pbe, mode = dal.ptr, dbe.ptr, 0
+        else:
+            pal, pbe, mode = orc.ptr(al), orc.ptr(be), 1
+        oh.check(oh.lib.och_gemm(dtype, ta.encode(), tb.encode(), n, n, K, pal, dA.ptr, rowsA, dB.ptr, rowsB, pbe, dC.ptr, n, mode, stream.handle))
+        got = dC.download(C0.dtype, C0.size)
+        for b in (dA, dB, dC):
+            b.free()
+        wide = np.int64 if exact else np.float64
+        num = (lambda a: a.astype(np.int64)) if exact else (lambda a: as_float(dtype, a).astype(np.float64))
+        mA, mB = num(A).reshape(colsA, rowsA).T, num(B).reshape(colsB, rowsB).T            # [row, col]
+        opA, opB = (mA if ta == "N" else mA.T), (mB if tb == "N" else mB.T)
+        c0, c = num(C0).reshape(n, n).T, num(got).reshape(n, n).T
+        what = "%s %s%s K=%d alpha=%r beta=%r" % (H.NAMES[dtype], ta, tb, K, alpha, beta)
+
+        def same(have, want, bound):
+            if exact:
+                assert np.array_equal(have % 256, want % 256), what
+            else:
+                assert (np.abs(have - want) <= TOL[dtype] * bound + 1e-30).all(), "%s: %.3e" % (what, np.abs(have - want).max())
+        for i in rng.integers(0, n, 8):
+            row = alpha * (opA[i, :] @ opB) + beta * c0[i, :]
+            same(c[i, :], row, abs(alpha) * (np.abs(opA[i, :]) @ np.abs(opB)) + abs(beta) * np.abs(c0[i, :]))
+            col = alpha * (opA @ opB[:, i]) + beta * c0[:, i]
+            same(c[:, i], col, abs(alpha) * (np.abs(opA) @ np.abs(opB[:, i])) + abs(beta) * np.abs(c0[:, i]))
+        X = rng.integers(-3, 4, (n, 6)).astype(wide)
+        want = alpha * (opA @ (opB @ X)) + beta * (c0 @ X)
+        have = c @ X
+        if exact:
+            assert np.array_equal(have % 256, want % 256), what + " (probe vectors)"
+        else:
+            bound = abs(alpha) * (np.abs(opA) @ (np.abs(opB) @ np.abs(X))) + abs(beta) * (np.abs(c0) @ np.abs(X))
+            assert np.linalg.norm(have - want) <= TOL[dtype] * np.linalg.norm(bound), what + " (probe vectors)"
 
 
 def test_gemm_errors_and_empty(hip, stream):
