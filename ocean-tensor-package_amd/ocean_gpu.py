@@ -242,6 +242,8 @@ class tensor(object):
             return tensor._converted(other, dtype, self._h.contents.device)
         if dtype is not None:
             return asTensor(other, dtype)
+        if isinstance(other, _np.ndarray) and other.ndim > 0:
+            return asTensor(other)                            # a numpy array keeps its own type
         if _np.ndim(other) == 0:
             return asTensor(other, _scalar_dtype(other, self.dtype))
         if _list_dtype(other) == bool:
