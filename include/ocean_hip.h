@@ -349,6 +349,11 @@ typedef struct {
 } och_reduce_axis_config;
 
 int och_reduce_axis(int op, int dtype, const och_reduce_axis_config *config, double p);
+/* One launch counts its outputs in 32 bits; a reduction with more outputs (the reference switches to 64-bit indices,     */
+/* solid/src/core/gpu/op/apply_elemwise.c:68-99) is cut along its outermost kept dimension into pieces that are launched   */
+/* one after the other. More than 2^32 reduced elements per output return an error. Test hook: the number of outputs per  */
+/* launch can be lowered (0 restores the default) so that small tensors are cut.                                          */
+void och_reduce_axis_set_output_limit(size_t outputs);
 
 /* ======================================================================== */
 /* GEMM: C <- alpha * op(A) * op(B) + beta * C, column-major, ld in elements*/

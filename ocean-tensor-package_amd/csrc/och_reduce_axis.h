@@ -302,6 +302,8 @@ __global__ __launch_bounds__(256) void axis_group_kernel(const AxisParams p, con
 }
 
 typedef int (*axis_fn)(const och_reduce_axis_config *c, double pnorm);
+/* outputs one launch handles (0xFFFFFF00 unless och_reduce_axis_set_output_limit has lowered it for a test) */
+uint64_t axis_output_limit();
 
 template <class T, int OP>
 static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
@@ -317,7 +319,24 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
    for (int d = 0; d < c->rdims; d++) relem *= c->rsize[d];
    if (nout == 0) return 0;
    if (relem == 0 && RD::NEEDS_DATA) return set_error("reduction over an empty range is undefined for this operation");
-   if (nout > 0xFFFFFF00ull || relem > 0xFFFFFF00ull) return set_error("axis reduction with more than 2^32 outputs or reduced elements is not supported");
+   if (relem > 0xFFFFFF00ull) return set_error("axis reduction over more than 2^32 elements per output is not supported");
+   /* more outputs than one launch counts in 32 bits (the reference switches to 64-bit indices): the outputs are
+      independent, so the outermost kept dimension is cut into runs that fit, or walked index by index when a single
+      index of it is still too much, and every piece is a reduction of its own on the same stream */
+   if (nout > axis_output_limit())
+   {  int last = -1;
+      for (int d = 0; d < c->ndims; d++) if (c->size[d] > 1) last = d;
+      const uint64_t inner = nout / c->size[last];
+      const uint64_t run = (inner <= axis_output_limit()) ? axis_output_limit() / inner : 1;
+      for (uint64_t start = 0; start < c->size[last]; start += run)
+      {  och_reduce_axis_config piece = *c;
+         piece.size[last] = (c->size[last] - start < run) ? (size_t)(c->size[last] - start) : (size_t)run;
+         piece.ptr1 = (char *)c->ptr1 + (int64_t)start * c->strides1[last];
+         piece.ptr2 = (char *)c->ptr2 + (int64_t)start * c->strides2[last];
+         if (launch_reduce_axis<T, OP>(&piece, pnorm) != 0) return -1;
+      }
+      return 0;
+   }
 
    AxisParams p;
    memset(&p, 0, sizeof(p));

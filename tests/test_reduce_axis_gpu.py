@@ -248,3 +248,24 @@ def test_axis_rows_that_are_not_whole_vectors(hip, stream, dtype):
             truth, scale = v.sum(axis=ax).T, np.abs(v).sum(axis=ax).T
             tol = 4e-3 if dtype == H.HALF else 1e-5
             assert np.all(np.abs(g - truth) <= tol * np.maximum(np.asarray(scale), 1e-6)), what
+
+
+def test_axis_reductions_with_more_outputs_than_a_launch_counts(hip, stream):
+    """A reduction with more outputs than one launch counts is cut along its outermost kept dimension into reductions of
+    their own (runs of that dimension, or single indices when one index is still too much). The limit is lowered so
+    that small tensors are cut; integer results are bit for bit those of the uncut call and of the oracle."""
+    rng = np.random.default_rng(41)
+    parent = rng.integers(-99, 99, size=(11, 30, 26, 40), dtype=np.int32)
+    view = parent[::2, 1::3, :, ::-2].transpose(3, 1, 2, 0)          # shape (20, 10, 26, 6), mixed strides
+    try:
+        for axes in ([0], [1], [3], [1, 2], [0, 3]):
+            for name in ("sum", "maximum", "nnz"):
+                oh.lib.och_reduce_axis_set_output_limit(0)
+                rd, whole, want = run_case(stream, name, H.INT32, parent, view, axes)
+                H.assert_same_bytes(whole, want, "uncut %s axes=%s" % (name, axes))
+                for limit in (1000, 250, 37, 5, 1):
+                    oh.lib.och_reduce_axis_set_output_limit(limit)
+                    rd, got, _ = run_case(stream, name, H.INT32, parent, view, axes)
+                    H.assert_same_bytes(got, whole, "%s axes=%s with at most %d outputs per launch" % (name, axes, limit))
+    finally:
+        oh.lib.och_reduce_axis_set_output_limit(0)
