@@ -84,14 +84,18 @@ def gpu_part(name):
     return [it for it in RF.parse_ref(text[cut:] if cut >= 0 else text) if isinstance(it, RF.RefTensor)]
 
 
-def assert_printed(printed, expected):
+def assert_printed(printed, expected, decimals=None):
+    """decimals: the expected file prints floating values rounded to that many decimals"""
     assert len(printed) == len(expected)
     for k, (t, ref) in enumerate(zip(printed, expected)):
         assert t.dtype == ref.dtype and list(t.size) == list(ref.shape) and t.device.name == ref.device, (k, t.footer(), ref)
         assert t.footer() == "<tensor.%s of size %s on %s>" % (OCEAN_NAME[ref.dtype], "x".join(map(str, ref.shape)), ref.device)
         got = t.asnumpy()
         got = got.transpose(*range(got.ndim)[::-1])          # Ocean index order A[i0, i1, ...]
-        assert np.array_equal(got.astype(ref.values.dtype), ref.values), (k, got, ref.values)
+        if decimals is not None and got.dtype.kind == "f":
+            assert np.allclose(got.astype(np.float64), ref.values, rtol=0, atol=0.51 * 10.0 ** -decimals), (k, got, ref.values)
+        else:
+            assert np.array_equal(got.astype(ref.values.dtype), ref.values), (k, got, ref.values)
 
 
 @pytest.mark.gpu
@@ -124,6 +128,38 @@ def test_replay_tensor_multiply_01(hip):
         a *= 3
         out.append(a.clone())
     assert_printed(out, gpu_part("tensor_multiply_01"))
+
+
+@pytest.mark.gpu
+def test_replay_tensor_subtract_01(hip):
+    import ocean_gpu as ocean
+    device, out = ocean.gpu[0], []
+    a = ocean.asTensor([True, True, False], device)
+    out += [a.clone(), -a, a - True]
+    a -= True
+    out.append(a.clone())
+    for dtype, three in ((ocean.int8, 3), (ocean.float, 3.0)):
+        a = ocean.asTensor([-2, -1, 0, 1, 2], dtype, device)
+        out += [a.clone(), -a, a - three]
+        a -= 3
+        out.append(a.clone())
+    assert_printed(out, gpu_part("tensor_subtract_01"))
+
+
+@pytest.mark.gpu
+def test_replay_tensor_divide_01(hip):
+    import ocean_gpu as ocean
+    device, out = ocean.gpu[0], []
+    a = ocean.asTensor([True, True, False], device)
+    out += [a.clone(), a / True]
+    a /= [True, False, True]
+    out.append(a.clone())
+    for dtype, three in ((ocean.int8, 3), (ocean.float, 3.0)):
+        a = ocean.asTensor([-10, -5, 0, 4, 6], dtype, device)
+        out += [a.clone(), a / three]
+        a /= 3
+        out.append(a.clone())
+    assert_printed(out, gpu_part("tensor_divide_01"), decimals=5)
 
 
 @pytest.mark.gpu
