@@ -580,6 +580,14 @@ static inline int gemm_pick_tile(const GemmArgs &g, const GemmTileChoice *choice
    return best;
 }
 
+/* base pointers, leading dimensions and batch strides of all three operands allow 16-byte accesses (es: element size) */
+static inline bool gemm_operands_aligned(const GemmArgs &g, int es)
+{  bool ok = ((uintptr_t)g.A % 16 == 0) && ((uintptr_t)g.B % 16 == 0) && ((uintptr_t)g.C % 16 == 0)
+          && ((int64_t)g.ldA * es) % 16 == 0 && ((int64_t)g.ldB * es) % 16 == 0 && ((int64_t)g.ldC * es) % 16 == 0;
+   for (int d = 0; d < g.batch.nb; d++) ok = ok && g.batch.sA[d] % 16 == 0 && g.batch.sB[d] % 16 == 0 && g.batch.sC[d] % 16 == 0;
+   return ok;
+}
+
 int gemm_float(const GemmArgs &g);
 int gemm_double(const GemmArgs &g);
 int gemm_cfloat(const GemmArgs &g);

@@ -506,6 +506,26 @@ int gemm_half(const GemmArgs &g)
    {  case 0:
          /* whole aligned tiles: four waves of 128 x 128 with the hand-pipelined loop; otherwise eight waves of 64 x 128 */
          if (g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0) return launch_gemm_half<128, 128, 2, 2, 64, true>(g);
+         if (g.K % 64 == 0 && g.M >= 256 && g.N >= 256 && gemm_operands_aligned(g, 2))
+         {  /* whole tiles first, on the pipelined loop; then the strip of columns to their right and the strip of rows below them */
+            const size_t Mi = g.M - g.M % 256, Ni = g.N - g.N % 256;
+            GemmArgs part = g;
+            part.M = Mi; part.N = Ni;
+            if (launch_gemm_half<128, 128, 2, 2, 64, true>(part) != 0) return -1;
+            if (g.N > Ni)
+            {  part = g; part.N = g.N - Ni;
+               part.B = (const char *)g.B + (int64_t)Ni * (g.transB == 'N' ? (int64_t)g.ldB : 1) * 2;
+               part.C = (char *)g.C + (int64_t)Ni * g.ldC * 2;
+               if (gemm_half(part) != 0) return -1;          /* K >= 64: never left to the generic kernel */
+            }
+            if (g.M > Mi)
+            {  part = g; part.M = g.M - Mi; part.N = Ni;
+               part.A = (const char *)g.A + (int64_t)Mi * (g.transA == 'N' ? 1 : (int64_t)g.ldA) * 2;
+               part.C = (char *)g.C + (int64_t)Mi * 2;
+               if (gemm_half(part) != 0) return -1;
+            }
+            return 0;
+         }
          return launch_gemm_half<64, 128, 4, 2, 64>(g);
       case 1:  return launch_gemm_half<64, 64, 2, 2, 64>(g);
       default: return launch_gemm_half<32, 32, 2, 2, 64>(g);

@@ -457,6 +457,26 @@ template <bool BOOL> static int gemm_byte_pick(const GemmArgs &g)
    {  case 0:
          /* whole tiles of 8-bit integers: four waves of 128 x 128 with the hand-pipelined loop; otherwise eight waves of 64 x 128 */
          if (!BOOL && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 128 == 0) return launch_gemm_byte<BOOL, 128, 128, 2, 2, 128, true>(g);
+         if (!BOOL && g.K % 128 == 0 && g.M >= 256 && g.N >= 256 && gemm_operands_aligned(g, 1))
+         {  /* whole tiles first, on the pipelined loop; then the strip of columns to their right and the strip of rows below them */
+            const size_t Mi = g.M - g.M % 256, Ni = g.N - g.N % 256;
+            GemmArgs part = g;
+            part.M = Mi; part.N = Ni;
+            if (launch_gemm_byte<BOOL, 128, 128, 2, 2, 128, true>(part) != 0) return -1;
+            if (g.N > Ni)
+            {  part = g; part.N = g.N - Ni;
+               part.B = (const char *)g.B + (int64_t)Ni * (g.transB == 'N' ? (int64_t)g.ldB : 1);
+               part.C = (char *)g.C + (int64_t)Ni * g.ldC;
+               if (gemm_byte_pick<BOOL>(part) != 0) return -1;        /* K >= 128: never left to the generic kernel */
+            }
+            if (g.M > Mi)
+            {  part = g; part.M = g.M - Mi; part.N = Ni;
+               part.A = (const char *)g.A + (int64_t)Mi * (g.transA == 'N' ? 1 : (int64_t)g.ldA);
+               part.C = (char *)g.C + (int64_t)Mi;
+               if (gemm_byte_pick<BOOL>(part) != 0) return -1;
+            }
+            return 0;
+         }
          return launch_gemm_byte<BOOL, 64, 128, 4, 2, 128>(g);
       case 1:  return launch_gemm_byte<BOOL, 64, 64, 2, 2, 128>(g);
       default: return launch_gemm_byte<BOOL, 32, 32, 2, 2, 128>(g);

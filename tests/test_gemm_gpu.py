@@ -164,24 +164,18 @@ def test_gemm_bytes_matrix_cores(hip, stream, dtype, ta, tb):
         run_case(stream, dtype, ta, tb, M, N, K, alpha, beta, rng, device_scalars=dev, pad=pad, kind="full")
 
 
-@pytest.mark.parametrize("dtype", [H.HALF, H.INT8, H.UINT8], ids=lambda d: H.NAMES[d])
-@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
-def test_gemm_pipelined_whole_tiles(hip, stream, dtype, ta, tb):
-    """Products that the tile choice gives to the 256 x 256 tile (256 tiles or more) and that consist of whole aligned
-    tiles run on the hand-pipelined loop: one slab (start-up only), three and five slabs (clamped loads past the end, both
-    LDS buffers reused), with and without beta, scalars in host and in device memory. Checked without O(n^3) host work:
-    eight complete rows and columns of C computed directly, and C times probe vectors against op(A) (op(B) x) -- in exact
-    arithmetic modulo 256 for the 8-bit types, to the half-precision bound for half."""
-    rng = np.random.default_rng(1200 + dtype + ord(ta) + 2 * ord(tb))
-    n = 4096
+def check_large_product(stream, dtype, ta, tb, M, N, cases, rng):
+    """Large products checked without O(n^3) host work: eight complete rows and columns of C computed directly, and C
+    times probe vectors against op(A) (op(B) x) -- in exact arithmetic modulo 256 for the 8-bit types, to the
+    half-precision bound for half. cases: (slabs of K, alpha, beta, scalars in device memory)."""
     kt = 64 if dtype == H.HALF else 128
     exact = dtype != H.HALF
-    for slabs, alpha, beta, dev in ((1, 1, 0, False), (3, 2, -1 if dtype != H.UINT8 else 3, True), (5, -1 if dtype != H.UINT8 else 5, 1, False)):
+    for slabs, alpha, beta, dev in cases:
         K = slabs * kt
-        rowsA, colsA = (n, K) if ta == "N" else (K, n)
-        rowsB, colsB = (K, n) if tb == "N" else (n, K)
+        rowsA, colsA = (M, K) if ta == "N" else (K, M)
+        rowsB, colsB = (K, N) if tb == "N" else (N, K)
         A, B, C0 = matrix(dtype, rowsA, colsA, rowsA, rng, "full" if exact else "small"), matrix(dtype, rowsB, colsB, rowsB, rng, "full" if exact else "small"), \
-            matrix(dtype, n, n, n, rng, "full" if exact else "small")
+            matrix(dtype, M, N, M, rng, "full" if exact else "small")
         al, be = scalar_of(dtype, alpha), scalar_of(dtype, beta)
         dA, dB, dC = oh.to_device(A, stream), oh.to_device(B, stream), oh.to_device(C0, stream)
         if dev:
@@ -189,7 +183,7 @@ def test_gemm_pipelined_whole_tiles(hip, stream, dtype, ta, tb):
             pal, pbe, mode = dal.ptr, dbe.ptr, 0
         else:
             pal, pbe, mode = orc.ptr(al), orc.ptr(be), 1
-        oh.check(oh.lib.och_gemm(dtype, ta.encode(), tb.encode(), n, n, K, pal, dA.ptr, rowsA, dB.ptr, rowsB, pbe, dC.ptr, n, mode, stream.handle))
+        oh.check(oh.lib.och_gemm(dtype, ta.encode(), tb.encode(), M, N, K, pal, dA.ptr, rowsA, dB.ptr, rowsB, pbe, dC.ptr, M, mode, stream.handle))
         got = dC.download(C0.dtype, C0.size)
         for b in (dA, dB, dC):
             b.free()
@@ -197,20 +191,21 @@ def test_gemm_pipelined_whole_tiles(hip, stream, dtype, ta, tb):
         num = (lambda a: a.astype(np.int64)) if exact else (lambda a: as_float(dtype, a).astype(np.float64))
         mA, mB = num(A).reshape(colsA, rowsA).T, num(B).reshape(colsB, rowsB).T            # [row, col]
         opA, opB = (mA if ta == "N" else mA.T), (mB if tb == "N" else mB.T)
-        c0, c = num(C0).reshape(n, n).T, num(got).reshape(n, n).T
-        what = "%s %s%s K=%d alpha=%r beta=%r" % (H.NAMES[dtype], ta, tb, K, alpha, beta)
+        c0, c = num(C0).reshape(N, M).T, num(got).reshape(N, M).T
+        what = "%s %s%s %dx%dx%d alpha=%r beta=%r" % (H.NAMES[dtype], ta, tb, M, N, K, alpha, beta)
 
         def same(have, want, bound):
             if exact:
                 assert np.array_equal(have % 256, want % 256), what
             else:
                 assert (np.abs(have - want) <= TOL[dtype] * bound + 1e-30).all(), "%s: %.3e" % (what, np.abs(have - want).max())
-        for i in rng.integers(0, n, 8):
+        for i in list(rng.integers(0, M, 7)) + [M - 1]:
             row = alpha * (opA[i, :] @ opB) + beta * c0[i, :]
             same(c[i, :], row, abs(alpha) * (np.abs(opA[i, :]) @ np.abs(opB)) + abs(beta) * np.abs(c0[i, :]))
-            col = alpha * (opA @ opB[:, i]) + beta * c0[:, i]
-            same(c[:, i], col, abs(alpha) * (np.abs(opA) @ np.abs(opB[:, i])) + abs(beta) * np.abs(c0[:, i]))
-        X = rng.integers(-3, 4, (n, 6)).astype(wide)
+        for j in list(rng.integers(0, N, 7)) + [N - 1]:
+            col = alpha * (opA @ opB[:, j]) + beta * c0[:, j]
+            same(c[:, j], col, abs(alpha) * (np.abs(opA) @ np.abs(opB[:, j])) + abs(beta) * np.abs(c0[:, j]))
+        X = rng.integers(-3, 4, (N, 6)).astype(wide)
         want = alpha * (opA @ (opB @ X)) + beta * (c0 @ X)
         have = c @ X
         if exact:
@@ -218,6 +213,26 @@ def test_gemm_pipelined_whole_tiles(hip, stream, dtype, ta, tb):
         else:
             bound = abs(alpha) * (np.abs(opA) @ (np.abs(opB) @ np.abs(X))) + abs(beta) * (np.abs(c0) @ np.abs(X))
             assert np.linalg.norm(have - want) <= TOL[dtype] * np.linalg.norm(bound), what + " (probe vectors)"
+
+
+@pytest.mark.parametrize("dtype", [H.HALF, H.INT8, H.UINT8], ids=lambda d: H.NAMES[d])
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+def test_gemm_pipelined_whole_tiles(hip, stream, dtype, ta, tb):
+    """Products that the tile choice gives to the 256 x 256 tile (256 tiles or more) and that consist of whole aligned
+    tiles run on the hand-pipelined loop: one slab (start-up only), three and five slabs (clamped loads past the end, both
+    LDS buffers reused), with and without beta, scalars in host and in device memory."""
+    rng = np.random.default_rng(1200 + dtype + ord(ta) + 2 * ord(tb))
+    check_large_product(stream, dtype, ta, tb, 4096, 4096,
+                        ((1, 1, 0, False), (3, 2, -1 if dtype != H.UINT8 else 3, True), (5, -1 if dtype != H.UINT8 else 5, 1, False)), rng)
+
+
+@pytest.mark.parametrize("dtype", [H.HALF, H.INT8], ids=lambda d: H.NAMES[d])
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+def test_gemm_whole_tiles_and_edge_strips(hip, stream, dtype, ta, tb):
+    """A large aligned product whose sizes are not multiples of the tile: the whole tiles run on the pipelined loop, the
+    columns to their right and the rows below them as products of their own; the last row and column are among those checked."""
+    rng = np.random.default_rng(1300 + dtype + ord(ta) + 2 * ord(tb))
+    check_large_product(stream, dtype, ta, tb, 8080, 8016, ((2, 2, -1, False),), rng)
 
 
 def test_gemm_errors_and_empty(hip, stream):
