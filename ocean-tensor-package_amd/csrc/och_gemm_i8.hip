@@ -135,7 +135,7 @@ struct ByteSlab
       reg[v] = *reinterpret_cast<const och_gu32x4 *>(base + step + toff);
    }
    __device__ __forceinline__ void stash_one(char *buffer, int piece) const
-   {  static_assert(KC || NV == 8, "a transposed piece is a store of 8 bytes");
+   {  static_assert(KC || NV == 8 || NV == 4, "a transposed piece is a store of 8 or 4 bytes");
       if (KC)
       {  uint32_t mn, k; where(piece, mn, k);
          *reinterpret_cast<och_gu32x4 *>(buffer + (k / 16) * PLANE + mn * 16) = reg[piece];
@@ -144,11 +144,12 @@ struct ByteSlab
       {  uint32_t mn, k; where(0, mn, k);
          char *at = buffer + (k / 16) * PLANE + (mn / 16) * 16 + k % 16 + piece * (G * 16);
          const uint32_t sel = 0x0C0C0400u + (uint32_t)(piece & 3) * 0x0101u;
-         uint32_t pair[4];
+         uint32_t pair[NV / 2];
 #pragma unroll
-         for (int w = 0; w < 4; w++) pair[w] = __builtin_amdgcn_perm(reg[NV > 2 * w + 1 ? 2 * w + 1 : 1][piece >> 2], reg[NV > 2 * w ? 2 * w : 0][piece >> 2], sel);
-         uint2 t; t.x = (pair[0] & 0xFFFFu) | (pair[1] << 16); t.y = (pair[2] & 0xFFFFu) | (pair[3] << 16);
-         *reinterpret_cast<uint2 *>(at) = t;
+         for (int w = 0; w < NV / 2; w++) pair[w] = __builtin_amdgcn_perm(reg[2 * w + 1][piece >> 2], reg[2 * w][piece >> 2], sel);
+         const uint32_t w0 = (pair[0] & 0xFFFFu) | (pair[1] << 16);
+         if (NV == 4) *reinterpret_cast<uint32_t *>(at) = w0;
+         else { uint2 t; t.x = w0; t.y = (pair[NV > 4 ? 2 : 0] & 0xFFFFu) | (pair[NV > 4 ? 3 : 1] << 16); *reinterpret_cast<uint2 *>(at) = t; }
       }
    }
    /* the sixteen k of slot `slot` that lane group `kg` (0 or 1) feeds to MFMA step `ks` (32 k per step) */
@@ -478,7 +479,9 @@ template <bool BOOL> static int gemm_byte_pick(const GemmArgs &g)
             return 0;
          }
          return launch_gemm_byte<BOOL, 64, 128, 4, 2, 128>(g);
-      case 1:  return launch_gemm_byte<BOOL, 64, 64, 2, 2, 128>(g);
+      case 1:
+         if (!BOOL && g.M % 128 == 0 && g.N % 128 == 0 && g.K % 128 == 0) return launch_gemm_byte<BOOL, 64, 64, 2, 2, 128, true>(g);
+         return launch_gemm_byte<BOOL, 64, 64, 2, 2, 128>(g);
       default: return launch_gemm_byte<BOOL, 32, 32, 2, 2, 128>(g);
    }
 }

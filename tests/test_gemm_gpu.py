@@ -140,6 +140,8 @@ def test_gemm_half_matrix_cores(hip, stream, ta, tb):
                                               (64, 64, 32, 0, -1, 0.5, False), (96, 160, 2048, 0, 0.5, 0, True), (33, 47, 17, 5, 1, 0, False),
                                               (2560, 2304, 48, 0, 1, 1, False), (2500, 2300, 40, 4, 1, 0, False), (4096, 3072, 64, 0, 1, 0, False),
                                               (4000, 3100, 70, 0, -1, 1, True),
+                                              # whole aligned 128 x 128 tiles, three and five slabs of K: the pipelined loop on the middle tile
+                                              (2048, 2048, 192, 0, 2, -1, True), (2048, 2304, 320, 0, 1, 0, False),
                                               # results narrower than a tile, vectors, K below one MFMA step, K not a multiple of 8
                                               (2000, 1, 1000, 0, 1, 0, False), (1, 1500, 999, 0, 1, 1, False), (700, 9, 3, 1, 2, 0, False), (31, 31, 15, 0, 1, 0, False),
                                               # few tiles and a long K: cut along K, float partial sums added in order
@@ -158,6 +160,8 @@ def test_gemm_bytes_matrix_cores(hip, stream, dtype, ta, tb):
     for (M, N, K, pad, alpha, beta, dev) in [(128, 128, 128, 0, 1, 0, False), (256, 384, 160, 16, 2, neg, False), (200, 136, 100, 3, 1, 1, True),
                                               (64, 64, 32, 0, neg, 1, False), (96, 160, 2048, 0, 3, 0, True), (33, 47, 37, 5, 1, 0, False),
                                               (2560, 2304, 256, 0, 1, 1, False), (2500, 2300, 130, 4, 1, 0, False), (4096, 3072, 128, 0, 1, 0, False),
+                                              # whole aligned 128 x 128 tiles, three and five slabs of K: the pipelined loop on the middle tile
+                                              (2048, 2048, 384, 0, 2, neg, True), (2048, 2304, 640, 0, 1, 0, False),
                                               (1, 1500, 999, 0, 1, 1, False), (128, 64, 8192, 0, 1, 0, False), (1, 1, 70000, 0, 1, neg, True)]:
         if dtype == H.BOOL:
             alpha, beta = (1 if alpha else 0), (1 if beta else 0)
