@@ -133,6 +133,45 @@ def main():
                 print("   %7.1f  %7.1f   %s" % r)
             print("   ... %d forms measured; slowest: %7.1f  %7.1f   %s" % ((len(rows),) + rows[-1]))
             sys.stdout.flush()
+        # an independent implementation on the same sizes: PyTorch's own elementwise, copy and reduction kernels
+        try:
+            import torch
+        except ImportError:
+            return
+        dev = torch.device("cuda:0")
+
+        def torch_time(fn):
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            ts = []
+            for _ in range(20):
+                e0.record()
+                for _ in range(10):
+                    fn()
+                e1.record(); torch.cuda.synchronize()
+                ts.append(e0.elapsed_time(e1) / 10)
+            ts.sort()
+            return ts[len(ts) // 2], ts[0]
+        print("== PyTorch %s on the same device, three operand sets rotated, random data (GB/s median, best)" % torch.__version__)
+        n = 1 << 24
+        sets = [[torch.randn(n, dtype=torch.float64, device=dev) for _ in range(3)] for _ in range(3)]
+        turn = [0]
+
+        def t_add():
+            turn[0] += 1; a, b, c = sets[turn[0] % 3]; torch.add(a, b, out=c)
+
+        def t_copy():
+            turn[0] += 1; a, b, c = sets[turn[0] % 3]; c.copy_(a)
+        med, best = torch_time(t_add); print("   %7.1f  %7.1f   torch.add, float64, 134 MB operands (2 reads : 1 write)" % (24 * n / med / 1e6, 24 * n / best / 1e6))
+        med, best = torch_time(t_copy); print("   %7.1f  %7.1f   Tensor.copy_, float64, 134 MB operands (1 read : 1 write)" % (16 * n / med / 1e6, 16 * n / best / 1e6))
+        del sets
+        xs = [torch.randn(1 << 26, dtype=torch.float32, device=dev) for _ in range(3)]
+
+        def t_sum():
+            turn[0] += 1; return xs[turn[0] % 3].sum()
+        med, best = torch_time(t_sum); print("   %7.1f  %7.1f   torch.sum, float32, 268 MB (read only)" % (4 * (1 << 26) / med / 1e6, 4 * (1 << 26) / best / 1e6))
         return
 
     def sample_launches(fn, samples=None, warm=3, target_ms=0.6):
