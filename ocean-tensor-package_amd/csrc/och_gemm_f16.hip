@@ -449,7 +449,9 @@ static int launch_gemm_half(const GemmArgs &g)
    };
    p.alignedA = aligned(g.A, g.ldA, g.batch.sA) ? 1 : 0; p.alignedB = aligned(g.B, g.ldB, g.batch.sB) ? 1 : 0;
    p.alignedC = aligned(g.C, g.ldC, g.batch.sC) ? 1 : 0;
-   const bool edge = !(g.M % BM == 0 && g.N % BN == 0 && g.K % KT == 0 && p.alignedA && p.alignedB && p.alignedC);
+   /* the pipelined loop keeps a thread's offset within a slab in 32 bits: columns further apart than 64 MB take the guarded kernel */
+   const bool far = PIPE && ((int64_t)g.ldA * 2 >= (1 << 26) || (int64_t)g.ldB * 2 >= (1 << 26));
+   const bool edge = far || !(g.M % BM == 0 && g.N % BN == 0 && g.K % KT == 0 && p.alignedA && p.alignedB && p.alignedC);
    /* few tiles and a long K: slices of K in grid z, at least 8 slabs each, about 512 blocks in all, partial sums within the workspace */
    uint32_t slices = 1;
    {  const uint64_t nslabs = (g.K + KT - 1) / KT;

@@ -1,0 +1,262 @@
+/* float GEMM for whole aligned 256 x 256 tiles: C <- alpha * op(A) * op(B) + beta * C, column-major.
+ *
+ * The counterpart of cublasSgemm in the reference (src/core/gpu/op/tensor_blas_gpu.c:183-197). Four waves per block,
+ * one per SIMD, each owning 128 x 128 of the tile as 4 x 4 tiles of v_mfma_f32_32x32x2_f32 (256 accumulator registers).
+ * On this device a vector-ALU instruction of a wave takes about eight cycles away from the matrix cores of its SIMD, and
+ * a 64-cycle MFMA hides none of that; LDS reads and scalar instructions are nearly free. So the main loop holds MFMAs,
+ * LDS reads, scalar instructions and loads that go from memory straight to LDS -- no vector arithmetic, no staging
+ * registers, no LDS stores:
+ *
+ *   - a slab is 32 k. An operand that is contiguous along k in memory ("k-contiguous": A of a T product, B of an N
+ *     product) lies in LDS as 16-byte chunks of 4 k, chunk-major: [chunk][row][4 floats]; lane l of a load instruction
+ *     fetches one chunk of row l of the wave's 64 rows. An operand that is contiguous along m / n lies in LDS as it
+ *     lies in memory, [k][256 rows]; a load instruction fetches one k of all 256 rows. Either way the 64 lanes of a load
+ *     write 1 KB of consecutive LDS, which is what loads to LDS do (M0 holds the address, the lanes follow each other).
+ *   - an MFMA step consumes one float per lane and operand (lanes 0-31: one k, lanes 32-63: another). One 16-byte
+ *     fragment read yields, for a k-contiguous operand, the values of one 32-row tile for four steps; for the other
+ *     kind, the values of four tiles for one step, the tiles then being made of every fourth row (tile i = rows 4 r + i),
+ *     which is undone when C is written. Four steps are a "quad"; in step t of quad q the lanes hold k = 8 q + 4 (l / 32) + t
+ *     for both operands.
+ *   - a quad is 64 MFMAs = 32 chunks of two, each closed by a scheduling fence; the 8 fragment reads of the NEXT quad go
+ *     one to every fourth chunk (two sets of fragment registers). The one barrier of a slab stands in front of quad 3,
+ *     behind a wait for the wave's own loads: after it slab s + 1 is complete in the other buffer (quad 3 reads its
+ *     first fragments) and nobody reads the rest of this buffer again, so quad 3 and quad 0 of the next slab issue the
+ *     16 loads of slab s + 2 into it, one to every fourth chunk. A load has three quads (12000 cycles) to arrive.
+ *   - the loop body has no branches: slab numbers past the end are clamped (the last slab is loaded again into a buffer
+ *     nobody reads); it is written out twice so that all LDS offsets are immediates.
+ *   - C leaves through LDS in passes of 64 columns, so that memory sees 16-byte accesses along the columns of C.
+ */
+#include "och_gemm.h"
+#pragma clang diagnostic ignored "-Winline-asm"
+
+namespace och {
+
+typedef float och_f32x4 __attribute__((ext_vector_type(4)));
+
+#define OCH_FP_BM 256
+#define OCH_FP_KT 32
+#define OCH_FP_THREADS 256
+#define OCH_FP_OPERAND 33792                 /* LDS bytes of one operand's slab, either layout */
+#define OCH_FP_BUFFER (2 * OCH_FP_OPERAND)
+
+struct FloatPipeParams
+{
+   const char *A, *B; char *C;
+   int64_t  ldA, ldB, ldC;              /* in elements */
+   uint32_t M, N, K;
+   float    alpha, beta;
+   const float *alpha_dev, *beta_dev;
+   uint32_t tiles_m, tiles_n;
+   GemmBatch batch;
+};
+
+/* one operand's slab: where its loads come from and go to, where the fragments are read, which row of the 256 a
+   fragment value belongs to */
+template <bool KC>
+struct FloatSlab
+{
+   static constexpr int PLANE = 256 * 16 + 128;      /* KC: bytes per chunk plane; the odd 32 banks keep the two lane halves apart */
+   static constexpr int ROW = 256 * 4 + 32;          /* !KC: bytes per k */
+   static_assert(8 * PLANE <= OCH_FP_OPERAND && 32 * ROW <= OCH_FP_OPERAND, "slab does not fit");
+   /* load j (0 .. 7) of wave w: byte offset in memory relative to the slab's first element, per lane */
+   static __device__ __forceinline__ uint32_t load_offset(int j, uint32_t wave, uint32_t lane, int64_t ld)
+   {  return KC ? (uint32_t)((int64_t)(wave * 64 + lane) * ld * 4 + j * 16) : (uint32_t)((int64_t)(wave * 8 + j) * ld * 4 + lane * 16); }
+   /* ... and its first byte in the operand's LDS area (lane l writes 16 bytes at + 16 l) */
+   static __device__ __forceinline__ uint32_t load_target(int j, uint32_t wave)
+   {  return KC ? (uint32_t)j * PLANE + wave * 1024 : (wave * 8 + j) * ROW; }
+   static __device__ __forceinline__ const char *slab_base(const char *mat, int64_t ld, uint32_t mn0, uint32_t k0)
+   {  return mat + (KC ? ((int64_t)k0 + (int64_t)mn0 * ld) : ((int64_t)mn0 + (int64_t)k0 * ld)) * 4; }
+   /* fragment read x (0 .. 3) of quad q: the lane's part of the address, and the immediate part */
+   static __device__ __forceinline__ uint32_t read_lane(uint32_t wbase, uint32_t lane)
+   {  const uint32_t r = lane % 32, kg = lane / 32;
+      return KC ? kg * PLANE + (wbase + r) * 16 : 4 * kg * ROW + (wbase + 4 * r) * 4;
+   }
+   static constexpr uint32_t read_offset(int x, int q) { return KC ? (uint32_t)(2 * q * PLANE + x * 32 * 16) : (uint32_t)((8 * q + x) * ROW); }
+   /* the value of tile i and step t within a quad's four reads */
+   static __device__ __forceinline__ float value(const och_f32x4 (&f)[4], int i, int t) { return KC ? f[i][t] : f[t][i]; }
+   /* row (of the wave's 128) of tile i, row-in-tile rr */
+   static __device__ __forceinline__ uint32_t row(int i, uint32_t rr) { return KC ? (uint32_t)i * 32 + rr : 4 * rr + (uint32_t)i; }
+};
+
+/* one load from memory straight to LDS: lane l brings 16 bytes from base + offset[l] to LDS byte target + 16 l */
+static __device__ __forceinline__ void load_to_lds(const char *base, uint32_t offset, uint32_t target)
+{
+   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(target), "v"(offset), "s"(base) : "memory");
+}
+
+template <bool AKC, bool BKC>
+__global__ __launch_bounds__(OCH_FP_THREADS) void gemm_float_pipe_kernel(const FloatPipeParams p)
+{
+   constexpr int T = 32, BM = OCH_FP_BM, BN = OCH_FP_BM, KT = OCH_FP_KT, TMS = 4, TNS = 4, WM = 128, WN = 128, THREADS = OCH_FP_THREADS;
+   constexpr uint32_t OP = OCH_FP_OPERAND, BUF = OCH_FP_BUFFER;
+   typedef FloatSlab<AKC> LA;
+   typedef FloatSlab<BKC> LB;
+   extern __shared__ __align__(16) char lds[];
+
+   int64_t oA, oB, oC, oAlpha, oBeta;
+   gemm_batch_offsets(p.batch, oA, oB, oC, oAlpha, oBeta);
+   const char *pA = p.A + oA, *pB = p.B + oB; char *pC = p.C + oC;
+   const uint32_t tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
+   const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+   const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+   const uint32_t wm = (wave % 2) * WM, wn = (wave / 2) * WN;
+
+   och_f32x16 acc[TMS][TNS];
+#pragma unroll
+   for (int i = 0; i < TMS; i++)
+#pragma unroll
+      for (int j = 0; j < TNS; j++)
+#pragma unroll
+         for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+
+   const uint32_t nslabs = p.K / KT, last = nslabs - 1;
+   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)lds;      /* where the array starts in LDS */
+   uint32_t offA[8], offB[8], tgtA[8], tgtB[8];
+#pragma unroll
+   for (int j = 0; j < 8; j++)
+   {  offA[j] = LA::load_offset(j, wave, lane, p.ldA); offB[j] = LB::load_offset(j, wave, lane, p.ldB);
+      tgtA[j] = lds0 + LA::load_target(j, wave); tgtB[j] = lds0 + OP + LB::load_target(j, wave);
+   }
+   /* the lane's read addresses in buffer 0 and buffer 1, in registers of their own (the empty asm keeps the compiler
+      from deriving the second from the first with an addition at every read: the distance is beyond a read's immediate) */
+   const char *readA[2], *readB[2];
+   {  uint32_t a1 = LA::read_lane(wm, lane) + BUF, b1 = OP + LB::read_lane(wn, lane) + BUF;
+      asm volatile("" : "+v"(a1), "+v"(b1));
+      readA[0] = lds + LA::read_lane(wm, lane); readA[1] = lds + a1;
+      readB[0] = lds + OP + LB::read_lane(wn, lane); readB[1] = lds + b1;
+   }
+   och_f32x4 fa[2][4], fb[2][4];
+
+   /* load number e (0 .. 15; A first) of slab `slab` into buffer `buf` */
+#define OCH_LOAD(e, baseA, baseB, buf)                                                                                 \
+   do { if ((e) < 8) load_to_lds(baseA, offA[(e) % 8], tgtA[(e) % 8] + (buf) * BUF);                                   \
+        else         load_to_lds(baseB, offB[(e) % 8], tgtB[(e) % 8] + (buf) * BUF); } while (0)
+   /* one quad: chunk c reads fragment c / 4 of quad QN from buffer RB into set NXT when c is a multiple of four, issues
+      load LOAD0 + c / 4 into buffer LBUF when c % 4 == 2 and LOADS is set, then runs its two MFMAs */
+#define OCH_QUAD(CUR, NXT, RB, QN, LOADS, LOAD0, LBUF)                                                                 \
+   do { _Pragma("unroll") for (int c = 0; c < 32; c++)                                                                \
+        {  if (c % 4 == 0)                                                                                             \
+           {  if (c / 4 < 4) fa[NXT][c / 4 % 4] = *reinterpret_cast<const och_f32x4 *>(readA[RB] + LA::read_offset(c / 4 % 4, QN)); \
+              else           fb[NXT][c / 4 % 4] = *reinterpret_cast<const och_f32x4 *>(readB[RB] + LB::read_offset(c / 4 % 4, QN)); \
+           }                                                                                                           \
+           if (LOADS && c % 4 == 2) OCH_LOAD(LOAD0 + c / 4, nextA, nextB, LBUF);                                       \
+           {  const int st = c / 8, m = (c % 8) * 2, i = m / TNS, j = m % TNS;                                         \
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(LA::value(fa[CUR], i, st), LB::value(fb[CUR], j, st), acc[i][j], 0, 0, 0); \
+              acc[i][j + 1] = __builtin_amdgcn_mfma_f32_32x32x2f32(LA::value(fa[CUR], i, st), LB::value(fb[CUR], j + 1, st), acc[i][j + 1], 0, 0, 0); \
+           }                                                                                                           \
+           __builtin_amdgcn_sched_barrier(0);                                                                          \
+        } } while (0)
+   /* slab s in buffer CB: quad 0 carries the second half of the loads of slab s + 1 (into the other buffer), quad 3 the
+      first half of the loads of slab s + 2 (into this one) */
+#define OCH_SLAB(s, CB)                                                                                                \
+   do { {  const uint32_t s1 = ((s) + 1 < last) ? (s) + 1 : last;                                                      \
+           const char *nextA = LA::slab_base(pA, p.ldA, m0, s1 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, s1 * KT);  \
+           OCH_QUAD(0, 1, CB, 1, true, 8, 1 - CB);                                                                     \
+        }                                                                                                              \
+        {  const char *nextA = nullptr, *nextB = nullptr;                                                              \
+           OCH_QUAD(1, 0, CB, 2, false, 0, 0);                                                                         \
+           OCH_QUAD(0, 1, CB, 3, false, 0, 0);                                                                         \
+        }                                                                                                              \
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                               \
+        __syncthreads();                                                                                               \
+        {  const uint32_t s2 = ((s) + 2 < last) ? (s) + 2 : last;                                                      \
+           const char *nextA = LA::slab_base(pA, p.ldA, m0, s2 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, s2 * KT);  \
+           OCH_QUAD(1, 0, 1 - CB, 0, true, 0, CB);                                                                     \
+        } } while (0)
+
+   {  /* slab 0 and the first half of slab 1 */
+      const uint32_t s1 = (1 < last) ? 1 : last;
+      const char *nextA = LA::slab_base(pA, p.ldA, m0, 0), *nextB = LB::slab_base(pB, p.ldB, n0, 0);
+#pragma unroll
+      for (int e = 0; e < 16; e++) OCH_LOAD(e, nextA, nextB, 0);
+      nextA = LA::slab_base(pA, p.ldA, m0, s1 * KT); nextB = LB::slab_base(pB, p.ldB, n0, s1 * KT);
+#pragma unroll
+      for (int e = 0; e < 8; e++) OCH_LOAD(e, nextA, nextB, 1);
+      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      __syncthreads();
+#pragma unroll
+      for (int x = 0; x < 4; x++)
+      {  fa[0][x] = *reinterpret_cast<const och_f32x4 *>(readA[0] + LA::read_offset(x, 0));
+         fb[0][x] = *reinterpret_cast<const och_f32x4 *>(readB[0] + LB::read_offset(x, 0));
+      }
+   }
+   uint32_t s = 0;
+   for (; s + 1 < nslabs; s += 2)
+   {  OCH_SLAB(s, 0);
+      OCH_SLAB(s + 1, 1);
+   }
+   if (s < nslabs) OCH_SLAB(s, 0);
+   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+   __syncthreads();
+#undef OCH_SLAB
+#undef OCH_QUAD
+#undef OCH_LOAD
+
+   /* epilogue: accumulator register r of lane l is row-in-tile 8 * (r / 4) + 4 * (l / 32) + r % 4 of A's tile and
+      row-in-tile l % 32 of B's. The scaled tile goes through LDS, 64 columns at a time with a pitch of BM + 4 floats, and
+      leaves (after beta * C has been added) in 16-byte pieces that follow the columns of C. */
+   float alpha = p.alpha, beta = p.beta;
+   if (p.alpha_dev) alpha = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(p.alpha_dev) + oAlpha);
+   if (p.beta_dev)  beta = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(p.beta_dev) + oBeta);
+   constexpr int CP = BM + 4, CPASS = 64, PASSES = BN / CPASS;
+   static_assert(CPASS * CP * 4 <= 2 * BUF, "a pass of the staged tile does not fit into the slab buffers");
+   float *stage = reinterpret_cast<float *>(lds);
+   for (int h = 0; h < PASSES; h++)
+   {
+#pragma unroll
+      for (int j = 0; j < TNS; j++)
+      {  const uint32_t col = wn + LB::row(j, lane % T);
+         if (col / CPASS != (uint32_t)h) continue;
+#pragma unroll
+         for (int i = 0; i < TMS; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+               stage[(col - h * CPASS) * CP + wm + LA::row(i, 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3))] = alpha * acc[i][j][r];
+      }
+      __syncthreads();
+      const uint32_t c0 = n0 + h * CPASS;
+      for (uint32_t q = threadIdx.x; q < CPASS * (BM / 4); q += THREADS)
+      {  const uint32_t c = q / (BM / 4), r4 = (q % (BM / 4)) * 4;
+         och_f32x4 v = *reinterpret_cast<const och_f32x4 *>(stage + c * CP + r4);
+         och_f32x4 *dst = reinterpret_cast<och_f32x4 *>(pC + ((int64_t)(m0 + r4) + (int64_t)(c0 + c) * p.ldC) * 4);
+         if (beta != 0) { const och_f32x4 old = *dst; v.x += beta * old.x; v.y += beta * old.y; v.z += beta * old.z; v.w += beta * old.w; }
+         *dst = v;
+      }
+      __syncthreads();
+   }
+}
+
+/* 0: launched; 1: not a case for this kernel (the caller's other kernels take it) */
+int gemm_float_pipe(const GemmArgs &g)
+{
+   if (g.M % OCH_FP_BM != 0 || g.N % OCH_FP_BM != 0 || g.K % OCH_FP_KT != 0 || g.K == 0 || !gemm_operands_aligned(g, 4)) return 1;
+   /* a lane's offset within a slab (up to 255 columns further on) is kept in 32 bits */
+   if ((int64_t)g.ldA * 4 >= (1 << 24) || (int64_t)g.ldB * 4 >= (1 << 24)) return 1;
+   FloatPipeParams p;
+   memset(&p, 0, sizeof(p));
+   p.A = (const char *)g.A; p.B = (const char *)g.B; p.C = (char *)g.C;
+   p.ldA = g.ldA; p.ldB = g.ldB; p.ldC = g.ldC;
+   p.M = (uint32_t)g.M; p.N = (uint32_t)g.N; p.K = (uint32_t)g.K;
+   if (g.scalar_mode_host) { memcpy(&p.alpha, g.alpha, 4); memcpy(&p.beta, g.beta, 4); }
+   else { p.alpha_dev = (const float *)g.alpha; p.beta_dev = (const float *)g.beta; }
+   p.batch = g.batch;
+   p.tiles_m = (uint32_t)(g.M / OCH_FP_BM); p.tiles_n = (uint32_t)(g.N / OCH_FP_BM);
+   const uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
+   if (blocks > 0x7FFFFFFFull) return set_error("gemm: too many tiles");
+   const bool akc = (g.transA != 'N'), bkc = (g.transB == 'N');
+   const dim3 grid((unsigned)blocks, 1, g.nz), block(OCH_FP_THREADS);
+   const size_t lds = 2 * (size_t)OCH_FP_BUFFER;
+#define OCH_FP_LAUNCH(AK, BK)                                                                                         \
+   do { auto kernel = gemm_float_pipe_kernel<AK, BK>;                                                                 \
+        OCH_CHECK_HIP(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+        hipLaunchKernelGGL(kernel, grid, block, lds, g.stream, p); } while (0)
+   if (!akc && !bkc) OCH_FP_LAUNCH(false, false);
+   else if (!akc)    OCH_FP_LAUNCH(false, true);
+   else if (!bkc)    OCH_FP_LAUNCH(true, false);
+   else              OCH_FP_LAUNCH(true, true);
+#undef OCH_FP_LAUNCH
+   OCH_CHECK_LAUNCH();
+   return 0;
+}
+
+} /* namespace och */

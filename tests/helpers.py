@@ -29,6 +29,11 @@ def f32_to_half_bits(a):
     a = np.ascontiguousarray(a, dtype=np.float32)
     out = np.empty(a.shape, dtype=np.uint16)
     flat_in, flat_out = a.reshape(-1), out.reshape(-1)
+    if flat_in.size >= 64:
+        # the same converter, applied by the oracle's converting copy instead of one call per element
+        n = flat_in.size
+        assert orc.lib.oracle_copy(FLOAT, HALF, 1, oh.sizes([n]), oh.strides([4]), orc.ptr(flat_in), 1, oh.sizes([n]), oh.strides([2]), orc.ptr(flat_out), 8) == 0
+        return out
     for i in range(flat_in.size):
         flat_out[i] = orc.lib.oracle_float_to_half(float(flat_in[i]))
     return out

@@ -168,18 +168,20 @@ def test_gemm_bytes_matrix_cores(hip, stream, dtype, ta, tb):
         run_case(stream, dtype, ta, tb, M, N, K, alpha, beta, rng, device_scalars=dev, pad=pad, kind="full")
 
 
-def check_large_product(stream, dtype, ta, tb, M, N, cases, rng):
+def check_large_product(stream, dtype, ta, tb, M, N, cases, rng, pad=0):
     """Large products checked without O(n^3) host work: eight complete rows and columns of C computed directly, and C
     times probe vectors against op(A) (op(B) x) -- in exact arithmetic modulo 256 for the 8-bit types, to the
-    half-precision bound for half. cases: (slabs of K, alpha, beta, scalars in device memory)."""
-    kt = 64 if dtype == H.HALF else 128
-    exact = dtype != H.HALF
+    precision's bound for half and float. cases: (slabs of K, alpha, beta, scalars in device memory); pad: rows of
+    junk between the columns of all three operands."""
+    kt = {H.HALF: 64, H.FLOAT: 32}.get(dtype, 128)
+    exact = dtype not in (H.HALF, H.FLOAT)
     for slabs, alpha, beta, dev in cases:
         K = slabs * kt
         rowsA, colsA = (M, K) if ta == "N" else (K, M)
         rowsB, colsB = (K, N) if tb == "N" else (N, K)
-        A, B, C0 = matrix(dtype, rowsA, colsA, rowsA, rng, "full" if exact else "small"), matrix(dtype, rowsB, colsB, rowsB, rng, "full" if exact else "small"), \
-            matrix(dtype, M, N, M, rng, "full" if exact else "small")
+        ldA, ldB, ldC = rowsA + pad, rowsB + pad, M + pad
+        A, B, C0 = matrix(dtype, rowsA, colsA, ldA, rng, "full" if exact else "small"), matrix(dtype, rowsB, colsB, ldB, rng, "full" if exact else "small"), \
+            matrix(dtype, M, N, ldC, rng, "full" if exact else "small")
         al, be = scalar_of(dtype, alpha), scalar_of(dtype, beta)
         dA, dB, dC = oh.to_device(A, stream), oh.to_device(B, stream), oh.to_device(C0, stream)
         if dev:
@@ -187,15 +189,16 @@ def check_large_product(stream, dtype, ta, tb, M, N, cases, rng):
             pal, pbe, mode = dal.ptr, dbe.ptr, 0
         else:
             pal, pbe, mode = orc.ptr(al), orc.ptr(be), 1
-        oh.check(oh.lib.och_gemm(dtype, ta.encode(), tb.encode(), M, N, K, pal, dA.ptr, rowsA, dB.ptr, rowsB, pbe, dC.ptr, M, mode, stream.handle))
+        oh.check(oh.lib.och_gemm(dtype, ta.encode(), tb.encode(), M, N, K, pal, dA.ptr, ldA, dB.ptr, ldB, pbe, dC.ptr, ldC, mode, stream.handle))
         got = dC.download(C0.dtype, C0.size)
         for b in (dA, dB, dC):
             b.free()
         wide = np.int64 if exact else np.float64
         num = (lambda a: a.astype(np.int64)) if exact else (lambda a: as_float(dtype, a).astype(np.float64))
-        mA, mB = num(A).reshape(colsA, rowsA).T, num(B).reshape(colsB, rowsB).T            # [row, col]
+        mA, mB = num(A).reshape(colsA, ldA)[:, :rowsA].T, num(B).reshape(colsB, ldB)[:, :rowsB].T            # [row, col]
         opA, opB = (mA if ta == "N" else mA.T), (mB if tb == "N" else mB.T)
-        c0, c = num(C0).reshape(N, M).T, num(got).reshape(N, M).T
+        c0, c = num(C0).reshape(N, ldC)[:, :M].T, num(got).reshape(N, ldC)[:, :M].T
+        assert np.array_equal(got.reshape(N, ldC)[:, M:], C0.reshape(N, ldC)[:, M:]), "padding of C written"
         what = "%s %s%s %dx%dx%d alpha=%r beta=%r" % (H.NAMES[dtype], ta, tb, M, N, K, alpha, beta)
 
         def same(have, want, bound):
@@ -219,6 +222,16 @@ def check_large_product(stream, dtype, ta, tb, M, N, cases, rng):
             assert np.linalg.norm(have - want) <= TOL[dtype] * np.linalg.norm(bound), what + " (probe vectors)"
 
 
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+def test_gemm_float_pipelined_whole_tiles(hip, stream, ta, tb):
+    """float products of 256 whole aligned 256 x 256 tiles or more run on the hand-pipelined kernel: one slab of 32 k
+    (start-up only), three and six slabs (clamped loads past the end, both LDS buffers reused), with and without beta,
+    scalars in host and in device memory, columns with and without junk between them."""
+    rng = np.random.default_rng(1300 + ord(ta) + 2 * ord(tb))
+    check_large_product(stream, H.FLOAT, ta, tb, 4096, 4096, ((1, 1, 0, False), (3, 2, -1, True)), rng)
+    check_large_product(stream, H.FLOAT, ta, tb, 4096, 4096, ((6, -1.5, 0.5, False),), rng, pad=12)
+
+
 @pytest.mark.parametrize("dtype", [H.HALF, H.INT8, H.UINT8], ids=lambda d: H.NAMES[d])
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
 def test_gemm_pipelined_whole_tiles(hip, stream, dtype, ta, tb):
@@ -230,7 +243,7 @@ def test_gemm_pipelined_whole_tiles(hip, stream, dtype, ta, tb):
                         ((1, 1, 0, False), (3, 2, -1 if dtype != H.UINT8 else 3, True), (5, -1 if dtype != H.UINT8 else 5, 1, False)), rng)
 
 
-@pytest.mark.parametrize("dtype", [H.HALF, H.INT8], ids=lambda d: H.NAMES[d])
+@pytest.mark.parametrize("dtype", [H.HALF, H.INT8, H.FLOAT], ids=lambda d: H.NAMES[d])
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
 def test_gemm_whole_tiles_and_edge_strips(hip, stream, dtype, ta, tb):
     """A large aligned product whose sizes are not multiples of the tile: the whole tiles run on the pipelined loop, the
