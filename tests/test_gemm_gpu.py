@@ -173,8 +173,8 @@ def check_large_product(stream, dtype, ta, tb, M, N, cases, rng, pad=0):
     times probe vectors against op(A) (op(B) x) -- in exact arithmetic modulo 256 for the 8-bit types, to the
     precision's bound for half and float. cases: (slabs of K, alpha, beta, scalars in device memory); pad: rows of
     junk between the columns of all three operands."""
-    kt = {H.HALF: 64, H.FLOAT: 32}.get(dtype, 128)
-    exact = dtype not in (H.HALF, H.FLOAT)
+    kt = {H.HALF: 64, H.FLOAT: 32, H.DOUBLE: 16}.get(dtype, 128)
+    exact = dtype not in (H.HALF, H.FLOAT, H.DOUBLE)
     for slabs, alpha, beta, dev in cases:
         K = slabs * kt
         rowsA, colsA = (M, K) if ta == "N" else (K, M)
@@ -232,6 +232,17 @@ def test_gemm_float_pipelined_whole_tiles(hip, stream, ta, tb):
     check_large_product(stream, H.FLOAT, ta, tb, 4096, 4096, ((6, -1.5, 0.5, False),), rng, pad=12)
 
 
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
+def test_gemm_double_pipelined_whole_tiles(hip, stream, ta, tb):
+    """double products of 256 whole aligned 256 x 128 tiles or more run on the hand-pipelined kernel, whose three slab
+    buffers rotate: one, two and three slabs of 16 k (start-up and each tail of the rotation), four and eight slabs (all
+    buffers reused, clamped loads past the end), with and without beta, scalars in host and in device memory, columns with
+    and without junk between them."""
+    rng = np.random.default_rng(1400 + ord(ta) + 2 * ord(tb))
+    check_large_product(stream, H.DOUBLE, ta, tb, 4096, 2048, ((1, 1, 0, False), (2, 2, -1, True), (3, -1, 1, False)), rng)
+    check_large_product(stream, H.DOUBLE, ta, tb, 4096, 2048, ((4, 1.5, 0, True), (8, -1.5, 0.5, False)), rng, pad=6)
+
+
 @pytest.mark.parametrize("dtype", [H.HALF, H.INT8, H.UINT8], ids=lambda d: H.NAMES[d])
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
 def test_gemm_pipelined_whole_tiles(hip, stream, dtype, ta, tb):
@@ -243,7 +254,7 @@ def test_gemm_pipelined_whole_tiles(hip, stream, dtype, ta, tb):
                         ((1, 1, 0, False), (3, 2, -1 if dtype != H.UINT8 else 3, True), (5, -1 if dtype != H.UINT8 else 5, 1, False)), rng)
 
 
-@pytest.mark.parametrize("dtype", [H.HALF, H.INT8, H.FLOAT], ids=lambda d: H.NAMES[d])
+@pytest.mark.parametrize("dtype", [H.HALF, H.INT8, H.FLOAT, H.DOUBLE], ids=lambda d: H.NAMES[d])
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
 def test_gemm_whole_tiles_and_edge_strips(hip, stream, dtype, ta, tb):
     """A large aligned product whose sizes are not multiples of the tile: the whole tiles run on the pipelined loop, the
