@@ -593,6 +593,7 @@ int gemm_float_pipe(const GemmArgs &g); /* whole aligned 256 x 256 tiles; 1: not
 int gemm_double(const GemmArgs &g);
 int gemm_double_pipe(const GemmArgs &g); /* whole aligned 256 x 128 tiles; 1: not taken */
 int gemm_cfloat(const GemmArgs &g);
+int gemm_cfloat_pipe(const GemmArgs &g); /* whole aligned 128 x 128 tiles; 1: not taken */
 int gemm_cdouble(const GemmArgs &g);
 int gemm_half(const GemmArgs &g);      /* 1: not taken, use the generic kernel */
 int gemm_int8(const GemmArgs &g);      /* int8 and uint8; 1: not taken */

@@ -173,8 +173,8 @@ def check_large_product(stream, dtype, ta, tb, M, N, cases, rng, pad=0):
     times probe vectors against op(A) (op(B) x) -- in exact arithmetic modulo 256 for the 8-bit types, to the
     precision's bound for half and float. cases: (slabs of K, alpha, beta, scalars in device memory); pad: rows of
     junk between the columns of all three operands."""
-    kt = {H.HALF: 64, H.FLOAT: 32, H.DOUBLE: 16}.get(dtype, 128)
-    exact = dtype not in (H.HALF, H.FLOAT, H.DOUBLE)
+    kt = {H.HALF: 64, H.FLOAT: 32, H.DOUBLE: 16, H.CFLOAT: 32}.get(dtype, 128)
+    exact = dtype not in (H.HALF, H.FLOAT, H.DOUBLE, H.CFLOAT)
     for slabs, alpha, beta, dev in cases:
         K = slabs * kt
         rowsA, colsA = (M, K) if ta == "N" else (K, M)
@@ -193,10 +193,11 @@ def check_large_product(stream, dtype, ta, tb, M, N, cases, rng, pad=0):
         got = dC.download(C0.dtype, C0.size)
         for b in (dA, dB, dC):
             b.free()
-        wide = np.int64 if exact else np.float64
-        num = (lambda a: a.astype(np.int64)) if exact else (lambda a: as_float(dtype, a).astype(np.float64))
+        wide = np.int64 if exact else (np.complex128 if dtype == H.CFLOAT else np.float64)
+        num = (lambda a: a.astype(np.int64)) if exact else (lambda a: as_float(dtype, a).astype(wide))
         mA, mB = num(A).reshape(colsA, ldA)[:, :rowsA].T, num(B).reshape(colsB, ldB)[:, :rowsB].T            # [row, col]
-        opA, opB = (mA if ta == "N" else mA.T), (mB if tb == "N" else mB.T)
+        op = {"N": lambda m: m, "T": lambda m: m.T, "C": lambda m: m.conj().T}
+        opA, opB = op[ta](mA), op[tb](mB)
         c0, c = num(C0).reshape(N, ldC)[:, :M].T, num(got).reshape(N, ldC)[:, :M].T
         assert np.array_equal(got.reshape(N, ldC)[:, M:], C0.reshape(N, ldC)[:, M:]), "padding of C written"
         what = "%s %s%s %dx%dx%d alpha=%r beta=%r" % (H.NAMES[dtype], ta, tb, M, N, K, alpha, beta)
@@ -232,6 +233,16 @@ def test_gemm_float_pipelined_whole_tiles(hip, stream, ta, tb):
     check_large_product(stream, H.FLOAT, ta, tb, 4096, 4096, ((6, -1.5, 0.5, False),), rng, pad=12)
 
 
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T"), ("C", "N"), ("N", "C"), ("C", "C"), ("T", "C")])
+def test_gemm_cfloat_pipelined_whole_tiles(hip, stream, ta, tb):
+    """complex float products of 256 whole aligned 128 x 128 tiles or more run on the hand-pipelined kernel, which sums
+    Ar Br, Ai Bi, Ar Bi and Ai Br apart and combines them with the signs the conjugations ask for: one, three and six
+    slabs of 32 k, complex alpha and beta, scalars in host and in device memory, columns with and without junk between them."""
+    rng = np.random.default_rng(1500 + ord(ta) + 2 * ord(tb))
+    check_large_product(stream, H.CFLOAT, ta, tb, 2048, 2048, ((1, 1, 0, False), (3, 2 - 1j, -1 + 0.5j, True)), rng)
+    check_large_product(stream, H.CFLOAT, ta, tb, 2048, 2048, ((6, -1.5j, 0.5, False),), rng, pad=6)
+
+
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
 def test_gemm_double_pipelined_whole_tiles(hip, stream, ta, tb):
     """double products of 256 whole aligned 256 x 128 tiles or more run on the hand-pipelined kernel, whose three slab
@@ -254,7 +265,7 @@ def test_gemm_pipelined_whole_tiles(hip, stream, dtype, ta, tb):
                         ((1, 1, 0, False), (3, 2, -1 if dtype != H.UINT8 else 3, True), (5, -1 if dtype != H.UINT8 else 5, 1, False)), rng)
 
 
-@pytest.mark.parametrize("dtype", [H.HALF, H.INT8, H.FLOAT, H.DOUBLE], ids=lambda d: H.NAMES[d])
+@pytest.mark.parametrize("dtype", [H.HALF, H.INT8, H.FLOAT, H.DOUBLE, H.CFLOAT], ids=lambda d: H.NAMES[d])
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
 def test_gemm_whole_tiles_and_edge_strips(hip, stream, dtype, ta, tb):
     """A large aligned product whose sizes are not multiples of the tile: the whole tiles run on the pipelined loop, the
