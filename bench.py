@@ -133,6 +133,27 @@ def main():
                 print("   %7.1f  %7.1f   %s" % r)
             print("   ... %d forms measured; slowest: %7.1f  %7.1f   %s" % ((len(rows),) + rows[-1]))
             sys.stdout.flush()
+        # matrix cores: a loop of nothing but MFMAs, and what other instructions of the same wave cost between them
+        def mfmabench(typ, kind, per, waves, iters=4000):
+            ms, flop = C.c_float(), C.c_double()
+            oh.check(lib.och_mfmabench(typ, kind, per, waves, iters, 7, C.byref(ms), C.byref(flop), h))
+            return ms.value, flop.value
+        print("== matrix cores (och_mfmabench): 16 independent MFMAs per iteration, one block of 4 waves per compute unit (one wave per SIMD)")
+        peaks = (("float 32x32x2", MFMA_PEAK["float"]), ("double 16x16x4", MFMA_PEAK["double"]), ("half 32x32x16", 2500.0), ("int8 32x32x32", 5000.0))
+        for typ, (name, peak) in enumerate(peaks):
+            mfmabench(typ, 0, 0, 4, 16000)                       # warm: the clock settles under this load
+            ms, flop = mfmabench(typ, 0, 0, 4, 16000)
+            print("   %-16s MFMAs alone: %8.1f T/s = %.3f of the nominal %.1f" % (name, flop / ms / 1e9, flop / ms / 1e9 / peak, peak))
+        print("   cost of an instruction between 64-cycle float MFMAs, in MFMA cycles (64 x time / time of the bare loop - 64) per instruction:")
+        for waves in (4, 8):
+            base, _ = mfmabench(0, 0, 0, waves)
+            for kind, name in ((1, "v_mov_b32"), (2, "v_add_f32"), (3, "s_nop"), (4, "s_add_u32"), (5, "s_waitcnt"), (6, "ds_read_b128")):
+                cells = []
+                for per in (1, 2, 4):
+                    ms, _ = mfmabench(0, kind, per, waves)
+                    cells.append("%5.1f" % ((ms / base - 1.0) * 64.0 / per))
+                print("   %d wave(s) per SIMD  %-13s 1 / 2 / 4 per MFMA: %s" % (waves // 4, name, "  ".join(cells)))
+        sys.stdout.flush()
         # an independent implementation on the same sizes: PyTorch's own elementwise, copy and reduction kernels
         try:
             import torch
