@@ -589,7 +589,7 @@ static inline bool gemm_operands_aligned(const GemmArgs &g, int es)
 }
 
 int gemm_float(const GemmArgs &g);
-int gemm_float_pipe(const GemmArgs &g); /* whole aligned 256 x 256 tiles; 1: not taken */
+int gemm_float_pipe(const GemmArgs &g, int tile); /* whole aligned tiles of 256 x 256 or 128 x 128; 1: not taken */
 int gemm_double(const GemmArgs &g);
 int gemm_double_pipe(const GemmArgs &g); /* whole aligned 256 x 128 tiles; 1: not taken */
 int gemm_cfloat(const GemmArgs &g);

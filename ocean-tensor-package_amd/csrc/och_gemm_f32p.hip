@@ -1,7 +1,9 @@
-/* float GEMM for whole aligned 256 x 256 tiles: C <- alpha * op(A) * op(B) + beta * C, column-major.
+/* float GEMM for whole aligned 256 x 256 or 128 x 128 tiles: C <- alpha * op(A) * op(B) + beta * C, column-major.
  *
  * The counterpart of cublasSgemm in the reference (src/core/gpu/op/tensor_blas_gpu.c:183-197). Four waves per block,
- * one per SIMD, each owning 128 x 128 of the tile as 4 x 4 tiles of v_mfma_f32_32x32x2_f32 (256 accumulator registers).
+ * one per SIMD, each owning 128 x 128 of the tile as 4 x 4 tiles of v_mfma_f32_32x32x2_f32 (256 accumulator registers);
+ * for products with fewer than one such tile per compute unit the same kernel with TS = 2: waves of 64 x 64 (2 x 2
+ * tiles), two blocks per compute unit. The description is for TS = 4.
  * On this device a vector-ALU instruction of a wave takes about eight cycles away from the matrix cores of its SIMD, and
  * a 64-cycle MFMA hides none of that; LDS reads and scalar instructions are nearly free. So the main loop holds MFMAs,
  * LDS reads, scalar instructions and loads that go from memory straight to LDS -- no vector arithmetic, no staging
@@ -33,11 +35,8 @@ namespace och {
 
 typedef float och_f32x4 __attribute__((ext_vector_type(4)));
 
-#define OCH_FP_BM 256
 #define OCH_FP_KT 32
 #define OCH_FP_THREADS 256
-#define OCH_FP_OPERAND 33792                 /* LDS bytes of one operand's slab, either layout */
-#define OCH_FP_BUFFER (2 * OCH_FP_OPERAND)
 
 struct FloatPipeParams
 {
@@ -50,32 +49,49 @@ struct FloatPipeParams
    GemmBatch batch;
 };
 
-/* one operand's slab: where its loads come from and go to, where the fragments are read, which row of the 256 a
-   fragment value belongs to */
-template <bool KC>
+/* one operand's slab of ROWS = 256 or 128 rows: where its loads come from and go to, where the fragments are read, which
+   row a fragment value belongs to. TS = ROWS / 64 tiles of 32 rows per wave. */
+template <bool KC, int ROWS>
 struct FloatSlab
 {
-   static constexpr int PLANE = 256 * 16 + 128;      /* KC: bytes per chunk plane; the odd 32 banks keep the two lane halves apart */
-   static constexpr int ROW = 256 * 4 + 32;          /* !KC: bytes per k */
-   static_assert(8 * PLANE <= OCH_FP_OPERAND && 32 * ROW <= OCH_FP_OPERAND, "slab does not fit");
-   /* load j (0 .. 7) of wave w: byte offset in memory relative to the slab's first element, per lane */
+   static constexpr int TS = ROWS / 64;
+   static constexpr int PLANE = ROWS * 16 + 128;     /* KC: bytes per chunk plane; the odd 32 banks keep the two lane halves apart */
+   static constexpr int KPI = 256 / ROWS;            /* !KC: k per load instruction (1 KB of rows) and ... */
+   static constexpr int UNIT = 1024 + 32 * KPI;      /* ... bytes from one instruction's rows to the next one's */
+   static constexpr int OPERAND = 8 * PLANE;         /* LDS bytes of the slab, either layout */
+   static_assert((32 / KPI) * UNIT <= OPERAND, "slab does not fit");
+   static constexpr int LOADS = ROWS / 32;           /* loads per wave and slab */
+   static constexpr int GROUPS = ROWS / 64;          /* KC: groups of 64 rows, one row per lane */
+   static constexpr int READS = KC ? TS : 4;         /* fragment reads per quad */
+   static constexpr uint32_t k_offset(int k) { return (uint32_t)((k / KPI) * UNIT + (k % KPI) * ROWS * 4); }      /* !KC: where k starts */
+   /* load j of wave w: byte offset in memory relative to the slab's first element, per lane. KC: chunk (w / GROUPS) * LOADS + j
+      of the rows of group w % GROUPS; !KC: k = (w * LOADS + j) * KPI + lane / (64 / KPI), 16 bytes of rows per lane */
    static __device__ __forceinline__ uint32_t load_offset(int j, uint32_t wave, uint32_t lane, int64_t ld)
-   {  return KC ? (uint32_t)((int64_t)(wave * 64 + lane) * ld * 4 + j * 16) : (uint32_t)((int64_t)(wave * 8 + j) * ld * 4 + lane * 16); }
+   {  if (KC) return (uint32_t)((int64_t)((wave % GROUPS) * 64 + lane) * ld * 4 + ((wave / GROUPS) * LOADS + j) * 16);
+      constexpr uint32_t LPK = 64 / KPI;
+      return (uint32_t)((int64_t)((wave * LOADS + j) * KPI + lane / LPK) * ld * 4 + (lane % LPK) * 16);
+   }
    /* ... and its first byte in the operand's LDS area (lane l writes 16 bytes at + 16 l) */
    static __device__ __forceinline__ uint32_t load_target(int j, uint32_t wave)
-   {  return KC ? (uint32_t)j * PLANE + wave * 1024 : (wave * 8 + j) * ROW; }
+   {  return KC ? ((wave / GROUPS) * LOADS + j) * PLANE + (wave % GROUPS) * 1024 : (wave * LOADS + j) * UNIT; }
    static __device__ __forceinline__ const char *slab_base(const char *mat, int64_t ld, uint32_t mn0, uint32_t k0)
    {  return mat + (KC ? ((int64_t)k0 + (int64_t)mn0 * ld) : ((int64_t)mn0 + (int64_t)k0 * ld)) * 4; }
-   /* fragment read x (0 .. 3) of quad q: the lane's part of the address, and the immediate part */
+   /* fragment read x (0 .. READS - 1) of quad q: the lane's part of the address, and the immediate part */
    static __device__ __forceinline__ uint32_t read_lane(uint32_t wbase, uint32_t lane)
    {  const uint32_t r = lane % 32, kg = lane / 32;
-      return KC ? kg * PLANE + (wbase + r) * 16 : 4 * kg * ROW + (wbase + 4 * r) * 4;
+      return KC ? kg * PLANE + (wbase + r) * 16 : kg * k_offset(4) + (wbase + TS * r) * 4;
    }
-   static constexpr uint32_t read_offset(int x, int q) { return KC ? (uint32_t)(2 * q * PLANE + x * 32 * 16) : (uint32_t)((8 * q + x) * ROW); }
-   /* the value of tile i and step t within a quad's four reads */
+   static constexpr uint32_t read_offset(int x, int q) { return KC ? (uint32_t)(2 * q * PLANE + x * 32 * 16) : k_offset(8 * q + x); }
+   /* KC: the four steps of one tile, 16 bytes; !KC: the TS tiles of one step, 4 TS bytes */
+   static __device__ __forceinline__ och_f32x4 read(const char *at)
+   {  if (KC || TS == 4) return *reinterpret_cast<const och_f32x4 *>(at);
+      const float2 v = *reinterpret_cast<const float2 *>(at);
+      return och_f32x4{v.x, v.y, 0.0f, 0.0f};
+   }
+   /* the value of tile i and step t within a quad's reads */
    static __device__ __forceinline__ float value(const och_f32x4 (&f)[4], int i, int t) { return KC ? f[i][t] : f[t][i]; }
-   /* row (of the wave's 128) of tile i, row-in-tile rr */
-   static __device__ __forceinline__ uint32_t row(int i, uint32_t rr) { return KC ? (uint32_t)i * 32 + rr : 4 * rr + (uint32_t)i; }
+   /* row (of the wave's 32 TS) of tile i, row-in-tile rr */
+   static __device__ __forceinline__ uint32_t row(int i, uint32_t rr) { return KC ? (uint32_t)i * 32 + rr : TS * rr + (uint32_t)i; }
 };
 
 /* one load from memory straight to LDS: lane l brings 16 bytes from base + offset[l] to LDS byte target + 16 l */
@@ -84,13 +100,17 @@ static __device__ __forceinline__ void load_to_lds(const char *base, uint32_t of
    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(target), "v"(offset), "s"(base) : "memory");
 }
 
-template <bool AKC, bool BKC>
-__global__ __launch_bounds__(OCH_FP_THREADS) void gemm_float_pipe_kernel(const FloatPipeParams p)
+template <bool AKC, bool BKC, int TS>
+__global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pipe_kernel(const FloatPipeParams p)
 {
-   constexpr int T = 32, BM = OCH_FP_BM, BN = OCH_FP_BM, KT = OCH_FP_KT, TMS = 4, TNS = 4, WM = 128, WN = 128, THREADS = OCH_FP_THREADS;
-   constexpr uint32_t OP = OCH_FP_OPERAND, BUF = OCH_FP_BUFFER;
-   typedef FloatSlab<AKC> LA;
-   typedef FloatSlab<BKC> LB;
+   constexpr int T = 32, BM = 64 * TS, BN = 64 * TS, KT = OCH_FP_KT, TMS = TS, TNS = TS, WM = 32 * TS, WN = 32 * TS, THREADS = OCH_FP_THREADS;
+   typedef FloatSlab<AKC, BM> LA;
+   typedef FloatSlab<BKC, BN> LB;
+   constexpr uint32_t OP = LA::OPERAND, BUF = 2 * OP;
+   constexpr int NLA = LA::LOADS, NL = 2 * NLA;            /* loads per wave and slab: of A, of both */
+   constexpr int CH = 2 * TS * TS;                         /* chunks of two MFMAs per quad */
+   constexpr int RA = LA::READS, NR = LA::READS + LB::READS; /* fragment reads per quad: of A, of both */
+   static_assert(TS == 4 || TS == 2, "wave tiles of 128 x 128 or 64 x 64");
    extern __shared__ __align__(16) char lds[];
 
    int64_t oA, oB, oC, oAlpha, oBeta;
@@ -111,9 +131,9 @@ __global__ __launch_bounds__(OCH_FP_THREADS) void gemm_float_pipe_kernel(const F
 
    const uint32_t nslabs = p.K / KT, last = nslabs - 1;
    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)lds;      /* where the array starts in LDS */
-   uint32_t offA[8], offB[8], tgtA[8], tgtB[8];
+   uint32_t offA[NLA], offB[NLA], tgtA[NLA], tgtB[NLA];
 #pragma unroll
-   for (int j = 0; j < 8; j++)
+   for (int j = 0; j < NLA; j++)
    {  offA[j] = LA::load_offset(j, wave, lane, p.ldA); offB[j] = LB::load_offset(j, wave, lane, p.ldB);
       tgtA[j] = lds0 + LA::load_target(j, wave); tgtB[j] = lds0 + OP + LB::load_target(j, wave);
    }
@@ -127,20 +147,20 @@ __global__ __launch_bounds__(OCH_FP_THREADS) void gemm_float_pipe_kernel(const F
    }
    och_f32x4 fa[2][4], fb[2][4];
 
-   /* load number e (0 .. 15; A first) of slab `slab` into buffer `buf` */
+   /* load number e (0 .. NL - 1; A's first) of a slab into buffer `buf` */
 #define OCH_LOAD(e, baseA, baseB, buf)                                                                                 \
-   do { if ((e) < 8) load_to_lds(baseA, offA[(e) % 8], tgtA[(e) % 8] + (buf) * BUF);                                   \
-        else         load_to_lds(baseB, offB[(e) % 8], tgtB[(e) % 8] + (buf) * BUF); } while (0)
-   /* one quad: chunk c reads fragment c / 4 of quad QN from buffer RB into set NXT when c is a multiple of four, issues
-      load LOAD0 + c / 4 into buffer LBUF when c % 4 == 2 and LOADS is set, then runs its two MFMAs */
+   do { if ((e) < NLA) load_to_lds(baseA, offA[(e) % NLA], tgtA[(e) % NLA] + (buf) * BUF);                             \
+        else           load_to_lds(baseB, offB[(e) % NLA], tgtB[(e) % NLA] + (buf) * BUF); } while (0)
+   /* one quad of CH chunks: chunk c issues its share of the NR fragment reads of quad QN from buffer RB into set NXT, and,
+      when LOADS is set and c % TS == TS / 2, load LOAD0 + c / TS into buffer LBUF; then it runs its two MFMAs */
 #define OCH_QUAD(CUR, NXT, RB, QN, LOADS, LOAD0, LBUF)                                                                 \
-   do { _Pragma("unroll") for (int c = 0; c < 32; c++)                                                                \
-        {  if (c % 4 == 0)                                                                                             \
-           {  if (c / 4 < 4) fa[NXT][c / 4 % 4] = *reinterpret_cast<const och_f32x4 *>(readA[RB] + LA::read_offset(c / 4 % 4, QN)); \
-              else           fb[NXT][c / 4 % 4] = *reinterpret_cast<const och_f32x4 *>(readB[RB] + LB::read_offset(c / 4 % 4, QN)); \
+   do { _Pragma("unroll") for (int c = 0; c < CH; c++)                                                                \
+        {  _Pragma("unroll") for (int f = c * NR / CH; f < (c + 1) * NR / CH; f++)                                     \
+           {  if (f < RA) fa[NXT][f < RA ? f : 0] = LA::read(readA[RB] + LA::read_offset(f < RA ? f : 0, QN));         \
+              else        fb[NXT][f >= RA ? f - RA : 0] = LB::read(readB[RB] + LB::read_offset(f >= RA ? f - RA : 0, QN)); \
            }                                                                                                           \
-           if (LOADS && c % 4 == 2) OCH_LOAD(LOAD0 + c / 4, nextA, nextB, LBUF);                                       \
-           {  const int st = c / 8, m = (c % 8) * 2, i = m / TNS, j = m % TNS;                                         \
+           if (LOADS && c % TS == TS / 2) OCH_LOAD(LOAD0 + c / TS, nextA, nextB, LBUF);                                \
+           {  const int st = c / (CH / 4), m = (c % (CH / 4)) * 2, i = m / TNS, j = m % TNS;                           \
               acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(LA::value(fa[CUR], i, st), LB::value(fb[CUR], j, st), acc[i][j], 0, 0, 0); \
               acc[i][j + 1] = __builtin_amdgcn_mfma_f32_32x32x2f32(LA::value(fa[CUR], i, st), LB::value(fb[CUR], j + 1, st), acc[i][j + 1], 0, 0, 0); \
            }                                                                                                           \
@@ -151,7 +171,7 @@ __global__ __launch_bounds__(OCH_FP_THREADS) void gemm_float_pipe_kernel(const F
 #define OCH_SLAB(s, CB)                                                                                                \
    do { {  const uint32_t s1 = ((s) + 1 < last) ? (s) + 1 : last;                                                      \
            const char *nextA = LA::slab_base(pA, p.ldA, m0, s1 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, s1 * KT);  \
-           OCH_QUAD(0, 1, CB, 1, true, 8, 1 - CB);                                                                     \
+           OCH_QUAD(0, 1, CB, 1, true, NL / 2, 1 - CB);                                                                     \
         }                                                                                                              \
         {  const char *nextA = nullptr, *nextB = nullptr;                                                              \
            OCH_QUAD(1, 0, CB, 2, false, 0, 0);                                                                         \
@@ -168,17 +188,16 @@ __global__ __launch_bounds__(OCH_FP_THREADS) void gemm_float_pipe_kernel(const F
       const uint32_t s1 = (1 < last) ? 1 : last;
       const char *nextA = LA::slab_base(pA, p.ldA, m0, 0), *nextB = LB::slab_base(pB, p.ldB, n0, 0);
 #pragma unroll
-      for (int e = 0; e < 16; e++) OCH_LOAD(e, nextA, nextB, 0);
+      for (int e = 0; e < NL; e++) OCH_LOAD(e, nextA, nextB, 0);
       nextA = LA::slab_base(pA, p.ldA, m0, s1 * KT); nextB = LB::slab_base(pB, p.ldB, n0, s1 * KT);
 #pragma unroll
-      for (int e = 0; e < 8; e++) OCH_LOAD(e, nextA, nextB, 1);
-      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      for (int e = 0; e < NL / 2; e++) OCH_LOAD(e, nextA, nextB, 1);
+      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NL / 2) : "memory");
       __syncthreads();
 #pragma unroll
-      for (int x = 0; x < 4; x++)
-      {  fa[0][x] = *reinterpret_cast<const och_f32x4 *>(readA[0] + LA::read_offset(x, 0));
-         fb[0][x] = *reinterpret_cast<const och_f32x4 *>(readB[0] + LB::read_offset(x, 0));
-      }
+      for (int x = 0; x < LA::READS; x++) fa[0][x] = LA::read(readA[0] + LA::read_offset(x, 0));
+#pragma unroll
+      for (int x = 0; x < LB::READS; x++) fb[0][x] = LB::read(readB[0] + LB::read_offset(x, 0));
    }
    uint32_t s = 0;
    for (; s + 1 < nslabs; s += 2)
@@ -226,10 +245,10 @@ __global__ __launch_bounds__(OCH_FP_THREADS) void gemm_float_pipe_kernel(const F
    }
 }
 
-/* 0: launched; 1: not a case for this kernel (the caller's other kernels take it) */
-int gemm_float_pipe(const GemmArgs &g)
+/* 0: launched; 1: not a case for this kernel (the caller's other kernels take it). tile: 256 or 128. */
+int gemm_float_pipe(const GemmArgs &g, int tile)
 {
-   if (g.M % OCH_FP_BM != 0 || g.N % OCH_FP_BM != 0 || g.K % OCH_FP_KT != 0 || g.K == 0 || !gemm_operands_aligned(g, 4)) return 1;
+   if (g.M % tile != 0 || g.N % tile != 0 || g.K % OCH_FP_KT != 0 || g.K == 0 || !gemm_operands_aligned(g, 4)) return 1;
    /* a lane's offset within a slab (up to 255 columns further on) is kept in 32 bits */
    if ((int64_t)g.ldA * 4 >= (1 << 24) || (int64_t)g.ldB * 4 >= (1 << 24)) return 1;
    FloatPipeParams p;
@@ -240,20 +259,23 @@ int gemm_float_pipe(const GemmArgs &g)
    if (g.scalar_mode_host) { memcpy(&p.alpha, g.alpha, 4); memcpy(&p.beta, g.beta, 4); }
    else { p.alpha_dev = (const float *)g.alpha; p.beta_dev = (const float *)g.beta; }
    p.batch = g.batch;
-   p.tiles_m = (uint32_t)(g.M / OCH_FP_BM); p.tiles_n = (uint32_t)(g.N / OCH_FP_BM);
+   p.tiles_m = (uint32_t)(g.M / tile); p.tiles_n = (uint32_t)(g.N / tile);
    const uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
    if (blocks > 0x7FFFFFFFull) return set_error("gemm: too many tiles");
    const bool akc = (g.transA != 'N'), bkc = (g.transB == 'N');
    const dim3 grid((unsigned)blocks, 1, g.nz), block(OCH_FP_THREADS);
-   const size_t lds = 2 * (size_t)OCH_FP_BUFFER;
-#define OCH_FP_LAUNCH(AK, BK)                                                                                         \
-   do { auto kernel = gemm_float_pipe_kernel<AK, BK>;                                                                 \
+#define OCH_FP_LAUNCH(AK, BK, TS)                                                                                     \
+   do { auto kernel = gemm_float_pipe_kernel<AK, BK, TS>;                                                             \
+        const size_t lds = 4 * (size_t)FloatSlab<AK, 64 * TS>::OPERAND;                                               \
         OCH_CHECK_HIP(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
         hipLaunchKernelGGL(kernel, grid, block, lds, g.stream, p); } while (0)
-   if (!akc && !bkc) OCH_FP_LAUNCH(false, false);
-   else if (!akc)    OCH_FP_LAUNCH(false, true);
-   else if (!bkc)    OCH_FP_LAUNCH(true, false);
-   else              OCH_FP_LAUNCH(true, true);
+#define OCH_FP_PICK(AK, BK) do { if (tile == 256) OCH_FP_LAUNCH(AK, BK, 4); else OCH_FP_LAUNCH(AK, BK, 2); } while (0)
+   if (tile != 256 && tile != 128) return 1;
+   if (!akc && !bkc) OCH_FP_PICK(false, false);
+   else if (!akc)    OCH_FP_PICK(false, true);
+   else if (!bkc)    OCH_FP_PICK(true, false);
+   else              OCH_FP_PICK(true, true);
+#undef OCH_FP_PICK
 #undef OCH_FP_LAUNCH
    OCH_CHECK_LAUNCH();
    return 0;

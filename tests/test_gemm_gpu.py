@@ -231,6 +231,9 @@ def test_gemm_float_pipelined_whole_tiles(hip, stream, ta, tb):
     rng = np.random.default_rng(1300 + ord(ta) + 2 * ord(tb))
     check_large_product(stream, H.FLOAT, ta, tb, 4096, 4096, ((1, 1, 0, False), (3, 2, -1, True)), rng)
     check_large_product(stream, H.FLOAT, ta, tb, 4096, 4096, ((6, -1.5, 0.5, False),), rng, pad=12)
+    # fewer than one 256 x 256 tile per compute unit: the same kernel on 128 x 128 tiles, two blocks per compute unit
+    check_large_product(stream, H.FLOAT, ta, tb, 2048, 2048, ((1, 1, 0, False), (3, 2, -1, True), (6, -1.5, 0.5, False)), rng)
+    check_large_product(stream, H.FLOAT, ta, tb, 2048 + 40, 2048 + 24, ((2, 0.5, 2, False),), rng, pad=4)
 
 
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T"), ("C", "N"), ("N", "C"), ("C", "C"), ("T", "C")])
