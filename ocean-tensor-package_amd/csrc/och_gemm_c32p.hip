@@ -1,4 +1,4 @@
-/* complex float GEMM for whole aligned 128 x 128 tiles: C <- alpha * op(A) * op(B) + beta * C, column-major, op = none,
+/* complex float GEMM on tiles of 128 x 128 for aligned operands with M and N multiples of 2 and K of 32: C <- alpha * op(A) * op(B) + beta * C, column-major, op = none,
  * transposition or conjugate transposition.
  *
  * The counterpart of cublasCgemm in the reference (src/core/gpu/op/tensor_blas_gpu.c:183-197). The float kernel
@@ -55,8 +55,19 @@ struct CFloatSlab
    static_assert(16 * PLANE <= OCH_CP_OPERAND && 32 * ROWP <= OCH_CP_OPERAND, "slab does not fit");
    /* load j (0 .. 7) of wave w: byte offset in memory relative to the slab's first element, per lane. KC: chunk
       (w / 2) * 8 + j of the 64 rows of group w % 2; !KC: k = 8 w + j */
-   static __device__ __forceinline__ uint32_t load_offset(int j, uint32_t wave, uint32_t lane, int64_t ld)
-   {  return KC ? (uint32_t)((int64_t)((wave % 2) * 64 + lane) * ld * 8 + ((wave / 2) * 8 + j) * 16) : (uint32_t)((int64_t)(wave * 8 + j) * ld * 8 + lane * 16); }
+   /* `rows`: how many of the tile's rows exist (a multiple of 2; fewer than 128 in the last tile of a matrix whose size is
+      not a multiple of the tile). Lanes whose rows do not exist fetch the last rows that do: loads stay inside the matrix,
+      and what they bring is multiplied into rows of the tile that are never written. */
+   static __device__ __forceinline__ uint32_t load_offset(int j, uint32_t wave, uint32_t lane, int64_t ld, uint32_t rows)
+   {  if (KC)
+      {  uint32_t row = (wave % 2) * 64 + lane;
+         row = row < rows ? row : rows - 1;
+         return (uint32_t)((int64_t)row * ld * 8 + ((wave / 2) * 8 + j) * 16);
+      }
+      uint32_t row = lane * 2;
+      row = row < rows ? row : rows - 2;
+      return (uint32_t)((int64_t)(wave * 8 + j) * ld * 8 + row * 8);
+   }
    /* ... and its first byte in the operand's LDS area (lane l writes 16 bytes at + 16 l) */
    static __device__ __forceinline__ uint32_t load_target(int j, uint32_t wave)
    {  return KC ? ((wave / 2) * 8 + j) * PLANE + (wave % 2) * 1024 : (wave * 8 + j) * ROWP; }
@@ -111,10 +122,11 @@ __global__ __launch_bounds__(OCH_CP_THREADS) void gemm_cfloat_pipe_kernel(const 
 
    const uint32_t nslabs = p.K / KT, last = nslabs - 1;
    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)lds;      /* where the array starts in LDS */
+   const uint32_t rowsA = p.M - m0 < (uint32_t)BM ? p.M - m0 : (uint32_t)BM, rowsB = p.N - n0 < (uint32_t)BN ? p.N - n0 : (uint32_t)BN;    /* of this tile */
    uint32_t offA[8], offB[8], tgtA[8], tgtB[8];
 #pragma unroll
    for (int j = 0; j < 8; j++)
-   {  offA[j] = LA::load_offset(j, wave, lane, p.ldA); offB[j] = LB::load_offset(j, wave, lane, p.ldB);
+   {  offA[j] = LA::load_offset(j, wave, lane, p.ldA, rowsA); offB[j] = LB::load_offset(j, wave, lane, p.ldB, rowsB);
       tgtA[j] = lds0 + LA::load_target(j, wave); tgtB[j] = lds0 + OP + LB::load_target(j, wave);
    }
    /* the lane's read addresses in buffer 0 and buffer 1, in registers of their own (the empty asm keeps the compiler
@@ -221,6 +233,7 @@ __global__ __launch_bounds__(OCH_CP_THREADS) void gemm_cfloat_pipe_kernel(const 
       const uint32_t c0 = n0 + h * CPASS;
       for (uint32_t q = threadIdx.x; q < CPASS * (BM / 2); q += THREADS)
       {  const uint32_t c = q / (BM / 2), r2 = (q % (BM / 2)) * 2;
+         if (r2 >= rowsA || h * CPASS + c >= rowsB) continue;          /* outside C */
          och_f32x4 v = *reinterpret_cast<const och_f32x4 *>(stage + c * CP + r2);
          och_f32x4 *dst = reinterpret_cast<och_f32x4 *>(pC + ((int64_t)(m0 + r2) + (int64_t)(c0 + c) * p.ldC) * 8);
          if (br != 0 || bi != 0)
@@ -237,7 +250,7 @@ __global__ __launch_bounds__(OCH_CP_THREADS) void gemm_cfloat_pipe_kernel(const 
 /* 0: launched; 1: not a case for this kernel (the caller's other kernels take it) */
 int gemm_cfloat_pipe(const GemmArgs &g)
 {
-   if (g.M % OCH_CP_BM != 0 || g.N % OCH_CP_BM != 0 || g.K % OCH_CP_KT != 0 || g.K == 0 || !gemm_operands_aligned(g, 8)) return 1;
+   if (g.M % 2 != 0 || g.N % 2 != 0 || g.M == 0 || g.N == 0 || g.K % OCH_CP_KT != 0 || g.K == 0 || !gemm_operands_aligned(g, 8)) return 1;
    /* a lane's offset within a slab (up to 127 columns further on) is kept in 32 bits */
    if ((int64_t)g.ldA * 8 >= (1 << 24) || (int64_t)g.ldB * 8 >= (1 << 24)) return 1;
    CFloatPipeParams p;
@@ -249,7 +262,7 @@ int gemm_cfloat_pipe(const GemmArgs &g)
    else { p.alpha_dev = (const float *)g.alpha; p.beta_dev = (const float *)g.beta; }
    p.batch = g.batch;
    p.conjA = (g.transA == 'C'); p.conjB = (g.transB == 'C');
-   p.tiles_m = (uint32_t)(g.M / OCH_CP_BM); p.tiles_n = (uint32_t)(g.N / OCH_CP_BM);
+   p.tiles_m = (uint32_t)((g.M + OCH_CP_BM - 1) / OCH_CP_BM); p.tiles_n = (uint32_t)((g.N + OCH_CP_BM - 1) / OCH_CP_BM);
    const uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
    if (blocks > 0x7FFFFFFFull) return set_error("gemm: too many tiles");
    const bool akc = (g.transA != 'N'), bkc = (g.transB == 'N');

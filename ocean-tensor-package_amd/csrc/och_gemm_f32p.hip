@@ -1,4 +1,4 @@
-/* float GEMM for whole aligned 256 x 256 or 128 x 128 tiles: C <- alpha * op(A) * op(B) + beta * C, column-major.
+/* float GEMM on tiles of 256 x 256 or 128 x 128 for aligned operands with M and N multiples of 4 and K of 32: C <- alpha * op(A) * op(B) + beta * C, column-major.
  *
  * The counterpart of cublasSgemm in the reference (src/core/gpu/op/tensor_blas_gpu.c:183-197). Four waves per block,
  * one per SIMD, each owning 128 x 128 of the tile as 4 x 4 tiles of v_mfma_f32_32x32x2_f32 (256 accumulator registers);
@@ -66,10 +66,19 @@ struct FloatSlab
    static constexpr uint32_t k_offset(int k) { return (uint32_t)((k / KPI) * UNIT + (k % KPI) * ROWS * 4); }      /* !KC: where k starts */
    /* load j of wave w: byte offset in memory relative to the slab's first element, per lane. KC: chunk (w / GROUPS) * LOADS + j
       of the rows of group w % GROUPS; !KC: k = (w * LOADS + j) * KPI + lane / (64 / KPI), 16 bytes of rows per lane */
-   static __device__ __forceinline__ uint32_t load_offset(int j, uint32_t wave, uint32_t lane, int64_t ld)
-   {  if (KC) return (uint32_t)((int64_t)((wave % GROUPS) * 64 + lane) * ld * 4 + ((wave / GROUPS) * LOADS + j) * 16);
+   /* `rows`: how many of the tile's rows exist (a multiple of 4; fewer than ROWS in the last tile of a matrix whose size is
+      not a multiple of the tile). Lanes whose rows do not exist fetch the last rows that do: loads stay inside the matrix,
+      and what they bring is multiplied into rows of the tile that are never written. */
+   static __device__ __forceinline__ uint32_t load_offset(int j, uint32_t wave, uint32_t lane, int64_t ld, uint32_t rows)
+   {  if (KC)
+      {  uint32_t row = (wave % GROUPS) * 64 + lane;
+         row = row < rows ? row : rows - 1;
+         return (uint32_t)((int64_t)row * ld * 4 + ((wave / GROUPS) * LOADS + j) * 16);
+      }
       constexpr uint32_t LPK = 64 / KPI;
-      return (uint32_t)((int64_t)((wave * LOADS + j) * KPI + lane / LPK) * ld * 4 + (lane % LPK) * 16);
+      uint32_t row = (lane % LPK) * 4;
+      row = row < rows ? row : rows - 4;
+      return (uint32_t)((int64_t)((wave * LOADS + j) * KPI + lane / LPK) * ld * 4 + row * 4);
    }
    /* ... and its first byte in the operand's LDS area (lane l writes 16 bytes at + 16 l) */
    static __device__ __forceinline__ uint32_t load_target(int j, uint32_t wave)
@@ -131,10 +140,11 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pi
 
    const uint32_t nslabs = p.K / KT, last = nslabs - 1;
    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)lds;      /* where the array starts in LDS */
+   const uint32_t rowsA = p.M - m0 < (uint32_t)BM ? p.M - m0 : (uint32_t)BM, rowsB = p.N - n0 < (uint32_t)BN ? p.N - n0 : (uint32_t)BN;    /* of this tile */
    uint32_t offA[NLA], offB[NLA], tgtA[NLA], tgtB[NLA];
 #pragma unroll
    for (int j = 0; j < NLA; j++)
-   {  offA[j] = LA::load_offset(j, wave, lane, p.ldA); offB[j] = LB::load_offset(j, wave, lane, p.ldB);
+   {  offA[j] = LA::load_offset(j, wave, lane, p.ldA, rowsA); offB[j] = LB::load_offset(j, wave, lane, p.ldB, rowsB);
       tgtA[j] = lds0 + LA::load_target(j, wave); tgtB[j] = lds0 + OP + LB::load_target(j, wave);
    }
    /* the lane's read addresses in buffer 0 and buffer 1, in registers of their own (the empty asm keeps the compiler
@@ -236,6 +246,7 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pi
       const uint32_t c0 = n0 + h * CPASS;
       for (uint32_t q = threadIdx.x; q < CPASS * (BM / 4); q += THREADS)
       {  const uint32_t c = q / (BM / 4), r4 = (q % (BM / 4)) * 4;
+         if (r4 >= rowsA || h * CPASS + c >= rowsB) continue;          /* outside C */
          och_f32x4 v = *reinterpret_cast<const och_f32x4 *>(stage + c * CP + r4);
          och_f32x4 *dst = reinterpret_cast<och_f32x4 *>(pC + ((int64_t)(m0 + r4) + (int64_t)(c0 + c) * p.ldC) * 4);
          if (beta != 0) { const och_f32x4 old = *dst; v.x += beta * old.x; v.y += beta * old.y; v.z += beta * old.z; v.w += beta * old.w; }
@@ -245,10 +256,11 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pi
    }
 }
 
-/* 0: launched; 1: not a case for this kernel (the caller's other kernels take it). tile: 256 or 128. */
+/* 0: launched; 1: not a case for this kernel (the caller's other kernels take it). tile: 256 or 128; M and N multiples
+   of 4, K of 32, operands aligned to 16 bytes. */
 int gemm_float_pipe(const GemmArgs &g, int tile)
 {
-   if (g.M % tile != 0 || g.N % tile != 0 || g.K % OCH_FP_KT != 0 || g.K == 0 || !gemm_operands_aligned(g, 4)) return 1;
+   if (g.M % 4 != 0 || g.N % 4 != 0 || g.M == 0 || g.N == 0 || g.K % OCH_FP_KT != 0 || g.K == 0 || !gemm_operands_aligned(g, 4)) return 1;
    /* a lane's offset within a slab (up to 255 columns further on) is kept in 32 bits */
    if ((int64_t)g.ldA * 4 >= (1 << 24) || (int64_t)g.ldB * 4 >= (1 << 24)) return 1;
    FloatPipeParams p;
@@ -259,7 +271,7 @@ int gemm_float_pipe(const GemmArgs &g, int tile)
    if (g.scalar_mode_host) { memcpy(&p.alpha, g.alpha, 4); memcpy(&p.beta, g.beta, 4); }
    else { p.alpha_dev = (const float *)g.alpha; p.beta_dev = (const float *)g.beta; }
    p.batch = g.batch;
-   p.tiles_m = (uint32_t)(g.M / tile); p.tiles_n = (uint32_t)(g.N / tile);
+   p.tiles_m = (uint32_t)((g.M + tile - 1) / tile); p.tiles_n = (uint32_t)((g.N + tile - 1) / tile);
    const uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
    if (blocks > 0x7FFFFFFFull) return set_error("gemm: too many tiles");
    const bool akc = (g.transA != 'N'), bkc = (g.transB == 'N');

@@ -6,32 +6,28 @@ namespace och {
 int gemm_double(const GemmArgs &g)
 {  static const GemmTileChoice choice[4] = { { 128, 128, 1.0 }, { 128, 64, 0.96 }, { 64, 128, 0.96 }, { 64, 64, 0.92 } };
    const int pick = gemm_pick_tile(g, choice, 4);
-   /* Large aligned products with K a multiple of 16: the whole 256 x 128 tiles run on the pipelined kernel, the strip of
-      columns to their right and the strip of rows below them as products of their own -- when that is cheaper by the model
-      of gemm_pick_tile (rounds of the compute units x tile area / efficiency, the kernels below at 0.87 of the pipelined one) */
-   if (g.M >= 256 && g.N >= 128 && g.K >= 16 && g.K % 16 == 0 && gemm_operands_aligned(g, 8))
+   /* Aligned products with M and N multiples of 2 and K of 16 run on the pipelined kernel on tiles of 256 x 128 when
+      that is cheaper by the model of gemm_pick_tile (rounds of the compute units x tile area / efficiency, the kernels
+      below at 0.87 of the pipelined one). A K that is not a multiple of 16 (scalars in host memory only): the whole
+      slabs there, the rest of K as a product of its own that adds to C. */
+   if (g.M >= 256 / 2 && g.N >= 128 / 2 && g.M % 2 == 0 && g.N % 2 == 0 && g.K >= 16 && (g.K % 16 == 0 || (g.scalar_mode_host && g.K >= 128)) && gemm_operands_aligned(g, 8))
    {  const uint64_t units = (uint64_t)gemm_compute_units();
-      auto cost = [&](uint64_t bm, uint64_t bn, double efficiency, bool whole)
-      {  const uint64_t tiles = (whole ? (g.M / bm) * (g.N / bn) : ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn)) * (uint64_t)g.nz;
+      auto cost = [&](uint64_t bm, uint64_t bn, double efficiency)
+      {  const uint64_t tiles = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * (uint64_t)g.nz;
          return (double)((tiles + units - 1) / units) * (double)(bm * bn) / efficiency;
       };
-      if (cost(256, 128, 1.0, true) < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87, false))
-      {  const size_t Mi = g.M - g.M % 256, Ni = g.N - g.N % 128;
-         GemmArgs part = g;
-         part.M = Mi; part.N = Ni;
+      if (cost(256, 128, 1.0) < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87))
+      {  GemmArgs part = g;
+         const size_t Kh = g.K - g.K % 16;
+         part.K = Kh;
          const int taken = gemm_double_pipe(part);
          if (taken < 0) return taken;
          if (taken == 0)
-         {  if (g.N > Ni)
-            {  part = g; part.N = g.N - Ni;
-               part.B = (const char *)g.B + (int64_t)Ni * (g.transB == 'N' ? (int64_t)g.ldB : 1) * 8;
-               part.C = (char *)g.C + (int64_t)Ni * g.ldC * 8;
-               if (gemm_double(part) != 0) return -1;
-            }
-            if (g.M > Mi)
-            {  part = g; part.M = g.M - Mi; part.N = Ni;
-               part.A = (const char *)g.A + (int64_t)Mi * (g.transA == 'N' ? 1 : (int64_t)g.ldA) * 8;
-               part.C = (char *)g.C + (int64_t)Mi * 8;
+         {  if (g.K > Kh)
+            {  static const double one = 1.0;
+               part.K = g.K - Kh; part.beta = &one;
+               part.A = (const char *)g.A + (int64_t)Kh * (g.transA == 'N' ? (int64_t)g.ldA : 1) * 8;
+               part.B = (const char *)g.B + (int64_t)Kh * (g.transB == 'N' ? 1 : (int64_t)g.ldB) * 8;
                if (gemm_double(part) != 0) return -1;
             }
             return 0;

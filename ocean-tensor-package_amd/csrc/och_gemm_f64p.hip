@@ -1,4 +1,4 @@
-/* double GEMM for whole aligned 256 x 128 tiles: C <- alpha * op(A) * op(B) + beta * C, column-major.
+/* double GEMM on tiles of 256 x 128 for aligned operands with M and N multiples of 2 and K of 16: C <- alpha * op(A) * op(B) + beta * C, column-major.
  *
  * The counterpart of cublasDgemm in the reference (src/core/gpu/op/tensor_blas_gpu.c:183-197). Four waves per block,
  * one per SIMD, each owning 128 x 64 of the tile as 8 x 4 tiles of v_mfma_f64_16x16x4_f64 (256 accumulator registers).
@@ -64,10 +64,19 @@ struct DoubleSlab
    static constexpr int GROUPS = ROWS / 64, PARTS = ROWS / 128;
    /* load j of wave w. KC: chunk (w / GROUPS) * LOADS + j of the 64 rows of group w % GROUPS; !KC: unit u = w * LOADS + j
       is part u % PARTS (128 rows) of k = u / PARTS */
-   static __device__ __forceinline__ uint32_t load_offset(int j, uint32_t wave, uint32_t lane, int64_t ld)
-   {  if (KC) return (uint32_t)((int64_t)((wave % GROUPS) * 64 + lane) * ld * 8 + ((wave / GROUPS) * LOADS + j) * 16);
+   /* `rows`: how many of the tile's rows exist (a multiple of 2; fewer than ROWS in the last tile of a matrix whose size is
+      not a multiple of the tile). Lanes whose rows do not exist fetch the last rows that do: loads stay inside the matrix,
+      and what they bring is multiplied into rows of the tile that are never written. */
+   static __device__ __forceinline__ uint32_t load_offset(int j, uint32_t wave, uint32_t lane, int64_t ld, uint32_t rows)
+   {  if (KC)
+      {  uint32_t row = (wave % GROUPS) * 64 + lane;
+         row = row < rows ? row : rows - 1;
+         return (uint32_t)((int64_t)row * ld * 8 + ((wave / GROUPS) * LOADS + j) * 16);
+      }
       const uint32_t u = wave * LOADS + j;
-      return (uint32_t)((int64_t)(u / PARTS) * ld * 8 + (u % PARTS) * 1024 + lane * 16);
+      uint32_t row = (u % PARTS) * 128 + lane * 2;
+      row = row < rows ? row : rows - 2;
+      return (uint32_t)((int64_t)(u / PARTS) * ld * 8 + row * 8);
    }
    static __device__ __forceinline__ uint32_t load_target(int j, uint32_t wave)
    {  if (KC) return ((wave / GROUPS) * LOADS + j) * PLANE + (wave % GROUPS) * 1024;
@@ -150,11 +159,12 @@ __global__ __launch_bounds__(OCH_DP_THREADS) void gemm_double_pipe_kernel(const 
 
    const uint32_t nslabs = p.K / KT, last = nslabs - 1;
    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)lds;      /* where the array starts in LDS */
+   const uint32_t rowsA = p.M - m0 < (uint32_t)BM ? p.M - m0 : (uint32_t)BM, rowsB = p.N - n0 < (uint32_t)BN ? p.N - n0 : (uint32_t)BN;    /* of this tile */
    uint32_t offA[8], offB[4], tgtA[8], tgtB[4];
 #pragma unroll
-   for (int j = 0; j < 8; j++) { offA[j] = LA::load_offset(j, wave, lane, p.ldA); tgtA[j] = lds0 + LA::load_target(j, wave); }
+   for (int j = 0; j < 8; j++) { offA[j] = LA::load_offset(j, wave, lane, p.ldA, rowsA); tgtA[j] = lds0 + LA::load_target(j, wave); }
 #pragma unroll
-   for (int j = 0; j < 4; j++) { offB[j] = LB::load_offset(j, wave, lane, p.ldB); tgtB[j] = lds0 + OPA + LB::load_target(j, wave); }
+   for (int j = 0; j < 4; j++) { offB[j] = LB::load_offset(j, wave, lane, p.ldB, rowsB); tgtB[j] = lds0 + OPA + LB::load_target(j, wave); }
    /* the lane's read addresses in the three buffers, in registers of their own (the empty asm keeps the compiler from
       deriving one from the other with an addition at every read: the distance is beyond a read's immediate) */
    uint32_t readA[3], readB[3];
@@ -257,6 +267,7 @@ __global__ __launch_bounds__(OCH_DP_THREADS) void gemm_double_pipe_kernel(const 
       const uint32_t c0 = n0 + h * CPASS;
       for (uint32_t q = threadIdx.x; q < CPASS * (BM / 2); q += THREADS)
       {  const uint32_t c = q / (BM / 2), r2 = (q % (BM / 2)) * 2;
+         if (r2 >= rowsA || h * CPASS + c >= rowsB) continue;          /* outside C */
          och_f64x2 v = *reinterpret_cast<const och_f64x2 *>(stage + c * CP + r2);
          och_f64x2 *dst = reinterpret_cast<och_f64x2 *>(pC + ((int64_t)(m0 + r2) + (int64_t)(c0 + c) * p.ldC) * 8);
          if (beta != 0) { const och_f64x2 old = *dst; v.x += beta * old.x; v.y += beta * old.y; }
@@ -266,10 +277,11 @@ __global__ __launch_bounds__(OCH_DP_THREADS) void gemm_double_pipe_kernel(const 
    }
 }
 
-/* 0: launched; 1: not a case for this kernel (the caller's other kernels take it) */
+/* 0: launched; 1: not a case for this kernel (the caller's other kernels take it): M and N multiples of 2, K of 16,
+   operands aligned to 16 bytes */
 int gemm_double_pipe(const GemmArgs &g)
 {
-   if (g.M % OCH_DP_BM != 0 || g.N % OCH_DP_BN != 0 || g.K % OCH_DP_KT != 0 || g.K == 0 || !gemm_operands_aligned(g, 8)) return 1;
+   if (g.M % 2 != 0 || g.N % 2 != 0 || g.M == 0 || g.N == 0 || g.K % OCH_DP_KT != 0 || g.K == 0 || !gemm_operands_aligned(g, 8)) return 1;
    /* a lane's offset within a slab (up to 255 columns further on) is kept in 32 bits */
    if ((int64_t)g.ldA * 8 >= (1 << 24) || (int64_t)g.ldB * 8 >= (1 << 24)) return 1;
    DoublePipeParams p;
@@ -280,7 +292,7 @@ int gemm_double_pipe(const GemmArgs &g)
    if (g.scalar_mode_host) { memcpy(&p.alpha, g.alpha, 8); memcpy(&p.beta, g.beta, 8); }
    else { p.alpha_dev = (const double *)g.alpha; p.beta_dev = (const double *)g.beta; }
    p.batch = g.batch;
-   p.tiles_m = (uint32_t)(g.M / OCH_DP_BM); p.tiles_n = (uint32_t)(g.N / OCH_DP_BN);
+   p.tiles_m = (uint32_t)((g.M + OCH_DP_BM - 1) / OCH_DP_BM); p.tiles_n = (uint32_t)((g.N + OCH_DP_BN - 1) / OCH_DP_BN);
    const uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
    if (blocks > 0x7FFFFFFFull) return set_error("gemm: too many tiles");
    const bool akc = (g.transA != 'N'), bkc = (g.transB == 'N');

@@ -176,7 +176,7 @@ def check_large_product(stream, dtype, ta, tb, M, N, cases, rng, pad=0):
     kt = {H.HALF: 64, H.FLOAT: 32, H.DOUBLE: 16, H.CFLOAT: 32}.get(dtype, 128)
     exact = dtype not in (H.HALF, H.FLOAT, H.DOUBLE, H.CFLOAT)
     for slabs, alpha, beta, dev in cases:
-        K = slabs * kt
+        K = int(round(slabs * kt))
         rowsA, colsA = (M, K) if ta == "N" else (K, M)
         rowsB, colsB = (K, N) if tb == "N" else (N, K)
         ldA, ldB, ldC = rowsA + pad, rowsB + pad, M + pad
@@ -234,6 +234,11 @@ def test_gemm_float_pipelined_whole_tiles(hip, stream, ta, tb):
     # fewer than one 256 x 256 tile per compute unit: the same kernel on 128 x 128 tiles, two blocks per compute unit
     check_large_product(stream, H.FLOAT, ta, tb, 2048, 2048, ((1, 1, 0, False), (3, 2, -1, True), (6, -1.5, 0.5, False)), rng)
     check_large_product(stream, H.FLOAT, ta, tb, 2048 + 40, 2048 + 24, ((2, 0.5, 2, False),), rng, pad=4)
+    # last tiles of four rows / four columns (the tile's loads are clamped to the rows that exist, the rest of the tile is not written)
+    check_large_product(stream, H.FLOAT, ta, tb, 2564, 2560, ((2, 1, -1, False),), rng)
+    check_large_product(stream, H.FLOAT, ta, tb, 2560, 2564, ((2, 1, 0, False),), rng, pad=8)
+    # K that is not a whole number of slabs (scalars in host memory): the whole slabs pipelined, the rest added by a product of its own
+    check_large_product(stream, H.FLOAT, ta, tb, 2048, 2048 + 24, ((9.25, 0.5, 2, False), (9.25, 0.5, 2, True)), rng)
 
 
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T"), ("C", "N"), ("N", "C"), ("C", "C"), ("T", "C")])
@@ -244,6 +249,8 @@ def test_gemm_cfloat_pipelined_whole_tiles(hip, stream, ta, tb):
     rng = np.random.default_rng(1500 + ord(ta) + 2 * ord(tb))
     check_large_product(stream, H.CFLOAT, ta, tb, 2048, 2048, ((1, 1, 0, False), (3, 2 - 1j, -1 + 0.5j, True)), rng)
     check_large_product(stream, H.CFLOAT, ta, tb, 2048, 2048, ((6, -1.5j, 0.5, False),), rng, pad=6)
+    check_large_product(stream, H.CFLOAT, ta, tb, 2048, 2048, ((8.125, 1 - 1j, 0.5j, False),), rng)            # a K of 8 slabs + 4
+    check_large_product(stream, H.CFLOAT, ta, tb, 4098, 4098, ((2, 1, -1, False),), rng)                        # last tiles of two rows / columns
 
 
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
@@ -255,6 +262,8 @@ def test_gemm_double_pipelined_whole_tiles(hip, stream, ta, tb):
     rng = np.random.default_rng(1400 + ord(ta) + 2 * ord(tb))
     check_large_product(stream, H.DOUBLE, ta, tb, 4096, 2048, ((1, 1, 0, False), (2, 2, -1, True), (3, -1, 1, False)), rng)
     check_large_product(stream, H.DOUBLE, ta, tb, 4096, 2048, ((4, 1.5, 0, True), (8, -1.5, 0.5, False)), rng, pad=6)
+    check_large_product(stream, H.DOUBLE, ta, tb, 4096, 2048, ((9.3125, 2, -1, False),), rng)                    # a K of 9 slabs + 5
+    check_large_product(stream, H.DOUBLE, ta, tb, 7938, 7938, ((2, 1, -1, False),), rng)                         # last tiles of two rows / columns
 
 
 @pytest.mark.parametrize("dtype", [H.HALF, H.INT8, H.UINT8], ids=lambda d: H.NAMES[d])
