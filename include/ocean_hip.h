@@ -391,6 +391,13 @@ int och_gemm_batched(int dtype, char transA, char transB, size_t M, size_t N, si
                      const ptrdiff_t *stride_beta, const ptrdiff_t *strideC,
                      int scalar_mode_host, och_stream stream);
 
+/* Which kernel large aligned float / double / complex-float products take is decided by a cost model (rounds of the   */
+/* compute units x tile area / efficiency). For tests and measurements the decision can be fixed: 0 the model decides */
+/* (default), 1 the pipelined kernel on its large tile wherever its conditions hold (M, N multiples of 4 or 2, K of   */
+/* the slab, 16-byte aligned operands), 2 the pipelined kernel on its small tile (float, double; complex float has    */
+/* one tile), 3 never the pipelined kernel. Process-wide; no counterpart in the reference.                            */
+int och_gemm_set_kernel_choice(int choice);
+
 /* Fused projection step of a modified Gram-Schmidt sweep. No counterpart in the reference, whose callers issue one    */
 /* dot product (gemm with M = N = 1) and one rank-1 update per pair of columns, i.e. 2 k launches for this:             */
 /*    for i = 0 .. k-1 (in this order):  r[i] = q_i^H v;   v <- v - r[i] q_i                                            */

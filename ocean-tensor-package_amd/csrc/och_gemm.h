@@ -559,6 +559,7 @@ static int launch_gemm_mfma(const GemmArgs &g)
 
 /* Compute units of the current device (cached per device). */
 int gemm_compute_units(void);
+int gemm_kernel_choice(void);            /* 0 automatic; 1 / 2: pipelined kernel, large / small tile; 3: never pipelined */
 
 /* Which block tile to use. The compute units work through the tiles in rounds, and the last round is as long as the others
    however few tiles it holds: 3000^3 double is 576 tiles of 128 x 128, i.e. 2.25 rounds on 256 units, and ran at 39
@@ -591,7 +592,7 @@ static inline bool gemm_operands_aligned(const GemmArgs &g, int es)
 int gemm_float(const GemmArgs &g);
 int gemm_float_pipe(const GemmArgs &g, int tile); /* whole aligned tiles of 256 x 256 or 128 x 128; 1: not taken */
 int gemm_double(const GemmArgs &g);
-int gemm_double_pipe(const GemmArgs &g); /* whole aligned 256 x 128 tiles; 1: not taken */
+int gemm_double_pipe(const GemmArgs &g, int tile_m); /* tiles of 256 x 128 or 128 x 128; 1: not taken */
 int gemm_cfloat(const GemmArgs &g);
 int gemm_cfloat_pipe(const GemmArgs &g); /* whole aligned 128 x 128 tiles; 1: not taken */
 int gemm_cdouble(const GemmArgs &g);

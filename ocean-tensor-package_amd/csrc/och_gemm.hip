@@ -116,6 +116,11 @@ template <class T> static int gemm_generic(const GemmArgs &g)
    return 0;
 }
 
+/* 0: the cost model chooses; 1: the pipelined kernel on its large tile wherever it applies; 2: on its small tile (float,
+   double); 3: never the pipelined kernel. For tests and measurements (och_gemm_set_kernel_choice). */
+static int g_gemm_kernel_choice = 0;
+int gemm_kernel_choice(void) { return g_gemm_kernel_choice; }
+
 int gemm_compute_units(void)
 {  static int cached[64];
    int device = 0;
@@ -244,5 +249,12 @@ extern "C" int och_gemm_batched(int dtype, char transA, char transB, size_t M, s
    {  b.z0 = (uint32_t)z0; g.nz = (unsigned)((total - z0 < 65535) ? total - z0 : 65535);
       if (gemm_dispatch(dtype, g) != 0) return -1;
    }
+   return 0;
+}
+
+extern "C" int och_gemm_set_kernel_choice(int choice)
+{
+   if (choice < 0 || choice > 3) return och::set_error("gemm: kernel choice %d (0 automatic, 1 pipelined large tile, 2 pipelined small tile, 3 tiled kernel)", choice);
+   och::g_gemm_kernel_choice = choice;
    return 0;
 }

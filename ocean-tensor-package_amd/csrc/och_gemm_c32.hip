@@ -14,7 +14,8 @@ int gemm_cfloat(const GemmArgs &g)
       {  const uint64_t tiles = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * (uint64_t)g.nz;
          return (double)((tiles + units - 1) / units) * (double)(bm * bn) / efficiency;
       };
-      if (cost(128, 128, 1.0) < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87))
+      const int forced = gemm_kernel_choice();
+      if (forced != 3 && (forced != 0 || cost(128, 128, 1.0) < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87)))
       {  GemmArgs part = g;
          const size_t Kh = g.K - g.K % 32;
          part.K = Kh;

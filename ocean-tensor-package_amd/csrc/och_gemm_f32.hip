@@ -19,8 +19,9 @@ int gemm_float(const GemmArgs &g)
       };
       const double others = cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.85);
       const double large = cost(256, 256, 1.0), small = cost(128, 128, 0.9);
-      const int tile = large <= small ? 256 : 128;
-      if ((tile == 256 ? large : small) < others)
+      const int forced = gemm_kernel_choice();
+      const int tile = forced == 1 ? 256 : (forced == 2 ? 128 : (large <= small ? 256 : 128));
+      if (forced != 3 && (forced != 0 || (tile == 256 ? large : small) < others))
       {  GemmArgs part = g;
          const size_t Kh = g.K - g.K % 32;
          part.K = Kh;

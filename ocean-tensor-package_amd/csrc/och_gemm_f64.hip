@@ -6,7 +6,7 @@ namespace och {
 int gemm_double(const GemmArgs &g)
 {  static const GemmTileChoice choice[4] = { { 128, 128, 1.0 }, { 128, 64, 0.96 }, { 64, 128, 0.96 }, { 64, 64, 0.92 } };
    const int pick = gemm_pick_tile(g, choice, 4);
-   /* Aligned products with M and N multiples of 2 and K of 16 run on the pipelined kernel on tiles of 256 x 128 when
+   /* Aligned products with M and N multiples of 2 and K of 16 run on the pipelined kernel on tiles of 256 x 128 or 128 x 128 (at 0.9) when
       that is cheaper by the model of gemm_pick_tile (rounds of the compute units x tile area / efficiency, the kernels
       below at 0.87 of the pipelined one). A K that is not a multiple of 16 (scalars in host memory only): the whole
       slabs there, the rest of K as a product of its own that adds to C. */
@@ -16,11 +16,14 @@ int gemm_double(const GemmArgs &g)
       {  const uint64_t tiles = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * (uint64_t)g.nz;
          return (double)((tiles + units - 1) / units) * (double)(bm * bn) / efficiency;
       };
-      if (cost(256, 128, 1.0) < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87))
+      const double large = cost(256, 128, 1.0), small = cost(128, 128, 0.9);
+      const int forced = gemm_kernel_choice();
+      const int tile_m = forced == 1 ? 256 : (forced == 2 ? 128 : (large <= small ? 256 : 128));
+      if (forced != 3 && (forced != 0 || (tile_m == 256 ? large : small) < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87)))
       {  GemmArgs part = g;
          const size_t Kh = g.K - g.K % 16;
          part.K = Kh;
-         const int taken = gemm_double_pipe(part);
+         const int taken = gemm_double_pipe(part, tile_m);
          if (taken < 0) return taken;
          if (taken == 0)
          {  if (g.K > Kh)

@@ -126,6 +126,10 @@ static __device__ __forceinline__ void acc_zero()
 {
    asm volatile(".set och_acc, 0\n\t.rept 256\n\tv_accvgpr_write_b32 a[och_acc], 0\n\t.set och_acc, och_acc + 1\n\t.endr" : : : "a255");
 }
+static __device__ __forceinline__ void acc_zero_half()                                 /* the 16 tiles of the small kernel */
+{
+   asm volatile(".set och_acc, 0\n\t.rept 128\n\tv_accvgpr_write_b32 a[och_acc], 0\n\t.set och_acc, och_acc + 1\n\t.endr" : : : "a127");
+}
 static __device__ __forceinline__ void mfma_f64(int tile, double a, double b)         /* tile += a b */
 {
    asm volatile("v_mfma_f64_16x16x4_f64 a[%2:%2+7], %0, %1, a[%2:%2+7]" : : "v"(a), "v"(b), "i"(8 * tile));
@@ -277,9 +281,142 @@ __global__ __launch_bounds__(OCH_DP_THREADS) void gemm_double_pipe_kernel(const 
    }
 }
 
+/* The same on tiles of 128 x 128 for products with too few tiles of 256 x 128: four waves of 64 x 64 (4 x 4 tiles, 128
+   accumulation registers), two slab buffers of 34 KB, so that two blocks share a compute unit and fill each other's
+   waits. Slab s in buffer s % 2: its first pair carries the second half of the 8 loads of slab s + 1 (into the other
+   buffer), the barrier behind a wait for all loads stands in front of its second pair, which reads the first fragments
+   of slab s + 1 and carries the first half of the loads of slab s + 2 (into this buffer). */
+template <bool AKC, bool BKC>
+__global__ __launch_bounds__(OCH_DP_THREADS, 2) void gemm_double_pipe_small_kernel(const DoublePipeParams p)
+{
+   constexpr int T = 16, BM = 128, BN = 128, KT = OCH_DP_KT, TMS = 4, TNS = 4, WM = 64, WN = 64, THREADS = OCH_DP_THREADS;
+   constexpr uint32_t OPA = OCH_DP_B, BUF = 2 * OCH_DP_B;
+   typedef DoubleSlab<AKC, BM> LA;
+   typedef DoubleSlab<BKC, BN> LB;
+   static_assert(LA::LOADS == 4 && LB::LOADS == 4 && LA::TILES == TMS && LB::TILES == TNS, "the schedule below is written for these");
+   extern __shared__ __align__(16) char lds[];
+
+   int64_t oA, oB, oC, oAlpha, oBeta;
+   gemm_batch_offsets(p.batch, oA, oB, oC, oAlpha, oBeta);
+   const char *pA = p.A + oA, *pB = p.B + oB; char *pC = p.C + oC;
+   const uint32_t tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
+   const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+   const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+   const uint32_t wm = (wave % 2) * WM, wn = (wave / 2) * WN;
+
+   acc_zero_half();
+
+   const uint32_t nslabs = p.K / KT, last = nslabs - 1;
+   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)lds;      /* where the array starts in LDS */
+   const uint32_t rowsA = p.M - m0 < (uint32_t)BM ? p.M - m0 : (uint32_t)BM, rowsB = p.N - n0 < (uint32_t)BN ? p.N - n0 : (uint32_t)BN;    /* of this tile */
+   uint32_t offA[4], offB[4], tgtA[4], tgtB[4];
+#pragma unroll
+   for (int j = 0; j < 4; j++)
+   {  offA[j] = LA::load_offset(j, wave, lane, p.ldA, rowsA); tgtA[j] = lds0 + LA::load_target(j, wave);
+      offB[j] = LB::load_offset(j, wave, lane, p.ldB, rowsB); tgtB[j] = lds0 + OPA + LB::load_target(j, wave);
+   }
+   uint32_t readA[2], readB[2];
+#pragma unroll
+   for (int b = 0; b < 2; b++)
+   {  readA[b] = lds0 + LA::read_lane(wm, lane) + b * BUF; readB[b] = lds0 + OPA + LB::read_lane(wn, lane) + b * BUF;
+      asm volatile("" : "+v"(readA[b]), "+v"(readB[b]));
+   }
+   och_f64x2 fa[2][TMS], fb[2][TNS];
+
+#define OCH_LOAD(e, baseA, baseB, buf)                                                                                 \
+   do { if ((e) < 4) load_to_lds(baseA, offA[(e) % 4], tgtA[(e) % 4] + (buf) * BUF);                                   \
+        else         load_to_lds(baseB, offB[(e) % 4], tgtB[(e) % 4] + (buf) * BUF); } while (0)
+   /* one pair of steps = 32 MFMAs = 16 chunks: chunk c reads fragment c / 2 of pair PN from buffer RB into set NXT when c
+      is even, issues load LOAD0 + c / 4 into buffer LBUF when c % 4 == 2, then runs its two MFMAs */
+#define OCH_PAIR(CUR, NXT, RB, PN, LOAD0, LBUF)                                                                        \
+   do { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                            \
+        _Pragma("unroll") for (int c = 0; c < 16; c++)                                                                \
+        {  if (c % 2 == 0)                                                                                             \
+           {  if (c / 2 < TMS) fa[NXT][c / 2 % TMS] = lds_read(readA[RB], LA::read_offset(c / 2 % TMS, PN));            \
+              else             fb[NXT][c / 2 % TNS] = lds_read(readB[RB], LB::read_offset(c / 2 % TNS, PN));            \
+           }                                                                                                           \
+           if (c % 4 == 2) OCH_LOAD(LOAD0 + c / 4, nextA, nextB, LBUF);                                                \
+           {  const int st = c / 8, m = (c % 8) * 2, i = m / TNS, j = m % TNS;                                         \
+              mfma_f64(i * TNS + j, LA::value(fa[CUR], i, st), LB::value(fb[CUR], j, st));                             \
+              mfma_f64(i * TNS + j + 1, LA::value(fa[CUR], i, st), LB::value(fb[CUR], j + 1, st));                     \
+           }                                                                                                           \
+           __builtin_amdgcn_sched_barrier(0);                                                                          \
+        } } while (0)
+#define OCH_SLAB(s, CB)                                                                                                \
+   do { {  const uint32_t s1 = ((s) + 1 < last) ? (s) + 1 : last;                                                      \
+           const char *nextA = LA::slab_base(pA, p.ldA, m0, s1 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, s1 * KT);  \
+           OCH_PAIR(0, 1, CB, 1, 4, 1 - CB);                                                                           \
+        }                                                                                                              \
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                                                    \
+        __syncthreads();                                                                                               \
+        {  const uint32_t s2 = ((s) + 2 < last) ? (s) + 2 : last;                                                      \
+           const char *nextA = LA::slab_base(pA, p.ldA, m0, s2 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, s2 * KT);  \
+           OCH_PAIR(1, 0, 1 - CB, 0, 0, CB);                                                                           \
+        } } while (0)
+
+   {  /* slab 0 and the first half of slab 1 */
+      const uint32_t s1 = (1 < last) ? 1 : last;
+      const char *nextA = LA::slab_base(pA, p.ldA, m0, 0), *nextB = LB::slab_base(pB, p.ldB, n0, 0);
+#pragma unroll
+      for (int e = 0; e < 8; e++) OCH_LOAD(e, nextA, nextB, 0);
+      nextA = LA::slab_base(pA, p.ldA, m0, s1 * KT); nextB = LB::slab_base(pB, p.ldB, n0, s1 * KT);
+#pragma unroll
+      for (int e = 0; e < 4; e++) OCH_LOAD(e, nextA, nextB, 1);
+      asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+      __syncthreads();
+#pragma unroll
+      for (int x = 0; x < TMS; x++) fa[0][x] = lds_read(readA[0], LA::read_offset(x, 0));
+#pragma unroll
+      for (int x = 0; x < TNS; x++) fb[0][x] = lds_read(readB[0], LB::read_offset(x, 0));
+   }
+   asm volatile("s_nop 7");                 /* the zeroed accumulators are in place */
+   uint32_t s = 0;
+   for (; s + 1 < nslabs; s += 2)
+   {  OCH_SLAB(s, 0);
+      OCH_SLAB(s + 1, 1);
+   }
+   if (s < nslabs) OCH_SLAB(s, 0);
+   asm volatile("s_nop 15\n\ts_nop 15\n\ts_waitcnt vmcnt(0)" ::: "memory");       /* the last MFMAs have left the pipeline; the last loads have landed */
+   __syncthreads();
+#undef OCH_SLAB
+#undef OCH_PAIR
+#undef OCH_LOAD
+
+   double alpha = p.alpha, beta = p.beta;
+   if (p.alpha_dev) alpha = *reinterpret_cast<const double *>(reinterpret_cast<const char *>(p.alpha_dev) + oAlpha);
+   if (p.beta_dev)  beta = *reinterpret_cast<const double *>(reinterpret_cast<const char *>(p.beta_dev) + oBeta);
+   constexpr int CP = BM + 2, CPASS = 32, PASSES = BN / CPASS;
+   static_assert(CPASS * CP * 8 <= 2 * BUF, "a pass of the staged tile does not fit into the slab buffers");
+   double *stage = reinterpret_cast<double *>(lds);
+   for (int h = 0; h < PASSES; h++)
+   {
+#pragma unroll
+      for (int j = 0; j < TNS; j++)
+      {  const uint32_t col = wn + LB::row(j, lane % T);
+         if (col / CPASS != (uint32_t)h) continue;
+#pragma unroll
+         for (int i = 0; i < TMS; i++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+               stage[(col - h * CPASS) * CP + wm + LA::row(i, 4 * r + (lane >> 4))] = alpha * acc_read(i * TNS + j, r);
+      }
+      __syncthreads();
+      const uint32_t c0 = n0 + h * CPASS;
+      for (uint32_t q = threadIdx.x; q < CPASS * (BM / 2); q += THREADS)
+      {  const uint32_t c = q / (BM / 2), r2 = (q % (BM / 2)) * 2;
+         if (r2 >= rowsA || h * CPASS + c >= rowsB) continue;          /* outside C */
+         och_f64x2 v = *reinterpret_cast<const och_f64x2 *>(stage + c * CP + r2);
+         och_f64x2 *dst = reinterpret_cast<och_f64x2 *>(pC + ((int64_t)(m0 + r2) + (int64_t)(c0 + c) * p.ldC) * 8);
+         if (beta != 0) { const och_f64x2 old = *dst; v.x += beta * old.x; v.y += beta * old.y; }
+         *dst = v;
+      }
+      __syncthreads();
+   }
+}
+
 /* 0: launched; 1: not a case for this kernel (the caller's other kernels take it): M and N multiples of 2, K of 16,
    operands aligned to 16 bytes */
-int gemm_double_pipe(const GemmArgs &g)
+int gemm_double_pipe(const GemmArgs &g, int tile_m)          /* tile_m: 256 (tiles of 256 x 128) or 128 (tiles of 128 x 128) */
 {
    if (g.M % 2 != 0 || g.N % 2 != 0 || g.M == 0 || g.N == 0 || g.K % OCH_DP_KT != 0 || g.K == 0 || !gemm_operands_aligned(g, 8)) return 1;
    /* a lane's offset within a slab (up to 255 columns further on) is kept in 32 bits */
@@ -292,14 +429,15 @@ int gemm_double_pipe(const GemmArgs &g)
    if (g.scalar_mode_host) { memcpy(&p.alpha, g.alpha, 8); memcpy(&p.beta, g.beta, 8); }
    else { p.alpha_dev = (const double *)g.alpha; p.beta_dev = (const double *)g.beta; }
    p.batch = g.batch;
-   p.tiles_m = (uint32_t)((g.M + OCH_DP_BM - 1) / OCH_DP_BM); p.tiles_n = (uint32_t)((g.N + OCH_DP_BN - 1) / OCH_DP_BN);
+   if (tile_m != 256 && tile_m != 128) return 1;
+   p.tiles_m = (uint32_t)((g.M + tile_m - 1) / tile_m); p.tiles_n = (uint32_t)((g.N + OCH_DP_BN - 1) / OCH_DP_BN);
    const uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
    if (blocks > 0x7FFFFFFFull) return set_error("gemm: too many tiles");
    const bool akc = (g.transA != 'N'), bkc = (g.transB == 'N');
    const dim3 grid((unsigned)blocks, 1, g.nz), block(OCH_DP_THREADS);
-   const size_t lds = OCH_DP_BUFFERS * (size_t)OCH_DP_BUFFER;
+   const size_t lds = tile_m == 256 ? OCH_DP_BUFFERS * (size_t)OCH_DP_BUFFER : 4 * (size_t)OCH_DP_B;
 #define OCH_DP_LAUNCH(AK, BK)                                                                                         \
-   do { auto kernel = gemm_double_pipe_kernel<AK, BK>;                                                                \
+   do { auto kernel = tile_m == 256 ? gemm_double_pipe_kernel<AK, BK> : gemm_double_pipe_small_kernel<AK, BK>;        \
         OCH_CHECK_HIP(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
         hipLaunchKernelGGL(kernel, grid, block, lds, g.stream, p); } while (0)
    if (!akc && !bkc) OCH_DP_LAUNCH(false, false);

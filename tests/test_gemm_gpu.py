@@ -223,6 +223,32 @@ def check_large_product(stream, dtype, ta, tb, M, N, cases, rng, pad=0):
             assert np.linalg.norm(have - want) <= TOL[dtype] * np.linalg.norm(bound), what + " (probe vectors)"
 
 
+@pytest.mark.parametrize("choice", [1, 2, 3], ids=["large_tile", "small_tile", "tiled_kernel"])
+@pytest.mark.parametrize("dtype", [H.FLOAT, H.DOUBLE, H.CFLOAT], ids=lambda d: H.NAMES[d])
+def test_gemm_pipelined_kernels_against_the_oracle(hip, stream, dtype, choice):
+    """With the kernel choice fixed (och_gemm_set_kernel_choice) the pipelined kernels take every aligned product whose M and
+    N are multiples of 4 (double, complex float: 2), however small: whole results against the oracle for single tiles, last
+    tiles of a few rows and columns, one to nine slabs of K, a K with a remainder (host scalars: pipelined head + additive
+    rest; device scalars: the tiled kernel), every transposition and conjugation. Choice 3 is the tiled kernel on the same
+    shapes."""
+    rng = np.random.default_rng(1600 + 10 * dtype + choice)
+    slab = 16 if dtype == H.DOUBLE else 32
+    cplx = dtype == H.CFLOAT
+    modes = ["N", "T"] + (["C"] if cplx else [])
+    shapes = [(128, 128, slab), (132, 260, 3 * slab), (388, 130 if dtype != H.FLOAT else 132, 2 * slab), (260, 516, 9 * slab + 8), (512, 256, 5 * slab),
+              (256, 384, 4 * slab)]
+    assert oh.lib.och_gemm_set_kernel_choice(7) != 0
+    oh.check(oh.lib.och_gemm_set_kernel_choice(choice))
+    try:
+        for n, (M, N, K) in enumerate(shapes):
+            for ta in modes:
+                for tb in modes:
+                    alpha, beta = ((2 - 1j, -1 + 0.5j) if cplx else (2, -1)) if (n + len(ta + tb) + ord(ta)) % 2 else (1, 0)
+                    run_case(stream, dtype, ta, tb, M, N, K, alpha, beta, rng, device_scalars=(n % 3 == 2), pad=4)
+    finally:
+        oh.check(oh.lib.och_gemm_set_kernel_choice(0))
+
+
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
 def test_gemm_float_pipelined_whole_tiles(hip, stream, ta, tb):
     """float products of 256 whole aligned 256 x 256 tiles or more run on the hand-pipelined kernel: one slab of 32 k
