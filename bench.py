@@ -538,7 +538,32 @@ def main():
             for buf in (a, b, c):
                 buf.free()
         if True:
-            # beyond the named configurations: half-precision and 8-bit products of the same size on the matrix cores
+            # beyond the named configurations: complex double of the complex-float size; a float product whose sizes are
+            # not multiples of any tile
+            dim = 4096
+            a, b, c = [oh.DeviceBuffer(16 * dim * dim, stream) for _ in range(3)]
+            block = rng.uniform(-1, 1, 1 << 22)
+            for buf in (a, b):
+                upload_tiled(buf, block, 16 * dim * dim)
+            onez = np.array([1.0, 0.0]); zeroz = np.zeros(2)
+            for ta, tb in ((b"N", b"N"), (b"T", b"N"), (b"N", b"T")):
+                fn = lambda: oh.check(lib.och_gemm(CD, ta, tb, dim, dim, dim, onez.ctypes.data, a.ptr, dim, b.ptr, dim,
+                                                   zeroz.ctypes.data, c.ptr, dim, 1, h))
+                configs["extra_gemm_cdouble_%d_%s%s" % (dim, ta.decode(), tb.decode())] = tflops(8 * dim ** 3, sample_launches(fn, warm=2), MFMA_PEAK["cdouble"])
+            for buf in (a, b, c):
+                buf.free()
+            dim = 7000
+            a, b, c = [oh.DeviceBuffer(4 * dim * dim, stream) for _ in range(3)]
+            block = rng.uniform(-1, 1, 1 << 22).astype(np.float32)
+            for buf in (a, b):
+                upload_tiled(buf, block, 4 * dim * dim)
+            onef = np.array([1, 0], np.float32); zerof = np.zeros(2, np.float32)
+            fn = lambda: oh.check(lib.och_gemm(F32, b"N", b"N", dim, dim, dim, onef.ctypes.data, a.ptr, dim, b.ptr, dim,
+                                               zerof.ctypes.data, c.ptr, dim, 1, h))
+            configs["extra_gemm_float_%d_NN" % dim] = tflops(2 * dim ** 3, sample_launches(fn, warm=2), MFMA_PEAK["float"])
+            for buf in (a, b, c):
+                buf.free()
+            # half-precision and 8-bit products of the size of the named configurations on the matrix cores
             dim = 8192
             a, b, c = [oh.DeviceBuffer(2 * dim * dim, stream) for _ in range(3)]
             block = rng.uniform(-1, 1, 1 << 22).astype(np.float16)

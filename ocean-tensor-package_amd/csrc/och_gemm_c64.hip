@@ -3,7 +3,37 @@
 namespace och {
 int gemm_cdouble(const GemmArgs &g)
 {  static const GemmTileChoice choice[2] = { { 128, 64, 1.0 }, { 64, 64, 0.94 } };
-   if (gemm_pick_tile(g, choice, 2) == 0) return launch_gemm_mfma<double, true, 64, 32, 8>(g);
+   const int pick = gemm_pick_tile(g, choice, 2);
+   /* Products with K a multiple of 16 run on the pipelined kernel (och_gemm_c64p.hip) on tiles of 128 x 64 when that is
+      cheaper by the model of gemm_pick_tile (rounds of the compute units x tile area / efficiency, the kernel below at
+      0.87 of the pipelined one). A K that is not a multiple of 16 (scalars in host memory only): the whole slabs there,
+      the rest of K as a product of its own that adds to C. */
+   if (g.M >= 64 && g.N >= 32 && g.K >= 16 && (g.K % 16 == 0 || (g.scalar_mode_host && g.K >= 128)) && gemm_operands_aligned(g, 16))
+   {  const uint64_t units = (uint64_t)gemm_compute_units();
+      auto cost = [&](uint64_t bm, uint64_t bn, double efficiency)
+      {  const uint64_t tiles = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * (uint64_t)g.nz;
+         return (double)((tiles + units - 1) / units) * (double)(bm * bn) / efficiency;
+      };
+      const int forced = gemm_kernel_choice();
+      if (forced != 3 && (forced != 0 || cost(128, 64, 1.0) < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87)))
+      {  GemmArgs part = g;
+         const size_t Kh = g.K - g.K % 16;
+         part.K = Kh;
+         const int taken = gemm_cdouble_pipe(part);
+         if (taken < 0) return taken;
+         if (taken == 0)
+         {  if (g.K > Kh)
+            {  static const double one[2] = { 1.0, 0.0 };
+               part.K = g.K - Kh; part.beta = one;
+               part.A = (const char *)g.A + (int64_t)Kh * (g.transA == 'N' ? (int64_t)g.ldA : 1) * 16;
+               part.B = (const char *)g.B + (int64_t)Kh * (g.transB == 'N' ? 1 : (int64_t)g.ldB) * 16;
+               if (gemm_cdouble(part) != 0) return -1;
+            }
+            return 0;
+         }
+      }
+   }
+   if (pick == 0) return launch_gemm_mfma<double, true, 64, 32, 8>(g);
    return launch_gemm_mfma<double, true, 32, 32, 8>(g);
 }
 }

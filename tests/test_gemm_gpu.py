@@ -173,8 +173,8 @@ def check_large_product(stream, dtype, ta, tb, M, N, cases, rng, pad=0):
     times probe vectors against op(A) (op(B) x) -- in exact arithmetic modulo 256 for the 8-bit types, to the
     precision's bound for half and float. cases: (slabs of K, alpha, beta, scalars in device memory); pad: rows of
     junk between the columns of all three operands."""
-    kt = {H.HALF: 64, H.FLOAT: 32, H.DOUBLE: 16, H.CFLOAT: 32}.get(dtype, 128)
-    exact = dtype not in (H.HALF, H.FLOAT, H.DOUBLE, H.CFLOAT)
+    kt = {H.HALF: 64, H.FLOAT: 32, H.DOUBLE: 16, H.CFLOAT: 32, H.CDOUBLE: 16}.get(dtype, 128)
+    exact = dtype not in (H.HALF, H.FLOAT, H.DOUBLE, H.CFLOAT, H.CDOUBLE)
     for slabs, alpha, beta, dev in cases:
         K = int(round(slabs * kt))
         rowsA, colsA = (M, K) if ta == "N" else (K, M)
@@ -193,7 +193,7 @@ def check_large_product(stream, dtype, ta, tb, M, N, cases, rng, pad=0):
         got = dC.download(C0.dtype, C0.size)
         for b in (dA, dB, dC):
             b.free()
-        wide = np.int64 if exact else (np.complex128 if dtype == H.CFLOAT else np.float64)
+        wide = np.int64 if exact else (np.complex128 if dtype in (H.CFLOAT, H.CDOUBLE) else np.float64)
         num = (lambda a: a.astype(np.int64)) if exact else (lambda a: as_float(dtype, a).astype(wide))
         mA, mB = num(A).reshape(colsA, ldA)[:, :rowsA].T, num(B).reshape(colsB, ldB)[:, :rowsB].T            # [row, col]
         op = {"N": lambda m: m, "T": lambda m: m.T, "C": lambda m: m.conj().T}
@@ -224,7 +224,7 @@ def check_large_product(stream, dtype, ta, tb, M, N, cases, rng, pad=0):
 
 
 @pytest.mark.parametrize("choice", [1, 2, 3], ids=["large_tile", "small_tile", "tiled_kernel"])
-@pytest.mark.parametrize("dtype", [H.FLOAT, H.DOUBLE, H.CFLOAT], ids=lambda d: H.NAMES[d])
+@pytest.mark.parametrize("dtype", [H.FLOAT, H.DOUBLE, H.CFLOAT, H.CDOUBLE], ids=lambda d: H.NAMES[d])
 def test_gemm_pipelined_kernels_against_the_oracle(hip, stream, dtype, choice):
     """With the kernel choice fixed (och_gemm_set_kernel_choice) the pipelined kernels take every aligned product whose M and
     N are multiples of 4 (double, complex float: 2), however small: whole results against the oracle for single tiles, last
@@ -232,8 +232,8 @@ def test_gemm_pipelined_kernels_against_the_oracle(hip, stream, dtype, choice):
     rest; device scalars: the tiled kernel), every transposition and conjugation. Choice 3 is the tiled kernel on the same
     shapes."""
     rng = np.random.default_rng(1600 + 10 * dtype + choice)
-    slab = 16 if dtype == H.DOUBLE else 32
-    cplx = dtype == H.CFLOAT
+    slab = 16 if dtype in (H.DOUBLE, H.CDOUBLE) else 32
+    cplx = dtype in (H.CFLOAT, H.CDOUBLE)
     modes = ["N", "T"] + (["C"] if cplx else [])
     shapes = [(128, 128, slab), (132, 260, 3 * slab), (388, 130 if dtype != H.FLOAT else 132, 2 * slab), (260, 516, 9 * slab + 8), (512, 256, 5 * slab),
               (256, 384, 4 * slab)]
@@ -277,6 +277,16 @@ def test_gemm_cfloat_pipelined_whole_tiles(hip, stream, ta, tb):
     check_large_product(stream, H.CFLOAT, ta, tb, 2048, 2048, ((6, -1.5j, 0.5, False),), rng, pad=6)
     check_large_product(stream, H.CFLOAT, ta, tb, 2048, 2048, ((8.125, 1 - 1j, 0.5j, False),), rng)            # a K of 8 slabs + 4
     check_large_product(stream, H.CFLOAT, ta, tb, 4098, 4098, ((2, 1, -1, False),), rng)                        # last tiles of two rows / columns
+
+
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "C"), ("C", "T")])
+def test_gemm_cdouble_pipelined_tiles(hip, stream, ta, tb):
+    """complex double products that fill the compute units with tiles of 128 x 64 run on the hand-pipelined kernel, whose
+    three slab buffers rotate: one to four slabs of 16 k, a K with a remainder, odd M and N (last tiles of one row and one
+    column), complex alpha and beta in host and in device memory."""
+    rng = np.random.default_rng(1700 + ord(ta) + 2 * ord(tb))
+    check_large_product(stream, H.CDOUBLE, ta, tb, 2048, 1024, ((1, 1, 0, False), (2, 2 - 1j, -1 + 0.5j, True), (3, -1j, 1, False), (4, 1, 0.5j, False)), rng)
+    check_large_product(stream, H.CDOUBLE, ta, tb, 2049, 2049, ((9.3125, 1 - 1j, 0.5, False),), rng, pad=3)
 
 
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
