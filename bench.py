@@ -143,7 +143,8 @@ def main():
         for typ, (name, peak) in enumerate(peaks):
             mfmabench(typ, 0, 0, 4, 16000)                       # warm: the clock settles under this load
             ms, flop = mfmabench(typ, 0, 0, 4, 16000)
-            print("   %-16s MFMAs alone: %8.1f T/s = %.3f of the nominal %.1f" % (name, flop / ms / 1e9, flop / ms / 1e9 / peak, peak))
+            ms1, flop1 = mfmabench(typ, 7, 0, 4, 16000)
+            print("   %-16s MFMAs alone: %8.1f T/s = %.3f of the nominal %.1f on 16 pseudo-random operand pairs in turn; %8.1f T/s on one pair" % (name, flop / ms / 1e9, flop / ms / 1e9 / peak, peak, flop1 / ms1 / 1e9))
         print("   cost of an instruction between 64-cycle float MFMAs, in MFMA cycles (64 x time / time of the bare loop - 64) per instruction:")
         for waves in (4, 8):
             base, _ = mfmabench(0, 0, 0, waves)
@@ -574,6 +575,16 @@ def main():
                 fn = lambda: oh.check(lib.och_gemm(oh.HALF, ta, tb, dim, dim, dim, one16.ctypes.data, a.ptr, dim, b.ptr, dim,
                                                    zero16.ctypes.data, c.ptr, dim, 1, h))
                 configs["extra_gemm_half_%d_%s%s" % (dim, ta.decode(), tb.decode())] = tflops(2 * dim ** 3, sample_launches(fn, warm=2), 2500.0)
+            # the same products on operands that are 1.0 everywhere: the same instructions at the same addresses, but hardly a
+            # bit changes from one MFMA to the next, the matrix cores draw less power and the clock stays up -- how much of
+            # the distance to nominal peak is the power limit and how much the kernel
+            block = np.full(1 << 22, 0x3C00, np.uint16)
+            for buf in (a, b):
+                upload_tiled(buf, block, 2 * dim * dim)
+            for ta, tb in ((b"N", b"N"), (b"T", b"N")):
+                fn = lambda: oh.check(lib.och_gemm(oh.HALF, ta, tb, dim, dim, dim, one16.ctypes.data, a.ptr, dim, b.ptr, dim,
+                                                   zero16.ctypes.data, c.ptr, dim, 1, h))
+                configs["extra_gemm_half_%d_%s%s_constant_operands" % (dim, ta.decode(), tb.decode())] = tflops(2 * dim ** 3, sample_launches(fn, warm=2), 2500.0)
             for buf in (a, b, c):
                 buf.free()
             a, b, c = [oh.DeviceBuffer(dim * dim, stream) for _ in range(3)]

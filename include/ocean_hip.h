@@ -145,7 +145,8 @@ int och_membench(int kind, int unr, int nt, int map, int block, int blocks, size
 
 /* Matrix-core micro-benchmark (no counterpart in the reference): the rate of a loop of nothing but MFMAs, and what     */
 /* other instructions of the same wave cost between them. type: 0 float 32x32x2, 1 double 16x16x4, 2 half 32x32x16,    */
-/* 3 int8 32x32x32. kind: 0 MFMAs alone, 1 v_mov_b32, 2 v_add_f32, 3 s_nop, 4 s_add_u32, 5 s_waitcnt, 6 ds_read_b128,   */
+/* 3 int8 32x32x32. kind: 0 MFMAs alone on 16 pseudo-random operand pairs in turn, 7 MFMAs alone on one operand pair   */
+/* (the power drawn, and with it the clock, depends on it), 1 v_mov_b32, 2 v_add_f32, 3 s_nop, 4 s_add_u32, 5 s_waitcnt, 6 ds_read_b128, */
 /* `per_mfma` (1, 2 or 4) of them after every MFMA. waves: 4 or 8 per block, one block per compute unit. Times `reps`  */
 /* launches of `iters` iterations of 16 MFMAs per wave with events on `stream`; returns the median time of a launch    */
 /* and the flop (or integer operations) it performs. Allocates and frees its own small buffers. Synchronous.           */

@@ -43,7 +43,8 @@ template <> struct MfbOp<3>
    static __device__ __forceinline__ Acc mma(In a, In b, Acc c) { return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0); }
 };
 
-/* KIND: 0 nothing, 1 v_mov_b32, 2 v_add_f32, 3 s_nop, 4 s_add_u32, 5 s_waitcnt (nothing to wait for), 6 ds_read_b128 */
+/* KIND: 0 nothing, 1 v_mov_b32, 2 v_add_f32, 3 s_nop, 4 s_add_u32, 5 s_waitcnt (nothing to wait for), 6 ds_read_b128,
+   7 nothing, and every MFMA on the same pair of operands */
 template <int TYPE, int KIND, int N, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void mfmabench_kernel(float *out, const float *in, int iters)
 {
@@ -71,8 +72,8 @@ __global__ __launch_bounds__(64 * WAVES) void mfmabench_kernel(float *out, const
    {
 #pragma unroll
       for (int c = 0; c < 16; c++)
-      {  if (TYPE == 1) asm volatile("v_mfma_f64_16x16x4_f64 a[%2:%2+7], %0, %1, a[%2:%2+7]" : : "v"(a[c % 4]), "v"(b[c / 4]), "i"(8 * (c % 16)));
-         else acc[c % Op::ACCS] = Op::mma(a[c % 4], b[c / 4], acc[c % Op::ACCS]);
+      {  if (TYPE == 1) asm volatile("v_mfma_f64_16x16x4_f64 a[%2:%2+7], %0, %1, a[%2:%2+7]" : : "v"(a[KIND == 7 ? 0 : c % 4]), "v"(b[KIND == 7 ? 0 : c / 4]), "i"(8 * (c % 16)));
+         else acc[c % Op::ACCS] = Op::mma(a[KIND == 7 ? 0 : c % 4], b[KIND == 7 ? 0 : c / 4], acc[c % Op::ACCS]);
 #pragma unroll
          for (int n = 0; n < N; n++)
          {  if (KIND == 1) asm volatile("v_mov_b32 %0, %1" : "=v"(t) : "v"(x));
@@ -107,6 +108,7 @@ template <int TYPE, int KIND> static mfb_kernel mfb_pick_n(int n, int waves)
 template <int TYPE> static mfb_kernel mfb_pick_kind(int kind, int n, int waves)
 {  switch (kind)
    {  case 0: return mfb_pick_n<TYPE, 0>(0, waves);
+      case 7: return mfb_pick_waves<TYPE, 7, 0>(waves);
       case 1: return mfb_pick_n<TYPE, 1>(n, waves); case 2: return mfb_pick_n<TYPE, 2>(n, waves); case 3: return mfb_pick_n<TYPE, 3>(n, waves);
       case 4: return mfb_pick_n<TYPE, 4>(n, waves); case 5: return mfb_pick_n<TYPE, 5>(n, waves); case 6: return mfb_pick_n<TYPE, 6>(n, waves);
    }
@@ -117,14 +119,15 @@ template <int TYPE> static mfb_kernel mfb_pick_kind(int kind, int n, int waves)
 
 using namespace och;
 
-/* type: 0 float, 1 double, 2 half, 3 int8 MFMA. kind: 0 MFMAs alone, 1 v_mov_b32, 2 v_add_f32, 3 s_nop, 4 s_add_u32,
-   5 s_waitcnt, 6 ds_read_b128 -- `per_mfma` (1, 2 or 4; ignored for kind 0) of them after every MFMA. waves: 4 or 8 per
+/* type: 0 float, 1 double, 2 half, 3 int8 MFMA. kind: 0 MFMAs alone (16 pairs of pseudo-random operands in turn), 7 MFMAs
+   alone on one pair of operands, 1 v_mov_b32, 2 v_add_f32, 3 s_nop, 4 s_add_u32, 5 s_waitcnt, 6 ds_read_b128 -- `per_mfma`
+   (1, 2 or 4; ignored for kinds 0 and 7) of them after every MFMA. waves: 4 or 8 per
    block (one block per compute unit). Times `reps` launches of `iters` iterations of 16 MFMAs per wave with events on
    `stream` after one untimed launch; returns the median time of a launch and the flop it performs. Synchronous. */
 extern "C" int och_mfmabench(int type, int kind, int per_mfma, int waves, int iters, int reps, float *median_ms, double *flop, och_stream stream_)
 {
    hipStream_t stream = as_stream(stream_);
-   if (type < 0 || type > 3 || kind < 0 || kind > 6) return set_error("mfmabench: unknown type %d or kind %d", type, kind);
+   if (type < 0 || type > 3 || kind < 0 || kind > 7) return set_error("mfmabench: unknown type %d or kind %d", type, kind);
    if (waves != 4 && waves != 8) return set_error("mfmabench: 4 or 8 waves per block");
    if (iters < 1 || iters > (1 << 20) || reps < 1 || reps > 1000) return set_error("mfmabench: iters / reps out of range");
    mfb_kernel fn = nullptr;

@@ -33,7 +33,7 @@ def test_mfmabench_rates_and_instruction_costs(hip, stream):
 
 def test_mfmabench_arguments(hip, stream):
     ms, flop = C.c_float(), C.c_double()
-    for args in ((4, 0, 0, 4, 10, 1), (0, 7, 1, 4, 10, 1), (0, 1, 3, 4, 10, 1), (0, 0, 0, 5, 10, 1), (0, 0, 0, 4, 0, 1), (0, 0, 0, 4, 10, 0)):
+    for args in ((4, 0, 0, 4, 10, 1), (0, 8, 1, 4, 10, 1), (0, 1, 3, 4, 10, 1), (0, 0, 0, 5, 10, 1), (0, 0, 0, 4, 0, 1), (0, 0, 0, 4, 10, 0)):
         assert oh.lib.och_mfmabench(*args, C.byref(ms), C.byref(flop), stream.handle) != 0, args
         assert b"mfmabench" in oh.lib.och_last_error()
 
