@@ -54,7 +54,7 @@ int fill_bytes(void *dst, int value, size_t nbytes, hipStream_t stream);
 #define OCH_RED_MAX_BLOCKS 512
 #define OCH_RED_SLOT 16                               /* bytes per partial of a full reduction */
 #define OCH_RED_SCRATCH (OCH_RED_MAX_BLOCKS * OCH_RED_SLOT + 256)
-#define OCH_GEMM_WORKSPACE (16u << 20)                /* partial products of the split-K matrix-vector kernels */
+#define OCH_GEMM_WORKSPACE (64u << 20)                /* partial products of the kernels that split K */
 struct StreamContext
 {  char *red_scratch;          /* OCH_RED_SCRATCH bytes, partial slots + ticket counter (zero between launches) */
    void *host_result;          /* 64 bytes of pinned host memory: result of a full reduction */

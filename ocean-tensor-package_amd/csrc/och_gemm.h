@@ -590,9 +590,11 @@ static inline bool gemm_operands_aligned(const GemmArgs &g, int es)
 }
 
 int gemm_float(const GemmArgs &g);
-int gemm_float_pipe(const GemmArgs &g, int tile); /* whole aligned tiles of 256 x 256 or 128 x 128; 1: not taken */
+int gemm_float_pipe(const GemmArgs &g, int tile); /* tiles of 256 x 256 or 128 x 128; 1: not taken */
+int gemm_float_pipe_split(const GemmArgs &g, int tile, double *rounds); /* shares of the tiles of the last round; rounds of the compute units */
 int gemm_double(const GemmArgs &g);
 int gemm_double_pipe(const GemmArgs &g, int tile_m); /* tiles of 256 x 128 or 128 x 128; 1: not taken */
+int gemm_double_pipe_split(const GemmArgs &g, int tile_m, double *rounds); /* shares of the tiles of the last round; rounds of the compute units */
 int gemm_cfloat(const GemmArgs &g);
 int gemm_cfloat_pipe(const GemmArgs &g); /* whole aligned 128 x 128 tiles; 1: not taken */
 int gemm_cdouble(const GemmArgs &g);

@@ -8,7 +8,7 @@ int gemm_float(const GemmArgs &g)
    const int pick = gemm_pick_tile(g, choice, 4);
    /* Aligned products with M and N multiples of 4 and K of 32 run on the pipelined kernel (och_gemm_f32p.hip) on tiles of
       256 x 256 or 128 x 128 when that is cheaper by the model of gemm_pick_tile: rounds of the compute units x tile area /
-      efficiency, with the kernels below at 0.85 of the pipelined kernel on 256 x 256 tiles and the 128 x 128 tiles at 0.9
+      efficiency, with the kernels below at 0.8 of the pipelined kernel on 256 x 256 tiles and the 128 x 128 tiles at 0.95
       (8192^3: 130 against 153 TFLOP/s; 2048^3: 84 against 135). A K that is not a multiple of 32 (scalars in host memory
       only): the whole slabs there, the rest of K as a product of its own that adds to C. */
    if (g.M >= 128 && g.N >= 128 && g.M % 4 == 0 && g.N % 4 == 0 && g.K >= 32 && (g.K % 32 == 0 || (g.scalar_mode_host && g.K >= 256)) && gemm_operands_aligned(g, 4))
@@ -17,8 +17,14 @@ int gemm_float(const GemmArgs &g)
       {  const uint64_t tiles = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * (uint64_t)g.nz;
          return (double)((tiles + units - 1) / units) * (double)(bm * bn) / efficiency;
       };
-      const double others = cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.85);
-      const double large = cost(256, 256, 1.0), small = cost(128, 128, 0.9);
+      const double others = cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.8);
+      /* the pipelined kernel cuts the tiles of a last round that is at most half full along K: that round then counts as
+         1 / shares of a round */
+      GemmArgs whole = g;
+      whole.K = g.K - g.K % 32;
+      double rounds_large = 0, rounds_small = 0;
+      gemm_float_pipe_split(whole, 256, &rounds_large); gemm_float_pipe_split(whole, 128, &rounds_small);
+      const double large = rounds_large * 65536.0, small = rounds_small * 16384.0 / 0.95;
       const int forced = gemm_kernel_choice();
       const int tile = forced == 1 ? 256 : (forced == 2 ? 128 : (large <= small ? 256 : 128));
       if (forced != 3 && (forced != 0 || (tile == 256 ? large : small) < others))

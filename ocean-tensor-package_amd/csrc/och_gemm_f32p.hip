@@ -46,6 +46,12 @@ struct FloatPipeParams
    float    alpha, beta;
    const float *alpha_dev, *beta_dev;
    uint32_t tiles_m, tiles_n;
+   /* the tiles of the last, partly filled round of the compute units are cut along K: tiles from split_first on are
+      computed by `split` blocks each, block q of them (counted from the first such block) leaving the raw sums of its
+      share of the slabs in partial[q] (a dense tile, column-major); gemm_float_pipe_finish_kernel adds the shares in
+      order and applies alpha / beta. split <= 1: no tile is cut. Only without a batch. */
+   uint32_t split_first, split;
+   float   *partial;
    GemmBatch batch;
 };
 
@@ -128,7 +134,10 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pi
    int64_t oA, oB, oC, oAlpha, oBeta;
    gemm_batch_offsets(p.batch, oA, oB, oC, oAlpha, oBeta);
    const char *pA = p.A + oA, *pB = p.B + oB; char *pC = p.C + oC;
-   const uint32_t tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
+   uint32_t tile = blockIdx.x, share = 0, shares = 1, cut = 0;           /* cut: index of this block among those of cut tiles */
+   if (p.split > 1 && blockIdx.x >= p.split_first)
+   {  cut = blockIdx.x - p.split_first; tile = p.split_first + cut / p.split; share = cut % p.split; shares = p.split; }
+   const uint32_t tile_m = tile % p.tiles_m, tile_n = tile / p.tiles_m;
    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
    const uint32_t wm = (wave % 2) * WM, wn = (wave / 2) * WN;
@@ -141,7 +150,9 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pi
 #pragma unroll
          for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
 
-   const uint32_t nslabs = p.K / KT, last = nslabs - 1;
+   /* this block's slabs: slab0 .. last of the product's K / KT (all of them unless the tile is cut) */
+   const uint32_t per_share = (p.K / KT + shares - 1) / shares, slab0 = share * per_share;
+   const uint32_t nslabs = slab0 + per_share <= p.K / KT ? per_share : p.K / KT - slab0, last = slab0 + nslabs - 1;
    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)lds;      /* where the array starts in LDS */
    const uint32_t rowsA = p.M - m0 < (uint32_t)BM ? p.M - m0 : (uint32_t)BM, rowsB = p.N - n0 < (uint32_t)BN ? p.N - n0 : (uint32_t)BN;    /* of this tile */
    uint32_t offA[NLA], offB[NLA], tgtA[NLA], tgtB[NLA];
@@ -182,7 +193,7 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pi
    /* slab s in buffer CB: quad 0 carries the second half of the loads of slab s + 1 (into the other buffer), quad 3 the
       first half of the loads of slab s + 2 (into this one) */
 #define OCH_SLAB(s, CB)                                                                                                \
-   do { {  const uint32_t s1 = ((s) + 1 < last) ? (s) + 1 : last;                                                      \
+   do { {  const uint32_t s1 = (slab0 + (s) + 1 < last) ? slab0 + (s) + 1 : last;                                      \
            const char *nextA = LA::slab_base(pA, p.ldA, m0, s1 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, s1 * KT);  \
            OCH_QUAD(0, 1, CB, 1, true, NL / 2, 1 - CB);                                                                     \
         }                                                                                                              \
@@ -192,14 +203,14 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pi
         }                                                                                                              \
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                               \
         __syncthreads();                                                                                               \
-        {  const uint32_t s2 = ((s) + 2 < last) ? (s) + 2 : last;                                                      \
+        {  const uint32_t s2 = (slab0 + (s) + 2 < last) ? slab0 + (s) + 2 : last;                                      \
            const char *nextA = LA::slab_base(pA, p.ldA, m0, s2 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, s2 * KT);  \
            OCH_QUAD(1, 0, 1 - CB, 0, true, 0, CB);                                                                     \
         } } while (0)
 
    {  /* slab 0 and the first half of slab 1 */
-      const uint32_t s1 = (1 < last) ? 1 : last;
-      const char *nextA = LA::slab_base(pA, p.ldA, m0, 0), *nextB = LB::slab_base(pB, p.ldB, n0, 0);
+      const uint32_t s1 = (slab0 + 1 < last) ? slab0 + 1 : last;
+      const char *nextA = LA::slab_base(pA, p.ldA, m0, slab0 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, slab0 * KT);
 #pragma unroll
       for (int e = 0; e < NL; e++) OCH_LOAD(e, nextA, nextB, 0);
       nextA = LA::slab_base(pA, p.ldA, m0, s1 * KT); nextB = LB::slab_base(pB, p.ldB, n0, s1 * KT);
@@ -230,6 +241,14 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pi
    float alpha = p.alpha, beta = p.beta;
    if (p.alpha_dev) alpha = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(p.alpha_dev) + oAlpha);
    if (p.beta_dev)  beta = *reinterpret_cast<const float *>(reinterpret_cast<const char *>(p.beta_dev) + oBeta);
+   /* a share of a cut tile leaves its raw sums, the whole tile, in the workspace */
+   char *out = pC + ((int64_t)m0 + (int64_t)n0 * p.ldC) * 4;
+   int64_t ldOut = p.ldC;
+   uint32_t rowsOut = rowsA, colsOut = rowsB;
+   if (shares > 1)
+   {  alpha = 1.0f; beta = 0.0f;
+      out = reinterpret_cast<char *>(p.partial + (size_t)cut * BM * BN); ldOut = BM; rowsOut = BM; colsOut = BN;
+   }
    constexpr int CP = BM + 4, CPASS = 64, PASSES = BN / CPASS;
    static_assert(CPASS * CP * 4 <= 2 * BUF, "a pass of the staged tile does not fit into the slab buffers");
    float *stage = reinterpret_cast<float *>(lds);
@@ -246,17 +265,68 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pi
                stage[(col - h * CPASS) * CP + wm + LA::row(i, 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3))] = alpha * acc[i][j][r];
       }
       __syncthreads();
-      const uint32_t c0 = n0 + h * CPASS;
       for (uint32_t q = threadIdx.x; q < CPASS * (BM / 4); q += THREADS)
       {  const uint32_t c = q / (BM / 4), r4 = (q % (BM / 4)) * 4;
-         if (r4 >= rowsA || h * CPASS + c >= rowsB) continue;          /* outside C */
+         if (r4 >= rowsOut || h * CPASS + c >= colsOut) continue;      /* outside C */
          och_f32x4 v = *reinterpret_cast<const och_f32x4 *>(stage + c * CP + r4);
-         och_f32x4 *dst = reinterpret_cast<och_f32x4 *>(pC + ((int64_t)(m0 + r4) + (int64_t)(c0 + c) * p.ldC) * 4);
+         och_f32x4 *dst = reinterpret_cast<och_f32x4 *>(out + ((int64_t)r4 + (int64_t)(h * CPASS + c) * ldOut) * 4);
          if (beta != 0) { const och_f32x4 old = *dst; v.x += beta * old.x; v.y += beta * old.y; v.z += beta * old.z; v.w += beta * old.w; }
          *dst = v;
       }
       __syncthreads();
    }
+}
+
+/* The shares of the cut tiles, added in the order of their slabs, times alpha, plus beta * C: a block per 32 columns of a
+   cut tile (grid y), 16 bytes of a column of C per thread and trip. */
+template <int TS>
+__global__ __launch_bounds__(256) void gemm_float_pipe_finish_kernel(const FloatPipeParams p)
+{
+   constexpr uint32_t BM = 64 * TS, BN = 64 * TS;
+   const uint32_t tile = p.split_first + blockIdx.x, tile_m = tile % p.tiles_m, tile_n = tile / p.tiles_m;
+   const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+   const uint32_t rows = p.M - m0 < BM ? p.M - m0 : BM, cols = p.N - n0 < BN ? p.N - n0 : BN;
+   const float alpha = p.alpha_dev ? *p.alpha_dev : p.alpha, beta = p.beta_dev ? *p.beta_dev : p.beta;
+   const float *shares = p.partial + (size_t)blockIdx.x * p.split * BM * BN;
+   for (uint32_t q = threadIdx.x; q < 32 * (BM / 4); q += 256)
+   {  const uint32_t c = blockIdx.y * 32 + q / (BM / 4), r4 = (q % (BM / 4)) * 4;
+      if (r4 >= rows || c >= cols) continue;
+      och_f32x4 v = *reinterpret_cast<const och_f32x4 *>(shares + (size_t)c * BM + r4);
+      for (uint32_t t = 1; t < p.split; t++)
+      {  const och_f32x4 w = *reinterpret_cast<const och_f32x4 *>(shares + (size_t)t * BM * BN + (size_t)c * BM + r4);
+         v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
+      }
+      v.x *= alpha; v.y *= alpha; v.z *= alpha; v.w *= alpha;
+      och_f32x4 *dst = reinterpret_cast<och_f32x4 *>(p.C + ((int64_t)(m0 + r4) + (int64_t)(n0 + c) * p.ldC) * 4);
+      if (beta != 0) { const och_f32x4 old = *dst; v.x += beta * old.x; v.y += beta * old.y; v.z += beta * old.z; v.w += beta * old.w; }
+      *dst = v;
+   }
+}
+
+/* Into how many shares the tiles of the last round are cut (1: not at all): the round must be at most half full, every
+   share at least 8 slabs long, and all shares must fit into the stream's workspace. *rounds: the rounds of the compute
+   units the product then takes (for the cost model of the caller); the cut round counts as the length of a share plus
+   what every block spends outside its main loop (about 6 slabs' worth) over the length of a whole tile. */
+int gemm_float_pipe_split(const GemmArgs &g, int tile, double *rounds)
+{
+   const uint64_t units = (uint64_t)gemm_compute_units();
+   const uint64_t tiles = ((g.M + tile - 1) / tile) * ((g.N + tile - 1) / tile) * (uint64_t)g.nz;
+   const uint64_t rest = tiles % units, slabs = g.K / OCH_FP_KT;
+   uint64_t shares = 1;
+   if (g.batch.nb == 0 && g.nz == 1 && rest > 0 && rest * 2 <= units && slabs >= 16)
+   {  shares = units / rest;
+      if (shares > 8) shares = 8;
+      if (shares > slabs / 8) shares = slabs / 8;
+      const uint64_t fit = OCH_GEMM_WORKSPACE / (rest * (uint64_t)tile * tile * 4);
+      if (shares > fit) shares = fit;
+      while (shares > 1 && ((slabs + shares - 1) / shares) * (shares - 1) >= slabs) shares--;      /* no empty share */
+      if (shares < 2) shares = 1;
+   }
+   if (rounds)
+   {  const double whole = (double)(slabs + 6), cut = (double)((slabs + shares - 1) / shares + 6) + 0.02 * whole;
+      *rounds = (double)(tiles / units) + (rest == 0 ? 0.0 : (shares > 1 ? cut / whole : 1.0));
+   }
+   return (int)shares;
 }
 
 /* 0: launched; 1: not a case for this kernel (the caller's other kernels take it). tile: 256 or 128; M and N multiples
@@ -275,8 +345,18 @@ int gemm_float_pipe(const GemmArgs &g, int tile)
    else { p.alpha_dev = (const float *)g.alpha; p.beta_dev = (const float *)g.beta; }
    p.batch = g.batch;
    p.tiles_m = (uint32_t)((g.M + tile - 1) / tile); p.tiles_n = (uint32_t)((g.N + tile - 1) / tile);
-   const uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
+   uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
    if (blocks > 0x7FFFFFFFull) return set_error("gemm: too many tiles");
+   if (tile != 256 && tile != 128) return 1;
+   const int shares = gemm_float_pipe_split(g, tile, nullptr);
+   uint32_t cut_tiles = 0;
+   if (shares > 1)
+   {  char *ws;
+      if (stream_gemm_workspace(g.stream, &ws) != 0) return -1;
+      cut_tiles = (uint32_t)(blocks % (uint64_t)gemm_compute_units());
+      p.split = (uint32_t)shares; p.split_first = (uint32_t)blocks - cut_tiles; p.partial = reinterpret_cast<float *>(ws);
+      blocks += (uint64_t)cut_tiles * (shares - 1);
+   }
    const bool akc = (g.transA != 'N'), bkc = (g.transB == 'N');
    const dim3 grid((unsigned)blocks, 1, g.nz), block(OCH_FP_THREADS);
 #define OCH_FP_LAUNCH(AK, BK, TS)                                                                                     \
@@ -285,13 +365,16 @@ int gemm_float_pipe(const GemmArgs &g, int tile)
         OCH_CHECK_HIP(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
         hipLaunchKernelGGL(kernel, grid, block, lds, g.stream, p); } while (0)
 #define OCH_FP_PICK(AK, BK) do { if (tile == 256) OCH_FP_LAUNCH(AK, BK, 4); else OCH_FP_LAUNCH(AK, BK, 2); } while (0)
-   if (tile != 256 && tile != 128) return 1;
    if (!akc && !bkc) OCH_FP_PICK(false, false);
    else if (!akc)    OCH_FP_PICK(false, true);
    else if (!bkc)    OCH_FP_PICK(true, false);
    else              OCH_FP_PICK(true, true);
 #undef OCH_FP_PICK
 #undef OCH_FP_LAUNCH
+   if (shares > 1)
+   {  if (tile == 256) hipLaunchKernelGGL(gemm_float_pipe_finish_kernel<4>, dim3(cut_tiles, 8), dim3(256), 0, g.stream, p);
+      else             hipLaunchKernelGGL(gemm_float_pipe_finish_kernel<2>, dim3(cut_tiles, 4), dim3(256), 0, g.stream, p);
+   }
    OCH_CHECK_LAUNCH();
    return 0;
 }

@@ -16,7 +16,13 @@ int gemm_double(const GemmArgs &g)
       {  const uint64_t tiles = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * (uint64_t)g.nz;
          return (double)((tiles + units - 1) / units) * (double)(bm * bn) / efficiency;
       };
-      const double large = cost(256, 128, 1.0), small = cost(128, 128, 0.9);
+      /* the pipelined kernel cuts the tiles of a last round that is at most half full along K: that round then counts as
+         1 / shares of a round */
+      GemmArgs whole = g;
+      whole.K = g.K - g.K % 16;
+      double rounds_large = 0, rounds_small = 0;
+      gemm_double_pipe_split(whole, 256, &rounds_large); gemm_double_pipe_split(whole, 128, &rounds_small);
+      const double large = rounds_large * 32768.0, small = rounds_small * 16384.0 / 0.95;
       const int forced = gemm_kernel_choice();
       const int tile_m = forced == 1 ? 256 : (forced == 2 ? 128 : (large <= small ? 256 : 128));
       if (forced != 3 && (forced != 0 || (tile_m == 256 ? large : small) < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87)))

@@ -249,6 +249,38 @@ def test_gemm_pipelined_kernels_against_the_oracle(hip, stream, dtype, choice):
         oh.check(oh.lib.och_gemm_set_kernel_choice(0))
 
 
+@pytest.mark.parametrize("choice,M,N", [(2, 2176, 2048), (2, 2180, 2052), (1, 4352, 4096)], ids=["small_tiles", "small_tiles_ragged", "large_tiles"])
+def test_gemm_float_last_round_cut_along_k(hip, stream, choice, M, N):
+    """When the last round of the compute units is at most half full (here 16 tiles, or 17 x 17 - 256 = 33, on 256 units) its
+    tiles are cut along K into shares of at least 8 slabs that fill the round; the shares are added in order by a second
+    kernel. 64 slabs give 8 shares of 8 (7 of 10 where 33 tiles are cut), 17 slabs two shares of 9 and 8; with beta, scalars in
+    host and device memory, a K with a remainder."""
+    if hip.device_properties(0).multiprocessor_count != 256:
+        pytest.skip("the sizes are chosen for 256 compute units")
+    rng = np.random.default_rng(1900 + choice + M)
+    oh.check(oh.lib.och_gemm_set_kernel_choice(choice))
+    try:
+        for ta, tb in (("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")):
+            check_large_product(stream, H.FLOAT, ta, tb, M, N, ((64, 2, -1, ta == "T"), (17, 1, 0, False), (20.25, -0.5, 1, False)), rng)
+    finally:
+        oh.check(oh.lib.och_gemm_set_kernel_choice(0))
+
+
+@pytest.mark.parametrize("choice,M,N", [(2, 2176, 2048), (2, 2178, 2050), (1, 4352, 2048)], ids=["small_tiles", "small_tiles_ragged", "large_tiles"])
+def test_gemm_double_last_round_cut_along_k(hip, stream, choice, M, N):
+    """The same for double: 16 tiles (ragged sizes: 18 x 17 - 256 = 50) in the last round of 256 compute units, cut into 8
+    (5) shares of the 64 slabs of 16 k, two shares of 17 slabs, a K with a remainder."""
+    if hip.device_properties(0).multiprocessor_count != 256:
+        pytest.skip("the sizes are chosen for 256 compute units")
+    rng = np.random.default_rng(2000 + choice + M)
+    oh.check(oh.lib.och_gemm_set_kernel_choice(choice))
+    try:
+        for ta, tb in (("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")):
+            check_large_product(stream, H.DOUBLE, ta, tb, M, N, ((64, 2, -1, ta == "T"), (17, 1, 0, False), (20.3125, -0.5, 1, False)), rng)
+    finally:
+        oh.check(oh.lib.och_gemm_set_kernel_choice(0))
+
+
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
 def test_gemm_float_pipelined_whole_tiles(hip, stream, ta, tb):
     """float products of 256 whole aligned 256 x 256 tiles or more run on the hand-pipelined kernel: one slab of 32 k
