@@ -596,9 +596,11 @@ int gemm_double(const GemmArgs &g);
 int gemm_double_pipe(const GemmArgs &g, int tile_m); /* tiles of 256 x 128 or 128 x 128; 1: not taken */
 int gemm_double_pipe_split(const GemmArgs &g, int tile_m, double *rounds); /* shares of the tiles of the last round; rounds of the compute units */
 int gemm_cfloat(const GemmArgs &g);
-int gemm_cfloat_pipe(const GemmArgs &g); /* whole aligned 128 x 128 tiles; 1: not taken */
+int gemm_cfloat_pipe(const GemmArgs &g); /* tiles of 128 x 128; 1: not taken */
+int gemm_cfloat_pipe_split(const GemmArgs &g, double *rounds);
 int gemm_cdouble(const GemmArgs &g);
 int gemm_cdouble_pipe(const GemmArgs &g); /* tiles of 128 x 64; 1: not taken */
+int gemm_cdouble_pipe_split(const GemmArgs &g, double *rounds);
 int gemm_half(const GemmArgs &g);      /* 1: not taken, use the generic kernel */
 int gemm_int8(const GemmArgs &g);      /* int8 and uint8; 1: not taken */
 int gemm_bool(const GemmArgs &g);      /* 1: not taken */

@@ -42,6 +42,12 @@ struct CFloatPipeParams
    const float *alpha_dev, *beta_dev;
    int      conjA, conjB;
    uint32_t tiles_m, tiles_n;
+   /* the tiles of the last, partly filled round of the compute units are cut along K: tiles from split_first on are
+      computed by `split` blocks each, block q of them (counted from the first such block) leaving the raw complex sums of
+      its share of the slabs in partial[q] (a dense tile, column-major); the finish kernel adds the shares in order and
+      applies alpha / beta. split <= 1: no tile is cut. Only without a batch. */
+   uint32_t split_first, split;
+   float *partial;
    GemmBatch batch;
 };
 
@@ -108,7 +114,10 @@ __global__ __launch_bounds__(OCH_CP_THREADS) void gemm_cfloat_pipe_kernel(const 
    int64_t oA, oB, oC, oAlpha, oBeta;
    gemm_batch_offsets(p.batch, oA, oB, oC, oAlpha, oBeta);
    const char *pA = p.A + oA, *pB = p.B + oB; char *pC = p.C + oC;
-   const uint32_t tile_m = blockIdx.x % p.tiles_m, tile_n = blockIdx.x / p.tiles_m;
+   uint32_t tile = blockIdx.x, share = 0, shares = 1, cut = 0;           /* cut: index of this block among those of cut tiles */
+   if (p.split > 1 && blockIdx.x >= p.split_first)
+   {  cut = blockIdx.x - p.split_first; tile = p.split_first + cut / p.split; share = cut % p.split; shares = p.split; }
+   const uint32_t tile_m = tile % p.tiles_m, tile_n = tile / p.tiles_m;
    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
    const uint32_t wm = (wave % 2) * WM, wn = (wave / 2) * WN;
@@ -123,7 +132,9 @@ __global__ __launch_bounds__(OCH_CP_THREADS) void gemm_cfloat_pipe_kernel(const 
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][a][r] = 0;
 
-   const uint32_t nslabs = p.K / KT, last = nslabs - 1;
+   /* this block's slabs: slab0 .. last of the product's K / KT (all of them unless the tile is cut) */
+   const uint32_t per_share = (p.K / KT + shares - 1) / shares, slab0 = share * per_share;
+   const uint32_t nslabs = slab0 + per_share <= p.K / KT ? per_share : p.K / KT - slab0, last = slab0 + nslabs - 1;
    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)lds;      /* where the array starts in LDS */
    const uint32_t rowsA = p.M - m0 < (uint32_t)BM ? p.M - m0 : (uint32_t)BM, rowsB = p.N - n0 < (uint32_t)BN ? p.N - n0 : (uint32_t)BN;    /* of this tile */
    uint32_t offA[8], offB[8], tgtA[8], tgtB[8];
@@ -164,7 +175,7 @@ __global__ __launch_bounds__(OCH_CP_THREADS) void gemm_cfloat_pipe_kernel(const 
    /* slab s in buffer CB: quad 0 carries the second half of the loads of slab s + 1 (into the other buffer), quad 3 the
       first half of the loads of slab s + 2 (into this one) */
 #define OCH_SLAB(s, CB)                                                                                                \
-   do { {  const uint32_t s1 = ((s) + 1 < last) ? (s) + 1 : last;                                                      \
+   do { {  const uint32_t s1 = (slab0 + (s) + 1 < last) ? slab0 + (s) + 1 : last;                                                      \
            const char *nextA = LA::slab_base(pA, p.ldA, m0, s1 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, s1 * KT);  \
            OCH_QUAD(0, 1, CB, 1, true, 8, 1 - CB);                                                                     \
         }                                                                                                              \
@@ -174,14 +185,14 @@ __global__ __launch_bounds__(OCH_CP_THREADS) void gemm_cfloat_pipe_kernel(const 
         }                                                                                                              \
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                               \
         __syncthreads();                                                                                               \
-        {  const uint32_t s2 = ((s) + 2 < last) ? (s) + 2 : last;                                                      \
+        {  const uint32_t s2 = (slab0 + (s) + 2 < last) ? slab0 + (s) + 2 : last;                                                      \
            const char *nextA = LA::slab_base(pA, p.ldA, m0, s2 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, s2 * KT);  \
            OCH_QUAD(1, 0, 1 - CB, 0, true, 0, CB);                                                                     \
         } } while (0)
 
    {  /* slab 0 and the first half of slab 1 */
-      const uint32_t s1 = (1 < last) ? 1 : last;
-      const char *nextA = LA::slab_base(pA, p.ldA, m0, 0), *nextB = LB::slab_base(pB, p.ldB, n0, 0);
+      const uint32_t s1 = (slab0 + 1 < last) ? slab0 + 1 : last;
+      const char *nextA = LA::slab_base(pA, p.ldA, m0, slab0 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, slab0 * KT);
 #pragma unroll
       for (int e = 0; e < 16; e++) OCH_LOAD(e, nextA, nextB, 0);
       nextA = LA::slab_base(pA, p.ldA, m0, s1 * KT); nextB = LB::slab_base(pB, p.ldB, n0, s1 * KT);
@@ -215,6 +226,14 @@ __global__ __launch_bounds__(OCH_CP_THREADS) void gemm_cfloat_pipe_kernel(const 
    if (p.alpha_dev) { const float *q = reinterpret_cast<const float *>(reinterpret_cast<const char *>(p.alpha_dev) + oAlpha); ar = q[0]; ai = q[1]; }
    if (p.beta_dev)  { const float *q = reinterpret_cast<const float *>(reinterpret_cast<const char *>(p.beta_dev) + oBeta); br = q[0]; bi = q[1]; }
    const float sq = (p.conjA != p.conjB) ? 1.0f : -1.0f, s1 = p.conjB ? -1.0f : 1.0f, s2 = p.conjA ? -1.0f : 1.0f;
+   /* a share of a cut tile leaves its raw sums, the whole tile, in the workspace */
+   char *out = pC + ((int64_t)m0 + (int64_t)n0 * p.ldC) * 8;
+   int64_t ldOut = p.ldC;
+   uint32_t rowsOut = rowsA, colsOut = rowsB;
+   if (shares > 1)
+   {  ar = 1; ai = 0; br = 0; bi = 0;
+      out = reinterpret_cast<char *>(p.partial + (size_t)cut * BM * BN * 2); ldOut = BM; rowsOut = BM; colsOut = BN;
+   }
    constexpr int CP = BM + 2, CPASS = 32, PASSES = BN / CPASS;
    static_assert(CPASS * CP * 8 <= 2 * BUF, "a pass of the staged tile does not fit into the slab buffers");
    float2 *stage = reinterpret_cast<float2 *>(lds);
@@ -233,12 +252,11 @@ __global__ __launch_bounds__(OCH_CP_THREADS) void gemm_cfloat_pipe_kernel(const 
             }
       }
       __syncthreads();
-      const uint32_t c0 = n0 + h * CPASS;
       for (uint32_t q = threadIdx.x; q < CPASS * (BM / 2); q += THREADS)
       {  const uint32_t c = q / (BM / 2), r2 = (q % (BM / 2)) * 2;
-         if (r2 >= rowsA || h * CPASS + c >= rowsB) continue;          /* outside C */
+         if (r2 >= rowsOut || h * CPASS + c >= colsOut) continue;      /* outside C */
          och_f32x4 v = *reinterpret_cast<const och_f32x4 *>(stage + c * CP + r2);
-         och_f32x4 *dst = reinterpret_cast<och_f32x4 *>(pC + ((int64_t)(m0 + r2) + (int64_t)(c0 + c) * p.ldC) * 8);
+         och_f32x4 *dst = reinterpret_cast<och_f32x4 *>(out + ((int64_t)r2 + (int64_t)(h * CPASS + c) * ldOut) * 8);
          if (br != 0 || bi != 0)
          {  const och_f32x4 old = *dst;
             v.x += br * old.x - bi * old.y; v.y += br * old.y + bi * old.x;
@@ -248,6 +266,58 @@ __global__ __launch_bounds__(OCH_CP_THREADS) void gemm_cfloat_pipe_kernel(const 
       }
       __syncthreads();
    }
+}
+
+/* The shares of the cut tiles, added in the order of their slabs, times alpha, plus beta * C: a block per 16 columns of a
+   cut tile (grid y), one element of C per thread and trip. */
+__global__ __launch_bounds__(256) void gemm_cfloat_pipe_finish_kernel(const CFloatPipeParams p)
+{
+   constexpr uint32_t BM = 128, BN = 128;
+   const uint32_t tile = p.split_first + blockIdx.x, tile_m = tile % p.tiles_m, tile_n = tile / p.tiles_m;
+   const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+   const uint32_t rows = p.M - m0 < BM ? p.M - m0 : BM, cols = p.N - n0 < BN ? p.N - n0 : BN;
+   const float ar = p.alpha_dev ? p.alpha_dev[0] : p.alpha[0], ai = p.alpha_dev ? p.alpha_dev[1] : p.alpha[1];
+   const float br = p.beta_dev ? p.beta_dev[0] : p.beta[0], bi = p.beta_dev ? p.beta_dev[1] : p.beta[1];
+   const float *shares = p.partial + (size_t)blockIdx.x * p.split * BM * BN * 2;
+   for (uint32_t q = threadIdx.x; q < 16 * BM; q += 256)
+   {  const uint32_t c = blockIdx.y * 16 + q / BM, r = q % BM;
+      if (r >= rows || c >= cols) continue;
+      float sr = 0, si = 0;
+      for (uint32_t t = 0; t < p.split; t++)
+      {  const float *w = shares + ((size_t)t * BM * BN + (size_t)c * BM + r) * 2;
+         sr += w[0]; si += w[1];
+      }
+      float vr = ar * sr - ai * si, vi = ar * si + ai * sr;
+      float *dst = reinterpret_cast<float *>(p.C + ((int64_t)(m0 + r) + (int64_t)(n0 + c) * p.ldC) * 8);
+      if (br != 0 || bi != 0) { const float cr = dst[0], ci = dst[1]; vr += br * cr - bi * ci; vi += br * ci + bi * cr; }
+      dst[0] = vr; dst[1] = vi;
+   }
+}
+
+/* Into how many shares the tiles of the last round are cut (1: not at all): the round must be at most half full, every
+   share at least 8 slabs long, and all shares must fit into the stream's workspace. *rounds: the rounds of the compute
+   units the product then takes (for the cost model of the caller); the cut round counts as the length of a share plus
+   what every block spends outside its main loop (about 6 slabs' worth) over the length of a whole tile. */
+int gemm_cfloat_pipe_split(const GemmArgs &g, double *rounds)
+{
+   const uint64_t units = (uint64_t)gemm_compute_units();
+   const uint64_t tiles = ((g.M + 128 - 1) / 128) * ((g.N + 128 - 1) / 128) * (uint64_t)g.nz;
+   const uint64_t rest = tiles % units, slabs = g.K / 32;
+   uint64_t shares = 1;
+   if (g.batch.nb == 0 && g.nz == 1 && rest > 0 && rest * 2 <= units && slabs >= 16)
+   {  shares = units / rest;
+      if (shares > 8) shares = 8;
+      if (shares > slabs / 8) shares = slabs / 8;
+      const uint64_t fit = OCH_GEMM_WORKSPACE / (rest * (uint64_t)128 * 128 * 8);
+      if (shares > fit) shares = fit;
+      while (shares > 1 && ((slabs + shares - 1) / shares) * (shares - 1) >= slabs) shares--;      /* no empty share */
+      if (shares < 2) shares = 1;
+   }
+   if (rounds)
+   {  const double whole = (double)(slabs + 6), cut = (double)((slabs + shares - 1) / shares + 6) + 0.02 * whole;
+      *rounds = (double)(tiles / units) + (rest == 0 ? 0.0 : (shares > 1 ? cut / whole : 1.0));
+   }
+   return (int)shares;
 }
 
 /* 0: launched; 1: not a case for this kernel (the caller's other kernels take it) */
@@ -266,8 +336,17 @@ int gemm_cfloat_pipe(const GemmArgs &g)
    p.batch = g.batch;
    p.conjA = (g.transA == 'C'); p.conjB = (g.transB == 'C');
    p.tiles_m = (uint32_t)((g.M + OCH_CP_BM - 1) / OCH_CP_BM); p.tiles_n = (uint32_t)((g.N + OCH_CP_BM - 1) / OCH_CP_BM);
-   const uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
+   uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
    if (blocks > 0x7FFFFFFFull) return set_error("gemm: too many tiles");
+   const int shares = gemm_cfloat_pipe_split(g, nullptr);
+   uint32_t cut_tiles = 0;
+   if (shares > 1)
+   {  char *ws;
+      if (stream_gemm_workspace(g.stream, &ws) != 0) return -1;
+      cut_tiles = (uint32_t)(blocks % (uint64_t)gemm_compute_units());
+      p.split = (uint32_t)shares; p.split_first = (uint32_t)blocks - cut_tiles; p.partial = reinterpret_cast<float *>(ws);
+      blocks += (uint64_t)cut_tiles * (shares - 1);
+   }
    const bool akc = (g.transA != 'N'), bkc = (g.transB == 'N');
    const dim3 grid((unsigned)blocks, 1, g.nz), block(OCH_CP_THREADS);
    const size_t lds = 2 * (size_t)OCH_CP_BUFFER;
@@ -280,6 +359,7 @@ int gemm_cfloat_pipe(const GemmArgs &g)
    else if (!bkc)    OCH_CP_LAUNCH(true, false);
    else              OCH_CP_LAUNCH(true, true);
 #undef OCH_CP_LAUNCH
+   if (shares > 1) hipLaunchKernelGGL(gemm_cfloat_pipe_finish_kernel, dim3(cut_tiles, 8), dim3(256), 0, g.stream, p);
    OCH_CHECK_LAUNCH();
    return 0;
 }

@@ -14,8 +14,15 @@ int gemm_cdouble(const GemmArgs &g)
       {  const uint64_t tiles = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * (uint64_t)g.nz;
          return (double)((tiles + units - 1) / units) * (double)(bm * bn) / efficiency;
       };
+      /* the pipelined kernel cuts the tiles of a last round that is at most half full along K: that round then counts as
+         a fraction of a round */
+      GemmArgs whole = g;
+      whole.K = g.K - g.K % 16;
+      double rounds = 0;
+      gemm_cdouble_pipe_split(whole, &rounds);
+      const double pipelined = rounds * 8192.0;
       const int forced = gemm_kernel_choice();
-      if (forced != 3 && (forced != 0 || cost(128, 64, 1.0) < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87)))
+      if (forced != 3 && (forced != 0 || pipelined < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87)))
       {  GemmArgs part = g;
          const size_t Kh = g.K - g.K % 16;
          part.K = Kh;

@@ -281,6 +281,22 @@ def test_gemm_double_last_round_cut_along_k(hip, stream, choice, M, N):
         oh.check(oh.lib.och_gemm_set_kernel_choice(0))
 
 
+@pytest.mark.parametrize("dtype,M,N", [(H.CFLOAT, 2176, 2048), (H.CFLOAT, 2178, 2050), (H.CDOUBLE, 2176, 1024), (H.CDOUBLE, 2177, 1025)],
+                         ids=["cfloat", "cfloat_ragged", "cdouble", "cdouble_ragged"])
+def test_gemm_complex_last_round_cut_along_k(hip, stream, dtype, M, N):
+    """The same for the complex types: the shares hold the complex sums before alpha (the four real accumulators already
+    combined with the signs of the conjugations); complex alpha and beta are applied once, by the kernel that adds the shares."""
+    if hip.device_properties(0).multiprocessor_count != 256:
+        pytest.skip("the sizes are chosen for 256 compute units")
+    rng = np.random.default_rng(2100 + dtype + M)
+    oh.check(oh.lib.och_gemm_set_kernel_choice(1))
+    try:
+        for ta, tb in (("N", "N"), ("T", "N"), ("N", "C"), ("C", "T")):
+            check_large_product(stream, dtype, ta, tb, M, N, ((64, 2 - 1j, -1 + 0.5j, ta == "T"), (17, 1, 0, False), (20.25, -0.5j, 1, False)), rng)
+    finally:
+        oh.check(oh.lib.och_gemm_set_kernel_choice(0))
+
+
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("T", "N"), ("N", "T"), ("T", "T")])
 def test_gemm_float_pipelined_whole_tiles(hip, stream, ta, tb):
     """float products of 256 whole aligned 256 x 256 tiles or more run on the hand-pipelined kernel: one slab of 32 k
