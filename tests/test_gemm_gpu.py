@@ -549,11 +549,37 @@ def test_gemm_batched_equals_loop(hip, stream, case):
     """och_gemm_batched (the reference's loop over the dimensions beyond the second, tensor_blas_gpu.c:171-252, as one
     launch) gives bit for bit what one och_gemm per product gives (those are held to the oracle above); integer
     results are also compared with the oracle directly."""
+    run_batched(stream, case, (2, 1, 3))
+
+
+PIPELINED_BATCH_CASES = [  # as above; aligned operands, sizes the pipelined kernels take when they are asked to
+    (H.FLOAT, "N", "T", 260, 132, 96, (3,), False, True),
+    (H.FLOAT, "T", "N", 128, 384, 64, (2, 2), True, False),
+    (H.DOUBLE, "N", "N", 258, 130, 48, (3,), False, True),
+    (H.DOUBLE, "T", "T", 384, 128, 32, (2,), False, "host"),
+    (H.CFLOAT, "C", "N", 130, 258, 64, (3,), True, True),
+    (H.CDOUBLE, "N", "C", 129, 67, 48, (2, 2), False, True),
+]
+
+
+@pytest.mark.parametrize("choice", [1, 2], ids=["large_tile", "small_tile"])
+@pytest.mark.parametrize("case", PIPELINED_BATCH_CASES, ids=lambda c: "%s-%s%s-%dx%dx%d-b%s" % (H.NAMES[c[0]], c[1], c[2], c[3], c[4], c[5], "x".join(map(str, c[6]))))
+def test_gemm_batched_on_the_pipelined_kernels(hip, stream, case, choice):
+    """The batch in grid z of the pipelined kernels (operand, scalar and result offsets per product; ragged last tiles):
+    bit for bit what one product at a time gives with the same kernel, which is held to the oracle above."""
+    oh.check(oh.lib.och_gemm_set_kernel_choice(choice))
+    try:
+        run_batched(stream, case, (4, 4, 4))
+    finally:
+        oh.check(oh.lib.och_gemm_set_kernel_choice(0))
+
+
+def run_batched(stream, case, pads):
     dtype, ta, tb, M, N, K, bsize, share_b, scalars = case
     rng = np.random.default_rng(99 + dtype + M)
     rowsA, colsA = (M, K) if ta == "N" else (K, M)
     rowsB, colsB = (K, N) if tb == "N" else (N, K)
-    ldA, ldB, ldC = rowsA + 2, rowsB + 1, M + 3
+    ldA, ldB, ldC = rowsA + pads[0], rowsB + pads[1], M + pads[2]
     total = int(np.prod(bsize))
     item = np.dtype(H.storage(dtype)).itemsize
     A = H.random_data(dtype, ldA * colsA * total, rng, "small")
