@@ -560,6 +560,7 @@ static int launch_gemm_mfma(const GemmArgs &g)
 /* Compute units of the current device (cached per device). */
 int gemm_compute_units(void);
 int gemm_kernel_choice(void);            /* 0 automatic; 1 / 2: pipelined kernel, large / small tile; 3: never pipelined */
+int gemm_pad_tail(const GemmArgs &g, size_t Kh, int slab, int es, GemmArgs *tail);   /* the rest of K as one zero-padded slab in the workspace */
 
 /* Which block tile to use. The compute units work through the tiles in rounds, and the last round is as long as the others
    however few tiles it holds: 3000^3 double is 576 tiles of 128 x 128, i.e. 2.25 rounds on 256 units, and ran at 39

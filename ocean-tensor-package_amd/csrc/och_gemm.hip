@@ -116,6 +116,51 @@ template <class T> static int gemm_generic(const GemmArgs &g)
    return 0;
 }
 
+/* dst (d0 x d1, dense, column-major) <- the v0 x v1 corner of src (leading dimension ld), zero elsewhere; elements of
+   sizeof(E) bytes */
+template <class E>
+__global__ __launch_bounds__(256) void gemm_pad_kernel(E *dst, const E *src, uint32_t d0, uint64_t total, uint32_t v0, uint32_t v1, int64_t ld)
+{
+   const uint64_t e = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+   if (e >= total) return;
+   const uint32_t j = (uint32_t)(e / d0), i = (uint32_t)(e - (uint64_t)j * d0);
+   E v = E();
+   if (i < v0 && j < v1) v = src[i + (int64_t)j * ld];
+   dst[e] = v;
+}
+
+/* The last K - Kh (< slab) of the inner dimension as a product of one whole slab: both operands' tails are copied into
+   the stream's workspace and filled up with zeros to `slab` k (the pipelined kernels take whole slabs only), laid out as
+   the operands themselves are, so that *tail = g with A, B, their leading dimensions and K replaced multiplies them with
+   the same transposition flags. es: bytes per element. 0: done; 1: the copies do not fit into the workspace. */
+int gemm_pad_tail(const GemmArgs &g, size_t Kh, int slab, int es, GemmArgs *tail)
+{
+   const size_t kt = g.K - Kh;
+   const size_t bytesA = g.M * (size_t)slab * es, bytesB = g.N * (size_t)slab * es;
+   if (g.batch.nb != 0 || g.nz != 1 || bytesA + bytesB > OCH_GEMM_WORKSPACE) return 1;
+   char *ws;
+   if (stream_gemm_workspace(g.stream, &ws) != 0) return -1;
+   *tail = g;
+   tail->K = (size_t)slab;
+   for (int operand = 0; operand < 2; operand++)
+   {  /* rows contiguous (A not transposed, B transposed): rows x slab, the tail's columns first; k contiguous: slab x rows */
+      const bool rows_contiguous = operand == 0 ? (g.transA == 'N') : (g.transB != 'N');
+      const size_t rows = operand == 0 ? g.M : g.N;
+      const ptrdiff_t ld = operand == 0 ? g.ldA : g.ldB;
+      const char *src = (const char *)(operand == 0 ? g.A : g.B) + (int64_t)Kh * (rows_contiguous ? (int64_t)ld : 1) * es;
+      char *dst = ws + (operand == 0 ? 0 : bytesA);
+      const uint32_t d0 = (uint32_t)(rows_contiguous ? rows : (size_t)slab), v0 = (uint32_t)(rows_contiguous ? rows : kt), v1 = (uint32_t)(rows_contiguous ? kt : rows);
+      const uint64_t total = (uint64_t)rows * slab;
+      const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+      if (es == 4)      hipLaunchKernelGGL(gemm_pad_kernel<uint32_t>, grid, block, 0, g.stream, (uint32_t *)dst, (const uint32_t *)src, d0, total, v0, v1, (int64_t)ld);
+      else if (es == 8) hipLaunchKernelGGL(gemm_pad_kernel<uint64_t>, grid, block, 0, g.stream, (uint64_t *)dst, (const uint64_t *)src, d0, total, v0, v1, (int64_t)ld);
+      else              hipLaunchKernelGGL(gemm_pad_kernel<uint4>, grid, block, 0, g.stream, (uint4 *)dst, (const uint4 *)src, d0, total, v0, v1, (int64_t)ld);
+      if (operand == 0) { tail->A = dst; tail->ldA = (ptrdiff_t)d0; } else { tail->B = dst; tail->ldB = (ptrdiff_t)d0; }
+   }
+   OCH_CHECK_LAUNCH();
+   return 0;
+}
+
 /* 0: the cost model chooses; 1: the pipelined kernel on its large tile wherever it applies; 2: on its small tile (float,
    double); 3: never the pipelined kernel. For tests and measurements (och_gemm_set_kernel_choice). */
 static int g_gemm_kernel_choice = 0;

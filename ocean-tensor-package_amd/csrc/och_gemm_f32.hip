@@ -36,6 +36,17 @@ int gemm_float(const GemmArgs &g)
          if (taken == 0)
          {  if (g.K > Kh)
             {  static const float one = 1.0f;
+               /* the rest of K, filled up with zeros to one slab in the workspace, on the pipelined kernel again; where
+                  that does not fit, on the kernels below */
+               GemmArgs tail;
+               const int padded = gemm_pad_tail(g, Kh, 32, 4, &tail);
+               if (padded < 0) return -1;
+               if (padded == 0)
+               {  tail.beta = &one;
+                  const int again = gemm_float_pipe(tail, tile);
+                  if (again < 0) return -1;
+                  if (again == 0) return 0;
+               }
                part.K = g.K - Kh; part.beta = &one;
                part.A = (const char *)g.A + (int64_t)Kh * (g.transA == 'N' ? (int64_t)g.ldA : 1) * 4;
                part.B = (const char *)g.B + (int64_t)Kh * (g.transB == 'N' ? 1 : (int64_t)g.ldB) * 4;
