@@ -27,6 +27,11 @@
  *   - the loop body has no branches: slab numbers past the end are clamped (the last slab is loaded again into a buffer
  *     nobody reads); it is written out twice so that all LDS offsets are immediates.
  *   - C leaves through LDS in passes of 64 columns, so that memory sees 16-byte accesses along the columns of C.
+ *   - the last tiles of a matrix whose size is not a multiple of the tile: lanes whose rows do not exist load the last
+ *     rows that do (every load stays inside the matrix, the loop is unchanged), and what lies outside C is not written.
+ *   - the compute units work through the tiles in rounds, and a last round of a few tiles would take as long as a full
+ *     one: when it is at most half full its tiles are cut along K into shares that fill it, each share leaves its raw sums
+ *     in the stream's workspace, and gemm_float_pipe_finish_kernel adds them in slab order and applies alpha and beta.
  */
 #include "och_gemm.h"
 #pragma clang diagnostic ignored "-Winline-asm"
