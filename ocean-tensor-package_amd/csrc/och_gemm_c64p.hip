@@ -312,7 +312,7 @@ __global__ __launch_bounds__(256) void gemm_cdouble_pipe_finish_kernel(const CDo
 }
 
 /* Into how many shares the tiles of the last round are cut (1: not at all): the round must be at most half full, every
-   share at least 8 slabs long, and all shares must fit into the stream's workspace. *rounds: the rounds of the compute
+   share at least 8 slabs long, at most 8 shares per tile (64 when the whole product is less than one round), and all shares must fit into the stream's workspace. *rounds: the rounds of the compute
    units the product then takes (for the cost model of the caller); the cut round counts as the length of a share plus
    what every block spends outside its main loop (about 6 slabs' worth) over the length of a whole tile. */
 int gemm_cdouble_pipe_split(const GemmArgs &g, double *rounds)
@@ -323,12 +323,12 @@ int gemm_cdouble_pipe_split(const GemmArgs &g, double *rounds)
    uint64_t shares = 1;
    if (g.batch.nb == 0 && g.nz == 1 && rest > 0 && rest * 2 <= units && slabs >= 16)
    {  shares = units / rest;
-      if (shares > 8) shares = 8;
+      if (shares > (tiles < units ? 64 : 8)) shares = tiles < units ? 64 : 8;       /* 64: a product of a few tiles and a long K */
       if (shares > slabs / 8) shares = slabs / 8;
       const uint64_t fit = OCH_GEMM_WORKSPACE / (rest * (uint64_t)128 * 64 * 16);
       if (shares > fit) shares = fit;
       while (shares > 1 && ((slabs + shares - 1) / shares) * (shares - 1) >= slabs) shares--;      /* no empty share */
-      if (shares < 2) shares = 1;
+      if (shares < 2 || rest * shares * 2 < units) shares = 1;      /* ... nor a cut that leaves most compute units idle */
    }
    if (rounds)
    {  const double whole = (double)(slabs + 6), cut = (double)((slabs + shares - 1) / shares + 6) + 0.02 * whole;

@@ -249,12 +249,14 @@ def test_gemm_pipelined_kernels_against_the_oracle(hip, stream, dtype, choice):
         oh.check(oh.lib.och_gemm_set_kernel_choice(0))
 
 
-@pytest.mark.parametrize("choice,M,N", [(2, 2176, 2048), (2, 2180, 2052), (1, 4352, 4096)], ids=["small_tiles", "small_tiles_ragged", "large_tiles"])
+@pytest.mark.parametrize("choice,M,N", [(2, 2176, 2048), (2, 2180, 2052), (1, 4352, 4096), (2, 2560, 2048)],
+                         ids=["small_tiles", "small_tiles_ragged", "large_tiles", "small_tiles_quarter_round"])
 def test_gemm_float_last_round_cut_along_k(hip, stream, choice, M, N):
     """When the last round of the compute units is at most half full (here 16 tiles, or 17 x 17 - 256 = 33, on 256 units) its
     tiles are cut along K into shares of at least 8 slabs that fill the round; the shares are added in order by a second
-    kernel. 64 slabs give 8 shares of 8 (7 of 10 where 33 tiles are cut), 17 slabs two shares of 9 and 8; with beta, scalars in
-    host and device memory, a K with a remainder."""
+    kernel. 64 slabs give 8 shares of 8 (7 of 10 where 33 tiles are cut, 4 of 16 where 64 are); 17 slabs give two shares of
+    9 and 8 where 64 tiles are cut and none where 16 are (two shares would leave most compute units idle); with beta, scalars
+    in host and device memory, a K with a remainder."""
     if hip.device_properties(0).multiprocessor_count != 256:
         pytest.skip("the sizes are chosen for 256 compute units")
     rng = np.random.default_rng(1900 + choice + M)
@@ -266,7 +268,8 @@ def test_gemm_float_last_round_cut_along_k(hip, stream, choice, M, N):
         oh.check(oh.lib.och_gemm_set_kernel_choice(0))
 
 
-@pytest.mark.parametrize("choice,M,N", [(2, 2176, 2048), (2, 2178, 2050), (1, 4352, 2048)], ids=["small_tiles", "small_tiles_ragged", "large_tiles"])
+@pytest.mark.parametrize("choice,M,N", [(2, 2176, 2048), (2, 2178, 2050), (1, 4352, 2048), (2, 2560, 2048)],
+                         ids=["small_tiles", "small_tiles_ragged", "large_tiles", "small_tiles_quarter_round"])
 def test_gemm_double_last_round_cut_along_k(hip, stream, choice, M, N):
     """The same for double: 16 tiles (ragged sizes: 18 x 17 - 256 = 50) in the last round of 256 compute units, cut into 8
     (5) shares of the 64 slabs of 16 k, two shares of 17 slabs, a K with a remainder."""
