@@ -150,6 +150,66 @@ def test_graph_with_half_gemm_split_k_projection_and_gather(hip, stream):
         b.free()
 
 
+def test_graph_with_pipelined_gemm(hip, stream):
+    """The pipelined float and double kernels in a recorded sequence: more than 64 KB of LDS, loads straight to LDS, and (for
+    the float product, 320 tiles on 256 compute units) the last round cut along K with its shares in the stream's workspace
+    and the kernel that adds them. Every replay equals the eager run of the same number, bit for bit; C accumulates
+    (beta = 1), so the runs differ."""
+    if hip.device_properties(0).multiprocessor_count != 256:
+        pytest.skip("the sizes are chosen for 256 compute units")
+    lib, h = oh.lib, stream.handle
+    rng = np.random.default_rng(41)
+    M, N, K = 2560, 2048, 17 * 32
+    a32, b32 = rng.uniform(-1, 1, M * K).astype(np.float32), rng.uniform(-1, 1, K * N).astype(np.float32)
+    a64, b64 = rng.uniform(-1, 1, 384 * 64), rng.uniform(-1, 1, 64 * 258)
+    dA, dB, dC = oh.to_device(a32, stream), oh.to_device(b32, stream), oh.DeviceBuffer(4 * M * N, stream)
+    eA, eB, eC = oh.to_device(a64, stream), oh.to_device(b64, stream), oh.DeviceBuffer(8 * 384 * 258, stream)
+    half32, one32, half64, one64 = np.float32([0.5]), np.float32([1.0]), np.float64([0.5]), np.float64([1.0])
+    p = lambda x: x.ctypes.data_as(C.c_void_p)
+
+    def sequence():
+        oh.check(lib.och_gemm(H.FLOAT, b"N", b"N", M, N, K, p(half32), dA.ptr, M, dB.ptr, K, p(one32), dC.ptr, M, 1, h))
+        oh.check(lib.och_gemm(H.DOUBLE, b"T", b"N", 384, 258, 64, p(half64), eA.ptr, 64, eB.ptr, 64, p(one64), eC.ptr, 384, 1, h))
+
+    def snapshot():
+        stream.synchronize()
+        return [dC.download(np.uint8).copy(), eC.download(np.uint8).copy()]
+
+    def reset():
+        for b in (dC, eC):
+            oh.check(lib.och_memset_async(b.ptr, 0, b.nbytes, h))
+        stream.synchronize()
+
+    oh.check(lib.och_gemm_set_kernel_choice(2))
+    try:
+        reset()
+        eager = []
+        for _ in range(3):
+            sequence()
+            eager.append(snapshot())
+        assert not np.array_equal(eager[0][0], eager[1][0])
+        # the float product against numpy, to a float bound
+        want = 0.5 * (a32.reshape(K, M).T.astype(np.float64) @ b32.reshape(N, K).T.astype(np.float64))
+        got = eager[0][0].view(np.float32).reshape(N, M).T
+        assert np.abs(got - want).max() <= 1e-5 * K
+        reset()
+        oh.check(lib.och_stream_begin_capture(h))
+        sequence()
+        graph = C.c_void_p()
+        oh.check(lib.och_stream_end_capture(h, C.byref(graph)))
+        assert not eC.download(np.uint8).any()                                      # recording executed nothing
+        for k in range(3):
+            oh.check(lib.och_graph_launch(graph, h))
+            got = snapshot()
+            assert np.array_equal(got[0], eager[k][0]) and np.array_equal(got[1], eager[k][1]), "replay %d differs from the eager run" % k
+            stream.synchronize()
+        oh.check(lib.och_graph_destroy(graph))
+    finally:
+        oh.check(lib.och_gemm_set_kernel_choice(0))
+    for b in (dA, dB, dC, eA, eB, eC):
+        b.free()
+
+
 def test_first_error_is_kept_until_it_is_checked(hip, stream):
     """The status protocol of src/core/gpu/cuda.c:84-120: the first failing runtime call is remembered, later ones do not
     replace it, och_status_check reports it once and forgets it. The failures are host-side argument errors."""
