@@ -17,14 +17,17 @@ int gemm_float(const GemmArgs &g)
       {  const uint64_t tiles = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * (uint64_t)g.nz;
          return (double)((tiles + units - 1) / units) * (double)(bm * bn) / efficiency;
       };
-      const double others = cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.8);
       /* the pipelined kernel cuts the tiles of a last round that is at most half full along K: that round then counts as
          1 / shares of a round */
       GemmArgs whole = g;
       whole.K = g.K - g.K % 32;
       double rounds_large = 0, rounds_small = 0;
       gemm_float_pipe_split(whole, 256, &rounds_large); gemm_float_pipe_split(whole, 128, &rounds_small);
-      const double large = rounds_large * 65536.0, small = rounds_small * 16384.0 / 0.95;
+      /* what a block spends outside its main loop, in slabs of 32 k: about three on the large tile and in the kernels
+         below, two on the small tile (8192 x 8192 x 256: 109, 93 and 118 TFLOP/s) */
+      const double slabs = (double)(whole.K / 32);
+      const double large = rounds_large * 65536.0 * (slabs + 3) / slabs, small = rounds_small * 16384.0 / 0.95 * (slabs + 2) / slabs;
+      const double others = cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.8) * (slabs + 3) / slabs;
       const int forced = gemm_kernel_choice();
       const int tile = forced == 1 ? 256 : (forced == 2 ? 128 : (large <= small ? 256 : 128));
       if (forced != 3 && (forced != 0 || (tile == 256 ? large : small) < others))

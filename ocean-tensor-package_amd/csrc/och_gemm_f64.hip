@@ -22,10 +22,13 @@ int gemm_double(const GemmArgs &g)
       whole.K = g.K - g.K % 16;
       double rounds_large = 0, rounds_small = 0;
       gemm_double_pipe_split(whole, 256, &rounds_large); gemm_double_pipe_split(whole, 128, &rounds_small);
-      const double large = rounds_large * 32768.0, small = rounds_small * 16384.0 / 0.95;
+      /* what a block spends outside its main loop, in slabs of 16 k: about three on the large tile, two on the small one,
+         four in the kernels below */
+      const double slabs = (double)(whole.K / 16);
+      const double large = rounds_large * 32768.0 * (slabs + 3) / slabs, small = rounds_small * 16384.0 / 0.95 * (slabs + 2) / slabs;
       const int forced = gemm_kernel_choice();
       const int tile_m = forced == 1 ? 256 : (forced == 2 ? 128 : (large <= small ? 256 : 128));
-      if (forced != 3 && (forced != 0 || (tile_m == 256 ? large : small) < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87)))
+      if (forced != 3 && (forced != 0 || (tile_m == 256 ? large : small) < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87) * (slabs + 4) / slabs))
       {  GemmArgs part = g;
          const size_t Kh = g.K - g.K % 16;
          part.K = Kh;
