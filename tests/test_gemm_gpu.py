@@ -657,3 +657,22 @@ def test_gemm_with_few_tiles_and_long_k(hip, stream, dtype):
         for ta, tb in (("N", "N"), ("T", "N"), ("N", "T"), ("C" if cplx else "T", "C" if cplx else "T")):
             alpha, beta = ((2 - 1j, -1 + 0.5j) if cplx else (2, -1)) if (M + len(ta)) % 2 else (1, 0)
             run_case(stream, dtype, ta, tb, M, N, K, alpha, beta, rng, device_scalars=(K % 2 == 0), pad=3 if (K % 2) else 0)
+
+
+@pytest.mark.parametrize("dtype", [H.FLOAT, H.DOUBLE, H.CFLOAT, H.CDOUBLE], ids=lambda d: H.NAMES[d])
+def test_gemm_seeded_shapes_under_the_automatic_choice(hip, stream, dtype):
+    """Shapes drawn from a fixed seed, left to the library's own choice of kernel: M and N from 128 to 1500 (even, mostly
+    multiples of 4, some odd), K from one slab to 6000 with and without a remainder, every mode pair, aligned and unaligned
+    leading dimensions, alpha / beta trivial or not, scalars in host or device memory. Whatever the model picks -- large or
+    small pipelined tile, last round cut along K, padded rest of K, tiled kernel -- the result is held to the same bound."""
+    rng = np.random.default_rng(4200 + dtype)
+    cplx = dtype in H.COMPLEX_TYPES
+    slab = 16 if dtype in (H.DOUBLE, H.CDOUBLE) else 32
+    modes = ["N", "T"] + (["C"] if cplx else [])
+    for n in range(32):
+        step = (4, 4, 2, 1)[n % 4]
+        M, N = (int(rng.integers(128 // step, 1500 // step)) * step for _ in range(2))
+        K = int(rng.integers(1, 6000 // slab)) * slab + (int(rng.integers(1, slab)) if n % 3 == 1 else 0)
+        ta, tb = modes[int(rng.integers(len(modes)))], modes[int(rng.integers(len(modes)))]
+        alpha, beta = ((2 - 1j, -1 + 0.5j) if cplx else (2, -1)) if n % 2 else (1, 0)
+        check_large_product(stream, dtype, ta, tb, M, N, [(K / slab, alpha, beta, n % 5 == 4)], rng, pad=(0, 4, 0, 3)[(n // 4) % 4])
