@@ -398,6 +398,12 @@ int och_gemm_batched(int dtype, char transA, char transB, size_t M, size_t N, si
 /* the slab, 16-byte aligned operands), 2 the pipelined kernel on its small tile (float, double; complex float has    */
 /* one tile), 3 never the pipelined kernel. Process-wide; no counterpart in the reference.                            */
 int och_gemm_set_kernel_choice(int choice);
+/* The pipelined kernels' plan for the last round of the compute units, host arithmetic only (no device is touched):   */
+/* a product of ceil(M / tile_m) x ceil(N / tile_n) block tiles on `units` compute units, K in slabs of `slab`, every   */
+/* element of C elem_size bytes. Returns into how many shares along K each tile of the last round is cut (1: no cut)   */
+/* and, in *rounds (may be null), the cost of the product in rounds of whole tiles. No counterpart in the reference.   */
+int och_gemm_split_plan(size_t M, size_t N, size_t K, unsigned tile_m, unsigned tile_n, unsigned slab, unsigned elem_size,
+                        unsigned units, double *rounds);
 
 /* Fused projection step of a modified Gram-Schmidt sweep. No counterpart in the reference, whose callers issue one    */
 /* dot product (gemm with M = N = 1) and one rank-1 update per pair of columns, i.e. 2 k launches for this:             */

@@ -560,6 +560,8 @@ static int launch_gemm_mfma(const GemmArgs &g)
 /* Compute units of the current device (cached per device). */
 int gemm_compute_units(void);
 int gemm_kernel_choice(void);            /* 0 automatic; 1 / 2: pipelined kernel, large / small tile; 3: never pipelined */
+int gemm_pipe_split_plan(uint64_t M, uint64_t N, uint64_t K, uint64_t batch, bool single, uint32_t tile_m, uint32_t tile_n,
+                         uint32_t slab, uint32_t elem_size, uint64_t units, double *rounds);   /* shares of the tiles of the last round */
 int gemm_pad_tail(const GemmArgs &g, size_t Kh, int slab, int es, GemmArgs *tail);   /* the rest of K as one zero-padded slab in the workspace */
 
 /* Which block tile to use. The compute units work through the tiles in rounds, and the last round is as long as the others

@@ -166,6 +166,36 @@ int gemm_pad_tail(const GemmArgs &g, size_t Kh, int slab, int es, GemmArgs *tail
 static int g_gemm_kernel_choice = 0;
 int gemm_kernel_choice(void) { return g_gemm_kernel_choice; }
 
+/* The last round of a pipelined product. `units` compute units work through tiles x batch block tiles in rounds, and
+   a last round of `rest` tiles takes as long as a full one. When it is at most half full (and the product is a single one,
+   not an entry of a batch, with at least 16 slabs of K) its tiles are cut along K into shares that fill the round: at most 8 per tile -- 64 when
+   the whole product is less than one round -- each of at least 8 slabs, none empty, together within the stream's
+   workspace (every share leaves tile_m x tile_n raw sums of elem_size bytes there); no cut that would still leave most
+   of the units idle. Returns the shares per tile (1: no cut). *rounds: what the product costs in rounds of whole tiles,
+   the cut round counted by the length of a share plus six slabs of fixed cost per block. Host arithmetic only. */
+int gemm_pipe_split_plan(uint64_t M, uint64_t N, uint64_t K, uint64_t batch, bool single, uint32_t tile_m, uint32_t tile_n,
+                         uint32_t slab, uint32_t elem_size, uint64_t units, double *rounds)
+{
+   if (tile_m == 0 || tile_n == 0 || slab == 0 || elem_size == 0 || units == 0) { if (rounds) *rounds = 0.0; return 1; }
+   const uint64_t tiles = ((M + tile_m - 1) / tile_m) * ((N + tile_n - 1) / tile_n) * batch;
+   const uint64_t rest = tiles % units, slabs = K / slab;
+   uint64_t shares = 1;
+   if (single && batch == 1 && rest > 0 && rest * 2 <= units && slabs >= 16)
+   {  shares = units / rest;
+      if (shares > (tiles < units ? 64 : 8)) shares = tiles < units ? 64 : 8;
+      if (shares > slabs / 8) shares = slabs / 8;
+      const uint64_t fit = OCH_GEMM_WORKSPACE / (rest * (uint64_t)tile_m * tile_n * elem_size);
+      if (shares > fit) shares = fit;
+      while (shares > 1 && ((slabs + shares - 1) / shares) * (shares - 1) >= slabs) shares--;
+      if (shares < 2 || rest * shares * 2 < units) shares = 1;
+   }
+   if (rounds)
+   {  const double whole = (double)(slabs + 6), cut = (double)((slabs + shares - 1) / shares + 6) + 0.02 * whole;
+      *rounds = (double)(tiles / units) + (rest == 0 ? 0.0 : (shares > 1 ? cut / whole : 1.0));
+   }
+   return (int)shares;
+}
+
 int gemm_compute_units(void)
 {  static int cached[64];
    int device = 0;
@@ -295,6 +325,12 @@ extern "C" int och_gemm_batched(int dtype, char transA, char transB, size_t M, s
       if (gemm_dispatch(dtype, g) != 0) return -1;
    }
    return 0;
+}
+
+extern "C" int och_gemm_split_plan(size_t M, size_t N, size_t K, unsigned tile_m, unsigned tile_n, unsigned slab, unsigned elem_size,
+                                   unsigned units, double *rounds)
+{
+   return och::gemm_pipe_split_plan(M, N, K, 1, true, tile_m, tile_n, slab, elem_size, units, rounds);
 }
 
 extern "C" int och_gemm_set_kernel_choice(int choice)

@@ -314,24 +314,7 @@ __global__ __launch_bounds__(256) void gemm_float_pipe_finish_kernel(const Float
    what every block spends outside its main loop (about 6 slabs' worth) over the length of a whole tile. */
 int gemm_float_pipe_split(const GemmArgs &g, int tile, double *rounds)
 {
-   const uint64_t units = (uint64_t)gemm_compute_units();
-   const uint64_t tiles = ((g.M + tile - 1) / tile) * ((g.N + tile - 1) / tile) * (uint64_t)g.nz;
-   const uint64_t rest = tiles % units, slabs = g.K / OCH_FP_KT;
-   uint64_t shares = 1;
-   if (g.batch.nb == 0 && g.nz == 1 && rest > 0 && rest * 2 <= units && slabs >= 16)
-   {  shares = units / rest;
-      if (shares > (tiles < units ? 64 : 8)) shares = tiles < units ? 64 : 8;       /* 64: a product of a few tiles and a long K */
-      if (shares > slabs / 8) shares = slabs / 8;
-      const uint64_t fit = OCH_GEMM_WORKSPACE / (rest * (uint64_t)tile * tile * 4);
-      if (shares > fit) shares = fit;
-      while (shares > 1 && ((slabs + shares - 1) / shares) * (shares - 1) >= slabs) shares--;      /* no empty share */
-      if (shares < 2 || rest * shares * 2 < units) shares = 1;      /* ... nor a cut that leaves most compute units idle */
-   }
-   if (rounds)
-   {  const double whole = (double)(slabs + 6), cut = (double)((slabs + shares - 1) / shares + 6) + 0.02 * whole;
-      *rounds = (double)(tiles / units) + (rest == 0 ? 0.0 : (shares > 1 ? cut / whole : 1.0));
-   }
-   return (int)shares;
+   return gemm_pipe_split_plan(g.M, g.N, g.K, (uint64_t)g.nz, g.batch.nb == 0, (uint32_t)tile, (uint32_t)tile, OCH_FP_KT, 4, (uint64_t)gemm_compute_units(), rounds);
 }
 
 /* 0: launched; 1: not a case for this kernel (the caller's other kernels take it). tile: 256 or 128; M and N multiples

@@ -208,6 +208,54 @@ def test_kernel_choice():
     assert p.div_d[0] == 1 and fastdiv(12345, 1, p.div_m[0], p.div_s1[0], p.div_s2[0]) == 12345
 
 
+def test_cutting_the_last_round_of_a_product_along_k():
+    """och_gemm_split_plan (host arithmetic only): known answers, and for shapes from a fixed seed the rules a cut has to
+    keep -- only a last round that is at most half full is cut, at most 8 shares per tile (64 for a product of less than
+    one round), every share at least 8 slabs and none empty, the shares of the round within the compute units and within
+    the 64 MB workspace, no cut that leaves most units idle, and a cost between the whole rounds and the rounds rounded up."""
+    import ocean_hip as oh
+    workspace = 1 << 26
+
+    def plan(M, N, K, tm, tn, slab, es, units=256):
+        rounds = C.c_double(-1.0)
+        shares = oh.lib.och_gemm_split_plan(M, N, K, tm, tn, slab, es, units, C.byref(rounds))
+        assert shares == oh.lib.och_gemm_split_plan(M, N, K, tm, tn, slab, es, units, None)
+        return shares, rounds.value
+    assert plan(8192, 8192, 8192, 256, 256, 32, 4) == (1, 4.0)                  # whole rounds: nothing to cut
+    shares, rounds = plan(3000, 3000, 3000 - 3000 % 32, 128, 128, 32, 4)        # 576 tiles = 2 rounds + 64 tiles, 93 slabs
+    assert shares == 4 and abs(rounds - (2 + (24 + 6 + 0.02 * 99) / 99)) < 1e-12
+    assert plan(512, 512, 65536, 256, 256, 32, 4)[0] == 64                      # four tiles and a long K
+    assert plan(128, 128, 262144, 128, 128, 32, 4)[0] == 1                      # one tile: 64 shares would leave 3/4 idle
+    assert plan(2176, 2048, 1024, 128, 128, 16, 8)[0] == 8                      # 272 tiles: 16 in the last round, 64 slabs
+    assert plan(2176, 2048, 240, 128, 128, 16, 8)[0] == 1                       # 15 slabs: too short to cut
+    assert plan(4352, 4096, 8192, 256, 256, 32, 4, units=0) == (1, 0.0)         # nothing to plan for
+    rng = np.random.default_rng(77)
+    tiles_of = [(256, 256, 32, 4), (128, 128, 32, 4), (256, 128, 16, 8), (128, 128, 16, 8), (128, 128, 32, 8), (128, 64, 16, 16)]
+    cut = 0
+    for n in range(4000):
+        tm, tn, slab, es = tiles_of[n % len(tiles_of)]
+        units = (256, 304, 64, 1)[(n // 7) % 4]
+        M, N = int(rng.integers(1, 9000)), int(rng.integers(1, 9000))
+        K = int(rng.integers(1, 3000 if n % 2 else 300)) * slab
+        shares, rounds = plan(M, N, K, tm, tn, slab, es, units)
+        tiles = -(-M // tm) * -(-N // tn)
+        rest, slabs = tiles % units, K // slab
+        assert 1 <= shares <= (64 if tiles < units else 8), (M, N, K, shares)
+        assert tiles // units <= rounds <= -(-tiles // units) + 1e-12
+        if rest == 0 or rest * 2 > units or slabs < 16:
+            assert shares == 1
+        if shares == 1:
+            assert rounds == -(-tiles // units)
+            continue
+        cut += 1
+        length = -(-slabs // shares)
+        assert length >= 8 and length * (shares - 1) < slabs, "a share shorter than 8 slabs, or an empty one"
+        assert rest * shares <= units and rest * shares * 2 >= units
+        assert rest * shares * tm * tn * es <= workspace
+        assert rounds < -(-tiles // units)
+    assert cut > 200
+
+
 def test_cutting_a_large_reduction_into_launches():
     """och_reduce_cut_parts (host arithmetic only): the boxes are disjoint, cover the tensor, hold at most `limit` elements
     each, and never cut dimension 0; a dimension 0 beyond the limit is refused."""
