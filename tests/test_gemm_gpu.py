@@ -676,3 +676,19 @@ def test_gemm_seeded_shapes_under_the_automatic_choice(hip, stream, dtype):
         ta, tb = modes[int(rng.integers(len(modes)))], modes[int(rng.integers(len(modes)))]
         alpha, beta = ((2 - 1j, -1 + 0.5j) if cplx else (2, -1)) if n % 2 else (1, 0)
         check_large_product(stream, dtype, ta, tb, M, N, [(K / slab, alpha, beta, n % 5 == 4)], rng, pad=(0, 4, 0, 3)[(n // 4) % 4])
+
+
+@pytest.mark.parametrize("dtype", [H.HALF, H.INT8, H.UINT8], ids=lambda d: H.NAMES[d])
+def test_gemm_seeded_shapes_of_the_matrix_core_types(hip, stream, dtype):
+    """The same for half (float accumulation, bound 2e-3) and the 8-bit integers (exact modulo 256): shapes from a fixed
+    seed with M and N from 64 to 1500, whole tiles, edge strips and odd sizes, K with and without whole slabs, aligned and
+    unaligned leading dimensions, both kinds of scalars."""
+    rng = np.random.default_rng(4300 + dtype)
+    slab = 64 if dtype == H.HALF else 128
+    for n in range(24):
+        step = (256, 128, 8, 1)[n % 4]
+        M, N = (max(step, int(rng.integers(64, 1500)) // step * step) for _ in range(2))
+        K = int(rng.integers(1, 4000 // slab)) * slab + (int(rng.integers(1, slab)) if n % 3 == 1 else 0)
+        ta, tb = "NT"[int(rng.integers(2))], "NT"[int(rng.integers(2))]
+        alpha, beta = (2, -1) if n % 2 else (1, 0)
+        check_large_product(stream, dtype, ta, tb, M, N, [(K / slab, alpha, beta, n % 5 == 4)], rng, pad=(0, 8, 0, 3)[(n // 4) % 4])
