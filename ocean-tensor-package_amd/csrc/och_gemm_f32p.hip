@@ -3,7 +3,8 @@
  * The counterpart of cublasSgemm in the reference (src/core/gpu/op/tensor_blas_gpu.c:183-197). Four waves per block,
  * one per SIMD, each owning 128 x 128 of the tile as 4 x 4 tiles of v_mfma_f32_32x32x2_f32 (256 accumulator registers);
  * for products with fewer than one such tile per compute unit the same kernel with TS = 2: waves of 64 x 64 (2 x 2
- * tiles), two blocks per compute unit. The description is for TS = 4.
+ * tiles), two blocks per compute unit (SINGLE: one slab buffer, three blocks, for a K of one or two slabs). The
+ * description is for TS = 4.
  * On this device a vector-ALU instruction of a wave takes about eight cycles away from the matrix cores of its SIMD, and
  * a 64-cycle MFMA hides none of that; LDS reads and scalar instructions are nearly free. So the main loop holds MFMAs,
  * LDS reads, scalar instructions and loads that go from memory straight to LDS -- no vector arithmetic, no staging
@@ -123,8 +124,8 @@ static __device__ __forceinline__ void load_to_lds(const char *base, uint32_t of
    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(target), "v"(offset), "s"(base) : "memory");
 }
 
-template <bool AKC, bool BKC, int TS>
-__global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pipe_kernel(const FloatPipeParams p)
+template <bool AKC, bool BKC, int TS, bool SINGLE = false>
+__global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : (SINGLE ? 3 : 2)) void gemm_float_pipe_kernel(const FloatPipeParams p)
 {
    constexpr int T = 32, BM = 64 * TS, BN = 64 * TS, KT = OCH_FP_KT, TMS = TS, TNS = TS, WM = 32 * TS, WN = 32 * TS, THREADS = OCH_FP_THREADS;
    typedef FloatSlab<AKC, BM> LA;
@@ -213,6 +214,30 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pi
            OCH_QUAD(1, 0, 1 - CB, 0, true, 0, CB);                                                                     \
         } } while (0)
 
+   if constexpr (SINGLE)
+   {  /* one slab buffer, three blocks per compute unit: a block's loads are not covered by its own MFMAs but by those of
+         its neighbours. For a K of a few slabs, where a block spends as long on its first loads and on writing C as in
+         its loop. */
+      for (uint32_t s = 0; s < nslabs; s++)
+      {  const char *nextA = LA::slab_base(pA, p.ldA, m0, (slab0 + s) * KT), *nextB = LB::slab_base(pB, p.ldB, n0, (slab0 + s) * KT);
+         if (s > 0) __syncthreads();
+#pragma unroll
+         for (int e = 0; e < NL; e++) OCH_LOAD(e, nextA, nextB, 0);
+         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+         __syncthreads();
+#pragma unroll
+         for (int x = 0; x < LA::READS; x++) fa[0][x] = LA::read(readA[0] + LA::read_offset(x, 0));
+#pragma unroll
+         for (int x = 0; x < LB::READS; x++) fb[0][x] = LB::read(readB[0] + LB::read_offset(x, 0));
+         OCH_QUAD(0, 1, 0, 1, false, 0, 0);
+         OCH_QUAD(1, 0, 0, 2, false, 0, 0);
+         OCH_QUAD(0, 1, 0, 3, false, 0, 0);
+         OCH_QUAD(1, 0, 0, 0, false, 0, 0);            /* (its reads are not used) */
+      }
+      __syncthreads();
+   }
+   else
+   {
    {  /* slab 0 and the first half of slab 1 */
       const uint32_t s1 = (slab0 + 1 < last) ? slab0 + 1 : last;
       const char *nextA = LA::slab_base(pA, p.ldA, m0, slab0 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, slab0 * KT);
@@ -236,6 +261,7 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pi
    if (s < nslabs) OCH_SLAB(s, 0);
    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
    __syncthreads();
+   }
 #undef OCH_SLAB
 #undef OCH_QUAD
 #undef OCH_LOAD
@@ -255,7 +281,7 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : 2) void gemm_float_pi
       out = reinterpret_cast<char *>(p.partial + (size_t)cut * BM * BN); ldOut = BM; rowsOut = BM; colsOut = BN;
    }
    constexpr int CP = BM + 4, CPASS = 64, PASSES = BN / CPASS;
-   static_assert(CPASS * CP * 4 <= 2 * BUF, "a pass of the staged tile does not fit into the slab buffers");
+   static_assert(CPASS * CP * 4 <= (SINGLE ? 1 : 2) * BUF, "a pass of the staged tile does not fit into the slab buffers");
    float *stage = reinterpret_cast<float *>(lds);
    for (int h = 0; h < PASSES; h++)
    {
@@ -346,13 +372,17 @@ int gemm_float_pipe(const GemmArgs &g, int tile)
       blocks += (uint64_t)cut_tiles * (shares - 1);
    }
    const bool akc = (g.transA != 'N'), bkc = (g.transB == 'N');
+   /* a K of one or two slabs on the small tile: one slab buffer and three blocks per compute unit instead of two buffers and
+      two blocks (8192 x 8192 x 64: 67-74 -> 78-80 TFLOP/s; from four slabs on the two buffers win). Same MFMAs in the
+      same order: the same bits. */
+   const bool single = tile == 128 && shares == 1 && g.K / OCH_FP_KT <= 2;
    const dim3 grid((unsigned)blocks, 1, g.nz), block(OCH_FP_THREADS);
-#define OCH_FP_LAUNCH(AK, BK, TS)                                                                                     \
-   do { auto kernel = gemm_float_pipe_kernel<AK, BK, TS>;                                                             \
-        const size_t lds = 4 * (size_t)FloatSlab<AK, 64 * TS>::OPERAND;                                               \
+#define OCH_FP_LAUNCH(AK, BK, TS, SINGLE)                                                                             \
+   do { auto kernel = gemm_float_pipe_kernel<AK, BK, TS, SINGLE>;                                                     \
+        const size_t lds = ((SINGLE) ? 2 : 4) * (size_t)FloatSlab<AK, 64 * TS>::OPERAND;                              \
         OCH_CHECK_HIP(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
         hipLaunchKernelGGL(kernel, grid, block, lds, g.stream, p); } while (0)
-#define OCH_FP_PICK(AK, BK) do { if (tile == 256) OCH_FP_LAUNCH(AK, BK, 4); else OCH_FP_LAUNCH(AK, BK, 2); } while (0)
+#define OCH_FP_PICK(AK, BK) do { if (tile == 256) OCH_FP_LAUNCH(AK, BK, 4, false); else if (single) OCH_FP_LAUNCH(AK, BK, 2, true); else OCH_FP_LAUNCH(AK, BK, 2, false); } while (0)
    if (!akc && !bkc) OCH_FP_PICK(false, false);
    else if (!akc)    OCH_FP_PICK(false, true);
    else if (!bkc)    OCH_FP_PICK(true, false);
