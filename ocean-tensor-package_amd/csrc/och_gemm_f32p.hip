@@ -3,7 +3,7 @@
  * The counterpart of cublasSgemm in the reference (src/core/gpu/op/tensor_blas_gpu.c:183-197). Four waves per block,
  * one per SIMD, each owning 128 x 128 of the tile as 4 x 4 tiles of v_mfma_f32_32x32x2_f32 (256 accumulator registers);
  * for products with fewer than one such tile per compute unit the same kernel with TS = 2: waves of 64 x 64 (2 x 2
- * tiles), two blocks per compute unit (SINGLE: one slab buffer, three blocks, for a K of one or two slabs). The
+ * tiles), two blocks per compute unit (SINGLE: one slab buffer of 34 KB and about a hundred registers, four blocks, for a K of one or two slabs). The
  * description is for TS = 4.
  * On this device a vector-ALU instruction of a wave takes about eight cycles away from the matrix cores of its SIMD, and
  * a 64-cycle MFMA hides none of that; LDS reads and scalar instructions are nearly free. So the main loop holds MFMAs,
@@ -125,7 +125,7 @@ static __device__ __forceinline__ void load_to_lds(const char *base, uint32_t of
 }
 
 template <bool AKC, bool BKC, int TS, bool SINGLE = false>
-__global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : (SINGLE ? 3 : 2)) void gemm_float_pipe_kernel(const FloatPipeParams p)
+__global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : (SINGLE ? 4 : 2)) void gemm_float_pipe_kernel(const FloatPipeParams p)
 {
    constexpr int T = 32, BM = 64 * TS, BN = 64 * TS, KT = OCH_FP_KT, TMS = TS, TNS = TS, WM = 32 * TS, WN = 32 * TS, THREADS = OCH_FP_THREADS;
    typedef FloatSlab<AKC, BM> LA;
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : (SINGLE ? 3 : 2)) voi
         } } while (0)
 
    if constexpr (SINGLE)
-   {  /* one slab buffer, three blocks per compute unit: a block's loads are not covered by its own MFMAs but by those of
+   {  /* one slab buffer, four blocks per compute unit: a block's loads are not covered by its own MFMAs but by those of
          its neighbours. For a K of a few slabs, where a block spends as long on its first loads and on writing C as in
          its loop. */
       for (uint32_t s = 0; s < nslabs; s++)
@@ -372,7 +372,7 @@ int gemm_float_pipe(const GemmArgs &g, int tile)
       blocks += (uint64_t)cut_tiles * (shares - 1);
    }
    const bool akc = (g.transA != 'N'), bkc = (g.transB == 'N');
-   /* a K of one or two slabs on the small tile: one slab buffer and three blocks per compute unit instead of two buffers and
+   /* a K of one or two slabs on the small tile: one slab buffer and four blocks per compute unit instead of two buffers and
       two blocks (8192 x 8192 x 64: 67-74 -> 78-80 TFLOP/s; from four slabs on the two buffers win). Same MFMAs in the
       same order: the same bits. */
    const bool single = tile == 128 && shares == 1 && g.K / OCH_FP_KT <= 2;
