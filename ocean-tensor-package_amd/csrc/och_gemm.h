@@ -557,6 +557,15 @@ static int launch_gemm_mfma(const GemmArgs &g)
    return 0;
 }
 
+/* one load from memory straight to LDS: lane l brings 16 bytes from base + offset[l] to LDS byte target + 16 l. The target
+   travels in M0, which the kernels that load this way use for nothing else (the compiler is not told: it counts M0 among the registers it
+   manages itself and warns about a clobber); the compiler does not see a load either, so the waits for these loads
+   (vmcnt) are written out in front of the barriers. */
+static __device__ __forceinline__ void load_to_lds(const char *base, uint32_t offset, uint32_t target)
+{
+   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(target), "v"(offset), "s"(base) : "memory");
+}
+
 /* Compute units of the current device (cached per device). */
 int gemm_compute_units(void);
 int gemm_kernel_choice(void);            /* 0 automatic; 1 / 2: pipelined kernel, large / small tile; 3: never pipelined */

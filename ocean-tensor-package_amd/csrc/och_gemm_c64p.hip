@@ -88,15 +88,6 @@ struct CDoubleSlab
 };
 static_assert(16 * CDoubleSlab<true, 128>::PLANE <= OCH_ZP_A && 16 * CDoubleSlab<true, 64>::PLANE <= OCH_ZP_B, "the slabs do not fit");
 
-/* one load from memory straight to LDS: lane l brings 16 bytes from base + offset[l] to LDS byte target + 16 l. The target
-   travels in M0, which nothing else in these kernels uses (the compiler is not told: it counts M0 among the registers it
-   manages itself and warns about a clobber); the compiler does not see a load either, so the waits for these loads
-   (vmcnt) are written out in front of the barriers. */
-static __device__ __forceinline__ void load_to_lds(const char *base, uint32_t offset, uint32_t target)
-{
-   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(target), "v"(offset), "s"(base) : "memory");
-}
-
 /* 16 bytes of LDS into two ordinary registers pairs. Written as an instruction of its own so that the value lands in the
    ordinary registers (left to itself the compiler reads fragments into accumulation registers and copies them on every
    use). The compiler does not know that the value arrives later: every pair of steps opens with a wait for all LDS reads. */

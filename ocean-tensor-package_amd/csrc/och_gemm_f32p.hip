@@ -115,15 +115,6 @@ struct FloatSlab
    static __device__ __forceinline__ uint32_t row(int i, uint32_t rr) { return KC ? (uint32_t)i * 32 + rr : TS * rr + (uint32_t)i; }
 };
 
-/* one load from memory straight to LDS: lane l brings 16 bytes from base + offset[l] to LDS byte target + 16 l. The target
-   travels in M0, which nothing else in these kernels uses (the compiler is not told: it counts M0 among the registers it
-   manages itself and warns about a clobber); the compiler does not see a load either, so the waits for these loads
-   (vmcnt) are written out in front of the barriers. */
-static __device__ __forceinline__ void load_to_lds(const char *base, uint32_t offset, uint32_t target)
-{
-   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(target), "v"(offset), "s"(base) : "memory");
-}
-
 template <bool AKC, bool BKC, int TS, bool SINGLE = false>
 __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : (SINGLE ? 4 : 2)) void gemm_float_pipe_kernel(const FloatPipeParams p)
 {
