@@ -573,6 +573,35 @@ int gemm_pipe_split_plan(uint64_t M, uint64_t N, uint64_t K, uint64_t batch, boo
                          uint32_t slab, uint32_t elem_size, uint64_t units, double *rounds);   /* shares of the tiles of the last round */
 int gemm_pad_tail(const GemmArgs &g, size_t Kh, int slab, int es, GemmArgs *tail);   /* the rest of K as one zero-padded slab in the workspace */
 
+/* A product on a pipelined kernel whose K need not be a whole number of slabs (the caller has checked that the scalars
+   are in host memory when it is not): the whole slabs through `pipelined` with the caller's beta, then the rest of K --
+   both operands' tails copied into the workspace and filled up with zeros to one slab -- through `pipelined` again with
+   beta = 1 (`one`: that scalar in the product's type); where the rest cannot be padded, through `others`, the type's own
+   entry. 0: done; 1: the pipelined kernel does not take the product, nothing was launched; -1: error. es: element size. */
+template <class Pipelined, class Others>
+static int gemm_pipelined_head_and_rest(const GemmArgs &g, int slab, int es, const void *one, Pipelined pipelined, Others others)
+{
+   GemmArgs part = g;
+   const size_t Kh = g.K - g.K % (size_t)slab;
+   part.K = Kh;
+   const int taken = pipelined(part);
+   if (taken != 0) return taken;
+   if (g.K == Kh) return 0;
+   GemmArgs tail;
+   const int padded = gemm_pad_tail(g, Kh, slab, es, &tail);
+   if (padded < 0) return -1;
+   if (padded == 0)
+   {  tail.beta = one;
+      const int again = pipelined(tail);
+      if (again < 0) return -1;
+      if (again == 0) return 0;
+   }
+   part.K = g.K - Kh; part.beta = one;
+   part.A = (const char *)g.A + (int64_t)Kh * (g.transA == 'N' ? (int64_t)g.ldA : 1) * es;
+   part.B = (const char *)g.B + (int64_t)Kh * (g.transB == 'N' ? 1 : (int64_t)g.ldB) * es;
+   return others(part) != 0 ? -1 : 0;
+}
+
 /* Which block tile to use. The compute units work through the tiles in rounds, and the last round is as long as the others
    however few tiles it holds: 3000^3 double is 576 tiles of 128 x 128, i.e. 2.25 rounds on 256 units, and ran at 39
    TFLOP/s where 4000^3 (exactly 4 rounds) reached 56. A candidate's cost is rounds x tile area / efficiency (its measured

@@ -23,32 +23,9 @@ int gemm_cfloat(const GemmArgs &g)
       const double pipelined = rounds * 16384.0;
       const int forced = gemm_kernel_choice();
       if (forced != 3 && (forced != 0 || pipelined < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87)))
-      {  GemmArgs part = g;
-         const size_t Kh = g.K - g.K % 32;
-         part.K = Kh;
-         const int taken = gemm_cfloat_pipe(part);
-         if (taken < 0) return taken;
-         if (taken == 0)
-         {  if (g.K > Kh)
-            {  static const float one[2] = { 1.0f, 0.0f };
-               /* the rest of K, filled up with zeros to one slab in the workspace, on the pipelined kernel again; where
-                  that does not fit, on the kernels below */
-               GemmArgs tail;
-               const int padded = gemm_pad_tail(g, Kh, 32, 8, &tail);
-               if (padded < 0) return -1;
-               if (padded == 0)
-               {  tail.beta = one;
-                  const int again = gemm_cfloat_pipe(tail);
-                  if (again < 0) return -1;
-                  if (again == 0) return 0;
-               }
-               part.K = g.K - Kh; part.beta = one;
-               part.A = (const char *)g.A + (int64_t)Kh * (g.transA == 'N' ? (int64_t)g.ldA : 1) * 8;
-               part.B = (const char *)g.B + (int64_t)Kh * (g.transB == 'N' ? 1 : (int64_t)g.ldB) * 8;
-               if (gemm_cfloat(part) != 0) return -1;
-            }
-            return 0;
-         }
+      {  static const float one[2] = { 1.0f, 0.0f };
+         const int done = gemm_pipelined_head_and_rest(g, 32, 8, one, [&](const GemmArgs &a) { return gemm_cfloat_pipe(a); }, gemm_cfloat);
+         if (done <= 0) return done;
       }
    }
    switch (pick)

@@ -31,32 +31,9 @@ int gemm_float(const GemmArgs &g)
       const int forced = gemm_kernel_choice();
       const int tile = forced == 1 ? 256 : (forced == 2 ? 128 : (large <= small ? 256 : 128));
       if (forced != 3 && (forced != 0 || (tile == 256 ? large : small) < others))
-      {  GemmArgs part = g;
-         const size_t Kh = g.K - g.K % 32;
-         part.K = Kh;
-         const int taken = gemm_float_pipe(part, tile);
-         if (taken < 0) return taken;
-         if (taken == 0)
-         {  if (g.K > Kh)
-            {  static const float one = 1.0f;
-               /* the rest of K, filled up with zeros to one slab in the workspace, on the pipelined kernel again; where
-                  that does not fit, on the kernels below */
-               GemmArgs tail;
-               const int padded = gemm_pad_tail(g, Kh, 32, 4, &tail);
-               if (padded < 0) return -1;
-               if (padded == 0)
-               {  tail.beta = &one;
-                  const int again = gemm_float_pipe(tail, tile);
-                  if (again < 0) return -1;
-                  if (again == 0) return 0;
-               }
-               part.K = g.K - Kh; part.beta = &one;
-               part.A = (const char *)g.A + (int64_t)Kh * (g.transA == 'N' ? (int64_t)g.ldA : 1) * 4;
-               part.B = (const char *)g.B + (int64_t)Kh * (g.transB == 'N' ? 1 : (int64_t)g.ldB) * 4;
-               if (gemm_float(part) != 0) return -1;
-            }
-            return 0;
-         }
+      {  static const float one = 1.0f;
+         const int done = gemm_pipelined_head_and_rest(g, 32, 4, &one, [&](const GemmArgs &a) { return gemm_float_pipe(a, tile); }, gemm_float);
+         if (done <= 0) return done;
       }
    }
    switch (pick)

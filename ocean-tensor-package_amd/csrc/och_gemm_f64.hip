@@ -29,32 +29,9 @@ int gemm_double(const GemmArgs &g)
       const int forced = gemm_kernel_choice();
       const int tile_m = forced == 1 ? 256 : (forced == 2 ? 128 : (large <= small ? 256 : 128));
       if (forced != 3 && (forced != 0 || (tile_m == 256 ? large : small) < cost(choice[pick].bm, choice[pick].bn, choice[pick].efficiency * 0.87) * (slabs + 4) / slabs))
-      {  GemmArgs part = g;
-         const size_t Kh = g.K - g.K % 16;
-         part.K = Kh;
-         const int taken = gemm_double_pipe(part, tile_m);
-         if (taken < 0) return taken;
-         if (taken == 0)
-         {  if (g.K > Kh)
-            {  static const double one = 1.0;
-               /* the rest of K, filled up with zeros to one slab in the workspace, on the pipelined kernel again; where
-                  that does not fit, on the kernels below */
-               GemmArgs tail;
-               const int padded = gemm_pad_tail(g, Kh, 16, 8, &tail);
-               if (padded < 0) return -1;
-               if (padded == 0)
-               {  tail.beta = &one;
-                  const int again = gemm_double_pipe(tail, tile_m);
-                  if (again < 0) return -1;
-                  if (again == 0) return 0;
-               }
-               part.K = g.K - Kh; part.beta = &one;
-               part.A = (const char *)g.A + (int64_t)Kh * (g.transA == 'N' ? (int64_t)g.ldA : 1) * 8;
-               part.B = (const char *)g.B + (int64_t)Kh * (g.transB == 'N' ? 1 : (int64_t)g.ldB) * 8;
-               if (gemm_double(part) != 0) return -1;
-            }
-            return 0;
-         }
+      {  static const double one = 1.0;
+         const int done = gemm_pipelined_head_and_rest(g, 16, 8, &one, [&](const GemmArgs &a) { return gemm_double_pipe(a, tile_m); }, gemm_double);
+         if (done <= 0) return done;
       }
    }
    switch (pick)
