@@ -3,6 +3,7 @@
  * square LDS tile; here each thread owns a 4 x 4 patch of a 64 x 64 tile).
  * bool: + is OR, * is AND. Integers wrap. half multiplies and accumulates in float. */
 #include "och_gemm.h"
+#include <atomic>
 #include "../../include/ocean_hip.h"
 
 namespace och {
@@ -163,8 +164,8 @@ int gemm_pad_tail(const GemmArgs &g, size_t Kh, int slab, int es, GemmArgs *tail
 
 /* 0: the cost model chooses; 1: the pipelined kernel on its large tile wherever it applies; 2: on its small tile (float,
    double); 3: never the pipelined kernel. For tests and measurements (och_gemm_set_kernel_choice). */
-static int g_gemm_kernel_choice = 0;
-int gemm_kernel_choice(void) { return g_gemm_kernel_choice; }
+static std::atomic<int> g_gemm_kernel_choice{0};
+int gemm_kernel_choice(void) { return g_gemm_kernel_choice.load(std::memory_order_relaxed); }
 
 /* The last round of a pipelined product. `units` compute units work through tiles x batch block tiles in rounds, and
    a last round of `rest` tiles takes as long as a full one. When it is at most half full (and the product is a single one,
@@ -197,15 +198,15 @@ int gemm_pipe_split_plan(uint64_t M, uint64_t N, uint64_t K, uint64_t batch, boo
 }
 
 int gemm_compute_units(void)
-{  static int cached[64];
+{  static std::atomic<int> cached[64];          /* zero-initialised; threads that meet an empty entry all store the same number */
    int device = 0;
    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
-   if (cached[device] == 0)
-   {  int n = 0;
-      if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0) n = 256;
-      cached[device] = n;
+   int n = cached[device].load(std::memory_order_relaxed);
+   if (n == 0)
+   {  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0) n = 256;
+      cached[device].store(n, std::memory_order_relaxed);
    }
-   return cached[device];
+   return n;
 }
 
 static char norm_trans(char t)
@@ -336,6 +337,6 @@ extern "C" int och_gemm_split_plan(size_t M, size_t N, size_t K, unsigned tile_m
 extern "C" int och_gemm_set_kernel_choice(int choice)
 {
    if (choice < 0 || choice > 3) return och::set_error("gemm: kernel choice %d (0 automatic, 1 pipelined large tile, 2 pipelined small tile, 3 tiled kernel)", choice);
-   och::g_gemm_kernel_choice = choice;
+   och::g_gemm_kernel_choice.store(choice, std::memory_order_relaxed);
    return 0;
 }
