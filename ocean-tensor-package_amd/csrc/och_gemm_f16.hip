@@ -18,6 +18,7 @@
 namespace och {
 
 typedef _Float16 och_h8 __attribute__((ext_vector_type(8)));
+typedef short och_i16x4 __attribute__((ext_vector_type(4)));
 
 struct HalfGemmParams
 {
@@ -35,29 +36,29 @@ struct HalfGemmParams
    float   *partial;
 };
 
-/* Moves a BMN x KT slab of an operand (2-byte elements) from memory to registers and on to LDS.
-   LDS layout: [chunk of 8 k][slot][8 halves], 32 bytes of padding after every chunk plane. A fragment read takes one
-   chunk of 32 neighbouring slots: 512 consecutive bytes.
-   KC (contiguous along k in memory): a thread loads 16 bytes = one chunk of one row; row r sits in slot r. Eight
-   neighbouring lanes store the eight chunks of a row; the padding moves each plane on by eight banks.
-   !KC (contiguous along the row index): a thread loads NV consecutive k for 8 neighbouring rows (16 bytes each),
-   transposes the 8 x NV block in registers and stores NV k for each of the 8 rows. Neighbouring lanes hold rows that are
-   8 apart, so row r sits in slot (r mod 8) * (BMN / 8) + r / 8: the stores of a wave cover consecutive slots. Which row
-   of the tile an MFMA lane works on is then a matter of bookkeeping when C is written (row_of_slot). */
+/* Moves a BMN x KT slab of an operand (2-byte elements) from memory to registers and on to LDS, 16 bytes at a time, and
+   reads MFMA fragments (eight consecutive k of one row per lane) from there.
+   KC (contiguous along k in memory): a thread loads one chunk of 8 k of one row; LDS holds [chunk of 8 k][row][8 halves],
+   32 bytes of padding after every chunk plane; eight neighbouring lanes store the eight chunks of a row, and a fragment
+   is one 16-byte read (32 neighbouring rows of one chunk plane: 512 consecutive bytes per half wave).
+   !KC (contiguous along the row index): a thread loads 8 neighbouring rows of one k, for NV consecutive k, and LDS holds
+   the slab as it lies in memory, [k][row] with a pitch of BMN + 16 halves. The fragments come out of transposing reads
+   (ds_read_b64_tr_b16): in every group of 16 lanes, lanes 4 q .. 4 q + 3 read 16 neighbouring rows of k + q, and lane i
+   of the group receives row i of k .. k + 3; two such reads make the eight k of a fragment. No register transposition,
+   no permuted rows. */
 template <bool KC, bool EDGE, int BMN, int KT, int THREADS>
 struct HalfSlab
 {
    static constexpr int NV = BMN * KT / 8 / THREADS;                   /* 16-byte loads per thread */
-   static constexpr int PLANE = BMN * 8 + 16;                          /* halves per chunk plane */
-   static constexpr int SIZE = (KT / 8) * PLANE;                       /* halves per LDS buffer */
+   static constexpr int PLANE = BMN * 8 + 16;                          /* KC: halves per chunk plane */
+   static constexpr int PITCH = BMN + 16;                              /* !KC: halves from one k to the next; 32 bytes more than the rows so that the four k of a transposing read meet different banks */
+   static constexpr int SIZE = KC ? (KT / 8) * PLANE : KT * PITCH;     /* halves per LDS buffer */
    static_assert(NV >= 1 && (BMN * KT) % (8 * THREADS) == 0, "slab does not divide among the threads");
-   static_assert(KC || NV == 2 || NV == 4 || NV == 8, "the transposing loader needs 2, 4 or 8 k per thread");
    och_gu32x4 reg[NV];
 
-   static __device__ __forceinline__ uint32_t row_of_slot(uint32_t slot)
-   {  return KC ? slot : (slot % (BMN / 8)) * 8 + slot / (BMN / 8); }
-   /* row_of_slot(s + o) - row_of_slot(s) for offsets o whose sum with s does not carry out of s mod (BMN / 8) */
-   static constexpr uint32_t row_step(uint32_t o) { return KC ? o : (o % (BMN / 8)) * 8 + o / (BMN / 8); }
+   /* LDS slot -> row of the tile: the same for both layouts (kept as the one place that says so) */
+   static __device__ __forceinline__ uint32_t row_of_slot(uint32_t slot) { return slot; }
+   static constexpr uint32_t row_step(uint32_t o) { return o; }
    static __device__ __forceinline__ void where(int v, uint32_t &mn, uint32_t &k)
    {  if (!KC) { mn = (threadIdx.x % (BMN / 8)) * 8; k = (threadIdx.x / (BMN / 8)) * NV + v; }
       else     { const uint32_t q = threadIdx.x + THREADS * v; k = (q % (KT / 8)) * 8; mn = q / (KT / 8); }
@@ -101,22 +102,9 @@ struct HalfSlab
          }
       }
       else
-      {  constexpr int WD = NV / 2;                     /* 32-bit words per row: k pairs */
-         uint32_t mn, k; where(0, mn, k);
-         uint16_t *dst = buffer + (k / 8) * PLANE + (mn / 8) * 8 + k % 8;          /* row mn + i: slot i * (BMN / 8) + mn / 8 */
+      {  uint32_t mn, k; where(0, mn, k);
 #pragma unroll
-         for (int i = 0; i < 8; i++)
-         {  uint32_t out[WD];
-#pragma unroll
-            for (int w = 0; w < WD; w++)
-            {  const uint32_t x = reg[2 * w][i >> 1], y = reg[2 * w + 1][i >> 1];
-               out[w] = (i & 1) ? ((x >> 16) | (y & 0xFFFF0000u)) : ((x & 0xFFFFu) | (y << 16));
-            }
-            uint16_t *at = dst + i * BMN;                /* BMN / 8 slots of 8 halves */
-            if (WD == 1) *reinterpret_cast<uint32_t *>(at) = out[0];
-            else if (WD == 2) { uint2 t; t.x = out[0]; t.y = out[WD > 1 ? 1 : 0]; *reinterpret_cast<uint2 *>(at) = t; }
-            else { och_gu32x4 t; t.x = out[0]; t.y = out[WD > 1 ? 1 : 0]; t.z = out[WD > 2 ? 2 : 0]; t.w = out[WD > 3 ? 3 : 0]; *reinterpret_cast<och_gu32x4 *>(at) = t; }
-         }
+         for (int v = 0; v < NV; v++) *reinterpret_cast<och_gu32x4 *>(buffer + (k + v) * PITCH + mn) = reg[v];
       }
    }
    /* the same in single instructions, for loops that place every one of them by hand: load number v (whole tiles only),
@@ -135,33 +123,29 @@ struct HalfSlab
       const int64_t step = KC ? (int64_t)(THREADS / (KT / 8)) * v * ld * 2 : (int64_t)v * ld * 2;
       reg[v] = *reinterpret_cast<const och_gu32x4 *>(base + step + toff);
    }
-   static constexpr int PIECES = KC ? NV : 8;                           /* stores that move the registers to LDS */
+   static constexpr int PIECES = NV;                                    /* stores that move the registers to LDS */
    __device__ __forceinline__ void stash_one(uint16_t *buffer, int piece) const
-   {  static_assert(KC || NV == 8 || NV == 4, "a transposed piece is a store of 16 or 8 bytes");
-      if (KC)
-      {  uint32_t mn, k; where(piece, mn, k);
-         *reinterpret_cast<och_gu32x4 *>(buffer + (k / 8) * PLANE + mn * 8) = reg[piece];
-      }
-      else
-      {  constexpr int WD = NV / 2;
-         uint32_t mn, k; where(0, mn, k);
-         uint16_t *at = buffer + (k / 8) * PLANE + (mn / 8) * 8 + k % 8 + piece * BMN;
-         uint32_t out[WD];
-#pragma unroll
-         for (int w = 0; w < WD; w++)
-         {  /* the low (even piece) or high (odd piece) halves of two words, side by side: one byte permutation */
-            const uint32_t x = reg[2 * w][piece >> 1], y = reg[2 * w + 1][piece >> 1];
-            out[w] = __builtin_amdgcn_perm(y, x, (piece & 1) ? 0x07060302u : 0x05040100u);
-         }
-         if (WD == 2) { uint2 t; t.x = out[0]; t.y = out[1]; *reinterpret_cast<uint2 *>(at) = t; }
-         else { och_gu32x4 t; t.x = out[0]; t.y = out[1]; t.z = out[WD > 2 ? 2 : 0]; t.w = out[WD > 3 ? 3 : 0]; *reinterpret_cast<och_gu32x4 *>(at) = t; }
-      }
+   {  uint32_t mn, k; where(piece, mn, k);
+      if (KC) *reinterpret_cast<och_gu32x4 *>(buffer + (k / 8) * PLANE + mn * 8) = reg[piece];
+      else    *reinterpret_cast<och_gu32x4 *>(buffer + k * PITCH + mn) = reg[piece];
    }
    /* the eight k of slot `slot` that lane group `kg` (0 or 1) feeds to MFMA step `ks` (16 k per step) */
    static __device__ __forceinline__ och_h8 fragment(const uint16_t *buffer, int slot, int ks, int kg)
    {  och_h8 f;
-      const och_gu32x4 raw = *reinterpret_cast<const och_gu32x4 *>(buffer + (ks * 2 + kg) * PLANE + slot * 8);
-      __builtin_memcpy(&f, &raw, 16);
+      if (KC)
+      {  const och_gu32x4 raw = *reinterpret_cast<const och_gu32x4 *>(buffer + (ks * 2 + kg) * PLANE + slot * 8);
+         __builtin_memcpy(&f, &raw, 16);
+      }
+      else
+      {  /* slot = first row of the tile + lane % 32; this lane reads rows (slot - lane % 16) + 4 (lane % 4) .. + 3 of
+            k + (lane % 16) / 4 and receives row `slot` of k .. k + 3 */
+         const int lane = threadIdx.x & 63;
+         const uint16_t *at = buffer + (ks * 16 + kg * 8 + ((lane & 15) >> 2)) * PITCH + (slot - (lane & 15)) + 4 * (lane & 3);
+         const och_i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) och_i16x4 *)at);
+         const och_i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) och_i16x4 *)(at + 4 * PITCH));
+         __builtin_memcpy(&f, &lo, 8);
+         __builtin_memcpy(reinterpret_cast<char *>(&f) + 8, &hi, 8);
+      }
       return f;
    }
 };
