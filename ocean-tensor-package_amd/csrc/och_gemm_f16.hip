@@ -9,9 +9,9 @@
  * A block of NWM x NWN waves owns a (NWM*WM) x (NWN*WN) tile of C, each wave WM x WN of it as 32 x 32 MFMA tiles. Per K
  * step of KT = 64 the block stages slabs of op(A) and op(B) through LDS, loading slab s+1 from memory into registers before the
  * MFMAs of slab s and writing it to the other LDS buffer afterwards. An MFMA operand is eight consecutive k of one row
- * (column) per lane, so LDS holds both operands as 16-byte chunks of 8 k and a fragment is one 16-byte LDS read per lane.
+ * (column) per lane: a k-contiguous operand lies in LDS as 16-byte chunks of 8 k and a fragment is one 16-byte LDS read.
  * An operand that is contiguous along k in memory ('T' for A, 'N' for B) arrives in that shape; one that is contiguous
- * along m / n is transposed in registers on its way to LDS. Which k a lane holds does not matter as long as A and B agree, and they do by construction.
+ * along m / n lies in LDS as in memory, and its fragments come out of transposing LDS reads (ds_read_b64_tr_b16).
  */
 #include "och_gemm.h"
 

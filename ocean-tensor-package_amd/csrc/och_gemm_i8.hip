@@ -9,8 +9,8 @@
  *
  * Structure as in the half-precision kernel: a block of NWM x NWN waves owns a tile of C, K steps of 128, slab s + 1 is
  * stored to the other LDS buffer half way through the MFMAs of slab s and the loads of slab s + 2 follow at once. LDS
- * holds 16-byte chunks of 16 k, chunk-major; an operand that is contiguous along m / n is transposed in registers
- * (bytes picked with v_perm_b32) and its rows sit in permuted slots, undone when C is written.
+ * holds an operand that is contiguous along k as 16-byte chunks of 16 k, chunk-major; one that is contiguous along m / n
+ * as it lies in memory, and its fragments come out of transposing LDS reads (ds_read_b64_tr_b8).
  */
 #include "och_gemm.h"
 
@@ -18,6 +18,7 @@ namespace och {
 
 typedef int och_i32x4  __attribute__((ext_vector_type(4)));
 typedef int och_i32x16 __attribute__((ext_vector_type(16)));
+typedef int och_i32x2  __attribute__((ext_vector_type(2)));
 
 struct ByteGemmParams
 {
@@ -37,25 +38,28 @@ struct ByteGemmParams
 __device__ __forceinline__ uint32_t bool_bytes(uint32_t x)
 {  return ((((x & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | x) & 0x80808080u) >> 7; }
 
-/* Moves a BMN x KT slab of an operand (1-byte elements) from memory to registers and on to LDS.
-   LDS layout: [chunk of 16 k][slot][16 bytes], 32 bytes of padding after every chunk plane.
-   KC (contiguous along k in memory): a thread loads one chunk of one row; row r sits in slot r.
-   !KC (contiguous along the row index): a thread loads NV consecutive k for 16 neighbouring rows, transposes the 16 x NV
-   block in registers and stores NV k for each of the 16 rows; row r sits in slot (r mod 16) * (BMN / 16) + r / 16, so
-   that the stores of a wave cover consecutive slots. */
+/* Moves a BMN x KT slab of an operand (1-byte elements) from memory to registers and on to LDS, 16 bytes at a time, and
+   reads MFMA fragments (sixteen consecutive k of one row per lane) from there.
+   KC (contiguous along k in memory): a thread loads one chunk of 16 k of one row; LDS holds [chunk of 16 k][row][16 bytes],
+   32 bytes of padding after every chunk plane; a fragment is one 16-byte read.
+   !KC (contiguous along the row index): a thread loads 16 neighbouring rows of one k, for NV consecutive k, and LDS holds
+   the slab as it lies in memory, [k][row] with a pitch of BMN + 16 bytes. The fragments come out of transposing reads
+   (ds_read_b64_tr_b8): in every group of 16 lanes, lanes 2 e and 2 e + 1 read 16 neighbouring rows of k + e, and lane i of
+   the group receives row i of k .. k + 7; two such reads make the sixteen k of a fragment. */
 template <bool KC, bool EDGE, bool BOOL, int BMN, int KT, int THREADS>
 struct ByteSlab
 {
    static constexpr int NV = BMN * KT / 16 / THREADS;                  /* 16-byte loads per thread */
    static constexpr int G = BMN / 16;                                  /* groups of 16 rows */
-   static constexpr int PLANE = BMN * 16 + 32;                         /* bytes per chunk plane */
-   static constexpr int SIZE = (KT / 16) * PLANE;                      /* bytes per LDS buffer */
+   static constexpr int PLANE = BMN * 16 + 32;                         /* KC: bytes per chunk plane */
+   static constexpr int PITCH = BMN + 16;                              /* !KC: bytes from one k to the next; 16 more than the rows so that the eight k of a transposing read meet different banks */
+   static constexpr int SIZE = KC ? (KT / 16) * PLANE : KT * PITCH;    /* bytes per LDS buffer */
    static_assert(NV >= 1 && (BMN * KT) % (16 * THREADS) == 0, "slab does not divide among the threads");
-   static_assert(KC || NV == 2 || NV == 4 || NV == 8, "the transposing loader needs 2, 4 or 8 k per thread");
    och_gu32x4 reg[NV];
 
-   static __device__ __forceinline__ uint32_t row_of_slot(uint32_t slot) { return KC ? slot : (slot % G) * 16 + slot / G; }
-   static constexpr uint32_t row_step(uint32_t o) { return KC ? o : (o % G) * 16 + o / G; }
+   /* LDS slot -> row of the tile: the same for both layouts (kept as the one place that says so) */
+   static __device__ __forceinline__ uint32_t row_of_slot(uint32_t slot) { return slot; }
+   static constexpr uint32_t row_step(uint32_t o) { return o; }
    static __device__ __forceinline__ void where(int v, uint32_t &mn, uint32_t &k)
    {  if (!KC) { mn = (threadIdx.x % G) * 16; k = (threadIdx.x / G) * NV + v; }
       else     { const uint32_t q = threadIdx.x + THREADS * v; k = (q % (KT / 16)) * 16; mn = q / (KT / 16); }
@@ -99,31 +103,14 @@ struct ByteSlab
       }
       else
       {  uint32_t mn, k; where(0, mn, k);
-         char *dst = buffer + (k / 16) * PLANE + (mn / 16) * 16 + k % 16;         /* row mn + i: slot i * G + mn / 16 */
 #pragma unroll
-         for (int i = 0; i < 16; i++)
-         {  /* byte i of every loaded vector, in the order of k */
-            const uint32_t sel = 0x0C0C0400u + (uint32_t)(i & 3) * 0x0101u;        /* bytes: b[i & 3] of the low, of the high operand, 0, 0 */
-            const uint32_t lo = __builtin_amdgcn_perm(reg[1][i >> 2], reg[0][i >> 2], sel);
-            if (NV == 2) *reinterpret_cast<uint16_t *>(dst + i * (G * 16)) = (uint16_t)lo;
-            else
-            {  const uint32_t hi = __builtin_amdgcn_perm(reg[NV > 2 ? 3 : 1][i >> 2], reg[NV > 2 ? 2 : 0][i >> 2], sel);
-               const uint32_t w0 = (lo & 0xFFFFu) | (hi << 16);
-               if (NV == 4) *reinterpret_cast<uint32_t *>(dst + i * (G * 16)) = w0;
-               else
-               {  const uint32_t lo2 = __builtin_amdgcn_perm(reg[NV > 4 ? 5 : 1][i >> 2], reg[NV > 4 ? 4 : 0][i >> 2], sel);
-                  const uint32_t hi2 = __builtin_amdgcn_perm(reg[NV > 4 ? 7 : 1][i >> 2], reg[NV > 4 ? 6 : 0][i >> 2], sel);
-                  uint2 t; t.x = w0; t.y = (lo2 & 0xFFFFu) | (hi2 << 16);
-                  *reinterpret_cast<uint2 *>(dst + i * (G * 16)) = t;
-               }
-            }
-         }
+         for (int v = 0; v < NV; v++) *reinterpret_cast<och_gu32x4 *>(buffer + (k + v) * PITCH + mn) = reg[v];
       }
    }
    /* The same in single instructions, for the loop that places every one of them by hand (whole tiles, no bool): load
       number v as a scalar base (the slab's first element, the same for all threads) + a step per v + the thread's own
       offset, which does not change from slab to slab; and store number `piece` of the PIECES that move the registers to LDS */
-   static constexpr int PIECES = KC ? NV : 16;
+   static constexpr int PIECES = NV;
    static __device__ __forceinline__ uint32_t thread_offset(int64_t ld)
    {  uint32_t mn, k; where(0, mn, k);
       return (uint32_t)(KC ? ((int64_t)k + (int64_t)mn * ld) : ((int64_t)mn + (int64_t)k * ld));
@@ -135,28 +122,26 @@ struct ByteSlab
       reg[v] = *reinterpret_cast<const och_gu32x4 *>(base + step + toff);
    }
    __device__ __forceinline__ void stash_one(char *buffer, int piece) const
-   {  static_assert(KC || NV == 8 || NV == 4, "a transposed piece is a store of 8 or 4 bytes");
-      if (KC)
-      {  uint32_t mn, k; where(piece, mn, k);
-         *reinterpret_cast<och_gu32x4 *>(buffer + (k / 16) * PLANE + mn * 16) = reg[piece];
-      }
-      else
-      {  uint32_t mn, k; where(0, mn, k);
-         char *at = buffer + (k / 16) * PLANE + (mn / 16) * 16 + k % 16 + piece * (G * 16);
-         const uint32_t sel = 0x0C0C0400u + (uint32_t)(piece & 3) * 0x0101u;
-         uint32_t pair[NV / 2];
-#pragma unroll
-         for (int w = 0; w < NV / 2; w++) pair[w] = __builtin_amdgcn_perm(reg[2 * w + 1][piece >> 2], reg[2 * w][piece >> 2], sel);
-         const uint32_t w0 = (pair[0] & 0xFFFFu) | (pair[1] << 16);
-         if (NV == 4) *reinterpret_cast<uint32_t *>(at) = w0;
-         else { uint2 t; t.x = w0; t.y = (pair[NV > 4 ? 2 : 0] & 0xFFFFu) | (pair[NV > 4 ? 3 : 1] << 16); *reinterpret_cast<uint2 *>(at) = t; }
-      }
+   {  uint32_t mn, k; where(piece, mn, k);
+      if (KC) *reinterpret_cast<och_gu32x4 *>(buffer + (k / 16) * PLANE + mn * 16) = reg[piece];
+      else    *reinterpret_cast<och_gu32x4 *>(buffer + k * PITCH + mn) = reg[piece];
    }
    /* the sixteen k of slot `slot` that lane group `kg` (0 or 1) feeds to MFMA step `ks` (32 k per step) */
    static __device__ __forceinline__ och_i32x4 fragment(const char *buffer, int slot, int ks, int kg)
    {  och_i32x4 f;
-      const och_gu32x4 raw = *reinterpret_cast<const och_gu32x4 *>(buffer + (ks * 2 + kg) * PLANE + slot * 16);
-      __builtin_memcpy(&f, &raw, 16);
+      if (KC)
+      {  const och_gu32x4 raw = *reinterpret_cast<const och_gu32x4 *>(buffer + (ks * 2 + kg) * PLANE + slot * 16);
+         __builtin_memcpy(&f, &raw, 16);
+      }
+      else
+      {  /* slot = first row of the tile + lane % 32; this lane reads rows (slot - lane % 16) + 8 (lane % 2) .. + 7 of
+            k + (lane % 16) / 2 and receives row `slot` of k .. k + 7 */
+         const int lane = threadIdx.x & 63;
+         const char *at = buffer + (ks * 32 + kg * 16 + ((lane & 15) >> 1)) * PITCH + (slot - (lane & 15)) + 8 * (lane & 1);
+         const och_i32x2 lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) och_i32x2 *)at);
+         const och_i32x2 hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) och_i32x2 *)(at + 8 * PITCH));
+         f.x = lo.x; f.y = lo.y; f.z = hi.x; f.w = hi.y;
+      }
       return f;
    }
 };
