@@ -208,6 +208,17 @@ def test_kernel_choice():
     assert p.div_d[0] == 1 and fastdiv(12345, 1, p.div_m[0], p.div_s1[0], p.div_s2[0]) == 12345
 
 
+def test_gemm_kernel_choice_knob_checks_its_argument():
+    """och_gemm_set_kernel_choice touches no device: 0 to 3 are accepted, anything else is refused with a message."""
+    import ocean_hip as oh
+    for choice in (1, 2, 3, 0):
+        assert oh.lib.och_gemm_set_kernel_choice(choice) == 0
+    for choice in (-1, 4, 99):
+        assert oh.lib.och_gemm_set_kernel_choice(choice) != 0
+        assert b"kernel choice" in oh.lib.och_last_error()
+    assert oh.lib.och_gemm_set_kernel_choice(0) == 0
+
+
 def test_cutting_the_last_round_of_a_product_along_k():
     """och_gemm_split_plan (host arithmetic only): known answers, and for shapes from a fixed seed the rules a cut has to
     keep -- only a last round that is at most half full is cut, at most 8 shares per tile (64 for a product of less than
