@@ -282,6 +282,58 @@ static OcTensor *scalar_tensor(OcScalar *s, OcDType dtype, double fallback)
    }
    return t;
 }
+/* value converted to the given type (OcScalar_castTo, src/base/scalar.c), through the one-element tensor above */
+static int scalar_cast(OcScalar *value, OcDType dtype, OcScalar *result)
+{  OcTensor *t;
+   if (value->dtype == dtype) { *result = *value; return 0; }
+   if ((t = scalar_tensor(value, dtype, 0)) == NULL) return -1;
+   memset(result, 0, sizeof(*result));
+   result->dtype = dtype;
+   memcpy(&result->value, OcTensor_data(t), (size_t)t->elemsize);
+   OcDecrefTensor(t);
+   return 0;
+}
+/* tensor_itf.c:2788-2826: NaN entries are replaced by the value in the tensor's type; integer tensors are left alone */
+int OcTensor_fillNaN(OcTensor *tensor, OcScalar *value)
+{  OcScalar v; MODULE_OR_FAIL(m, tensor->device);
+   if (m->Tensor_fillNaN == NULL) OcError(-1, "Tensor fill NaN is not supported on device %s", tensor->device->name);
+   if (!OcDType_isFloat(tensor->dtype)) return 0;
+   if (scalar_cast(value, tensor->dtype, &v) != 0) return -1;
+   return m->Tensor_fillNaN(tensor, &v);
+}
+/* tensor_itf.c:2864-2908: the value is converted to the tensor's type, the mask is broadcast to the tensor's shape
+   and brought to bool on the tensor's device, then the device function runs */
+int OcTensor_maskedFill(OcTensor *tensor, OcTensor *mask, OcScalar *value)
+{  OcScalar v; OcTensor *view = NULL, *m1 = NULL; int result = -1;
+   MODULE_OR_FAIL(m, tensor->device);
+   if (m->Tensor_maskedFill == NULL) OcError(-1, "Tensor masked fill is not supported on device %s", tensor->device->name);
+   if (scalar_cast(value, tensor->dtype, &v) != 0) return -1;
+   m1 = OcIncrefTensor(mask);
+   if (tensor_ensure(&m1, OcDTypeBool, tensor->device, 1) != 0) goto final;
+   if ((view = OcTensor_broadcastTo(m1, tensor->ndims, tensor->size)) == NULL) goto final;
+   if (OcTensor_isByteswapped(tensor))
+   {  /* the stored bytes are in the other order: fill with the swapped value (each part of a complex value by itself) */
+      int parts = OcDType_isComplex(tensor->dtype) ? 2 : 1, w = tensor->elemsize / parts, i, j; char *b = (char *)&v.value;
+      for (j = 0; j < parts; j++) for (i = 0; i < w / 2; i++) { char c = b[j * w + i]; b[j * w + i] = b[j * w + w - 1 - i]; b[j * w + w - 1 - i] = c; }
+   }
+   result = m->Tensor_maskedFill(tensor, view, &v);
+final:
+   if (view) OcDecrefTensor(view);
+   if (m1) OcDecrefTensor(m1);
+   return result;
+}
+/* value(i) = offset + i * step over the flat index, first dimension fastest (the building block of OcTensor_range and
+   OcTensor_linspace, tensor_itf.c:2965-3075) */
+int OcTensor_stepsInt64(OcTensor *tensor, OcInt64 offset, OcInt64 step)
+{  MODULE_OR_FAIL(m, tensor->device);
+   if (m->Tensor_stepsInt64 == NULL) OcError(-1, "Tensor steps is not supported on device %s", tensor->device->name);
+   return m->Tensor_stepsInt64(tensor, offset, step);
+}
+int OcTensor_stepsDouble(OcTensor *tensor, OcDouble offset, OcDouble step)
+{  MODULE_OR_FAIL(m, tensor->device);
+   if (m->Tensor_stepsDouble == NULL) OcError(-1, "Tensor steps is not supported on device %s", tensor->device->name);
+   return m->Tensor_stepsDouble(tensor, offset, step);
+}
 /* leading dimension of a matrix operand, flipping the mode when only its rows are contiguous */
 static int gemm_operand(OcTensor **t, char *mode, OcIndex *ld, int complex_type)
 {  OcTensor *x = *t; int es = x->elemsize;

@@ -24,6 +24,10 @@ OcTensor *OcTensor_broadcastTo(OcTensor *tensor, int ndims, const OcSize *size);
 int OcTensor_copy(OcTensor *src, OcTensor *dst);                                   /* any device, dtype, byte order */
 int OcTensor_ensure(OcTensor **tensor, OcDType dtype, OcDevice *device);           /* replaces *tensor by a converted native-order copy when needed */
 int OcTensor_fill(OcTensor *tensor, OcScalar *value);
+int OcTensor_fillNaN(OcTensor *tensor, OcScalar *value);                           /* value converted to the tensor's type */
+int OcTensor_maskedFill(OcTensor *tensor, OcTensor *mask, OcScalar *value);        /* mask: any type / device, broadcast to the tensor */
+int OcTensor_stepsInt64(OcTensor *tensor, OcInt64 offset, OcInt64 step);           /* value(i) = offset + i * step, flat index */
+int OcTensor_stepsDouble(OcTensor *tensor, OcDouble offset, OcDouble step);
 OcTensor *OcTensor_find(OcTensor *mask);                                         /* ndims x nnz indices of the non-zero elements */
 OcTensor *OcTensor_maskToOffset(OcTensor *mask, OcIndex *strides);               /* nnz offsets sum(index * strides) */
 int OcTensor_binary(int op, OcTensor *src1, OcTensor *src2, OcTensor **dst);       /* op: index into the table's binary block */

@@ -19,13 +19,17 @@
 typedef struct { OcStream HEAD; och_stream handle; } OcStreamGPU;
 typedef struct { OcEvent HEAD; och_event handle; } OcEventGPU;
 typedef struct { OcStorage HEAD; } OcStorageGPU;
+/* the module's device object: the public part (OcDeviceGPU of include/ocean_gpu_module.h: properties under the
+   reference's names, free lists) followed by what only this file uses */
 typedef struct
-{  OcDevice        HEAD;
-   och_device_prop properties;
-   OcStream       *freeStreams;  int nFreeStreams;
-   OcEvent        *freeEvents;   int nFreeEvents;
+{  OcDeviceGPU     pub;
+   och_device_prop hip;                                                /* as the device library reports them */
    long            eventsRecorded, eventsWaited, streamsCreated;      /* activity counters (OcDeviceGPU_activity) */
-} OcDeviceGPU;
+} OcDeviceGPUFull;
+#define freeStreams  pub.streamBuffer
+#define nFreeStreams pub.streamCount
+#define freeEvents   pub.eventBuffer
+#define nFreeEvents  pub.eventCount
 /* the context of the core module on a GPU device: the interface's part first (module_core_gpu.h:28-32 has the BLAS
    handle behind it; the MFMA GEMM kernels need none) */
 typedef struct { OcModuleCore_Context HEAD; int deviceIndex; } OcModuleCoreGPU_Context;
@@ -41,7 +45,7 @@ static OcModuleCore oc_module_core_gpu;          /* the table that registration 
 static int activate(OcDevice *device) { if (och_device_set(device->index) != 0) OcError(-1, "%s", och_last_error()); return 0; }
 
 static OcStream *OcDeviceGPU_createStream(OcDevice *device)
-{  OcDeviceGPU *g = (OcDeviceGPU *)device; OcStreamGPU *s;
+{  OcDeviceGPUFull *g = (OcDeviceGPUFull *)device; OcStreamGPU *s;
    if (g->freeStreams)
    {  s = (OcStreamGPU *)g->freeStreams; g->freeStreams = s->HEAD.next; g->nFreeStreams--; }
    else
@@ -56,14 +60,14 @@ static OcStream *OcDeviceGPU_createStream(OcDevice *device)
 }
 /* called by OcDecrefStream when the last reference goes (device.c:225-236, after synchronising the stream) */
 static void OcDeviceGPU_deleteStream(OcStream *stream)
-{  OcDeviceGPU *g;
+{  OcDeviceGPUFull *g;
    if (stream == NULL) return;
-   g = (OcDeviceGPU *)stream->device;
+   g = (OcDeviceGPUFull *)stream->device;
    if (g->nFreeStreams < OC_GPU_MAX_FREE) { stream->next = g->freeStreams; g->freeStreams = stream; g->nFreeStreams++; }
    else { och_stream_destroy(((OcStreamGPU *)stream)->handle); OcFree(stream); }
 }
 static int OcDeviceGPU_createEvent(OcDevice *device, OcEvent **event)
-{  OcDeviceGPU *g = (OcDeviceGPU *)device; OcEventGPU *e;
+{  OcDeviceGPUFull *g = (OcDeviceGPUFull *)device; OcEventGPU *e;
    if (g->freeEvents) { e = (OcEventGPU *)g->freeEvents; g->freeEvents = e->HEAD.next; g->nFreeEvents--; }
    else
    {  if (activate(device) != 0) return -1;
@@ -75,7 +79,7 @@ static int OcDeviceGPU_createEvent(OcDevice *device, OcEvent **event)
    return 0;
 }
 static void OcDeviceGPU_deleteEvent(OcDevice *device, OcEvent *event)
-{  OcDeviceGPU *g = (OcDeviceGPU *)device;
+{  OcDeviceGPUFull *g = (OcDeviceGPUFull *)device;
    if (event == NULL) return;
    if (g->nFreeEvents < OC_GPU_MAX_FREE) { event->next = g->freeEvents; g->freeEvents = event; g->nFreeEvents++; }
    else { och_event_destroy(((OcEventGPU *)event)->handle); OcFree(event); }
@@ -83,23 +87,43 @@ static void OcDeviceGPU_deleteEvent(OcDevice *device, OcEvent *event)
 static int OcStreamGPU_synchronize(OcStream *s)  { OCH_CALL(och_stream_synchronize(((OcStreamGPU *)s)->handle)); return 0; }
 static int OcEventGPU_synchronize(OcEvent *e)    { OCH_CALL(och_event_synchronize(((OcEventGPU *)e)->handle)); return 0; }
 static int OcEventGPU_record(OcEvent *e, OcStream *s)
-{  ((OcDeviceGPU *)s->device)->eventsRecorded++;
+{  ((OcDeviceGPUFull *)s->device)->eventsRecorded++;
    OCH_CALL(och_event_record(((OcEventGPU *)e)->handle, ((OcStreamGPU *)s)->handle)); return 0;
 }
 static int OcStreamGPU_waitEvent(OcStream *s, OcEvent *e)
-{  ((OcDeviceGPU *)s->device)->eventsWaited++;
+{  ((OcDeviceGPUFull *)s->device)->eventsWaited++;
    OCH_CALL(och_stream_wait_event(((OcStreamGPU *)s)->handle, ((OcEventGPU *)e)->handle)); return 0;
 }
 static void OcFreeDeviceGPU(OcDevice *device)
-{  OcDeviceGPU *g = (OcDeviceGPU *)device;
+{  OcDeviceGPUFull *g = (OcDeviceGPUFull *)device;
    och_device_set(device->index);
    while (g->freeStreams) { OcStream *s = g->freeStreams; g->freeStreams = s->next; och_stream_destroy(((OcStreamGPU *)s)->handle); OcFree(s); }
    while (g->freeEvents)  { OcEvent *e = g->freeEvents; g->freeEvents = e->next; och_event_destroy(((OcEventGPU *)e)->handle); OcFree(e); }
 }
+/* device_gpu.c:471-616: the properties under the reference's field names */
+static void fill_public_properties(OcDevicePropGPU *q, const och_device_prop *p)
+{  int i;
+   memset(q, 0, sizeof(*q));
+   memcpy(q->name, p->name, sizeof(q->name)); q->name[sizeof(q->name) - 1] = 0;
+   q->totalGlobalMem = p->total_global_mem; q->freeGlobalMem = p->free_global_mem; q->sharedMemPerBlock = p->shared_mem_per_block;
+   q->regsPerBlock = p->regs_per_block; q->warpSize = p->wavefront_size; q->memPitch = p->mem_pitch;
+   q->maxThreadsPerBlock = p->max_threads_per_block;
+   for (i = 0; i < 3; i++) { q->maxThreadsDim[i] = p->max_threads_dim[i]; q->maxGridSize[i] = p->max_grid_size[i]; }
+   q->clockRate = p->clock_rate_khz; q->totalConstMem = p->total_const_mem; q->major = p->major; q->minor = p->minor;
+   q->deviceOverlap = p->async_engine_count > 0; q->multiProcessorCount = p->multiprocessor_count;
+   q->kernelExecTimeoutEnabled = p->kernel_exec_timeout_enabled; q->integrated = p->integrated;
+   q->canMapHostMemory = p->can_map_host_memory; q->computeMode = p->compute_mode; q->concurrentKernels = p->concurrent_kernels;
+   q->ECCEnabled = p->ecc_enabled; q->pciBusID = p->pci_bus_id; q->pciDeviceID = p->pci_device_id; q->pciDomainID = p->pci_domain_id;
+   q->tccDriver = p->tcc_driver; q->asyncEngineCount = p->async_engine_count; q->unifiedAddressing = 1;
+   q->memoryClockRate = p->memory_clock_rate_khz; q->memoryBusWidth = p->memory_bus_width; q->l2CacheSize = p->l2_cache_size;
+   q->maxThreadsPerMultiProcessor = p->max_threads_per_multiprocessor;
+   q->sharedMemPerMultiprocessor = p->shared_mem_per_block; q->maxSharedMemPerSM = (int)p->shared_mem_per_block;
+   q->maxWarpsPerMultiProcessor = p->wavefront_size > 0 ? p->max_threads_per_multiprocessor / p->wavefront_size : 0;
+}
 /* device_gpu.c:81-122. A GPU device has NO default stream: every storage gets a stream of its own (storage.c:94-103),
    so that operations on different tensors overlap and are ordered by the read / write protocol only. */
 static OcDevice *OcCreateDeviceGPU(OcDeviceType *type, int index, const char *name)
-{  OcDevice *device = OcCreateDevice(type, index, name, sizeof(OcDeviceGPU)); OcDeviceGPU *g = (OcDeviceGPU *)device;
+{  OcDevice *device = OcCreateDevice(type, index, name, sizeof(OcDeviceGPUFull)); OcDeviceGPUFull *g = (OcDeviceGPUFull *)device;
    if (device == NULL) return NULL;
    device->finalize = OcFreeDeviceGPU; device->endianness = 0; device->requiresAlignedData = 1;
    device->create_stream = OcDeviceGPU_createStream; device->create_event = OcDeviceGPU_createEvent;
@@ -108,8 +132,9 @@ static OcDevice *OcCreateDeviceGPU(OcDeviceType *type, int index, const char *na
    device->record_event = OcEventGPU_record;          device->wait_event = OcStreamGPU_waitEvent;
    g->freeStreams = NULL; g->nFreeStreams = 0; g->freeEvents = NULL; g->nFreeEvents = 0;
    g->eventsRecorded = g->eventsWaited = g->streamsCreated = 0;
-   if (och_device_properties(index, &g->properties) != 0 || och_device_warmup(index) != 0)          /* device_gpu.c:155-196, 471-616 */
+   if (och_device_properties(index, &g->hip) != 0 || och_device_warmup(index) != 0)                /* device_gpu.c:155-196, 471-616 */
    {  OcErrorMessage("%s", och_last_error()); OcDecrefDevice(device); return NULL; }
+   fill_public_properties(&g->pub.properties, &g->hip);
    return device;
 }
 
@@ -139,7 +164,7 @@ error:
    OcDecrefStorage(storage);
    return NULL;
 }
-static int OcBufferGPU_copy(OcStorage *src, void *srcData, OcStorage *dst, void *dstData, OcDType dtype, OcSize n)
+int OcBufferGPU_copy(OcStorage *src, void *srcData, OcStorage *dst, void *dstData, OcDType dtype, OcSize n)
 {  if (n == 0) return 0;
    if (src->stream->device != dst->stream->device) OcError(-1, "Copies between GPU devices are not part of this build (one device)");
    if (OcStorage_startRead(dst, src) != 0 || activate(dst->stream->device) != 0) return -1;
@@ -149,38 +174,38 @@ static int OcBufferGPU_copy(OcStorage *src, void *srcData, OcStorage *dst, void 
 }
 /* the transfers between host and device block, as the reference's do (storage_gpu.c:165-250): wait for the storage's
    outstanding work, copy, record */
-static int OcBufferGPU_copyFromCPU(OcStorage *src, void *srcData, OcStorage *dst, void *dstData, OcDType dtype, OcSize n)
+int OcBufferGPU_copyFromCPU(OcStorage *src, void *srcData, OcStorage *dst, void *dstData, OcDType dtype, OcSize n)
 {  (void)src;
    if (OcStorage_synchronize(dst) != 0 || activate(dst->stream->device) != 0) return -1;
    OCH_CALL(och_memcpy_htod(dstData, srcData, (size_t)(n * OcDType_size(dtype)), ((OcStreamGPU *)dst->stream)->handle));
    return OcStorage_update(dst);
 }
-static int OcBufferGPU_copyToCPU(OcStorage *src, void *srcData, OcStorage *dst, void *dstData, OcDType dtype, OcSize n)
+int OcBufferGPU_copyToCPU(OcStorage *src, void *srcData, OcStorage *dst, void *dstData, OcDType dtype, OcSize n)
 {  if (OcStorage_synchronize(src) != 0 || activate(src->stream->device) != 0) return -1;
    OCH_CALL(och_memcpy_dtoh(dstData, srcData, (size_t)(n * OcDType_size(dtype)), ((OcStreamGPU *)src->stream)->handle));
    if (OcStorage_update(dst) != 0) return -1;
    return OcStorage_finishRead(src, src);                              /* updates the read event */
 }
-static int OcBufferGPU_copyHostStorage(OcStorage *storage, OcSize offset, OcSize nbytes, void *ptr)
+int OcBufferGPU_copyHostToStorage(OcStorage *storage, OcIndex offset, OcSize nbytes, void *ptr)
 {  if (OcStorage_synchronize(storage) != 0 || activate(storage->stream->device) != 0) return -1;
    OCH_CALL(och_memcpy_htod(storage->data + offset, ptr, (size_t)nbytes, ((OcStreamGPU *)storage->stream)->handle));
    return OcStorage_update(storage);
 }
-static int OcBufferGPU_copyStorageHost(OcStorage *storage, OcSize offset, OcSize nbytes, void *ptr)
+int OcBufferGPU_copyStorageToHost(OcStorage *storage, OcIndex offset, OcSize nbytes, void *ptr)
 {  if (OcStorage_synchronize(storage) != 0 || activate(storage->stream->device) != 0) return -1;
    OCH_CALL(och_memcpy_dtoh(ptr, storage->data + offset, (size_t)nbytes, ((OcStreamGPU *)storage->stream)->handle));
    return OcStorage_finishRead(storage, storage);
 }
-static int OcBufferGPU_zero(OcStorage *storage, void *data, OcDType dtype, OcSize size)
+int OcBufferGPU_zero(OcStorage *storage, void *data, OcDType dtype, OcSize size)
 {  if (activate(storage->stream->device) != 0) return -1;
    OCH_CALL(och_memset_async(data, 0, (size_t)(size * OcDType_size(dtype)), ((OcStreamGPU *)storage->stream)->handle));
    return OcStorage_update(storage);
 }
 static int OcDeviceGPU_formatInfo(OcDevice *device, char **str, const char *header, const char *footer)
-{  OcDeviceGPU *g = (OcDeviceGPU *)device; size_t n = 512 + (header ? strlen(header) : 0) + (footer ? strlen(footer) : 0);
+{  OcDeviceGPUFull *g = (OcDeviceGPUFull *)device; size_t n = 512 + (header ? strlen(header) : 0) + (footer ? strlen(footer) : 0);
    if ((*str = (char *)OcMalloc(n)) == NULL) OcError(-1, "Insufficient memory for the device description");
-   snprintf(*str, n, "%sDevice %s: %s (%s), %d compute units, %.1f GiB%s", header ? header : "", device->name, g->properties.name,
-            g->properties.arch, g->properties.multiprocessor_count, g->properties.total_global_mem / 1073741824.0, footer ? footer : "");
+   snprintf(*str, n, "%sDevice %s: %s (%s), %d compute units, %.1f GiB%s", header ? header : "", device->name, g->hip.name,
+            g->hip.arch, g->hip.multiprocessor_count, g->hip.total_global_mem / 1073741824.0, footer ? footer : "");
    return 0;
 }
 
@@ -567,25 +592,38 @@ static void finalizeContext(OcDevice *device, OcDeviceModule *deviceModule, void
 }
 static void finalizeModule(OcDeviceModule *deviceModule) { (void)deviceModule; }
 
-static void initializeFunctions(OcModuleCore *m)
-{  memset(m, 0, sizeof(*m));
-   m->HEAD.module = &oc_module_core;               /* registration increments its reference count */
-   m->HEAD.initializeContext = initializeContext; m->HEAD.finalizeContext = finalizeContext; m->HEAD.finalizeModule = finalizeModule;
-   m->Device_formatInfo = OcDeviceGPU_formatInfo;
+/* The table is assembled from the same pieces as the reference's (module_core_gpu.c:40-63, tensor_gpu.c:35-50) */
+int OcRegisterDevicesGPU(OcModuleCore *m) { m->Device_formatInfo = OcDeviceGPU_formatInfo; return 0; }
+int OcRegisterStorageGPU(OcModuleCore *m)
+{  m->Storage_create = OcStorageGPU_create; m->Storage_fromObject = NULL;
    m->Buffer_copy = OcBufferGPU_copy; m->Buffer_copyFromCPU = OcBufferGPU_copyFromCPU; m->Buffer_copyToCPU = OcBufferGPU_copyToCPU;
-   m->Buffer_copyHostStorage = OcBufferGPU_copyHostStorage; m->Buffer_copyStorageHost = OcBufferGPU_copyStorageHost; m->Buffer_zero = OcBufferGPU_zero;
-   m->Storage_create = OcStorageGPU_create; m->Storage_fromObject = NULL;
-   m->Tensor_copy = OcTensorGPU_copy; m->Tensor_copyFromCPU = OcTensorGPU_copyFromCPU; m->Tensor_copyToCPU = OcTensorGPU_copyToCPU;
-   m->Tensor_byteswapNoFlag = OcTensorGPU_byteswapNoFlag;
-   m->Tensor_fill = OcTensorGPU_fill; m->Tensor_fillNaN = OcTensorGPU_fillNaN; m->Tensor_maskedFill = OcTensorGPU_maskedFill;
-   m->Tensor_stepsInt64 = OcTensorGPU_stepsInt64; m->Tensor_stepsDouble = OcTensorGPU_stepsDouble; m->Tensor_stepsCDouble = OcTensorGPU_stepsCDouble;
-   m->Tensor_find = OcTensorGPU_find; m->Tensor_maskToOffset = OcTensorGPU_maskToOffset;   /* empty in the reference's GPU table (docs/future_work.md:33) */
+   m->Buffer_copyHostStorage = OcBufferGPU_copyHostToStorage; m->Buffer_copyStorageHost = OcBufferGPU_copyStorageToHost; m->Buffer_zero = OcBufferGPU_zero;
+   return 0;
+}
+void OcTensorGPU_initializeCopyOps(OcModuleCore *m)
+{  m->Tensor_copy = OcTensorGPU_copy; m->Tensor_copyFromCPU = OcTensorGPU_copyFromCPU; m->Tensor_copyToCPU = OcTensorGPU_copyToCPU;
+   m->Tensor_byteswapNoFlag = OcTensorGPU_byteswapNoFlag;          /* CPU-only in the reference (template_byteswap.c:27-34) */
+}
+void OcTensorGPU_initializeFillOps(OcModuleCore *m)
+{  m->Tensor_fill = OcTensorGPU_fill; m->Tensor_fillNaN = OcTensorGPU_fillNaN; m->Tensor_maskedFill = OcTensorGPU_maskedFill; }
+void OcTensorGPU_initializeStepOps(OcModuleCore *m)
+{  m->Tensor_stepsInt64 = OcTensorGPU_stepsInt64; m->Tensor_stepsDouble = OcTensorGPU_stepsDouble; m->Tensor_stepsCDouble = OcTensorGPU_stepsCDouble; }
+void OcTensorGPU_initializeIndexOps(OcModuleCore *m)
+{  m->Tensor_find = OcTensorGPU_find; m->Tensor_maskToOffset = OcTensorGPU_maskToOffset;   /* empty in the reference's GPU table (docs/future_work.md:33) */
    m->Tensor_indexToOffset = OcTensorGPU_indexToOffset; m->Tensor_addIfNegative = OcTensorGPU_addIfNegative;
    m->Tensor_getIndex = OcTensorGPU_getIndex; m->Tensor_setIndex = OcTensorGPU_setIndex; m->Tensor_fillIndex = OcTensorGPU_fillIndex;
+}
 #define OC_X(NAME, OP) m->Tensor_##NAME = OcTensorGPU_##NAME;
-   OC_UNARY_TABLE(OC_X) OC_BINARY_TABLE(OC_X) OC_AXIS_TABLE(OC_X)
+void OcTensorGPU_initializeUnaryOps(OcModuleCore *m)  { OC_UNARY_TABLE(OC_X) }
+void OcTensorGPU_initializeBinaryOps(OcModuleCore *m) { OC_BINARY_TABLE(OC_X) }
+void OcTensorGPU_initializeReduceAxisOps(OcModuleCore *m)
+{  OC_AXIS_TABLE(OC_X)
+   m->Tensor_axisNorm = OcTensorGPU_axisNorm; m->Tensor_axisNormNaN = OcTensorGPU_axisNormNaN;
+}
 #undef OC_X
-   m->Tensor_allGELE = OcTensorGPU_allGELE; m->Tensor_allGELT = OcTensorGPU_allGELT; m->Tensor_allGTLE = OcTensorGPU_allGTLE; m->Tensor_allGTLT = OcTensorGPU_allGTLT;
+void OcTensorGPU_initializeBlasOps(OcModuleCore *m) { m->Tensor_gemm = OcTensorGPU_gemm; m->Tensor_gemmSupportedOn = OcTensorGPU_gemmSupportedOn; }
+void OcTensorGPU_initializeReduceAllOps(OcModuleCore *m)
+{  m->Tensor_allGELE = OcTensorGPU_allGELE; m->Tensor_allGELT = OcTensorGPU_allGELT; m->Tensor_allGTLE = OcTensorGPU_allGTLE; m->Tensor_allGTLT = OcTensorGPU_allGTLT;
    m->Tensor_allLE = OcTensorGPU_allLE; m->Tensor_allLT = OcTensorGPU_allLT; m->Tensor_allGE = OcTensorGPU_allGE; m->Tensor_allGT = OcTensorGPU_allGT;
    m->Tensor_any = OcTensorGPU_any; m->Tensor_all = OcTensorGPU_all; m->Tensor_allFinite = OcTensorGPU_allFinite; m->Tensor_anyInf = OcTensorGPU_anyInf;
    m->Tensor_anyNaN = OcTensorGPU_anyNaN; m->Tensor_nnz = OcTensorGPU_nnz; m->Tensor_nnzNaN = OcTensorGPU_nnzNaN;
@@ -593,8 +631,19 @@ static void initializeFunctions(OcModuleCore *m)
    m->Tensor_sumAbs = OcTensorGPU_sumAbs; m->Tensor_sumAbsNaN = OcTensorGPU_sumAbsNaN; m->Tensor_maximum = OcTensorGPU_maximum; m->Tensor_minimum = OcTensorGPU_minimum;
    m->Tensor_maximumAbs = OcTensorGPU_maximumAbs; m->Tensor_minimumAbs = OcTensorGPU_minimumAbs; m->Tensor_norm2 = OcTensorGPU_norm2; m->Tensor_norm2NaN = OcTensorGPU_norm2NaN;
    m->Tensor_norm = OcTensorGPU_norm; m->Tensor_normNaN = OcTensorGPU_normNaN;
-   m->Tensor_axisNorm = OcTensorGPU_axisNorm; m->Tensor_axisNormNaN = OcTensorGPU_axisNormNaN;
-   m->Tensor_gemm = OcTensorGPU_gemm; m->Tensor_gemmSupportedOn = OcTensorGPU_gemmSupportedOn;
+}
+int OcRegisterTensorGPU(OcModuleCore *m)
+{  OcTensorGPU_initializeCopyOps(m); OcTensorGPU_initializeFillOps(m); OcTensorGPU_initializeStepOps(m);
+   OcTensorGPU_initializeIndexOps(m); OcTensorGPU_initializeUnaryOps(m); OcTensorGPU_initializeBinaryOps(m);
+   OcTensorGPU_initializeBlasOps(m); OcTensorGPU_initializeReduceAllOps(m); OcTensorGPU_initializeReduceAxisOps(m);
+   return 0;
+}
+static int initializeFunctions(OcModuleCore *m)
+{  memset(m, 0, sizeof(*m));
+   m->HEAD.module = &oc_module_core;               /* registration increments its reference count */
+   m->HEAD.initializeContext = initializeContext; m->HEAD.finalizeContext = finalizeContext; m->HEAD.finalizeModule = finalizeModule;
+   if (OcRegisterDevicesGPU(m) != 0 || OcRegisterStorageGPU(m) != 0 || OcRegisterTensorGPU(m) != 0) return -1;
+   return 0;
 }
 
 int OcDeviceGPUCount(void) { return oc_gpu_count; }
@@ -607,16 +656,26 @@ int OcDeviceGPU_peerAccess(int device1, int device2)
    return result;
 }
 int OcDeviceGPU_properties(OcDevice *device, void *och_device_prop_out)
-{  OcDeviceGPU *g = (OcDeviceGPU *)device; size_t total = 0;
+{  OcDeviceGPUFull *g = (OcDeviceGPUFull *)device; size_t total = 0;
    if (!OcDeviceGPU_isInstance(device) || och_device_prop_out == NULL) OcError(-1, "Device properties: not a GPU device");
-   OCH_CALL(och_device_mem_info(device->index, &g->properties.free_global_mem, &total));
-   memcpy(och_device_prop_out, &g->properties, sizeof(g->properties));
+   OCH_CALL(och_device_mem_info(device->index, &g->hip.free_global_mem, &total));
+   g->pub.properties.freeGlobalMem = g->hip.free_global_mem;
+   memcpy(och_device_prop_out, &g->hip, sizeof(g->hip));
+   return 0;
+}
+/* device_gpu.c:620-637 */
+int OcDeviceGPU_updateProperties(OcDeviceGPU *device)
+{  OcDeviceGPUFull *g = (OcDeviceGPUFull *)device; size_t total = 0;
+   if (!OcDeviceGPU_isInstance((OcDevice *)device)) OcError(-1, "Update properties: not a GPU device");
+   if (och_device_mem_info(((OcDevice *)device)->index, &g->hip.free_global_mem, &total) != 0)
+      OcError(-1, "Error getting memory info in update properties function: %s", och_last_error());
+   device->properties.freeGlobalMem = g->hip.free_global_mem;
    return 0;
 }
 /* events recorded, stream waits issued and streams created on a GPU device since it was created (no counterpart in the
    reference): what a test needs to see that operands on different streams really go through the event protocol */
 int OcDeviceGPU_activity(OcDevice *device, long *eventsRecorded, long *eventsWaited, long *streamsCreated)
-{  OcDeviceGPU *g = (OcDeviceGPU *)device;
+{  OcDeviceGPUFull *g = (OcDeviceGPUFull *)device;
    if (!OcDeviceGPU_isInstance(device)) OcError(-1, "Device activity: not a GPU device");
    if (eventsRecorded) *eventsRecorded = g->eventsRecorded;
    if (eventsWaited) *eventsWaited = g->eventsWaited;
@@ -635,7 +694,7 @@ static void OcFinalizeDevicesGPU(void)
    }
    oc_gpu_count = 0;
 }
-static int OcInitDevicesGPU(void)
+int OcInitDevicesGPU(void)
 {  OcDeviceType *type; OcDevice *device; char name[16]; int count = 0, index;
    if (och_device_count(&count) != 0) count = 0;
    if ((type = OcCreateDeviceType("GPU")) == NULL) return -1;
@@ -654,9 +713,9 @@ static int OcInitDevicesGPU(void)
    return 0;
 }
 /* module_core_gpu.c:127-145 */
-static int OcInitModuleCore_GPU(void)
+int OcInitModuleCore_GPU(void)
 {  if (OcModuleCore_initialize() != 0) return -1;
-   initializeFunctions(&oc_module_core_gpu);
+   if (initializeFunctions(&oc_module_core_gpu) != 0) return -1;
    return OcRegisterModule("GPU", (OcDeviceModule *)&oc_module_core_gpu, sizeof(oc_module_core_gpu));
 }
 void OcFinalizeGPU(void)

@@ -47,7 +47,9 @@ class deviceGPU(object):
     deviceName = property(lambda self: self._prop().name.decode(), doc="device name")
     totalGlobalMem = property(lambda self: int(self._prop().total_global_mem), doc="total amount of global memory on the device in bytes")
     totalMem = totalGlobalMem
-    freeMem = property(lambda self: int(self._prop().free_global_mem), doc="free amount of global memory on the device in bytes")
+    # pyOcean_device_gpu.c:199-206: refreshed through OcDeviceGPU_updateProperties, then read from the device object
+    freeMem = property(lambda self: int(_host.gpu_public_properties(self._handle, update=True).freeGlobalMem),
+                       doc="free amount of global memory on the device in bytes")
     sharedMemPerBlock = property(lambda self: int(self._prop().shared_mem_per_block), doc="maximum amount of shared memory available to a thread block")
     regsPerBlock = property(lambda self: self._prop().regs_per_block, doc="maximum number of 32-bit registers available to a thread block")
     warpSize = property(lambda self: self._prop().wavefront_size, doc="warp size in threads")

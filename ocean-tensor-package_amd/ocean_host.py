@@ -62,6 +62,35 @@ class ReduceAxis(C.Structure):
                 ("strides2", C.c_ssize_t * 8), ("rstrides", C.c_ssize_t * 8), ("ptr1", C.c_void_p), ("ptr2", C.c_void_p)]
 
 
+class DevicePropGPU(C.Structure):
+    """OcDevicePropGPU (include/ocean_gpu_module.h; the reference's include/ocean/core/gpu/device_gpu.h:31-106)."""
+    _fields_ = ([("name", C.c_char * 256), ("totalGlobalMem", C.c_size_t), ("freeGlobalMem", C.c_size_t), ("sharedMemPerBlock", C.c_size_t),
+                 ("regsPerBlock", C.c_int), ("warpSize", C.c_int), ("memPitch", C.c_size_t), ("maxThreadsPerBlock", C.c_int),
+                 ("maxThreadsDim", C.c_int * 3), ("maxGridSize", C.c_int * 3), ("clockRate", C.c_int), ("totalConstMem", C.c_size_t)]
+                + [(n, C.c_int) for n in ("major", "minor", "deviceOverlap", "multiProcessorCount", "kernelExecTimeoutEnabled", "integrated",
+                                          "canMapHostMemory", "computeMode", "concurrentKernels", "ECCEnabled", "pciBusID", "pciDeviceID",
+                                          "pciDomainID", "tccDriver", "asyncEngineCount", "unifiedAddressing", "memoryClockRate",
+                                          "memoryBusWidth", "l2CacheSize", "maxThreadsPerMultiProcessor", "streamPrioritiesSupported",
+                                          "globalL1CacheSupported", "localL1CacheSupported")]
+                + [("sharedMemPerMultiprocessor", C.c_size_t)]
+                + [(n, C.c_int) for n in ("regsPerMultiprocessor", "managedMemSupported", "isMultiGpuBoard", "multiGpuBoardGroupID",
+                                          "singleToDoublePrecisionPerfRatio", "pageableMemoryAccess", "concurrentManagedAccess",
+                                          "hostNativeAtomicSupported", "maxBlocksPerMultiProcessor", "maxWarpsPerMultiProcessor",
+                                          "maxSharedMemPerSM")])
+
+
+def gpu_public_properties(device_handle, update=False):
+    """The OcDevicePropGPU inside an OcDeviceGPU object (it follows the OcDevice head), read in place the way
+    pyOcean_device_gpu.c:181-420 reads it; update=True calls OcDeviceGPU_updateProperties first (freeMem does)."""
+    import json
+    handle = device_handle.value if isinstance(device_handle, C.c_void_p) else device_handle
+    if update:
+        lib.OcDeviceGPU_updateProperties.argtypes = [C.c_void_p]
+        check(lib.OcDeviceGPU_updateProperties(handle))
+    head = json.loads(lib.OcHost_abiLayout())["sizeof(OcDevice)"]
+    return DevicePropGPU.from_address(handle + head)
+
+
 TP = C.POINTER(Tensor)
 _ss = C.POINTER(C.c_ssize_t)
 lib.OcError_lastMessage.restype = C.c_char_p
@@ -86,6 +115,10 @@ lib.OcTensor_axisReduce.argtypes = [C.c_int, TP, C.c_int, C.POINTER(C.c_int), C.
 lib.OcTensor_gemm.argtypes = [C.POINTER(Scalar), TP, C.c_char, TP, C.c_char, C.POINTER(Scalar), C.POINTER(TP)]
 lib.OcTensor_mtimes.argtypes = [TP, TP, C.POINTER(TP)]
 lib.OcTensor_fill.argtypes = [TP, C.POINTER(Scalar)]
+lib.OcTensor_fillNaN.argtypes = [TP, C.POINTER(Scalar)]
+lib.OcTensor_maskedFill.argtypes = [TP, TP, C.POINTER(Scalar)]
+lib.OcTensor_stepsInt64.argtypes = [TP, C.c_int64, C.c_int64]
+lib.OcTensor_stepsDouble.argtypes = [TP, C.c_double, C.c_double]
 lib.OcTensorGPU_projectColumns.argtypes = [TP, TP, TP]
 lib.OcTensor_find.restype = TP
 lib.OcTensor_find.argtypes = [TP]

@@ -156,6 +156,11 @@ def test_steps(hip, stream, dtype):
         cases[0] = ("int64", (0, 1) if dtype != H.BOOL else (0, 0))
         cases[1] = ("double", (0.0, 0.25))
         cases[2] = ("cdouble", (oh.CDouble(0.0, 0.0), oh.CDouble(0.25, 0.125)))
+    # integer parameters wrap as an unsigned 64-bit sum before the conversion (template_steps.c:31-40): negative
+    # values, wrap-around of the narrow types and a sum that passes 2^64 must all come out as on the CPU
+    cases += [("int64", (-5, 3)), ("int64", (250, 1)), ("int64", (1 << 40, -(1 << 33))), ("int64", (-1, -1))]
+    if dtype >= H.HALF or dtype in (H.INT16, H.INT32, H.INT64):
+        cases += [("double", (-7.5, 1.75)), ("double", (1e-3, 1.0 / 3))]
     for kind, (a, b) in cases:
         x = H.Operand(parent, view, dtype).upload(stream)
         want = parent.copy()

@@ -194,3 +194,78 @@ def test_views_and_errors():
     # without OcInitGPU no device module is registered for a made-up device
     with pytest.raises(host.OceanError):
         host.check(host.lib.OcTensor_binary(99, t, t, C.byref(host.TP())))
+
+
+REF_GPU_HEADERS = "/root/reference/include/ocean/core/gpu"
+# Names the reference's GPU headers export that this module deliberately does not, and why:
+EXEMPT_EXPORTS = {
+    "OcInitCuda": "cuda.h:30 -- CUDA runtime bring-up; the device library initialises HIP on first use",
+    "OcCuda_setDevice": "cuda.h:33 -- takes no CUDA-typed argument, but belongs to the CUDA status helpers below; och_device_set",
+    "OcCuda_setStatus": "cuda.h:36 -- argument is a cudaError_t; the device library keeps the first-error status (och_status_check)",
+    "OcCuda_clearStatus": "cuda.h:37 -- same protocol, och_status_clear",
+    "OcCuda_checkStatus": "cuda.h:38 -- same protocol, och_status_check",
+    "OcModuleCoreGPU_cublasHandle": "module_core_gpu.h:40 -- returns a cublasHandle_t; the MFMA GEMM kernels need no handle",
+}
+
+
+def exported_symbols(path):
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", path], check=True, capture_output=True, text=True).stdout
+    return {line.split()[-1] for line in out.splitlines() if line.strip()}
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_GPU_HEADERS), reason="reference tree not present")
+def test_every_public_name_of_the_reference_gpu_headers_is_exported():
+    """Every OC_API function of include/ocean/core/gpu/**/*.h is an exported symbol of the host library, except
+    the CUDA-typed helpers listed above."""
+    import re
+    names = set()
+    for folder, _, files in os.walk(REF_GPU_HEADERS):
+        for f in files:
+            if f.endswith(".h"):
+                text = open(os.path.join(folder, f)).read()
+                names.update(re.findall(r"OC_API\s+[\w\s\*]*?\b(\w+)\s*\(", text))
+    assert len(names) >= 30 and "OcDeviceGPU_updateProperties" in names and "OcBufferGPU_zero" in names
+    have = exported_symbols(host.LIB_PATH)
+    missing = sorted(n for n in names if n not in have and n not in EXEMPT_EXPORTS)
+    assert not missing, missing
+    assert not [n for n in EXEMPT_EXPORTS if n not in names], "exemption for a name the reference does not have"
+    assert "OcGPU" in have and "OcInitGPU" in have and "OcFinalizeGPU" in have           # include/ocean_gpu.h
+
+
+def test_module_header_declares_what_the_library_exports():
+    """include/ocean_gpu_module.h and the library agree: every function the header declares is exported."""
+    import re
+    text = open(os.path.join(ROOT, "include", "ocean_gpu_module.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = set(re.findall(r"\b(Oc\w+)\s*\(", text))
+    assert {"OcInitGPU", "OcDeviceGPU_updateProperties", "OcInitDevicesGPU", "OcInitModuleCore_GPU", "OcRegisterStorageGPU",
+            "OcBufferGPU_copyHostToStorage", "OcBufferGPU_copyStorageToHost", "OcRegisterTensorGPU"} <= declared
+    have = exported_symbols(host.LIB_PATH)
+    assert not sorted(declared - have), sorted(declared - have)
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_GPU_HEADERS), reason="reference tree not present")
+def test_public_device_properties_have_the_reference_fields_in_order():
+    """OcDevicePropGPU of include/ocean_gpu_module.h lists the live fields of the reference's struct
+    (device_gpu.h:31-106) with the same types in the same order, and the ctypes mirror agrees with both."""
+    import re
+
+    def fields(text, closing):
+        body = text[:text.index(closing)]
+        body = body[body.rindex("typedef struct"):]
+        body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+        out = []
+        for ctype, decl in re.findall(r"\b(char|size_t|int)\s+([^;]+);", body):
+            for d in decl.split(","):
+                m = re.match(r"\s*(\w+)\s*(\[\d+\])?\s*$", d)
+                out.append((ctype, m.group(1), m.group(2) or ""))
+        return out
+    ref = fields(open(os.path.join(REF_GPU_HEADERS, "device_gpu.h")).read(), "} OcDevicePropGPU;")
+    mine = fields(open(os.path.join(ROOT, "include", "ocean_gpu_module.h")).read(), "} OcDevicePropGPU;")
+    assert len(ref) >= 45 and mine == ref
+    assert [n for n, _ in host.DevicePropGPU._fields_] == [n for _, n, _ in ref]
+    sizes = {"char": 1, "size_t": 8, "int": 4}
+    for (ctype, name, dim), (fname, ftype) in zip(ref, host.DevicePropGPU._fields_):
+        count = int(dim[1:-1]) if dim else 1
+        assert C.sizeof(ftype) == sizes[ctype] * count, name

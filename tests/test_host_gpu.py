@@ -194,6 +194,99 @@ def test_unary_and_fill(gpu):
     assert (host.to_numpy(t) == 3.25).all()
 
 
+def test_masked_fill_fill_nan_and_steps_through_the_table(gpu):
+    """Tensor_maskedFill, Tensor_fillNaN, Tensor_stepsInt64 and Tensor_stepsDouble reached the way Ocean's interface
+    reaches them (tensor_itf.c:2788-2908, 2965-3075): the value converted to the tensor's type, the mask of another
+    type and shape brought to bool and broadcast. Expected values: numpy.where and offset + i * step."""
+    rng = np.random.default_rng(77)
+    x = rng.uniform(-5, 5, (20, 33)).astype(np.float32)                       # Ocean shape (33, 20)
+    t = host.from_numpy(x, host.FLOAT, gpu)
+    mask = (rng.random((20, 33)) < 0.4).astype(np.uint8)
+    tm = host.from_numpy(mask, host.BOOL, gpu)
+    val = host.scalar(host.DOUBLE, 2.5)                                       # a double scalar into a float tensor
+    host.check(host.lib.OcTensor_maskedFill(t, tm, C.byref(val)))
+    want = np.where(mask != 0, np.float32(2.5), x)
+    assert host.to_numpy(t).tobytes() == want.tobytes()
+    # an int32 mask on the HOST with one row (Ocean shape (33, 1)), broadcast along the second dimension
+    row = rng.integers(-1, 2, (1, 33)).astype(np.int32)
+    trow = host.from_numpy(row, host.INT32)
+    val = host.scalar(host.INT64, -7)
+    host.check(host.lib.OcTensor_maskedFill(t, trow, C.byref(val)))
+    want = np.where(np.broadcast_to(row != 0, (20, 33)), np.float32(-7), want)
+    assert host.to_numpy(t).tobytes() == want.tobytes()
+    # a transposed view as destination: the mask follows the view's shape
+    tt = host.lib.OcTensor_transpose(t)                                       # Ocean shape (20, 33)
+    mask2 = (rng.random((33, 20)) < 0.3).astype(np.uint8)
+    tm2 = host.from_numpy(mask2, host.BOOL, gpu)
+    val = host.scalar(host.FLOAT, 0.125)
+    host.check(host.lib.OcTensor_maskedFill(tt, tm2, C.byref(val)))
+    want = np.where(mask2.T != 0, np.float32(0.125), want)
+    assert host.to_numpy(t).tobytes() == want.tobytes()
+    # a mask of the wrong shape is refused
+    bad = host.from_numpy(np.zeros((3, 5), np.uint8), host.BOOL, gpu)
+    assert host.lib.OcTensor_maskedFill(t, bad, C.byref(val)) != 0
+    # integer destination: the value is converted with C's rule
+    xi = rng.integers(-100, 100, (7, 9)).astype(np.int16)
+    ti = host.from_numpy(xi, host.INT16, gpu)
+    mi = (rng.random((7, 9)) < 0.5).astype(np.uint8)
+    val = host.scalar(host.DOUBLE, -3.75)
+    host.check(host.lib.OcTensor_maskedFill(ti, host.from_numpy(mi, host.BOOL, gpu), C.byref(val)))
+    assert np.array_equal(host.to_numpy(ti), np.where(mi != 0, np.int16(-3), xi))
+    # fillNaN
+    y = rng.uniform(-1, 1, (6, 11)); y[rng.random((6, 11)) < 0.3] = np.nan
+    ty = host.from_numpy(y, host.DOUBLE, gpu)
+    val = host.scalar(host.FLOAT, 9.5)
+    host.check(host.lib.OcTensor_fillNaN(ty, C.byref(val)))
+    assert host.to_numpy(ty).tobytes() == np.where(np.isnan(y), 9.5, y).tobytes()
+    host.check(host.lib.OcTensor_fillNaN(ti, C.byref(val)))                   # integers hold no NaN: untouched
+    assert np.array_equal(host.to_numpy(ti), np.where(mi != 0, np.int16(-3), xi))
+    # steps: the flat index runs over Ocean's first dimension fastest = numpy's C order of the reversed shape
+    ts = host.create([5, 4, 3], host.INT32, gpu)
+    host.check(host.lib.OcTensor_stepsInt64(ts, -4, 3))
+    assert np.array_equal(host.to_numpy(ts), (-4 + 3 * np.arange(60)).reshape(3, 4, 5).astype(np.int32))
+    td = host.create([8, 5], host.FLOAT, gpu)
+    host.check(host.lib.OcTensor_stepsDouble(td, 0.1, 0.3))
+    assert host.to_numpy(td).tobytes() == (0.1 + np.arange(40).astype(np.float64) * 0.3).astype(np.float32).reshape(5, 8).tobytes()
+    tdt = host.lib.OcTensor_transpose(td)                                     # Ocean shape (5, 8) over the same memory
+    host.check(host.lib.OcTensor_stepsInt64(tdt, 100, 1))
+    assert np.array_equal(host.to_numpy(td), (100 + np.arange(40)).reshape(8, 5).T.astype(np.float32))
+
+
+def test_public_device_object_and_reference_named_helpers(gpu):
+    """OcDeviceGPU_updateProperties (device_gpu.c:620-637) refreshes freeGlobalMem inside the device object, whose public
+    part carries the reference's field names; the buffer functions are callable under the reference's names."""
+    pub = host.gpu_public_properties(gpu)
+    assert pub.warpSize == 64 and pub.multiProcessorCount >= 64 and pub.totalGlobalMem >= (1 << 30)
+    assert pub.maxWarpsPerMultiProcessor * 64 == pub.maxThreadsPerMultiProcessor and pub.major >= 9
+    before = host.gpu_public_properties(gpu, update=True).freeGlobalMem
+    assert 0 < before <= pub.totalGlobalMem
+    big = host.create([1 << 26], host.DOUBLE, gpu)
+    after = host.gpu_public_properties(gpu, update=True).freeGlobalMem
+    assert after <= before - (1 << 28)
+    cpu_dev = host.cpu_device()
+    host.lib.OcDeviceGPU_updateProperties.argtypes = [C.c_void_p]
+    assert host.lib.OcDeviceGPU_updateProperties(cpu_dev) == -1               # not a GPU device
+    # OcBufferGPU_copyHostToStorage / copyStorageToHost / zero on the storage of `big` (storage_gpu.c:252-302)
+    st = big.contents.storage
+    data = np.arange(1000, dtype=np.float64)
+    back = np.zeros(1000)
+    for fn in (host.lib.OcBufferGPU_copyHostToStorage, host.lib.OcBufferGPU_copyStorageToHost):
+        fn.argtypes = [C.POINTER(host.Storage), C.c_ssize_t, C.c_ssize_t, C.c_void_p]
+    host.lib.OcBufferGPU_zero.argtypes = [C.POINTER(host.Storage), C.c_void_p, C.c_int, C.c_ssize_t]
+    host.check(host.lib.OcBufferGPU_copyHostToStorage(st, 4096, data.nbytes, data.ctypes.data))
+    host.check(host.lib.OcBufferGPU_copyStorageToHost(st, 4096, back.nbytes, back.ctypes.data))
+    assert np.array_equal(back, data)
+    host.check(host.lib.OcBufferGPU_zero(st, st.contents.data + 4096 + 80, host.DOUBLE, 500))
+    host.check(host.lib.OcBufferGPU_copyStorageToHost(st, 4096, back.nbytes, back.ctypes.data))
+    assert np.array_equal(back[:10], data[:10]) and not back[10:510].any() and np.array_equal(back[510:], data[510:])
+    host.lib.OcDecrefTensor(big)
+    # the registration pieces fill a caller's table: the same entries as the registered one
+    table = (C.c_void_p * 256)()
+    host.lib.OcRegisterStorageGPU.argtypes = [C.c_void_p]; host.lib.OcRegisterTensorGPU.argtypes = [C.c_void_p]
+    assert host.lib.OcRegisterStorageGPU(table) == 0 and host.lib.OcRegisterTensorGPU(table) == 0
+    assert sum(1 for v in table if v) > 120
+
+
 def test_find_and_mask_to_offset_through_the_table(gpu):
     rng = np.random.default_rng(12)
     mask = (rng.random((9, 40, 33)) < 0.2).astype(np.uint8)                 # Ocean dims (33, 40, 9)
