@@ -358,11 +358,15 @@ typedef struct {
 } och_reduce_axis_config;
 
 int och_reduce_axis(int op, int dtype, const och_reduce_axis_config *config, double p);
-/* One launch counts its outputs in 32 bits; a reduction with more outputs (the reference switches to 64-bit indices,     */
-/* solid/src/core/gpu/op/apply_elemwise.c:68-99) is cut along its outermost kept dimension into pieces that are launched   */
-/* one after the other. More than 2^32 reduced elements per output return an error. Test hook: the number of outputs per  */
-/* launch can be lowered (0 restores the default) so that small tensors are cut.                                          */
+/* One launch counts its outputs, and the reduced elements of one output, in 32 bits; the reference switches to 64-bit  */
+/* indices instead (solid/src/core/gpu/op/apply_elemwise.c:66-99). A reduction with more outputs is cut along its        */
+/* outermost kept dimension into pieces that are launched one after the other. A reduced range of more elements is cut  */
+/* along its outermost reduced dimension: every piece is a launch that leaves raw accumulators in the stream's workspace */
+/* and one finish kernel folds them in the order of the reduced index (a fixed order: results are reproducible). Test   */
+/* hooks: the number of outputs and of reduced elements per launch can be lowered (0 restores the default) so that      */
+/* small tensors are cut.                                                                                               */
 void och_reduce_axis_set_output_limit(size_t outputs);
+void och_reduce_axis_set_range_limit(size_t nelem);
 
 /* ======================================================================== */
 /* GEMM: C <- alpha * op(A) * op(B) + beta * C, column-major, ld in elements*/
@@ -480,6 +484,15 @@ typedef struct {
 } och_elemwise_plan;
 int och_elemwise_analyze(int noperands, const int *elemsize, int ndims, const size_t *size,
                          const ptrdiff_t *const *strides, void *const *ptrs, och_elemwise_plan *plan);
+/* One launch of the elementwise engine (binary, unary, copy / cast / byteswap, fill, steps, the index kernels) counts    */
+/* its work items in 32 bits: at most 0xFFFF0000 elements. The reference switches its kernels to 64-bit indices above   */
+/* that (solid/src/core/gpu/op/apply_elemwise.c:66-99); here a larger call is cut along its outermost dimension into    */
+/* runs that are launched one after the other on the stream (a one-dimensional call into runs of a multiple of 64       */
+/* elements), a copy between different shapes along the flat index both sides share, and the gather / scatter kernels   */
+/* decompose a 64-bit work-item number. Test hook: the limit can be lowered (64 ... 0xFFFF0000; 0 restores the default) */
+/* so that small tensors take these paths; och_elemwise_analyze reports the launches a call would make. Returns -1 for  */
+/* a value outside that range.                                                                                          */
+int och_elemwise_set_launch_limit(size_t nelem);
 /* OCH_KERNEL_ROWS (unit-stride rows that are not whole aligned vectors: an odd width, a start or a pitch that is not  */
 /* a multiple of the vector width): a work item is one aligned unit of `vec` elements of a destination row. For unit   */
 /* number `unit` of a row of row_elements elements of elemsize bytes that starts `misalignment` bytes into such a unit: */

@@ -72,11 +72,56 @@ static int side_normalize(Side &s, int ndims, const size_t *size, const ptrdiff_
    return 0;
 }
 
+/* the same for element counts above the launch limit of the elementwise engine: sizes and the flat index are 64 bits
+   wide and decomposed with plain divisions; one launch covers elements [first, first + count) */
+struct ReshapeBigParams
+{
+   char *src, *dst;
+   int nd1, nd2;
+   uint64_t size1[OCH_MAX_DIMS], size2[OCH_MAX_DIMS];
+   int64_t st1[OCH_MAX_DIMS], st2[OCH_MAX_DIMS];
+   uint64_t first, count;
+};
+template <int ES>
+__global__ __launch_bounds__(256) void reshape_big_kernel(const ReshapeBigParams p)
+{
+   const uint64_t local = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+   if (local >= p.count) return;
+   const uint64_t e = p.first + local;
+   int64_t o1 = 0, o2 = 0;
+   uint64_t q = e;
+   for (int d = 0; d < p.nd1 - 1; d++) { const uint64_t q2 = q / p.size1[d]; o1 += (int64_t)(q - q2 * p.size1[d]) * p.st1[d]; q = q2; }
+   o1 += (int64_t)q * p.st1[p.nd1 - 1];
+   q = e;
+   for (int d = 0; d < p.nd2 - 1; d++) { const uint64_t q2 = q / p.size2[d]; o2 += (int64_t)(q - q2 * p.size2[d]) * p.st2[d]; q = q2; }
+   o2 += (int64_t)q * p.st2[p.nd2 - 1];
+   *reinterpret_cast<Blob<ES> *>(p.dst + o2) = *reinterpret_cast<const Blob<ES> *>(p.src + o1);
+}
+
 static int reshape_launch(int es, const Side &a, char *src, const Side &b, char *dst, hipStream_t stream)
 {
-   /* chunks of < 2^32 elements along the flat index are cut on the outermost dimension of
-      both sides only when they coincide; otherwise large reshapes are refused */
-   if (a.nelem >= 0xFFFFFF00ull) return set_error("reshape copy of more than 2^32 elements is not supported");
+   if (a.nelem > ew_launch_limit())
+   {  /* the two sides are cut differently by their dimensions, so the cut is made along the flat index they share
+         (the reference runs its kernel with 64-bit indices, solid/src/core/gpu/op/apply_elemwise.c:66-99) */
+      ReshapeBigParams p;
+      p.src = src; p.dst = dst; p.nd1 = a.nd; p.nd2 = b.nd;
+      for (int d = 0; d < a.nd; d++) { p.size1[d] = a.size[d]; p.st1[d] = a.st[d]; }
+      for (int d = 0; d < b.nd; d++) { p.size2[d] = b.size[d]; p.st2[d] = b.st[d]; }
+      const uint64_t run = ew_launch_limit();
+      for (uint64_t first = 0; first < a.nelem; first += run)
+      {  p.first = first; p.count = (a.nelem - first < run) ? a.nelem - first : run;
+         dim3 grid((unsigned)((p.count + 255) / 256)), block(256);
+         switch (es)
+         {  case 1:  hipLaunchKernelGGL(reshape_big_kernel<1>,  grid, block, 0, stream, p); break;
+            case 2:  hipLaunchKernelGGL(reshape_big_kernel<2>,  grid, block, 0, stream, p); break;
+            case 4:  hipLaunchKernelGGL(reshape_big_kernel<4>,  grid, block, 0, stream, p); break;
+            case 8:  hipLaunchKernelGGL(reshape_big_kernel<8>,  grid, block, 0, stream, p); break;
+            default: hipLaunchKernelGGL(reshape_big_kernel<16>, grid, block, 0, stream, p); break;
+         }
+         OCH_CHECK_LAUNCH();
+      }
+      return 0;
+   }
    ReshapeParams p;
    p.src = src; p.dst = dst; p.nd1 = a.nd; p.nd2 = b.nd; p.nelem = (uint32_t)a.nelem;
    for (int d = 0; d < a.nd; d++) { p.div1[d] = make_fastdiv((uint32_t)a.size[d]); p.st1[d] = a.st[d]; }

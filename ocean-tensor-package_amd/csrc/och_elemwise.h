@@ -727,16 +727,25 @@ static int ew_normalize(EwShape<NOPS> &s, int ndims, const size_t *size,
    return 0;
 }
 
-/* Launcher signature: (shape with every size < 2^32 and nelem < 2^32, vec flag, first flat index) */
+/* Elements one launch of the elementwise engine handles: 0xFFFF0000 (keeps block base + thread offset from wrapping in
+   32 bits) unless och_elemwise_set_launch_limit has lowered it so that small tensors take the cutting path below. The
+   reference switches its kernels to 64-bit indices instead (solid/src/core/gpu/op/apply_elemwise.c:66-99). */
+uint64_t ew_launch_limit();
+
+/* Launcher signature: (shape with every size < 2^32 and nelem < 2^32, vec flag, first flat index). A shape above the
+   limit is cut along its outermost dimension into runs that fit (or walked index by index and cut further inside when
+   one index of it is still too much); a one-dimensional shape into runs of a multiple of 64 elements, so that every
+   run starts as aligned as the whole. The runs are launched one after the other on the caller's stream. */
 template <int NOPS, class L>
 static int ew_launch_chunked(EwShape<NOPS> s, uint64_t flat0, L &&launch)
 {
-   const uint64_t LIMIT = 0xFFFF0000ull;          /* keeps block base + thread offset from wrapping */
+   const uint64_t LIMIT = ew_launch_limit();
    if (s.nelem == 0) return 0;
    if (s.nelem <= LIMIT) return launch(s, flat0);
    int last = s.ndims - 1;
    uint64_t inner = s.nelem / s.size[last];
-   uint64_t chunk = (s.ndims == 1) ? (1ull << 30) : (inner <= LIMIT ? LIMIT / inner : 0);
+   const uint64_t run1 = (LIMIT >= (1ull << 30)) ? (1ull << 30) : ((LIMIT & ~63ull) ? (LIMIT & ~63ull) : 64);
+   uint64_t chunk = (s.ndims == 1) ? run1 : (inner <= LIMIT ? LIMIT / inner : 0);
    if (chunk >= 1)
    {  for (uint64_t start = 0; start < s.size[last]; start += chunk)
       {  EwShape<NOPS> c = s;

@@ -26,6 +26,7 @@ struct IndexParams
    char          *ptr1, *ptr2;
    uint64_t       nelem;
    int            ndims;
+   int            small;                       /* nelem fits one launch's 32-bit index arithmetic: div[] is filled */
 };
 struct ToOffsetStrides { int64_t s[OCH_MAX_DIMS]; };
 
@@ -48,7 +49,7 @@ __global__ __launch_bounds__(256) void index_to_offset_kernel(uint64_t nelem, in
 template <class E, int MODE, int V>
 __global__ __launch_bounds__(256) void index_kernel(const IndexParams p, const E value)
 {
-   const bool small = p.nelem <= 0xFFFFFFFFull;
+   const bool small = p.small != 0;
    for (uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x; idx < p.nelem; idx += (uint64_t)gridDim.x * 256)
    {  int64_t o1 = 0, o2 = 0;
       if (small)
@@ -96,7 +97,10 @@ static int launch_index(IndexParams &p, const och_scalar &value, hipStream_t str
    const bool runs = p.ndims >= 1 && p.offsets[0] == nullptr && p.size[0] % V == 0 && p.strides1[0] == (int64_t)sizeof(E) &&
                      (MODE == 2 || p.strides2[0] == (int64_t)sizeof(E));
    if (runs) { p.size[0] /= V; p.nelem /= V; p.strides1[0] = 16; if (MODE != 2) p.strides2[0] = 16; }
-   if (p.nelem <= 0xFFFFFFFFull)
+   /* above the launch limit of the elementwise engine (2^32 - 2^16 elements unless a test has lowered it) the kernel
+      decomposes the 64-bit work-item number with plain divisions; its grid-stride loop covers any count */
+   p.small = (p.nelem <= ew_launch_limit()) ? 1 : 0;
+   if (p.small)
       for (int d = 0; d < p.ndims; d++) p.div[d] = make_fastdiv((uint32_t)p.size[d]);
    uint64_t blocks = (p.nelem + 255) / 256; if (blocks > (1u << 20)) blocks = 1u << 20;
    if (runs) hipLaunchKernelGGL((index_kernel<E, MODE, V>), dim3((unsigned)blocks), dim3(256), 0, stream, p, v);
@@ -155,8 +159,8 @@ extern "C" int och_index_to_offset(int dtype, int nstrides, const int64_t *strid
    ToOffsetStrides st; memset(&st, 0, sizeof(st));
    for (int i = 0; i < nstrides; i++) st.s[i] = strides[i];
    /* launches of at most 2^31 elements each (the grid of one launch is 32 bits of blocks wide, and the runtime accepts
-      far fewer blocks than that) */
-   const size_t per_launch = (size_t)1 << 31;
+      far fewer blocks than that), or of the launch limit of the elementwise engine when a test has lowered it */
+   const size_t per_launch = (ew_launch_limit() < ((size_t)1 << 31)) ? (size_t)ew_launch_limit() : ((size_t)1 << 31);
    for (size_t first = 0; first < nelem; first += per_launch)
    {  const size_t n = (nelem - first < per_launch) ? nelem - first : per_launch;
       const dim3 grid((unsigned)((n + 255) / 256)), block(256);

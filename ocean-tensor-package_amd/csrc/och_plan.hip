@@ -4,6 +4,9 @@
 
 namespace och {
 
+static uint64_t g_ew_launch_limit = 0;
+uint64_t ew_launch_limit() { return g_ew_launch_limit ? g_ew_launch_limit : 0xFFFF0000ull; }
+
 template <int NOPS>
 static int analyze(const int *elemsize, int ndims, const size_t *size, const ptrdiff_t *const *strides, void *const *ptrs,
                    och_elemwise_plan *plan)
@@ -94,4 +97,12 @@ extern "C" int och_elemwise_analyze(int noperands, const int *elemsize, int ndim
       case 3: return analyze<3>(elemsize, ndims, size, strides, ptrs, plan);
    }
    return set_error("elemwise_analyze: %d operands are not supported (1 to 3)", noperands);
+}
+
+extern "C" int och_elemwise_set_launch_limit(size_t nelem)
+{
+   if (nelem != 0 && (nelem < 64 || nelem > 0xFFFF0000ull))
+      return och::set_error("och_elemwise_set_launch_limit: the limit must be 0 (default) or between 64 and 0xFFFF0000 elements");
+   och::g_ew_launch_limit = nelem;
+   return 0;
 }

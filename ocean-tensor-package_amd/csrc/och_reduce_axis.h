@@ -12,6 +12,7 @@
  * Accumulator types, NaN rules and result types are those of the full reductions.
  */
 #pragma once
+#include <vector>
 #include "och_reduce_all.h"
 
 namespace och {
@@ -28,6 +29,10 @@ struct AxisParams
       loads); every piece leaves its accumulator in partials[slice][output] (16-byte slots) and axis_finish_kernel
       folds the pieces in order */
    uint32_t slices, slice_len; int slice_rows;
+   /* partial: the accumulators go to partials[slice_base + slice][output] instead of the destination (always when the
+      range is cut into slices; also for a single slice when the call is one of several that cover a reduced range too
+      long for one launch, whose pieces occupy consecutive slots and are folded together) */
+   int partial; uint32_t slice_base;
    int64_t  rowbytes;                            /* row mode of the cooperative kernels: bytes of one row of the first reduced dimension */
    /* row mode of the per-thread kernel: the rows of the first outer dimension are not whole aligned groups, but every row
       starts at the same position row_m within a 16-byte unit; a thread owns the aligned chunk c of a row, i.e. the
@@ -154,12 +159,12 @@ __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, co
          for (int k = 0; k < VEC; k++)
          {  const int i = first + k;                   /* position in the row; elements of the chunk outside the row are dropped */
             if (i >= 0 && (uint32_t)i < p.row_n0)
-            {  if (p.slices > 1) *reinterpret_cast<Acc *>(p.partials + ((size_t)blockIdx.y * p.nout + o + (uint32_t)i) * 16) = acc[k];
+            {  if (p.partial) *reinterpret_cast<Acc *>(p.partials + ((size_t)(p.slice_base + blockIdx.y) * p.nout + o + (uint32_t)i) * 16) = acc[k];
                else *reinterpret_cast<Res *>(p.dst + o2 + (int64_t)i * p.st2[0]) = RD::finalize(acc[k], prm);
             }
          }
       }
-      else if (VEC > 1 && p.dst_wide && p.slices <= 1)
+      else if (VEC > 1 && p.dst_wide && !p.partial)
       {
 #pragma unroll
          for (int q = 0; q < VEC / PV; q++)
@@ -173,7 +178,7 @@ __global__ __launch_bounds__(256) void axis_thread_kernel(const AxisParams p, co
       {
 #pragma unroll
          for (int k = 0; k < VEC; k++)
-         {  if (p.slices > 1) *reinterpret_cast<Acc *>(p.partials + ((size_t)blockIdx.y * p.nout + o + k) * 16) = acc[k];
+         {  if (p.partial) *reinterpret_cast<Acc *>(p.partials + ((size_t)(p.slice_base + blockIdx.y) * p.nout + o + k) * 16) = acc[k];
             else *reinterpret_cast<Res *>(p.dst + o2 + (int64_t)k * p.st2[0]) = RD::finalize(acc[k], prm);
          }
       }
@@ -296,7 +301,7 @@ __global__ __launch_bounds__(256) void axis_group_kernel(const AxisParams p, con
       if (threadIdx.x == 0) { acc = RD::combine(RD::combine(lds[0], lds[1]), RD::combine(lds[2], lds[3])); }
    }
    if (active && lane == 0)
-   {  if (p.slices > 1) *reinterpret_cast<Acc *>(p.partials + ((size_t)blockIdx.y * p.nout + o) * 16) = acc;
+   {  if (p.partial) *reinterpret_cast<Acc *>(p.partials + ((size_t)(p.slice_base + blockIdx.y) * p.nout + o) * 16) = acc;
       else *reinterpret_cast<typename RD::Res *>(p.dst + o2) = RD::finalize(acc, prm);
    }
 }
@@ -304,6 +309,44 @@ __global__ __launch_bounds__(256) void axis_group_kernel(const AxisParams p, con
 typedef int (*axis_fn)(const och_reduce_axis_config *c, double pnorm);
 /* outputs one launch handles (0xFFFFFF00 unless och_reduce_axis_set_output_limit has lowered it for a test) */
 uint64_t axis_output_limit();
+/* elements of the reduced range (per output) one launch handles: 0xFFFFFF00 unless och_reduce_axis_set_range_limit has
+   lowered it for a test */
+uint64_t axis_range_limit();
+
+/* One launch of several that together cover a reduced range too long for one: it leaves its accumulators in the slots
+   base, base + 1, ... of the stream's workspace (at most `room` of them) and reports how many it used. */
+struct AxisPiece { uint32_t base, room, used; AxisParams params; };
+
+/* Cuts the reduced range of c into pieces of at most `limit` elements, in the order of the flat reduced index: runs
+   along the outermost reduced dimension, or -- when a single index of it is still too long -- index by index, each cut
+   further inside. */
+static void axis_cut_range(const och_reduce_axis_config &c, uint64_t limit, std::vector<och_reduce_axis_config> &out)
+{
+   uint64_t relem = 1; int last = -1;
+   for (int d = 0; d < c.rdims; d++) { relem *= c.rsize[d]; if (c.rsize[d] > 1) last = d; }
+   if (relem <= limit || last < 0) { out.push_back(c); return; }
+   const uint64_t inner = relem / c.rsize[last];
+   if (inner <= limit)
+   {  const uint64_t run = limit / inner;
+      for (uint64_t start = 0; start < c.rsize[last]; start += run)
+      {  och_reduce_axis_config piece = c;
+         piece.rsize[last] = (c.rsize[last] - start < run) ? (size_t)(c.rsize[last] - start) : (size_t)run;
+         piece.ptr1 = (char *)c.ptr1 + (int64_t)start * c.rstrides[last];
+         out.push_back(piece);
+      }
+      return;
+   }
+   for (uint64_t i = 0; i < c.rsize[last]; i++)
+   {  och_reduce_axis_config piece = c;
+      piece.rsize[last] = 1;
+      piece.ptr1 = (char *)c.ptr1 + (int64_t)i * c.rstrides[last];
+      axis_cut_range(piece, limit, out);
+   }
+}
+
+template <class T, int OP>
+static int launch_reduce_axis_one(const och_reduce_axis_config *c, const typename Reduce<T, OP>::Param &prm,
+                                  uint64_t nout, uint64_t relem, AxisPiece *piece);
 
 template <class T, int OP>
 static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
@@ -319,7 +362,6 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
    for (int d = 0; d < c->rdims; d++) relem *= c->rsize[d];
    if (nout == 0) return 0;
    if (relem == 0 && RD::NEEDS_DATA) return set_error("reduction over an empty range is undefined for this operation");
-   if (relem > 0xFFFFFF00ull) return set_error("axis reduction over more than 2^32 elements per output is not supported");
    /* more outputs than one launch counts in 32 bits (the reference switches to 64-bit indices): the outputs are
       independent, so the outermost kept dimension is cut into runs that fit, or walked index by index when a single
       index of it is still too much, and every piece is a reduction of its own on the same stream */
@@ -337,7 +379,39 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
       }
       return 0;
    }
+   if (relem <= axis_range_limit()) return launch_reduce_axis_one<T, OP>(c, prm, nout, relem, nullptr);
+   /* a reduced range longer than one launch counts in 32 bits (solid/src/core/gpu/op/apply_elemwise.c:66-99: the
+      reference switches to 64-bit indices): the range is cut into pieces, every piece is a launch that leaves raw
+      accumulators in consecutive slots of the stream's workspace -- cut into slices of its own while there is room -- and
+      one finish kernel folds all slots in the order of the reduced index */
+   std::vector<och_reduce_axis_config> pieces;
+   axis_cut_range(*c, axis_range_limit(), pieces);
+   const uint64_t rows = OCH_GEMM_WORKSPACE / (nout * 16);
+   if (pieces.size() > rows) return set_error("axis reduction: the reduced range needs %llu pieces of partial results, the workspace holds %llu",
+                                              (unsigned long long)pieces.size(), (unsigned long long)rows);
+   AxisPiece pc; uint32_t base = 0;
+   for (size_t i = 0; i < pieces.size(); i++)
+   {  uint64_t n = 1;
+      for (int d = 0; d < pieces[i].rdims; d++) n *= pieces[i].rsize[d];
+      pc.base = base; pc.used = 0;
+      pc.room = (uint32_t)(rows - base - (pieces.size() - 1 - i));           /* every later piece needs at least one slot */
+      if (launch_reduce_axis_one<T, OP>(&pieces[i], prm, nout, n, &pc) != 0) return -1;
+      base += pc.used;
+   }
+   AxisParams p = pc.params;
+   p.slices = base; p.slice_base = 0;
+   uint32_t lanes = 1;
+   while (lanes < 64 && lanes * 16 <= p.slices && (uint64_t)p.nout * lanes * 2 <= (1u << 20)) lanes *= 2;
+   hipLaunchKernelGGL((axis_finish_kernel<RD, T>), dim3((unsigned)(((uint64_t)p.nout * lanes + 255) / 256)), dim3(256), 0, as_stream(c->stream), p, prm, lanes);
+   OCH_CHECK_LAUNCH();
+   return 0;
+}
 
+template <class T, int OP>
+static int launch_reduce_axis_one(const och_reduce_axis_config *c, const typename Reduce<T, OP>::Param &prm,
+                                  uint64_t nout, uint64_t relem, AxisPiece *piece)
+{
+   typedef Reduce<T, OP> RD;
    AxisParams p;
    memset(&p, 0, sizeof(p));
    p.src = (char *)c->ptr1; p.dst = (char *)c->ptr2;
@@ -370,17 +444,21 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
       every piece at least min_len long, the partial accumulators within the stream's workspace */
    auto plan_slices = [&](uint64_t blocks, uint64_t range, uint64_t min_len) -> int
    {  p.slices = 1; p.slice_len = 0; p.partials = nullptr;
-      if (blocks >= 512 || range < 2 * min_len) return 0;
-      uint64_t want = (1024 + blocks - 1) / blocks;
-      if (want > range / min_len) want = range / min_len;
-      const uint64_t fit = OCH_GEMM_WORKSPACE / ((uint64_t)p.nout * 16);
-      if (want > fit) want = fit;
-      if (want > 65535) want = 65535;
-      if (want < 2) return 0;
-      p.slice_len = (uint32_t)((range + want - 1) / want);
-      p.slices = (uint32_t)((range + p.slice_len - 1) / p.slice_len);
-      if (p.slices < 2) { p.slices = 1; return 0; }
-      return stream_gemm_workspace(stream, &p.partials);
+      p.partial = piece ? 1 : 0; p.slice_base = piece ? piece->base : 0;
+      if (blocks < 512 && range >= 2 * min_len)
+      {  uint64_t want = (1024 + blocks - 1) / blocks;
+         if (want > range / min_len) want = range / min_len;
+         const uint64_t fit = piece ? (uint64_t)piece->room : OCH_GEMM_WORKSPACE / ((uint64_t)p.nout * 16);
+         if (want > fit) want = fit;
+         if (want > 65535) want = 65535;
+         if (want >= 2)
+         {  p.slice_len = (uint32_t)((range + want - 1) / want);
+            p.slices = (uint32_t)((range + p.slice_len - 1) / p.slice_len);
+            if (p.slices < 2) p.slices = 1;
+         }
+      }
+      if (p.slices > 1) p.partial = 1;
+      return p.partial ? stream_gemm_workspace(stream, &p.partials) : 0;
    };
    if (!cooperative)
    {  /* VEC outputs per thread when the first outer dimension has unit source stride and
@@ -485,6 +563,7 @@ static int launch_reduce_axis(const och_reduce_axis_config *c, double pnorm)
          else      hipLaunchKernelGGL((axis_group_kernel<RD, T, 256>), grid, dim3(256), 0, stream, p, prm);
       }
    }
+   if (piece) { OCH_CHECK_LAUNCH(); piece->used = p.slices; piece->params = p; return 0; }
    if (p.slices > 1)
    {  uint32_t lanes = 1;                        /* at least eight pieces per lane, at most 2^20 threads */
       while (lanes < 64 && lanes * 16 <= p.slices && (uint64_t)p.nout * lanes * 2 <= (1u << 20)) lanes *= 2;

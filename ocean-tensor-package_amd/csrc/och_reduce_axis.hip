@@ -6,6 +6,8 @@
 namespace och {
 static std::atomic<uint64_t> g_axis_output_limit(0xFFFFFF00ull);
 uint64_t axis_output_limit() { return g_axis_output_limit.load(); }
+static std::atomic<uint64_t> g_axis_range_limit(0xFFFFFF00ull);
+uint64_t axis_range_limit() { return g_axis_range_limit.load(); }
 /* the instantiations are spread over eight translation units (build time); each knows its own operations */
 #define OCH_AXIS_PARTS(X) X(a) X(b) X(c) X(d) X(e) X(f) X(g) X(h)
 #define OCH_X(part) axis_fn axis_lookup_##part(int op, int dtype);
@@ -14,6 +16,8 @@ OCH_AXIS_PARTS(OCH_X)
 }
 extern "C" void och_reduce_axis_set_output_limit(size_t outputs)
 {  och::g_axis_output_limit.store((outputs == 0 || outputs > 0xFFFFFF00ull) ? 0xFFFFFF00ull : (uint64_t)outputs); }
+extern "C" void och_reduce_axis_set_range_limit(size_t nelem)
+{  och::g_axis_range_limit.store((nelem == 0 || nelem > 0xFFFFFF00ull) ? 0xFFFFFF00ull : (uint64_t)nelem); }
 extern "C" int och_reduce_axis(int op, int dtype, const och_reduce_axis_config *config, double p)
 {
    using namespace och;

@@ -139,6 +139,8 @@ PROTOTYPES = {
     "och_reduce_cut_parts": (C.c_longlong, [_i, C.POINTER(C.c_size_t), C.c_size_t, C.c_longlong, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "och_reduce_set_part_limit": (None, [C.c_size_t]),
     "och_reduce_axis_set_output_limit": (None, [C.c_size_t]),
+    "och_reduce_axis_set_range_limit": (None, [C.c_size_t]),
+    "och_elemwise_set_launch_limit": (C.c_int, [C.c_size_t]),
     "och_device_count": (_i, [C.POINTER(_i)]),
     "och_device_set": (_i, [_i]),
     "och_device_get": (_i, [C.POINTER(_i)]),

@@ -332,3 +332,30 @@ def test_units_of_a_row_partition_it():
                         if lo.value == 0 and hi.value == vec:
                             assert (m + first.value * es) % wd == 0
                     assert (covered == 1).all(), (es, vec, n0, m)
+
+
+def test_elementwise_launch_limit_cuts_calls_into_runs():
+    """och_elemwise_set_launch_limit lowers the number of elements per launch, so that the cutting of tensors above
+    2^32 - 2^16 elements can be seen on small ones: och_elemwise_analyze reports the launches of a call without a GPU."""
+    import ocean_hip as oh
+    a = 1 << 20
+    try:
+        assert oh.lib.och_elemwise_set_launch_limit(63) == -1 and oh.lib.och_elemwise_set_launch_limit((1 << 32) + 5) == -1
+        assert oh.lib.och_elemwise_set_launch_limit(1000) == 0
+        # one dimension: runs of the largest multiple of 64 below the limit (960), 5000 = 5 * 960 + 200
+        p = oh.elemwise_analyze([4, 4], [5000], [[4], [4]], [a, a])
+        assert p.launches == 6 and p.kernel == oh.KERNEL_WIDE
+        # one dimension whose last run is not a whole number of vectors: body + tail in that run only
+        p = oh.elemwise_analyze([4, 4], [5003], [[4], [4]], [a, a])
+        assert p.launches == 7
+        # two dimensions that do not merge: runs of whole indices of the outer one (1000 // 48 = 20 of 45 -> 3 launches)
+        p = oh.elemwise_analyze([4, 4], [48, 45], [[4, 256], [4, 192]], [a, a])
+        assert p.launches == 3 and p.ndims == 2
+        # one index of the outer dimension is still too long: walked index by index, each cut inside (3 x 3 runs)
+        p = oh.elemwise_analyze([4, 4], [2560, 3], [[4, 16384], [4, 10240]], [a, a])
+        assert p.launches == 9
+        assert oh.lib.och_elemwise_set_launch_limit(0) == 0
+        p = oh.elemwise_analyze([4, 4], [5000], [[4], [4]], [a, a])
+        assert p.launches == 1
+    finally:
+        oh.lib.och_elemwise_set_launch_limit(0)
