@@ -520,6 +520,168 @@ def main():
         for src, dst in c4:
             src.free(); dst.free()
 
+    # ------------------------------------------------------------------ beyond the named configurations: the other kernel families
+    # (unary functions, arithmetic-heavy binary operations, the software half types, fill, gather / scatter / find): the same
+    # sampling, two operand sets alternating, algorithmic bytes = every input element read once + every output written once
+    if args.only is None:
+        U = oh.U
+        ne = 1 << 26
+        HALF_T, CHALF_T, I64, I32 = oh.HALF, oh.CHALF, oh.INT64, oh.INT32
+
+        def extra_sets(es_in, es_out, n_in, fill):
+            """two sets of n_in inputs + 1 output of ne elements; fill(k) gives a host block for input k"""
+            out = []
+            for _ in range(2):
+                ins = []
+                for k in range(n_in):
+                    b = oh.DeviceBuffer(es_in * ne, stream)
+                    upload_tiled(b, fill(k), es_in * ne)
+                    ins.append(b)
+                out.append((ins, oh.DeviceBuffer(es_out * ne, stream)))
+            return out
+
+        def free_sets(sets_):
+            for ins, o in sets_:
+                for b in ins + [o]:
+                    b.free()
+        se = oh.sizes([ne])
+        # unary functions
+        for dt, es, nm, npt in ((F32, 4, "f32", np.float32), (F64, 8, "f64", np.float64)):
+            sets_ = extra_sets(es, es, 1, lambda k: rng.uniform(0.5, 4.0, 1 << 22).astype(npt))
+            stx = oh.strides([es]); ut = [0]
+            for opn in ("sqrt", "exp", "sin", "tanh"):
+                def un(opn=opn):
+                    ins, o = sets_[ut[0] % 2]; ut[0] += 1
+                    oh.check(lib.och_unary(U[opn], dt, 1, se, stx, ins[0].ptr, stx, o.ptr, h))
+                configs["extra_unary_%s_%s_2^26" % (opn, nm)] = gbps(2 * es * ne, sample_launches(un), ceil_of("copy_134MB_operands"))
+            free_sets(sets_)
+        sets_ = extra_sets(8, 8, 1, lambda k: (rng.uniform(-2, 2, 1 << 21) + 1j * rng.uniform(-2, 2, 1 << 21)).astype(np.complex64))
+        outr = [oh.DeviceBuffer(4 * ne, stream) for _ in range(2)]
+        stc, stf = oh.strides([8]), oh.strides([4]); ut = [0]
+
+        def un_cexp():
+            ins, o = sets_[ut[0] % 2]; ut[0] += 1
+            oh.check(lib.och_unary(U["exp"], CF, 1, se, stc, ins[0].ptr, stc, o.ptr, h))
+
+        def un_cabs():
+            ins, o = sets_[ut[0] % 2]; ut[0] += 1
+            oh.check(lib.och_unary(U["absolute"], CF, 1, se, stc, ins[0].ptr, stf, outr[ut[0] % 2].ptr, h))
+        configs["extra_unary_exp_cfloat_2^26"] = gbps(16 * ne, sample_launches(un_cexp), ceil_of("copy_134MB_operands"))
+        configs["extra_unary_absolute_cfloat_to_f32_2^26"] = gbps(12 * ne, sample_launches(un_cabs), ceil_of("copy_134MB_operands"))
+        free_sets(sets_)
+        for b in outr:
+            b.free()
+        # binary operations with real arithmetic behind them: integer division and remainder (floor rules), powers
+        def int_block(npt, k):
+            v = rng.integers(-(1 << 20), 1 << 20, 1 << 22).astype(npt)
+            if k == 1:
+                v = rng.integers(1, 1000, 1 << 22).astype(npt) * rng.choice(np.array([-1, 1], npt), 1 << 22)
+            return v
+        for dt, es, nm, npt in ((I32, 4, "int32", np.int32), (I64, 8, "int64", np.int64)):
+            sets_ = extra_sets(es, es, 2, lambda k: int_block(npt, k))
+            stx = oh.strides([es]); bt = [0]
+            for opn in ("divide", "mod"):
+                def bn(opn=opn):
+                    ins, o = sets_[bt[0] % 2]; bt[0] += 1
+                    oh.check(lib.och_binary(B[opn], dt, 1, se, stx, ins[0].ptr, stx, ins[1].ptr, stx, o.ptr, h))
+                configs["extra_binary_%s_%s_2^26" % (opn, nm)] = gbps(3 * es * ne, sample_launches(bn), ceil_of("add_134MB_operands"))
+            free_sets(sets_)
+        for dt, es, nm, fillf, es2 in ((I32, 4, "int32", lambda k: (rng.integers(-9, 9, 1 << 22) if k == 0 else rng.integers(0, 9, 1 << 22)).astype(np.int32 if k == 0 else np.int16), 2),
+                                        (F32, 4, "f32", lambda k: rng.uniform(0.5, 2.0, 1 << 22).astype(np.float32), 4)):
+            # integer powers take int16 exponents (the second operand type of the table's power entry)
+            sets_ = []
+            for _ in range(2):
+                a_ = oh.DeviceBuffer(es * ne, stream); b_ = oh.DeviceBuffer(es2 * ne, stream); o_ = oh.DeviceBuffer(es * ne, stream)
+                upload_tiled(a_, fillf(0), es * ne); upload_tiled(b_, fillf(1), es2 * ne)
+                sets_.append(([a_, b_], o_))
+            stx, stb = oh.strides([es]), oh.strides([es2]); bt = [0]
+
+            def bp():
+                ins, o = sets_[bt[0] % 2]; bt[0] += 1
+                oh.check(lib.och_binary(B["power"], dt, 1, se, stx, ins[0].ptr, stb, ins[1].ptr, stx, o.ptr, h))
+            configs["extra_binary_power_%s_2^26" % nm] = gbps((2 * es + es2) * ne, sample_launches(bp), ceil_of("add_134MB_operands"))
+            free_sets(sets_)
+        # the half types: storage is half, arithmetic is float, conversions by the library's own rounding rules
+        for dt, es, nm in ((HALF_T, 2, "half"), (CHALF_T, 4, "chalf")):
+            sets_ = extra_sets(es, es, 2, lambda k: rng.uniform(-2, 2, 1 << 22).astype(np.float16))
+            stx = oh.strides([es]); bt = [0]
+            for opn in ("add", "multiply"):
+                def bh(opn=opn):
+                    ins, o = sets_[bt[0] % 2]; bt[0] += 1
+                    oh.check(lib.och_binary(B[opn], dt, 1, se, stx, ins[0].ptr, stx, ins[1].ptr, stx, o.ptr, h))
+                configs["extra_binary_%s_%s_2^26" % (opn, nm)] = gbps(3 * es * ne, sample_launches(bh), ceil_of("add_67MB_operands"))
+            free_sets(sets_)
+        # fill and masked fill, float32
+        fbufs = [oh.DeviceBuffer(4 * ne, stream) for _ in range(2)]
+        mbufs = [oh.to_device((rng.random(ne) < 0.5).astype(np.uint8), stream) for _ in range(2)]
+        fval = oh.make_scalar(F32, 1.5); ft = [0]
+
+        def k_fill():
+            ft[0] += 1
+            oh.check(lib.och_fill(F32, 1, se, stf, fbufs[ft[0] % 2].ptr, fval, h))
+
+        def k_masked_fill():
+            ft[0] += 1
+            oh.check(lib.och_masked_fill(F32, 1, se, stf, fbufs[ft[0] % 2].ptr, oh.strides([1]), mbufs[ft[0] % 2].ptr, fval, h))
+        configs["extra_fill_f32_2^26"] = gbps(4 * ne, sample_launches(k_fill), ceil_of("write_268MB"))
+        e = gbps(9 * ne, sample_launches(k_masked_fill), ceil_of("copy_134MB_operands"))
+        e["note"] = ("half of the mask set at random, so every 16-byte group holds kept and replaced elements: the result is where(mask, value, old) -- "
+                     "the mask (1 byte) and the old element (4 bytes) are read, the element (4 bytes) is written: 9 bytes per element")
+        configs["extra_masked_fill_f32_2^26_half_set"] = e
+        for b in fbufs + mbufs:
+            b.free()
+        # gather / scatter of 65536 rows of 8 KB through an offset table, 16M random 8-byte elements, and find on a 64M-element mask
+        rows_n, row_bytes = 65536, 8192
+        gsrc = [oh.DeviceBuffer(rows_n * row_bytes, stream) for _ in range(2)]
+        gdst = [oh.DeviceBuffer(rows_n * row_bytes, stream) for _ in range(2)]
+        for b in gsrc:
+            upload_tiled(b, rng.standard_normal(1 << 21), rows_n * row_bytes)
+        perm = rng.permutation(rows_n).astype(np.int64) * row_bytes
+        dperm = oh.to_device(perm, stream)
+        tabs = (C.POINTER(C.c_int64) * 2)(None, C.cast(dperm.ptr, C.POINTER(C.c_int64)))
+        gsz = oh.sizes([row_bytes // 8, rows_n]); gst1 = oh.strides([8, 0]); gst2 = oh.strides([8, row_bytes]); gt = [0]
+
+        def k_gather():
+            gt[0] += 1
+            oh.check(lib.och_get_index(F64, 2, gsz, tabs, gst1, gsrc[gt[0] % 2].ptr, gst2, gdst[gt[0] % 2].ptr, h))
+
+        def k_scatter():
+            gt[0] += 1
+            oh.check(lib.och_set_index(F64, 2, gsz, tabs, gst1, gdst[gt[0] % 2].ptr, gst2, gsrc[gt[0] % 2].ptr, h))
+        configs["extra_gather_65536_rows_of_8KB"] = gbps(2 * rows_n * row_bytes, sample_launches(k_gather), ceil_of("copy_134MB_operands"))
+        configs["extra_scatter_65536_rows_of_8KB"] = gbps(2 * rows_n * row_bytes, sample_launches(k_scatter), ceil_of("copy_134MB_operands"))
+        nr = 1 << 24
+        eperm = (rng.integers(0, rows_n * row_bytes // 8, nr).astype(np.int64)) * 8
+        deperm = oh.to_device(eperm, stream)
+        tab1 = (C.POINTER(C.c_int64) * 1)(C.cast(deperm.ptr, C.POINTER(C.c_int64)))
+
+        def k_gather_elements():
+            gt[0] += 1
+            oh.check(lib.och_get_index(F64, 1, oh.sizes([nr]), tab1, oh.strides([0]), gsrc[gt[0] % 2].ptr, oh.strides([8]), gdst[gt[0] % 2].ptr, h))
+        e = gbps(16 * nr, sample_launches(k_gather_elements))
+        e["Gelements_per_s"] = round(nr / e["ms"] / 1e6, 1)
+        e["note"] = "16M random 8-byte elements out of 537 MB: every element costs the memory system a whole sector"
+        configs["extra_gather_16M_random_8B_elements"] = e
+        for b in gsrc + gdst + [dperm, deperm]:
+            b.free()
+        nm_ = 1 << 26
+        masks = [oh.to_device((rng.random(nm_) < 0.3).astype(np.uint8), stream) for _ in range(2)]
+        work = oh.DeviceBuffer(lib.och_find_workspace_size(nm_), stream)
+        fout = oh.DeviceBuffer(8 * nm_ // 2, stream)
+        nnz = C.c_size_t(); fsz, fst = oh.sizes([nm_]), oh.strides([1]); fturn = [0]
+
+        def k_find():
+            fturn[0] += 1
+            m_ = masks[fturn[0] % 2]
+            oh.check(lib.och_find_count(1, fsz, fst, m_.ptr, work.ptr, C.byref(nnz), h))
+            oh.check(lib.och_find_apply(1, fsz, fst, m_.ptr, work.ptr, None, fout.ptr, h))
+        k_find()
+        e = gbps(2 * nm_ + 8 * nnz.value, sample_launches(k_find))
+        e["note"] = "count (with its read-back of the total) + apply on a 64M-element mask, 30 %% set: the mask read twice, %d positions of 8 bytes written" % nnz.value
+        configs["extra_find_64M_mask_30pct"] = e
+        for b in masks + [work, fout]:
+            b.free()
+
     # ------------------------------------------------------------------ configuration 5 (GEMM)
     if args.only in (None, "c5"):
         def tflops(flop, timing, peak):

@@ -124,6 +124,13 @@ int och_device_synchronize(void);
 int och_stream_create(och_stream *stream);                 /* device_gpu.c:251-288 */
 int och_stream_destroy(och_stream stream);                 /* device_gpu.c:324-346 */
 int och_stream_synchronize(och_stream stream);             /* device_gpu.c:374-382 */
+/* No counterpart in the reference. Products that are cut along K, matrix-vector products and sliced axis reductions  */
+/* keep partial results in a 64 MB workspace that belongs to the stream (taken from the stream-ordered pool at the     */
+/* first such call, or by och_stream_begin_capture; released with the stream). A caller that retires a stream without */
+/* destroying it -- Ocean's device layer recycles up to 64 of them -- gives the workspace back with this call; it is   */
+/* freed behind the work already queued on the stream and the next call that needs one takes a new one. A graph         */
+/* recorded on the stream addresses the old workspace and must not be launched after this call.                        */
+int och_stream_release_workspace(och_stream stream);
 int och_stream_wait_event(och_stream stream, och_event event); /* device_gpu.c:411-420 */
 int och_event_create(och_event *event, int timing);        /* device_gpu.c:292-320; timing=0: disable timing */
 int och_event_destroy(och_event event);                    /* device_gpu.c:350-370 */

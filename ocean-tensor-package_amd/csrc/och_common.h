@@ -62,6 +62,7 @@ struct StreamContext
 };
 int stream_context(hipStream_t stream, StreamContext **ctx);
 int stream_gemm_workspace(hipStream_t stream, char **workspace);
+int stream_release_workspace(hipStream_t stream);
 void stream_context_release(hipStream_t stream);
 /* device address, on the current device, of the file-scope scratch array of och_reduce_all_device_noalloc (och_reduce.hip) */
 int reduce_static_scratch(char **scratch);

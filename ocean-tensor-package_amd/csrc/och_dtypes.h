@@ -76,17 +76,17 @@ template <class T> constexpr bool is_real_v    = !is_complex_v<T>;
 OCH_HD float bits_to_float(uint32_t u) { union { uint32_t u; float f; } c; c.u = u; return c.f; }
 OCH_HD uint32_t float_to_bits(float f) { union { uint32_t u; float f; } c; c.f = f; return c.u; }
 
-OCH_HD float half_to_float(half_t hh)
+/* The reference's routines in integer arithmetic, bit for bit (half.c:26-149): both zeros map to +0, subnormal halves
+   are normalised, Inf / NaN keep their payload; float -> half returns zero below 2^-15, rounds ties (and above) up in
+   magnitude with the carry running into the exponent, encodes the exponents 2^-15 and 2^16 as it does every other
+   (which gives a subnormal pattern and a NaN pattern), and gives 0x7F00 for NaN. */
+OCH_HD float half_to_float_soft(half_t hh)
 {
    uint32_t h = hh.v;
    uint32_t s = (h & 0x8000u) << 16;
    h &= 0x7FFFu;
    if (h == 0) return 0.f;                       /* both zeros map to +0 */
    uint32_t e = h & 0x7C00u;
-#if defined(__HIP_DEVICE_COMPILE__)
-   /* finite non-zero values: the hardware conversion is exact, as is the normalisation loop below (subnormals included) */
-   if (e != 0x7C00u) { _Float16 x; __builtin_memcpy(&x, &hh.v, 2); return (float)x; }
-#endif
    if (e == 0)
    {  /* subnormal: normalise the mantissa */
       uint32_t shift = 1; h <<= 1;
@@ -98,7 +98,7 @@ OCH_HD float half_to_float(half_t hh)
    return bits_to_float(((h << 13) + 0x38000000u) | s);
 }
 
-OCH_HD half_t float_to_half(float f)
+OCH_HD half_t float_to_half_soft(float f)
 {
    uint32_t raw = float_to_bits(f);
    uint32_t d   = raw & 0x007FFFFFu;
@@ -116,6 +116,46 @@ OCH_HD half_t float_to_half(float f)
    r.v = (uint16_t)v;
    return r;
 }
+
+#if defined(__HIP_DEVICE_COMPILE__)
+/* On the device the common case is a few instructions around the hardware converters, without a divergent branch:
+   half -> float is exact in hardware for every value but a NaN (whose payload the integer routine carries over bit by
+   bit), subnormals included, and adding +0 turns -0 into +0; float -> half with rounding toward zero gives, for
+   2^-14 <= |f| < 2^16, exactly the reference's truncated pattern ((exponent - 112) << 10 | mantissa >> 13 | sign), to
+   which the reference's rounding adds bit 12 of the float. Only lanes with a NaN half, or a float whose exponent is one
+   of the two that the reference encodes in its own way or lies above them, take the integer routine -- behind a branch
+   that is uniform over the wave, so waves without such a value never execute it. (The empty asm statements keep the
+   compiler from turning those branches into unconditional arithmetic.) */
+OCH_D float half_to_float(half_t hh)
+{
+   _Float16 x; __builtin_memcpy(&x, &hh.v, 2);
+   float r = (float)x + 0.0f;
+   if (__builtin_amdgcn_ballot_w64(r != r) != 0)
+   {  asm volatile("" ::: "memory");
+      if (r != r) r = bits_to_float(((uint32_t)(hh.v & 0x7FFFu) << 13) | 0x7F800000u | ((uint32_t)(hh.v & 0x8000u) << 16));
+   }
+   return r;
+}
+OCH_D half_t float_to_half(float f)
+{
+   const uint32_t raw = float_to_bits(f), a = raw & 0x7FFFFFFFu;
+   const auto pk = __builtin_amdgcn_cvt_pkrtz(f, 0.0f);
+   uint32_t t; __builtin_memcpy(&t, &pk, 4);
+   const bool under = a < 0x38000000u;                               /* below 2^-15: zero, sign dropped */
+   const uint32_t v = under ? 0u : t + ((raw >> 12) & 1u);
+   /* exponent 2^-15, or 2^16 and above (values below 2^-15 are moved into the ordinary range for this test) */
+   const uint32_t c = (under ? 0x38800000u : a) - 0x38800000u;
+   half_t r; r.v = (uint16_t)v;
+   if (__builtin_amdgcn_uicmp(c, 0x0F000000u, 35 /* unsigned >= : the lanes' results as one 64-bit mask */) != 0)
+   {  asm volatile("" ::: "memory");
+      if (c >= 0x0F000000u) r = float_to_half_soft(f);
+   }
+   return r;
+}
+#else
+OCH_HD float half_to_float(half_t hh) { return half_to_float_soft(hh); }
+OCH_HD half_t float_to_half(float f) { return float_to_half_soft(f); }
+#endif
 
 /* ---- float -> integer with x86-64 scalar converter results ------------- */
 template <class F> OCH_HD int32_t cvtt_i32(F x)

@@ -869,8 +869,11 @@ template <class A, class B, class C> constexpr int vec_for3()
 /* Launcher signature: (parameters, workgroups, threads per workgroup) */
 template <int NOPS, class LW, class LM, class LS, class LR>
 static int ew_dispatch(const EwShape<NOPS> &s, uint64_t flat0, int vec, const int (&es)[NOPS],
-                       LW &&wide, LM &&mixed, LS &&single, LR &&rows)
+                       LW &&wide, LM &&mixed, LS &&single, LR &&rows, bool streaming_form = true)
 {
+   /* streaming_form = false: a launch that only writes keeps the plain stores and the 256-thread workgroups whatever
+      its size (a float32 fill of 268 MB: 6.0 TB/s in the streaming form, the write ceiling of 6.6 - 6.8 is reached
+      by plain stores) */
    EwParams<NOPS> p;
    /* unit-stride rows that are not whole aligned vectors (see the row kernels): a width that VEC does not divide (a
       one-dimensional shape of such a length is cut into body and tail below instead), or a unit-stride operand whose
@@ -883,6 +886,7 @@ static int ew_dispatch(const EwShape<NOPS> &s, uint64_t flat0, int vec, const in
    }
    auto run = [&](const EwShape<NOPS> &sh, uint64_t f0) -> bool
    {  if (!ew_params<NOPS>(p, sh, vec, es, f0, NOPS - 1)) return false;      /* vec = 1 (16-byte elements) always fits */
+      if (!streaming_form) p.nt = 0;
       bool all = true;
       for (int k = 0; k < NOPS; k++) all = all && (p.vecmode[k] == 1);
       const uint32_t block = p.nt ? OCH_EW_BLOCK_STREAM : OCH_EW_BLOCK;
@@ -1083,7 +1087,7 @@ static int launch_ew1(int ndims, const size_t *size, const ptrdiff_t *st, void *
          {  if constexpr (VEC > 1)
             {  if (p.nt) hipLaunchKernelGGL((ew1_rows_kernel<F, VEC, true>), dim3(blocks), dim3(threads), 0, stream, p, prm);
                else      hipLaunchKernelGGL((ew1_rows_kernel<F, VEC, false>), dim3(blocks), dim3(threads), 0, stream, p, prm);
-            } });
+            } }, F::RMW);
    });
 }
 

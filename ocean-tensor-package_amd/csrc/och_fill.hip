@@ -68,7 +68,12 @@ static const fill_fn fillnan_table[DT_COUNT] = { 0, 0, 0, 0, 0, 0, 0, 0, 0,
    &launch_fill<FillNaNOp, half_t>, &launch_fill<FillNaNOp, float>, &launch_fill<FillNaNOp, double>,
    &launch_fill<FillNaNOp, chalf_t>, &launch_fill<FillNaNOp, cfloat_t>, &launch_fill<FillNaNOp, cdouble_t> };
 
-/* ---- masked fill: data[i] = value where mask[i] ---- */
+/* ---- masked fill: data[i] = value where mask[i] ----
+   A thread owns VEC neighbouring elements (16 bytes of the tensor, VEC mask bytes). Where the tensor is unit-stride and
+   aligned, the group moves as a whole: nothing when no mask byte of the group is set, one 16-byte store when all are,
+   otherwise the group is read, the set elements are replaced and the group is written back -- stores of single
+   elements leave the memory system to merge them into the lines it holds, which runs at about half the rate. Otherwise
+   element by element. */
 template <class T, int VEC>
 __global__ __launch_bounds__(OCH_EW_BLOCK) void masked_fill_kernel(const EwParams<2> p, const T value)
 {
@@ -78,6 +83,18 @@ __global__ __launch_bounds__(OCH_EW_BLOCK) void masked_fill_kernel(const EwParam
    group_offsets<2>(p, g, off);
    Pack<obool, VEC> m;
    load_pack<obool, VEC>(m, p.ptr[1] + off[1], p.estride[1], p.vecmode[1]);
+   if (VEC > 1 && p.vecmode[0] == 1)
+   {  bool any = false, all = true;
+#pragma unroll
+      for (int k = 0; k < VEC; k++) { any = any || (m.v[k].v != 0); all = all && (m.v[k].v != 0); }
+      if (!any) return;
+      Pack<T, VEC> d;
+      if (!all) load_wide<T, VEC>(d, p.ptr[0] + off[0]);
+#pragma unroll
+      for (int k = 0; k < VEC; k++) if (all || m.v[k].v) d.v[k] = value;
+      store_wide<T, VEC>(d, p.ptr[0] + off[0]);
+      return;
+   }
 #pragma unroll
    for (int k = 0; k < VEC; k++)
       if (m.v[k].v) *reinterpret_cast<T *>(p.ptr[0] + off[0] + k * p.estride[0]) = value;
@@ -91,10 +108,10 @@ static int launch_masked_fill(int nd, const size_t *size, const ptrdiff_t *st1, 
    if (ew_normalize<2>(shape, nd, size, strides, ptrs, 0, true) != 0) return -1;
    const int es[2] = { (int)sizeof(T), 1 };
    T v = scalar_as<T>(value);
-   constexpr int VEC = 4;
+   constexpr int VEC = vec_for<T>();
    return ew_launch_chunked<2>(shape, 0, [&](const EwShape<2> &s, uint64_t flat0) -> int
    {  EwParams<2> p;
-      if (ew_params<2>(p, s, VEC, es, flat0))
+      if (VEC > 1 && ew_params<2>(p, s, VEC, es, flat0))
          hipLaunchKernelGGL((masked_fill_kernel<T, VEC>), dim3((p.ngroups + OCH_EW_BLOCK - 1) / OCH_EW_BLOCK), dim3(OCH_EW_BLOCK), 0, stream, p, v);
       else
       {  ew_params<2>(p, s, 1, es, flat0);

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void index_to_offset_kernel(uint64_t nelem, in
    V > 1: a work item is a run of V elements (16 bytes) along a dense dimension 0 that has no offset table; the host has
    divided size[0] by V and set both strides of dimension 0 to 16. Offset tables are device data, so whether a run is
    16-byte aligned is only known here: aligned runs move in one access, others element by element. */
-template <class E, int MODE, int V>
+template <class E, int MODE, int V, bool NT = false>
 __global__ __launch_bounds__(256) void index_kernel(const IndexParams p, const E value)
 {
    const bool small = p.small != 0;
@@ -70,7 +70,12 @@ __global__ __launch_bounds__(256) void index_kernel(const IndexParams p, const E
       }
       char *a = p.ptr1 + o1, *b = p.ptr2 + o2;
       if (V > 1 && ((((uintptr_t)a) | (MODE != 2 ? (uintptr_t)b : 0)) & 15) == 0)
-      {  if (MODE == 0) *reinterpret_cast<uint4 *>(b) = *reinterpret_cast<const uint4 *>(a);
+      {  typedef typename RawVec<16>::type W;
+         if constexpr (NT && MODE != 2)
+         {  if (MODE == 0) __builtin_nontemporal_store(__builtin_nontemporal_load(reinterpret_cast<const W *>(a)), reinterpret_cast<W *>(b));
+            else           *reinterpret_cast<W *>(a) = __builtin_nontemporal_load(reinterpret_cast<const W *>(b));     /* scattered rows: plain stores */
+         }
+         else if (MODE == 0) *reinterpret_cast<uint4 *>(b) = *reinterpret_cast<const uint4 *>(a);
          else if (MODE == 1) *reinterpret_cast<uint4 *>(a) = *reinterpret_cast<const uint4 *>(b);
          else { union { uint4 w; E e[V]; } u; for (int k = 0; k < V; k++) u.e[k] = value; *reinterpret_cast<uint4 *>(a) = u.w; }
          continue;
@@ -100,10 +105,13 @@ static int launch_index(IndexParams &p, const och_scalar &value, hipStream_t str
    /* above the launch limit of the elementwise engine (2^32 - 2^16 elements unless a test has lowered it) the kernel
       decomposes the 64-bit work-item number with plain divisions; its grid-stride loop covers any count */
    p.small = (p.nelem <= ew_launch_limit()) ? 1 : 0;
+   /* the call moves more than the caches hold: 16-byte runs with the nontemporal hint (a compile-time property of the kernel) */
+   const bool nt = runs && MODE != 2 && p.nelem * 32 >= OCH_EW_STREAM_BYTES;
    if (p.small)
       for (int d = 0; d < p.ndims; d++) p.div[d] = make_fastdiv((uint32_t)p.size[d]);
    uint64_t blocks = (p.nelem + 255) / 256; if (blocks > (1u << 20)) blocks = 1u << 20;
-   if (runs) hipLaunchKernelGGL((index_kernel<E, MODE, V>), dim3((unsigned)blocks), dim3(256), 0, stream, p, v);
+   if (nt)   hipLaunchKernelGGL((index_kernel<E, MODE, V, true>), dim3((unsigned)blocks), dim3(256), 0, stream, p, v);
+   else if (runs) hipLaunchKernelGGL((index_kernel<E, MODE, V>), dim3((unsigned)blocks), dim3(256), 0, stream, p, v);
    else      hipLaunchKernelGGL((index_kernel<E, MODE, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, p, v);
    OCH_CHECK_LAUNCH();
    return 0;

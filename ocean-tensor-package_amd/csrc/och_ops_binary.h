@@ -44,12 +44,24 @@ template <class T> OCH_D bool prod_negative(T x, T y)
    else return int_mul<T>(x, y) < 0;
 }
 
+/* magnitude of a signed value as its unsigned twin (the most negative value keeps its bit pattern, 2^(bits-1)) */
+template <class T> OCH_D typename uwrap<T>::type int_magnitude(T x)
+{  typedef typename uwrap<T>::type U; return (x < 0) ? (U)((U)0 - (U)x) : (U)x; }
+
 /* Quotient of the reference's integer expressions, evaluated in `int` for
-   8/16-bit operands (so -128 / -1 wraps on the final store only). */
+   8/16-bit operands (so -128 / -1 wraps on the final store only). 64-bit signed operands divide as magnitudes: the
+   unsigned division takes its short form (one 32-bit division) whenever both magnitudes fit 32 bits -- the signed one
+   only when both operands are non-negative, so mixed signs in a wave ran the short and the long form one after the other
+   -- and the most negative value divided by -1 comes out wrapped without a case of its own. */
 template <class T> OCH_D T int_quot(T x, T y)
 {
    if constexpr (is_uint_v<T>) return (T)(x / y);
    else if constexpr (sizeof(T) < 4) return (T)((int32_t)x / (int32_t)y);
+   else if constexpr (sizeof(T) == 8)
+   {  typedef typename uwrap<T>::type U;
+      const U q = int_magnitude<T>(x) / int_magnitude<T>(y);
+      return (T)(((x < 0) != (y < 0)) ? (U)((U)0 - q) : q);
+   }
    else
    {  /* most-negative / -1 overflows; the x86 result the CPU path would trap on is not
          reproducible, return the wrapped value */
@@ -61,6 +73,12 @@ template <class T> OCH_D T int_rem(T x, T y)
 {
    if constexpr (is_uint_v<T>) return (T)(x % y);
    else if constexpr (sizeof(T) < 4) return (T)((int32_t)x % (int32_t)y);
+   else if constexpr (sizeof(T) == 8)
+   {  /* the remainder takes the sign of the dividend; x % -1 = 0 follows */
+      typedef typename uwrap<T>::type U;
+      const U r = int_magnitude<T>(x) % int_magnitude<T>(y);
+      return (T)((x < 0) ? (U)((U)0 - r) : r);
+   }
    else { if (y == (T)-1) return (T)0; return (T)(x % y); }
 }
 

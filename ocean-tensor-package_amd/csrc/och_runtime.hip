@@ -64,11 +64,26 @@ int stream_gemm_workspace(hipStream_t stream, char **workspace)
    if (stream_context(stream, &c) != 0) return -1;
    std::lock_guard<std::mutex> lock(g_stream_ctx_mutex);
    if (c->gemm_workspace == nullptr)
-   {  void *w = nullptr;
-      OCH_CHECK_HIP(hipMalloc(&w, OCH_GEMM_WORKSPACE));
+   {  /* from the stream-ordered pool: no device-wide synchronisation, and what och_stream_release_workspace gives back
+         serves the next stream that needs one */
+      void *w = nullptr;
+      OCH_CHECK_HIP(hipMallocAsync(&w, OCH_GEMM_WORKSPACE, stream));
       c->gemm_workspace = (char *)w;
    }
    *workspace = c->gemm_workspace;
+   return 0;
+}
+/* gives the stream's workspace back to the pool, behind the work already queued on the stream */
+int stream_release_workspace(hipStream_t stream)
+{
+   int dev;
+   OCH_CHECK_HIP(hipGetDevice(&dev));
+   std::lock_guard<std::mutex> lock(g_stream_ctx_mutex);
+   auto it = g_stream_ctx.find(std::make_pair(dev, stream));
+   if (it == g_stream_ctx.end() || it->second.gemm_workspace == nullptr) return 0;
+   char *w = it->second.gemm_workspace;
+   it->second.gemm_workspace = nullptr;
+   OCH_CHECK_HIP(hipFreeAsync(w, stream));
    return 0;
 }
 void stream_context_release(hipStream_t stream)
@@ -79,7 +94,7 @@ void stream_context_release(hipStream_t stream)
    auto it = g_stream_ctx.find(std::make_pair(dev, stream));
    if (it == g_stream_ctx.end()) return;
    (void)hipFree(it->second.red_scratch); (void)hipHostFree(it->second.host_result);
-   if (it->second.gemm_workspace) (void)hipFree(it->second.gemm_workspace);
+   if (it->second.gemm_workspace) (void)hipFreeAsync(it->second.gemm_workspace, stream);
    g_stream_ctx.erase(it);
 }
 
@@ -211,6 +226,7 @@ int och_stream_destroy(och_stream stream)
    OCH_CHECK_HIP(hipStreamDestroy((hipStream_t)stream));
    return 0;
 }
+int och_stream_release_workspace(och_stream stream) { return och::stream_release_workspace((hipStream_t)stream); }
 int och_stream_synchronize(och_stream stream) { OCH_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream)); OCH_CHECK_AFTER_WAIT("a stream"); return 0; }
 int och_stream_wait_event(och_stream stream, och_event event)
 {  OCH_CHECK_HIP(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0)); return 0; }

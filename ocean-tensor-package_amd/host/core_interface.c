@@ -100,7 +100,13 @@ int OcTensor_binary(int op, OcTensor *src1, OcTensor *src2, OcTensor **dst)
    if (is_logical) dtype = OcDTypeBool;
    dtype2 = dtype;
    if (is_shift) dtype2 = OcDTypeInt8;
-   if (op == 6 && !OcDType_isFloat(dtype)) dtype2 = OcDTypeInt16;
+   if (op == 6)
+   {  /* power (tensor_itf.c:4736-4760): the base keeps its type (widened by a given destination's); two integer
+         operands take an int16 exponent, anything else the common type for both */
+      dtype = (*dst) ? OcDType_getCommonType(src1->dtype, (*dst)->dtype) : src1->dtype;
+      if (!OcDType_isFloat(dtype) && !OcDType_isFloat(src2->dtype)) dtype2 = OcDTypeInt16;
+      else { dtype = OcDType_getCommonType(dtype, src2->dtype); dtype2 = dtype; }
+   }
    rtype = is_compare ? OcDTypeBool : dtype;
    a = OcIncrefTensor(src1); b = OcIncrefTensor(src2);
    /* converted operands live in the device's ring of temporary storages: releasing them does not wait for the device */
@@ -146,6 +152,7 @@ int OcTensor_unary(int op, OcTensor *src, OcTensor **dst)
       static const OcDType signed_of[5] = { OcDTypeInt16, OcDTypeInt16, OcDTypeInt32, OcDTypeInt64, OcDTypeDouble };
       OcDType work = a->dtype;
       if (op == 0 && work >= OcDTypeUInt8 && work <= OcDTypeUInt64) work = signed_of[work];
+      if (op == 2) work = OcDTypeBool;                                      /* logical not works on truth values (tensor_itf.c:3669-3676) */
       if (OcTensor_ensure(&a, work, a->device) != 0) goto final;
    }
    rtype = a->dtype;
@@ -179,6 +186,35 @@ int OcTensor_reduceAll(int which, OcTensor *tensor, double p, OcScalar *result)
          case 27: r = m->Tensor_norm2(a, result); break;      case 28: r = m->Tensor_norm2NaN(a, result); break;
          default: OcErrorMessage("Reduction %d does not return a scalar", which);
       }
+   }
+   OcDecrefTensor(a);
+   return r;
+}
+/* the logical reductions (any, all, allFinite, anyInf, anyNaN: which = 0 ... 4) and the counts (nnz, nnzNaN: 5, 6) of
+   tensor_itf.c:5299-5400, through the same table */
+int OcTensor_reduceLogical(int which, OcTensor *tensor, int *result)
+{  OcTensor *a = OcIncrefTensor(tensor); int r = -1;
+   if (OcTensor_ensure(&a, a->dtype, a->device) == 0)
+   {  OcModuleCore *m = OcModuleCore_forDevice(a->device);
+      if (m == NULL) OcErrorMessage("No core module is registered for device %s", a->device->name);
+      else switch (which)
+      {  case 0: r = m->Tensor_any(a, result); break;        case 1: r = m->Tensor_all(a, result); break;
+         case 2: r = m->Tensor_allFinite(a, result); break;  case 3: r = m->Tensor_anyInf(a, result); break;
+         case 4: r = m->Tensor_anyNaN(a, result); break;
+         default: OcErrorMessage("Reduction %d does not return a truth value", which);
+      }
+   }
+   OcDecrefTensor(a);
+   return r;
+}
+int OcTensor_reduceCount(int which, OcTensor *tensor, OcUInt64 *result)
+{  OcTensor *a = OcIncrefTensor(tensor); int r = -1;
+   if (OcTensor_ensure(&a, a->dtype, a->device) == 0)
+   {  OcModuleCore *m = OcModuleCore_forDevice(a->device);
+      if (m == NULL) OcErrorMessage("No core module is registered for device %s", a->device->name);
+      else if (which == 5) r = m->Tensor_nnz(a, result);
+      else if (which == 6) r = m->Tensor_nnzNaN(a, result);
+      else OcErrorMessage("Reduction %d does not return a count", which);
    }
    OcDecrefTensor(a);
    return r;
@@ -475,6 +511,19 @@ static int index_view(OcTensor *tensor, OcTensor *indices, OcTensorIndexView *vi
       if (OcTensor_copy(indices, idx) != 0) { OcDecrefTensor(idx); return -1; }
       for (d = 0; d < k; d++)              /* negative indices: add the dimension's size, row by row */
       {  OcTensor *row = OcTensor_slice(idx, 0, d, 1, 1);
+         /* every index must lie in [-size, size): checked with the module's own full reductions before anything is
+            addressed through it, as the interface does when an index is bound (index_itf.c:1311-1336, which keeps the
+            minimum and maximum of every index row) */
+         if (row != NULL && n > 0)
+         {  OcScalar lo, hi;
+            if (m->Tensor_minimum == NULL || m->Tensor_maximum == NULL || m->Tensor_minimum(row, &lo) != 0 || m->Tensor_maximum(row, &hi) != 0)
+            {  OcDecrefTensor(row); OcDecrefTensor(idx); OcError(-1, "Could not determine the range of the tensor indices"); }
+            if (lo.value.sInt64 < -(OcInt64)tensor->size[d] || hi.value.sInt64 >= (OcInt64)tensor->size[d])
+            {  long bad = (long)((lo.value.sInt64 < -(OcInt64)tensor->size[d]) ? lo.value.sInt64 : hi.value.sInt64);
+               OcDecrefTensor(row); OcDecrefTensor(idx);
+               OcError(-1, "Tensor index (%ld) out of range (%lu) at dimension %d", bad, (unsigned long)tensor->size[d], d);
+            }
+         }
          s.dtype = OcDTypeInt64; s.value.sInt64 = tensor->size[d];
          if (row == NULL || m->Tensor_addIfNegative(row, &s) != 0) { if (row) OcDecrefTensor(row); OcDecrefTensor(idx); return -1; }
          OcDecrefTensor(row);

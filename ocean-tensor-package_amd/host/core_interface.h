@@ -33,6 +33,8 @@ OcTensor *OcTensor_maskToOffset(OcTensor *mask, OcIndex *strides);              
 int OcTensor_binary(int op, OcTensor *src1, OcTensor *src2, OcTensor **dst);       /* op: index into the table's binary block */
 int OcTensor_unary(int op, OcTensor *src, OcTensor **dst);
 int OcTensor_reduceAll(int which, OcTensor *tensor, double p, OcScalar *result);    /* which: och reduction index of an OcScalar-valued reduction */
+int OcTensor_reduceLogical(int which, OcTensor *tensor, int *result);            /* which: 0 any, 1 all, 2 allFinite, 3 anyInf, 4 anyNaN */
+int OcTensor_reduceCount(int which, OcTensor *tensor, OcUInt64 *result);         /* which: 5 nnz, 6 nnzNaN */
 int OcTensor_axisReduce(int which, OcTensor *src, int n, int *axes, int keepdims, double p, OcTensor **dst);
 int OcTensor_gemm(OcScalar *alpha, OcTensor *A, char modeA, OcTensor *B, char modeB, OcScalar *beta, OcTensor **C);
 int OcTensor_gemmTensors(OcTensor *alpha, OcTensor *A, char modeA, OcTensor *B, char modeB, OcTensor *beta, OcTensor **C);   /* scalars as tensors (one per product), NULL: 1 and 0 */

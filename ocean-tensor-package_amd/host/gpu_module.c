@@ -63,7 +63,12 @@ static void OcDeviceGPU_deleteStream(OcStream *stream)
 {  OcDeviceGPUFull *g;
    if (stream == NULL) return;
    g = (OcDeviceGPUFull *)stream->device;
-   if (g->nFreeStreams < OC_GPU_MAX_FREE) { stream->next = g->freeStreams; g->freeStreams = stream; g->nFreeStreams++; }
+   if (g->nFreeStreams < OC_GPU_MAX_FREE)
+   {  /* a retired stream keeps its small reduction scratch but gives its 64 MB workspace back to the pool */
+      och_device_set(stream->device->index);
+      och_stream_release_workspace(((OcStreamGPU *)stream)->handle);
+      stream->next = g->freeStreams; g->freeStreams = stream; g->nFreeStreams++;
+   }
    else { och_stream_destroy(((OcStreamGPU *)stream)->handle); OcFree(stream); }
 }
 static int OcDeviceGPU_createEvent(OcDevice *device, OcEvent **event)

@@ -140,6 +140,7 @@ PROTOTYPES = {
     "och_reduce_set_part_limit": (None, [C.c_size_t]),
     "och_reduce_axis_set_output_limit": (None, [C.c_size_t]),
     "och_reduce_axis_set_range_limit": (None, [C.c_size_t]),
+    "och_stream_release_workspace": (C.c_int, [C.c_void_p]),
     "och_elemwise_set_launch_limit": (C.c_int, [C.c_size_t]),
     "och_device_count": (_i, [C.POINTER(_i)]),
     "och_device_set": (_i, [_i]),

@@ -41,6 +41,11 @@ class Scalar(C.Structure):
 
     def get(self):
         v = self.value
+        if self.dtype == HALF:
+            return float(np.array([v.u16], np.uint16).view(np.float16)[0])
+        if self.dtype == CHALF:
+            parts = np.array([v.u32 & 0xFFFF, v.u32 >> 16], np.uint16).view(np.float16)
+            return complex(float(parts[0]), float(parts[1]))
         return {BOOL: v.u8, UINT8: v.u8, UINT16: v.u16, UINT32: v.u32, UINT64: v.u64, INT8: v.i8, INT16: v.i16, INT32: v.i32,
                 INT64: v.i64, FLOAT: v.f32, DOUBLE: v.f64, CFLOAT: complex(*v.c64), CDOUBLE: complex(*v.c128)}[self.dtype]
 

@@ -359,3 +359,35 @@ def test_elementwise_launch_limit_cuts_calls_into_runs():
         assert p.launches == 1
     finally:
         oh.lib.och_elemwise_set_launch_limit(0)
+
+
+PIPELINED_GEMM_SOURCES = ["och_gemm_f32p.hip", "och_gemm_f64p.hip", "och_gemm_c32p.hip", "och_gemm_c64p.hip"]
+
+
+@pytest.mark.parametrize("source", PIPELINED_GEMM_SOURCES)
+def test_m0_is_used_by_the_loads_to_lds_only(source):
+    """The pipelined GEMM kernels pass the LDS target of `global_load_lds_dwordx4` in M0 from inline assembly without
+    the compiler knowing. That is sound only while the compiler itself keeps nothing in M0 across those statements
+    (dynamic register indexing, LDS-direct reads, s_sendmsg and v_readlane with M0 would): every mention of M0 in the
+    generated code of these kernels must be the `s_mov_b32 m0, <sgpr>` of such a load, followed by the load within the
+    next two instructions."""
+    import re
+    import shutil
+    import subprocess
+    import tempfile
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc is not available")
+    src = os.path.join(ROOT, "ocean-tensor-package_amd", "csrc", source)
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "k.s")
+        subprocess.run([hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang",
+                        "-packed-fp32-ops", "-Wno-unused-command-line-argument", "--cuda-device-only", "-S", src, "-o", out],
+                       check=True, capture_output=True)
+        lines = [ln.split(";")[0].strip() for ln in open(out)]
+    code = [ln for ln in lines if ln and not ln.startswith(".") and not ln.endswith(":")]
+    uses = [i for i, ln in enumerate(code) if re.search(r"\bm0\b", ln)]
+    assert len(uses) >= 8, "no load to LDS found in %s" % source
+    for i in uses:
+        assert re.fullmatch(r"s_mov_b32 m0, s\d+", code[i]), code[i]
+        assert any(c.startswith("global_load_lds_dwordx4") for c in code[i + 1:i + 3]), code[i:i + 3]

@@ -303,3 +303,70 @@ def test_memset_is_exact_at_any_alignment_and_size(hip, stream):
     got = big.download(np.uint8)
     assert got.min() == 0x5A and got.max() == 0x5A
     big.free()
+
+
+def half_conversion_floats():
+    """float32 bit patterns that reach every branch of the float -> half rule (half.c:101-149) on both sides of each
+    boundary: every exponent with mantissas just below, at and above the rounding tie, with the kept bits all clear, all
+    set (the carry runs into the exponent) and mixed; both signs; zeros, subnormals, infinities and NaNs."""
+    low = np.array([0x0000, 0x0001, 0x0FFF, 0x1000, 0x1001, 0x1FFF], np.uint32)                  # the 13 bits that are dropped
+    kept = np.array([0x000, 0x001, 0x155, 0x2AA, 0x3FE, 0x3FF], np.uint32) << 13              # the 10 bits that are kept
+    mant = (kept[:, None] | low[None, :]).reshape(-1)
+    ex = np.arange(256, dtype=np.uint32) << 23
+    bits = (ex[:, None] | mant[None, :]).reshape(-1)
+    bits = np.concatenate([bits, bits | np.uint32(0x80000000)])
+    rng = np.random.default_rng(99)
+    extra = rng.integers(0, 1 << 32, 200000, dtype=np.uint64).astype(np.uint32)
+    near = (rng.integers(100, 150, 200000).astype(np.uint32) << 23) | rng.integers(0, 1 << 23, 200000).astype(np.uint32) | (rng.integers(0, 2, 200000).astype(np.uint32) << 31)
+    return np.concatenate([bits, extra, near]).view(np.float32)
+
+
+def test_half_conversions_cover_every_rule(hip, stream):
+    """All 65536 half patterns to float and double, and a set of floats built to hit every branch of the float -> half
+    rule (ties, the carry into the exponent, the flush below 2^-15, the exponents 2^-15 and 2^16 that the CPU routine
+    encodes in its own way, overflow, NaN), bit for bit against the oracle, whose converter is pinned exhaustively
+    against the reference's half.c. Lanes that take the integer routine sit next to lanes that do not."""
+    halfs = np.arange(65536, dtype=np.uint16)
+    rng = np.random.default_rng(7)
+    halfs = np.concatenate([halfs, rng.permutation(halfs)])                  # special values scattered among ordinary ones
+    n = halfs.size
+    src = oh.to_device(halfs, stream)
+    for dst_type, npt in ((H.FLOAT, np.float32), (H.DOUBLE, np.float64)):
+        es = np.dtype(npt).itemsize
+        dst = oh.DeviceBuffer(es * n, stream)
+        oh.check(oh.lib.och_copy(H.HALF, dst_type, 1, oh.sizes([n]), oh.strides([2]), src.ptr, 1, oh.sizes([n]), oh.strides([es]), dst.ptr, stream.handle))
+        got = dst.download(npt)
+        want = np.empty(n, npt)
+        assert orc.lib.oracle_copy(H.HALF, dst_type, 1, oh.sizes([n]), oh.strides([2]), orc.ptr(halfs), 1, oh.sizes([n]), oh.strides([es]), orc.ptr(want), 4) == 0
+        assert got.tobytes() == want.tobytes(), "half -> %s" % H.NAMES[dst_type]
+        dst.free()
+    src.free()
+    floats = half_conversion_floats()
+    n = floats.size
+    src = oh.to_device(floats, stream)
+    dst = oh.DeviceBuffer(2 * n, stream)
+    oh.check(oh.lib.och_copy(H.FLOAT, H.HALF, 1, oh.sizes([n]), oh.strides([4]), src.ptr, 1, oh.sizes([n]), oh.strides([2]), dst.ptr, stream.handle))
+    got = dst.download(np.uint16)
+    want = np.empty(n, np.uint16)
+    assert orc.lib.oracle_copy(H.FLOAT, H.HALF, 1, oh.sizes([n]), oh.strides([4]), orc.ptr(floats), 1, oh.sizes([n]), oh.strides([2]), orc.ptr(want), 4) == 0
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, "float -> half: %d differ, first %r -> got %#06x want %#06x" % (bad.size, floats[bad[0]], got[bad[0]], want[bad[0]])
+    src.free(); dst.free()
+    # arithmetic on the half types goes through both converters: x + y, x * y and x / y on every pairing of a few hundred
+    # patterns that include both zeros, subnormals, the largest finite value, infinities and NaNs
+    pats = np.concatenate([np.array([0x0000, 0x8000, 0x0001, 0x8001, 0x03FF, 0x0400, 0x7BFF, 0xFBFF, 0x7C00, 0xFC00, 0x7C01, 0x7E00, 0xFE01, 0x3C00, 0xBC00,
+                                     0x0200, 0x8200, 0x3555, 0x7800, 0xF800], np.uint16),
+                           rng.integers(0, 65536, 236).astype(np.uint16)])
+    x = np.repeat(pats, pats.size); y = np.tile(pats, pats.size)
+    n = x.size
+    dx, dy, dz = oh.to_device(x, stream), oh.to_device(y, stream), oh.DeviceBuffer(2 * n, stream)
+    sz, st = oh.sizes([n]), oh.strides([2])
+    for opname in ("add", "multiply", "divide", "subtract"):
+        oh.check(oh.lib.och_binary(oh.B[opname], H.HALF, 1, sz, st, dx.ptr, st, dy.ptr, st, dz.ptr, stream.handle))
+        got = dz.download(np.uint16)
+        want = np.empty(n, np.uint16)
+        assert orc.lib.oracle_binary(oh.B[opname], H.HALF, 1, sz, st, orc.ptr(x), st, orc.ptr(y), st, orc.ptr(want)) == 0
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "half %s: %d differ, first %#06x, %#06x -> got %#06x want %#06x" % (opname, bad.size, x[bad[0]], y[bad[0]], got[bad[0]], want[bad[0]])
+    for b in (dx, dy, dz):
+        b.free()

@@ -82,7 +82,11 @@ def test_promotion_compare_shift_power(gpu):
     te = host.from_numpy(e, host.INT64, gpu)
     small = host.from_numpy((a % 7).astype(np.int16), host.INT16, gpu)
     pw = binary(POWER, small, te)
-    assert pw.contents.dtype == host.INT64 and np.array_equal(host.to_numpy(pw), (a % 7).astype(np.int64) ** e)
+    # an integer base keeps its type and the exponent is taken as int16 (OcTensor_power, tensor_itf.c:4753-4756)
+    assert pw.contents.dtype == host.INT16 and np.array_equal(host.to_numpy(pw), ((a % 7).astype(np.int64) ** e).astype(np.int16))
+    tf = host.from_numpy(np.full((7, 33), 0.5, np.float32), host.FLOAT, gpu)
+    pf = binary(POWER, small, tf)                   # a floating exponent: both operands in the common type
+    assert pf.contents.dtype == host.FLOAT and np.allclose(host.to_numpy(pf), np.sqrt((a % 7).astype(np.float32)), rtol=1e-6)
     # destination of another type: computed in the common type, then converted
     out = host.create([33, 7], host.DOUBLE, gpu)
     binary(ADD, ta, tb, out=out)
@@ -502,6 +506,20 @@ def test_index_tables_on_their_own_streams(gpu):
     host.check(host.lib.OcTensor_getIndexed(t, tp, C.byref(out2)))
     sel = [rows - 1, 0, 5, rows - cols]
     assert np.array_equal(host.to_numpy(out2), want[:, sel])
+    # indices outside [-size, size) are refused before anything is addressed through them (index_itf.c:1311-1336): the
+    # call returns the reference's error, launches no gather or scatter, and leaves the tensor as it was
+    before = host.to_numpy(t)
+    for bad_value, dim in ((rows, 0), (-rows - 1, 0), (cols, 1), (-cols - 1, 1), (1 << 40, 0)):
+        bad = idx2.copy()
+        bad[picks // 2, dim] = bad_value
+        tb = host.from_numpy(bad, host.INT64, gpu)
+        out3 = host.TP()
+        assert host.lib.OcTensor_getIndexed(t, tb, C.byref(out3)) == -1 and not out3
+        msg = host.lib.OcError_lastMessage().decode()
+        assert "out of range" in msg and "(%d)" % bad_value in msg and "dimension %d" % dim in msg, msg
+        assert host.lib.OcTensor_setIndexed(t, tb, tv) == -1
+        host.lib.OcDecrefTensor(tb)
+    assert np.array_equal(host.to_numpy(t), before)
     for x in (t, ti, out, ti2, tv, tp, out2):
         host.lib.OcDecrefTensor(x)
 
