@@ -99,6 +99,7 @@ def main():
 
     import numpy as np
     import ocean_hip as oh
+    import ocean_hip_bench as ohb
 
     oh.check(oh.lib.och_device_set(0))
     oh.check(oh.lib.och_device_warmup(0))
@@ -114,7 +115,7 @@ def main():
 
     def membench(kind, unr, nt, mp, block, blocks, reps, nbytes=None):
         med, best, moved = C.c_float(), C.c_float(), C.c_size_t()
-        oh.check(lib.och_membench(kind, unr, nt, mp, block, blocks, nbytes or MEMBENCH_BYTES[kind], 3, reps, C.byref(med), C.byref(best), C.byref(moved), h))
+        oh.check(ohb.lib.och_membench(kind, unr, nt, mp, block, blocks, nbytes or MEMBENCH_BYTES[kind], 3, reps, C.byref(med), C.byref(best), C.byref(moved), h))
         return moved.value / med.value / 1e6, moved.value / best.value / 1e6
 
     if args.ceiling:
@@ -136,7 +137,7 @@ def main():
         # matrix cores: a loop of nothing but MFMAs, and what other instructions of the same wave cost between them
         def mfmabench(typ, kind, per, waves, iters=4000):
             ms, flop = C.c_float(), C.c_double()
-            oh.check(lib.och_mfmabench(typ, kind, per, waves, iters, 7, C.byref(ms), C.byref(flop), h))
+            oh.check(ohb.lib.och_mfmabench(typ, kind, per, waves, iters, 7, C.byref(ms), C.byref(flop), h))
             return ms.value, flop.value
         print("== matrix cores (och_mfmabench): 16 independent MFMAs per iteration, one block of 4 waves per compute unit (one wave per SIMD)")
         peaks = (("float 32x32x2", MFMA_PEAK["float"]), ("double 16x16x4", MFMA_PEAK["double"]), ("half 32x32x16", 2500.0), ("int8 32x32x32", 5000.0))
@@ -194,6 +195,39 @@ def main():
         def t_sum():
             turn[0] += 1; return xs[turn[0] % 3].sum()
         med, best = torch_time(t_sum); print("   %7.1f  %7.1f   torch.sum, float32, 268 MB (read only)" % (4 * (1 << 26) / med / 1e6, 4 * (1 << 26) / best / 1e6))
+        del xs
+        # the vendor library's matrix products through torch.matmul / torch._int_mm at 8192^3 (T/s median, best): an
+        # independent figure for what the matrix cores sustain on random and on constant operands
+        print("== vendor GEMM through PyTorch at 8192^3, two operand sets alternating (TFLOP/s or TOP/s median, best)")
+        dim = 8192
+
+        def gemm_line(name, make, op, peak):
+            for label, const in (("random operands", False), ("constant operands (1.0 / 1 everywhere)", True)):
+                ops = [(make(const), make(const)) for _ in range(2)]
+                gturn = [0]
+
+                def run():
+                    gturn[0] += 1
+                    a_, b_ = ops[gturn[0] % 2]
+                    return op(a_, b_)
+                try:
+                    med, best = torch_time(run)
+                except Exception as e:                                  # a product the installed library does not offer
+                    print("   %-28s %-40s not available: %s" % (name, label, str(e).splitlines()[0][:80]))
+                    return
+                flop = 2.0 * dim ** 3
+                print("   %8.1f  %8.1f   %-28s %-40s (%.3f of the nominal %.0f)" % (flop / med / 1e9, flop / best / 1e9, name, label, flop / med / 1e9 / peak, peak))
+                del ops
+        gemm_line("float32 NN", lambda c: torch.ones(dim, dim, device=dev) if c else torch.rand(dim, dim, device=dev) * 2 - 1, torch.matmul, MFMA_PEAK["float"])
+        gemm_line("float64 NN", lambda c: torch.ones(dim, dim, device=dev, dtype=torch.float64) if c else torch.rand(dim, dim, device=dev, dtype=torch.float64) * 2 - 1, torch.matmul, MFMA_PEAK["double"])
+        gemm_line("float16 NN", lambda c: torch.ones(dim, dim, device=dev, dtype=torch.float16) if c else (torch.rand(dim, dim, device=dev) * 2 - 1).half(), torch.matmul, 2500.0)
+        gemm_line("float16 TN (A.T @ B)", lambda c: torch.ones(dim, dim, device=dev, dtype=torch.float16) if c else (torch.rand(dim, dim, device=dev) * 2 - 1).half(),
+                  lambda a_, b_: torch.matmul(a_.t(), b_), 2500.0)
+        gemm_line("bfloat16 NN", lambda c: torch.ones(dim, dim, device=dev, dtype=torch.bfloat16) if c else (torch.rand(dim, dim, device=dev) * 2 - 1).bfloat16(), torch.matmul, 2500.0)
+        gemm_line("int8 NN (torch._int_mm)", lambda c: torch.ones(dim, dim, device=dev, dtype=torch.int8) if c else torch.randint(-128, 128, (dim, dim), device=dev, dtype=torch.int8),
+                  lambda a_, b_: torch._int_mm(a_, b_), 5000.0)
+        gemm_line("int8 NT (torch._int_mm)", lambda c: torch.ones(dim, dim, device=dev, dtype=torch.int8) if c else torch.randint(-128, 128, (dim, dim), device=dev, dtype=torch.int8),
+                  lambda a_, b_: torch._int_mm(a_, b_.t()), 5000.0)
         return
 
     def sample_launches(fn, samples=None, warm=3, target_ms=0.6):

@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void index_kernel(const IndexParams p, const E
       {  typedef typename RawVec<16>::type W;
          if constexpr (NT && MODE != 2)
          {  if (MODE == 0) __builtin_nontemporal_store(__builtin_nontemporal_load(reinterpret_cast<const W *>(a)), reinterpret_cast<W *>(b));
-            else           *reinterpret_cast<W *>(a) = __builtin_nontemporal_load(reinterpret_cast<const W *>(b));     /* scattered rows: plain stores */
+            else           *reinterpret_cast<W *>(a) = *reinterpret_cast<const W *>(b);
          }
          else if (MODE == 0) *reinterpret_cast<uint4 *>(b) = *reinterpret_cast<const uint4 *>(a);
          else if (MODE == 1) *reinterpret_cast<uint4 *>(a) = *reinterpret_cast<const uint4 *>(b);
@@ -106,7 +106,7 @@ static int launch_index(IndexParams &p, const och_scalar &value, hipStream_t str
       decomposes the 64-bit work-item number with plain divisions; its grid-stride loop covers any count */
    p.small = (p.nelem <= ew_launch_limit()) ? 1 : 0;
    /* the call moves more than the caches hold: 16-byte runs with the nontemporal hint (a compile-time property of the kernel) */
-   const bool nt = runs && MODE != 2 && p.nelem * 32 >= OCH_EW_STREAM_BYTES;
+   const bool nt = runs && MODE == 0 && p.nelem * 32 >= OCH_EW_STREAM_BYTES;      /* gathers only: scattered rows are written faster by plain stores */
    if (p.small)
       for (int d = 0; d < p.ndims; d++) p.div[d] = make_fastdiv((uint32_t)p.size[d]);
    uint64_t blocks = (p.nelem + 255) / 256; if (blocks > (1u << 20)) blocks = 1u << 20;

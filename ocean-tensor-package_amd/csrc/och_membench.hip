@@ -13,6 +13,7 @@
  * that nothing is served from the 256 MB last-level cache.
  */
 #include "och_common.h"
+#include "../../include/ocean_hip_bench.h"
 #include "och_dtypes.h"
 #include <algorithm>
 #include <vector>

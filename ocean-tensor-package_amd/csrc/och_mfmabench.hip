@@ -7,6 +7,7 @@
  * 64 * waves threads per compute unit, waves = 4 or 8 (one or two waves per SIMD).
  */
 #include "och_common.h"
+#include "../../include/ocean_hip_bench.h"
 #include <vector>
 #include <algorithm>
 #pragma clang diagnostic ignored "-Winline-asm"

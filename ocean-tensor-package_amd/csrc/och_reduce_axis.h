@@ -306,6 +306,43 @@ __global__ __launch_bounds__(256) void axis_group_kernel(const AxisParams p, con
    }
 }
 
+/* Short contiguous rows (one reduced dimension of 1 ... 64 aligned 16-byte groups, a power of two of them): p.glanes =
+   groups per row lanes share an output, every lane loads ONE group per output, and a lane group takes four outputs, one
+   per load instruction, so that each instruction of a wave reads 1 KB of consecutive rows and four are in flight. With one
+   output per lane group a lane had a single load in flight (rows of two groups), or read its row's groups one after the
+   other from lines it shared with its neighbours (8 floats per output: 5.3 TB/s). */
+template <class RD, class T, int VEC, bool NT>
+__global__ __launch_bounds__(256) void axis_short_rows_kernel(const AxisParams p, const typename RD::Param prm)
+{
+   typedef typename RD::Acc Acc;
+   constexpr int U = 4;
+   const uint32_t G = p.glanes, gpw = 64u / G;
+   const uint32_t wave = (blockIdx.x * 256u + threadIdx.x) >> 6, lane = threadIdx.x & 63u, g = lane / G, li = lane % G;
+   Pack<T, VEC> v[U]; int64_t o2[U]; bool active[U];
+#pragma unroll
+   for (int u = 0; u < U; u++)
+   {  const uint32_t o = (wave * U + u) * gpw + g;
+      active[u] = o < p.nout;
+      int64_t o1 = 0; o2[u] = 0;
+      if (active[u])
+      {  axis_outer_offsets(p, o, o1, o2[u]);
+         load_wide<T, VEC, NT>(v[u], p.src + o1 + (int64_t)li * 16);
+      }
+   }
+#pragma unroll
+   for (int u = 0; u < U; u++)
+   {  Acc acc = RD::identity();
+      if (active[u])
+      {
+#pragma unroll
+         for (int k = 0; k < VEC; k++) acc = RD::combine(acc, RD::load(v[u].v[k], prm));
+      }
+#pragma unroll
+      for (int m = 32; m >= 1; m >>= 1) if ((uint32_t)m < G) acc = RD::combine(acc, shfl_xor_any<Acc>(acc, m));
+      if (active[u] && li == 0) *reinterpret_cast<typename RD::Res *>(p.dst + o2[u]) = RD::finalize(acc, prm);
+   }
+}
+
 typedef int (*axis_fn)(const och_reduce_axis_config *c, double pnorm);
 /* outputs one launch handles (0xFFFFFF00 unless och_reduce_axis_set_output_limit has lowered it for a test) */
 uint64_t axis_output_limit();
@@ -539,6 +576,18 @@ static int launch_reduce_axis_one(const och_reduce_axis_config *c, const typenam
       p.slice_rows = 0;
       {  const uint64_t range = (p.rd <= 1) ? (wide ? p.rsize0 / VEC : (rows ? p.rgdiv.d : p.rsize0)) : loads;
          if (plan_slices(blocks, range, (uint64_t)(wave ? p.glanes : 256) * 8) != 0) return -1;
+      }
+      /* short rows: one load per lane and output, four outputs per lane group (see axis_short_rows_kernel) */
+      if (VEC > 1 && wide && wave && p.rd == 1 && p.slices == 1 && !p.partial && loads <= 64 && (loads & (loads - 1)) == 0)
+      {  if constexpr (VEC > 1)
+         {  p.glanes = loads;
+            const uint64_t waves = ((uint64_t)p.nout + 4 * (64 / loads) - 1) / (4 * (64 / loads));
+            const unsigned sblocks = (unsigned)((waves + 3) / 4);
+            if (streaming) hipLaunchKernelGGL((axis_short_rows_kernel<RD, T, VEC, true>), dim3(sblocks), dim3(256), 0, stream, p, prm);
+            else           hipLaunchKernelGGL((axis_short_rows_kernel<RD, T, VEC, false>), dim3(sblocks), dim3(256), 0, stream, p, prm);
+            OCH_CHECK_LAUNCH();
+            return 0;
+         }
       }
       const dim3 grid(blocks, p.slices);
       /* the nontemporal hint only where one load instruction of a wave covers whole cache lines: with fewer than eight

@@ -217,8 +217,6 @@ PROTOTYPES = {
     "och_elemwise_row_units": (C.c_size_t, [C.c_size_t, _i, _i]),
     "och_gemm_set_kernel_choice": (_i, [_i]),
     "och_gemm_split_plan": (_i, [C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_uint, C.c_uint, C.c_uint, C.c_uint, C.POINTER(C.c_double)]),
-    "och_mfmabench": (_i, [_i, _i, _i, _i, _i, _i, C.POINTER(C.c_float), C.POINTER(C.c_double), _vp]),
-    "och_membench": (_i, [_i, _i, _i, _i, _i, _i, C.c_size_t, _i, _i, C.POINTER(C.c_float), C.POINTER(C.c_float), C.POINTER(C.c_size_t), _vp]),
 }
 
 

@@ -391,3 +391,17 @@ def test_m0_is_used_by_the_loads_to_lds_only(source):
     for i in uses:
         assert re.fullmatch(r"s_mov_b32 m0, s\d+", code[i]), code[i]
         assert any(c.startswith("global_load_lds_dwordx4") for c in code[i + 1:i + 3]), code[i:i + 3]
+
+
+def test_microbenchmarks_live_in_their_own_library():
+    """The product header declares no measurement tool; the two micro-benchmarks are declared in include/ocean_hip_bench.h and
+    exported by csrc/libocean_hip_bench.so only."""
+    import ocean_hip_bench as ohb
+    assert not [n for n in declared_functions() if "bench" in n]
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "ocean_hip_bench.h")).read(), flags=re.S)
+    names = sorted(set(re.findall(r"\b(och_[a-z0-9_]+)\s*\(", text)))
+    assert names == ["och_membench", "och_mfmabench"]
+    raw = C.CDLL(ohb.LIB_PATH)
+    assert all(hasattr(raw, n) for n in names)
+    product = C.CDLL(oh.LIB_PATH)
+    assert not any(hasattr(product, n) for n in names)

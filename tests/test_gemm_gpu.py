@@ -257,8 +257,8 @@ def test_gemm_float_last_round_cut_along_k(hip, stream, choice, M, N):
     kernel. 64 slabs give 8 shares of 8 (7 of 10 where 33 tiles are cut, 4 of 16 where 64 are); 17 slabs give two shares of
     9 and 8 where 64 tiles are cut and none where 16 are (two shares would leave most compute units idle); with beta, scalars
     in host and device memory, a K with a remainder."""
-    if hip.device_properties(0).multiprocessor_count != 256:
-        pytest.skip("the sizes are chosen for 256 compute units")
+    # (the sizes are chosen for 256 compute units; on another device the planner cuts differently or not at all, and the
+    #  results are checked all the same)
     rng = np.random.default_rng(1900 + choice + M)
     oh.check(oh.lib.och_gemm_set_kernel_choice(choice))
     try:
@@ -273,8 +273,8 @@ def test_gemm_float_last_round_cut_along_k(hip, stream, choice, M, N):
 def test_gemm_double_last_round_cut_along_k(hip, stream, choice, M, N):
     """The same for double: 16 tiles (ragged sizes: 18 x 17 - 256 = 50) in the last round of 256 compute units, cut into 8
     (5) shares of the 64 slabs of 16 k, two shares of 17 slabs, a K with a remainder."""
-    if hip.device_properties(0).multiprocessor_count != 256:
-        pytest.skip("the sizes are chosen for 256 compute units")
+    # (the sizes are chosen for 256 compute units; on another device the planner cuts differently or not at all, and the
+    #  results are checked all the same)
     rng = np.random.default_rng(2000 + choice + M)
     oh.check(oh.lib.och_gemm_set_kernel_choice(choice))
     try:
@@ -289,8 +289,8 @@ def test_gemm_double_last_round_cut_along_k(hip, stream, choice, M, N):
 def test_gemm_complex_last_round_cut_along_k(hip, stream, dtype, M, N):
     """The same for the complex types: the shares hold the complex sums before alpha (the four real accumulators already
     combined with the signs of the conjugations); complex alpha and beta are applied once, by the kernel that adds the shares."""
-    if hip.device_properties(0).multiprocessor_count != 256:
-        pytest.skip("the sizes are chosen for 256 compute units")
+    # (the sizes are chosen for 256 compute units; on another device the planner cuts differently or not at all, and the
+    #  results are checked all the same)
     rng = np.random.default_rng(2100 + dtype + M)
     oh.check(oh.lib.och_gemm_set_kernel_choice(1))
     try:

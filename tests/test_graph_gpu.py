@@ -155,8 +155,8 @@ def test_graph_with_pipelined_gemm(hip, stream):
     the float product, 320 tiles on 256 compute units) the last round cut along K with its shares in the stream's workspace
     and the kernel that adds them. Every replay equals the eager run of the same number, bit for bit; C accumulates
     (beta = 1), so the runs differ."""
-    if hip.device_properties(0).multiprocessor_count != 256:
-        pytest.skip("the sizes are chosen for 256 compute units")
+    # (the sizes are chosen for 256 compute units; on another device the planner cuts differently or not at all, and the
+    #  results are checked all the same)
     lib, h = oh.lib, stream.handle
     rng = np.random.default_rng(41)
     M, N, K = 2560, 2048, 17 * 32

@@ -269,3 +269,31 @@ def test_axis_reductions_with_more_outputs_than_a_launch_counts(hip, stream):
                     H.assert_same_bytes(got, whole, "%s axes=%s with at most %d outputs per launch" % (name, axes, limit))
     finally:
         oh.lib.och_reduce_axis_set_output_limit(0)
+
+
+SHORT_ROWS = [(H.FLOAT, 8, 5000), (H.FLOAT, 4, 4099), (H.INT32, 16, 3001), (H.DOUBLE, 64, 1100), (H.DOUBLE, 2, 70001), (H.INT8, 256, 1030), (H.INT8, 16, 9000),
+              (H.HALF, 32, 2050), (H.CFLOAT, 8, 2049), (H.INT16, 512, 1025), (H.INT64, 128, 1024)]
+
+
+@pytest.mark.parametrize("dtype,row,nrows", SHORT_ROWS, ids=["%s-%dx%d" % (H.NAMES[d], r, n) for d, r, n in SHORT_ROWS])
+def test_axis_short_contiguous_rows(hip, stream, dtype, row, nrows):
+    """Many outputs, each the reduction of one short contiguous row of 1 ... 64 aligned 16-byte groups: the lanes that
+    share an output load one group each and every lane group takes four outputs, so the last wave has outputs that do
+    not exist. Counts, extremes and integer sums are exact; floating sums within the usual bound."""
+    rng = np.random.default_rng(5200 + dtype + row)
+    parent = H.random_data(dtype, row * nrows, rng, "general").reshape(nrows, row)
+    view = parent.T                                                          # Ocean shape (row, nrows): the row is dimension 0
+    v = to_f64(dtype, view)
+    for name in ("sum", "maximum", "nnz", "any", "norm2", "minimum_abs"):
+        if not oh.lib.och_reduce_supported(oh.R[name], dtype):
+            continue
+        rd, got, want = run_case(stream, name, dtype, parent, view, [0])
+        what = "%s %s rows of %d x %d" % (name, H.NAMES[dtype], row, nrows)
+        if (dtype <= H.INT64 and name != "norm2") or name in ("maximum", "nnz", "any") or (name == "minimum_abs" and dtype < H.CHALF):
+            H.assert_same_bytes(got, want, what)
+            continue
+        g = to_f64(rd, got)
+        truth = {"sum": v.sum(axis=0), "norm2": np.sqrt((np.abs(v) ** 2).sum(axis=0)), "minimum_abs": np.abs(v).min(axis=0)}[name]
+        scale = np.abs(v).sum(axis=0) if name == "sum" else np.abs(truth)
+        tol = 1e-12 if dtype == H.DOUBLE else (4e-3 if dtype == H.HALF else 1e-5)
+        assert np.all(np.abs(g - truth) <= tol * np.maximum(np.asarray(scale), 1e-6)), what

@@ -272,6 +272,39 @@ def test_reductions_on_two_streams_do_not_share_scratch(hip, stream):
     other.synchronize(); other.destroy()
 
 
+def test_cross_block_hand_over_of_full_reductions_under_load(hip, stream):
+    """The blocks of a full reduction hand their partial results to the block that draws the last ticket through device
+    memory, with relaxed device-scope atomics and a wait for the writer's stores in front of the ticket. A partial that
+    the last block read before it had arrived would give a wrong sum. Six streams run long series of full reductions at
+    once -- large sources (one block per compute unit, all their partials in flight) and small ones (few blocks, the last
+    block arrives almost at once), interleaved -- on integer data whose sums are known exactly; every result is compared,
+    and the first mismatch stops the test with its position."""
+    rng = np.random.default_rng(78)
+    nstreams, reps = 6, 150
+    streams = [stream] + [oh.Stream() for _ in range(nstreams - 1)]
+    big, small = 1 << 23, 1 << 14
+    data = [rng.integers(-1000, 1000, big).astype(np.int32) for _ in range(nstreams)]
+    prefix = [np.concatenate([[0], np.cumsum(d.astype(np.int64))]) for d in data]
+    bufs = [oh.to_device(d, s) for d, s in zip(data, streams)]
+    outs = [oh.DeviceBuffer(8 * reps, s) for s in streams]
+    lengths = [[(big - 17 * r - k) if (r + k) % 3 else (small + 5 * r + k) for r in range(reps)] for k in range(nstreams)]
+    for s in streams:
+        s.synchronize()
+    for r in range(reps):
+        for k in range(nstreams):
+            oh.check(oh.lib.och_reduce_all_device(oh.R["sum"], H.INT32, 1, oh.sizes([lengths[k][r]]), oh.strides([4]), bufs[k].ptr, None, None, 0.0,
+                                                  C.c_void_p(outs[k].address + 8 * r), None, streams[k].handle))
+    for k in range(nstreams):
+        got = outs[k].download(np.int64, reps)
+        want = np.array([prefix[k][lengths[k][r]] for r in range(reps)])
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "stream %d, reduction %d of %d elements: got %d, want %d" % (k, bad[0], lengths[k][bad[0]], got[bad[0]], want[bad[0]])
+    for b in bufs + outs:
+        b.free()
+    for s in streams[1:]:
+        s.synchronize(); s.destroy()
+
+
 ROW_TYPES = [H.BOOL, H.INT8, H.UINT8, H.INT16, H.UINT16, H.HALF, H.INT32, H.FLOAT, H.INT64, H.DOUBLE, H.CHALF, H.CFLOAT]
 
 
