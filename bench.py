@@ -760,6 +760,20 @@ def main():
             configs["extra_gemm_float_%d_NN" % dim] = tflops(2 * dim ** 3, sample_launches(fn, warm=2), MFMA_PEAK["float"])
             for buf in (a, b, c):
                 buf.free()
+            # away from 8192^3: products of one or a few rounds of the compute units, and products with a short K (whose
+            # blocks spend as long on their first loads and on writing C as in their loop)
+            for dt, es, nm, npt in ((F32, 4, "float", np.float32), (F64, 8, "double", np.float64)):
+                cap = 8192 * 8192
+                a, b, c = [oh.DeviceBuffer(es * cap, stream) for _ in range(3)]
+                block = rng.uniform(-1, 1, 1 << 22).astype(npt)
+                for buf in (a, b):
+                    upload_tiled(buf, block, es * cap)
+                one_, zero_ = np.array([1, 0], npt), np.zeros(2, npt)
+                for m_, n_, k_ in ((1024, 1024, 1024), (1536, 1536, 1536), (2048, 2048, 2048), (3000, 3000, 3000), (4096, 4096, 4096), (8192, 8192, 64), (8192, 8192, 256)):
+                    fn = lambda: oh.check(lib.och_gemm(dt, b"N", b"N", m_, n_, k_, one_.ctypes.data, a.ptr, m_, b.ptr, k_, zero_.ctypes.data, c.ptr, m_, 1, h))
+                    configs["extra_gemm_%s_%dx%dx%d_NN" % (nm, m_, n_, k_)] = tflops(2.0 * m_ * n_ * k_, sample_launches(fn, warm=2), MFMA_PEAK[nm])
+                for buf in (a, b, c):
+                    buf.free()
             # half-precision and 8-bit products of the size of the named configurations on the matrix cores
             dim = 8192
             a, b, c = [oh.DeviceBuffer(2 * dim * dim, stream) for _ in range(3)]
