@@ -386,8 +386,15 @@ int och_gemm_batched(int dtype, char transA, char transB, size_t M, size_t N, si
 /* compute units x tile area / efficiency). For tests and measurements the decision can be fixed: 0 the model decides */
 /* (default), 1 the pipelined kernel on its large tile wherever its conditions hold (M, N multiples of 4 or 2, K of   */
 /* the slab, 16-byte aligned operands), 2 the pipelined kernel on its small tile (float, double; complex float has    */
-/* one tile), 3 never the pipelined kernel. Process-wide; no counterpart in the reference.                            */
+/* one tile), 3 never the pipelined kernel, 4 the pipelined kernel on its smallest tile (float: 64 x 64; the other    */
+/* types: the tile the model prefers), 5 as 4 with four slab buffers in a ring instead of two. Process-wide; no       */
+/* counterpart in the reference.                                                                                      */
 int och_gemm_set_kernel_choice(int choice);
+/* Which kernel the model gives an aligned float product of `batch` entries (0 or 1: a single product) with scalars  */
+/* in host memory: 256, 128 or 64 for the pipelined kernel on tiles of that edge, 0 for the tiled kernels. Host      */
+/* arithmetic only (no device is touched; without a device the model assumes 256 compute units). No counterpart in   */
+/* the reference.                                                                                                     */
+int och_gemm_float_plan(size_t M, size_t N, size_t K, unsigned batch);
 /* The pipelined kernels' plan for the last round of the compute units, host arithmetic only (no device is touched):   */
 /* a product of ceil(M / tile_m) x ceil(N / tile_n) block tiles on `units` compute units, K in slabs of `slab`, every   */
 /* element of C elem_size bytes. Returns into how many shares along K each tile of the last round is cut (1: no cut)   */

@@ -568,7 +568,7 @@ static __device__ __forceinline__ void load_to_lds(const char *base, uint32_t of
 
 /* Compute units of the current device (cached per device). */
 int gemm_compute_units(void);
-int gemm_kernel_choice(void);            /* 0 automatic; 1 / 2: pipelined kernel, large / small tile; 3: never pipelined */
+int gemm_kernel_choice(void);            /* 0 automatic; 1 / 2 / 4: pipelined kernel, large / small / smallest tile; 3: never pipelined */
 int gemm_pipe_split_plan(uint64_t M, uint64_t N, uint64_t K, uint64_t batch, bool single, uint32_t tile_m, uint32_t tile_n,
                          uint32_t slab, uint32_t elem_size, uint64_t units, double *rounds);   /* shares of the tiles of the last round */
 int gemm_pad_tail(const GemmArgs &g, size_t Kh, int slab, int es, GemmArgs *tail);   /* the rest of K as one zero-padded slab in the workspace */
@@ -631,7 +631,8 @@ static inline bool gemm_operands_aligned(const GemmArgs &g, int es)
 }
 
 int gemm_float(const GemmArgs &g);
-int gemm_float_pipe(const GemmArgs &g, int tile); /* tiles of 256 x 256 or 128 x 128; 1: not taken */
+int gemm_float_pipe(const GemmArgs &g, int tile); /* tiles of 256 x 256, 128 x 128 or 64 x 64; 1: not taken */
+int gemm_float_plan_query(uint64_t M, uint64_t N, uint64_t K, unsigned batch); /* the tile an aligned product takes; 0: the tiled kernels */
 int gemm_float_pipe_split(const GemmArgs &g, int tile, double *rounds); /* shares of the tiles of the last round; rounds of the compute units */
 int gemm_double(const GemmArgs &g);
 int gemm_double_pipe(const GemmArgs &g, int tile_m); /* tiles of 256 x 128 or 128 x 128; 1: not taken */

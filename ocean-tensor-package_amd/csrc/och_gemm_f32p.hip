@@ -1,10 +1,16 @@
-/* float GEMM on tiles of 256 x 256 or 128 x 128 for aligned operands with M and N multiples of 4 and K of 32: C <- alpha * op(A) * op(B) + beta * C, column-major.
+/* float GEMM on tiles of 256 x 256, 128 x 128 or 64 x 64 for aligned operands with M and N multiples of 4 and K of 32: C <- alpha * op(A) * op(B) + beta * C, column-major.
  *
  * The counterpart of cublasSgemm in the reference (src/core/gpu/op/tensor_blas_gpu.c:183-197). Four waves per block,
  * one per SIMD, each owning 128 x 128 of the tile as 4 x 4 tiles of v_mfma_f32_32x32x2_f32 (256 accumulator registers);
  * for products with fewer than one such tile per compute unit the same kernel with TS = 2: waves of 64 x 64 (2 x 2
- * tiles), two blocks per compute unit (SINGLE: one slab buffer of 34 KB and about a hundred registers, four blocks, for a K of one or two slabs). The
- * description is for TS = 4.
+ * tiles), two blocks per compute unit (SINGLE: one slab buffer of 34 KB and about a hundred registers, four blocks, for a K of one or two slabs);
+ * for products of a few hundred tiles at most, TS = 1: waves of 32 x 32 (one tile, a chunk being two steps of it), 36 KB
+ * of LDS and under 48 registers, up to four blocks per compute unit (1024^3: 69 TFLOP/s against 53 on the 128 x 128 tile,
+ * whose 64 tiles have to be cut along K; 1536^3: 107 against 75). With one block on a compute unit its loads have only
+ * three quads of four MFMAs (770 cycles) to arrive and the block waits for them: it runs at 0.7 of the matrix rate, at 0.9
+ * with a second block beside it. NB = 4 keeps four slab buffers in a ring instead of two, so that a load has three
+ * slabs to arrive; only the knob of the dispatcher reaches it.
+ * The description is for TS = 4.
  * On this device a vector-ALU instruction of a wave takes about eight cycles away from the matrix cores of its SIMD, and
  * a 64-cycle MFMA hides none of that; LDS reads and scalar instructions are nearly free. So the main loop holds MFMAs,
  * LDS reads, scalar instructions and loads that go from memory straight to LDS -- no vector arithmetic, no staging
@@ -106,6 +112,7 @@ struct FloatSlab
    /* KC: the four steps of one tile, 16 bytes; !KC: the TS tiles of one step, 4 TS bytes */
    static __device__ __forceinline__ och_f32x4 read(const char *at)
    {  if (KC || TS == 4) return *reinterpret_cast<const och_f32x4 *>(at);
+      if (TS == 1) return och_f32x4{*reinterpret_cast<const float *>(at), 0.0f, 0.0f, 0.0f};
       const float2 v = *reinterpret_cast<const float2 *>(at);
       return och_f32x4{v.x, v.y, 0.0f, 0.0f};
    }
@@ -115,8 +122,8 @@ struct FloatSlab
    static __device__ __forceinline__ uint32_t row(int i, uint32_t rr) { return KC ? (uint32_t)i * 32 + rr : TS * rr + (uint32_t)i; }
 };
 
-template <bool AKC, bool BKC, int TS, bool SINGLE = false>
-__global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : (SINGLE ? 4 : 2)) void gemm_float_pipe_kernel(const FloatPipeParams p)
+template <bool AKC, bool BKC, int TS, bool SINGLE = false, int NB = 2>
+__global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : (SINGLE || TS == 1 ? 4 : 2)) void gemm_float_pipe_kernel(const FloatPipeParams p)
 {
    constexpr int T = 32, BM = 64 * TS, BN = 64 * TS, KT = OCH_FP_KT, TMS = TS, TNS = TS, WM = 32 * TS, WN = 32 * TS, THREADS = OCH_FP_THREADS;
    typedef FloatSlab<AKC, BM> LA;
@@ -125,7 +132,8 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : (SINGLE ? 4 : 2)) voi
    constexpr int NLA = LA::LOADS, NL = 2 * NLA;            /* loads per wave and slab: of A, of both */
    constexpr int CH = 2 * TS * TS;                         /* chunks of two MFMAs per quad */
    constexpr int RA = LA::READS, NR = LA::READS + LB::READS; /* fragment reads per quad: of A, of both */
-   static_assert(TS == 4 || TS == 2, "wave tiles of 128 x 128 or 64 x 64");
+   static_assert(TS == 4 || TS == 2 || TS == 1, "wave tiles of 128 x 128, 64 x 64 or 32 x 32");
+   static_assert(NB == 2 || (NB == 4 && !SINGLE && BUF + 2 * OP < 65536), "two slab buffers, or a ring of four within reach of the immediates of two read addresses");
    extern __shared__ __align__(16) char lds[];
 
    int64_t oA, oB, oC, oAlpha, oBeta;
@@ -161,7 +169,7 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : (SINGLE ? 4 : 2)) voi
    /* the lane's read addresses in buffer 0 and buffer 1, in registers of their own (the empty asm keeps the compiler
       from deriving the second from the first with an addition at every read: the distance is beyond a read's immediate) */
    const char *readA[2], *readB[2];
-   {  uint32_t a1 = LA::read_lane(wm, lane) + BUF, b1 = OP + LB::read_lane(wn, lane) + BUF;
+   {  uint32_t a1 = LA::read_lane(wm, lane) + (NB / 2) * BUF, b1 = OP + LB::read_lane(wn, lane) + (NB / 2) * BUF;
       asm volatile("" : "+v"(a1), "+v"(b1));
       readA[0] = lds + LA::read_lane(wm, lane); readA[1] = lds + a1;
       readB[0] = lds + OP + LB::read_lane(wn, lane); readB[1] = lds + b1;
@@ -177,32 +185,32 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : (SINGLE ? 4 : 2)) voi
 #define OCH_QUAD(CUR, NXT, RB, QN, LOADS, LOAD0, LBUF)                                                                 \
    do { _Pragma("unroll") for (int c = 0; c < CH; c++)                                                                \
         {  _Pragma("unroll") for (int f = c * NR / CH; f < (c + 1) * NR / CH; f++)                                     \
-           {  if (f < RA) fa[NXT][f < RA ? f : 0] = LA::read(readA[RB] + LA::read_offset(f < RA ? f : 0, QN));         \
-              else        fb[NXT][f >= RA ? f - RA : 0] = LB::read(readB[RB] + LB::read_offset(f >= RA ? f - RA : 0, QN)); \
+           {  if (f < RA) fa[NXT][f < RA ? f : 0] = LA::read(readA[(RB) / (NB / 2)] + ((RB) % (NB / 2)) * BUF + LA::read_offset(f < RA ? f : 0, QN)); \
+              else        fb[NXT][f >= RA ? f - RA : 0] = LB::read(readB[(RB) / (NB / 2)] + ((RB) % (NB / 2)) * BUF + LB::read_offset(f >= RA ? f - RA : 0, QN)); \
            }                                                                                                           \
            if (LOADS && c % TS == TS / 2) OCH_LOAD(LOAD0 + c / TS, nextA, nextB, LBUF);                                \
-           {  const int st = c / (CH / 4), m = (c % (CH / 4)) * 2, i = m / TNS, j = m % TNS;                           \
+           _Pragma("unroll") for (int x = 2 * c; x < 2 * c + 2; x++)                                                   \
+           {  const int st = x / (TMS * TNS), i = x % (TMS * TNS) / TNS, j = x % TNS;                                  \
               acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(LA::value(fa[CUR], i, st), LB::value(fb[CUR], j, st), acc[i][j], 0, 0, 0); \
-              acc[i][j + 1] = __builtin_amdgcn_mfma_f32_32x32x2f32(LA::value(fa[CUR], i, st), LB::value(fb[CUR], j + 1, st), acc[i][j + 1], 0, 0, 0); \
            }                                                                                                           \
            __builtin_amdgcn_sched_barrier(0);                                                                          \
         } } while (0)
    /* slab s in buffer CB: quad 0 carries the second half of the loads of slab s + 1 (into the other buffer), quad 3 the
       first half of the loads of slab s + 2 (into this one) */
 #define OCH_SLAB(s, CB)                                                                                                \
-   do { {  const uint32_t s1 = (slab0 + (s) + 1 < last) ? slab0 + (s) + 1 : last;                                      \
+   do { {  const uint32_t s1 = (slab0 + (s) + (NB - 1) < last) ? slab0 + (s) + (NB - 1) : last;                        \
            const char *nextA = LA::slab_base(pA, p.ldA, m0, s1 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, s1 * KT);  \
-           OCH_QUAD(0, 1, CB, 1, true, NL / 2, 1 - CB);                                                                     \
+           OCH_QUAD(0, 1, CB, 1, true, NL / 2, ((CB) + NB - 1) % NB);                                                  \
         }                                                                                                              \
         {  const char *nextA = nullptr, *nextB = nullptr;                                                              \
            OCH_QUAD(1, 0, CB, 2, false, 0, 0);                                                                         \
            OCH_QUAD(0, 1, CB, 3, false, 0, 0);                                                                         \
         }                                                                                                              \
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                               \
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"((NB - 2) * NL) : "memory");                                         \
         __syncthreads();                                                                                               \
-        {  const uint32_t s2 = (slab0 + (s) + 2 < last) ? slab0 + (s) + 2 : last;                                      \
+        {  const uint32_t s2 = (slab0 + (s) + NB < last) ? slab0 + (s) + NB : last;                                    \
            const char *nextA = LA::slab_base(pA, p.ldA, m0, s2 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, s2 * KT);  \
-           OCH_QUAD(1, 0, 1 - CB, 0, true, 0, CB);                                                                     \
+           OCH_QUAD(1, 0, ((CB) + 1) % NB, 0, true, 0, CB);                                                            \
         } } while (0)
 
    if constexpr (SINGLE)
@@ -229,15 +237,20 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : (SINGLE ? 4 : 2)) voi
    }
    else
    {
-   {  /* slab 0 and the first half of slab 1 */
-      const uint32_t s1 = (slab0 + 1 < last) ? slab0 + 1 : last;
-      const char *nextA = LA::slab_base(pA, p.ldA, m0, slab0 * KT), *nextB = LB::slab_base(pB, p.ldB, n0, slab0 * KT);
+   {  /* slabs 0 .. NB - 2 and the first half of slab NB - 1 */
+      const uint32_t s1 = (slab0 + (NB - 1) < last) ? slab0 + (NB - 1) : last;
+      const char *nextA, *nextB;
 #pragma unroll
-      for (int e = 0; e < NL; e++) OCH_LOAD(e, nextA, nextB, 0);
+      for (int b = 0; b < NB - 1; b++)
+      {  const uint32_t sb = (b == 0 || slab0 + b < last) ? slab0 + b : last;
+         nextA = LA::slab_base(pA, p.ldA, m0, sb * KT); nextB = LB::slab_base(pB, p.ldB, n0, sb * KT);
+#pragma unroll
+         for (int e = 0; e < NL; e++) OCH_LOAD(e, nextA, nextB, b);
+      }
       nextA = LA::slab_base(pA, p.ldA, m0, s1 * KT); nextB = LB::slab_base(pB, p.ldB, n0, s1 * KT);
 #pragma unroll
-      for (int e = 0; e < NL / 2; e++) OCH_LOAD(e, nextA, nextB, 1);
-      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NL / 2) : "memory");
+      for (int e = 0; e < NL / 2; e++) OCH_LOAD(e, nextA, nextB, NB - 1);
+      asm volatile("s_waitcnt vmcnt(%0)" : : "n"((NB - 2) * NL + NL / 2) : "memory");
       __syncthreads();
 #pragma unroll
       for (int x = 0; x < LA::READS; x++) fa[0][x] = LA::read(readA[0] + LA::read_offset(x, 0));
@@ -245,11 +258,24 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : (SINGLE ? 4 : 2)) voi
       for (int x = 0; x < LB::READS; x++) fb[0][x] = LB::read(readB[0] + LB::read_offset(x, 0));
    }
    uint32_t s = 0;
-   for (; s + 1 < nslabs; s += 2)
-   {  OCH_SLAB(s, 0);
-      OCH_SLAB(s + 1, 1);
+   if constexpr (NB == 2)
+   {  for (; s + 1 < nslabs; s += 2)
+      {  OCH_SLAB(s, 0);
+         OCH_SLAB(s + 1, 1);
+      }
+      if (s < nslabs) OCH_SLAB(s, 0);
    }
-   if (s < nslabs) OCH_SLAB(s, 0);
+   else
+   {  for (; s + 3 < nslabs; s += 4)
+      {  OCH_SLAB(s, 0);
+         OCH_SLAB(s + 1, 1);
+         OCH_SLAB(s + 2, 2 % NB);
+         OCH_SLAB(s + 3, 3 % NB);
+      }
+      if (s < nslabs) OCH_SLAB(s, 0);
+      if (s + 1 < nslabs) OCH_SLAB(s + 1, 1);
+      if (s + 2 < nslabs) OCH_SLAB(s + 2, 2 % NB);
+   }
    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
    __syncthreads();
    }
@@ -272,7 +298,7 @@ __global__ __launch_bounds__(OCH_FP_THREADS, TS == 4 ? 1 : (SINGLE ? 4 : 2)) voi
       out = reinterpret_cast<char *>(p.partial + (size_t)cut * BM * BN); ldOut = BM; rowsOut = BM; colsOut = BN;
    }
    constexpr int CP = BM + 4, CPASS = 64, PASSES = BN / CPASS;
-   static_assert(CPASS * CP * 4 <= (SINGLE ? 1 : 2) * BUF, "a pass of the staged tile does not fit into the slab buffers");
+   static_assert(CPASS * CP * 4 <= (SINGLE ? 1 : NB) * BUF, "a pass of the staged tile does not fit into the slab buffers");
    float *stage = reinterpret_cast<float *>(lds);
    for (int h = 0; h < PASSES; h++)
    {
@@ -352,7 +378,9 @@ int gemm_float_pipe(const GemmArgs &g, int tile)
    p.tiles_m = (uint32_t)((g.M + tile - 1) / tile); p.tiles_n = (uint32_t)((g.N + tile - 1) / tile);
    uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
    if (blocks > 0x7FFFFFFFull) return set_error("gemm: too many tiles");
-   if (tile != 256 && tile != 128) return 1;
+   const bool ring = (tile == 65);                       /* the smallest tile on four slab buffers instead of two */
+   if (ring) tile = 64;
+   if (tile != 256 && tile != 128 && tile != 64) return 1;
    const int shares = gemm_float_pipe_split(g, tile, nullptr);
    uint32_t cut_tiles = 0;
    if (shares > 1)
@@ -368,12 +396,12 @@ int gemm_float_pipe(const GemmArgs &g, int tile)
       same order: the same bits. */
    const bool single = tile == 128 && shares == 1 && g.K / OCH_FP_KT <= 2;
    const dim3 grid((unsigned)blocks, 1, g.nz), block(OCH_FP_THREADS);
-#define OCH_FP_LAUNCH(AK, BK, TS, SINGLE)                                                                             \
-   do { auto kernel = gemm_float_pipe_kernel<AK, BK, TS, SINGLE>;                                                     \
-        const size_t lds = ((SINGLE) ? 2 : 4) * (size_t)FloatSlab<AK, 64 * TS>::OPERAND;                              \
+#define OCH_FP_LAUNCH(AK, BK, TS, SINGLE, NB)                                                                         \
+   do { auto kernel = gemm_float_pipe_kernel<AK, BK, TS, SINGLE, NB>;                                                 \
+        const size_t lds = ((SINGLE) ? 2 : 2 * (NB)) * (size_t)FloatSlab<AK, 64 * TS>::OPERAND;                       \
         OCH_CHECK_HIP(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
         hipLaunchKernelGGL(kernel, grid, block, lds, g.stream, p); } while (0)
-#define OCH_FP_PICK(AK, BK) do { if (tile == 256) OCH_FP_LAUNCH(AK, BK, 4, false); else if (single) OCH_FP_LAUNCH(AK, BK, 2, true); else OCH_FP_LAUNCH(AK, BK, 2, false); } while (0)
+#define OCH_FP_PICK(AK, BK) do { if (tile == 256) OCH_FP_LAUNCH(AK, BK, 4, false, 2); else if (tile == 64 && ring) OCH_FP_LAUNCH(AK, BK, 1, false, 4); else if (tile == 64) OCH_FP_LAUNCH(AK, BK, 1, false, 2); else if (single) OCH_FP_LAUNCH(AK, BK, 2, true, 2); else OCH_FP_LAUNCH(AK, BK, 2, false, 2); } while (0)
    if (!akc && !bkc) OCH_FP_PICK(false, false);
    else if (!akc)    OCH_FP_PICK(false, true);
    else if (!bkc)    OCH_FP_PICK(true, false);
@@ -382,7 +410,8 @@ int gemm_float_pipe(const GemmArgs &g, int tile)
 #undef OCH_FP_LAUNCH
    if (shares > 1)
    {  if (tile == 256) hipLaunchKernelGGL(gemm_float_pipe_finish_kernel<4>, dim3(cut_tiles, 8), dim3(256), 0, g.stream, p);
-      else             hipLaunchKernelGGL(gemm_float_pipe_finish_kernel<2>, dim3(cut_tiles, 4), dim3(256), 0, g.stream, p);
+      else if (tile == 128) hipLaunchKernelGGL(gemm_float_pipe_finish_kernel<2>, dim3(cut_tiles, 4), dim3(256), 0, g.stream, p);
+      else             hipLaunchKernelGGL(gemm_float_pipe_finish_kernel<1>, dim3(cut_tiles, 2), dim3(256), 0, g.stream, p);
    }
    OCH_CHECK_LAUNCH();
    return 0;

@@ -216,6 +216,7 @@ PROTOTYPES = {
     "och_elemwise_row_unit": (_i, [C.c_uint, _i, _i, _i, C.c_size_t, C.POINTER(C.c_longlong), C.POINTER(_i), C.POINTER(_i)]),
     "och_elemwise_row_units": (C.c_size_t, [C.c_size_t, _i, _i]),
     "och_gemm_set_kernel_choice": (_i, [_i]),
+    "och_gemm_float_plan": (_i, [C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint]),
     "och_gemm_split_plan": (_i, [C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint, C.c_uint, C.c_uint, C.c_uint, C.c_uint, C.POINTER(C.c_double)]),
 }
 

@@ -209,14 +209,40 @@ def test_kernel_choice():
 
 
 def test_gemm_kernel_choice_knob_checks_its_argument():
-    """och_gemm_set_kernel_choice touches no device: 0 to 3 are accepted, anything else is refused with a message."""
+    """och_gemm_set_kernel_choice touches no device: 0 to 5 are accepted, anything else is refused with a message."""
     import ocean_hip as oh
-    for choice in (1, 2, 3, 0):
+    for choice in (1, 2, 3, 4, 5, 0):
         assert oh.lib.och_gemm_set_kernel_choice(choice) == 0
-    for choice in (-1, 4, 99):
+    for choice in (-1, 6, 99):
         assert oh.lib.och_gemm_set_kernel_choice(choice) != 0
         assert b"kernel choice" in oh.lib.och_last_error()
     assert oh.lib.och_gemm_set_kernel_choice(0) == 0
+
+
+def test_float_products_and_the_tile_the_model_gives_them():
+    """och_gemm_float_plan is host arithmetic on 256 compute units when there is no device. The expectations are the
+    winners of measurements on an MI355X (TFLOP/s, NN products; tiled kernels / 128 x 128 / 64 x 64 tiles):
+    512^3 10 / 7 / 16, 768^3 26 / 17 / 41, 1024^3 49 / 53 / 69, 1536^3 65 / 75 / 107, 1792^3 71 / 104 / 98,
+    2048^3 91 / 136 / 125, 1024 x 2048 x 1024 65 / 92 / 102, 1024 x 1024 x 4096 63 / 104 / 97."""
+    import ocean_hip as oh
+    plan = oh.lib.och_gemm_float_plan
+    assert oh.lib.och_gemm_set_kernel_choice(0) == 0
+    for m, n, k, tile in [(512, 512, 512, 64), (768, 768, 768, 64), (1024, 1024, 1024, 64), (1536, 1536, 1536, 64),
+                          (1024, 2048, 1024, 64), (1792, 1792, 1792, 128), (2048, 2048, 2048, 128), (1024, 1024, 4096, 128),
+                          (4096, 4096, 4096, 256), (8192, 8192, 8192, 256), (8192, 8192, 64, 128)]:
+        assert plan(m, n, k, 1) == tile, (m, n, k)
+    # what the pipelined kernel does not take: M or N below 128 or not a multiple of 4, K below a slab
+    for m, n, k in [(64, 4096, 4096), (4096, 126, 4096), (1026, 1024, 1024), (1024, 1024, 16)]:
+        assert plan(m, n, k, 1) == 0, (m, n, k)
+    # a batch of small products counts its tiles over all entries
+    assert plan(256, 256, 256, 100) in (64, 128)
+    # the knob overrides the model
+    for choice, tile in [(1, 256), (2, 128), (3, 0), (4, 64)]:
+        assert oh.lib.och_gemm_set_kernel_choice(choice) == 0
+        try:
+            assert plan(1024, 1024, 1024, 1) == tile
+        finally:
+            assert oh.lib.och_gemm_set_kernel_choice(0) == 0
 
 
 def test_cutting_the_last_round_of_a_product_along_k():
