@@ -17,6 +17,22 @@
 
 namespace och {
 
+/* The conversions of the epilogue. The library's general device conversions (och_dtypes.h) keep their rare cases behind
+   wave-uniform branches, which pays in a streaming kernel; unrolled over the 256 accumulators of a wave here they cost the
+   kernel its registers (a kilobyte and more of scratch per lane, and the 8192^3 product 21 ms instead of 1). So: the
+   integer routine for float -> half, and the hardware converter for finite halves with the integer routine for the rest. */
+static __device__ __forceinline__ float gemm_half_to_float(half_t hh)
+{
+   uint32_t h = hh.v;
+   uint32_t s = (h & 0x8000u) << 16;
+   h &= 0x7FFFu;
+   if (h == 0) return 0.f;                       /* both zeros map to +0 */
+   uint32_t e = h & 0x7C00u;
+   if (e != 0x7C00u) { _Float16 x; __builtin_memcpy(&x, &hh.v, 2); return (float)x; }      /* exact, subnormals included */
+   return bits_to_float((h << 13) | 0x7F800000u | s);                                       /* Inf, NaN with its payload */
+}
+static __device__ __forceinline__ half_t gemm_float_to_half(float f) { return float_to_half_soft(f); }
+
 typedef _Float16 och_h8 __attribute__((ext_vector_type(8)));
 typedef short och_i16x4 __attribute__((ext_vector_type(4)));
 
@@ -330,7 +346,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
    half_t al = p.alpha, be = p.beta;
    if (p.alpha_dev) al = *reinterpret_cast<const half_t *>(reinterpret_cast<const char *>(p.alpha_dev) + oAlpha);
    if (p.beta_dev)  be = *reinterpret_cast<const half_t *>(reinterpret_cast<const char *>(p.beta_dev) + oBeta);
-   const float alpha = half_to_float(al), beta = half_to_float(be);
+   const float alpha = gemm_half_to_float(al), beta = gemm_half_to_float(be);
    /* this lane's part of tile (i, j): rows row0 + row_step(32 i + 8 (r / 4) + r % 4), column col0 + row_step(32 j); the
       slot offsets added here never carry out of a group of BM / 8 (BN / 8) slots, so the steps are compile-time numbers */
    if (beta == 0)
@@ -349,7 +365,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
             for (int i = 0; i < TMS; i++)
 #pragma unroll
                for (int r = 0; r < 16; r++)
-                  mine[LB::row_step(j * T) * CP + LA::row_step(i * T + 8 * (r >> 2) + (r & 3))] = float_to_half(alpha * acc[i][j][r]).v;
+                  mine[LB::row_step(j * T) * CP + LA::row_step(i * T + 8 * (r >> 2) + (r & 3))] = gemm_float_to_half(alpha * acc[i][j][r]).v;
          }
          __syncthreads();
          const uint32_t c0 = n0 + h * CPASS;
@@ -382,7 +398,7 @@ __global__ __launch_bounds__(64 * NWM * NWN) void gemm_half_kernel(const HalfGem
             const uint32_t dr = LA::row_step(i * T + 8 * (r >> 2) + (r & 3));
             if (EDGE && m0 + row0 + dr >= p.M) continue;
             half_t *c = reinterpret_cast<half_t *>(mine + ((int64_t)dr + (int64_t)LB::row_step(j * T) * p.ldC) * 2);
-            *c = float_to_half(alpha * acc[i][j][r] + beta * half_to_float(*c));
+            *c = gemm_float_to_half(alpha * acc[i][j][r] + beta * gemm_half_to_float(*c));
          }
    }
 }
@@ -403,11 +419,11 @@ __global__ __launch_bounds__(256) void gemm_half_finish_kernel(const HalfGemmPar
       for (int u = 0; u < 8; u++) s += v[u];
    }
    for (; t < slices; t++) s += p.partial[(size_t)t * mn + e];
-   const float alpha = half_to_float(p.alpha_dev ? *p.alpha_dev : p.alpha), beta = half_to_float(p.beta_dev ? *p.beta_dev : p.beta);
+   const float alpha = gemm_half_to_float(p.alpha_dev ? *p.alpha_dev : p.alpha), beta = gemm_half_to_float(p.beta_dev ? *p.beta_dev : p.beta);
    half_t *c = reinterpret_cast<half_t *>(p.C) + ((int64_t)row + (int64_t)col * p.ldC);
    float v = alpha * s;
-   if (beta != 0) v += beta * half_to_float(*c);
-   *c = float_to_half(v);
+   if (beta != 0) v += beta * gemm_half_to_float(*c);
+   *c = gemm_float_to_half(v);
 }
 
 template <int WM, int WN, int NWM, int NWN, int KT, bool PIPE = false>

@@ -223,14 +223,15 @@ def check_large_product(stream, dtype, ta, tb, M, N, cases, rng, pad=0):
             assert np.linalg.norm(have - want) <= TOL[dtype] * np.linalg.norm(bound), what + " (probe vectors)"
 
 
-@pytest.mark.parametrize("choice", [1, 2, 3], ids=["large_tile", "small_tile", "tiled_kernel"])
+@pytest.mark.parametrize("choice", [1, 2, 3, 4], ids=["large_tile", "small_tile", "tiled_kernel", "smallest_tile"])
 @pytest.mark.parametrize("dtype", [H.FLOAT, H.DOUBLE, H.CFLOAT, H.CDOUBLE], ids=lambda d: H.NAMES[d])
 def test_gemm_pipelined_kernels_against_the_oracle(hip, stream, dtype, choice):
     """With the kernel choice fixed (och_gemm_set_kernel_choice) the pipelined kernels take every aligned product whose M and
     N are multiples of 4 (double, complex float: 2), however small: whole results against the oracle for single tiles, last
     tiles of a few rows and columns, one to nine slabs of K, a K with a remainder (host scalars: pipelined head + additive
     rest; device scalars: the tiled kernel), every transposition and conjugation. Choice 3 is the tiled kernel on the same
-    shapes."""
+    shapes; choice 4 the 64 x 64 tiles of the float kernel (the other types have no such tile and take the one their model
+    prefers)."""
     rng = np.random.default_rng(1600 + 10 * dtype + choice)
     slab = 16 if dtype in (H.DOUBLE, H.CDOUBLE) else 32
     cplx = dtype in (H.CFLOAT, H.CDOUBLE)
@@ -249,8 +250,8 @@ def test_gemm_pipelined_kernels_against_the_oracle(hip, stream, dtype, choice):
         oh.check(oh.lib.och_gemm_set_kernel_choice(0))
 
 
-@pytest.mark.parametrize("choice,M,N", [(2, 2176, 2048), (2, 2180, 2052), (1, 4352, 4096), (2, 2560, 2048)],
-                         ids=["small_tiles", "small_tiles_ragged", "large_tiles", "small_tiles_quarter_round"])
+@pytest.mark.parametrize("choice,M,N", [(2, 2176, 2048), (2, 2180, 2052), (1, 4352, 4096), (2, 2560, 2048), (4, 1088, 1024), (4, 1092, 1028)],
+                         ids=["small_tiles", "small_tiles_ragged", "large_tiles", "small_tiles_quarter_round", "smallest_tiles", "smallest_tiles_ragged"])
 def test_gemm_float_last_round_cut_along_k(hip, stream, choice, M, N):
     """When the last round of the compute units is at most half full (here 16 tiles, or 17 x 17 - 256 = 33, on 256 units) its
     tiles are cut along K into shares of at least 8 slabs that fill the round; the shares are added in order by a second
@@ -565,7 +566,7 @@ PIPELINED_BATCH_CASES = [  # as above; aligned operands, sizes the pipelined ker
 ]
 
 
-@pytest.mark.parametrize("choice", [1, 2], ids=["large_tile", "small_tile"])
+@pytest.mark.parametrize("choice", [1, 2, 4], ids=["large_tile", "small_tile", "smallest_tile"])
 @pytest.mark.parametrize("case", PIPELINED_BATCH_CASES, ids=lambda c: "%s-%s%s-%dx%dx%d-b%s" % (H.NAMES[c[0]], c[1], c[2], c[3], c[4], c[5], "x".join(map(str, c[6]))))
 def test_gemm_batched_on_the_pipelined_kernels(hip, stream, case, choice):
     """The batch in grid z of the pipelined kernels (operand, scalar and result offsets per product; ragged last tiles):
