@@ -419,6 +419,74 @@ def test_m0_is_used_by_the_loads_to_lds_only(source):
         assert any(c.startswith("global_load_lds_dwordx4") for c in code[i + 1:i + 3]), code[i:i + 3]
 
 
+def library_kernel_metadata():
+    """(kernel name, scratch bytes per lane, vector registers) of every gfx950 kernel in csrc/libocean_hip.so, read from the
+    notes of the code objects it carries: the .hip_fatbin section is a row of clang offload bundles (magic, entry count,
+    then per entry offset, size and target triple), each holding one translation unit's code object."""
+    import shutil
+    import struct
+    import subprocess
+    import tempfile
+    tools = "/opt/rocm/llvm/bin"
+    objcopy, readelf = os.path.join(tools, "llvm-objcopy"), os.path.join(tools, "llvm-readelf")
+    if not (os.path.exists(objcopy) and os.path.exists(readelf)):
+        pytest.skip("the LLVM binary tools of ROCm are not available")
+    magic = b"__CLANG_OFFLOAD_BUNDLE__"
+    kernels = []
+    with tempfile.TemporaryDirectory() as tmp:
+        fat = os.path.join(tmp, "fat.bin")
+        subprocess.run([objcopy, "-O", "binary", "--only-section=.hip_fatbin", oh.LIB_PATH, fat], check=True, capture_output=True)
+        blob = open(fat, "rb").read()
+        at = blob.find(magic)
+        while at >= 0:
+            (entries,) = struct.unpack_from("<Q", blob, at + len(magic))
+            pos = at + len(magic) + 8
+            for _ in range(entries):
+                offset, size, tlen = struct.unpack_from("<QQQ", blob, pos)
+                triple = blob[pos + 24:pos + 24 + tlen].decode()
+                pos += 24 + tlen
+                if "gfx950" not in triple or size == 0:
+                    continue
+                co = os.path.join(tmp, "k.co")
+                with open(co, "wb") as out:
+                    out.write(blob[at + offset:at + offset + size])
+                notes = subprocess.run([readelf, "--notes", co], check=True, capture_output=True, text=True).stdout
+                name = scratch = vgprs = None
+                for line in notes.splitlines():
+                    line = line.strip()
+                    if line.startswith(".name:"):
+                        name = line.split(":", 1)[1].strip()
+                    elif line.startswith(".private_segment_fixed_size:"):
+                        scratch = int(line.split(":")[1])
+                    elif line.startswith(".vgpr_count:"):
+                        vgprs = int(line.split(":")[1])
+                    elif line.startswith(".wavefront_size:") and name is not None and scratch is not None:
+                        kernels.append((name, scratch, vgprs))
+                        name = scratch = vgprs = None
+            at = blob.find(magic, at + len(magic))
+    return kernels
+
+
+def test_no_kernel_of_the_library_lives_in_scratch_memory():
+    """A change far from a kernel (a conversion routine in a shared header, say) can cost a kernel with hundreds of live
+    accumulators its registers without any test of results noticing: the half GEMM once went from 1100 to 50 TFLOP/s that
+    way, with a kilobyte and more of scratch per lane. So the scratch every kernel of the built library asks for is held
+    to what it is known to need: nothing for the float, double and complex pipelined GEMM kernels beyond a few spilled
+    registers, at most 128 bytes per lane for the 8-bit kernels and the half kernels of whole tiles, 320 for the half
+    kernels of ragged ones, 768 for anything else."""
+    kernels = library_kernel_metadata()
+    assert len(kernels) > 5000
+    limits = [("gemm_float_pipe_kernel", 32), ("gemm_double_pipe", 32), ("gemm_cfloat_pipe", 64), ("gemm_cdouble_pipe", 64),
+              ("Li128ELi128ELi2ELi2ELi64E", 128),          # the half kernels of whole 256 x 256 tiles: waves of 128 x 128
+              ("gemm_half_kernel", 320), ("gemm_byte_kernel", 128), ("", 768)]
+    seen = set()
+    for name, scratch, _ in kernels:
+        prefix, limit = next((p, l) for p, l in limits if p in name)
+        seen.add(prefix)
+        assert scratch <= limit, "%s: %d bytes of scratch per lane (limit %d)" % (name, scratch, limit)
+    assert seen == {p for p, _ in limits}
+
+
 def test_microbenchmarks_live_in_their_own_library():
     """The product header declares no measurement tool; the two micro-benchmarks are declared in include/ocean_hip_bench.h and
     exported by csrc/libocean_hip_bench.so only."""
