@@ -13,6 +13,7 @@
  */
 #pragma once
 #include "och_dtypes.h"
+#include "och_math.h"
 #include <math.h>
 
 namespace och {
@@ -230,8 +231,8 @@ template <class T> struct BinPower
          return z;
       }
       else if constexpr (std::is_same<T, double>::value)
-         return (double)powf((float)x, (float)y);   /* the CPU path evaluates double pow in single precision */
-      else if constexpr (is_float_v<T>) return from_work<T>(powf(to_work(x), to_work(y)));
+         return (double)och_powf((float)x, (float)y);   /* the CPU path evaluates double pow in single precision */
+      else if constexpr (is_float_v<T>) return from_work<T>(och_powf(to_work(x), to_work(y)));
       else
       {  typedef typename traits<T>::elem E; typedef elemwork_t<T> W; R z;
          W xr = to_work(x.real), xi = to_work(x.imag), yr = to_work(y.real), yi = to_work(y.imag);

@@ -13,6 +13,7 @@
  */
 #pragma once
 #include "och_dtypes.h"
+#include "och_math.h"
 #include <math.h>
 
 namespace och {
@@ -21,7 +22,7 @@ namespace och {
 #define OCH_MATH1(NAME, FN, DN) \
    template <class W> OCH_D W NAME(W x) { if constexpr (std::is_same<W, float>::value) return FN(x); else return DN(x); }
 OCH_MATH1(m_sin, sinf, sin)       OCH_MATH1(m_cos, cosf, cos)       OCH_MATH1(m_tan, tanf, tan)
-OCH_MATH1(m_sinh, sinhf, sinh)    OCH_MATH1(m_cosh, coshf, cosh)    OCH_MATH1(m_tanh, tanhf, tanh)
+OCH_MATH1(m_sinh, sinhf, sinh)    OCH_MATH1(m_cosh, coshf, cosh)    OCH_MATH1(m_tanh, tanhf, och_tanh)   /* double: och_math.h */
 OCH_MATH1(m_asin, asinf, asin)    OCH_MATH1(m_acos, acosf, acos)    OCH_MATH1(m_atan, atanf, atan)
 OCH_MATH1(m_asinh, asinhf, asinh) OCH_MATH1(m_acosh, acoshf, acosh) OCH_MATH1(m_atanh, atanhf, atanh)
 OCH_MATH1(m_sqrt, sqrtf, sqrt)    OCH_MATH1(m_cbrt, cbrtf, cbrt)
@@ -34,8 +35,8 @@ OCH_MATH1(m_trunc, truncf, trunc) OCH_MATH1(m_round, roundf, round)
 template <class W> OCH_D W m_atan2(W y, W x) { if constexpr (std::is_same<W, float>::value) return atan2f(y, x); else return atan2(y, x); }
 template <class W> OCH_D W m_hypot(W x, W y) { if constexpr (std::is_same<W, float>::value) return hypotf(x, y); else return hypot(x, y); }
 template <class W> OCH_D W m_copysign(W x, W y) { if constexpr (std::is_same<W, float>::value) return copysignf(x, y); else return copysign(x, y); }
-/* pow in the CPU table: powf for BOTH float and double */
-template <class W> OCH_D W m_pow(W x, W y) { return (W)powf((float)x, (float)y); }
+/* pow in the CPU table: powf for BOTH float and double (och_math.h: the correctly rounded power in all but one case in 10^5) */
+template <class W> OCH_D W m_pow(W x, W y) { return (W)och_powf((float)x, (float)y); }
 /* exp10(x) is evaluated as exp(ln10 * x) */
 template <class W> OCH_D W m_exp10(W x)
 {  if constexpr (std::is_same<W, float>::value) return expf(((float)2.3025850929940459) * x);
