@@ -245,12 +245,14 @@ template <class T> struct BinPower
          if constexpr (std::is_same<W, float>::value)
          {  zi = atan2f(xi, xr); zr = (W)(logf(scale) * 0.5);
             xr = yr * zr - yi * zi; xi = yr * zi + yi * zr;
-            scale = expf(xr); xr = scale * cosf(xi); xi = scale * sinf(xi);
+            W sn, cs; sincosf(xi, &sn, &cs);          /* one argument reduction for both */
+            scale = expf(xr); xr = scale * cs; xi = scale * sn;
          }
          else
          {  zi = atan2(xi, xr); zr = log(scale) * 0.5;
             xr = yr * zr - yi * zi; xi = yr * zi + yi * zr;
-            scale = exp(xr); xr = scale * cos(xi); xi = scale * sin(xi);
+            W sn, cs; sincos(xi, &sn, &cs);
+            scale = exp(xr); xr = scale * cs; xi = scale * sn;
          }
          z.real = from_work<E>(xr); z.imag = from_work<E>(xi);
          return z;

@@ -32,6 +32,8 @@ OCH_MATH1(m_log1p, log1pf, log1p)
 OCH_MATH1(m_fabs, fabsf, fabs)    OCH_MATH1(m_ceil, ceilf, ceil)    OCH_MATH1(m_floor, floorf, floor)
 OCH_MATH1(m_trunc, truncf, trunc) OCH_MATH1(m_round, roundf, round)
 #undef OCH_MATH1
+/* sine and cosine of one argument share their argument reduction */
+template <class W> OCH_D void m_sincos(W x, W &s, W &c) { if constexpr (std::is_same<W, float>::value) sincosf(x, &s, &c); else sincos(x, &s, &c); }
 template <class W> OCH_D W m_atan2(W y, W x) { if constexpr (std::is_same<W, float>::value) return atan2f(y, x); else return atan2(y, x); }
 template <class W> OCH_D W m_hypot(W x, W y) { if constexpr (std::is_same<W, float>::value) return hypotf(x, y); else return hypot(x, y); }
 template <class W> OCH_D W m_copysign(W x, W y) { if constexpr (std::is_same<W, float>::value) return copysignf(x, y); else return copysign(x, y); }
@@ -187,19 +189,20 @@ template <class T, int ID> struct UnaryOp
             else if constexpr (ID == U_CONJ) { y.real = x.real; y.imag = from_work<E>((W)-1 * xi); return y; }
             else if constexpr (ID == U_RECIPROCAL)
             {  W scale = (W)1 / ((xr * xr) + (xi * xi)); yr = xr * scale; yi = xi * scale * (W)-1; }
-            else if constexpr (ID == U_SIN)  { yr = m_sin(xr) * m_cosh(xi);  yi = m_cos(xr) * m_sinh(xi); }
-            else if constexpr (ID == U_COS)  { yr = m_cos(xr) * m_cosh(xi);  yi = m_sin(xr) * m_sinh(xi) * (W)-1; }
+            else if constexpr (ID == U_SIN)  { W sn, cs; m_sincos(xr, sn, cs); yr = sn * m_cosh(xi);  yi = cs * m_sinh(xi); }
+            else if constexpr (ID == U_COS)  { W sn, cs; m_sincos(xr, sn, cs); yr = cs * m_cosh(xi);  yi = sn * m_sinh(xi) * (W)-1; }
             else if constexpr (ID == U_TAN)
-            {  W a = 2 * xr, b = 2 * xi, r = m_cos(a) + m_cosh(b); yr = m_sin(a) / r; yi = m_sinh(b) / r; }
-            else if constexpr (ID == U_SINH) { yr = m_sinh(xr) * m_cos(xi);  yi = m_cosh(xr) * m_sin(xi); }
-            else if constexpr (ID == U_COSH) { yr = m_cosh(xr) * m_cos(xi);  yi = m_sinh(xr) * m_sin(xi); }
+            {  W a = 2 * xr, b = 2 * xi, sn, cs; m_sincos(a, sn, cs); W r = cs + m_cosh(b); yr = sn / r; yi = m_sinh(b) / r; }
+            else if constexpr (ID == U_SINH) { W sn, cs; m_sincos(xi, sn, cs); yr = m_sinh(xr) * cs;  yi = m_cosh(xr) * sn; }
+            else if constexpr (ID == U_COSH) { W sn, cs; m_sincos(xi, sn, cs); yr = m_cosh(xr) * cs;  yi = m_sinh(xr) * sn; }
             else if constexpr (ID == U_TANH)
-            {  W a = 2 * xr, b = 2 * xi, r = (W)1 / (m_cosh(a) + m_cos(b)); yr = m_sinh(a) * r; yi = m_sin(b) * r; }
+            {  W a = 2 * xr, b = 2 * xi, sn, cs; m_sincos(b, sn, cs); W r = (W)1 / (m_cosh(a) + cs); yr = m_sinh(a) * r; yi = sn * r; }
             else if constexpr (ID == U_ARCSIN || ID == U_ARCCOS)
             {  W v1 = 1 - (xr * xr) + (xi * xi), v2 = -2 * xr * xi;
-               W gamma = m_sqrt(m_hypot(v1, v2)), theta = m_atan2(v2, v1) / 2;
-               if constexpr (ID == U_ARCSIN) { v1 = -xi + gamma * m_cos(theta); v2 = xr + gamma * m_sin(theta); }
-               else                          { v1 = xr - gamma * m_sin(theta); v2 = xi + gamma * m_cos(theta); }
+               W gamma = m_sqrt(m_hypot(v1, v2)), theta = m_atan2(v2, v1) / 2, sn, cs;
+               m_sincos(theta, sn, cs);
+               if constexpr (ID == U_ARCSIN) { v1 = -xi + gamma * cs; v2 = xr + gamma * sn; }
+               else                          { v1 = xr - gamma * sn; v2 = xi + gamma * cs; }
                yr = m_atan2(v2, v1); yi = m_log(v1 * v1 + v2 * v2) / -2;
             }
             else if constexpr (ID == U_ARCTAN)
@@ -212,8 +215,9 @@ template <class T, int ID> struct UnaryOp
             {  W v1, v2;
                if constexpr (ID == U_ARCSINH) v1 = 1 + (xr * xr) - (xi * xi); else v1 = (xr * xr) - (xi * xi) - 1;
                v2 = 2 * xr * xi;
-               W gamma = m_sqrt(m_hypot(v1, v2)), theta = m_atan2(v2, v1) / 2;
-               v1 = xr + gamma * m_cos(theta); v2 = xi + gamma * m_sin(theta);
+               W gamma = m_sqrt(m_hypot(v1, v2)), theta = m_atan2(v2, v1) / 2, sn, cs;
+               m_sincos(theta, sn, cs);
+               v1 = xr + gamma * cs; v2 = xi + gamma * sn;
                yr = m_log(v1 * v1 + v2 * v2) / 2; yi = m_atan2(v2, v1);
             }
             else if constexpr (ID == U_ARCTANH)
@@ -240,16 +244,17 @@ template <class T, int ID> struct UnaryOp
             else if constexpr (ID == U_CBRT)
             {  W scale = (xr * xr) + (xi * xi);
                if (scale > 0)
-               {  scale = m_pow(scale, (W)(1. / 6)); W angle = m_atan2(xi, xr) / 3;
-                  yr = scale * m_cos(angle); yi = scale * m_sin(angle);
+               {  scale = m_pow(scale, (W)(1. / 6)); W angle = m_atan2(xi, xr) / 3, sn, cs;
+                  m_sincos(angle, sn, cs);
+                  yr = scale * cs; yi = scale * sn;
                }
                else { y.real = ezero; y.imag = ezero; return y; }
             }
             else if constexpr (ID == U_SQUARE) { yr = xr * xr - xi * xi; yi = 2 * xr * xi; }
-            else if constexpr (ID == U_EXP)   { W s = m_exp(xr); yr = s * m_cos(xi); yi = s * m_sin(xi); }
-            else if constexpr (ID == U_EXP2)  { W b = xi * c_ln2<W>();  W s = m_exp2(xr);  yr = s * m_cos(b); yi = s * m_sin(b); }
-            else if constexpr (ID == U_EXP10) { W b = xi * c_ln10<W>(); W s = m_exp10(xr); yr = s * m_cos(b); yi = s * m_sin(b); }
-            else if constexpr (ID == U_EXPM1) { W s = m_exp(xr); yr = s * m_cos(xi) - 1; yi = s * m_sin(xi); }
+            else if constexpr (ID == U_EXP)   { W s = m_exp(xr), sn, cs; m_sincos(xi, sn, cs); yr = s * cs; yi = s * sn; }
+            else if constexpr (ID == U_EXP2)  { W b = xi * c_ln2<W>();  W s = m_exp2(xr), sn, cs;  m_sincos(b, sn, cs); yr = s * cs; yi = s * sn; }
+            else if constexpr (ID == U_EXP10) { W b = xi * c_ln10<W>(); W s = m_exp10(xr), sn, cs; m_sincos(b, sn, cs); yr = s * cs; yi = s * sn; }
+            else if constexpr (ID == U_EXPM1) { W s = m_exp(xr), sn, cs; m_sincos(xi, sn, cs); yr = s * cs - 1; yi = s * sn; }
             else if constexpr (ID == U_LOG)   { W s = xr * xr + xi * xi; yr = m_log(s) * (W)0.5;   yi = m_atan2(xi, xr); }
             else if constexpr (ID == U_LOG2)  { W s = xr * xr + xi * xi; yr = m_log2(s) * (W)0.5;  yi = m_atan2(xi, xr) / c_ln2<W>(); }
             else if constexpr (ID == U_LOG10) { W s = xr * xr + xi * xi; yr = m_log10(s) * (W)0.5; yi = m_atan2(xi, xr) / c_ln10<W>(); }
