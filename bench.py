@@ -228,6 +228,16 @@ def main():
                   lambda a_, b_: torch._int_mm(a_, b_), 5000.0)
         gemm_line("int8 NT (torch._int_mm)", lambda c: torch.ones(dim, dim, device=dev, dtype=torch.int8) if c else torch.randint(-128, 128, (dim, dim), device=dev, dtype=torch.int8),
                   lambda a_, b_: torch._int_mm(a_, b_.t()), 5000.0)
+        # the same library away from 8192^3, at the sizes of the extra_gemm_<type>_MxNxK lines of the default run
+        print("== vendor GEMM through PyTorch at the sizes of the extra_gemm_ lines (NN, random operands, TFLOP/s median, microseconds)")
+        for tdt, tname in ((torch.float32, "float32"), (torch.float64, "float64"), (torch.float16, "float16")):
+            for m_, n_, k_ in ((1024, 1024, 1024), (1536, 1536, 1536), (2048, 2048, 2048), (3000, 3000, 3000), (4096, 4096, 4096), (8192, 8192, 64), (8192, 8192, 256)):
+                ta_ = (torch.rand(m_, k_, device=dev) * 2 - 1).to(tdt)
+                tb_ = (torch.rand(k_, n_, device=dev) * 2 - 1).to(tdt)
+                tc_ = torch.empty(m_, n_, device=dev, dtype=tdt)
+                med, best = torch_time(lambda: torch.matmul(ta_, tb_, out=tc_))
+                print("   %8.1f  %8.1f us   %s %5d x %5d x %5d" % (2.0 * m_ * n_ * k_ / med / 1e9, med * 1e3, tname, m_, n_, k_))
+                del ta_, tb_, tc_
         return
 
     def sample_launches(fn, samples=None, warm=3, target_ms=0.6):
