@@ -46,7 +46,7 @@ static int gemm_float_plan(const GemmArgs &g, int *pick)
    if (!((tile == 256 ? large : small) < others)) tile = 0;
    const uint64_t tiles64 = ((g.M + 63) / 64) * ((g.N + 63) / 64) * (uint64_t)g.nz;
    if (tiles64 <= 4 * units)
-   {  if (tile == 0) return 64;
+   {  if (tile == 0) return slabs <= 256 ? 64 : 0;      /* (measured up to K = 4096; a longer K stays where it was) */
       if (slabs <= 2) return tile;          /* the small tile has a kernel of its own for a K of one or two slabs */
       /* microseconds of a launch: `slab_us` per slab and block, the whole rounds, then the last round, cut or not */
       auto micros = [&](uint64_t edge, int shares, double fixed, double slab_us, double cut_us)
