@@ -473,12 +473,14 @@ def test_no_kernel_of_the_library_lives_in_scratch_memory():
     way, with a kilobyte and more of scratch per lane. So the scratch every kernel of the built library asks for is held
     to what it is known to need: nothing for the float, double and complex pipelined GEMM kernels beyond a few spilled
     registers, at most 128 bytes per lane for the 8-bit kernels and the half kernels of whole tiles, 320 for the half
-    kernels of ragged ones, 768 for anything else."""
+    kernels of ragged ones, 768 for the fused projection, 32 for the per-thread axis reduction, none for anything
+    else (every elementwise, copy, fill, index and other reduction kernel)."""
     kernels = library_kernel_metadata()
     assert len(kernels) > 5000
     limits = [("gemm_float_pipe_kernel", 32), ("gemm_double_pipe", 32), ("gemm_cfloat_pipe", 64), ("gemm_cdouble_pipe", 64),
               ("Li128ELi128ELi2ELi2ELi64E", 128),          # the half kernels of whole 256 x 256 tiles: waves of 128 x 128
-              ("gemm_half_kernel", 320), ("gemm_byte_kernel", 128), ("", 768)]
+              ("gemm_half_kernel", 320), ("gemm_byte_kernel", 128), ("mgs_project_kernel", 768), ("axis_thread_kernel", 32),
+              ("", 0)]                                        # every elementwise, copy, fill, index and other reduction kernel: none
     seen = set()
     for name, scratch, _ in kernels:
         prefix, limit = next((p, l) for p, l in limits if p in name)
