@@ -1,0 +1,77 @@
+/* Host walk through the LDS layout of the pipelined float GEMM (csrc/och_gemm_f32p_slab.h), for
+   tests/test_gemm_layout_cpu.py. For every operand layout (contiguous along k or along the rows) and every block tile
+   (256, 128, 64 rows) a slab of a synthetic matrix is brought into an LDS image by exactly the offsets the kernel's load
+   instructions use (4 waves x LOADS instructions x 64 lanes x 16 bytes), and every value an MFMA would get -- tile i of a
+   wave, step t of quad q, lane l -- is compared with the matrix element it has to be: row wbase + row(i, l % 32),
+   k = 8 q + 4 (l / 32) + t. Also checked: loads stay inside the slab of the rows that exist, no two loads write the same
+   LDS bytes, everything lies inside the operand's LDS area. Returns the number of violations. */
+#include <stdint.h>
+#include <string.h>
+#include <stdio.h>
+#include <vector>
+#include "och_gemm_f32p_slab.h"
+
+using namespace och;
+
+template <bool KC, int ROWS>
+static long check(uint32_t rows /* rows of the tile that exist: a multiple of 4 */, int64_t ld, int verbose)
+{
+   typedef FloatSlab<KC, ROWS> L;
+   constexpr int KT = 32, TS = L::TS;
+   long bad = 0;
+   /* the matrix around the slab: element (row r, k) = 1000 r + k + 1, stored as the kernel's operand layout says */
+   const int64_t nrow = ROWS, nk = KT;
+   std::vector<float> mat((size_t)(KC ? nrow * ld : nk * ld), -1.0f);
+   auto element = [&](int64_t r, int64_t k) -> float & { return mat[(size_t)(KC ? r * ld + k : k * ld + r)]; };
+   for (int64_t r = 0; r < (int64_t)rows; r++) for (int64_t k = 0; k < nk; k++) element(r, k) = (float)(1000 * r + k + 1);
+   const char *base = L::slab_base(reinterpret_cast<const char *>(mat.data()), ld, 0, 0);
+   std::vector<char> lds(L::OPERAND, 0);
+   std::vector<unsigned char> written(L::OPERAND, 0);
+   for (uint32_t wave = 0; wave < 4; wave++)
+      for (int j = 0; j < L::LOADS; j++)
+         for (uint32_t lane = 0; lane < 64; lane++)
+         {  const uint32_t off = L::load_offset(j, wave, lane, ld, rows), tgt = L::load_target(j, wave) + 16 * lane;
+            if (tgt % 16 != 0 || tgt + 16 > (uint32_t)L::OPERAND) { bad++; continue; }
+            if ((size_t)off + 16 > mat.size() * 4) { bad++; continue; }
+            float v[4]; memcpy(v, base + off, 16);
+            for (int e = 0; e < 4; e++) if (v[e] < 0) bad++;                  /* a load outside the rows that exist */
+            for (int e = 0; e < 16; e++) { if (written[tgt + e]) bad++; written[tgt + e] = 1; }
+            memcpy(lds.data() + tgt, base + off, 16);
+         }
+   /* rows past the end of the matrix hold the last rows that exist (the kernel never writes their results) */
+   auto expected = [&](uint32_t r, uint32_t k) -> float
+   {  uint32_t src = r;
+      if (r >= rows) src = KC ? rows - 1 : rows - 4 + r % 4;
+      return (float)(1000 * src + k + 1);
+   };
+   const int wave_rows = 32 * TS;
+   for (uint32_t wbase = 0; wbase < (uint32_t)ROWS; wbase += wave_rows)
+      for (uint32_t lane = 0; lane < 64; lane++)
+         for (int q = 0; q < 4; q++)
+         {  och_f32x4 f[4];
+            for (int x = 0; x < 4; x++) f[x] = och_f32x4{0, 0, 0, 0};
+            for (int x = 0; x < L::READS; x++)
+            {  const uint32_t at = L::read_lane(wbase, lane) + L::read_offset(x, q);
+               const uint32_t width = (KC || TS == 4) ? 16 : 4 * TS;                  /* bytes of the fragment read */
+               if (at % width != 0 || at + width > (uint32_t)L::OPERAND) { bad++; continue; }
+               f[x] = L::read(lds.data() + at);
+            }
+            for (int i = 0; i < TS; i++)
+               for (int t = 0; t < 4; t++)
+               {  const uint32_t r = wbase + L::row(i, lane % 32), k = 8 * q + 4 * (lane / 32) + t;
+                  const float got = L::value(f, i, t), want = expected(r, k);
+                  if (got != want)
+                  {  if (verbose && bad < 10) printf("KC=%d ROWS=%d rows=%u: tile %d step %d quad %d lane %u: got %g, want %g\n", (int)KC, ROWS, rows, i, t, q, lane, got, want);
+                     bad++;
+                  }
+               }
+         }
+   return bad;
+}
+
+extern "C" long gemm_slab_check(int kc, int rows_of_tile, unsigned rows, long ld, int verbose)
+{
+   if (kc) { if (rows_of_tile == 256) return check<true, 256>(rows, ld, verbose); if (rows_of_tile == 128) return check<true, 128>(rows, ld, verbose); if (rows_of_tile == 64) return check<true, 64>(rows, ld, verbose); }
+   else    { if (rows_of_tile == 256) return check<false, 256>(rows, ld, verbose); if (rows_of_tile == 128) return check<false, 128>(rows, ld, verbose); if (rows_of_tile == 64) return check<false, 64>(rows, ld, verbose); }
+   return -1;
+}
