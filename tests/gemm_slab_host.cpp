@@ -1,4 +1,4 @@
-/* Host walk through the LDS layout of the pipelined float GEMM (csrc/och_gemm_f32p_slab.h), for
+/* Host walk through the LDS layout of the pipelined float and double GEMM (csrc/och_gemm_f32p_slab.h, och_gemm_f64p_slab.h), for
    tests/test_gemm_layout_cpu.py. For every operand layout (contiguous along k or along the rows) and every block tile
    (256, 128, 64 rows) a slab of a synthetic matrix is brought into an LDS image by exactly the offsets the kernel's load
    instructions use (4 waves x LOADS instructions x 64 lanes x 16 bytes), and every value an MFMA would get -- tile i of a
@@ -10,6 +10,7 @@
 #include <stdio.h>
 #include <vector>
 #include "och_gemm_f32p_slab.h"
+#include "och_gemm_f64p_slab.h"
 
 using namespace och;
 
@@ -73,5 +74,65 @@ extern "C" long gemm_slab_check(int kc, int rows_of_tile, unsigned rows, long ld
 {
    if (kc) { if (rows_of_tile == 256) return check<true, 256>(rows, ld, verbose); if (rows_of_tile == 128) return check<true, 128>(rows, ld, verbose); if (rows_of_tile == 64) return check<true, 64>(rows, ld, verbose); }
    else    { if (rows_of_tile == 256) return check<false, 256>(rows, ld, verbose); if (rows_of_tile == 128) return check<false, 128>(rows, ld, verbose); if (rows_of_tile == 64) return check<false, 64>(rows, ld, verbose); }
+   return -1;
+}
+
+/* The double kernel: slabs of 16 k, a wave owns half the rows of its operand as TILES tiles of 16 rows; v_mfma_f64_16x16x4
+   takes one double per lane and operand, lanes 16 g .. 16 g + 15 holding k-group g: in step t of pair P, k = 8 P + 2 g + t. */
+template <bool KC, int ROWS>
+static long check_double(uint32_t rows /* a multiple of 2 */, int64_t ld, int verbose)
+{
+   typedef DoubleSlab<KC, ROWS> L;
+   constexpr int KT = OCH_DP_KT, TILES = L::TILES, AREA = KC ? 8 * L::PLANE : 16 * L::ROWP;
+   long bad = 0;
+   std::vector<double> mat((size_t)(KC ? (int64_t)ROWS * ld : (int64_t)KT * ld), -1.0);
+   auto element = [&](int64_t r, int64_t k) -> double & { return mat[(size_t)(KC ? r * ld + k : k * ld + r)]; };
+   for (int64_t r = 0; r < (int64_t)rows; r++) for (int64_t k = 0; k < KT; k++) element(r, k) = (double)(1000 * r + k + 1);
+   const char *base = L::slab_base(reinterpret_cast<const char *>(mat.data()), ld, 0, 0);
+   std::vector<char> lds(AREA, 0);
+   std::vector<unsigned char> written(AREA, 0);
+   for (uint32_t wave = 0; wave < 4; wave++)
+      for (int j = 0; j < L::LOADS; j++)
+         for (uint32_t lane = 0; lane < 64; lane++)
+         {  const uint32_t off = L::load_offset(j, wave, lane, ld, rows), tgt = L::load_target(j, wave) + 16 * lane;
+            if (tgt % 16 != 0 || tgt + 16 > (uint32_t)AREA) { bad++; continue; }
+            if ((size_t)off + 16 > mat.size() * 8) { bad++; continue; }
+            double v[2]; memcpy(v, base + off, 16);
+            for (int e = 0; e < 2; e++) if (v[e] < 0) bad++;
+            for (int e = 0; e < 16; e++) { if (written[tgt + e]) bad++; written[tgt + e] = 1; }
+            memcpy(lds.data() + tgt, base + off, 16);
+         }
+   auto expected = [&](uint32_t r, uint32_t k) -> double
+   {  uint32_t src = r;
+      if (r >= rows) src = KC ? rows - 1 : rows - 2 + r % 2;
+      return (double)(1000 * src + k + 1);
+   };
+   for (uint32_t wbase = 0; wbase < (uint32_t)ROWS; wbase += ROWS / 2)
+      for (uint32_t lane = 0; lane < 64; lane++)
+         for (int P = 0; P < KT / 8; P++)
+         {  och_f64x2 f[TILES];
+            for (int x = 0; x < TILES; x++)
+            {  f[x] = och_f64x2{0, 0};
+               const uint32_t at = L::read_lane(wbase, lane) + L::read_offset(x, P);
+               if (at % 16 != 0 || at + 16 > (uint32_t)AREA) { bad++; continue; }
+               memcpy(&f[x], lds.data() + at, 16);
+            }
+            for (int i = 0; i < TILES; i++)
+               for (int t = 0; t < 2; t++)
+               {  const uint32_t r = wbase + L::row(i, lane % 16), k = 8 * P + 2 * (lane / 16) + t;
+                  const double got = L::value(f, i, t), want = expected(r, k);
+                  if (got != want)
+                  {  if (verbose && bad < 10) printf("double KC=%d ROWS=%d rows=%u: tile %d step %d pair %d lane %u: got %g, want %g\n", (int)KC, ROWS, rows, i, t, P, lane, got, want);
+                     bad++;
+                  }
+               }
+         }
+   return bad;
+}
+
+extern "C" long gemm_slab_check_double(int kc, int rows_of_tile, unsigned rows, long ld, int verbose)
+{
+   if (kc) { if (rows_of_tile == 256) return check_double<true, 256>(rows, ld, verbose); if (rows_of_tile == 128) return check_double<true, 128>(rows, ld, verbose); }
+   else    { if (rows_of_tile == 256) return check_double<false, 256>(rows, ld, verbose); if (rows_of_tile == 128) return check_double<false, 128>(rows, ld, verbose); }
    return -1;
 }

@@ -1,4 +1,4 @@
-"""The LDS layout of the pipelined float GEMM kernel, walked through on the host.
+"""The LDS layout of the pipelined float and double GEMM kernels, walked through on the host.
 
 csrc/och_gemm_f32p_slab.h holds the index arithmetic of gemm_float_pipe_kernel (the counterpart of cublasSgemm in
 src/core/gpu/op/tensor_blas_gpu.c:183-197): which 16 bytes every lane of every load instruction fetches and where in LDS
@@ -26,6 +26,8 @@ def slab(tmp_path_factory):
     lib = C.CDLL(so)
     lib.gemm_slab_check.restype = C.c_long
     lib.gemm_slab_check.argtypes = [C.c_int, C.c_int, C.c_uint, C.c_long, C.c_int]
+    lib.gemm_slab_check_double.restype = C.c_long
+    lib.gemm_slab_check_double.argtypes = [C.c_int, C.c_int, C.c_uint, C.c_long, C.c_int]
     return lib
 
 
@@ -39,5 +41,16 @@ def test_every_mfma_operand_is_the_matrix_element_it_has_to_be(slab, kc, tile):
             assert slab.gemm_slab_check(kc, tile, rows, ld, 1) == 0, (kc, tile, rows, ld)
 
 
+@pytest.mark.parametrize("tile", [256, 128])
+@pytest.mark.parametrize("kc", [0, 1], ids=["contiguous_along_rows", "contiguous_along_k"])
+def test_every_double_mfma_operand_is_the_matrix_element_it_has_to_be(slab, kc, tile):
+    """The same walk for gemm_double_pipe_kernel (csrc/och_gemm_f64p_slab.h): slabs of 16 k, operands of 256 rows (A of the
+    large tile) and 128 rows, tiles of 16 rows, last tiles of which only a few rows exist (multiples of 2)."""
+    for rows in sorted({tile, tile - 2, tile // 2 + 2, tile // 2, 34, 6, 2}):
+        for ld in ((16, 18, 1000) if kc else (tile, tile + 6, 4 * tile + 2)):
+            assert slab.gemm_slab_check_double(kc, tile, rows, ld, 1) == 0, (kc, tile, rows, ld)
+
+
 def test_unknown_tile_is_refused(slab):
     assert slab.gemm_slab_check(0, 96, 96, 96, 0) == -1
+    assert slab.gemm_slab_check_double(0, 64, 64, 64, 0) == -1
