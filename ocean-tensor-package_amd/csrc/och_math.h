@@ -1,9 +1,11 @@
-/* Two elementary functions written out in IEEE basic operations: powf and tanh (double).
+/* Elementary functions written out in IEEE basic operations: powf, tanh (double), sinh, cosh, log1p, asinh, acosh, atanh.
  *
- * The device math library's routines for these two cost more arithmetic than the memory system leaves time for (powf
- * about 210 instructions per element, tanh on double about 140 double-precision operations, most of them the
- * double-double arithmetic of its extended exponential); a streaming kernel built on them runs at half the rate of its
- * neighbours. The routines below need a third of that. They use additions, multiplications, fused multiply-adds,
+ * The device math library's routines for these cost more arithmetic than the memory system leaves time for (powf about
+ * 210 instructions per element, tanh on double about 140 double-precision operations, most of them the double-double
+ * arithmetic of its extended exponential; sinh, cosh, log1p and the inverse hyperbolic functions 125 to 200 instructions
+ * in either precision, against the 48 (float) and 96 (double) that fit under the memory time of a unary kernel); a
+ * streaming kernel built on them runs at half the rate of its neighbours or less. The routines below need a third to a
+ * half of that. The float versions evaluate in double precision with shorter polynomials and round once. They use additions, multiplications, fused multiply-adds,
  * divisions, conversions and integer operations on the bits only -- no library call -- so a host build of this header
  * gives bit for bit what the device gives, and the accuracy against the host's libm (the reference's CPU functions:
  * solid/include/solid/core/cpu/unary_ops_cpu.h:24-140, powf for the power of both float and double) is established on the
@@ -19,6 +21,13 @@
  *   och_tanh(x)      E / (E + 2) with E = exp(2|x|) - 1 built without cancellation from a reduction by ln 2 in two parts
  *                    and a degree-13 polynomial for e^g - 1; 1 from 20 on. Within 2 units in the last place of the
  *                    host's tanh.
+ *   och_sinh, och_cosh   from the same exponential: (E + E / (E + 1)) / 2 below 1, e^a / 2 -+ 1 / (2 e^a) above, overflowing
+ *                    where the functions do (not where e^a does). Within 3 units in the last place of the host's.
+ *   och_log1p, och_atanh, och_asinh, och_acosh   fdlibm's formulas (s_log1p.c, e_atanh.c, s_asinh.c, e_acosh.c) on a log of
+ *                    this file's own (atanh series of (m - 1) / (m + 1), e ln 2 added in two parts), every case of each
+ *                    function as one log1p of a selected argument. Within 3 units in the last place of the host's.
+ *   och_*f           the same in double precision with shorter series, rounded to float once: within 2 units of the
+ *                    host's float functions (which are themselves not correctly rounded).
  */
 #pragma once
 #include <stdint.h>
@@ -149,5 +158,179 @@ OCH_MATH_FN double och_tanh(double x)
    r = math_from_bits(math_to_bits(r) | (bx & 0x8000000000000000ull));
    return a == a ? r : x + x;                                               /* NaN stays NaN */
 }
+
+/* ---- hyperbolic sine and cosine ----------------------------------------------------------------------------------
+   e^u for u >= 0 in two parts: k, the nearest integer to u / ln 2, and e^g - 1 for the rest g (|g| <= 0.347), which is
+   g + g^2 (1/2 + g/6 + ...) without a rounded 1 in it. FULL: degree 13, for results in double; otherwise degree 9
+   (relative truncation 2e-11), for results that are rounded to float. */
+template <bool FULL>
+OCH_MATH_FN double math_exp_rest(double u, double &k)
+{
+   k = __builtin_rint(u * 1.4426950408889634074);
+   double g = __builtin_fma(k, -6.93147180369123816490e-01, u);
+   g = __builtin_fma(k, -1.90821492927058770002e-10, g);
+   double q;
+   if (FULL)
+   {  q = 1.0 / 6227020800.0;
+      q = __builtin_fma(q, g, 1.0 / 479001600.0); q = __builtin_fma(q, g, 1.0 / 39916800.0); q = __builtin_fma(q, g, 1.0 / 3628800.0);
+      q = __builtin_fma(q, g, 1.0 / 362880.0);
+   }
+   else q = 1.0 / 362880.0;
+   q = __builtin_fma(q, g, 1.0 / 40320.0); q = __builtin_fma(q, g, 1.0 / 5040.0); q = __builtin_fma(q, g, 1.0 / 720.0);
+   q = __builtin_fma(q, g, 1.0 / 120.0);   q = __builtin_fma(q, g, 1.0 / 24.0);   q = __builtin_fma(q, g, 1.0 / 6.0);
+   q = __builtin_fma(q, g, 0.5);
+   return __builtin_fma(g * g, q, g);
+}
+
+/* e^a / 2 for 0 <= a <= 711 without an early overflow: (e^g 2^(k - 1 - c)) 2^c, c = 64 for the largest k */
+OCH_MATH_FN double math_half_exp(double em1, double k)
+{
+   const int ik = (int)k, c = ik > 1000 ? 64 : 0;
+   return ((em1 + 1.0) * math_pow2i(ik - 1 - c)) * math_pow2i(c);
+}
+
+/* sinh a = (E + E / (E + 1)) / 2 with E = e^a - 1 below 1 (no cancellation: E = 2^k (e^g - 1) + (2^k - 1), k = 0 or 1),
+   e^a / 2 - 1 / (2 e^a) from 1 on; cosh a = e^a / 2 + 1 / (2 e^a). Overflow to infinity where the functions overflow
+   (710.4758...), not where e^a does. */
+template <bool FULL>
+OCH_MATH_FN double math_sinh(double x)
+{
+   const uint64_t bx = math_to_bits(x);
+   const double a = math_from_bits(bx & 0x7FFFFFFFFFFFFFFFull);
+   double k;
+   const double em1 = math_exp_rest<FULL>(a < 711.0 ? a : 711.0, k);
+   const double pk = k < 2.0 ? k + 1.0 : 1.0;                              /* 2^k for k = 0, 1 (only used below 1) */
+   const double E = __builtin_fma(pk, em1, pk - 1.0);
+   const double th = math_half_exp(em1, k);
+   const bool small = a < 1.0;
+   const double q = (small ? E : 0.25) / (small ? E + 1.0 : th);          /* one division for both forms */
+   double r = small ? 0.5 * (E + q) : th - q;
+   r = math_from_bits(math_to_bits(r) | (bx & 0x8000000000000000ull));
+   return a == a ? r : x + x;
+}
+template <bool FULL>
+OCH_MATH_FN double math_cosh(double x)
+{
+   const double a = math_from_bits(math_to_bits(x) & 0x7FFFFFFFFFFFFFFFull);
+   double k;
+   const double em1 = math_exp_rest<FULL>(a < 711.0 ? a : 711.0, k);
+   const double th = math_half_exp(em1, k);
+   const double r = th + 0.25 / th;
+   return a == a ? r : x + x;
+}
+OCH_MATH_FN double och_sinh(double x) { return math_sinh<true>(x); }
+OCH_MATH_FN double och_cosh(double x) { return math_cosh<true>(x); }
+OCH_MATH_FN float  och_sinhf(float x) { return (float)math_sinh<false>((double)x); }
+OCH_MATH_FN float  och_coshf(float x) { return (float)math_cosh<false>((double)x); }
+
+/* ---- log1p and the inverse hyperbolic functions ---------------------------------------------------------------------
+   log of a positive normal double: v = 2^e m with m in [0.707, 1.414), log m = 2 atanh s = 2 s (1 + z / 3 + z^2 / 5 + ...),
+   s = (m - 1) / (m + 1), z = s^2 <= 0.0295. FULL: terms up to z^9 / 19 (truncation 2e-17); otherwise up to z^5 / 11
+   (1e-10, for results rounded to float). e ln 2 is added in two parts. */
+template <bool FULL>
+OCH_MATH_FN double math_log_normal(double v)
+{
+   const uint64_t u = math_to_bits(v);
+   int e = (int)(u >> 52) - 1023;
+   double m = math_from_bits((u & 0x000FFFFFFFFFFFFFull) | 0x3FF0000000000000ull);
+   const bool upper = m >= 1.4142135623730951;
+   m = upper ? m * 0.5 : m;
+   e = upper ? e + 1 : e;
+   const double s = (m - 1.0) / (m + 1.0), z = s * s;
+   double t;
+   if (FULL)
+   {  t = 1.0 / 19.0;
+      t = __builtin_fma(t, z, 1.0 / 17.0); t = __builtin_fma(t, z, 1.0 / 15.0); t = __builtin_fma(t, z, 1.0 / 13.0);
+      t = __builtin_fma(t, z, 1.0 / 11.0);
+   }
+   else t = 1.0 / 11.0;
+   t = __builtin_fma(t, z, 1.0 / 9.0); t = __builtin_fma(t, z, 1.0 / 7.0); t = __builtin_fma(t, z, 1.0 / 5.0);
+   t = __builtin_fma(t, z, 1.0 / 3.0);
+   const double two_s = s + s, de = (double)e;
+   const double logm = __builtin_fma(two_s * z, t, two_s);
+   return __builtin_fma(de, 6.93147180369123816490e-01, __builtin_fma(de, 1.90821492927058770002e-10, logm));
+}
+
+/* log(1 + y) for y > -1, finite: the log of the rounded sum plus what the rounding took away, (y - (u - 1)) / u */
+template <bool FULL>
+OCH_MATH_FN double math_log1p_core(double y)
+{
+   const double u = 1.0 + y;
+   const double c = (u - 1.0 == y) ? 0.0 : (y - (u - 1.0)) / u;          /* (the division only where the sum was rounded) */
+   return math_log_normal<FULL>(u) + c;
+}
+
+template <bool FULL>
+OCH_MATH_FN double math_log1p(double x)
+{
+   const double inf = math_from_bits(0x7FF0000000000000ull);
+   const bool plain = x > -1.0 && x < inf;
+   double r = math_log1p_core<FULL>(plain ? x : 0.0);
+   /* 1 + x = 1 for tiny x: the correction term alone gives x (also for -0 and subnormal x, where log 1 + x / 1 = x) */
+   if (x == 0.0) r = x;                                                    /* keeps the sign of zero */
+   if (x == inf) r = inf;
+   if (x == -1.0) r = -inf;
+   if (x < -1.0 || x != x) r = math_from_bits(0x7FF8000000000000ull);
+   return r;
+}
+
+/* atanh a = log1p(2a / (1 - a)) / 2, below 0.5 as log1p(2a + 2a a / (1 - a)) / 2 (e_atanh.c of fdlibm) */
+template <bool FULL>
+OCH_MATH_FN double math_atanh(double x)
+{
+   const uint64_t bx = math_to_bits(x);
+   const double a = math_from_bits(bx & 0x7FFFFFFFFFFFFFFFull);
+   const bool plain = a < 1.0;
+   const double b = plain ? a : 0.0, t = b + b, q = b / (1.0 - b);                  /* (2a / (1 - a) = 2 q: one division) */
+   double r = 0.5 * math_log1p_core<FULL>(b < 0.5 ? __builtin_fma(t, q, t) : q + q);
+   if (a == 1.0) r = math_from_bits(0x7FF0000000000000ull);
+   r = math_from_bits(math_to_bits(r) | (bx & 0x8000000000000000ull));
+   if (a > 1.0 || a != a) r = math_from_bits(0x7FF8000000000000ull);
+   return r;
+}
+
+/* asinh a = log1p(a + a^2 / (1 + sqrt(1 + a^2))) up to 2, log(a + sqrt(a^2 + 1)) = log1p((a - 1) + sqrt(a^2 + 1)) above (no
+   cancellation there), log a + log 2 from 2^28 on (the cases of s_asinh.c of fdlibm); all three as one log1p */
+template <bool FULL>
+OCH_MATH_FN double math_asinh(double x)
+{
+   const uint64_t bx = math_to_bits(x);
+   const double a = math_from_bits(bx & 0x7FFFFFFFFFFFFFFFull);
+   const bool big = a >= 268435456.0, finite = a < math_from_bits(0x7FF0000000000000ull);
+   const double b = (big || !finite) ? 1.0 : a, t = b * b, root = __builtin_sqrt(t + 1.0);
+   const double low = b + t / (1.0 + root);
+   const double high = (b - 1.0) + root;
+   double w = b <= 2.0 ? low : high;
+   w = big && finite ? a - 1.0 : w;
+   double r = math_log1p_core<FULL>(w) + (big ? 6.93147180559945286227e-01 : 0.0);
+   r = finite ? r : a;                                                      /* infinity, NaN */
+   r = math_from_bits(math_to_bits(r) | (bx & 0x8000000000000000ull));
+   return a == a ? r : x + x;
+}
+
+/* acosh x = log(x + sqrt(x^2 - 1)) = log1p(t + sqrt(t^2 + 2 t)), t = x - 1: sums of positive terms for every x >= 1;
+   log x + log 2 from 2^28 on (e_acosh.c of fdlibm has the same cases with a log instead of a log1p above 2) */
+template <bool FULL>
+OCH_MATH_FN double math_acosh(double x)
+{
+   const double inf = math_from_bits(0x7FF0000000000000ull);
+   const bool big = x >= 268435456.0, plain = x >= 1.0 && x < inf;
+   const double b = (plain && !big) ? x : 1.0, t = b - 1.0;
+   double w = t + __builtin_sqrt(__builtin_fma(t, t, t + t));
+   w = big && plain ? x - 1.0 : w;
+   double r = math_log1p_core<FULL>(w) + ((big && plain) ? 6.93147180559945286227e-01 : 0.0);
+   if (x == inf) r = inf;
+   if (x < 1.0 || x != x) r = math_from_bits(0x7FF8000000000000ull);
+   return r;
+}
+
+OCH_MATH_FN double och_log1p(double x) { return math_log1p<true>(x); }
+OCH_MATH_FN double och_atanh(double x) { return math_atanh<true>(x); }
+OCH_MATH_FN double och_asinh(double x) { return math_asinh<true>(x); }
+OCH_MATH_FN double och_acosh(double x) { return math_acosh<true>(x); }
+OCH_MATH_FN float  och_log1pf(float x) { return (float)math_log1p<false>((double)x); }
+OCH_MATH_FN float  och_atanhf(float x) { return (float)math_atanh<false>((double)x); }
+OCH_MATH_FN float  och_asinhf(float x) { return (float)math_asinh<false>((double)x); }
+OCH_MATH_FN float  och_acoshf(float x) { return (float)math_acosh<false>((double)x); }
 
 } /* namespace och */

@@ -22,13 +22,13 @@ namespace och {
 #define OCH_MATH1(NAME, FN, DN) \
    template <class W> OCH_D W NAME(W x) { if constexpr (std::is_same<W, float>::value) return FN(x); else return DN(x); }
 OCH_MATH1(m_sin, sinf, sin)       OCH_MATH1(m_cos, cosf, cos)       OCH_MATH1(m_tan, tanf, tan)
-OCH_MATH1(m_sinh, sinhf, sinh)    OCH_MATH1(m_cosh, coshf, cosh)    OCH_MATH1(m_tanh, tanhf, och_tanh)   /* double: och_math.h */
+OCH_MATH1(m_sinh, och_sinhf, och_sinh) OCH_MATH1(m_cosh, och_coshf, och_cosh) OCH_MATH1(m_tanh, tanhf, och_tanh)   /* och_*: och_math.h */
 OCH_MATH1(m_asin, asinf, asin)    OCH_MATH1(m_acos, acosf, acos)    OCH_MATH1(m_atan, atanf, atan)
-OCH_MATH1(m_asinh, asinhf, asinh) OCH_MATH1(m_acosh, acoshf, acosh) OCH_MATH1(m_atanh, atanhf, atanh)
+OCH_MATH1(m_asinh, och_asinhf, och_asinh) OCH_MATH1(m_acosh, och_acoshf, och_acosh) OCH_MATH1(m_atanh, och_atanhf, och_atanh)
 OCH_MATH1(m_sqrt, sqrtf, sqrt)    OCH_MATH1(m_cbrt, cbrtf, cbrt)
 OCH_MATH1(m_exp, expf, exp)       OCH_MATH1(m_exp2, exp2f, exp2)    OCH_MATH1(m_expm1, expm1f, expm1)
 OCH_MATH1(m_log, logf, log)       OCH_MATH1(m_log2, log2f, log2)    OCH_MATH1(m_log10, log10f, log10)
-OCH_MATH1(m_log1p, log1pf, log1p)
+OCH_MATH1(m_log1p, och_log1pf, och_log1p)
 OCH_MATH1(m_fabs, fabsf, fabs)    OCH_MATH1(m_ceil, ceilf, ceil)    OCH_MATH1(m_floor, floorf, floor)
 OCH_MATH1(m_trunc, truncf, trunc) OCH_MATH1(m_round, roundf, round)
 #undef OCH_MATH1

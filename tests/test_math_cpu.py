@@ -1,5 +1,5 @@
-"""The two elementary functions the device library evaluates itself (csrc/och_math.h: powf, tanh on double) against the
-host's libm, the functions the reference's CPU module calls (solid/include/solid/core/cpu/unary_ops_cpu.h:24-140; powf
+"""The elementary functions the device library evaluates itself (csrc/och_math.h: powf, tanh on double, sinh, cosh, log1p
+and the inverse hyperbolic functions in both precisions) against the host's libm, the functions the reference's CPU module calls (solid/include/solid/core/cpu/unary_ops_cpu.h:24-140; powf
 for the power of float and double alike, binary_ops.h). The header uses IEEE basic operations only, so its host build
 (tests/math_host.cpp, compiled here with g++) computes bit for bit what the kernels compute; what is established here on
 millions of arguments holds on the device."""
@@ -123,3 +123,50 @@ def test_tanh_special_values_and_monotone_ends(mathlib):
     assert np.array_equal(got[:4].view(np.uint64), want[:4].view(np.uint64))            # signed zeros, +-1 at the infinities
     assert np.array_equal(got[5:8], x[5:8])                                              # tanh x = x for subnormal x
     assert np.all(got[9:13] == 1.0) and got[13] == -1.0 and got[14] == 1.0 and got[15] == -1.0
+
+
+ONE_ARGUMENT = {
+    # name: (ranges in double, ranges in float)
+    "sinh": [(-1, 1), (0, 1e-3), (0.9, 1.1), (-22, 22), (-709, 709), (709, 712)],
+    "cosh": [(-1, 1), (0, 1e-3), (0.9, 1.1), (-22, 22), (-709, 709), (709, 712)],
+    "log1p": [(-0.999, 1), (-1e-3, 1e-3), (-0.5, 0.5), (0, 100), (1e10, 1e300), (-1, -0.99)],
+    "atanh": [(-0.999, 0.999), (-1e-3, 1e-3), (0.4, 0.6), (0.99, 1.0)],
+    "asinh": [(-1, 1), (-1e-3, 1e-3), (1.9, 2.1), (-100, 100), (1e8, 1e9), (1e100, 1e300)],
+    "acosh": [(1, 1.001), (1, 2), (1.9, 2.1), (2, 100), (1e8, 1e9), (1e100, 1e300)],
+}
+SPECIAL = [0.0, -0.0, np.inf, -np.inf, np.nan, 1e-300, -1e-300, 1e-40, -1.0, 1.0, -2.0, 0.5, -0.5, 2.0, 2.0 ** 28, 2.0 ** 28 + 1, 1e-20, -1e-20, 3e38,
+           -3e38, 710.4, 710.5, 89.4, 89.5, 88.7, 1.0 - 2.0 ** -53, -1.0 + 2.0 ** -53, 1.0 + 2.0 ** -52]
+
+
+@pytest.mark.parametrize("single", [False, True], ids=["double", "float"])
+@pytest.mark.parametrize("name", list(ONE_ARGUMENT))
+def test_hyperbolic_and_log1p_routines_stay_within_three_units_of_the_host(mathlib, name, single):
+    """double: within 3 units in the last place of the host's function; float (evaluated in double precision and rounded
+    once): within 2 of the host's float function and within 1 of the host's double function rounded to float. NaN, the
+    infinities and signed zeros exactly as the host gives them."""
+    dt = np.float32 if single else np.float64
+    fn = name + ("f" if single else "")
+    rng = np.random.default_rng(sum(map(ord, fn)))
+    for lo, hi in ONE_ARGUMENT[name]:
+        if single:
+            if lo >= 1e100:
+                lo, hi = 1e30, 3e38
+            elif abs(hi) >= 700:
+                lo, hi = (lo / 709 * 88, hi / 709 * 88) if hi <= 709 else (88, 91)
+        x = rng.uniform(lo, hi, N // 2).astype(dt)
+        got, want = call1(mathlib, "host_och_" + fn, x), call1(mathlib, "host_libm_" + fn, x)
+        d = ulps(got, want)
+        worst = int(np.argmax(d))
+        assert d[worst] <= (2 if single else 3), "%s(%r) = %r, host %r" % (fn, x[worst], got[worst], want[worst])
+        if single:
+            with np.errstate(all="ignore"):
+                rounded = call1(mathlib, "host_libm_" + name, x.astype(np.float64)).astype(np.float32)
+            assert ulps(got, rounded).max() <= 1
+            assert (ulps(got, rounded) != 0).mean() < 1e-4          # the correctly rounded value but for a few cases
+    x = np.array(SPECIAL, dtype=dt)
+    got, want = call1(mathlib, "host_och_" + fn, x), call1(mathlib, "host_libm_" + fn, x)
+    d = ulps(got, want)
+    assert d.max() <= 3, [(a, b, c) for a, b, c in zip(x, got, want) if not (a == a and b == c)][:5]
+    unusual = ~np.isfinite(want) | (want == 0)
+    assert np.array_equal(got[unusual & ~np.isnan(want)].view(np.uint32 if single else np.uint64),
+                          want[unusual & ~np.isnan(want)].view(np.uint32 if single else np.uint64))
