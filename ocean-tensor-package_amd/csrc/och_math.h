@@ -228,7 +228,7 @@ OCH_MATH_FN float  och_coshf(float x) { return (float)math_cosh<false>((double)x
    s = (m - 1) / (m + 1), z = s^2 <= 0.0295. FULL: terms up to z^9 / 19 (truncation 2e-17); otherwise up to z^5 / 11
    (1e-10, for results rounded to float). e ln 2 is added in two parts. */
 template <bool FULL>
-OCH_MATH_FN double math_log_normal(double v)
+OCH_MATH_FN void math_log_parts(double v, double &de, double &f, double &tail)
 {
    const uint64_t u = math_to_bits(v);
    int e = (int)(u >> 52) - 1023;
@@ -236,19 +236,29 @@ OCH_MATH_FN double math_log_normal(double v)
    const bool upper = m >= 1.4142135623730951;
    m = upper ? m * 0.5 : m;
    e = upper ? e + 1 : e;
-   const double s = (m - 1.0) / (m + 1.0), z = s * s;
+   f = m - 1.0;                                                             /* exact */
+   const double s = f / (2.0 + f), z = s * s;
    double t;
    if (FULL)
-   {  t = 1.0 / 19.0;
-      t = __builtin_fma(t, z, 1.0 / 17.0); t = __builtin_fma(t, z, 1.0 / 15.0); t = __builtin_fma(t, z, 1.0 / 13.0);
-      t = __builtin_fma(t, z, 1.0 / 11.0);
+   {  t = 2.0 / 19.0;
+      t = __builtin_fma(t, z, 2.0 / 17.0); t = __builtin_fma(t, z, 2.0 / 15.0); t = __builtin_fma(t, z, 2.0 / 13.0);
+      t = __builtin_fma(t, z, 2.0 / 11.0);
    }
-   else t = 1.0 / 11.0;
-   t = __builtin_fma(t, z, 1.0 / 9.0); t = __builtin_fma(t, z, 1.0 / 7.0); t = __builtin_fma(t, z, 1.0 / 5.0);
-   t = __builtin_fma(t, z, 1.0 / 3.0);
-   const double two_s = s + s, de = (double)e;
-   const double logm = __builtin_fma(two_s * z, t, two_s);
-   return __builtin_fma(de, 6.93147180369123816490e-01, __builtin_fma(de, 1.90821492927058770002e-10, logm));
+   else t = 2.0 / 11.0;
+   t = __builtin_fma(t, z, 2.0 / 9.0); t = __builtin_fma(t, z, 2.0 / 7.0); t = __builtin_fma(t, z, 2.0 / 5.0);
+   t = __builtin_fma(t, z, 2.0 / 3.0);
+   /* log m = 2 s + s R, R = z t; with 2 s = f - s f and f^2 / 2 split off: log m = f - (f^2 / 2 - s (f^2 / 2 + R)), the
+      arrangement of fdlibm's e_log.c: the leading term is exact and everything after it is small */
+   const double hfsq = 0.5 * f * f;
+   tail = hfsq - s * __builtin_fma(z, t, hfsq);                             /* log m = f - tail */
+   de = (double)e;
+}
+template <bool FULL>
+OCH_MATH_FN double math_log_normal(double v)
+{
+   double de, f, tail;
+   math_log_parts<FULL>(v, de, f, tail);
+   return __builtin_fma(de, 6.93147180369123816490e-01, -((tail - de * 1.90821492927058770002e-10) - f));
 }
 
 /* log(1 + y) for y > -1, finite: the log of the rounded sum plus what the rounding took away, (y - (u - 1)) / u */
