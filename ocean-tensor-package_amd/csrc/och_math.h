@@ -224,9 +224,10 @@ OCH_MATH_FN float  och_sinhf(float x) { return (float)math_sinh<false>((double)x
 OCH_MATH_FN float  och_coshf(float x) { return (float)math_cosh<false>((double)x); }
 
 /* ---- log1p and the inverse hyperbolic functions ---------------------------------------------------------------------
-   log of a positive normal double: v = 2^e m with m in [0.707, 1.414), log m = 2 atanh s = 2 s (1 + z / 3 + z^2 / 5 + ...),
-   s = (m - 1) / (m + 1), z = s^2 <= 0.0295. FULL: terms up to z^9 / 19 (truncation 2e-17); otherwise up to z^5 / 11
-   (1e-10, for results rounded to float). e ln 2 is added in two parts. */
+   log of a positive normal double: v = 2^e m with m in [0.707, 1.414), f = m - 1, log m = 2 atanh s = 2 s + s R with
+   s = f / (2 + f), z = s^2 <= 0.0295, R = z (2/3 + 2/5 z + 2/7 z^2 + ...). FULL: terms up to 2/19 z^9 (truncation 2e-17);
+   otherwise up to 2/11 z^5 (1e-10, for results rounded to float). math_log_parts returns e, f and the small part of
+   log m = f - tail; e ln 2 is added in two parts. */
 template <bool FULL>
 OCH_MATH_FN void math_log_parts(double v, double &de, double &f, double &tail)
 {
