@@ -593,7 +593,7 @@ def main():
         for dt, es, nm, npt in ((F32, 4, "f32", np.float32), (F64, 8, "f64", np.float64)):
             sets_ = extra_sets(es, es, 1, lambda k: rng.uniform(0.5, 4.0, 1 << 22).astype(npt))
             stx = oh.strides([es]); ut = [0]
-            for opn in ("sqrt", "exp", "sin", "tanh"):
+            for opn in ("sqrt", "exp", "sin", "tanh", "sinh", "cosh", "log1p", "arcsinh"):
                 def un(opn=opn):
                     ins, o = sets_[ut[0] % 2]; ut[0] += 1
                     oh.check(lib.och_unary(U[opn], dt, 1, se, stx, ins[0].ptr, stx, o.ptr, h))
