@@ -267,7 +267,8 @@ template <bool FULL>
 OCH_MATH_FN double math_log1p_core(double y)
 {
    const double u = 1.0 + y;
-   const double c = (u - 1.0 == y) ? 0.0 : (y - (u - 1.0)) / u;          /* (the division only where the sum was rounded) */
+   /* for a result rounded to float the lost part matters only where u is within 2^-29 of 1: no division by u there */
+   const double c = FULL ? ((u - 1.0 == y) ? 0.0 : (y - (u - 1.0)) / u) : y - (u - 1.0);
    return math_log_normal<FULL>(u) + c;
 }
 
