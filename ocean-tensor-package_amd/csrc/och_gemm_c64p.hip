@@ -18,15 +18,14 @@
  *   - any M and N: an element is a whole 16-byte piece of C. The last tiles clamp their loads to the rows that exist.
  */
 #include "och_gemm.h"
+#include "och_gemm_c64p_slab.h"
 #pragma clang diagnostic ignored "-Winline-asm"
 
 namespace och {
 
-typedef double och_f64x2 __attribute__((ext_vector_type(2)));
 
 #define OCH_ZP_BM 128
 #define OCH_ZP_BN 64
-#define OCH_ZP_KT 16
 #define OCH_ZP_THREADS 256
 #define OCH_ZP_A 33792                       /* LDS bytes of A's slab (128 rows of 16 k) */
 #define OCH_ZP_B 17408                       /* LDS bytes of B's slab (64 rows) */
@@ -51,41 +50,6 @@ struct CDoublePipeParams
    GemmBatch batch;
 };
 
-/* one operand's slab of ROWS = 128 or 64 rows and 16 k, [k][row][re, im] in LDS: where its loads come from and go to,
-   where the fragments are read */
-template <bool KC, int ROWS>
-struct CDoubleSlab
-{
-   static constexpr int PLANE = ROWS * 16 + 64;      /* bytes per k */
-   static constexpr int LOADS = ROWS * OCH_ZP_KT * 16 / 1024 / 4;     /* loads per wave and slab: 8 or 4 */
-   static constexpr int TILES = ROWS / 2 / 16;       /* tiles per wave: 4 or 2 */
-   static constexpr int READS = 2 * TILES;           /* fragment reads per pair of steps */
-   static constexpr int PARTS = ROWS / 64;           /* groups of 64 rows: one load instruction each per k */
-   /* load j of wave w: unit u = w * LOADS + j is the rows 64 (u % PARTS) ... of k = u / PARTS; lane l fetches row l of them.
-      `rows`: how many of the tile's rows exist; lanes whose row does not exist fetch the last one that does */
-   static __device__ __forceinline__ uint32_t load_offset(int j, uint32_t wave, uint32_t lane, int64_t ld, uint32_t rows)
-   {  const uint32_t u = wave * LOADS + j, k = u / PARTS;
-      uint32_t row = (u % PARTS) * 64 + lane;
-      row = row < rows ? row : rows - 1;
-      return (uint32_t)((KC ? (int64_t)row * ld + k : (int64_t)k * ld + row) * 16);
-   }
-   static __device__ __forceinline__ uint32_t load_target(int j, uint32_t wave)
-   {  const uint32_t u = wave * LOADS + j;
-      return (u / PARTS) * PLANE + (u % PARTS) * 1024;
-   }
-   static __device__ __forceinline__ const char *slab_base(const char *mat, int64_t ld, uint32_t mn0, uint32_t k0)
-   {  return mat + (KC ? ((int64_t)k0 + (int64_t)mn0 * ld) : ((int64_t)mn0 + (int64_t)k0 * ld)) * 16; }
-   /* fragment read x (0 .. READS - 1) of pair P -- tile x % TILES in step x / TILES: the lane's part of the address, and the immediate part */
-   static __device__ __forceinline__ uint32_t read_lane(uint32_t wbase, uint32_t lane)
-   {  const uint32_t r = lane % 16, kg = lane / 16;
-      return kg * PLANE + (wbase + r) * 16;
-   }
-   static constexpr uint32_t read_offset(int x, int P) { return (uint32_t)(4 * (2 * P + x / TILES) * PLANE + (x % TILES) * 256); }
-   /* part c (0: real, 1: imaginary) of the value of tile i in step t within a pair's reads */
-   static __device__ __forceinline__ double value(const och_f64x2 (&f)[READS], int i, int t, int c) { return f[t * TILES + i][c]; }
-   /* row (of the wave's rows) of tile i, row-in-tile rr */
-   static __device__ __forceinline__ uint32_t row(int i, uint32_t rr) { return (uint32_t)i * 16 + rr; }
-};
 static_assert(16 * CDoubleSlab<true, 128>::PLANE <= OCH_ZP_A && 16 * CDoubleSlab<true, 64>::PLANE <= OCH_ZP_B, "the slabs do not fit");
 
 /* 16 bytes of LDS into two ordinary registers pairs. Written as an instruction of its own so that the value lands in the

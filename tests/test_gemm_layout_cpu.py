@@ -1,4 +1,4 @@
-"""The LDS layout of the pipelined float and double GEMM kernels, walked through on the host.
+"""The LDS layout of the four pipelined GEMM kernels (float, double, complex float, complex double), walked through on the host.
 
 csrc/och_gemm_f32p_slab.h holds the index arithmetic of gemm_float_pipe_kernel (the counterpart of cublasSgemm in
 src/core/gpu/op/tensor_blas_gpu.c:183-197): which 16 bytes every lane of every load instruction fetches and where in LDS
@@ -28,6 +28,10 @@ def slab(tmp_path_factory):
     lib.gemm_slab_check.argtypes = [C.c_int, C.c_int, C.c_uint, C.c_long, C.c_int]
     lib.gemm_slab_check_double.restype = C.c_long
     lib.gemm_slab_check_double.argtypes = [C.c_int, C.c_int, C.c_uint, C.c_long, C.c_int]
+    lib.gemm_slab_check_cfloat.restype = C.c_long
+    lib.gemm_slab_check_cfloat.argtypes = [C.c_int, C.c_uint, C.c_long, C.c_int]
+    lib.gemm_slab_check_cdouble.restype = C.c_long
+    lib.gemm_slab_check_cdouble.argtypes = [C.c_int, C.c_int, C.c_uint, C.c_long, C.c_int]
     return lib
 
 
@@ -49,6 +53,19 @@ def test_every_double_mfma_operand_is_the_matrix_element_it_has_to_be(slab, kc, 
     for rows in sorted({tile, tile - 2, tile // 2 + 2, tile // 2, 34, 6, 2}):
         for ld in ((16, 18, 1000) if kc else (tile, tile + 6, 4 * tile + 2)):
             assert slab.gemm_slab_check_double(kc, tile, rows, ld, 1) == 0, (kc, tile, rows, ld)
+
+
+@pytest.mark.parametrize("kc", [0, 1], ids=["contiguous_along_rows", "contiguous_along_k"])
+def test_every_complex_mfma_operand_is_the_matrix_element_it_has_to_be(slab, kc):
+    """gemm_cfloat_pipe_kernel (och_gemm_c32p_slab.h: 128 rows, 32 k) and gemm_cdouble_pipe_kernel (och_gemm_c64p_slab.h: 128
+    and 64 rows, 16 k): real and imaginary part of every operand value, whole and ragged tiles."""
+    for rows in (128, 126, 66, 64, 34, 2):
+        for ld in ((32, 34, 1000) if kc else (128, 130, 517)):
+            assert slab.gemm_slab_check_cfloat(kc, rows, ld, 1) == 0, (kc, rows, ld)
+    for tile in (128, 64):
+        for rows in sorted({tile, tile - 1, tile // 2 + 1, tile // 2, 17, 1}):
+            for ld in ((16, 18, 1000) if kc else (tile, tile + 3, 4 * tile + 1)):
+                assert slab.gemm_slab_check_cdouble(kc, tile, rows, ld, 1) == 0, (kc, tile, rows, ld)
 
 
 def test_unknown_tile_is_refused(slab):
