@@ -387,8 +387,7 @@ int och_gemm_batched(int dtype, char transA, char transB, size_t M, size_t N, si
 /* (default), 1 the pipelined kernel on its large tile wherever its conditions hold (M, N multiples of 4 or 2, K of   */
 /* the slab, 16-byte aligned operands), 2 the pipelined kernel on its small tile (float, double; complex float has    */
 /* one tile), 3 never the pipelined kernel, 4 the pipelined kernel on its smallest tile (float: 64 x 64; the other    */
-/* types: the tile the model prefers), 5 as 4 with four slab buffers in a ring instead of two. Process-wide; no       */
-/* counterpart in the reference.                                                                                      */
+/* types: the tile the model prefers). Process-wide; no counterpart in the reference.                                 */
 int och_gemm_set_kernel_choice(int choice);
 /* Which kernel the model gives an aligned float product of `batch` entries (0 or 1: a single product) with scalars  */
 /* in host memory: 256, 128 or 64 for the pipelined kernel on tiles of that edge, 0 for the tiled kernels. Host      */

@@ -163,8 +163,7 @@ int gemm_pad_tail(const GemmArgs &g, size_t Kh, int slab, int es, GemmArgs *tail
 }
 
 /* 0: the cost model chooses; 1: the pipelined kernel on its large tile wherever it applies; 2: on its small tile (float,
-   double); 3: never the pipelined kernel; 4: on its smallest tile (float; the other types: the tile the model prefers); 5: as 4, with
-   four slab buffers in a ring. For tests and measurements (och_gemm_set_kernel_choice). */
+   double); 3: never the pipelined kernel; 4: on its smallest tile (float; the other types: the tile the model prefers). For tests and measurements (och_gemm_set_kernel_choice). */
 static std::atomic<int> g_gemm_kernel_choice{0};
 int gemm_kernel_choice(void) { return g_gemm_kernel_choice.load(std::memory_order_relaxed); }
 
@@ -342,7 +341,7 @@ extern "C" int och_gemm_float_plan(size_t M, size_t N, size_t K, unsigned batch)
 
 extern "C" int och_gemm_set_kernel_choice(int choice)
 {
-   if (choice < 0 || choice > 5) return och::set_error("gemm: kernel choice %d (0 automatic, 1 pipelined large tile, 2 pipelined small tile, 3 tiled kernel, 4 pipelined smallest tile, 5 the same on four slab buffers)", choice);
+   if (choice < 0 || choice > 4) return och::set_error("gemm: kernel choice %d (0 automatic, 1 pipelined large tile, 2 pipelined small tile, 3 tiled kernel, 4 pipelined smallest tile)", choice);
    och::g_gemm_kernel_choice.store(choice, std::memory_order_relaxed);
    return 0;
 }

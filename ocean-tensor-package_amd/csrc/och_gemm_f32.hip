@@ -41,7 +41,6 @@ static int gemm_float_plan(const GemmArgs &g, int *pick)
    if (forced == 2) return 128;
    if (forced == 3) return 0;
    if (forced == 4) return 64;
-   if (forced == 5) return 65;          /* the smallest tile with a ring of four slab buffers: measurements only */
    int tile = large <= small ? 256 : 128;
    if (!((tile == 256 ? large : small) < others)) tile = 0;
    const uint64_t tiles64 = ((g.M + 63) / 64) * ((g.N + 63) / 64) * (uint64_t)g.nz;

@@ -8,8 +8,8 @@
  * of LDS and under 48 registers, up to four blocks per compute unit (1024^3: 69 TFLOP/s against 53 on the 128 x 128 tile,
  * whose 64 tiles have to be cut along K; 1536^3: 107 against 75). With one block on a compute unit its loads have only
  * three quads of four MFMAs (770 cycles) to arrive and the block waits for them: it runs at 0.7 of the matrix rate, at 0.9
- * with a second block beside it. NB = 4 keeps four slab buffers in a ring instead of two, so that a load has three
- * slabs to arrive; only the knob of the dispatcher reaches it.
+ * with a second block beside it. NB = 4 would keep four slab buffers in a ring instead of two, so that a load has three
+ * slabs to arrive; the kernel is written for it, but that form has not run on a device and is not instantiated.
  * The description is for TS = 4.
  * On this device a vector-ALU instruction of a wave takes about eight cycles away from the matrix cores of its SIMD, and
  * a 64-cycle MFMA hides none of that; LDS reads and scalar instructions are nearly free. So the main loop holds MFMAs,
@@ -323,8 +323,6 @@ int gemm_float_pipe(const GemmArgs &g, int tile)
    p.tiles_m = (uint32_t)((g.M + tile - 1) / tile); p.tiles_n = (uint32_t)((g.N + tile - 1) / tile);
    uint64_t blocks = (uint64_t)p.tiles_m * p.tiles_n;
    if (blocks > 0x7FFFFFFFull) return set_error("gemm: too many tiles");
-   const bool ring = (tile == 65);                       /* the smallest tile on four slab buffers instead of two */
-   if (ring) tile = 64;
    if (tile != 256 && tile != 128 && tile != 64) return 1;
    const int shares = gemm_float_pipe_split(g, tile, nullptr);
    uint32_t cut_tiles = 0;
@@ -346,7 +344,7 @@ int gemm_float_pipe(const GemmArgs &g, int tile)
         const size_t lds = ((SINGLE) ? 2 : 2 * (NB)) * (size_t)FloatSlab<AK, 64 * TS>::OPERAND;                       \
         OCH_CHECK_HIP(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
         hipLaunchKernelGGL(kernel, grid, block, lds, g.stream, p); } while (0)
-#define OCH_FP_PICK(AK, BK) do { if (tile == 256) OCH_FP_LAUNCH(AK, BK, 4, false, 2); else if (tile == 64 && ring) OCH_FP_LAUNCH(AK, BK, 1, false, 4); else if (tile == 64) OCH_FP_LAUNCH(AK, BK, 1, false, 2); else if (single) OCH_FP_LAUNCH(AK, BK, 2, true, 2); else OCH_FP_LAUNCH(AK, BK, 2, false, 2); } while (0)
+#define OCH_FP_PICK(AK, BK) do { if (tile == 256) OCH_FP_LAUNCH(AK, BK, 4, false, 2); else if (tile == 64) OCH_FP_LAUNCH(AK, BK, 1, false, 2); else if (single) OCH_FP_LAUNCH(AK, BK, 2, true, 2); else OCH_FP_LAUNCH(AK, BK, 2, false, 2); } while (0)
    if (!akc && !bkc) OCH_FP_PICK(false, false);
    else if (!akc)    OCH_FP_PICK(false, true);
    else if (!bkc)    OCH_FP_PICK(true, false);

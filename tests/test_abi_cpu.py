@@ -209,11 +209,11 @@ def test_kernel_choice():
 
 
 def test_gemm_kernel_choice_knob_checks_its_argument():
-    """och_gemm_set_kernel_choice touches no device: 0 to 5 are accepted, anything else is refused with a message."""
+    """och_gemm_set_kernel_choice touches no device: 0 to 4 are accepted, anything else is refused with a message."""
     import ocean_hip as oh
-    for choice in (1, 2, 3, 4, 5, 0):
+    for choice in (1, 2, 3, 4, 0):
         assert oh.lib.och_gemm_set_kernel_choice(choice) == 0
-    for choice in (-1, 6, 99):
+    for choice in (-1, 5, 99):
         assert oh.lib.och_gemm_set_kernel_choice(choice) != 0
         assert b"kernel choice" in oh.lib.och_last_error()
     assert oh.lib.och_gemm_set_kernel_choice(0) == 0
